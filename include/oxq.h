@@ -1,0 +1,192 @@
+/*
+ * oxq.h -- C ABI of liboxq_hip.so: oxillama-quant's quantized matmul hot path on
+ * one MI355X (gfx950), hand-written HIP.
+ *
+ * The entry points are what an `impl QuantKernel for HipKernel` in the reference
+ * crate would bind over `extern "C"`: plain pointers and sizes, an int status per
+ * call, nothing retained beyond the call unless a handle says so.  Citations name
+ * the reference interface each one stands in for (paths relative to the reference
+ * tree, Q/ = crates/oxillama-quant/src).
+ *
+ * Weight bytes are raw GGUF blocks exactly as `GgufModel::tensor_data` hands them
+ * out (crates/oxillama-gguf/src/loader.rs:115), row-major, row_bytes =
+ * ceil(n_cols / block_size) * block_bytes (Q/reference/q4_k.rs:130-131).  They go
+ * to HBM unchanged; nothing is repacked.
+ *
+ * Supported formats: Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS.  Shapes whose n_cols is not
+ * a multiple of the format's block size return OXQ_ERR_UNSUPPORTED_SHAPE so the
+ * caller can fall back to its CPU kernel.
+ *
+ * Thread safety: every function may be called from several host threads; calls
+ * taking host slices serialise on an internal lock.
+ */
+#ifndef OXQ_H
+#define OXQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GgufTensorType discriminants, crates/oxillama-gguf/src/types.rs:72-150. */
+#define OXQ_TYPE_Q4_0 2u
+#define OXQ_TYPE_Q8_0 8u
+#define OXQ_TYPE_Q4_K 12u
+#define OXQ_TYPE_Q6_K 14u
+#define OXQ_TYPE_IQ4_XS 23u
+
+/* Status codes: 1..7 are the QuantError variants of Q/error.rs:10-71 in order;
+ * the (expected, got) / (needed, available) pair of the failing check is kept per
+ * thread and read back with oxq_last_error(). */
+#define OXQ_OK 0
+#define OXQ_ERR_UNSUPPORTED_TYPE 1     /* QuantError::UnsupportedType */
+#define OXQ_ERR_BLOCK_SIZE_MISMATCH 2  /* QuantError::BlockSizeMismatch */
+#define OXQ_ERR_DIMENSION_MISMATCH 3   /* QuantError::DimensionMismatch{expected, got} */
+#define OXQ_ERR_KERNEL 4               /* QuantError::KernelError{message} (HIP failures) */
+#define OXQ_ERR_BLOCK_COUNT_MISMATCH 5 /* QuantError::BlockCountMismatch */
+#define OXQ_ERR_BUFFER_TOO_SMALL 6     /* QuantError::BufferTooSmall{needed, available} */
+#define OXQ_ERR_INTERNAL 7             /* QuantError::Internal{message} */
+#define OXQ_ERR_UNSUPPORTED_SHAPE 8    /* no reference counterpart: fall back to the CPU kernel */
+#define OXQ_ERR_NO_DEVICE 9            /* no reference counterpart: no usable GPU */
+
+typedef struct oxq_device_props {
+    int device;
+    int compute_units;
+    int clock_khz;        /* peak engine clock */
+    int memory_clock_khz;
+    int memory_bus_bits;
+    size_t total_memory;
+    char name[128];
+    char arch[64];
+} oxq_device_props;
+
+/* Opaque handle to weights resident in HBM. */
+typedef struct oxq_weights *oxq_weights_t;
+
+/* ---- lifetime ---------------------------------------------------------- */
+
+/* Select the GPU used by this library (KernelDispatcher::new + SimdCapabilities::
+ * detect, Q/dispatch.rs:42,131: the run-time capability probe of the tier).
+ * Idempotent.  OXQ_ERR_NO_DEVICE when no gfx950-class device is visible. */
+int oxq_init(int device);
+/* Free cached weights and scratch memory.  Handles become invalid. */
+int oxq_shutdown(void);
+int oxq_device_info(oxq_device_props *out);
+
+/* Detail of the last failing call on this thread.  `a` = expected / needed,
+ * `b` = got / available; `message` may be NULL. */
+int oxq_last_error(size_t *a, size_t *b, char *message, size_t message_len);
+const char *oxq_status_name(int status);
+
+/* ---- format metadata: QuantKernel::block_size / block_bytes / name ----- */
+/* Q/traits.rs:175-182; values of crates/oxillama-gguf/src/types.rs:199-262.  0 /
+ * NULL for a format this library has no kernel for. */
+size_t oxq_block_size(uint32_t type);
+size_t oxq_block_bytes(uint32_t type);
+const char *oxq_type_name(uint32_t type);
+/* KernelDispatcher::get_kernel, Q/dispatch.rs:141: OXQ_OK if a HIP kernel exists
+ * for `type`, else OXQ_ERR_UNSUPPORTED_TYPE (the shim then tries the next tier). */
+int oxq_get_kernel(uint32_t type);
+
+/* ---- QuantKernel methods on host slices (the drop-in route) ------------ */
+
+/* QuantKernel::dequant_block, Q/traits.rs:28.  Checks as Q/reference/q4_k.rs:
+ * 53-64: block_len < block_bytes -> BUFFER_TOO_SMALL, then out_len < block_size
+ * -> BUFFER_TOO_SMALL.  Runs on the GPU. */
+int oxq_dequant_block(uint32_t type, const uint8_t *block, size_t block_len, float *output,
+                      size_t output_len);
+
+/* quantize_f32_to_q8_0, Q/quantize.rs:58-75.  n % 32 != 0 -> DIMENSION_MISMATCH
+ * {expected: (n/32+1)*32, got: n}.  out_len must hold n/32 * 34 bytes.  Output
+ * bytes are bit-identical to the reference encoder (Q/quantize.rs:190-210). */
+int oxq_quantize_f32_to_q8_0(const float *data, size_t n, uint8_t *out, size_t out_len);
+
+/* QuantKernel::matvec_q8_fused, Q/traits.rs:89-96: out[r] += W[r,:] . acts
+ * (ACCUMULATE).  Validation order of Q/reference/q4_k.rs:226-250: out_len <
+ * n_rows -> DIMENSION_MISMATCH{n_rows, out_len}; weights_len < n_rows*row_bytes
+ * -> BUFFER_TOO_SMALL; acts_len < blocks_per_row*(block_size/32)*34 ->
+ * BUFFER_TOO_SMALL. */
+int oxq_matvec_q8_fused(uint32_t type, const uint8_t *weights, size_t weights_len,
+                        const uint8_t *acts_q8, size_t acts_len, float *out, size_t out_len,
+                        size_t n_rows, size_t n_cols);
+
+/* QuantKernel::gemv, Q/traits.rs:39-44, on a QuantTensor given as (data, shape,
+ * type) (Q/types.rs:11-18).  output[r] is overwritten.  n_rows = shape[0], n_cols
+ * = shape[1] (or n_elements / n_rows for a 1-d shape), Q/reference/q4_k.rs:110-115;
+ * input_len < n_cols -> DIMENSION_MISMATCH{n_cols, input_len}; output_len <
+ * n_rows -> DIMENSION_MISMATCH{n_rows, output_len} (:117-128).
+ * The activation vector is quantized to Q8_0 on the GPU and fed to the fused
+ * kernel: results equal oxq_quantize_f32_to_q8_0 + oxq_matvec_q8_fused into
+ * zeros, and differ from the reference's f32-activation gemv by the Q8_0
+ * rounding of the input.  n_cols must be a multiple of 32. */
+int oxq_gemv(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape,
+             size_t n_dims, const float *input, size_t input_len, float *output,
+             size_t output_len);
+
+/* QuantKernel::gemm, Q/traits.rs:58-66: input [m x k] row-major, output [m x n]
+ * row-major, overwritten; same activation handling as oxq_gemv, row by row
+ * (Q/reference/q4_k.rs:186-201). */
+int oxq_gemm(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape,
+             size_t n_dims, const float *input, size_t input_len, float *output,
+             size_t output_len, size_t m, size_t n, size_t k);
+
+/* Debug: exact int32 group sums of the fused kernel, sums[r * groups + g] with
+ * groups = n_cols/32 (n_cols/16 for Q6_K).  Q4_0: sum (q-8)a; Q8_0: sum w a;
+ * Q4_K: sum q a; Q6_K: sum (q-32)a; IQ4_XS: sum kvalues[q] a.  No reference
+ * counterpart (the reference's AVX2 rows form the same sums in registers,
+ * Q/simd/avx2/q4_k.rs:298-318). */
+int oxq_block_sums(uint32_t type, const uint8_t *weights, size_t weights_len,
+                   const uint8_t *acts_q8, size_t acts_len, int32_t *sums, size_t sums_len,
+                   size_t n_rows, size_t n_cols);
+
+/* When enabled, host-slice calls keep a device copy of each weight buffer keyed
+ * by (pointer, length, type) plus a fingerprint of sampled bytes, so repeated
+ * calls with the same QuantTensor do not cross PCIe again.  Off by default: the
+ * caller must not mutate cached buffers.  Stands in for the ownership the
+ * reference gets for free from host slices (Q/types.rs:11-18). */
+int oxq_weight_cache_enable(int enabled);
+int oxq_weight_cache_clear(void);
+
+/* ---- weights resident in HBM ------------------------------------------- */
+
+/* Copy a weight matrix to HBM once (what load_quant_linear's data.to_vec() is to
+ * the CPU path, crates/oxillama-arch/src/llama/model.rs:805-822). */
+int oxq_weights_register(uint32_t type, size_t n_rows, size_t n_cols, const uint8_t *bytes,
+                         size_t len, oxq_weights_t *handle);
+int oxq_weights_release(oxq_weights_t handle);
+/* Device address / byte length of the registered blocks. */
+void *oxq_weights_device_ptr(oxq_weights_t handle);
+size_t oxq_weights_nbytes(oxq_weights_t handle);
+
+/* ---- device-pointer entry points (no copies, asynchronous) ------------- */
+/* All pointers are device memory; `stream` is a hipStream_t (NULL = default
+ * stream).  Shapes are validated as above (lengths are the caller's promise);
+ * kernels are enqueued and the call returns. */
+
+/* quantize_f32_to_q8_0 over `rows` rows of n floats each (rows*n contiguous). */
+int oxq_quantize_q8_0_dev(const float *d_x, size_t n_total, uint8_t *d_out, void *stream);
+
+/* matvec_q8_fused: d_out[r] += ... ; accumulate = 0 overwrites instead (gemv). */
+int oxq_matvec_q8_fused_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
+                            float *d_out, size_t n_rows, size_t n_cols, int accumulate,
+                            void *stream);
+
+/* Prefill: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched form
+ * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  Q4_K uses
+ * the int8-MFMA tile kernel; other formats run m fused matvecs. */
+int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
+                    float *d_out, size_t m, size_t n, size_t k, int accumulate, void *stream);
+
+int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
+                       int32_t *d_sums, size_t n_rows, size_t n_cols, void *stream);
+
+/* Launch width of the GEMV kernels: resident waves per compute unit (tuning
+ * knob for benchmarks; 0 restores the default). */
+int oxq_set_gemv_waves_per_cu(unsigned waves);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OXQ_H */

@@ -1,0 +1,124 @@
+/*
+ * oxq_oracle.h -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * Scalar C restatement of oxillama-quant's CPU kernels for the quantized-matmul
+ * path (reference = /root/reference/crates/oxillama-quant/src, abbreviated Q/).
+ * Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may load
+ * this library; the shipped HIP path never calls it.
+ *
+ * Every function names the reference lines whose operation order it follows.
+ * Build with -O2 -ffp-contract=off -fno-fast-math: Rust neither contracts
+ * a*b+c into an fma nor reassociates floating point.
+ *
+ * Pinning (what each group of functions is checked against, see tests/):
+ *   f16 <-> f32            all 65 536 halves and random floats vs F16C hardware
+ *   quantizers             closed-form invariants and the reference's own test
+ *                          vectors (Q/quantize.rs:225-445)
+ *   dequant_block, gemv    the reference's hand-built block tests
+ *                          (Q/reference/{q4_0,q8_0,q4_k,q6_k,iq4_xs}.rs tests)
+ *   matvec_q8_fused        fused == unfused identities, accumulate semantics,
+ *                          zero cases, AVX2-tier fixtures (Q/simd/avx2/ tests)
+ *   block integer sums     brute force from dequantized integer weights
+ *   IQ4_XS fused           the reference has no working implementation (the
+ *                          trait default indexes a 32-entry scratch with 256
+ *                          weights, Q/traits.rs:135,158-166); the integer form
+ *                          defined here is pinned against the reference gemv
+ *                          applied to dequantized activations.
+ */
+#ifndef OXQ_ORACLE_H
+#define OXQ_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* GgufTensorType ids, crates/oxillama-gguf/src/types.rs:72-150 */
+enum {
+    OXQ_REF_Q4_0 = 2,
+    OXQ_REF_Q8_0 = 8,
+    OXQ_REF_Q4_K = 12,
+    OXQ_REF_Q6_K = 14,
+    OXQ_REF_IQ4_XS = 23
+};
+
+/* QuantError variants, Q/error.rs:10-71 */
+enum {
+    OXQ_REF_OK = 0,
+    OXQ_REF_UNSUPPORTED_TYPE = 1,
+    OXQ_REF_BLOCK_SIZE_MISMATCH = 2,
+    OXQ_REF_DIMENSION_MISMATCH = 3, /* a = expected, b = got */
+    OXQ_REF_KERNEL_ERROR = 4,
+    OXQ_REF_BLOCK_COUNT_MISMATCH = 5,
+    OXQ_REF_BUFFER_TOO_SMALL = 6, /* a = needed, b = available */
+    OXQ_REF_INTERNAL = 7
+};
+
+/* matvec_q8_fused tiers */
+enum {
+    OXQ_REF_TIER_SCALAR = 0,     /* what the *Ref kernels run */
+    OXQ_REF_TIER_AVX2 = 1,       /* operation order of Q/simd/avx2 fused rows */
+    OXQ_REF_TIER_Q4_0_STANDALONE = 2 /* Q/reference/q4_0.rs:159 */
+};
+
+typedef struct {
+    int code;
+    size_t a;
+    size_t b;
+} oxq_ref_status;
+
+size_t oxq_ref_block_size(uint32_t type);
+size_t oxq_ref_block_bytes(uint32_t type);
+
+uint16_t oxq_ref_f32_to_f16(float v);
+float oxq_ref_f16_to_f32(uint16_t h);
+
+oxq_ref_status oxq_ref_quantize_f32_to_q8_0(const float *x, size_t n, uint8_t *out);
+oxq_ref_status oxq_ref_quantize_f32_to_q4_0(const float *x, size_t n, uint8_t *out);
+
+oxq_ref_status oxq_ref_dequant_block(uint32_t type, const uint8_t *block, size_t block_len,
+                                     float *out, size_t out_len);
+
+oxq_ref_status oxq_ref_gemv(uint32_t type, const uint8_t *w, size_t w_len, size_t n_rows,
+                            size_t n_cols, const float *x, size_t x_len, float *y, size_t y_len);
+
+oxq_ref_status oxq_ref_gemm(uint32_t type, const uint8_t *w, size_t w_len, const float *x,
+                            float *y, size_t m, size_t n, size_t k);
+
+oxq_ref_status oxq_ref_matvec_q8_fused(uint32_t type, int tier, const uint8_t *w, size_t w_len,
+                                       const uint8_t *acts, size_t acts_len, float *out,
+                                       size_t out_len, size_t n_rows, size_t n_cols);
+
+/* Integer-dot form shared by every format: per (row, integer group) the exact
+ * int32 sum, then one fp32 term per group.  Group = 32 weights (one Q8_0
+ * activation block) for Q4_0/Q8_0/Q4_K/IQ4_XS and 16 weights for Q6_K. */
+oxq_ref_status oxq_ref_matvec_q8_intdot(uint32_t type, const uint8_t *w, size_t w_len,
+                                        const uint8_t *acts, size_t acts_len, float *out,
+                                        size_t out_len, size_t n_rows, size_t n_cols);
+
+/* sums[row * groups_per_row + g]; groups_per_row = n_cols/32 (n_cols/16 for Q6_K).
+ * Q4_0: sum (q-8)*a; Q8_0: sum w*a; Q4_K: sum q*a (unsigned nibble); Q6_K:
+ * sum (q-32)*a; IQ4_XS: sum kvalues[q]*a.  n_cols must be a block multiple. */
+oxq_ref_status oxq_ref_block_sums(uint32_t type, const uint8_t *w, size_t w_len,
+                                  const uint8_t *acts, size_t acts_len, int32_t *sums,
+                                  size_t n_rows, size_t n_cols);
+
+/* Prefill: quantize each of the m activation rows to Q8_0, then m fused matvecs
+ * into a zeroed y[m x n] (gemm semantics of Q/reference/q4_k.rs:186-201 applied
+ * to the Q8_0-activation path). */
+oxq_ref_status oxq_ref_gemm_q8(uint32_t type, int tier, const uint8_t *w, size_t w_len,
+                               const float *x, float *y, size_t m, size_t n, size_t k);
+
+/* Multi-threaded row split of the AVX2-order fused matvec: parallel_gemv
+ * semantics (Q/parallel.rs:70-77), used only for the CPU baseline timing. */
+oxq_ref_status oxq_ref_matvec_q8_fused_mt(uint32_t type, int tier, const uint8_t *w, size_t w_len,
+                                          const uint8_t *acts, size_t acts_len, float *out,
+                                          size_t out_len, size_t n_rows, size_t n_cols,
+                                          int n_threads);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,56 @@
+"""Build the native libraries of this package in-tree.
+
+`python -m oxillama_amd.build` compiles
+  * oxillama_amd/liboxq_hip.so   -- HIP kernels + C ABI (include/oxq.h), gfx950 only
+  * oxillama_amd/liboxq_synth.so -- host-side synthetic weight generator
+hipcc cross-compiles gfx950 code objects without a GPU present.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+HIP_SOURCES = ["oxq_api.hip", "oxq_gemv.hip", "oxq_gemm.hip", "oxq_quantize.hip"]
+HIP_LIB = os.path.join(HERE, "liboxq_hip.so")
+SYNTH_LIB = os.path.join(HERE, "liboxq_synth.so")
+
+# -ffp-contract=off: the fp32 epilogues follow the reference's operation order (Rust
+# never fuses a*b+c).  Packed fp32 instructions are switched off.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall", "-Wno-unused-function",
+]
+
+
+def run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+
+
+def build_hip(extra=()):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objs = []
+    for src in HIP_SOURCES:
+        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        run([hipcc, *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj])
+        objs.append(obj)
+    run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB, *objs])
+    return HIP_LIB
+
+
+def build_synth():
+    run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-pthread", "-ffp-contract=off",
+         "-o", SYNTH_LIB, os.path.join(CSRC, "synth.cpp")])
+    return SYNTH_LIB
+
+
+def build_all():
+    build_hip()
+    build_synth()
+
+
+if __name__ == "__main__":
+    build_all()
+    sys.exit(0)

@@ -1,0 +1,108 @@
+"""ctypes binding of liboxq_hip.so (the C ABI declared in include/oxq.h).
+
+Plumbing for the Python tests and bench.py.  There is no fallback: if the HIP
+library has not been built, loading raises.
+"""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "liboxq_hip.so")
+
+OK = 0
+ERR_UNSUPPORTED_TYPE = 1
+ERR_BLOCK_SIZE_MISMATCH = 2
+ERR_DIMENSION_MISMATCH = 3
+ERR_KERNEL = 4
+ERR_BLOCK_COUNT_MISMATCH = 5
+ERR_BUFFER_TOO_SMALL = 6
+ERR_INTERNAL = 7
+ERR_UNSUPPORTED_SHAPE = 8
+ERR_NO_DEVICE = 9
+
+TYPE_Q4_0, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q6_K, TYPE_IQ4_XS = 2, 8, 12, 14, 23
+
+# Every symbol include/oxq.h declares, with its signature.
+_u8p = C.POINTER(C.c_uint8)
+_f32p = C.POINTER(C.c_float)
+_i32p = C.POINTER(C.c_int32)
+_szp = C.POINTER(C.c_size_t)
+
+
+class DeviceProps(C.Structure):
+    _fields_ = [
+        ("device", C.c_int),
+        ("compute_units", C.c_int),
+        ("clock_khz", C.c_int),
+        ("memory_clock_khz", C.c_int),
+        ("memory_bus_bits", C.c_int),
+        ("total_memory", C.c_size_t),
+        ("name", C.c_char * 128),
+        ("arch", C.c_char * 64),
+    ]
+
+
+SIGNATURES = {
+    "oxq_init": (C.c_int, [C.c_int]),
+    "oxq_shutdown": (C.c_int, []),
+    "oxq_device_info": (C.c_int, [C.POINTER(DeviceProps)]),
+    "oxq_last_error": (C.c_int, [_szp, _szp, C.c_char_p, C.c_size_t]),
+    "oxq_status_name": (C.c_char_p, [C.c_int]),
+    "oxq_block_size": (C.c_size_t, [C.c_uint32]),
+    "oxq_block_bytes": (C.c_size_t, [C.c_uint32]),
+    "oxq_type_name": (C.c_char_p, [C.c_uint32]),
+    "oxq_get_kernel": (C.c_int, [C.c_uint32]),
+    "oxq_dequant_block": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t]),
+    "oxq_quantize_f32_to_q8_0": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t]),
+    "oxq_matvec_q8_fused": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                      C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]),
+    "oxq_gemv": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, _szp, C.c_size_t, C.c_void_p,
+                           C.c_size_t, C.c_void_p, C.c_size_t]),
+    "oxq_gemm": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, _szp, C.c_size_t, C.c_void_p,
+                           C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t]),
+    "oxq_block_sums": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                 C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]),
+    "oxq_weight_cache_enable": (C.c_int, [C.c_int]),
+    "oxq_weight_cache_clear": (C.c_int, []),
+    "oxq_weights_register": (C.c_int, [C.c_uint32, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t,
+                                       C.POINTER(C.c_void_p)]),
+    "oxq_weights_release": (C.c_int, [C.c_void_p]),
+    "oxq_weights_device_ptr": (C.c_void_p, [C.c_void_p]),
+    "oxq_weights_nbytes": (C.c_size_t, [C.c_void_p]),
+    "oxq_quantize_q8_0_dev": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]),
+    "oxq_matvec_q8_fused_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
+                                          C.c_size_t, C.c_int, C.c_void_p]),
+    "oxq_gemm_q8_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
+                                  C.c_size_t, C.c_size_t, C.c_int, C.c_void_p]),
+    "oxq_block_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
+                                     C.c_size_t, C.c_void_p]),
+    "oxq_set_gemv_waves_per_cu": (C.c_int, [C.c_uint]),
+}
+
+_lib = None
+
+
+def load():
+    """Load liboxq_hip.so and attach signatures.  Raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m oxillama_amd.build` "
+            "(there is no CPU fallback for the HIP path)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the ABI lost a symbol
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def last_error():
+    lib = load()
+    a, b = C.c_size_t(0), C.c_size_t(0)
+    msg = C.create_string_buffer(256)
+    status = lib.oxq_last_error(C.byref(a), C.byref(b), msg, 256)
+    return status, a.value, b.value, msg.value.decode("utf-8", "replace")

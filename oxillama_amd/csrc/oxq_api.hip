@@ -1,0 +1,597 @@
+// C ABI of liboxq_hip.so (see include/oxq.h): argument validation in the
+// reference's order, HBM residency of weights, scratch buffers for the
+// host-slice route, and kernel launches.  No exception or abort crosses the ABI.
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <unordered_map>
+#include <vector>
+
+#include "oxq_internal.hpp"
+
+namespace oxq {
+hipError_t launch_dequant(uint32_t type, const uint8_t *blocks, size_t n_blocks, float *out, hipStream_t stream);
+}
+
+struct oxq_weights {
+    uint32_t type;
+    size_t n_rows, n_cols, nbytes;
+    uint8_t *dev;
+};
+
+namespace {
+
+struct ErrorDetail {
+    int status = OXQ_OK;
+    size_t a = 0, b = 0;
+    char message[256] = {0};
+};
+thread_local ErrorDetail g_err;
+
+int fail(int status, size_t a, size_t b, const char *msg) {
+    g_err.status = status;
+    g_err.a = a;
+    g_err.b = b;
+    std::snprintf(g_err.message, sizeof(g_err.message), "%s", msg ? msg : "");
+    return status;
+}
+
+int fail_hip(hipError_t e, const char *what) {
+    char buf[256];
+    std::snprintf(buf, sizeof(buf), "%s: %s", what, hipGetErrorString(e));
+    return fail(OXQ_ERR_KERNEL, (size_t)e, 0, buf);
+}
+
+#define OXQ_HIP(call)                                     \
+    do {                                                  \
+        hipError_t e_ = (call);                           \
+        if (e_ != hipSuccess) return fail_hip(e_, #call); \
+    } while (0)
+
+// A growable device buffer.
+struct Scratch {
+    void *ptr = nullptr;
+    size_t cap = 0;
+    int reserve(size_t n) {
+        if (n <= cap) return OXQ_OK;
+        if (ptr) (void)hipFree(ptr);
+        ptr = nullptr;
+        cap = 0;
+        size_t want = n + n / 4 + 256;
+        hipError_t e = hipMalloc(&ptr, want);
+        if (e != hipSuccess) return fail_hip(e, "hipMalloc(scratch)");
+        cap = want;
+        return OXQ_OK;
+    }
+    void release() {
+        if (ptr) (void)hipFree(ptr);
+        ptr = nullptr;
+        cap = 0;
+    }
+};
+
+struct CacheKey {
+    const void *ptr;
+    size_t len;
+    uint32_t type;
+    bool operator==(const CacheKey &o) const { return ptr == o.ptr && len == o.len && type == o.type; }
+};
+struct CacheKeyHash {
+    size_t operator()(const CacheKey &k) const {
+        return std::hash<const void *>()(k.ptr) ^ (k.len * 0x9E3779B97F4A7C15ull) ^ k.type;
+    }
+};
+struct CacheEntry {
+    uint8_t *dev;
+    uint64_t fingerprint;
+};
+
+struct State {
+    std::mutex mu;
+    bool initialised = false;
+    int device = -1;
+    uint32_t cus = 0;
+    uint32_t waves_per_cu = 0;  // 0 = default
+    bool cache_enabled = false;
+    std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
+    Scratch s_weights, s_acts, s_x, s_out, s_sums;
+};
+State g;
+
+constexpr uint32_t DEFAULT_WAVES_PER_CU = 8;
+
+// FNV-1a over up to 64 samples of 64 bytes spread across the buffer, plus its length.
+uint64_t fingerprint(const uint8_t *p, size_t len) {
+    uint64_t h = 1469598103934665603ull ^ len;
+    const size_t chunk = 64, samples = 64;
+    if (len <= chunk * samples) {
+        for (size_t i = 0; i < len; i++) h = (h ^ p[i]) * 1099511628211ull;
+        return h;
+    }
+    const size_t stride = (len - chunk) / (samples - 1);
+    for (size_t s = 0; s < samples; s++) {
+        const uint8_t *q = p + s * stride;
+        for (size_t i = 0; i < chunk; i++) h = (h ^ q[i]) * 1099511628211ull;
+    }
+    return h;
+}
+
+bool known_type(uint32_t type) { return oxq_block_size(type) != 0; }
+
+int ensure_init() {
+    if (g.initialised) return OXQ_OK;
+    return oxq_init(0);
+}
+
+// Device copy of a host weight buffer: cached when the cache is on, else staged
+// in scratch.  Caller holds g.mu.
+int stage_weights(uint32_t type, const uint8_t *host, size_t len, const uint8_t **dev) {
+    if (g.cache_enabled) {
+        CacheKey key{host, len, type};
+        const uint64_t fp = fingerprint(host, len);
+        auto it = g.cache.find(key);
+        if (it != g.cache.end() && it->second.fingerprint == fp) {
+            *dev = it->second.dev;
+            return OXQ_OK;
+        }
+        if (it != g.cache.end()) {
+            (void)hipFree(it->second.dev);
+            g.cache.erase(it);
+        }
+        uint8_t *d = nullptr;
+        OXQ_HIP(hipMalloc((void **)&d, len ? len : 1));
+        hipError_t e = hipMemcpy(d, host, len, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(d);
+            return fail_hip(e, "hipMemcpy(weights)");
+        }
+        g.cache.emplace(key, CacheEntry{d, fp});
+        *dev = d;
+        return OXQ_OK;
+    }
+    int st = g.s_weights.reserve(len ? len : 1);
+    if (st != OXQ_OK) return st;
+    OXQ_HIP(hipMemcpy(g.s_weights.ptr, host, len, hipMemcpyHostToDevice));
+    *dev = (const uint8_t *)g.s_weights.ptr;
+    return OXQ_OK;
+}
+
+struct FusedShape {
+    size_t bpr, row_bytes, acts_needed;
+};
+
+// Validation order of the reference's matvec_q8_fused
+// (crates/oxillama-quant/src/reference/q4_k.rs:226-250, traits.rs:99-130).
+int validate_fused(uint32_t type, size_t weights_len, size_t acts_len, size_t out_len, size_t n_rows,
+                   size_t n_cols, FusedShape *fs) {
+    if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
+    if (out_len < n_rows) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_rows, out_len, "out shorter than n_rows");
+    const size_t bs = oxq_block_size(type), bb = oxq_block_bytes(type);
+    fs->bpr = (n_cols + bs - 1) / bs;
+    fs->row_bytes = fs->bpr * bb;
+    fs->acts_needed = fs->bpr * (bs / 32) * 34;
+    if (weights_len < n_rows * fs->row_bytes)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * fs->row_bytes, weights_len, "weights buffer too small");
+    if (acts_len < fs->acts_needed)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, fs->acts_needed, acts_len, "activation buffer too small");
+    if (n_cols % bs != 0)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows > n_cols ? n_rows : n_cols, "dimension exceeds 2^32-1");
+    return OXQ_OK;
+}
+
+oxq::GemvArgs gemv_args(const uint8_t *W, const uint8_t *A, float *out, int32_t *sums, size_t n_rows,
+                        size_t n_cols, int accumulate) {
+    oxq::GemvArgs a;
+    a.W = W;
+    a.A = A;
+    a.out = out;
+    a.sums = sums;
+    a.n_rows = (uint32_t)n_rows;
+    a.n_cols = (uint32_t)n_cols;
+    a.accumulate = accumulate;
+    a.waves_per_cu = g.waves_per_cu ? g.waves_per_cu : DEFAULT_WAVES_PER_CU;
+    return a;
+}
+
+// Resolve (n_rows, n_cols) of a QuantTensor as the reference's gemv does
+// (reference/q4_k.rs:110-115).
+int tensor_dims(uint32_t type, size_t data_len, const size_t *shape, size_t n_dims, size_t *n_rows,
+                size_t *n_cols) {
+    if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
+    if (!shape || n_dims == 0) return fail(OXQ_ERR_DIMENSION_MISMATCH, 1, 0, "tensor shape is empty");
+    *n_rows = shape[0];
+    if (n_dims > 1) {
+        *n_cols = shape[1];
+    } else {
+        if (shape[0] == 0) return fail(OXQ_ERR_DIMENSION_MISMATCH, 1, 0, "tensor has zero rows");
+        size_t n_elems = 1;
+        for (size_t i = 0; i < n_dims; i++) n_elems *= shape[i];
+        *n_cols = n_elems / shape[0];
+    }
+    (void)data_len;
+    return OXQ_OK;
+}
+
+}  // namespace
+
+namespace oxq {
+uint32_t device_cus() { return g.cus ? g.cus : 256; }
+}  // namespace oxq
+
+extern "C" {
+
+int oxq_init(int device) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    if (g.initialised && g.device == device) return OXQ_OK;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(OXQ_ERR_NO_DEVICE, 0, 0, "no HIP device visible");
+    }
+    if (device < 0 || device >= count) return fail(OXQ_ERR_NO_DEVICE, (size_t)count, (size_t)device, "device index out of range");
+    OXQ_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    OXQ_HIP(hipGetDeviceProperties(&prop, device));
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        char msg[200];
+        std::snprintf(msg, sizeof(msg), "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+        return fail(OXQ_ERR_NO_DEVICE, 0, 0, msg);
+    }
+    g.device = device;
+    g.cus = (uint32_t)prop.multiProcessorCount;
+    g.initialised = true;
+    return OXQ_OK;
+}
+
+int oxq_shutdown(void) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    if (!g.initialised) return OXQ_OK;
+    for (auto &kv : g.cache) (void)hipFree(kv.second.dev);
+    g.cache.clear();
+    g.s_weights.release();
+    g.s_acts.release();
+    g.s_x.release();
+    g.s_out.release();
+    g.s_sums.release();
+    g.initialised = false;
+    g.device = -1;
+    return OXQ_OK;
+}
+
+int oxq_device_info(oxq_device_props *out) {
+    if (!out) return fail(OXQ_ERR_INTERNAL, 0, 0, "null output");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    hipDeviceProp_t prop;
+    OXQ_HIP(hipGetDeviceProperties(&prop, g.device));
+    std::memset(out, 0, sizeof(*out));
+    out->device = g.device;
+    out->compute_units = prop.multiProcessorCount;
+    out->clock_khz = prop.clockRate;
+    out->memory_clock_khz = prop.memoryClockRate;
+    out->memory_bus_bits = prop.memoryBusWidth;
+    out->total_memory = prop.totalGlobalMem;
+    std::snprintf(out->name, sizeof(out->name), "%s", prop.name);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", prop.gcnArchName);
+    return OXQ_OK;
+}
+
+int oxq_last_error(size_t *a, size_t *b, char *message, size_t message_len) {
+    if (a) *a = g_err.a;
+    if (b) *b = g_err.b;
+    if (message && message_len) std::snprintf(message, message_len, "%s", g_err.message);
+    return g_err.status;
+}
+
+const char *oxq_status_name(int status) {
+    switch (status) {
+    case OXQ_OK: return "Ok";
+    case OXQ_ERR_UNSUPPORTED_TYPE: return "UnsupportedType";
+    case OXQ_ERR_BLOCK_SIZE_MISMATCH: return "BlockSizeMismatch";
+    case OXQ_ERR_DIMENSION_MISMATCH: return "DimensionMismatch";
+    case OXQ_ERR_KERNEL: return "KernelError";
+    case OXQ_ERR_BLOCK_COUNT_MISMATCH: return "BlockCountMismatch";
+    case OXQ_ERR_BUFFER_TOO_SMALL: return "BufferTooSmall";
+    case OXQ_ERR_INTERNAL: return "Internal";
+    case OXQ_ERR_UNSUPPORTED_SHAPE: return "UnsupportedShape";
+    case OXQ_ERR_NO_DEVICE: return "NoDevice";
+    default: return "Unknown";
+    }
+}
+
+size_t oxq_block_size(uint32_t type) {
+    switch (type) {
+    case OXQ_TYPE_Q4_0:
+    case OXQ_TYPE_Q8_0: return 32;
+    case OXQ_TYPE_Q4_K:
+    case OXQ_TYPE_Q6_K:
+    case OXQ_TYPE_IQ4_XS: return 256;
+    default: return 0;
+    }
+}
+
+size_t oxq_block_bytes(uint32_t type) {
+    switch (type) {
+    case OXQ_TYPE_Q4_0: return 18;
+    case OXQ_TYPE_Q8_0: return 34;
+    case OXQ_TYPE_Q4_K: return 144;
+    case OXQ_TYPE_Q6_K: return 210;
+    case OXQ_TYPE_IQ4_XS: return 136;
+    default: return 0;
+    }
+}
+
+const char *oxq_type_name(uint32_t type) {
+    switch (type) {
+    case OXQ_TYPE_Q4_0: return "Q4_0";
+    case OXQ_TYPE_Q8_0: return "Q8_0";
+    case OXQ_TYPE_Q4_K: return "Q4_K";
+    case OXQ_TYPE_Q6_K: return "Q6_K";
+    case OXQ_TYPE_IQ4_XS: return "IQ4_XS";
+    default: return nullptr;
+    }
+}
+
+int oxq_get_kernel(uint32_t type) {
+    if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
+    return OXQ_OK;
+}
+
+int oxq_set_gemv_waves_per_cu(unsigned waves) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    g.waves_per_cu = waves > 64 ? 64 : waves;
+    return OXQ_OK;
+}
+
+int oxq_weight_cache_enable(int enabled) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    g.cache_enabled = enabled != 0;
+    return OXQ_OK;
+}
+
+int oxq_weight_cache_clear(void) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    for (auto &kv : g.cache) (void)hipFree(kv.second.dev);
+    g.cache.clear();
+    return OXQ_OK;
+}
+
+// ---- host-slice route ---------------------------------------------------
+
+int oxq_dequant_block(uint32_t type, const uint8_t *block, size_t block_len, float *output, size_t output_len) {
+    if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
+    const size_t bs = oxq_block_size(type), bb = oxq_block_bytes(type);
+    if (block_len < bb) return fail(OXQ_ERR_BUFFER_TOO_SMALL, bb, block_len, "block too small");
+    if (output_len < bs) return fail(OXQ_ERR_BUFFER_TOO_SMALL, bs, output_len, "output too small");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    std::lock_guard<std::mutex> lock(g.mu);
+    if ((st = g.s_acts.reserve(bb)) != OXQ_OK) return st;
+    if ((st = g.s_out.reserve(bs * sizeof(float))) != OXQ_OK) return st;
+    OXQ_HIP(hipMemcpy(g.s_acts.ptr, block, bb, hipMemcpyHostToDevice));
+    OXQ_HIP(oxq::launch_dequant(type, (const uint8_t *)g.s_acts.ptr, 1, (float *)g.s_out.ptr, nullptr));
+    OXQ_HIP(hipMemcpy(output, g.s_out.ptr, bs * sizeof(float), hipMemcpyDeviceToHost));
+    return OXQ_OK;
+}
+
+int oxq_quantize_f32_to_q8_0(const float *data, size_t n, uint8_t *out, size_t out_len) {
+    if (n % 32 != 0) return fail(OXQ_ERR_DIMENSION_MISMATCH, (n / 32 + 1) * 32, n, "length is not a multiple of 32");
+    const size_t need = n / 32 * 34;
+    if (out_len < need) return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, out_len, "output too small");
+    if (n == 0) return OXQ_OK;
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    std::lock_guard<std::mutex> lock(g.mu);
+    if ((st = g.s_x.reserve(n * sizeof(float))) != OXQ_OK) return st;
+    if ((st = g.s_acts.reserve(need)) != OXQ_OK) return st;
+    OXQ_HIP(hipMemcpy(g.s_x.ptr, data, n * sizeof(float), hipMemcpyHostToDevice));
+    OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, n, (uint8_t *)g.s_acts.ptr, nullptr));
+    OXQ_HIP(hipMemcpy(out, g.s_acts.ptr, need, hipMemcpyDeviceToHost));
+    return OXQ_OK;
+}
+
+int oxq_matvec_q8_fused(uint32_t type, const uint8_t *weights, size_t weights_len, const uint8_t *acts_q8,
+                        size_t acts_len, float *out, size_t out_len, size_t n_rows, size_t n_cols) {
+    FusedShape fs;
+    int st = validate_fused(type, weights_len, acts_len, out_len, n_rows, n_cols, &fs);
+    if (st != OXQ_OK) return st;
+    if (n_rows == 0 || n_cols == 0) return OXQ_OK;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    std::lock_guard<std::mutex> lock(g.mu);
+    const uint8_t *dW = nullptr;
+    if ((st = stage_weights(type, weights, n_rows * fs.row_bytes, &dW)) != OXQ_OK) return st;
+    if ((st = g.s_acts.reserve(fs.acts_needed)) != OXQ_OK) return st;
+    if ((st = g.s_out.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+    OXQ_HIP(hipMemcpy(g.s_acts.ptr, acts_q8, fs.acts_needed, hipMemcpyHostToDevice));
+    OXQ_HIP(hipMemcpy(g.s_out.ptr, out, n_rows * sizeof(float), hipMemcpyHostToDevice));
+    OXQ_HIP(oxq::launch_gemv_q8(type, gemv_args(dW, (const uint8_t *)g.s_acts.ptr, (float *)g.s_out.ptr, nullptr,
+                                                n_rows, n_cols, 1), nullptr));
+    OXQ_HIP(hipMemcpy(out, g.s_out.ptr, n_rows * sizeof(float), hipMemcpyDeviceToHost));
+    return OXQ_OK;
+}
+
+int oxq_block_sums(uint32_t type, const uint8_t *weights, size_t weights_len, const uint8_t *acts_q8,
+                   size_t acts_len, int32_t *sums, size_t sums_len, size_t n_rows, size_t n_cols) {
+    FusedShape fs;
+    int st = validate_fused(type, weights_len, acts_len, n_rows, n_rows, n_cols, &fs);
+    if (st != OXQ_OK) return st;
+    const size_t groups = n_cols / (type == OXQ_TYPE_Q6_K ? 16 : 32);
+    if (sums_len < n_rows * groups) return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * groups, sums_len, "sums buffer too small");
+    if (n_rows == 0 || n_cols == 0) return OXQ_OK;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    std::lock_guard<std::mutex> lock(g.mu);
+    const uint8_t *dW = nullptr;
+    if ((st = stage_weights(type, weights, n_rows * fs.row_bytes, &dW)) != OXQ_OK) return st;
+    if ((st = g.s_acts.reserve(fs.acts_needed)) != OXQ_OK) return st;
+    if ((st = g.s_out.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+    if ((st = g.s_sums.reserve(n_rows * groups * sizeof(int32_t))) != OXQ_OK) return st;
+    OXQ_HIP(hipMemcpy(g.s_acts.ptr, acts_q8, fs.acts_needed, hipMemcpyHostToDevice));
+    OXQ_HIP(oxq::launch_gemv_q8(type, gemv_args(dW, (const uint8_t *)g.s_acts.ptr, (float *)g.s_out.ptr,
+                                                (int32_t *)g.s_sums.ptr, n_rows, n_cols, 0), nullptr));
+    OXQ_HIP(hipMemcpy(sums, g.s_sums.ptr, n_rows * groups * sizeof(int32_t), hipMemcpyDeviceToHost));
+    return OXQ_OK;
+}
+
+int oxq_gemm(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
+             const float *input, size_t input_len, float *output, size_t output_len, size_t m, size_t n, size_t k) {
+    size_t n_rows = 0, n_cols = 0;
+    int st = tensor_dims(type, data_len, shape, n_dims, &n_rows, &n_cols);
+    if (st != OXQ_OK) return st;
+    // The reference slices input[row*k..(row+1)*k] and output[row*n..(row+1)*n] and calls gemv
+    // (reference/q4_k.rs:195-199): a short slice or k < n_cols / n < n_rows is a dimension error.
+    if (input_len < m * k) return fail(OXQ_ERR_DIMENSION_MISMATCH, m * k, input_len, "input shorter than m*k");
+    if (output_len < m * n) return fail(OXQ_ERR_DIMENSION_MISMATCH, m * n, output_len, "output shorter than m*n");
+    if (m == 0) return OXQ_OK;
+    if (k < n_cols) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_cols, k, "k smaller than the tensor's columns");
+    if (n < n_rows) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_rows, n, "n smaller than the tensor's rows");
+    const size_t bs = oxq_block_size(type), bb = oxq_block_bytes(type);
+    const size_t bpr = (n_cols + bs - 1) / bs, row_bytes = bpr * bb;
+    if (data_len < n_rows * row_bytes)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * row_bytes, data_len, "tensor data too small");
+    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
+    if (n_rows == 0 || n_cols == 0) return OXQ_OK;
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull || m > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows, "dimension exceeds 2^32-1");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    std::lock_guard<std::mutex> lock(g.mu);
+    const uint8_t *dW = nullptr;
+    if ((st = stage_weights(type, data, n_rows * row_bytes, &dW)) != OXQ_OK) return st;
+    const size_t act_row_bytes = n_cols / 32 * 34;
+    if ((st = g.s_x.reserve(m * n_cols * sizeof(float))) != OXQ_OK) return st;
+    if ((st = g.s_acts.reserve(m * act_row_bytes)) != OXQ_OK) return st;
+    if ((st = g.s_out.reserve(m * n_rows * sizeof(float))) != OXQ_OK) return st;
+    // Gather the first n_cols floats of each input row (k may exceed n_cols).
+    OXQ_HIP(hipMemcpy2D(g.s_x.ptr, n_cols * sizeof(float), input, k * sizeof(float), n_cols * sizeof(float), m,
+                        hipMemcpyHostToDevice));
+    OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, m * n_cols, (uint8_t *)g.s_acts.ptr, nullptr));
+    oxq::GemmArgs ga;
+    ga.W = dW;
+    ga.A = (const uint8_t *)g.s_acts.ptr;
+    ga.out = (float *)g.s_out.ptr;
+    ga.sums = nullptr;
+    ga.m = (uint32_t)m;
+    ga.n = (uint32_t)n_rows;
+    ga.k = (uint32_t)n_cols;
+    ga.accumulate = 0;
+    OXQ_HIP(oxq::launch_gemm_q8(type, ga, nullptr));
+    OXQ_HIP(hipMemcpy2D(output, n * sizeof(float), g.s_out.ptr, n_rows * sizeof(float), n_rows * sizeof(float), m,
+                        hipMemcpyDeviceToHost));
+    return OXQ_OK;
+}
+
+int oxq_gemv(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
+             const float *input, size_t input_len, float *output, size_t output_len) {
+    size_t n_rows = 0, n_cols = 0;
+    int st = tensor_dims(type, data_len, shape, n_dims, &n_rows, &n_cols);
+    if (st != OXQ_OK) return st;
+    if (input_len < n_cols) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_cols, input_len, "input shorter than n_cols");
+    if (output_len < n_rows) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_rows, output_len, "output shorter than n_rows");
+    const size_t shape2[2] = {n_rows, n_cols};
+    return oxq_gemm(type, data, data_len, shape2, 2, input, n_cols, output, n_rows, 1, n_rows, n_cols);
+}
+
+// ---- weights resident in HBM --------------------------------------------
+
+int oxq_weights_register(uint32_t type, size_t n_rows, size_t n_cols, const uint8_t *bytes, size_t len,
+                         oxq_weights_t *handle) {
+    if (!handle) return fail(OXQ_ERR_INTERNAL, 0, 0, "null handle pointer");
+    *handle = nullptr;
+    if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
+    const size_t bs = oxq_block_size(type), bb = oxq_block_bytes(type);
+    const size_t need = n_rows * ((n_cols + bs - 1) / bs) * bb;
+    if (len < need) return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, len, "weights buffer too small");
+    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    oxq_weights *w = new (std::nothrow) oxq_weights{type, n_rows, n_cols, need, nullptr};
+    if (!w) return fail(OXQ_ERR_INTERNAL, 0, 0, "out of host memory");
+    hipError_t e = hipMalloc((void **)&w->dev, need ? need : 1);
+    if (e == hipSuccess && need) e = hipMemcpy(w->dev, bytes, need, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        if (w->dev) (void)hipFree(w->dev);
+        delete w;
+        return fail_hip(e, "weights upload");
+    }
+    *handle = w;
+    return OXQ_OK;
+}
+
+int oxq_weights_release(oxq_weights_t handle) {
+    if (!handle) return OXQ_OK;
+    if (handle->dev) (void)hipFree(handle->dev);
+    delete handle;
+    return OXQ_OK;
+}
+
+void *oxq_weights_device_ptr(oxq_weights_t handle) { return handle ? handle->dev : nullptr; }
+size_t oxq_weights_nbytes(oxq_weights_t handle) { return handle ? handle->nbytes : 0; }
+
+// ---- device-pointer route -------------------------------------------------
+
+int oxq_quantize_q8_0_dev(const float *d_x, size_t n_total, uint8_t *d_out, void *stream) {
+    if (n_total % 32 != 0)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, (n_total / 32 + 1) * 32, n_total, "length is not a multiple of 32");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_quantize_q8_0(d_x, n_total, d_out, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+static int check_dev_shape(uint32_t type, size_t n_rows, size_t n_cols) {
+    if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
+    const size_t bs = oxq_block_size(type);
+    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows, "dimension exceeds 2^32-1");
+    return OXQ_OK;
+}
+
+int oxq_matvec_q8_fused_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out,
+                            size_t n_rows, size_t n_cols, int accumulate, void *stream) {
+    int st = check_dev_shape(type, n_rows, n_cols);
+    if (st != OXQ_OK) return st;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_gemv_q8(type, gemv_args(d_weights, d_acts_q8, d_out, nullptr, n_rows, n_cols, accumulate ? 1 : 0),
+                                (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, int32_t *d_sums,
+                       size_t n_rows, size_t n_cols, void *stream) {
+    int st = check_dev_shape(type, n_rows, n_cols);
+    if (st != OXQ_OK) return st;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (n_rows == 0 || n_cols == 0) return OXQ_OK;
+    std::lock_guard<std::mutex> lock(g.mu);
+    if ((st = g.s_out.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_gemv_q8(type, gemv_args(d_weights, d_acts_q8, (float *)g.s_out.ptr, d_sums, n_rows, n_cols, 0),
+                                (hipStream_t)stream));
+    OXQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, size_t m,
+                    size_t n, size_t k, int accumulate, void *stream) {
+    int st = check_dev_shape(type, n, k);
+    if (st != OXQ_OK) return st;
+    if (m > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, m, "dimension exceeds 2^32-1");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (m == 0 || n == 0 || k == 0) return OXQ_OK;
+    oxq::GemmArgs ga;
+    ga.W = d_weights;
+    ga.A = d_acts_q8;
+    ga.out = d_out;
+    ga.sums = nullptr;
+    ga.m = (uint32_t)m;
+    ga.n = (uint32_t)n;
+    ga.k = (uint32_t)k;
+    ga.accumulate = accumulate ? 1 : 0;
+    OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+}  // extern "C"

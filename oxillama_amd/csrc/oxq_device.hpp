@@ -1,0 +1,66 @@
+// Device-side helpers shared by the gfx950 kernels: unaligned vector loads of raw
+// GGUF bytes, half -> float, DPP lane exchange and the wave64 sum.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace oxq {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// GGUF blocks are 18/34/136/144/210 bytes: fields sit at 2-byte (or worse)
+// alignment.  gfx950 runs global memory in unaligned-access mode, so a packed
+// wrapper yields one global_load_dwordx{2,4} whatever the address.
+struct __attribute__((packed, aligned(1))) PackedU4 { u32x4 v; };
+struct __attribute__((packed, aligned(1))) PackedU2 { u32x2 v; };
+struct __attribute__((packed, aligned(1))) PackedU1 { uint32_t v; };
+struct __attribute__((packed, aligned(1))) PackedH1 { uint16_t v; };
+
+__device__ __forceinline__ u32x4 ld16(const uint8_t *p) { return reinterpret_cast<const PackedU4 *>(p)->v; }
+__device__ __forceinline__ u32x2 ld8(const uint8_t *p) { return reinterpret_cast<const PackedU2 *>(p)->v; }
+__device__ __forceinline__ uint32_t ld4(const uint8_t *p) { return reinterpret_cast<const PackedU1 *>(p)->v; }
+__device__ __forceinline__ uint32_t ld2(const uint8_t *p) { return reinterpret_cast<const PackedH1 *>(p)->v; }
+
+__device__ __forceinline__ void st2(uint8_t *p, uint32_t v) { reinterpret_cast<PackedH1 *>(p)->v = (uint16_t)v; }
+
+// IEEE binary16 bits -> float (v_cvt_f32_f16; subnormals are kept).
+__device__ __forceinline__ float h2f(uint32_t bits) {
+    return (float)__builtin_bit_cast(_Float16, (uint16_t)bits);
+}
+// float -> binary16 bits, round to nearest even (v_cvt_f16_f32).
+__device__ __forceinline__ uint32_t f2h(float f) {
+    return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
+}
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// DPP controls: quad_perm [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E, row_ror:n = 0x120+n.
+template <int CTRL> __device__ __forceinline__ int dpp_i(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL> __device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, dpp_i<CTRL>(__builtin_bit_cast(int, v)));
+}
+// Value held by lane ^ 1 / lane ^ 2.
+__device__ __forceinline__ int xor1_i(int v) { return dpp_i<0xB1>(v); }
+__device__ __forceinline__ int xor2_i(int v) { return dpp_i<0x4E>(v); }
+
+__device__ __forceinline__ float readlane_f(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
+// Sum over the 64 lanes, same value and same order in every lane: butterflies in
+// each quad, rotations inside each row of 16, then the four row sums.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f<0xB1>(v);
+    v += dpp_f<0x4E>(v);
+    v += dpp_f<0x124>(v);
+    v += dpp_f<0x128>(v);
+    float r0 = readlane_f(v, 0), r1 = readlane_f(v, 16), r2 = readlane_f(v, 32), r3 = readlane_f(v, 48);
+    return (r0 + r1) + (r2 + r3);
+}
+
+}  // namespace oxq

@@ -1,0 +1,40 @@
+// Host-side declarations shared by the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/oxq.h"
+
+namespace oxq {
+
+struct GemvArgs {
+    const uint8_t *W;     // raw GGUF blocks, row-major, device memory
+    const uint8_t *A;     // Q8_0 activation blocks, device memory
+    float *out;           // n_rows floats, device memory
+    int32_t *sums;        // optional: per-row integer group sums (debug), else null
+    uint32_t n_rows;
+    uint32_t n_cols;      // multiple of the format's block size
+    int accumulate;       // 1: out[r] += y (matvec_q8_fused), 0: out[r] = y (gemv)
+    uint32_t waves_per_cu;  // launch width: resident waves per compute unit
+};
+
+// Number of compute units of the current device (cached per device).
+uint32_t device_cus();
+
+hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream);
+
+// x: n floats (n % 32 == 0) -> n/32 Q8_0 blocks of 34 bytes.
+hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *out, hipStream_t stream);
+
+struct GemmArgs {
+    const uint8_t *W;   // raw GGUF blocks [n x k]
+    const uint8_t *A;   // Q8_0 blocks of the m activation rows, row-major, k/32 blocks per row
+    float *out;         // [m x n] row-major
+    int32_t *sums;      // optional debug dump [m][n][k/group]
+    uint32_t m, n, k;
+    int accumulate;
+};
+hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
+
+}  // namespace oxq

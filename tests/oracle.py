@@ -1,0 +1,232 @@
+"""ctypes binding of oracle/liboxq_oracle.so -- the CPU oracle (test infrastructure)."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ORACLE_DIR = os.path.join(ROOT, "oracle")
+LIB_PATH = os.path.join(ORACLE_DIR, "liboxq_oracle.so")
+F16C_PATH = os.path.join(ORACLE_DIR, "liboxq_f16c_check.so")
+
+Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS = 2, 8, 12, 14, 23
+ALL_TYPES = [Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS]
+BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), IQ4_XS: (256, 136)}
+NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS"}
+
+TIER_SCALAR, TIER_AVX2, TIER_Q4_0_STANDALONE = 0, 1, 2
+OK, UNSUPPORTED_TYPE, DIMENSION_MISMATCH, KERNEL_ERROR, BUFFER_TOO_SMALL = 0, 1, 3, 4, 6
+
+
+class Status(C.Structure):
+    _fields_ = [("code", C.c_int), ("a", C.c_size_t), ("b", C.c_size_t)]
+
+
+class OracleError(Exception):
+    def __init__(self, st):
+        super().__init__(f"oracle status {st.code} ({st.a}, {st.b})")
+        self.code, self.a, self.b = st.code, st.a, st.b
+
+
+_lib = None
+
+
+def build():
+    subprocess.run(["make", "-C", ORACLE_DIR, "-s", "liboxq_oracle.so", "liboxq_f16c_check.so"], check=True)
+
+
+def load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        build()
+    lib = C.CDLL(LIB_PATH)
+    vp, sz, u32 = C.c_void_p, C.c_size_t, C.c_uint32
+    lib.oxq_ref_block_size.restype = sz
+    lib.oxq_ref_block_size.argtypes = [u32]
+    lib.oxq_ref_block_bytes.restype = sz
+    lib.oxq_ref_block_bytes.argtypes = [u32]
+    lib.oxq_ref_f32_to_f16.restype = C.c_uint16
+    lib.oxq_ref_f32_to_f16.argtypes = [C.c_float]
+    lib.oxq_ref_f16_to_f32.restype = C.c_float
+    lib.oxq_ref_f16_to_f32.argtypes = [C.c_uint16]
+    for name, args in {
+        "oxq_ref_quantize_f32_to_q8_0": [vp, sz, vp],
+        "oxq_ref_quantize_f32_to_q4_0": [vp, sz, vp],
+        "oxq_ref_dequant_block": [u32, vp, sz, vp, sz],
+        "oxq_ref_gemv": [u32, vp, sz, sz, sz, vp, sz, vp, sz],
+        "oxq_ref_gemm": [u32, vp, sz, vp, vp, sz, sz, sz],
+        "oxq_ref_matvec_q8_fused": [u32, C.c_int, vp, sz, vp, sz, vp, sz, sz, sz],
+        "oxq_ref_matvec_q8_intdot": [u32, vp, sz, vp, sz, vp, sz, sz, sz],
+        "oxq_ref_block_sums": [u32, vp, sz, vp, sz, vp, sz, sz],
+        "oxq_ref_gemm_q8": [u32, C.c_int, vp, sz, vp, vp, sz, sz, sz],
+        "oxq_ref_matvec_q8_fused_mt": [u32, C.c_int, vp, sz, vp, sz, vp, sz, sz, sz, C.c_int],
+    }.items():
+        fn = getattr(lib, name)
+        fn.restype = Status
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _chk(st):
+    if st.code != OK:
+        raise OracleError(st)
+
+
+def _u8(a):
+    return np.ascontiguousarray(a).view(np.uint8).ravel()
+
+
+def groups_per_row(t, n_cols):
+    return n_cols // (16 if t == Q6_K else 32)
+
+
+def row_bytes(t, n_cols):
+    bs, bb = BLOCK[t]
+    return -(-n_cols // bs) * bb
+
+
+def f32_to_f16(v):
+    return load().oxq_ref_f32_to_f16(float(v))
+
+
+def f16_to_f32(h):
+    return load().oxq_ref_f16_to_f32(int(h))
+
+
+def quantize_q8_0(x):
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.zeros(x.size // 32 * 34 + 34, dtype=np.uint8)
+    _chk(load().oxq_ref_quantize_f32_to_q8_0(_p(x), x.size, _p(out)))
+    return out[: x.size // 32 * 34]
+
+
+def quantize_q4_0(x):
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.zeros(x.size // 32 * 18 + 18, dtype=np.uint8)
+    _chk(load().oxq_ref_quantize_f32_to_q4_0(_p(x), x.size, _p(out)))
+    return out[: x.size // 32 * 18]
+
+
+def dequant_block(t, block, out_len=None):
+    block = _u8(block)
+    n = BLOCK[t][0] if out_len is None else out_len
+    out = np.zeros(max(n, 1), dtype=np.float32)
+    _chk(load().oxq_ref_dequant_block(t, _p(block), block.size, _p(out), n))
+    return out[:n]
+
+
+def dequant_rows(t, w, n_rows, n_cols):
+    """Dequantize a whole matrix with dequant_block, block by block."""
+    w = _u8(w)
+    bs, bb = BLOCK[t]
+    bpr = n_cols // bs
+    out = np.zeros((n_rows, n_cols), dtype=np.float32)
+    for r in range(n_rows):
+        for b in range(bpr):
+            off = (r * bpr + b) * bb
+            out[r, b * bs:(b + 1) * bs] = dequant_block(t, w[off:off + bb])
+    return out
+
+
+def gemv(t, w, n_rows, n_cols, x, y_len=None, x_len=None):
+    w = _u8(w)
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    y = np.zeros(max(n_rows if y_len is None else y_len, 1), dtype=np.float32)
+    _chk(load().oxq_ref_gemv(t, _p(w), w.size, n_rows, n_cols, _p(x), x.size if x_len is None else x_len,
+                             _p(y), n_rows if y_len is None else y_len))
+    return y[:n_rows]
+
+
+def gemm(t, w, x, m, n, k):
+    w = _u8(w)
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    y = np.zeros(m * n, dtype=np.float32)
+    _chk(load().oxq_ref_gemm(t, _p(w), w.size, _p(x), _p(y), m, n, k))
+    return y.reshape(m, n)
+
+
+def matvec_q8_fused(t, w, acts, n_rows, n_cols, tier=TIER_AVX2, out=None, out_len=None):
+    w, acts = _u8(w), _u8(acts)
+    if out is None:
+        out = np.zeros(max(n_rows, 1), dtype=np.float32)
+    _chk(load().oxq_ref_matvec_q8_fused(t, tier, _p(w), w.size, _p(acts), acts.size, _p(out),
+                                        out.size if out_len is None else out_len, n_rows, n_cols))
+    return out[:n_rows]
+
+
+def matvec_q8_intdot(t, w, acts, n_rows, n_cols):
+    w, acts = _u8(w), _u8(acts)
+    out = np.zeros(max(n_rows, 1), dtype=np.float32)
+    _chk(load().oxq_ref_matvec_q8_intdot(t, _p(w), w.size, _p(acts), acts.size, _p(out), out.size,
+                                         n_rows, n_cols))
+    return out[:n_rows]
+
+
+def matvec_q8_fused_mt(t, w, acts, n_rows, n_cols, threads, tier=TIER_AVX2):
+    w, acts = _u8(w), _u8(acts)
+    out = np.zeros(max(n_rows, 1), dtype=np.float32)
+    _chk(load().oxq_ref_matvec_q8_fused_mt(t, tier, _p(w), w.size, _p(acts), acts.size, _p(out), out.size,
+                                           n_rows, n_cols, threads))
+    return out[:n_rows]
+
+
+def block_sums(t, w, acts, n_rows, n_cols):
+    w, acts = _u8(w), _u8(acts)
+    g = groups_per_row(t, n_cols)
+    sums = np.zeros(n_rows * g, dtype=np.int32)
+    _chk(load().oxq_ref_block_sums(t, _p(w), w.size, _p(acts), acts.size, _p(sums), n_rows, n_cols))
+    return sums.reshape(n_rows, g)
+
+
+def gemm_q8(t, w, x, m, n, k, tier=TIER_AVX2):
+    w = _u8(w)
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    y = np.zeros(m * n, dtype=np.float32)
+    _chk(load().oxq_ref_gemm_q8(t, tier, _p(w), w.size, _p(x), _p(y), m, n, k))
+    return y.reshape(m, n)
+
+
+# ---- block builders mirroring the reference tests' make_*_block helpers ----
+
+def f16_bytes(v):
+    h = f32_to_f16(v)
+    return bytes([h & 0xFF, h >> 8])
+
+
+def make_q4_0_block(scale, nibbles):  # Q/reference/q4_0.rs:238-244
+    assert len(nibbles) == 16
+    return f16_bytes(scale) + bytes(nibbles)
+
+
+def make_q8_0_block(scale, qs):  # Q/reference/q8_0.rs:137-145
+    assert len(qs) == 32
+    return f16_bytes(scale) + bytes((q & 0xFF) for q in qs)
+
+
+def make_q4_k_block(d, dmin, scales, qs):  # Q/reference/q4_k.rs:359-366
+    assert len(scales) == 12 and len(qs) == 128
+    return f16_bytes(d) + f16_bytes(dmin) + bytes(scales) + bytes(qs)
+
+
+def make_q6k_block(d, ql, qh, scales):  # Q/simd/avx2/q6_k.rs make_q6k_block
+    assert len(ql) == 128 and len(qh) == 64 and len(scales) == 16
+    return bytes(ql) + bytes(qh) + bytes((s & 0xFF) for s in scales) + f16_bytes(d)
+
+
+def make_iq4_xs_block(scale, sub_scales, nibbles):  # Q/reference/iq4_xs.rs:211-249
+    assert len(sub_scales) == 8 and len(nibbles) == 128
+    scales_h, scales_l = 0, [0, 0, 0, 0]
+    for i, v in enumerate(sub_scales):
+        v &= 0x3F
+        low, high = v & 0x0F, (v >> 4) & 0x03
+        scales_l[i // 2] |= low if i % 2 == 0 else (low << 4)
+        scales_h |= high << (2 * i)
+    return f16_bytes(scale) + bytes([scales_h & 0xFF, scales_h >> 8]) + bytes(scales_l) + bytes(nibbles)

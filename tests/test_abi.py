@@ -1,0 +1,106 @@
+"""The C-ABI library loads and exports every symbol include/oxq.h declares, and the
+checks that precede any GPU work behave as the reference's do.  CPU only: no entry
+point that would touch a device is called with valid arguments here."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+from oxillama_amd import capi, quant
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "oxq.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(oxq_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_and_binding_list_the_same_symbols():
+    assert declared_symbols() == sorted(capi.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = C.CDLL(capi.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_format_metadata_matches_reference_tables():
+    # crates/oxillama-gguf/src/types.rs:199-262
+    lib = capi.load()
+    table = {2: (32, 18, b"Q4_0"), 8: (32, 34, b"Q8_0"), 12: (256, 144, b"Q4_K"), 14: (256, 210, b"Q6_K"),
+             23: (256, 136, b"IQ4_XS")}
+    for t, (bs, bb, name) in table.items():
+        assert lib.oxq_block_size(t) == bs and lib.oxq_block_bytes(t) == bb and lib.oxq_type_name(t) == name
+        assert lib.oxq_get_kernel(t) == capi.OK
+    for t in (0, 1, 3, 13, 15, 39):  # formats this library has no kernel for
+        assert lib.oxq_block_size(t) == 0 and lib.oxq_type_name(t) is None
+        assert lib.oxq_get_kernel(t) == capi.ERR_UNSUPPORTED_TYPE
+    with pytest.raises(quant.UnsupportedType):
+        quant.KernelDispatcher().get_kernel(13)
+
+
+def test_status_names_follow_quant_error_variants():
+    lib = capi.load()
+    names = [lib.oxq_status_name(i).decode() for i in range(10)]
+    assert names == ["Ok", "UnsupportedType", "BlockSizeMismatch", "DimensionMismatch", "KernelError",
+                     "BlockCountMismatch", "BufferTooSmall", "Internal", "UnsupportedShape", "NoDevice"]
+
+
+def test_quantize_rejects_unaligned_length_before_touching_the_gpu():
+    # Q/quantize.rs:59-64
+    with pytest.raises(quant.DimensionMismatch) as e:
+        quant.quantize_f32_to_q8_0(np.zeros(31, dtype=np.float32))
+    assert (e.value.expected, e.value.got) == (32, 31)
+
+
+@pytest.mark.parametrize("t", [2, 8, 12, 14, 23])
+def test_fused_validation_order_before_touching_the_gpu(t):
+    # Q/reference/q4_k.rs:226-250: out, then weights, then activations
+    k = quant.HipKernel(t)
+    bs, bb = k.block_size(), k.block_bytes()
+    n_rows, n_cols = 3, 2 * bs
+    w = np.zeros(n_rows * 2 * bb, dtype=np.uint8)
+    acts_needed = 2 * (bs // 32) * 34
+    a = np.zeros(acts_needed, dtype=np.uint8)
+    with pytest.raises(quant.DimensionMismatch) as e:
+        k.matvec_q8_fused(w[:-1], a[:-1], np.zeros(2, dtype=np.float32), n_rows, n_cols)
+    assert (e.value.expected, e.value.got) == (3, 2)
+    with pytest.raises(quant.BufferTooSmall) as e:
+        k.matvec_q8_fused(w[:-1], a[:-1], np.zeros(3, dtype=np.float32), n_rows, n_cols)
+    assert (e.value.needed, e.value.available) == (w.size, w.size - 1)
+    with pytest.raises(quant.BufferTooSmall) as e:
+        k.matvec_q8_fused(w, a[:-1], np.zeros(3, dtype=np.float32), n_rows, n_cols)
+    assert (e.value.needed, e.value.available) == (acts_needed, acts_needed - 1)
+    with pytest.raises(quant.UnsupportedShape):  # partial blocks: the shim falls back to the CPU kernel
+        k.matvec_q8_fused(w, a, np.zeros(3, dtype=np.float32), n_rows, n_cols - 1)
+
+
+@pytest.mark.parametrize("t", [2, 8, 12, 14, 23])
+def test_dequant_and_gemv_argument_errors(t):
+    k = quant.HipKernel(t)
+    bs, bb = k.block_size(), k.block_bytes()
+    with pytest.raises(quant.BufferTooSmall) as e:  # e.g. Q/reference/q4_0.rs:348-355
+        k.dequant_block(np.zeros(4, dtype=np.uint8), np.zeros(bs, dtype=np.float32))
+    assert (e.value.needed, e.value.available) == (bb, 4)
+    with pytest.raises(quant.BufferTooSmall) as e:  # Q/reference/q4_0.rs:358-366
+        k.dequant_block(np.zeros(bb, dtype=np.uint8), np.zeros(1, dtype=np.float32))
+    assert (e.value.needed, e.value.available) == (bs, 1)
+    tensor = quant.QuantTensor(np.zeros(2 * bb, dtype=np.uint8), [2, bs], t)
+    with pytest.raises(quant.DimensionMismatch) as e:  # Q/reference/q4_0.rs:311-321
+        k.gemv(tensor, np.zeros(4, dtype=np.float32), np.zeros(2, dtype=np.float32))
+    assert (e.value.expected, e.value.got) == (bs, 4)
+    with pytest.raises(quant.DimensionMismatch) as e:  # Q/reference/q4_0.rs:324-337
+        k.gemv(tensor, np.zeros(bs, dtype=np.float32), np.zeros(1, dtype=np.float32))
+    assert (e.value.expected, e.value.got) == (2, 1)
+
+
+def test_quant_tensor_bookkeeping():
+    # Q/types.rs:31-50
+    t = quant.QuantTensor(np.zeros(144 * 6, dtype=np.uint8), [3, 512], 12)
+    assert t.n_elements() == 1536 and t.n_blocks() == 6 and t.expected_data_size() == 864
+    assert quant.QuantTensor(b"", [], 12).n_elements() == 0

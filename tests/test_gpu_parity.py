@@ -1,0 +1,325 @@
+"""Parity of the HIP path (through the C ABI) against the CPU oracle on identical
+seeded inputs.  Bars: Q8_0 activation bytes and integer group sums bit-exact; fp32
+outputs within 1e-5 * |y_ref|_inf (block-accumulation order differs)."""
+import sys
+
+import numpy as np
+import pytest
+
+import fixtures as FX
+import oracle as O
+from oxillama_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+FP32_REL_TOL = 1e-5  # max|y - y_ref| <= 1e-5 * max|y_ref|
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def assert_close(y, y_ref, what):
+    scale = float(np.abs(y_ref).max())
+    err = float(np.abs(y.astype(np.float64) - y_ref.astype(np.float64)).max())
+    assert err <= FP32_REL_TOL * scale + 1e-30, f"{what}: max err {err:.3e} > 1e-5 * {scale:.3e}"
+
+
+def canonical_ref(ref, t, w, a, n_rows, n_cols, threads=8):
+    """Reference-order result the GPU is held to: the AVX2 tier for Q4_0/Q8_0/Q4_K, the
+    (scalar-bodied) fused kernel for Q6_K, the integer form for IQ4_XS."""
+    return ref.matvec_q8_fused_mt(t, w, a, n_rows, n_cols, threads, tier=O.TIER_AVX2)
+
+
+# ---- (1) Q8_0 activation quantizer -----------------------------------------------------
+
+def test_quantize_q8_0_bit_exact_random(hip, ref):
+    for seed, n, sigma in ((1, 4096, 1.0), (2, 14336, 1.0), (3, 32, 1.0), (4, 64 * 4096, 3.0), (5, 4096, 1e-4)):
+        x = synth.normal_f32(seed, n, sigma)
+        say("quantize seed", seed, "n", n)
+        assert np.array_equal(hip.quantize_f32_to_q8_0(x), ref.quantize_q8_0(x))
+
+
+def test_quantize_q8_0_bit_exact_edge_cases(hip, ref):
+    rng = np.random.default_rng(7)
+    blocks = []
+    blocks.append(np.zeros(32, dtype=np.float32))                                   # d = 0
+    b = np.zeros(32, dtype=np.float32); b[:8] = [127, .5, 1.5, 2.5, -.5, -1.5, -2.5, 3.49]; blocks.append(b)
+    b = np.zeros(32, dtype=np.float32); b[0] = 1000; b[1] = -1000; b[31] = 500; blocks.append(b)  # quantize.rs:425
+    blocks.append(np.full(32, -0.0, dtype=np.float32))
+    blocks.append((np.arange(32, dtype=np.float32) / np.float32(15.5)) - 1)        # quantize.rs:263
+    blocks.append(np.full(32, 1e-30, dtype=np.float32))                            # d underflows f16
+    blocks.append(np.full(32, 6e-6, dtype=np.float32))                             # d subnormal in f16
+    blocks.append((rng.standard_normal(32) * 1e4).astype(np.float32))
+    blocks.append((rng.standard_normal(32) * 6e6).astype(np.float32))              # d overflows f16 -> inf
+    b = rng.standard_normal(32).astype(np.float32); b[5] = np.float32(3.0e38); blocks.append(b)
+    for k in range(40):                                                            # exact .5 ties after scaling
+        b = (rng.integers(-254, 255, size=32) * 0.5).astype(np.float32); b[0] = 127.0; blocks.append(b)
+    x = np.concatenate(blocks)
+    got, want = hip.quantize_f32_to_q8_0(x), ref.quantize_q8_0(x)
+    bad = np.nonzero(got != want)[0]
+    assert bad.size == 0, f"first mismatch at byte {bad[:5]} (block {bad[:5] // 34})"
+    assert hip.quantize_f32_to_q8_0(np.zeros(0, dtype=np.float32)).size == 0       # quantize.rs:432
+
+
+# ---- (2) dequant_block -------------------------------------------------------------------
+
+@pytest.mark.parametrize("case", FX.dequant_cases(), ids=lambda c: c[0])
+def test_dequant_block_known_answers(hip, ref, case):
+    _, t, block, expected, tol = case
+    out = np.zeros(O.BLOCK[t][0], dtype=np.float32)
+    hip.HipKernel(t).dequant_block(block, out)
+    for i, v in expected.items():
+        assert abs(out[i] - v) <= tol
+    assert np.array_equal(out, ref.dequant_block(t, block))
+
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_dequant_block_bit_exact_random(hip, ref, t):
+    bs, bb = O.BLOCK[t]
+    w = synth.weights(t, 100 + t, 8, bs)
+    k = hip.HipKernel(t)
+    for i in range(8):
+        out = np.zeros(bs, dtype=np.float32)
+        k.dequant_block(w[i * bb:(i + 1) * bb], out)
+        assert np.array_equal(out, ref.dequant_block(t, w[i * bb:(i + 1) * bb]))
+
+
+# ---- (3) fused matvec: the reference's own fixtures ------------------------------------------
+
+@pytest.mark.parametrize("case", FX.fused_cases(), ids=lambda c: c[0])
+def test_fused_reference_fixtures(hip, ref, case):
+    name, t, w, a, n_rows, n_cols, tol = case
+    say("fixture", name)
+    out = np.zeros(n_rows, dtype=np.float32)
+    hip.HipKernel(t).matvec_q8_fused(w, a, out, n_rows, n_cols)
+    for tier in (O.TIER_SCALAR, O.TIER_AVX2):
+        assert np.abs(out - ref.matvec_q8_fused(t, w, a, n_rows, n_cols, tier=tier)).max() < tol
+    assert np.array_equal(hip.HipKernel(t).block_sums(w, a, n_rows, n_cols), ref.block_sums(t, w, a, n_rows, n_cols))
+
+
+@pytest.mark.parametrize("case", FX.accumulate_cases(), ids=lambda c: c[0])
+def test_fused_accumulate_semantics(hip, case):
+    _, t, w, a, n_cols, preset = case
+    out = np.full(1, preset, dtype=np.float32)
+    hip.HipKernel(t).matvec_q8_fused(w, a, out, 1, n_cols)
+    assert out[0] == preset
+
+
+def test_fused_zero_activations(hip):
+    w = np.frombuffer(O.make_q4_k_block(1.0, 0.0, FX.Q4K_SCALES_ONES, [0x88] * 128), dtype=np.uint8)
+    a = np.frombuffer(O.make_q8_0_block(1.0, [0] * 32) * 8, dtype=np.uint8)
+    out = np.zeros(1, dtype=np.float32)
+    hip.HipKernel(O.Q4_K).matvec_q8_fused(w, a, out, 1, 256)
+    assert out[0] == 0.0
+
+
+# ---- (4) seeded random shapes: every launch variant -------------------------------------------
+
+def _shapes(t):
+    """n_cols covering 1..8 cached steps, ragged last steps and the uncached path."""
+    unit = 64 if t == O.Q6_K else 32
+    bs = O.BLOCK[t][0]
+    cols = set()
+    for units in (1, 8, 63, 64, 65, 128, 130, 192, 250, 256, 300, 448, 512, 520, 1100):
+        c = units * unit
+        c = -(-c // bs) * bs
+        cols.add(c)
+    return sorted(cols)
+
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_fused_random_shapes(hip, ref, t):
+    k = hip.HipKernel(t)
+    for i, n_cols in enumerate(_shapes(t)):
+        n_rows = (1, 3, 4, 5, 257, 64, 7)[i % 7]
+        say(O.NAMES[t], "n_rows", n_rows, "n_cols", n_cols)
+        w = synth.weights(t, 1000 + i, n_rows, n_cols)
+        a = ref.quantize_q8_0(synth.normal_f32(2000 + i, n_cols))
+        preset = synth.normal_f32(3000 + i, n_rows)
+        out = preset.copy()
+        k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+        y_ref = canonical_ref(ref, t, w, a, n_rows, n_cols)
+        assert_close(out - preset, y_ref, f"{O.NAMES[t]} {n_rows}x{n_cols}")
+        assert np.array_equal(k.block_sums(w, a, n_rows, n_cols), ref.block_sums(t, w, a, n_rows, n_cols))
+
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_fused_extreme_bytes(hip, ref, t):
+    """Uniformly random block payloads (all nibble / 6-bit / int8 codes, extreme scales kept finite)
+    against saturated activations: integer sums must still be exact."""
+    rng = np.random.default_rng(900 + t)
+    bs, bb = O.BLOCK[t]
+    n_rows, n_cols = 9, 8 * 256
+    w = rng.integers(0, 256, size=n_rows * (n_cols // bs) * bb, dtype=np.uint8).reshape(-1, bb)
+    one = np.frombuffer(O.f16_bytes(0.0078125), dtype=np.uint8)
+    if t == O.Q6_K:
+        w[:, 208:210] = one
+    else:
+        w[:, 0:2] = one
+    if t == O.Q4_K:
+        w[:, 2:4] = one
+    w = w.ravel()
+    q = rng.choice(np.array([-128, -127, 127, 0, 1, -1], dtype=np.int8), size=n_cols)
+    a = np.concatenate([np.frombuffer(O.make_q8_0_block(0.5, [int(v) for v in q[i:i + 32]]), dtype=np.uint8)
+                        for i in range(0, n_cols, 32)])
+    k = hip.HipKernel(t)
+    assert np.array_equal(k.block_sums(w, a, n_rows, n_cols), ref.block_sums(t, w, a, n_rows, n_cols))
+    out = np.zeros(n_rows, dtype=np.float32)
+    k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+    assert_close(out, canonical_ref(ref, t, w, a, n_rows, n_cols), O.NAMES[t])
+
+
+def test_empty_inputs(hip):
+    for t in O.ALL_TYPES:
+        k = hip.HipKernel(t)
+        out = np.full(2, 3.0, dtype=np.float32)
+        k.matvec_q8_fused(np.zeros(0, dtype=np.uint8), np.zeros(0, dtype=np.uint8), out, 0, 0)
+        assert (out == 3.0).all()
+
+
+# ---- (5) the benchmark configurations at full size ---------------------------------------------
+
+CONFIGS = [
+    ("C1 Q4_0 4096x4096", O.Q4_0, 4096, 4096),
+    ("C2 q_proj Q8_0 4096x4096", O.Q8_0, 4096, 4096),
+    ("C2 ffn_gate Q4_K 14336x4096", O.Q4_K, 14336, 4096),
+    ("C2 ffn_down Q6_K 4096x14336", O.Q6_K, 4096, 14336),
+    ("C5 expert gate IQ4_XS 14336x4096", O.IQ4_XS, 14336, 4096),
+    ("C5 expert down IQ4_XS 4096x14336", O.IQ4_XS, 4096, 14336),
+]
+
+
+@pytest.mark.parametrize("cfg", CONFIGS, ids=lambda c: c[0])
+def test_full_size_configs(hip, ref, cfg):
+    import torch
+    name, t, n_rows, n_cols = cfg
+    say(name)
+    w = synth.weights(t, 11, n_rows, n_cols)
+    x = synth.normal_f32(12, n_cols)
+    a_ref = ref.quantize_q8_0(x)
+    dw = torch.from_numpy(w).cuda()
+    dx = torch.from_numpy(x).cuda()
+    da = torch.empty(a_ref.size, dtype=torch.uint8, device="cuda")
+    hip.quantize_q8_0_dev(dx, da)
+    assert np.array_equal(da.cpu().numpy(), a_ref)                      # activation bytes bit-exact
+    k = hip.HipKernel(t)
+    dy = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+    k.matvec_q8_fused_dev(dw, da, dy, n_rows, n_cols, accumulate=True)
+    sums = torch.empty((n_rows, O.groups_per_row(t, n_cols)), dtype=torch.int32, device="cuda")
+    k.block_sums_dev(dw, da, sums, n_rows, n_cols)
+    torch.cuda.synchronize()
+    y_ref = canonical_ref(ref, t, w, a_ref, n_rows, n_cols)
+    assert_close(dy.cpu().numpy(), y_ref, name)
+    assert np.array_equal(sums.cpu().numpy(), ref.block_sums(t, w, a_ref, n_rows, n_cols))
+    # linearity in the accumulator: a second call adds the same vector again
+    k.matvec_q8_fused_dev(dw, da, dy, n_rows, n_cols, accumulate=True)
+    torch.cuda.synchronize()
+    assert_close(dy.cpu().numpy(), 2 * y_ref, name + " (accumulated twice)")
+
+
+def test_lm_head_full_size(hip, ref):
+    """C3: 128256 x 4096 Q6_K, the largest matrix.  Oracle on every row (threaded row split)."""
+    import torch
+    n_rows, n_cols, t = 128256, 4096, O.Q6_K
+    say("C3 lm_head: generating")
+    w = synth.weights(t, 21, n_rows, n_cols)
+    a = ref.quantize_q8_0(synth.normal_f32(22, n_cols))
+    dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(a).cuda()
+    dy = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+    hip.HipKernel(t).matvec_q8_fused_dev(dw, da, dy, n_rows, n_cols, accumulate=False)
+    torch.cuda.synchronize()
+    say("C3 lm_head: oracle")
+    y_ref = canonical_ref(ref, t, w, a, n_rows, n_cols, threads=16)
+    assert_close(dy.cpu().numpy(), y_ref, "lm_head")
+    # row-permutation equivariance on the device copy: rows are independent
+    perm = torch.randperm(n_rows, generator=torch.Generator().manual_seed(5))
+    rb = O.row_bytes(t, n_cols)
+    dwp = dw.view(n_rows, rb)[perm.cuda()].contiguous()
+    dyp = torch.zeros_like(dy)
+    hip.HipKernel(t).matvec_q8_fused_dev(dwp, da, dyp, n_rows, n_cols, accumulate=False)
+    torch.cuda.synchronize()
+    assert torch.equal(dyp, dy[perm.cuda()])
+
+
+# ---- (6) gemv / gemm on host slices ---------------------------------------------------------
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_gemv_is_quantize_plus_fused(hip, ref, t):
+    n_rows, n_cols = 33, 1024
+    w = synth.weights(t, 301, n_rows, n_cols)
+    x = synth.normal_f32(302, n_cols)
+    k = hip.HipKernel(t)
+    y = np.full(n_rows, 9.0, dtype=np.float32)  # overwritten, not accumulated (Q/traits.rs:39)
+    k.gemv(hip.QuantTensor(w, [n_rows, n_cols], t), x, y)
+    y_ref = canonical_ref(ref, t, w, ref.quantize_q8_0(x), n_rows, n_cols)
+    assert_close(y, y_ref, "gemv")
+    # and close to the reference's f32-activation gemv up to the Q8_0 rounding of x
+    y_f32 = ref.gemv(t, w, n_rows, n_cols, x)
+    assert np.abs(y - y_f32).max() < 0.02 * np.abs(y_f32).max()
+
+
+def test_gemv_known_answers(hip):
+    # Q/reference/q4_k.rs:411-436 (256) and Q/reference/q8_0.rs:175-190 (6.0): exact even after Q8_0
+    w = np.frombuffer(O.make_q4_k_block(1.0, 0.0, FX.Q4K_SCALES_ONES, [0x11] * 128), dtype=np.uint8)
+    y = np.zeros(1, dtype=np.float32)
+    hip.HipKernel(O.Q4_K).gemv(hip.QuantTensor(w, [1, 256], O.Q4_K), np.ones(256, dtype=np.float32), y)
+    assert abs(y[0] - 256.0) < 1.0
+    q = [0] * 32
+    q[0] = 1
+    x = np.zeros(32, dtype=np.float32)
+    x[0] = 3.0
+    w = np.frombuffer(O.make_q8_0_block(2.0, q), dtype=np.uint8)
+    hip.HipKernel(O.Q8_0).gemv(hip.QuantTensor(w, [1, 32], O.Q8_0), x, y)
+    assert abs(y[0] - 6.0) < 0.1
+
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_gemm_matches_oracle(hip, ref, t):
+    m, n, k_ = 5, 40, 768
+    w = synth.weights(t, 401, n, k_)
+    x = synth.normal_f32(402, m * k_).reshape(m, k_)
+    y = np.zeros((m, n), dtype=np.float32)
+    hip.HipKernel(t).gemm(hip.QuantTensor(w, [n, k_], t), x, y, m, n, k_)
+    assert_close(y, ref.gemm_q8(t, w, x, m, n, k_), "gemm")
+
+
+# ---- (7) residency helpers -----------------------------------------------------------------
+
+def test_registered_weights_and_cache(hip, ref):
+    import ctypes as C
+    from oxillama_amd import capi
+    lib = capi.load()
+    t, n_rows, n_cols = O.Q4_K, 64, 1024
+    w = synth.weights(t, 501, n_rows, n_cols)
+    a = ref.quantize_q8_0(synth.normal_f32(502, n_cols))
+    h = C.c_void_p()
+    assert lib.oxq_weights_register(t, n_rows, n_cols, w.ctypes.data, w.size, C.byref(h)) == capi.OK
+    assert lib.oxq_weights_nbytes(h) == w.size
+    import torch
+    da = torch.from_numpy(a).cuda()
+    dy = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+    st = lib.oxq_matvec_q8_fused_dev(t, lib.oxq_weights_device_ptr(h), da.data_ptr(), dy.data_ptr(), n_rows, n_cols,
+                                     0, None)
+    assert st == capi.OK
+    torch.cuda.synchronize()
+    y_ref = canonical_ref(ref, t, w, a, n_rows, n_cols)
+    assert_close(dy.cpu().numpy(), y_ref, "registered")
+    assert lib.oxq_weights_release(h) == capi.OK
+    # host-slice route with the cache on: same answer, and a changed buffer is noticed
+    lib.oxq_weight_cache_enable(1)
+    try:
+        k = hip.HipKernel(t)
+        for _ in range(2):
+            out = np.zeros(n_rows, dtype=np.float32)
+            k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+            assert_close(out, y_ref, "cached")
+        w2 = synth.weights(t, 503, n_rows, n_cols)
+        w[:] = w2
+        out = np.zeros(n_rows, dtype=np.float32)
+        k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+        assert_close(out, canonical_ref(ref, t, w2, a, n_rows, n_cols), "cache refreshed")
+    finally:
+        lib.oxq_weight_cache_enable(0)
+        lib.oxq_weight_cache_clear()
