@@ -225,13 +225,20 @@ def main():
               "up": layers[0]["up"].cpu().numpy(), "down": layers[0]["down"].cpu().numpy()}
         hx, hh = x.cpu().numpy(), h.cpu().numpy()
 
+        avx2 = O.load_avx2() is not None
+
+        def fused(t, w, a, n_rows, n_cols, threads):
+            if avx2:
+                return O.avx2_matvec_q8_fused(t, w, a, n_rows, n_cols, threads)
+            return O.matvec_q8_fused_mt(t, w, a, n_rows, n_cols, threads)
+
         def cpu_step(threads):
             a = O.quantize_q8_0(hx)
-            O.matvec_q8_fused_mt(O.Q8_0, hw["q"], a, H, H, threads)
-            O.matvec_q8_fused_mt(O.Q4_K, hw["gate"], a, F, H, threads)
-            O.matvec_q8_fused_mt(O.Q4_K, hw["up"], a, F, H, threads)
+            fused(O.Q8_0, hw["q"], a, H, H, threads)
+            fused(O.Q4_K, hw["gate"], a, F, H, threads)
+            fused(O.Q4_K, hw["up"], a, F, H, threads)
             b = O.quantize_q8_0(hh)
-            O.matvec_q8_fused_mt(O.Q6_K, hw["down"], b, H, F, threads)
+            fused(O.Q6_K, hw["down"], b, H, F, threads)
 
         def time_cpu(threads, budget_s):
             cpu_step(threads)
@@ -247,7 +254,8 @@ def main():
         s_1t, n_1t = time_cpu(1, 8.0)
         cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                "sample": f"one layer (same 4 matrices + 2 quantizations), {n_mt} repeats, static row split over "
-                         f"{cores} threads; C restatement of the reference's AVX2-tier fused rows (scalar code)",
+                         f"{cores} threads; " + ("AVX2 intrinsics twin of the reference's fused rows (Q6_K body is scalar "
+                         "there too)" if avx2 else "scalar C restatement of the reference's AVX2-tier fused rows"),
                "ms_per_step": round(s_mt * 1e3, 3),
                "single_thread": {"value": round(step_weight_bytes / s_1t / 1e9, 3), "ms_per_step": round(s_1t * 1e3, 3),
                                  "repeats": n_1t}}

@@ -22,7 +22,10 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (valid) {
         const u32x4 raw = ld16(reinterpret_cast<const uint8_t *>(x + blk * 32 + 4 * j));
-        for (int i = 0; i < 4; i++) v[i] = __builtin_bit_cast(float, raw[i]);
+        for (int i = 0; i < 4; i++) {
+            const uint32_t bits = raw[i];  // copy out first: bit_cast must not see the vector element lvalue
+            v[i] = __builtin_bit_cast(float, bits);
+        }
     }
     float m = 0.0f;
     for (int i = 0; i < 4; i++) m = fmaxf(m, fabsf(v[i]));

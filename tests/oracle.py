@@ -9,6 +9,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ORACLE_DIR = os.path.join(ROOT, "oracle")
 LIB_PATH = os.path.join(ORACLE_DIR, "liboxq_oracle.so")
 F16C_PATH = os.path.join(ORACLE_DIR, "liboxq_f16c_check.so")
+AVX2_PATH = os.path.join(ORACLE_DIR, "liboxq_cpu_avx2.so")
 
 Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS = 2, 8, 12, 14, 23
 ALL_TYPES = [Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS]
@@ -34,6 +35,46 @@ _lib = None
 
 def build():
     subprocess.run(["make", "-C", ORACLE_DIR, "-s", "liboxq_oracle.so", "liboxq_f16c_check.so"], check=True)
+
+
+def host_has(flag):
+    try:
+        with open("/proc/cpuinfo") as f:
+            return f" {flag}" in f.read()
+    except OSError:
+        return False
+
+
+_avx2 = None
+
+
+def load_avx2():
+    """AVX2 intrinsics twin of the reference's SIMD fused rows (CPU baseline); None when the
+    host CPU lacks AVX2/FMA/F16C."""
+    global _avx2
+    if _avx2 is not None:
+        return _avx2
+    if not (host_has("avx2") and host_has("fma") and host_has("f16c")):
+        return None
+    if not os.path.exists(AVX2_PATH):
+        subprocess.run(["make", "-C", ORACLE_DIR, "-s", "liboxq_cpu_avx2.so"], check=True)
+    lib = C.CDLL(AVX2_PATH)
+    lib.oxq_avx2_matvec_q8_fused.restype = C.c_int
+    lib.oxq_avx2_matvec_q8_fused.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
+                                             C.c_size_t, C.c_int]
+    _avx2 = lib
+    return lib
+
+
+def avx2_matvec_q8_fused(t, w, acts, n_rows, n_cols, threads=1, out=None):
+    lib = load_avx2()
+    w, acts = _u8(w), _u8(acts)
+    if out is None:
+        out = np.zeros(max(n_rows, 1), dtype=np.float32)
+    rc = lib.oxq_avx2_matvec_q8_fused(t, _p(w), _p(acts), _p(out), n_rows, n_cols, threads)
+    if rc != 0:
+        raise ValueError("unsupported type or partial block")
+    return out[:n_rows]
 
 
 def load():

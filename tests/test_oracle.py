@@ -522,3 +522,18 @@ def test_threaded_row_split_is_bit_identical(ref):
     w = synth.weights(O.Q4_K, 91, 37, 512)
     a = ref.quantize_q8_0(synth.normal_f32(92, 512))
     assert np.array_equal(ref.matvec_q8_fused_mt(O.Q4_K, w, a, 37, 512, 4), ref.matvec_q8_fused(O.Q4_K, w, a, 37, 512))
+
+
+@pytest.mark.parametrize("t", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K], ids=lambda t: O.NAMES[t])
+def test_avx2_twin_is_bit_identical_to_the_avx2_tier_restatement(ref, t):
+    """The intrinsics twin timed as the CPU baseline computes exactly what the oracle's
+    AVX2-order rows compute (integer sums are exact; the fp32 order is the same)."""
+    from oxillama_amd import synth
+    if ref.load_avx2() is None:
+        pytest.skip("host CPU lacks AVX2/FMA/F16C")
+    n_rows, n_cols = 19, 2048
+    w = synth.weights(t, 95, n_rows, n_cols)
+    a = ref.quantize_q8_0(synth.normal_f32(96, n_cols))
+    want = ref.matvec_q8_fused(t, w, a, n_rows, n_cols, tier=O.TIER_AVX2)
+    assert np.array_equal(ref.avx2_matvec_q8_fused(t, w, a, n_rows, n_cols, threads=1), want)
+    assert np.array_equal(ref.avx2_matvec_q8_fused(t, w, a, n_rows, n_cols, threads=3), want)
