@@ -185,6 +185,12 @@ int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d
 /* Launch width of the GEMV kernels: resident waves per compute unit (tuning
  * knob for benchmarks; 0 restores the default). */
 int oxq_set_gemv_waves_per_cu(unsigned waves);
+/* Rows a wave loads per batch in the GEMV kernels (1, 2 or 4; tuning knob; 0 restores
+ * the per-shape default). */
+int oxq_set_gemv_rows_per_batch(unsigned rows);
+/* Waves that share one row in the GEMV kernels (1 or 4; tuning knob; 0 restores the
+ * per-shape default: 4 for rows of three or more 64-unit steps). */
+int oxq_set_gemv_waves_per_row(unsigned waves);
 
 #ifdef __cplusplus
 }

@@ -3,6 +3,7 @@
 `python -m oxillama_amd.build` compiles
   * oxillama_amd/liboxq_hip.so   -- HIP kernels + C ABI (include/oxq.h), gfx950 only
   * oxillama_amd/liboxq_synth.so -- host-side synthetic weight generator
+  * oxillama_amd/liboxq_benchkit.so -- copy / streaming-read kernels for measurement calibration
 hipcc cross-compiles gfx950 code objects without a GPU present.
 """
 import os
@@ -14,6 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 HIP_SOURCES = ["oxq_api.hip", "oxq_gemv.hip", "oxq_gemm.hip", "oxq_quantize.hip"]
 HIP_LIB = os.path.join(HERE, "liboxq_hip.so")
 SYNTH_LIB = os.path.join(HERE, "liboxq_synth.so")
+BENCHKIT_LIB = os.path.join(HERE, "liboxq_benchkit.so")
 
 # -ffp-contract=off: the fp32 epilogues follow the reference's operation order (Rust
 # never fuses a*b+c).  Packed fp32 instructions are switched off.
@@ -46,9 +48,16 @@ def build_synth():
     return SYNTH_LIB
 
 
+def build_benchkit():
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    run([hipcc, *HIPCC_FLAGS, "-shared", "-o", BENCHKIT_LIB, os.path.join(CSRC, "benchkit.hip")])
+    return BENCHKIT_LIB
+
+
 def build_all():
     build_hip()
     build_synth()
+    build_benchkit()
 
 
 if __name__ == "__main__":

@@ -77,6 +77,8 @@ SIGNATURES = {
     "oxq_block_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                      C.c_size_t, C.c_void_p]),
     "oxq_set_gemv_waves_per_cu": (C.c_int, [C.c_uint]),
+    "oxq_set_gemv_rows_per_batch": (C.c_int, [C.c_uint]),
+    "oxq_set_gemv_waves_per_row": (C.c_int, [C.c_uint]),
 }
 
 _lib = None

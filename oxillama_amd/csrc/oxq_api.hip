@@ -93,6 +93,8 @@ struct State {
     int device = -1;
     uint32_t cus = 0;
     uint32_t waves_per_cu = 0;  // 0 = default
+    uint32_t rows_per_batch = 0;  // 0 = chosen per shape
+    uint32_t waves_per_row = 0;   // 0 = chosen per shape
     bool cache_enabled = false;
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
     Scratch s_weights, s_acts, s_x, s_out, s_sums;
@@ -193,6 +195,8 @@ oxq::GemvArgs gemv_args(const uint8_t *W, const uint8_t *A, float *out, int32_t 
     a.n_cols = (uint32_t)n_cols;
     a.accumulate = accumulate;
     a.waves_per_cu = g.waves_per_cu ? g.waves_per_cu : DEFAULT_WAVES_PER_CU;
+    a.rows_per_batch = g.rows_per_batch;
+    a.waves_per_row = g.waves_per_row;
     return a;
 }
 
@@ -344,6 +348,18 @@ int oxq_get_kernel(uint32_t type) {
 int oxq_set_gemv_waves_per_cu(unsigned waves) {
     std::lock_guard<std::mutex> lock(g.mu);
     g.waves_per_cu = waves > 64 ? 64 : waves;
+    return OXQ_OK;
+}
+
+int oxq_set_gemv_rows_per_batch(unsigned rows) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    g.rows_per_batch = rows > 4 ? 4 : rows;
+    return OXQ_OK;
+}
+
+int oxq_set_gemv_waves_per_row(unsigned waves) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    g.waves_per_row = waves >= 4 ? 4 : (waves ? 1 : 0);
     return OXQ_OK;
 }
 

@@ -22,6 +22,25 @@ __device__ __forceinline__ u32x2 ld8(const uint8_t *p) { return reinterpret_cast
 __device__ __forceinline__ uint32_t ld4(const uint8_t *p) { return reinterpret_cast<const PackedU1 *>(p)->v; }
 __device__ __forceinline__ uint32_t ld2(const uint8_t *p) { return reinterpret_cast<const PackedH1 *>(p)->v; }
 
+// 16 bytes at an address that is only 2-byte aligned, without a sub-dword-misaligned
+// vector load (those cost ~15% of streaming bandwidth on gfx950): read five dwords from
+// the 4-byte-aligned address at or just below p and funnel-shift by 0, 8, 16 or 24 bits.  The
+// fifth dword is only fetched when p is misaligned (otherwise the fourth is re-read), so
+// nothing past the dword that holds byte p+15 is touched.
+__device__ __forceinline__ u32x4 ld16_h(const uint8_t *p) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    const uint32_t sh = (uint32_t)(a & 3) * 8;
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(a & ~(uintptr_t)3);
+    const u32x4 lo = reinterpret_cast<const PackedU4 *>(q)->v;
+    const uint32_t hi = q[sh ? 4 : 3];
+    u32x4 r;
+    r[0] = __builtin_amdgcn_alignbit(lo[1], lo[0], sh);
+    r[1] = __builtin_amdgcn_alignbit(lo[2], lo[1], sh);
+    r[2] = __builtin_amdgcn_alignbit(lo[3], lo[2], sh);
+    r[3] = __builtin_amdgcn_alignbit(hi, lo[3], sh);
+    return r;
+}
+
 __device__ __forceinline__ void st2(uint8_t *p, uint32_t v) { reinterpret_cast<PackedH1 *>(p)->v = (uint16_t)v; }
 
 // IEEE binary16 bits -> float (v_cvt_f32_f16; subnormals are kept).

@@ -2,13 +2,27 @@
 //
 // A row of n_cols weights is cut into "units"; lane l of a wave owns unit
 // 64*step + l.  For each format this file says which raw GGUF bytes the lane
-// loads for its unit (Wt), which Q8_0 activation bytes it keeps in registers for
-// every row (Act), and how the exact int32 group sums and the fp32 term are
-// formed from them.  Byte layouts follow the reference decoders cited below
-// (Q/ = crates/oxillama-quant/src in the reference tree).
+// loads for its unit (Wt), which Q8_0 activation bytes and derived constants it
+// keeps in registers for every row (Act), and how the exact int32 group sums
+// and the fp32 contribution are formed from them.  Byte layouts follow the
+// reference decoders cited below (Q/ = crates/oxillama-quant/src in the
+// reference tree).
 //
 // Integer groups (the unit of the bit-exact check): 32 weights = one Q8_0
 // activation block for Q4_0 / Q8_0 / Q4_K / IQ4_XS, 16 weights for Q6_K.
+//
+// Loads are unconditional: a lane past the end of the row (`valid` false) reads
+// the row's last unit instead and carries all-zero activation constants, so it
+// contributes exactly 0 without any divergent control flow.
+//
+// fp32 form.  With I = integer group sum, the reference's fused rows compute
+// (d*sc*I - dmin*mn*S) * d_a per group (Q/simd/avx2/q4_k.rs:329).  d*sc, dmin*mn
+// and the products sc*I, mn*S are exact in fp32 (11-bit f16 significand times a
+// 6..8-bit integer; |sc*I| < 2^24), so d*float(sc*I) rounds exactly as
+// (d*sc)*float(I) does.  The kernels use that to do the scale multiplications in
+// integer arithmetic, and they accumulate the groups of one unit with fused
+// multiply-adds before the cross-lane sum; only the accumulation order and the
+// placement of roundings differ from the reference, within the 1e-5*|y|inf bar.
 #pragma once
 #include "oxq_device.hpp"
 
@@ -16,79 +30,91 @@ namespace oxq {
 
 constexpr uint32_t Q8_BLOCK_BYTES = 34;  // Q/traits.rs:12: f16 d + 32 x i8
 
+// v_mul_i32_i24: exact product of two values that fit in 24 signed bits.
+__device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
+
 // ---------------------------------------------------------------------------
 // Q4_K, Q/reference/q4_k.rs:27-99,218-333.  144 B = d, dmin (f16), 12 B packed
-// 6-bit scales/mins, 128 B nibbles.  Unit = one 16-byte chunk c (0..7) of qs:
-// low nibbles are 16 weights of sub-block 2g, high nibbles 16 weights of
-// sub-block 2g+1 (g = c/2), at bytes 16h.. of those activation blocks (h = c&1).
-// The two lanes of a pair (h = 0, 1) add their halves; lane h then owns the fp32
-// term of sub-block 2g+h = c.
+// 6-bit scales/mins, 128 B nibbles.  Unit = one 64-weight group g (0..3) of a
+// super-block: qs[32g..32g+32], low nibbles = sub-block 2g, high nibbles =
+// sub-block 2g+1, against activation blocks 8b+2g and 8b+2g+1.  Four lanes per
+// super-block; the 16-byte header is read by each of them (same cache line).
 struct FmtQ4K {
-    static constexpr uint32_t BLOCK_BYTES = 144, BLOCK_COLS = 256, UNIT_COLS = 32;
+    static constexpr uint32_t BLOCK_BYTES = 144, BLOCK_COLS = 256, UNIT_COLS = 64;
     struct Lane {
-        uint32_t c, h, sh;
+        uint32_t g, sh;
         bool upper;
     };
     struct Act {
-        u32x4 lo, hi;
-        float d_a, fasum;
+        u32x4 lo0, lo1, hi0, hi1;
+        float a_lo, a_hi;  // d_a of the two activation blocks
+        float b_lo, b_hi;  // d_a * sum(q_a)
     };
     struct Wt {
-        u32x4 hdr, qs;
+        u32x4 hdr, q0, q1;
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t lane) {
         Lane k;
-        k.c = lane & 7;
-        k.h = lane & 1;
-        k.sh = (k.c & 3) * 8;
-        k.upper = k.c >= 4;
+        k.g = lane & 3;
+        k.sh = (k.g & 1) * 16;
+        k.upper = k.g >= 2;
         return k;
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
                                                     const Lane &k) {
-        const uint32_t b = u >> 3, g = k.c >> 1;
-        const uint8_t *blo = A + (size_t)(8 * b + 2 * g) * Q8_BLOCK_BYTES;
+        const uint8_t *blo = A + (size_t)(8 * (u >> 2) + 2 * k.g) * Q8_BLOCK_BYTES;
         const uint8_t *bhi = blo + Q8_BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        a.lo = valid ? ld16(blo + 2 + 16 * k.h) : z;
-        a.hi = valid ? ld16(bhi + 2 + 16 * k.h) : z;
+        a.lo0 = ld16(blo + 2);
+        a.lo1 = ld16(blo + 18);
+        a.hi0 = ld16(bhi + 2);
+        a.hi1 = ld16(bhi + 18);
         int slo = 0, shi = 0;
         for (int i = 0; i < 4; i++) {
-            slo = sdot4(a.lo[i], 0x01010101u, slo);
-            shi = sdot4(a.hi[i], 0x01010101u, shi);
+            slo = sdot4(a.lo0[i], 0x01010101u, slo);
+            slo = sdot4(a.lo1[i], 0x01010101u, slo);
+            shi = sdot4(a.hi0[i], 0x01010101u, shi);
+            shi = sdot4(a.hi1[i], 0x01010101u, shi);
         }
-        slo += xor1_i(slo);
-        shi += xor1_i(shi);
-        a.fasum = (float)(k.h ? shi : slo);
-        a.d_a = valid ? h2f(ld2(k.h ? bhi : blo)) : 0.0f;
+        const float dlo = h2f(ld2(blo)), dhi = h2f(ld2(bhi));
+        a.a_lo = valid ? dlo : 0.0f;
+        a.a_hi = valid ? dhi : 0.0f;
+        a.b_lo = valid ? dlo * (float)slo : 0.0f;
+        a.b_hi = valid ? dhi * (float)shi : 0.0f;
     }
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, bool valid,
-                                                  const Lane &k) {
-        const uint8_t *blk = row + (size_t)(u >> 3) * BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        w.hdr = valid ? ld16(blk) : z;
-        w.qs = valid ? ld16(blk + 16 + 16 * k.c) : z;
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &k) {
+        const uint8_t *blk = row + (size_t)(u >> 2) * BLOCK_BYTES;
+        w.hdr = ld16(blk);
+        w.q0 = ld16(blk + 16 + 32 * k.g);
+        w.q1 = ld16(blk + 32 + 32 * k.g);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &k, int32_t *sums,
                                                 uint32_t u, bool valid) {
         int plo = 0, phi = 0;
         for (int i = 0; i < 4; i++) {
-            plo = sdot4(w.qs[i] & 0x0F0F0F0Fu, a.lo[i], plo);
-            phi = sdot4((w.qs[i] >> 4) & 0x0F0F0F0Fu, a.hi[i], phi);
+            plo = sdot4(w.q0[i] & 0x0F0F0F0Fu, a.lo0[i], plo);
+            phi = sdot4((w.q0[i] >> 4) & 0x0F0F0F0Fu, a.hi0[i], phi);
+            plo = sdot4(w.q1[i] & 0x0F0F0F0Fu, a.lo1[i], plo);
+            phi = sdot4((w.q1[i] >> 4) & 0x0F0F0F0Fu, a.hi1[i], phi);
         }
-        plo += xor1_i(plo);
-        phi += xor1_i(phi);
-        const int isum = k.h ? phi : plo;
-        // 6-bit scale / min of sub-block j = c (decode_scales_mins, q4_k.rs:27-49)
-        const uint32_t s_a = (w.hdr[1] >> k.sh) & 0xFF, s_b = (w.hdr[2] >> k.sh) & 0xFF,
-                       s_c = (w.hdr[3] >> k.sh) & 0xFF;
-        const uint32_t sc = k.upper ? ((s_c & 0x0F) | ((s_a >> 6) << 4)) : (s_a & 0x3F);
-        const uint32_t mn = k.upper ? ((s_c >> 4) | ((s_b >> 6) << 4)) : (s_b & 0x3F);
+        if (DUMP && valid) {
+            sums[2 * u] = plo;
+            sums[2 * u + 1] = phi;
+        }
+        // 6-bit scales / mins of sub-blocks 2g, 2g+1 as byte pairs (decode_scales_mins,
+        // q4_k.rs:27-49): j < 4: sc = s[j] & 63, mn = s[j+4] & 63; j >= 4: sc = (s[j+4] & 15) |
+        // (s[j-4] >> 6) << 4, mn = (s[j+4] >> 4) | (s[j] >> 6) << 4.
+        const uint32_t sa = w.hdr[1] >> k.sh, sb = w.hdr[2] >> k.sh, sc3 = w.hdr[3] >> k.sh;
+        const uint32_t x = k.upper ? sc3 : sa, y = k.upper ? (sc3 >> 4) : sb;
+        const uint32_t m1 = k.upper ? 0x0F0Fu : 0x3F3Fu, m2 = k.upper ? 0x3030u : 0u;
+        const uint32_t sc2 = (x & m1) | ((sa >> 2) & m2);
+        const uint32_t mn2 = (y & m1) | ((sb >> 2) & m2);
         const float d = h2f(w.hdr[0] & 0xFFFF), dmin = h2f(w.hdr[0] >> 16);
-        const float da = d * (float)sc, m = dmin * (float)mn;  // q4_k.rs:280-281
-        if (DUMP && valid) sums[u] = isum;
-        return (da * (float)isum - m * a.fasum) * a.d_a;  // q4_k.rs:307 / avx2/q4_k.rs:329
+        float su = a.a_lo * (float)mul24(plo, (int)(sc2 & 0xFF));
+        su = fmaf(a.a_hi, (float)mul24(phi, (int)((sc2 >> 8) & 0xFF)), su);
+        float sv = a.b_lo * (float)(mn2 & 0xFF);
+        sv = fmaf(a.b_hi, (float)((mn2 >> 8) & 0xFF), sv);
+        return fmaf(d, su, -(dmin * sv));
     }
 };
 
@@ -96,8 +122,8 @@ struct FmtQ4K {
 // Q6_K, Q/reference/q6_k.rs:39-72,246-351.  210 B = ql[128], qh[64], i8
 // scales[16], f16 d.  Unit = (half hh, sixteen is) of a super-block: bytes
 // ql[64hh+16is..+16], ql[64hh+32+16is..+16], qh[32hh+16is..+16] give four
-// 16-weight sub-blocks at columns 128hh + 32k + 16is (k = 0..3), scale index
-// 8hh + is + 2k, activation block 8b + 4hh + k bytes 16is..+16.
+// 16-weight sub-blocks at columns 128hh + 32j + 16is (j = 0..3), scale index
+// 8hh + is + 2j, activation block 8b + 4hh + j bytes 16is..+16.
 struct FmtQ6K {
     static constexpr uint32_t BLOCK_BYTES = 210, BLOCK_COLS = 256, UNIT_COLS = 64;
     struct Lane {
@@ -106,7 +132,7 @@ struct FmtQ6K {
     struct Act {
         u32x4 q[4];
         float d_a[4];
-        int asum32[4];  // 32 * sum of the 16 activation bytes
+        int nasum32[4];  // -32 * sum of the 16 activation bytes
     };
     struct Wt {
         u32x4 ql0, ql1, qh;
@@ -121,57 +147,57 @@ struct FmtQ6K {
     }
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
                                                     const Lane &k) {
-        const uint32_t b = u >> 2;
         const u32x4 z = {0, 0, 0, 0};
         for (int j = 0; j < 4; j++) {
-            const uint8_t *blk = A + (size_t)(8 * b + 4 * k.hh + j) * Q8_BLOCK_BYTES;
-            a.q[j] = valid ? ld16(blk + 2 + 16 * k.is) : z;
+            const uint8_t *blk = A + (size_t)(8 * (u >> 2) + 4 * k.hh + j) * Q8_BLOCK_BYTES;
+            const u32x4 q = ld16(blk + 2 + 16 * k.is);
+            a.q[j] = valid ? q : z;
             a.d_a[j] = valid ? h2f(ld2(blk)) : 0.0f;
             int s = 0;
             for (int i = 0; i < 4; i++) s = sdot4(a.q[j][i], 0x01010101u, s);
-            a.asum32[j] = 32 * s;
+            a.nasum32[j] = -32 * s;
         }
     }
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, bool valid,
-                                                  const Lane &k) {
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &k) {
         const uint8_t *blk = row + (size_t)(u >> 2) * BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        const u32x2 z2 = {0, 0};
-        w.ql0 = valid ? ld16(blk + 64 * k.hh + 16 * k.is) : z;
-        w.ql1 = valid ? ld16(blk + 64 * k.hh + 32 + 16 * k.is) : z;
-        w.qh = valid ? ld16(blk + 128 + 32 * k.hh + 16 * k.is) : z;
-        w.sc = valid ? ld8(blk + 192 + 8 * k.hh) : z2;
-        w.d = valid ? ld2(blk + 208) : 0u;
+        w.ql0 = ld16(blk + 64 * k.hh + 16 * k.is);
+        w.ql1 = ld16(blk + 64 * k.hh + 32 + 16 * k.is);
+        w.qh = ld16(blk + 128 + 32 * k.hh + 16 * k.is);
+        w.sc = ld8(blk + 192 + 8 * k.hh);
+        w.d = ld2(blk + 208);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &k, int32_t *sums,
                                                 uint32_t u, bool valid) {
-        int p0 = 0, p1 = 0, p2 = 0, p3 = 0;
+        // sum (q - 32) a = sum q a - 32 sum a: the accumulators start at -32 sum a
+        int p0 = a.nasum32[0], p1 = a.nasum32[1], p2 = a.nasum32[2], p3 = a.nasum32[3];
         for (int i = 0; i < 4; i++) {
             const uint32_t l0 = w.ql0[i], l1 = w.ql1[i], h = w.qh[i];
-            // q6_k.rs:55-60, four bytes at a time
-            const uint32_t q0 = (l0 & 0x0F0F0F0Fu) | ((h << 4) & 0x30303030u);
-            const uint32_t q1 = (l1 & 0x0F0F0F0Fu) | ((h << 2) & 0x30303030u);
-            const uint32_t q2 = ((l0 >> 4) & 0x0F0F0F0Fu) | (h & 0x30303030u);
-            const uint32_t q3 = ((l1 >> 4) & 0x0F0F0F0Fu) | ((h >> 2) & 0x30303030u);
+            // q6_k.rs:55-60, four bytes at a time.  hm holds the 2-bit fields of q1 (bits 0-1)
+            // and q3 (bits 4-5) of every byte, hn those of q2 and q4; a bitfield insert under
+            // the low-nibble mask joins them with the ql nibbles.
+            const uint32_t hm = h & 0x33333333u, hn = (h >> 2) & 0x33333333u;
+            const uint32_t q0 = (l0 & 0x0F0F0F0Fu) | ((hm << 4) & 0xF0F0F0F0u);
+            const uint32_t q1 = (l1 & 0x0F0F0F0Fu) | ((hn << 4) & 0xF0F0F0F0u);
+            const uint32_t q2 = ((l0 >> 4) & 0x0F0F0F0Fu) | (hm & 0xF0F0F0F0u);
+            const uint32_t q3 = ((l1 >> 4) & 0x0F0F0F0Fu) | (hn & 0xF0F0F0F0u);
             p0 = sdot4(q0, a.q[0][i], p0);
             p1 = sdot4(q1, a.q[1][i], p1);
             p2 = sdot4(q2, a.q[2][i], p2);
             p3 = sdot4(q3, a.q[3][i], p3);
         }
-        const int isum[4] = {p0 - a.asum32[0], p1 - a.asum32[1], p2 - a.asum32[2], p3 - a.asum32[3]};
+        const int isum[4] = {p0, p1, p2, p3};
         // scales[8hh + is + 2j]: bytes is, is+2 of sc[0], then of sc[1]
         const uint32_t s0 = w.sc[0] >> (8 * k.is), s1 = w.sc[1] >> (8 * k.is);
         const int scv[4] = {(int)(int8_t)(s0 & 0xFF), (int)(int8_t)((s0 >> 16) & 0xFF),
                             (int)(int8_t)(s1 & 0xFF), (int)(int8_t)((s1 >> 16) & 0xFF)};
-        const float d = h2f(w.d);
         float t = 0.0f;
         for (int j = 0; j < 4; j++) {
-            const float s = d * (float)scv[j];  // q6_k.rs:285
-            t += s * (float)isum[j] * a.d_a[j];
+            // |sc * isum| <= 128 * 16 * 63 * 128 < 2^24: exact as int24 operands and as fp32
+            t = fmaf(a.d_a[j], (float)mul24(isum[j], scv[j]), t);
             if (DUMP && valid) sums[16 * (u >> 2) + 8 * k.hh + 2 * j + k.is] = isum[j];
         }
-        return t;
+        return h2f(w.d) * t;
     }
 };
 
@@ -193,18 +219,15 @@ struct FmtQ8_0 {
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
                                                     const Lane &) {
         const uint8_t *blk = A + (size_t)u * Q8_BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        a.q0 = valid ? ld16(blk + 2) : z;
-        a.q1 = valid ? ld16(blk + 18) : z;
+        a.q0 = ld16(blk + 2);
+        a.q1 = ld16(blk + 18);
         a.d_a = valid ? h2f(ld2(blk)) : 0.0f;
     }
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, bool valid,
-                                                  const Lane &) {
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        w.q0 = valid ? ld16(blk + 2) : z;
-        w.q1 = valid ? ld16(blk + 18) : z;
-        w.d = valid ? ld2(blk) : 0u;
+        w.q0 = ld16_h(blk + 2);
+        w.q1 = ld16_h(blk + 18);
+        w.d = ld2(blk);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &, int32_t *sums,
@@ -242,7 +265,7 @@ struct FmtQ4_0 {
     struct Act {
         uint32_t ev[4], od[4];
         float d_a;
-        int asum8;
+        int nasum8;  // -8 * sum of the 32 activation bytes
     };
     struct Wt {
         u32x4 q;
@@ -252,33 +275,29 @@ struct FmtQ4_0 {
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
                                                     const Lane &) {
         const uint8_t *blk = A + (size_t)u * Q8_BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        const u32x4 q0 = valid ? ld16(blk + 2) : z, q1 = valid ? ld16(blk + 18) : z;
+        const u32x4 q0 = ld16(blk + 2), q1 = ld16(blk + 18);
         split_even_odd(q0, q1, a.ev, a.od);
         int s = 0;
         for (int i = 0; i < 4; i++) {
             s = sdot4(q0[i], 0x01010101u, s);
             s = sdot4(q1[i], 0x01010101u, s);
         }
-        a.asum8 = 8 * s;
+        a.nasum8 = -8 * s;
         a.d_a = valid ? h2f(ld2(blk)) : 0.0f;
     }
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, bool valid,
-                                                  const Lane &) {
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        w.q = valid ? ld16(blk + 2) : z;
-        w.d = valid ? ld2(blk) : 0u;
+        w.q = ld16_h(blk + 2);
+        w.d = ld2(blk);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &, int32_t *sums,
                                                 uint32_t u, bool valid) {
-        int p = 0;
+        int p = a.nasum8;
         for (int i = 0; i < 4; i++) {
             p = sdot4(w.q[i] & 0x0F0F0F0Fu, a.ev[i], p);
             p = sdot4((w.q[i] >> 4) & 0x0F0F0F0Fu, a.od[i], p);
         }
-        p -= a.asum8;
         if (DUMP && valid) sums[u] = p;
         const float scale = h2f(w.d) * a.d_a;  // avx2/q4_0.rs:211
         return scale * (float)p;               // avx2/q4_0.rs:265
@@ -289,7 +308,7 @@ struct FmtQ4_0 {
 // IQ4_XS, Q/reference/iq4_xs.rs:47-97; codebook Q/reference/iq_shared.rs:16-18.
 // 136 B = f16 d, u16 scales_h, 4 B scales_l, 128 B nibble indices.  Unit = one
 // 32-weight sub-block i: qs[16i..16i+16], interleaved nibbles.  Term:
-// (d * (ls - 32)) * float(sum kvalues[idx] * a) * d_a.
+// d * float((ls - 32) * sum kvalues[idx] * a) * d_a.
 struct FmtIQ4XS {
     static constexpr uint32_t BLOCK_BYTES = 136, BLOCK_COLS = 256, UNIT_COLS = 32;
     struct Lane {
@@ -307,18 +326,14 @@ struct FmtIQ4XS {
     static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
                                                     const Lane &) {
         const uint8_t *blk = A + (size_t)u * Q8_BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        const u32x4 q0 = valid ? ld16(blk + 2) : z, q1 = valid ? ld16(blk + 18) : z;
+        const u32x4 q0 = ld16(blk + 2), q1 = ld16(blk + 18);
         split_even_odd(q0, q1, a.ev, a.od);
         a.d_a = valid ? h2f(ld2(blk)) : 0.0f;
     }
-    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, bool valid,
-                                                  const Lane &k) {
+    static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &k) {
         const uint8_t *blk = row + (size_t)(u >> 3) * BLOCK_BYTES;
-        const u32x4 z = {0, 0, 0, 0};
-        const u32x2 z2 = {0, 0};
-        w.hdr = valid ? ld8(blk) : z2;
-        w.q = valid ? ld16(blk + 8 + 16 * k.i) : z;
+        w.hdr = ld8(blk);
+        w.q = ld16(blk + 8 + 16 * k.i);
     }
     // Four 4-bit indices (one per byte) -> four codebook bytes: two 8-entry byte
     // permutes, then a third permute picks the upper table where bit 3 is set.
@@ -342,8 +357,8 @@ struct FmtIQ4XS {
         const uint32_t ls_low = (w.hdr[1] >> (4 * k.i)) & 0x0F;
         const uint32_t ls_high = ((w.hdr[0] >> 16) >> (2 * k.i)) & 0x03;
         const int ls = (int)(ls_low | (ls_high << 4)) - 32;
-        const float scale = h2f(w.hdr[0] & 0xFFFF) * (float)ls;  // iq4_xs.rs:81
-        return scale * (float)p * a.d_a;
+        // |ls * p| <= 32 * 32 * 127 * 128 < 2^24: exact
+        return h2f(w.hdr[0] & 0xFFFF) * ((float)mul24(p, ls) * a.d_a);
     }
 };
 

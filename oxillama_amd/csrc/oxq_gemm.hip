@@ -18,6 +18,8 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
         g.n_cols = a.k;
         g.accumulate = a.accumulate;
         g.waves_per_cu = 8;
+        g.rows_per_batch = 0;
+        g.waves_per_row = 0;
         hipError_t e = launch_gemv_q8(type, g, stream);
         if (e != hipSuccess) return e;
     }

@@ -1,0 +1,177 @@
+// Kernel templates of the Q8_0-activation GEMV (see oxq_gemv.hip for the design).
+#pragma once
+#include "oxq_formats.hpp"
+
+namespace oxq {
+
+// Cached-activation kernel.  A work group is four waves.  KS waves share a row
+// (wave `part` owns steps [part*STEPS, (part+1)*STEPS) of it, i.e. a contiguous
+// slice of the columns) and 4/KS such groups work on different rows.  The
+// activation constants of a wave's steps live in registers for the whole kernel.
+// Rows are taken in batches of RB; the weight loads of the next batch are issued
+// (into a second register set) before the current batch is reduced, so every
+// wave always has loads in flight.  With KS > 1 the per-wave row sums are added
+// through LDS in a fixed order (part 0, 1, ...), one barrier per batch.
+template <class F, int STEPS, int RB>
+struct Batch {
+    typename F::Wt w[RB][STEPS];
+    float old;
+};
+
+template <class F, int STEPS, int RB>
+__device__ __forceinline__ void load_batch(Batch<F, STEPS, RB> &b, const uint8_t *__restrict__ W,
+                                           const float *__restrict__ out, uint32_t batch, uint32_t n_rows,
+                                           size_t row_bytes, uint32_t units, uint32_t unit0, uint32_t lane,
+                                           const typename F::Lane &k, bool want_old) {
+    const uint32_t row0 = batch * RB;
+    b.old = 0.0f;
+    if (want_old && lane < RB && row0 + lane < n_rows) b.old = out[row0 + lane];
+#pragma unroll
+    for (int r = 0; r < RB; r++) {
+        const uint32_t row = min(row0 + r, n_rows - 1);  // past the last row: re-read it, result unused
+        const uint8_t *rp = W + (size_t)row * row_bytes;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const uint32_t u = min(unit0 + (uint32_t)(s * 64) + lane, units - 1);  // past the end: last unit
+            F::load_w(b.w[r][s], rp, u, k);
+        }
+    }
+}
+
+// Lane r (r < RB) returns the wave's sum for row r of the batch.
+template <class F, int STEPS, int RB, bool DUMP>
+__device__ __forceinline__ float reduce_batch(const Batch<F, STEPS, RB> &b, const typename F::Act (&act)[STEPS],
+                                              int32_t *__restrict__ sums, uint32_t batch, uint32_t n_rows,
+                                              uint32_t units, uint32_t unit0, uint32_t groups_per_row, uint32_t lane,
+                                              const typename F::Lane &k) {
+    const uint32_t row0 = batch * RB;
+    float res = 0.0f;
+#pragma unroll
+    for (int r = 0; r < RB; r++) {
+        const uint32_t row = min(row0 + r, n_rows - 1);
+        float acc = 0.0f;
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
+            acc += F::template dot<DUMP>(b.w[r][s], act[s], k, DUMP ? sums + (size_t)row * groups_per_row : nullptr, u,
+                                         u < units);
+        }
+        const float total = wave_sum(acc);
+        if (lane == (uint32_t)r) res = total;
+    }
+    return res;
+}
+
+template <class F, int STEPS, int RB, int KS, bool DUMP>
+__global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict__ W,
+                                                     const uint8_t *__restrict__ A,
+                                                     float *__restrict__ out, int32_t *__restrict__ sums,
+                                                     uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
+                                                     size_t row_bytes, int accumulate) {
+    static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
+    constexpr uint32_t G = 4 / KS;  // row groups per work group
+    __shared__ float part_sums[2][4][4];
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const uint32_t part = wave_in_wg % KS, grp = wave_in_wg / KS;
+    const uint32_t group = blockIdx.x * G + grp;
+    const uint32_t n_groups = gridDim.x * G;
+    const uint32_t unit0 = part * STEPS * 64;
+    const typename F::Lane k = F::lane_consts(lane);
+    const uint32_t n_batches = (n_rows + RB - 1) / RB;
+    // With KS > 1 every wave of the work group runs the same number of trips (barriers);
+    // trips past the last batch re-read the last rows and store nothing.
+    const uint32_t n_trips = KS == 1 ? n_batches : ((n_batches + n_groups - 1) / n_groups) * n_groups;
+    if (KS == 1 && group >= n_batches) return;
+    const bool want_old = accumulate && part == 0;
+
+    // Activations first (they sit in L2 and arrive early), then the first batch of
+    // weights: the activation constants are derived while HBM is being read.
+    typename F::Act act[STEPS];
+#pragma unroll
+    for (int s = 0; s < STEPS; s++) {
+        const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
+        F::load_act(act[s], A, min(u, units - 1), u < units, k);  // all-zero constants past the end
+    }
+    Batch<F, STEPS, RB> b0, b1;
+    load_batch<F, STEPS, RB>(b0, W, out, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
+
+    uint32_t trip = 0;
+    auto finish = [&](float res, float old, uint32_t batch) {
+        const uint32_t row = batch * RB + lane;
+        if (KS == 1) {
+            if (lane < RB && row < n_rows) out[row] = old + res;
+        } else {
+            if (lane < RB) part_sums[trip & 1][wave_in_wg][lane] = res;
+            __syncthreads();
+            if (part == 0 && lane < RB && batch < n_batches && row < n_rows) {
+                float t = part_sums[trip & 1][grp * KS][lane];
+#pragma unroll
+                for (int p = 1; p < KS; p++) t += part_sums[trip & 1][grp * KS + p][lane];
+                out[row] = old + t;
+            }
+            trip++;
+        }
+    };
+
+    // Each reduce_batch call site has a fixed set of loads in flight behind it, so the
+    // compiler can wait for exactly the batch it needs and leave the prefetch outstanding.
+    uint32_t batch = group;
+    while (true) {
+        const uint32_t next = batch + n_groups;
+        if (next >= n_trips) {
+            const float r0 = reduce_batch<F, STEPS, RB, DUMP>(b0, act, sums, min(batch, n_batches - 1), n_rows, units,
+                                                              unit0, groups_per_row, lane, k);
+            finish(r0, b0.old, batch);
+            break;
+        }
+        load_batch<F, STEPS, RB>(b1, W, out, min(next, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
+        const float r0 = reduce_batch<F, STEPS, RB, DUMP>(b0, act, sums, min(batch, n_batches - 1), n_rows, units, unit0,
+                                                          groups_per_row, lane, k);
+        finish(r0, b0.old, batch);
+        const uint32_t next2 = next + n_groups;
+        if (next2 >= n_trips) {
+            const float r1 = reduce_batch<F, STEPS, RB, DUMP>(b1, act, sums, min(next, n_batches - 1), n_rows, units,
+                                                              unit0, groups_per_row, lane, k);
+            finish(r1, b1.old, next);
+            break;
+        }
+        load_batch<F, STEPS, RB>(b0, W, out, min(next2, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
+        const float r1 = reduce_batch<F, STEPS, RB, DUMP>(b1, act, sums, min(next, n_batches - 1), n_rows, units, unit0,
+                                                          groups_per_row, lane, k);
+        finish(r1, b1.old, next);
+        batch = next2;
+    }
+}
+
+// Any number of steps: activations re-read (from L2) for every row.
+template <class F, bool DUMP>
+__global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict__ W,
+                                                      const uint8_t *__restrict__ A,
+                                                      float *__restrict__ out, int32_t *__restrict__ sums,
+                                                      uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
+                                                      size_t row_bytes, int accumulate) {
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    const uint32_t n_waves = (gridDim.x * blockDim.x) >> 6;
+    const typename F::Lane k = F::lane_consts(lane);
+    const uint32_t steps = (units + 63) / 64;
+    for (uint32_t row = wave; row < n_rows; row += n_waves) {
+        const uint8_t *rp = W + (size_t)row * row_bytes;
+        float acc = 0.0f;
+        for (uint32_t s = 0; s < steps; s++) {
+            const uint32_t u = s * 64 + lane;
+            const bool valid = u < units;
+            typename F::Act a;
+            typename F::Wt w;
+            const uint32_t uc = min(u, units - 1);
+            F::load_w(w, rp, uc, k);
+            F::load_act(a, A, uc, valid, k);
+            acc += F::template dot<DUMP>(w, a, k, DUMP ? sums + (size_t)row * groups_per_row : nullptr, u, valid);
+        }
+        const float total = wave_sum(acc);
+        if (lane == 0) out[row] = (accumulate ? out[row] : 0.0f) + total;
+    }
+}
+
+}  // namespace oxq
