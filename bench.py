@@ -190,15 +190,16 @@ def main():
         xsq = torch.empty(M * (H // 32 * 34), dtype=torch.uint8, device=dev)
         ys = torch.zeros(M * F, dtype=torch.float32, device=dev)
         wp = [layers[i % L]["gate"] for i in range(min(L, 8))]
+        ws = torch.empty(max(k_q4k.gemm_workspace_bytes(M, F, H), 256), dtype=torch.uint8, device=dev)
         with torch.cuda.stream(stream):
             quant.quantize_q8_0_dev(xs, xsq)
-            k_q4k.gemm_q8_dev(wp[0], xsq, ys, M, F, H)
+            k_q4k.gemm_q8_dev(wp[0], xsq, ys, M, F, H, workspace=ws)
             stream.synchronize()
             reps = 8
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
             for i in range(reps):
-                k_q4k.gemm_q8_dev(wp[i % len(wp)], xsq, ys, M, F, H)
+                k_q4k.gemm_q8_dev(wp[i % len(wp)], xsq, ys, M, F, H, workspace=ws)
             e1.record(stream)
             e1.synchronize()
             gemm_us = e0.elapsed_time(e1) * 1e3 / reps

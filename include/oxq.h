@@ -174,10 +174,22 @@ int oxq_matvec_q8_fused_dev(uint32_t type, const uint8_t *d_weights, const uint8
                             void *stream);
 
 /* Prefill: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched form
- * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  Q4_K uses
- * the int8-MFMA tile kernel; other formats run m fused matvecs. */
+ * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  Q4_K with
+ * m >= 8 uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()
+ * bytes of 256-byte-aligned device scratch: pass it and the call is asynchronous
+ * and allocation-free; pass NULL and the library uses its own scratch (the call
+ * then serialises and waits for the stream).  Other formats, and shapes for which
+ * the workspace size is 0, run m fused matvecs and ignore the workspace. */
+size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k);
 int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
-                    float *d_out, size_t m, size_t n, size_t k, int accumulate, void *stream);
+                    float *d_out, size_t m, size_t n, size_t k, int accumulate,
+                    void *d_workspace, size_t workspace_bytes, void *stream);
+/* Debug: as oxq_gemm_q8_dev (overwrite), and the exact int32 group sums of the tile
+ * kernel, d_sums[(r * n + c) * (k/32) + g].  OXQ_ERR_UNSUPPORTED_SHAPE when the shape
+ * has no tile kernel. */
+int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
+                            float *d_out, int32_t *d_sums, size_t m, size_t n, size_t k,
+                            void *d_workspace, size_t workspace_bytes, void *stream);
 
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                        int32_t *d_sums, size_t n_rows, size_t n_cols, void *stream);

@@ -97,7 +97,7 @@ struct State {
     uint32_t waves_per_row = 0;   // 0 = chosen per shape
     bool cache_enabled = false;
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
-    Scratch s_weights, s_acts, s_x, s_out, s_sums;
+    Scratch s_weights, s_acts, s_x, s_out, s_sums, s_work;
 };
 State g;
 
@@ -261,6 +261,7 @@ int oxq_shutdown(void) {
     g.s_x.release();
     g.s_out.release();
     g.s_sums.release();
+    g.s_work.release();
     g.initialised = false;
     g.device = -1;
     return OXQ_OK;
@@ -489,6 +490,11 @@ int oxq_gemm(uint32_t type, const uint8_t *data, size_t data_len, const size_t *
     ga.A = (const uint8_t *)g.s_acts.ptr;
     ga.out = (float *)g.s_out.ptr;
     ga.sums = nullptr;
+    ga.workspace = nullptr;
+    if (oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n_cols)) {
+        if ((st = g.s_work.reserve(oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)n_cols))) != OXQ_OK) return st;
+        ga.workspace = (uint8_t *)g.s_work.ptr;
+    }
     ga.m = (uint32_t)m;
     ga.n = (uint32_t)n_rows;
     ga.k = (uint32_t)n_cols;
@@ -590,8 +596,15 @@ int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d
     return OXQ_OK;
 }
 
-int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, size_t m,
-                    size_t n, size_t k, int accumulate, void *stream) {
+size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k) {
+    (void)n;
+    if (m > 0xFFFFFFFFull || k > 0xFFFFFFFFull || !oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)k)) return 0;
+    return oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k);
+}
+
+static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, int32_t *d_sums,
+                    size_t m, size_t n, size_t k, int accumulate, void *d_workspace, size_t workspace_bytes,
+                    void *stream) {
     int st = check_dev_shape(type, n, k);
     if (st != OXQ_OK) return st;
     if (m > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, m, "dimension exceeds 2^32-1");
@@ -601,13 +614,47 @@ int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
     ga.W = d_weights;
     ga.A = d_acts_q8;
     ga.out = d_out;
-    ga.sums = nullptr;
+    ga.sums = d_sums;
+    ga.workspace = nullptr;
     ga.m = (uint32_t)m;
     ga.n = (uint32_t)n;
     ga.k = (uint32_t)k;
     ga.accumulate = accumulate ? 1 : 0;
+    const size_t need = oxq_gemm_q8_workspace_bytes(type, m, n, k);
+    if (need && d_workspace) {
+        if (workspace_bytes < need) return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, workspace_bytes, "workspace too small");
+        if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
+            return fail(OXQ_ERR_KERNEL, 256, reinterpret_cast<uintptr_t>(d_workspace) & 255, "workspace must be 256-byte aligned");
+        ga.workspace = (uint8_t *)d_workspace;
+        OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
+        return OXQ_OK;
+    }
+    if (need) {
+        // Library-owned scratch: calls serialise on the lock and wait for the stream, because
+        // the scratch is shared.
+        std::lock_guard<std::mutex> lock(g.mu);
+        if ((st = g.s_work.reserve(need)) != OXQ_OK) return st;
+        ga.workspace = (uint8_t *)g.s_work.ptr;
+        OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
+        OXQ_HIP(hipStreamSynchronize((hipStream_t)stream));
+        return OXQ_OK;
+    }
     OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
     return OXQ_OK;
+}
+
+int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, size_t m,
+                    size_t n, size_t k, int accumulate, void *d_workspace, size_t workspace_bytes, void *stream) {
+    return gemm_dev(type, d_weights, d_acts_q8, d_out, nullptr, m, n, k, accumulate, d_workspace, workspace_bytes, stream);
+}
+
+int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out,
+                            int32_t *d_sums, size_t m, size_t n, size_t k, void *d_workspace, size_t workspace_bytes,
+                            void *stream) {
+    if (!d_sums) return fail(OXQ_ERR_INTERNAL, 0, 0, "null sums");
+    if (oxq_gemm_q8_workspace_bytes(type, m, n, k) == 0)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, m, "no tile kernel for this type/shape");
+    return gemm_dev(type, d_weights, d_acts_q8, d_out, d_sums, m, n, k, 0, d_workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

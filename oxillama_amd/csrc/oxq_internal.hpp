@@ -33,10 +33,15 @@ struct GemmArgs {
     const uint8_t *W;   // raw GGUF blocks [n x k]
     const uint8_t *A;   // Q8_0 blocks of the m activation rows, row-major, k/32 blocks per row
     float *out;         // [m x n] row-major
-    int32_t *sums;      // optional debug dump [m][n][k/group]
+    int32_t *sums;      // optional debug dump [m][n][k/32]
+    uint8_t *workspace; // gemm_workspace_bytes(m, k) bytes, 256-byte aligned; null: row-by-row matvecs
     uint32_t m, n, k;
     int accumulate;
 };
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
+// Device scratch the tile kernel needs for m tokens of k columns (activation re-layout).
+size_t gemm_workspace_bytes(uint32_t m, uint32_t k);
+// True when (type, m, k) is served by the int8-MFMA tile kernel.
+bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t k);
 
 }  // namespace oxq

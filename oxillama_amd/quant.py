@@ -232,9 +232,22 @@ class HipKernel:
                                                  d_out.data_ptr(), n_rows, n_cols, int(accumulate),
                                                  self._stream()))
 
-    def gemm_q8_dev(self, d_weights, d_acts, d_out, m, n, k, accumulate=False):
+    def gemm_workspace_bytes(self, m, n, k):
+        return self._lib.oxq_gemm_q8_workspace_bytes(self.tensor_type, m, n, k)
+
+    def gemm_q8_dev(self, d_weights, d_acts, d_out, m, n, k, accumulate=False, workspace=None):
+        """workspace: uint8 CUDA tensor of gemm_workspace_bytes(m, n, k) bytes (256-byte aligned), or None."""
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_len = workspace.numel() if workspace is not None else 0
         _check(self._lib.oxq_gemm_q8_dev(self.tensor_type, d_weights.data_ptr(), d_acts.data_ptr(),
-                                         d_out.data_ptr(), m, n, k, int(accumulate), self._stream()))
+                                         d_out.data_ptr(), m, n, k, int(accumulate), ws_ptr, ws_len, self._stream()))
+
+    def gemm_block_sums_dev(self, d_weights, d_acts, d_out, d_sums, m, n, k, workspace=None):
+        ws_ptr = workspace.data_ptr() if workspace is not None else None
+        ws_len = workspace.numel() if workspace is not None else 0
+        _check(self._lib.oxq_gemm_block_sums_dev(self.tensor_type, d_weights.data_ptr(), d_acts.data_ptr(),
+                                                 d_out.data_ptr(), d_sums.data_ptr(), m, n, k, ws_ptr, ws_len,
+                                                 self._stream()))
 
     def block_sums_dev(self, d_weights, d_acts, d_sums, n_rows, n_cols):
         _check(self._lib.oxq_block_sums_dev(self.tensor_type, d_weights.data_ptr(), d_acts.data_ptr(),

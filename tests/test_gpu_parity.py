@@ -311,6 +311,80 @@ def test_gemm_matches_oracle(hip, ref, t):
     assert_close(y, ref.gemm_q8(t, w, x, m, n, k_), "gemm")
 
 
+def _oracle_prefill(ref, t, w, acts, m, n, k_, rows=None):
+    """m fused matvecs (threaded row split) on already-quantized activation rows."""
+    arb = k_ // 32 * 34
+    rows = range(m) if rows is None else rows
+    return np.stack([canonical_ref(ref, t, w, acts[r * arb:(r + 1) * arb], n, k_, threads=16) for r in rows])
+
+
+@pytest.mark.parametrize("shape", [(8, 32, 256), (33, 100, 1024), (128, 160, 512), (200, 257, 1024), (64, 64, 4096),
+                                   (130, 129, 2048)], ids=lambda s: "x".join(map(str, s)))
+def test_prefill_tile_kernel_q4k(hip, ref, shape):
+    """Q4_K x Q8_0 int8-MFMA tile kernel: integer sub-block sums bit-exact, fp32 within 1e-5,
+    ragged tile edges in both directions, overwrite and accumulate."""
+    import torch
+    m, n, k_ = shape
+    t = O.Q4_K
+    say("prefill", shape)
+    w = synth.weights(t, 600 + m, n, k_)
+    x = synth.normal_f32(700 + n, m * k_)
+    acts = ref.quantize_q8_0(x)
+    kern = hip.HipKernel(t)
+    ws_bytes = kern.gemm_workspace_bytes(m, n, k_)
+    assert ws_bytes > 0
+    dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    dy = torch.full((m, n), 7.0, dtype=torch.float32, device="cuda")
+    kern.gemm_q8_dev(dw, da, dy, m, n, k_, accumulate=False, workspace=ws)
+    torch.cuda.synchronize()
+    y_ref = _oracle_prefill(ref, t, w, acts, m, n, k_)
+    assert_close(dy.cpu().numpy(), y_ref, f"prefill {shape}")
+    # accumulate adds the same values to what is there; library-owned scratch gives the same bits
+    dy2 = dy.clone()
+    kern.gemm_q8_dev(dw, da, dy2, m, n, k_, accumulate=True, workspace=None)
+    torch.cuda.synchronize()
+    assert torch.equal(dy2, dy + dy)
+    # exact integer sums of every (token, weight row, sub-block)
+    dsum = torch.empty((m, n, k_ // 32), dtype=torch.int32, device="cuda")
+    dy3 = torch.empty_like(dy)
+    kern.gemm_block_sums_dev(dw, da, dy3, dsum, m, n, k_, workspace=ws)
+    torch.cuda.synchronize()
+    arb = k_ // 32 * 34
+    want = np.stack([ref.block_sums(t, w, acts[r * arb:(r + 1) * arb], n, k_) for r in range(m)])
+    assert np.array_equal(dsum.cpu().numpy(), want)
+    assert torch.equal(dy3, dy)
+
+
+def test_prefill_full_size_c4(hip, ref):
+    """C4: 512 tokens x Q4_K 14336 x 4096.  Oracle on every 16th token (all 14336 outputs each)."""
+    import torch
+    m, n, k_, t = 512, 14336, 4096, O.Q4_K
+    w = synth.weights(t, 31, n, k_)
+    x = synth.normal_f32(32, m * k_)
+    kern = hip.HipKernel(t)
+    dw, dx = torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda()
+    da = torch.empty(m * (k_ // 32 * 34), dtype=torch.uint8, device="cuda")
+    hip.quantize_q8_0_dev(dx, da)
+    acts = ref.quantize_q8_0(x)
+    assert np.array_equal(da.cpu().numpy(), acts)  # row-wise Q8_0 bytes bit-exact
+    ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
+    dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    kern.gemm_q8_dev(dw, da, dy, m, n, k_, accumulate=False, workspace=ws)
+    torch.cuda.synchronize()
+    rows = list(range(0, m, 16)) + [m - 1]
+    y_ref = _oracle_prefill(ref, t, w, acts, m, n, k_, rows=rows)
+    assert_close(dy.cpu().numpy()[rows], y_ref, "C4 prefill")
+    # every token row also equals the batch-1 fused matvec of the same activations, to fp32 order
+    yv = torch.zeros(n, dtype=torch.float32, device="cuda")
+    arb = k_ // 32 * 34
+    for r in (1, 255, 510):
+        yv.zero_()
+        kern.matvec_q8_fused_dev(dw, da[r * arb:(r + 1) * arb], yv, n, k_, accumulate=False)
+        torch.cuda.synchronize()
+        assert_close(dy[r].cpu().numpy(), yv.cpu().numpy(), f"row {r} vs matvec")
+
+
 # ---- (7) residency helpers -----------------------------------------------------------------
 
 def test_registered_weights_and_cache(hip, ref):
