@@ -203,6 +203,8 @@ int oxq_set_gemv_rows_per_batch(unsigned rows);
 /* Waves that share one row in the GEMV kernels (1 or 4; tuning knob; 0 restores the
  * per-shape default: 4 for rows of three or more 64-unit steps). */
 int oxq_set_gemv_waves_per_row(unsigned waves);
+/* Tile shape / prefetch depth of the prefill kernel (tuning knob; 0 restores the default). */
+int oxq_set_gemm_variant(int variant);
 
 #ifdef __cplusplus
 }

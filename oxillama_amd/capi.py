@@ -82,6 +82,7 @@ SIGNATURES = {
     "oxq_set_gemv_waves_per_cu": (C.c_int, [C.c_uint]),
     "oxq_set_gemv_rows_per_batch": (C.c_int, [C.c_uint]),
     "oxq_set_gemv_waves_per_row": (C.c_int, [C.c_uint]),
+    "oxq_set_gemm_variant": (C.c_int, [C.c_int]),
 }
 
 _lib = None

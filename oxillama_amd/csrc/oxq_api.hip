@@ -11,6 +11,7 @@
 #include "oxq_internal.hpp"
 
 namespace oxq {
+extern int g_gemm_variant;
 hipError_t launch_dequant(uint32_t type, const uint8_t *blocks, size_t n_blocks, float *out, hipStream_t stream);
 }
 
@@ -361,6 +362,11 @@ int oxq_set_gemv_rows_per_batch(unsigned rows) {
 int oxq_set_gemv_waves_per_row(unsigned waves) {
     std::lock_guard<std::mutex> lock(g.mu);
     g.waves_per_row = waves >= 4 ? 4 : (waves ? 1 : 0);
+    return OXQ_OK;
+}
+
+int oxq_set_gemm_variant(int variant) {
+    oxq::g_gemm_variant = variant;
     return OXQ_OK;
 }
 

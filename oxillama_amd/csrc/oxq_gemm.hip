@@ -66,12 +66,14 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
     da16[(size_t)j * mpad + t] = (uint16_t)dbits;
 }
 
-// Work group = 4 waves as 2 (tokens) x 2 (weight rows); each wave owns a 64 x 64 tile
-// = 2 x 2 MFMA tiles of 32 x 32.  Lane l: c = l % 32 is the token (A operand) /
+// Work group = 4 waves as 2 (tokens) x 2 (weight rows); each wave owns a 64 x (32*NT)
+// tile = 2 x NT MFMA tiles of 32 x 32.  Lane l: c = l % 32 is the token (A operand) /
 // weight row (B operand) / output column it feeds, h = l / 32 the 16-byte half of
 // the 32-byte block.  C layout of the 32x32 MFMAs: register v of lane l holds row
 // 8*(v/4) + 4*h + v%4 (token), column c (weight row).
-template <bool DUMP>
+// Operands are fetched DIST 64-column groups ahead into a ring of register slots
+// (DIST divides 4, so the slot of a group is fixed at compile time).
+template <int NT, int DIST, bool DUMP>
 __global__ __launch_bounds__(256) void gemm_q4k_q8_kernel(const uint8_t *__restrict__ W,
                                                          const uint8_t *__restrict__ q8t,
                                                          const float *__restrict__ P,
@@ -79,12 +81,13 @@ __global__ __launch_bounds__(256) void gemm_q4k_q8_kernel(const uint8_t *__restr
                                                          float *__restrict__ out, int32_t *__restrict__ sums,
                                                          uint32_t m, uint32_t mpad, uint32_t n, uint32_t k,
                                                          int accumulate) {
+    static_assert(DIST == 1 || DIST == 2 || DIST == 4, "prefetch distance in groups");
     extern __shared__ uint16_t lds_da[];  // [nsb][4 m-tiles][2 halves][16] f16 token scales of this work group
-    const uint32_t nsb = k / 32, nblk = k / 256;
+    const uint32_t nsb = k / 32, nblk = k / 256, ngrp = nblk * 4;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
     const uint32_t wm = wave & 1, wn = wave >> 1;
-    const uint32_t m_wg = blockIdx.x * 128, n_wave = blockIdx.y * 128 + wn * 64;
+    const uint32_t m_wg = blockIdx.x * 128, n_wave = blockIdx.y * (64 * NT) + wn * (32 * NT);
     const uint32_t m_wave = m_wg + wm * 64;
 
     // Token scales of the 128 tokens of this work group, permuted so that the 16 values a
@@ -97,83 +100,107 @@ __global__ __launch_bounds__(256) void gemm_q4k_q8_kernel(const uint8_t *__restr
     }
     __syncthreads();
 
-    v16f acc[2][2], acc2[2][2];
+    v16f acc[2][NT], acc2[2][NT];
     v16i magic;
     for (int i = 0; i < 16; i++) magic[i] = (int)MAGIC_BITS;
     for (int a = 0; a < 2; a++)
-        for (int b = 0; b < 2; b++)
+        for (int b = 0; b < NT; b++)
             for (int i = 0; i < 16; i++) {
                 acc[a][b][i] = 0.0f;
                 acc2[a][b][i] = 0.0f;
             }
 
     // rows past n are clamped for loads and masked at the store
-    uint32_t nrow[2];
-    const uint8_t *wrow[2];
-    for (int nt = 0; nt < 2; nt++) {
+    uint32_t nrow[NT];
+    const uint8_t *wrow[NT];
+    for (int nt = 0; nt < NT; nt++) {
         nrow[nt] = n_wave + nt * 32 + c;
         wrow[nt] = W + (size_t)min(nrow[nt], n - 1) * nblk * 144;
     }
     const uint32_t mtok[2] = {m_wave + c, m_wave + 32 + c};  // always < mpad
 
-    for (uint32_t blk = 0; blk < nblk; blk++) {
-        // scales of this super-block for the lane's two weight rows (decode_scales_mins,
-        // reference/q4_k.rs:27-49)
-        float dsc[2][8], nc2[2][8], qneg[2][8];
-        for (int nt = 0; nt < 2; nt++) {
-            const u32x4 hd = ld16(wrow[nt] + (size_t)blk * 144);
-            const float d = h2f(hd[0] & 0xFFFF), dmin = h2f(hd[0] >> 16);
+    struct Slot {
+        u32x4 qs[NT];     // 16 nibble bytes per weight row: low nibbles -> sub-block 2g, high -> 2g+1
+        u32x4 aop[2][2];  // [half][mt] 16 activation bytes
+        float pv[2];      // P of sub-block 2g + h
+    };
+    Slot slot[DIST];
+    u32x4 hdr[NT];
+    // group index G = 4*blk + g; groups past the end re-read the last one (result unused)
+    auto fill = [&](Slot &sl, uint32_t G) {
+        G = min(G, ngrp - 1);
+        const uint32_t blk = G >> 2, g = G & 3;
+        for (int nt = 0; nt < NT; nt++) sl.qs[nt] = ld16(wrow[nt] + (size_t)blk * 144 + 16 + 32 * g + 16 * h);
+        for (int half = 0; half < 2; half++)
+            for (int mt = 0; mt < 2; mt++)
+                sl.aop[half][mt] = *reinterpret_cast<const u32x4 *>(
+                    q8t + ((size_t)(2 * G + half) * mpad + mtok[mt]) * 32 + 16 * h);
+        for (int mt = 0; mt < 2; mt++) sl.pv[mt] = P[(size_t)(2 * G + h) * mpad + mtok[mt]];
+    };
+    for (int nt = 0; nt < NT; nt++) hdr[nt] = ld16(wrow[nt]);
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                uint32_t sc, mn;
-                if (s < 4) {
-                    sc = (hd[1] >> (8 * s)) & 63;
-                    mn = (hd[2] >> (8 * s)) & 63;
-                } else {
-                    sc = ((hd[3] >> (8 * (s - 4))) & 15) | (((hd[1] >> (8 * (s - 4) + 6)) & 3) << 4);
-                    mn = ((hd[3] >> (8 * (s - 4) + 4)) & 15) | (((hd[2] >> (8 * (s - 4) + 6)) & 3) << 4);
-                }
-                dsc[nt][s] = d * (float)sc;            // reference/q4_k.rs:280, exact
-                nc2[nt][s] = -(MAGIC_F * dsc[nt][s]);  // exact
-                qneg[nt][s] = -(dmin * (float)mn);     // reference/q4_k.rs:281, exact
-            }
+    for (int g = 0; g < DIST; g++) fill(slot[g], g);
+
+    for (uint32_t blk = 0; blk < nblk; blk++) {
+        const uint32_t nxt = min(blk + 1, nblk - 1);  // last trip: harmless re-read
+        u32x4 hd[NT];
+        for (int nt = 0; nt < NT; nt++) {
+            hd[nt] = hdr[nt];
+            hdr[nt] = ld16(wrow[nt] + (size_t)nxt * 144);
         }
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            // 16 nibble bytes per weight row: low nibbles -> sub-block 2g, high -> 2g+1
-            v4i blo[2], bhi[2];
-            for (int nt = 0; nt < 2; nt++) {
-                const u32x4 q = ld16(wrow[nt] + (size_t)blk * 144 + 16 + 32 * g + 16 * h);
+            Slot &sl = slot[g % DIST];
+            v4i blo[NT], bhi[NT];
+            for (int nt = 0; nt < NT; nt++)
                 for (int i = 0; i < 4; i++) {
-                    blo[nt][i] = (int)(q[i] & 0x0F0F0F0Fu);
-                    bhi[nt][i] = (int)((q[i] >> 4) & 0x0F0F0F0Fu);
+                    blo[nt][i] = (int)(sl.qs[nt][i] & 0x0F0F0F0Fu);
+                    bhi[nt][i] = (int)((sl.qs[nt][i] >> 4) & 0x0F0F0F0Fu);
+                }
+            v4i aop[2][2];
+            for (int half = 0; half < 2; half++)
+                for (int mt = 0; mt < 2; mt++)
+                    for (int i = 0; i < 4; i++) aop[half][mt][i] = (int)sl.aop[half][mt][i];
+            const float pv[2] = {sl.pv[0], sl.pv[1]};
+            fill(sl, blk * 4 + g + DIST);  // slot consumed: refill it DIST groups ahead
+            // scales of sub-blocks 2g, 2g+1 for the lane's weight rows (decode_scales_mins,
+            // reference/q4_k.rs:27-49)
+            float dsc[NT][2], nc2[NT][2], qneg[NT][2];
+            for (int nt = 0; nt < NT; nt++) {
+                const float d = h2f(hd[nt][0] & 0xFFFF), dmin = h2f(hd[nt][0] >> 16);
+#pragma unroll
+                for (int half = 0; half < 2; half++) {
+                    const int s = 2 * g + half;
+                    uint32_t sc, mn;
+                    if (s < 4) {
+                        sc = (hd[nt][1] >> (8 * s)) & 63;
+                        mn = (hd[nt][2] >> (8 * s)) & 63;
+                    } else {
+                        sc = ((hd[nt][3] >> (8 * (s - 4))) & 15) | (((hd[nt][1] >> (8 * (s - 4) + 6)) & 3) << 4);
+                        mn = ((hd[nt][3] >> (8 * (s - 4) + 4)) & 15) | (((hd[nt][2] >> (8 * (s - 4) + 6)) & 3) << 4);
+                    }
+                    dsc[nt][half] = d * (float)sc;               // reference/q4_k.rs:280, exact
+                    nc2[nt][half] = -(MAGIC_F * dsc[nt][half]);  // exact
+                    qneg[nt][half] = -(dmin * (float)mn);        // reference/q4_k.rs:281, exact
                 }
             }
 #pragma unroll
             for (int half = 0; half < 2; half++) {
-                const int s = 2 * g + half;
-                const uint32_t j = blk * 8 + s;
-                v4i aop[2];
-                u32x4 dav[2][2];
+                const uint32_t j = blk * 8 + 2 * g + half;
+                v16i dres[2][NT];
+                for (int mt = 0; mt < 2; mt++)
+                    for (int nt = 0; nt < NT; nt++)
+                        dres[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop[half][mt], half ? bhi[nt] : blo[nt], magic, 0, 0, 0);
                 for (int mt = 0; mt < 2; mt++) {
-                    const u32x4 av = *reinterpret_cast<const u32x4 *>(q8t + ((size_t)j * mpad + mtok[mt]) * 32 + 16 * h);
-                    for (int i = 0; i < 4; i++) aop[mt][i] = (int)av[i];
                     const u32x4 *dp = reinterpret_cast<const u32x4 *>(&lds_da[((j * 4 + wm * 2 + mt) * 2 + h) * 16]);
-                    dav[mt][0] = dp[0];
-                    dav[mt][1] = dp[1];
-                }
-                v16i dres[2][2];
-                for (int mt = 0; mt < 2; mt++)
-                    for (int nt = 0; nt < 2; nt++)
-                        dres[mt][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aop[mt], half ? bhi[nt] : blo[nt], magic, 0, 0, 0);
-                for (int mt = 0; mt < 2; mt++)
-                    for (int nt = 0; nt < 2; nt++) {
+                    const u32x4 dav[2] = {dp[0], dp[1]};
+                    for (int nt = 0; nt < NT; nt++) {
 #pragma unroll
                         for (int i = 0; i < 16; i++) {
                             const uint32_t dbits = (uint32_t)dres[mt][nt][i];
                             // fl(dsc * I), then += * da  (da is an f16 value, exact in fp32)
-                            const float t = fmaf(__builtin_bit_cast(float, dbits), dsc[nt][s], nc2[nt][s]);
-                            const uint32_t pair = dav[mt][i >> 3][(i >> 1) & 3];
+                            const float t = fmaf(__builtin_bit_cast(float, dbits), dsc[nt][half], nc2[nt][half]);
+                            const uint32_t pair = dav[i >> 3][(i >> 1) & 3];
                             const float da = h2f((i & 1) ? (pair >> 16) : (pair & 0xFFFF));
                             acc[mt][nt][i] = fmaf(t, da, acc[mt][nt][i]);
                             if (DUMP) {
@@ -183,21 +210,19 @@ __global__ __launch_bounds__(256) void gemm_q4k_q8_kernel(const uint8_t *__restr
                             }
                         }
                     }
-            }
-            // min term of sub-blocks 2g (lanes h = 0) and 2g+1 (lanes h = 1)
-            const uint32_t jp = blk * 8 + 2 * g + h;
-            for (int mt = 0; mt < 2; mt++) {
-                const float pv = P[(size_t)jp * mpad + mtok[mt]];
-                for (int nt = 0; nt < 2; nt++) {
-                    const float qv = h ? qneg[nt][2 * g + 1] : qneg[nt][2 * g];
-                    acc2[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pv, qv, acc2[mt][nt], 0, 0, 0);
                 }
             }
+            // min term of sub-blocks 2g (lanes h = 0) and 2g+1 (lanes h = 1)
+            for (int mt = 0; mt < 2; mt++)
+                for (int nt = 0; nt < NT; nt++) {
+                    const float qv = h ? qneg[nt][1] : qneg[nt][0];
+                    acc2[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pv[mt], qv, acc2[mt][nt], 0, 0, 0);
+                }
         }
     }
 
     for (int mt = 0; mt < 2; mt++)
-        for (int nt = 0; nt < 2; nt++) {
+        for (int nt = 0; nt < NT; nt++) {
             if (nrow[nt] >= n) continue;
 #pragma unroll
             for (int i = 0; i < 16; i++) {
@@ -233,6 +258,42 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
     return hipSuccess;
 }
 
+int g_gemm_variant = 0;  // tuning: 0 = default
+
+template <int NT, int DIST>
+static hipError_t launch_tile_variant(const GemmArgs &a, const uint8_t *q8t, const float *P, const uint16_t *da16,
+                                      uint32_t mpad, size_t lds, hipStream_t stream) {
+    const dim3 grid(mpad / 128, (a.n + 64 * NT - 1) / (64 * NT));
+    hipError_t e = hipSuccess;
+    if (lds > 64 * 1024) {  // beyond the default dynamic LDS limit: opt in (up to the 160 KB of a CU)
+        e = a.sums ? hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8_kernel<NT, DIST, true>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
+                   : hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8_kernel<NT, DIST, false>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return e;
+    }
+    if (a.sums)
+        hipLaunchKernelGGL((gemm_q4k_q8_kernel<NT, DIST, true>), grid, dim3(256), lds, stream, a.W, q8t, P, da16, a.out,
+                           a.sums, a.m, mpad, a.n, a.k, a.accumulate);
+    else
+        hipLaunchKernelGGL((gemm_q4k_q8_kernel<NT, DIST, false>), grid, dim3(256), lds, stream, a.W, q8t, P, da16, a.out,
+                           a.sums, a.m, mpad, a.n, a.k, a.accumulate);
+    return hipGetLastError();
+}
+
+static hipError_t launch_tiles(const GemmArgs &a, const uint8_t *q8t, const float *P, const uint16_t *da16,
+                               uint32_t mpad, size_t lds, hipStream_t stream) {
+    switch (g_gemm_variant) {
+    case 1: return launch_tile_variant<1, 1>(a, q8t, P, da16, mpad, lds, stream);
+    case 2: return launch_tile_variant<1, 2>(a, q8t, P, da16, mpad, lds, stream);
+    case 3: return launch_tile_variant<1, 4>(a, q8t, P, da16, mpad, lds, stream);
+    case 4: return launch_tile_variant<2, 1>(a, q8t, P, da16, mpad, lds, stream);
+    case 5: return launch_tile_variant<2, 2>(a, q8t, P, da16, mpad, lds, stream);
+    case 6: return launch_tile_variant<2, 4>(a, q8t, P, da16, mpad, lds, stream);
+    default: return launch_tile_variant<1, 2>(a, q8t, P, da16, mpad, lds, stream);
+    }
+}
+
 bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t k) {
     // LDS holds the f16 token scales of 128 tokens for the whole k: k/32 * 256 bytes
     return type == OXQ_TYPE_Q4_K && m >= 8 && (size_t)(k / 32) * 256 <= 160 * 1024;
@@ -248,22 +309,8 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
                        mpad, nsb);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
-    const dim3 grid(mpad / 128, (a.n + 127) / 128);
     const size_t lds = (size_t)nsb * 256;
-    if (lds > 64 * 1024) {  // beyond the default dynamic LDS limit: opt in (up to the 160 KB of a CU)
-        e = a.sums ? hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8_kernel<true>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds)
-                   : hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_q4k_q8_kernel<false>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-    }
-    if (a.sums)
-        hipLaunchKernelGGL(gemm_q4k_q8_kernel<true>, grid, dim3(256), lds, stream, a.W, q8t, P, da16, a.out, a.sums,
-                           a.m, mpad, a.n, a.k, a.accumulate);
-    else
-        hipLaunchKernelGGL(gemm_q4k_q8_kernel<false>, grid, dim3(256), lds, stream, a.W, q8t, P, da16, a.out, a.sums,
-                           a.m, mpad, a.n, a.k, a.accumulate);
-    return hipGetLastError();
+    return launch_tiles(a, q8t, P, da16, mpad, lds, stream);
 }
 
 }  // namespace oxq
