@@ -262,7 +262,7 @@ def main():
                                  "repeats": n_1t}}
 
     out = {
-        "metric": "Q4_K/Q6_K/Q8_0 GEMV weight GB/s, Llama-3-8B decode projections (batch 1)",
+        "metric": "Q4_K GEMV weight GB/s (% HBM peak); batch-512 prefill int8-MFMA TOPS",
         "value": round(value, 1),
         "unit": "GB/s",
         "n_gpus": 1,
