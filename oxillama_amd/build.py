@@ -4,6 +4,7 @@
   * oxillama_amd/liboxq_hip.so   -- HIP kernels + C ABI (include/oxq.h), gfx950 only
   * oxillama_amd/liboxq_synth.so -- host-side synthetic weight generator
   * oxillama_amd/liboxq_benchkit.so -- copy / streaming-read kernels for measurement calibration
+  * tests/cpp/test_quant_kernel.bin -- C++ mirror of the reference interface + its replayed unit tests
 hipcc cross-compiles gfx950 code objects without a GPU present.
 """
 import os
@@ -16,6 +17,7 @@ HIP_SOURCES = ["oxq_api.hip", "oxq_gemv.hip", "oxq_gemm.hip", "oxq_quantize.hip"
 HIP_LIB = os.path.join(HERE, "liboxq_hip.so")
 SYNTH_LIB = os.path.join(HERE, "liboxq_synth.so")
 BENCHKIT_LIB = os.path.join(HERE, "liboxq_benchkit.so")
+CPP_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp", "test_quant_kernel.bin")
 
 # -ffp-contract=off: the fp32 epilogues follow the reference's operation order (Rust
 # never fuses a*b+c).  Packed fp32 instructions are switched off.
@@ -54,10 +56,22 @@ def build_benchkit():
     return BENCHKIT_LIB
 
 
+def build_cpp_tests():
+    """The C++ mirror of the reference interface (include/oxq/quant_kernel.hpp) and the
+    program that replays the reference's unit tests through it."""
+    root = os.path.dirname(HERE)
+    run(["g++", "-O1", "-std=c++17", "-Wall", "-I", os.path.join(root, "include"),
+         os.path.join(root, "tests", "cpp", "test_quant_kernel.cpp"), "-o", CPP_TEST_BIN,
+         "-L", HERE, "-loxq_hip", "-Wl,-rpath,$ORIGIN/../../oxillama_amd",
+         "-Wl,-rpath-link,/opt/rocm/lib", "-Wl,--allow-shlib-undefined"])
+    return CPP_TEST_BIN
+
+
 def build_all():
     build_hip()
     build_synth()
     build_benchkit()
+    build_cpp_tests()
 
 
 if __name__ == "__main__":

@@ -1,0 +1,438 @@
+// Replays the reference crate's own unit tests against the C++ mirror of its
+// interface (include/oxq/quant_kernel.hpp), which calls liboxq_hip.so through the C ABI.
+// Each case names the reference test it follows (Q/ = crates/oxillama-quant/src).
+//
+//   test_quant_kernel --host   metadata, error variants and validation order (no GPU work)
+//   test_quant_kernel --gpu    the numeric cases (needs an MI355X)
+//
+// Exit status 0 = all passed.  `gemv`/`gemm` of this library quantize the f32 input to
+// Q8_0 first, so their closed-form expectations hold to the Q8_0 rounding of the input
+// (|rel err| <= 2e-3 here) instead of exactly; dequant and fused cases keep the
+// reference's own tolerances.
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+#include "oxq/quant_kernel.hpp"
+
+using namespace oxq;
+
+static int g_failed = 0, g_run = 0;
+#define CHECK(cond)                                                                  \
+    do {                                                                             \
+        if (!(cond)) {                                                               \
+            std::printf("    CHECK failed %s:%d: %s\n", __FILE__, __LINE__, #cond);  \
+            ++g_failed;                                                              \
+            return;                                                                  \
+        }                                                                            \
+    } while (0)
+#define CHECK_NEAR(a, b, tol)                                                                        \
+    do {                                                                                             \
+        const double va = (a), vb = (b);                                                             \
+        if (!(std::fabs(va - vb) <= (tol))) {                                                        \
+            std::printf("    CHECK_NEAR failed %s:%d: %s = %.9g vs %s = %.9g (tol %g)\n", __FILE__,  \
+                        __LINE__, #a, va, #b, vb, (double)(tol));                                    \
+            ++g_failed;                                                                              \
+            return;                                                                                  \
+        }                                                                                            \
+    } while (0)
+
+static void run(const char *name, const std::function<void()> &fn) {
+    const int before = g_failed;
+    std::printf("test %s ... ", name);
+    std::fflush(stdout);
+    fn();
+    ++g_run;
+    std::printf("%s\n", g_failed == before ? "ok" : "FAILED");
+    std::fflush(stdout);
+}
+
+// ---- block builders (little-endian f16 scale + payload) ------------------------------
+static uint16_t f16_bits(float f) {  // exact for the scales used here (0.5, 0.25, 1, 2, 0.1 -> RNE)
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    int32_t e = (int32_t)((x >> 23) & 0xFF) - 127 + 15;
+    uint32_t m = x & 0x7FFFFFu;
+    if ((x & 0x7FFFFFFFu) == 0) return (uint16_t)sign;
+    if (e <= 0 || e >= 31) return (uint16_t)(sign | 0x7C00u);  // not needed by these tests
+    uint32_t h = (uint32_t)(e << 10) | (m >> 13);
+    const uint32_t rem = m & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) ++h;
+    return (uint16_t)(sign | h);
+}
+static float f16_value(uint16_t h) {
+    const int e = (h >> 10) & 31, m = h & 1023;
+    const float v = e == 0 ? std::ldexp((float)m, -24) : std::ldexp((float)(m + 1024), e - 25);
+    return (h & 0x8000) ? -v : v;
+}
+static void put_f16(std::vector<uint8_t> &b, size_t at, float f) {
+    const uint16_t h = f16_bits(f);
+    b[at] = (uint8_t)(h & 0xFF);
+    b[at + 1] = (uint8_t)(h >> 8);
+}
+static std::vector<uint8_t> q4_0_block(float d, const std::vector<uint8_t> &nib16) {
+    std::vector<uint8_t> b(18, 0);
+    put_f16(b, 0, d);
+    for (int i = 0; i < 16; ++i) b[2 + i] = nib16[i];
+    return b;
+}
+static std::vector<uint8_t> q8_0_block(float d, const std::vector<int> &q32) {
+    std::vector<uint8_t> b(34, 0);
+    put_f16(b, 0, d);
+    for (int i = 0; i < 32; ++i) b[2 + i] = (uint8_t)(int8_t)q32[i];
+    return b;
+}
+static std::vector<uint8_t> q4_k_block(float d, float dmin, const std::vector<uint8_t> &scales12, uint8_t qs_fill) {
+    std::vector<uint8_t> b(144, 0);
+    put_f16(b, 0, d);
+    put_f16(b, 2, dmin);
+    for (int i = 0; i < 12; ++i) b[4 + i] = scales12[i];
+    for (int i = 0; i < 128; ++i) b[16 + i] = qs_fill;
+    return b;
+}
+static void append(std::vector<uint8_t> &dst, const std::vector<uint8_t> &src) {
+    dst.insert(dst.end(), src.begin(), src.end());
+}
+// Dequantized Q8_0 activations: q * d_a (the "unfused" operand of the reference's comparisons).
+static std::vector<float> dequant_acts(const std::vector<uint8_t> &acts) {
+    std::vector<float> x;
+    for (size_t b = 0; b + 34 <= acts.size(); b += 34) {
+        const float d = f16_value((uint16_t)(acts[b] | (acts[b + 1] << 8)));
+        for (int i = 0; i < 32; ++i) x.push_back((float)(int8_t)acts[b + 2 + i] * d);
+    }
+    return x;
+}
+// Unfused expectation as the reference's tests build it: dequant_block each weight block, dot in f32.
+static float unfused_row(const QuantKernel &k, const uint8_t *row, size_t n_cols, const std::vector<float> &x) {
+    const size_t bs = k.block_size(), bb = k.block_bytes();
+    std::vector<float> w(bs);
+    float sum = 0.0f;
+    for (size_t b = 0; b < n_cols / bs; ++b) {
+        if (!k.dequant_block(Slice<const uint8_t>(row + b * bb, bb), w)) return NAN;
+        for (size_t i = 0; i < bs; ++i) sum += w[i] * x[b * bs + i];
+    }
+    return sum;
+}
+
+static const std::vector<int> Q8_ALT16 = {1, -2, 3, -4, 5, -6, 7, -8, 9, -10, 11, -12, 13, -14, 15, -16,
+                                          -1, 2, -3, 4, -5, 6, -7, 8, -9, 10, -11, 12, -13, 14, -15, 16};
+static const std::vector<uint8_t> NIB_A = {0x5A, 0xF0, 0x13, 0x7E, 0xC2, 0x48, 0x9D, 0x6B,
+                                           0xA3, 0x2F, 0x71, 0xE4, 0x0C, 0x58, 0xB6, 0xD9};
+
+// ======================================================================================
+//  host-only cases
+// ======================================================================================
+static void host_tests() {
+    KernelDispatcher dispatcher;  // may have no device here; metadata and validation still work
+
+    run("block_info_matches_gguf_tables (gguf/src/types.rs:199-262)", [&] {
+        struct { GgufTensorType t; size_t bs, bb; } rows[] = {{GgufTensorType::Q4_0, 32, 18},
+                                                              {GgufTensorType::Q8_0, 32, 34},
+                                                              {GgufTensorType::Q4K, 256, 144},
+                                                              {GgufTensorType::Q6K, 256, 210},
+                                                              {GgufTensorType::Iq4Xs, 256, 136}};
+        for (auto &r : rows) {
+            HipKernel k(r.t);
+            CHECK(k.block_size() == r.bs);
+            CHECK(k.block_bytes() == r.bb);
+            CHECK(k.name() != nullptr && std::strlen(k.name()) > 0);
+        }
+    });
+
+    run("dispatcher_unknown_type_is_unsupported (Q/dispatch.rs:236-242)", [&] {
+        std::unique_ptr<QuantKernel> k;
+        const QuantResult r = dispatcher.get_kernel(999u, k);
+        CHECK(r.is_err());
+        CHECK(r.error().kind == QuantError::UnsupportedType);
+        CHECK(!k);
+        CHECK(dispatcher.get_kernel(GgufTensorType::Q4K, k).is_ok());
+        CHECK(k && k->block_size() == 256);
+    });
+
+    run("quant_tensor_bookkeeping (Q/types.rs:30-50)", [&] {
+        QuantTensor t(std::vector<uint8_t>(4 * 144), {2, 512}, GgufTensorType::Q4K);
+        CHECK(t.n_elements() == 1024);
+        CHECK(t.n_blocks() == 4);
+        CHECK(t.expected_data_size() == 4 * 144);
+        QuantTensor e({}, {}, GgufTensorType::Q8_0);
+        CHECK(e.n_elements() == 0 && e.n_blocks() == 0);
+    });
+
+    run("quantize_q8_0_rejects_unaligned_length (Q/quantize.rs:59-64,307-317)", [&] {
+        std::vector<float> x(33, 1.0f);
+        std::vector<uint8_t> out;
+        const QuantResult r = quantize_f32_to_q8_0(x, out);
+        CHECK(r.is_err());
+        CHECK(r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 64 && r.error().got == 33);
+        CHECK(r.error().to_string() == "dimension mismatch: expected 64, got 33");
+    });
+
+    run("fused_validation_order: out, weights, acts (Q/reference/q4_k.rs:226-250)", [&] {
+        HipKernel k(GgufTensorType::Q4K);
+        std::vector<uint8_t> w(2 * 144), a(8 * 34);
+        std::vector<float> out(2);
+        // everything too small: the output check fires first
+        QuantResult r = k.matvec_q8_fused(Slice<const uint8_t>(w.data(), 10), Slice<const uint8_t>(a.data(), 10),
+                                          Slice<float>(out.data(), 1), 2, 256);
+        CHECK(r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 2 && r.error().got == 1);
+        // output fine: weights next
+        r = k.matvec_q8_fused(Slice<const uint8_t>(w.data(), 287), Slice<const uint8_t>(a.data(), 10), out, 2, 256);
+        CHECK(r.error().kind == QuantError::BufferTooSmall);
+        CHECK(r.error().expected == 288 && r.error().got == 287);
+        // then activations: 8 Q8_0 blocks per super-block
+        r = k.matvec_q8_fused(w, Slice<const uint8_t>(a.data(), 271), out, 2, 256);
+        CHECK(r.error().kind == QuantError::BufferTooSmall);
+        CHECK(r.error().expected == 272 && r.error().got == 271);
+        CHECK(r.error().to_string() == "buffer too small: need 272 bytes, have 271");
+    });
+
+    run("gemv_dimension_checks: input then output (Q/reference/q4_k.rs:117-128)", [&] {
+        HipKernel k(GgufTensorType::Q8_0);
+        QuantTensor t(std::vector<uint8_t>(2 * 34), {2, 32}, GgufTensorType::Q8_0);
+        std::vector<float> x(31), y(1);
+        QuantResult r = k.gemv(t, x, y);
+        CHECK(r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 32 && r.error().got == 31);
+        x.resize(32);
+        r = k.gemv(t, x, y);
+        CHECK(r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 2 && r.error().got == 1);
+    });
+
+    run("dequant_block_buffer_checks (Q/reference/q4_k.rs:53-64)", [&] {
+        HipKernel k(GgufTensorType::Q6K);
+        std::vector<uint8_t> b(209);
+        std::vector<float> o(256);
+        QuantResult r = k.dequant_block(b, o);
+        CHECK(r.error().kind == QuantError::BufferTooSmall);
+        CHECK(r.error().expected == 210 && r.error().got == 209);
+        b.resize(210);
+        o.resize(255);
+        r = k.dequant_block(b, o);
+        CHECK(r.error().kind == QuantError::BufferTooSmall);
+        CHECK(r.error().expected == 256 && r.error().got == 255);
+    });
+}
+
+// ======================================================================================
+//  GPU cases
+// ======================================================================================
+static void gpu_tests() {
+    KernelDispatcher dispatcher;
+    if (!dispatcher.has_device()) {
+        std::printf("no usable GPU: oxq_init failed\n");
+        ++g_failed;
+        return;
+    }
+    auto kernel = [&](GgufTensorType t) {
+        std::unique_ptr<QuantKernel> k;
+        dispatcher.get_kernel(t, k);
+        return k;
+    };
+
+    run("q4_0 dequant_known_values (Q/reference/q4_0.rs:259-270)", [&] {
+        auto k = kernel(GgufTensorType::Q4_0);
+        std::vector<uint8_t> nib(16, 0x88);
+        nib[0] = 0xF0;
+        auto b = q4_0_block(0.5f, nib);
+        std::vector<float> w(32, 99.0f);
+        CHECK(k->dequant_block(b, w).is_ok());
+        CHECK(w[0] == -4.0f);  // (0 - 8) * 0.5
+        CHECK(w[1] == 3.5f);   // (15 - 8) * 0.5
+        for (int i = 2; i < 32; ++i) CHECK(w[i] == 0.0f);
+    });
+
+    run("q8_0 dequant_known_values (Q/reference/q8_0.rs:159-172)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        std::vector<int> q(32, 0);
+        q[0] = 10; q[1] = -5; q[31] = 127;
+        auto b = q8_0_block(0.5f, q);
+        std::vector<float> w(32);
+        CHECK(k->dequant_block(b, w).is_ok());
+        CHECK(w[0] == 5.0f && w[1] == -2.5f && w[31] == 63.5f);
+    });
+
+    run("q8_0 gemv_simple 1*2.0*3.0 (Q/reference/q8_0.rs:175-190)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        std::vector<int> q(32, 0);
+        q[0] = 1;
+        QuantTensor t(q8_0_block(2.0f, q), {1, 32}, GgufTensorType::Q8_0);
+        std::vector<float> x(32, 0.0f), y(1, -1.0f);
+        x[0] = 3.0f;
+        CHECK(k->gemv(t, x, y).is_ok());
+        CHECK_NEAR(y[0], 6.0, 6.0 * 2e-3);
+    });
+
+    run("q8_0 gemm two rows 4*0.5*3 (Q/reference/q8_0.rs:216-232)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        std::vector<int> q(32, 0);
+        q[0] = 4;
+        QuantTensor t(q8_0_block(0.5f, q), {1, 32}, GgufTensorType::Q8_0);
+        std::vector<float> x(64, 0.0f), y(2, -1.0f);
+        x[0] = 3.0f;
+        x[32] = -3.0f;
+        CHECK(k->gemm(t, x, y, 2, 1, 32).is_ok());
+        CHECK_NEAR(y[0], 6.0, 6.0 * 2e-3);
+        CHECK_NEAR(y[1], -6.0, 6.0 * 2e-3);
+    });
+
+    run("q4_k dequant all 8.0 (Q/reference/q4_k.rs:381-408)", [&] {
+        auto k = kernel(GgufTensorType::Q4K);
+        auto b = q4_k_block(1.0f, 0.0f, {1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1}, 0x88);
+        std::vector<float> w(256);
+        CHECK(k->dequant_block(b, w).is_ok());
+        for (float v : w) CHECK(v == 8.0f);
+    });
+
+    run("q4_k gemv ones = 256 (Q/reference/q4_k.rs:411-436)", [&] {
+        auto k = kernel(GgufTensorType::Q4K);
+        QuantTensor t(q4_k_block(1.0f, 0.0f, {1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1}, 0x11), {1, 256},
+                      GgufTensorType::Q4K);
+        std::vector<float> x(256, 1.0f), y(1);
+        CHECK(k->gemv(t, x, y).is_ok());
+        CHECK_NEAR(y[0], 256.0, 256.0 * 2e-3);
+    });
+
+    run("q6_k zero block and qh=0xAA (Q/reference/q6_k.rs:369-414)", [&] {
+        auto k = kernel(GgufTensorType::Q6K);
+        std::vector<uint8_t> b(210, 0);
+        std::vector<float> w(256, 1.0f);
+        CHECK(k->dequant_block(b, w).is_ok());
+        for (float v : w) CHECK(v == 0.0f);
+        for (int i = 0; i < 64; ++i) b[128 + i] = 0xAA;  // every q6 = 32 -> q - 32 = 0
+        for (int i = 0; i < 16; ++i) b[192 + i] = 1;
+        put_f16(b, 208, 1.0f);
+        CHECK(k->dequant_block(b, w).is_ok());
+        for (float v : w) CHECK(v == 0.0f);
+    });
+
+    run("iq4_xs ls=33, qs=0x88: first 32 weights 1.0 (Q/reference/iq4_xs.rs:266-285)", [&] {
+        auto k = kernel(GgufTensorType::Iq4Xs);
+        std::vector<uint8_t> b(136, 0);
+        put_f16(b, 0, 1.0f);
+        // sub-block 0: ls = 33 -> low nibble 1 in scales_l[0], high bits 2 in scales_h bits 0..1;
+        // every other sub-block: ls = 32 (low 0, high 2) -> scale 0
+        uint16_t sh = 0;
+        for (int i = 0; i < 8; ++i) sh |= (uint16_t)(2u << (2 * i));
+        b[2] = (uint8_t)(sh & 0xFF);
+        b[3] = (uint8_t)(sh >> 8);
+        b[4] = 0x01;
+        for (int i = 0; i < 128; ++i) b[8 + i] = 0x88;  // kvalues[8] = 1
+        std::vector<float> w(256);
+        CHECK(k->dequant_block(b, w).is_ok());
+        for (int i = 0; i < 32; ++i) CHECK(w[i] == 1.0f);
+        for (int i = 32; i < 256; ++i) CHECK(w[i] == 0.0f);
+    });
+
+    run("q4_0 fused accumulates: preset 42 survives zero acts (Q/reference/q4_0.rs:382-420)", [&] {
+        auto k = kernel(GgufTensorType::Q4_0);
+        auto w = q4_0_block(0.25f, NIB_A);
+        auto a = q8_0_block(0.5f, std::vector<int>(32, 0));
+        std::vector<float> out(1, 42.0f);
+        CHECK(k->matvec_q8_fused(w, a, out, 1, 32).is_ok());
+        CHECK(out[0] == 42.0f);
+    });
+
+    run("q4_k fused accumulates: preset 77 (Q/reference/q4_k.rs:474-493)", [&] {
+        auto k = kernel(GgufTensorType::Q4K);
+        auto w = q4_k_block(1.0f, 0.0f, {1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1}, 0x11);
+        std::vector<uint8_t> a;
+        for (int i = 0; i < 8; ++i) append(a, q8_0_block(0.5f, std::vector<int>(32, 0)));
+        std::vector<float> out(1, 77.0f);
+        CHECK(k->matvec_q8_fused(w, a, out, 1, 256).is_ok());
+        CHECK(out[0] == 77.0f);
+    });
+
+    run("q4_0 fused matches unfused, single block (Q/reference/q4_0.rs:423-464)", [&] {
+        auto k = kernel(GgufTensorType::Q4_0);
+        auto w = q4_0_block(0.25f, NIB_A);
+        auto a = q8_0_block(0.5f, Q8_ALT16);
+        std::vector<float> out(1, 0.0f);
+        CHECK(k->matvec_q8_fused(w, a, out, 1, 32).is_ok());
+        CHECK_NEAR(out[0], unfused_row(*k, w.data(), 32, dequant_acts(a)), 1e-3);
+    });
+
+    run("q4_k fused matches unfused, mixed scales (Q/reference/q4_k.rs:496-559)", [&] {
+        auto k = kernel(GgufTensorType::Q4K);
+        auto w = q4_k_block(0.5f, 0.1f, {5, 3, 7, 2, 4, 6, 1, 3, 9, 11, 13, 15}, 0xA5);
+        std::vector<uint8_t> a;
+        for (int i = 0; i < 8; ++i) append(a, q8_0_block(0.25f, Q8_ALT16));
+        std::vector<float> out(1, 0.0f);
+        CHECK(k->matvec_q8_fused(w, a, out, 1, 256).is_ok());
+        const float want = unfused_row(*k, w.data(), 256, dequant_acts(a));
+        CHECK_NEAR(out[0], want, 1e-3 * std::fmax(1.0, std::fabs(want)));
+    });
+
+    run("q4_k fused multi-row matches unfused (Q/reference/q4_k.rs:562-625)", [&] {
+        auto k = kernel(GgufTensorType::Q4K);
+        std::vector<uint8_t> w, a;
+        for (float s : {0.5f, 1.0f, 0.25f, 0.1f}) append(w, q4_k_block(s, 0.0f, {1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1}, 0x55));
+        const std::vector<int> q = {2, -1, 4, -3, 6, -5, 8, -7, 1, -2, 3, -4, 5, -6, 7, -8,
+                                    -2, 1, -4, 3, -6, 5, -8, 7, -1, 2, -3, 4, -5, 6, -7, 8};
+        for (int i = 0; i < 8; ++i) append(a, q8_0_block(0.5f, q));
+        std::vector<float> out(4, 0.0f);
+        CHECK(k->matvec_q8_fused(w, a, out, 4, 256).is_ok());
+        const auto x = dequant_acts(a);
+        for (int r = 0; r < 4; ++r) CHECK_NEAR(out[r], unfused_row(*k, w.data() + r * 144, 256, x), 1e-3);
+    });
+
+    run("q6_k fused matches unfused on the pattern block (Q/simd/avx2/q6_k.rs:939-980)", [&] {
+        auto k = kernel(GgufTensorType::Q6K);
+        std::vector<uint8_t> w(210);
+        for (int i = 0; i < 128; ++i) w[i] = (uint8_t)((i * 5 + 11) & 0xFF);
+        for (int i = 0; i < 64; ++i) w[128 + i] = (uint8_t)((i * 13 + 7) & 0xFF);
+        for (int i = 0; i < 16; ++i) w[192 + i] = (uint8_t)(i + 1);
+        put_f16(w, 208, 0.01f);
+        const std::vector<int> q = {1, -2, 3, -4, 5, -6, 7, -8, 9, -10, 11, -12, 13, -14, 15, -16,
+                                    0, 1, -1, 2, -2, 3, -3, 4, -4, 5, -5, 6, -6, 7, -7, 8};
+        std::vector<uint8_t> a;
+        for (int i = 0; i < 8; ++i) append(a, q8_0_block(0.1f, q));
+        std::vector<float> out(1, 0.0f);
+        CHECK(k->matvec_q8_fused(w, a, out, 1, 256).is_ok());
+        CHECK_NEAR(out[0], unfused_row(*k, w.data(), 256, dequant_acts(a)), 1e-3);
+    });
+
+    run("quantize_q8_0: max maps to +-127, zero block (Q/quantize.rs:320-379)", [&] {
+        std::vector<float> x(64, 0.0f);
+        for (int i = 0; i < 32; ++i) x[i] = (float)(i - 16) * 0.25f;  // extreme = -4.0 at i = 0
+        std::vector<uint8_t> out;
+        CHECK(quantize_f32_to_q8_0(x, out).is_ok());
+        CHECK(out.size() == 68);
+        CHECK((int8_t)out[2] == -127);
+        for (int i = 0; i < 34; ++i) CHECK(out[34 + i] == 0);  // all-zero block: d = 0, q = 0
+    });
+
+    run("gemv equals quantize + fused into zeros, bit for bit", [&] {
+        auto k = kernel(GgufTensorType::Q4K);
+        std::vector<uint8_t> w;
+        for (float s : {0.5f, 1.0f, 0.25f}) append(w, q4_k_block(s, 0.1f, {5, 3, 7, 2, 4, 6, 1, 3, 9, 11, 13, 15}, 0xA5));
+        QuantTensor t(w, {3, 256}, GgufTensorType::Q4K);
+        std::vector<float> x(256), y(3, -1.0f), z(3, 0.0f);
+        for (int i = 0; i < 256; ++i) x[i] = std::sin(0.37f * (float)i);
+        CHECK(k->gemv(t, x, y).is_ok());
+        std::vector<uint8_t> a;
+        CHECK(quantize_f32_to_q8_0(x, a).is_ok());
+        CHECK(k->matvec_q8_fused(w, a, z, 3, 256).is_ok());
+        for (int r = 0; r < 3; ++r) CHECK(y[r] == z[r]);
+    });
+}
+
+int main(int argc, char **argv) {
+    const std::string mode = argc > 1 ? argv[1] : "--host";
+    if (mode == "--host") {
+        host_tests();
+    } else if (mode == "--gpu") {
+        gpu_tests();
+    } else {
+        std::printf("usage: %s --host | --gpu\n", argv[0]);
+        return 2;
+    }
+    std::printf("%d cases, %d failed\n", g_run, g_failed);
+    return g_failed == 0 ? 0 : 1;
+}
