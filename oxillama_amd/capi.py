@@ -7,7 +7,7 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "liboxq_hip.so")
+LIB_PATH = os.environ.get("OXQ_HIP_LIB") or os.path.join(HERE, "liboxq_hip.so")
 
 OK = 0
 ERR_UNSUPPORTED_TYPE = 1
