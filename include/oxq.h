@@ -175,7 +175,7 @@ int oxq_matvec_q8_fused_dev(uint32_t type, const uint8_t *d_weights, const uint8
 
 /* Prefill: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched form
  * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  Q4_K with
- * m >= 8 uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()
+ * m >= 8 (and IQ4_XS likewise) uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()
  * bytes of 256-byte-aligned device scratch: pass it and the call is asynchronous
  * and allocation-free; pass NULL and the library uses its own scratch (the call
  * then serialises and waits for the stream).  Other formats, and shapes for which
@@ -190,6 +190,24 @@ int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
 int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                             float *d_out, int32_t *d_sums, size_t m, size_t n, size_t k,
                             void *d_workspace, size_t workspace_bytes, void *stream);
+
+/* Grouped (mixture-of-experts) matmul: the batched form of the per-token expert calls of
+ * MoeFfn::forward (crates/oxillama-arch/src/common/moe.rs:236-252: for each selected expert,
+ * expert.forward(input) -> QuantLinear::forward -> gemv).  Token rows are grouped by
+ * expert: expert e multiplies rows d_row_offsets[e] .. d_row_offsets[e+1]-1 of d_acts_q8
+ * (total_rows rows of k/32 Q8_0 blocks) by the n x k weights at d_weights + e *
+ * expert_stride_bytes and writes the same rows of d_out [total_rows x n].  d_row_offsets is
+ * device memory (n_experts + 1 ascending int32 values, last = total_rows), so the call neither
+ * copies nor synchronises; max_rows_per_expert bounds any one group (0 = total_rows) and only
+ * sizes the launch.  Q4_K and IQ4_XS; needs oxq_moe_gemm_q8_workspace_bytes() bytes of
+ * 256-byte-aligned device scratch.  d_sums (optional, else NULL): exact int32 group sums
+ * [(row * n + c) * (k/32) + g] as in oxq_gemm_block_sums_dev. */
+size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k);
+int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes,
+                        size_t n_experts, const uint8_t *d_acts_q8, const int32_t *d_row_offsets,
+                        size_t total_rows, size_t max_rows_per_expert, float *d_out, int32_t *d_sums,
+                        size_t n, size_t k, int accumulate, void *d_workspace,
+                        size_t workspace_bytes, void *stream);
 
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                        int32_t *d_sums, size_t n_rows, size_t n_cols, void *stream);

@@ -663,4 +663,47 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
     return gemm_dev(type, d_weights, d_acts_q8, d_out, d_sums, m, n, k, 0, d_workspace, workspace_bytes, stream);
 }
 
+size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k) {
+    return oxq_gemm_q8_workspace_bytes(type, total_rows < 8 ? 8 : total_rows, n, k);
+}
+
+int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
+                        const uint8_t *d_acts_q8, const int32_t *d_row_offsets, size_t total_rows,
+                        size_t max_rows_per_expert, float *d_out, int32_t *d_sums, size_t n, size_t k, int accumulate,
+                        void *d_workspace, size_t workspace_bytes, void *stream) {
+    int st = check_dev_shape(type, n, k);
+    if (st != OXQ_OK) return st;
+    if (total_rows > 0x7FFFFFFFull || n_experts > 65535)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0x7FFFFFFFull, total_rows, "too many rows or experts");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (total_rows == 0 || n_experts == 0 || n == 0 || k == 0) return OXQ_OK;
+    if (!d_row_offsets) return fail(OXQ_ERR_INTERNAL, 0, 0, "null row offsets");
+    const size_t row_bytes = k / oxq_block_size(type) * oxq_block_bytes(type);
+    if (expert_stride_bytes < n * row_bytes)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, n * row_bytes, expert_stride_bytes, "expert stride smaller than one expert");
+    const size_t need = oxq_moe_gemm_q8_workspace_bytes(type, total_rows, n, k);
+    if (need == 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, k, "no grouped kernel for this type/shape");
+    if (!d_workspace || workspace_bytes < need)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, d_workspace ? workspace_bytes : 0, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
+        return fail(OXQ_ERR_KERNEL, 256, reinterpret_cast<uintptr_t>(d_workspace) & 255, "workspace must be 256-byte aligned");
+    oxq::GemmArgs ga;
+    ga.W = d_weights;
+    ga.A = d_acts_q8;
+    ga.out = d_out;
+    ga.sums = d_sums;
+    ga.workspace = (uint8_t *)d_workspace;
+    ga.m = (uint32_t)(total_rows < 8 ? 8 : total_rows);  // the tile kernel's minimum; rows past the offsets are never stored
+    ga.n = (uint32_t)n;
+    ga.k = (uint32_t)k;
+    ga.accumulate = accumulate ? 1 : 0;
+    ga.offsets = d_row_offsets;
+    ga.n_experts = (uint32_t)n_experts;
+    ga.max_rows = (uint32_t)(max_rows_per_expert ? (max_rows_per_expert < total_rows ? max_rows_per_expert : total_rows)
+                                                 : total_rows);
+    ga.w_stride = expert_stride_bytes;
+    OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
 }  // extern "C"

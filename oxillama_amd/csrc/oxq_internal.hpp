@@ -35,8 +35,14 @@ struct GemmArgs {
     float *out;         // [m x n] row-major
     int32_t *sums;      // optional debug dump [m][n][k/32]
     uint8_t *workspace; // gemm_workspace_bytes(m, k) bytes, 256-byte aligned; null: row-by-row matvecs
-    uint32_t m, n, k;
+    uint32_t m, n, k;   // m = all token rows (of all experts in the grouped form)
     int accumulate;
+    // Grouped (mixture-of-experts) form: expert e multiplies token rows offsets[e] ..
+    // offsets[e+1]-1 by the weights at W + e * w_stride.  offsets == null: plain matmul.
+    const int32_t *offsets = nullptr;  // device memory, n_experts + 1 entries
+    uint32_t n_experts = 0;
+    uint32_t max_rows = 0;             // upper bound of the rows of any one expert
+    size_t w_stride = 0;
 };
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
 // Device scratch the tile kernel needs for m tokens of k columns (activation re-layout).

@@ -249,6 +249,19 @@ class HipKernel:
                                                  d_out.data_ptr(), d_sums.data_ptr(), m, n, k, ws_ptr, ws_len,
                                                  self._stream()))
 
+    def moe_gemm_workspace_bytes(self, total_rows, n, k):
+        return self._lib.oxq_moe_gemm_q8_workspace_bytes(self.tensor_type, total_rows, n, k)
+
+    def moe_gemm_q8_dev(self, d_weights, expert_stride, n_experts, d_acts, d_offsets, total_rows, max_rows, d_out,
+                        n, k, workspace, accumulate=False, d_sums=None):
+        """Grouped expert matmul: rows d_offsets[e]..d_offsets[e+1]-1 of d_acts times expert e's weights
+        (d_weights + e * expert_stride bytes) -> the same rows of d_out [total_rows x n]."""
+        _check(self._lib.oxq_moe_gemm_q8_dev(self.tensor_type, d_weights.data_ptr(), expert_stride, n_experts,
+                                             d_acts.data_ptr(), d_offsets.data_ptr(), total_rows, max_rows,
+                                             d_out.data_ptr(), d_sums.data_ptr() if d_sums is not None else None,
+                                             n, k, int(accumulate), workspace.data_ptr(), workspace.numel(),
+                                             self._stream()))
+
     def block_sums_dev(self, d_weights, d_acts, d_sums, n_rows, n_cols):
         _check(self._lib.oxq_block_sums_dev(self.tensor_type, d_weights.data_ptr(), d_acts.data_ptr(),
                                             d_sums.data_ptr(), n_rows, n_cols, self._stream()))

@@ -320,13 +320,13 @@ def _oracle_prefill(ref, t, w, acts, m, n, k_, rows=None):
 
 @pytest.mark.parametrize("shape", [(8, 32, 256), (33, 100, 1024), (128, 160, 512), (200, 257, 1024), (64, 64, 4096),
                                    (130, 129, 2048)], ids=lambda s: "x".join(map(str, s)))
-def test_prefill_tile_kernel_q4k(hip, ref, shape):
-    """Q4_K x Q8_0 int8-MFMA tile kernel: integer sub-block sums bit-exact, fp32 within 1e-5,
-    ragged tile edges in both directions, overwrite and accumulate."""
+@pytest.mark.parametrize("t", [O.Q4_K, O.IQ4_XS], ids=lambda t: O.NAMES[t])
+def test_prefill_tile_kernel(hip, ref, shape, t):
+    """Q4_K / IQ4_XS x Q8_0 int8-MFMA tile kernel: integer sub-block sums bit-exact, fp32 within
+    1e-5, ragged tile edges in both directions, overwrite and accumulate."""
     import torch
     m, n, k_ = shape
-    t = O.Q4_K
-    say("prefill", shape)
+    say("prefill", O.NAMES[t], shape)
     w = synth.weights(t, 600 + m, n, k_)
     x = synth.normal_f32(700 + n, m * k_)
     acts = ref.quantize_q8_0(x)
@@ -386,6 +386,84 @@ def test_prefill_full_size_c4(hip, ref):
 
 
 # ---- (7) residency helpers -----------------------------------------------------------------
+
+def _moe_case(ref, t, n_experts, n_tok, top_k, n, k_, seed):
+    """Seeded uniform router logits -> top-k routing -> pairs grouped by expert."""
+    from oxillama_amd import moe
+    rng = np.random.default_rng(seed)
+    logits = rng.random((n_tok, n_experts), dtype=np.float32)
+    experts, weights = moe.route_top_k(logits, top_k)
+    offsets, tok, slot = moe.group_by_expert(experts, n_experts)
+    x = synth.normal_f32(seed + 1, n_tok * k_).reshape(n_tok, k_)
+    acts_tok = ref.quantize_q8_0(x.reshape(-1)).reshape(n_tok, k_ // 32 * 34)
+    acts = np.ascontiguousarray(acts_tok[tok])  # one activation row per (token, expert) pair
+    w = np.stack([synth.weights(t, seed + 10 + e, n, k_) for e in range(n_experts)])
+    return offsets, tok, slot, weights, acts, w
+
+
+@pytest.mark.parametrize("t", [O.IQ4_XS, O.Q4_K], ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("cfg", [(8, 64, 2, 96, 1024), (4, 7, 2, 300, 512), (8, 200, 2, 64, 256), (3, 5, 1, 33, 2048)],
+                         ids=lambda c: "e%d_t%d_k%d_n%d_k%d" % c)
+def test_moe_grouped_matmul(hip, ref, t, cfg):
+    """Grouped expert matmul: every (token, expert) pair equals the fused matvec of that expert's
+    weights with the token's Q8_0 row (fp32 within 1e-5, integer sums bit-exact); rows of experts
+    with no tokens and tile padding are never written."""
+    import torch
+    n_experts, n_tok, top_k, n, k_ = cfg
+    say("moe", O.NAMES[t], cfg)
+    offsets, tok, slot, weights, acts, w = _moe_case(ref, t, n_experts, n_tok, top_k, n, k_, 900 + n_tok)
+    rows = int(offsets[-1])
+    assert rows == n_tok * top_k
+    kern = hip.HipKernel(t)
+    ws = torch.empty(kern.moe_gemm_workspace_bytes(rows, n, k_), dtype=torch.uint8, device="cuda")
+    dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
+    doff = torch.from_numpy(offsets).cuda()
+    dy = torch.full((rows + 3, n), 7.0, dtype=torch.float32, device="cuda")  # 3 guard rows
+    dsum = torch.full((rows, n, k_ // 32), -1, dtype=torch.int32, device="cuda")
+    max_rows = int(np.diff(offsets).max())
+    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy, n, k_, ws, d_sums=dsum)
+    torch.cuda.synchronize()
+    y = dy.cpu().numpy()
+    assert np.all(y[rows:] == 7.0)
+    y_ref = np.empty((rows, n), dtype=np.float32)
+    s_ref = np.empty((rows, n, k_ // 32), dtype=np.int32)
+    for e in range(n_experts):
+        for r in range(offsets[e], offsets[e + 1]):
+            y_ref[r] = canonical_ref(ref, t, w[e], acts[r], n, k_)
+            s_ref[r] = ref.block_sums(t, w[e], acts[r], n, k_)
+    assert_close(y[:rows], y_ref, f"moe {cfg}")
+    assert np.array_equal(dsum.cpu().numpy(), s_ref)
+    # production launch (no sums), overwrite then accumulate, max_rows = 0 (unknown)
+    dy2 = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
+    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, 0, dy2, n, k_, ws)
+    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy2, n, k_, ws, accumulate=True)
+    torch.cuda.synchronize()
+    assert torch.equal(dy2, dy[:rows] + dy[:rows])
+
+
+def test_moe_full_size_c5_one_projection(hip, ref):
+    """C5 shapes: 8 experts of IQ4_XS 14336 x 4096 (gate) and 4096 x 14336 (down), 64 tokens top-2.
+    Oracle on a sample of pairs (every row of the sampled pairs)."""
+    import torch
+    t, n_experts, n_tok, top_k = O.IQ4_XS, 8, 64, 2
+    kern = hip.HipKernel(t)
+    for n, k_ in ((14336, 4096), (4096, 14336)):
+        offsets, tok, slot, weights, acts, w = _moe_case(ref, t, n_experts, n_tok, top_k, n, k_, 5000 + n)
+        rows = int(offsets[-1])
+        ws = torch.empty(kern.moe_gemm_workspace_bytes(rows, n, k_), dtype=torch.uint8, device="cuda")
+        dw, da, doff = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda(), torch.from_numpy(offsets).cuda()
+        dy = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
+        kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, int(np.diff(offsets).max()), dy, n, k_, ws)
+        torch.cuda.synchronize()
+        y = dy.cpu().numpy()
+        for r in range(0, rows, 9):
+            e = int(np.searchsorted(offsets, r, side="right") - 1)
+            y_ref = canonical_ref(ref, t, w[e], acts[r], n, k_, threads=16)
+            assert_close(y[r], y_ref, f"c5 {n}x{k_} pair row {r} expert {e}")
+        del dw, da, dy, ws
+
+
+
 
 def test_registered_weights_and_cache(hip, ref):
     import ctypes as C
