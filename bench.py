@@ -15,6 +15,7 @@ Prints ONE JSON line.  Extra objects:
                events on the launch stream, algorithmic bytes / duration vs 8 TB/s
   kernels      the same figure for each GEMV shape, the lm_head and C1 shapes
   prefill      batch-512 Q4_K prefill matmul, int8 TOPS vs the 5.0 POPS peak
+  moe          IQ4_XS grouped expert matmuls (8 experts, 64 tokens, top-2), weight GB/s
   cpu_baseline the CPU restatement of the reference's fused rows on this host
 """
 import argparse
@@ -53,6 +54,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra-kernels", action="store_true")
+    ap.add_argument("--no-moe", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives or sharding here)",
@@ -215,6 +217,63 @@ def main():
                    "TOPS": round(ops / gemm_us / 1e6, 2), "peak_TOPS": INT8_PEAK_TOPS,
                    "frac_int8_peak": round(ops / gemm_us / 1e6 / INT8_PEAK_TOPS, 4)}
 
+    # ---- C5: Mixtral-shaped IQ4_XS expert matmuls, 64 tokens, top-2 of 8 experts ------------
+    moe_out = None
+    if not args.no_moe:
+        from oxillama_amd import moe
+        E, NTOK, TOPK = 8, 64, 2
+        k_iq = quant.HipKernel(IQ4_XS)
+        rng = np.random.default_rng(5)
+        experts, _ = moe.route_top_k(rng.random((NTOK, E), dtype=np.float32), TOPK)
+        offsets, tok, _slot = moe.group_by_expert(experts, E)
+        rows, max_rows = int(offsets[-1]), int(np.diff(offsets).max())
+
+        def expert_set(seed, n_rows, n_cols):
+            return torch.from_numpy(np.stack([synth.weights(IQ4_XS, seed + e, n_rows, n_cols) for e in range(E)])).to(dev)
+        wg, wu, wd = expert_set(7000, F, H), expert_set(7100, F, H), expert_set(7200, H, F)
+        stride = wg[0].numel()
+        xt = torch.from_numpy(synth.normal_f32(7, NTOK * H)).to(dev).reshape(NTOK, H)
+        xp = xt[torch.from_numpy(tok.astype(np.int64)).to(dev)].contiguous()      # one row per (token, expert) pair
+        hp = torch.from_numpy(synth.normal_f32(8, rows * F)).to(dev)
+        xpq = torch.empty(rows * (H // 32 * 34), dtype=torch.uint8, device=dev)
+        hpq = torch.empty(rows * (F // 32 * 34), dtype=torch.uint8, device=dev)
+        doff = torch.from_numpy(offsets).to(dev)
+        og = torch.zeros(rows * F, dtype=torch.float32, device=dev)
+        ou = torch.zeros(rows * F, dtype=torch.float32, device=dev)
+        od = torch.zeros(rows * H, dtype=torch.float32, device=dev)
+        wsm = torch.empty(max(k_iq.moe_gemm_workspace_bytes(rows, F, H), k_iq.moe_gemm_workspace_bytes(rows, H, F)),
+                          dtype=torch.uint8, device=dev)
+
+        def moe_step():
+            quant.quantize_q8_0_dev(xp, xpq)
+            k_iq.moe_gemm_q8_dev(wg, stride, E, xpq, doff, rows, max_rows, og, F, H, wsm)
+            k_iq.moe_gemm_q8_dev(wu, stride, E, xpq, doff, rows, max_rows, ou, F, H, wsm)
+            quant.quantize_q8_0_dev(hp, hpq)
+            k_iq.moe_gemm_q8_dev(wd, stride, E, hpq, doff, rows, max_rows, od, H, F, wsm)
+
+        with torch.cuda.stream(stream):
+            moe_step()
+            stream.synchronize()
+            reps = 6
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(reps):
+                moe_step()
+            e1.record(stream)
+            e1.synchronize()
+            moe_us = e0.elapsed_time(e1) * 1e3 / reps
+        moe_bytes = 3 * E * stride
+        moe_ops = 2 * rows * 3 * F * H
+        moe_out = {"workload": "IQ4_XS, 8 experts x (gate, up 14336x4096; down 4096x14336), 64 tokens, top-2 "
+                               "(seeded uniform logits), pairs grouped per expert",
+                   "pairs": rows, "rows_per_expert": np.diff(offsets).tolist(), "us_per_step": round(moe_us, 1),
+                   "weight_bytes": moe_bytes, "weight_GBps": round(moe_bytes / moe_us / 1e3, 1),
+                   "frac_hbm_peak": round(moe_bytes / moe_us / 1e3 / HBM_PEAK_GBPS, 4),
+                   "int8_TOPS": round(moe_ops / moe_us / 1e6, 1),
+                   "timed": "2 activation quantizations + 3 grouped int8-MFMA matmuls (the 749 MB of expert weights "
+                            "exceed the 256 MB Infinity Cache, so every step streams them from HBM)"}
+        del wg, wu, wd
+
     # ---- CPU baseline: the reference's fused rows restated in C, same layer -------------
     cpu = None
     if not args.no_cpu_baseline:
@@ -282,6 +341,7 @@ def main():
         "cpu_baseline": cpu,
         "kernels": kernels,
         "prefill": prefill,
+        "moe": moe_out,
         "device": {"name": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
                    "clock_mhz": info["clock_khz"] / 1000.0, "weight_generation_s": round(gen_s, 1)},
     }

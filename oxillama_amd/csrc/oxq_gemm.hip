@@ -424,8 +424,11 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     case 15: return launch_tile<F, 1, 1, 1, 4, false>(a, p, stream);
     case 16: return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
     default:
-        return rows > 32 ? launch_tile<F, 2, 2, 2, 1, false>(a, p, stream)
-                         : launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
+        if (rows > 32) return launch_tile<F, 2, 2, 2, 1, false>(a, p, stream);
+        // few tokens: 256-row tiles unless that leaves compute units without a work group
+        if ((size_t)((a.n + 255) / 256) * (a.offsets ? a.n_experts : 1) >= device_cus())
+            return launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
+        return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
     }
 }
 
