@@ -173,6 +173,16 @@ int oxq_matvec_q8_fused_dev(uint32_t type, const uint8_t *d_weights, const uint8
                             float *d_out, size_t n_rows, size_t n_cols, int accumulate,
                             void *stream);
 
+/* The same for up to 4 weight matrices of one format and shape that share the activation
+ * vector -- wq/wk/wv or ffn_gate/ffn_up of one layer, which the reference runs as separate
+ * QuantLinear::forward calls on the same input (crates/oxillama-arch/src/llama/model.rs:
+ * 295-310): d_outs[i][r] (+)= d_weights[i][r,:] . acts.  One launch streams all of them, which
+ * saves the fill and drain of the memory pipeline between them.  d_weights / d_outs are host
+ * arrays of n_mats device pointers.  Results are bit-identical to n_mats single calls. */
+int oxq_matvec_q8_fused_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_weights,
+                                  const uint8_t *d_acts_q8, float *const *d_outs, size_t n_rows,
+                                  size_t n_cols, int accumulate, void *stream);
+
 /* Prefill: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched form
  * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  Q4_K with
  * m >= 8 (and IQ4_XS likewise) uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()

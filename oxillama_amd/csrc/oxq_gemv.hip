@@ -19,15 +19,25 @@ template <class F, int STEPS, int RB, int KS, bool DUMP>
 static hipError_t launch_cached(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
                                 hipStream_t stream) {
     constexpr uint32_t G = 4 / KS;  // row groups per work group
+    const uint32_t n_mats = a.n_mats ? a.n_mats : 1;
+    const uint8_t *w[4];
+    float *o[4];
+    for (uint32_t i = 0; i < 4; i++) {
+        w[i] = i > 0 && i < n_mats ? a.W_more[i - 1] : a.W;
+        o[i] = i > 0 && i < n_mats ? a.out_more[i - 1] : a.out;
+    }
     const uint32_t n_batches = (a.n_rows + RB - 1) / RB;
-    const uint32_t max_groups = device_cus() * a.waves_per_cu / KS;
+    // the launch width is shared by the matrices of the call
+    uint32_t max_groups = device_cus() * a.waves_per_cu / KS / n_mats;
+    if (max_groups == 0) max_groups = 1;
     // Equal share per group: ceil(n_batches / passes) groups, each doing `passes` batches.
     const uint32_t passes = (n_batches + max_groups - 1) / max_groups;
     const uint32_t groups = (n_batches + passes - 1) / passes;
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
-    hipLaunchKernelGGL((gemv_q8_cached<F, STEPS, RB, KS, DUMP>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.out,
-                       a.sums, a.n_rows, units, groups_per_row, row_bytes, a.accumulate);
+    hipLaunchKernelGGL((gemv_q8_cached<F, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), 0, stream, w[0], w[1],
+                       w[2], w[3], o[0], o[1], o[2], o[3], a.A, a.sums, a.n_rows, units, groups_per_row, row_bytes,
+                       a.accumulate);
     return hipGetLastError();
 }
 
@@ -90,8 +100,39 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     return hipGetLastError();
 }
 
+// True when one launch can take the n_mats matrices of `a` (the register-cached kernel, whole
+// batches per matrix); otherwise the caller gets one launch per matrix.
+template <class F>
+static bool multi_in_one_launch(const GemvArgs &a) {
+    return (a.n_cols / F::UNIT_COLS + 63) / 64 <= 32 && !a.sums;
+}
+
 hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream) {
     if (a.n_rows == 0 || a.n_cols == 0) return hipSuccess;
+    if (a.n_mats > 1) {
+        bool one = false;
+        switch (type) {
+        case OXQ_TYPE_Q4_0: one = multi_in_one_launch<FmtQ4_0>(a); break;
+        case OXQ_TYPE_Q8_0: one = multi_in_one_launch<FmtQ8_0>(a); break;
+        case OXQ_TYPE_Q4_K: one = multi_in_one_launch<FmtQ4K>(a); break;
+        case OXQ_TYPE_Q6_K: one = multi_in_one_launch<FmtQ6K>(a); break;
+        case OXQ_TYPE_IQ4_XS: one = multi_in_one_launch<FmtIQ4XS>(a); break;
+        default: return hipErrorInvalidValue;
+        }
+        if (!one) {
+            for (uint32_t i = 0; i < a.n_mats; i++) {
+                GemvArgs s = a;
+                s.n_mats = 1;
+                if (i) {
+                    s.W = a.W_more[i - 1];
+                    s.out = a.out_more[i - 1];
+                }
+                hipError_t e = launch_gemv_q8(type, s, stream);
+                if (e != hipSuccess) return e;
+            }
+            return hipSuccess;
+        }
+    }
     switch (type) {
     case OXQ_TYPE_Q4_0: return launch_format<FmtQ4_0>(a, 32, stream);
     case OXQ_TYPE_Q8_0: return launch_format<FmtQ8_0>(a, 32, stream);

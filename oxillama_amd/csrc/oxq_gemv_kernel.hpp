@@ -63,12 +63,20 @@ __device__ __forceinline__ float reduce_batch(const Batch<F, STEPS, RB> &b, cons
 }
 
 template <class F, int STEPS, int RB, int KS, bool DUMP>
-__global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict__ W,
-                                                     const uint8_t *__restrict__ A,
-                                                     float *__restrict__ out, int32_t *__restrict__ sums,
+__global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
+                                                     const uint8_t *__restrict__ W2, const uint8_t *__restrict__ W3,
+                                                     float *__restrict__ out0, float *__restrict__ out1,
+                                                     float *__restrict__ out2, float *__restrict__ out3,
+                                                     const uint8_t *__restrict__ A, int32_t *__restrict__ sums,
                                                      uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
                                                      size_t row_bytes, int accumulate) {
     static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
+    // Up to four matrices of one shape and format that share the activation vector (wq/wk/wv,
+    // ffn_gate/ffn_up) ride in one launch: blockIdx.y picks the matrix, and each matrix gets
+    // its own gridDim.x work groups.
+    const uint32_t mat = blockIdx.y;
+    const uint8_t *__restrict__ W = mat == 0 ? W0 : mat == 1 ? W1 : mat == 2 ? W2 : W3;
+    float *__restrict__ out = mat == 0 ? out0 : mat == 1 ? out1 : mat == 2 ? out2 : out3;
     constexpr uint32_t G = 4 / KS;  // row groups per work group
     __shared__ float part_sums[2][4][4];
     const uint32_t lane = threadIdx.x & 63;

@@ -19,6 +19,11 @@ struct GemvArgs {
     uint32_t waves_per_cu;  // launch width: resident waves per compute unit
     uint32_t rows_per_batch;  // rows a wave loads at once (1, 2 or 4); 0 = chosen from the row size
     uint32_t waves_per_row;   // 1 or 4 waves share a row; 0 = chosen from the row length
+    // Further matrices of the same shape and format sharing A (q/k/v, gate/up): n_mats - 1
+    // entries; each has n_rows rows and its own output vector.
+    uint32_t n_mats = 1;
+    const uint8_t *W_more[3] = {nullptr, nullptr, nullptr};
+    float *out_more[3] = {nullptr, nullptr, nullptr};
 };
 
 // Number of compute units of the current device (cached per device).

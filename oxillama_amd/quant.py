@@ -232,6 +232,15 @@ class HipKernel:
                                                  d_out.data_ptr(), n_rows, n_cols, int(accumulate),
                                                  self._stream()))
 
+    def matvec_q8_fused_multi_dev(self, d_weights, d_acts, d_outs, n_rows, n_cols, accumulate=True):
+        """Up to 4 matrices of one shape sharing d_acts, one launch (wq/wk/wv, ffn_gate/ffn_up)."""
+        import ctypes as C
+        n = len(d_weights)
+        wp = (C.c_void_p * n)(*[w.data_ptr() for w in d_weights])
+        op = (C.c_void_p * n)(*[o.data_ptr() for o in d_outs])
+        _check(self._lib.oxq_matvec_q8_fused_multi_dev(self.tensor_type, n, wp, d_acts.data_ptr(), op, n_rows, n_cols,
+                                                       int(accumulate), self._stream()))
+
     def gemm_workspace_bytes(self, m, n, k):
         return self._lib.oxq_gemm_q8_workspace_bytes(self.tensor_type, m, n, k)
 

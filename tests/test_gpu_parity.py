@@ -197,6 +197,28 @@ def test_fused_extreme_bytes(hip, ref, t):
     assert_close(out, canonical_ref(ref, t, w, a, n_rows, n_cols), O.NAMES[t])
 
 
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("n_mats", [2, 3, 4])
+def test_fused_multi_matrix_launch_is_bit_identical(hip, ref, t, n_mats):
+    """wq/wk/wv- or gate/up-style launch of several matrices sharing one activation vector:
+    the same bits as one call per matrix, overwrite and accumulate, for row counts that are
+    and are not a multiple of the kernel's batch (the latter falls back to separate launches)."""
+    import torch
+    for n_rows, n_cols in ((64, 4096), (36, 1024), (30, 512), (8, 14336)):
+        ws = [torch.from_numpy(synth.weights(t, 800 + i, n_rows, n_cols)).cuda() for i in range(n_mats)]
+        a = torch.from_numpy(ref.quantize_q8_0(synth.normal_f32(810, n_cols))).cuda()
+        kern = hip.HipKernel(t)
+        single = [torch.full((n_rows,), 3.0, dtype=torch.float32, device="cuda") for _ in range(n_mats)]
+        multi = [torch.full((n_rows,), 3.0, dtype=torch.float32, device="cuda") for _ in range(n_mats)]
+        for acc in (False, True):
+            for w, y in zip(ws, single):
+                kern.matvec_q8_fused_dev(w, a, y, n_rows, n_cols, accumulate=acc)
+            kern.matvec_q8_fused_multi_dev(ws, a, multi, n_rows, n_cols, accumulate=acc)
+            torch.cuda.synchronize()
+            for y1, y2 in zip(single, multi):
+                assert torch.equal(y1, y2), (O.NAMES[t], n_mats, n_rows, n_cols, acc)
+
+
 def test_empty_inputs(hip):
     for t in O.ALL_TYPES:
         k = hip.HipKernel(t)
