@@ -41,6 +41,7 @@ __device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
 // super-block; the 16-byte header is read by each of them (same cache line).
 struct FmtQ4K {
     static constexpr uint32_t BLOCK_BYTES = 144, BLOCK_COLS = 256, UNIT_COLS = 64;
+    static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {
         uint32_t g, sh;
         bool upper;
@@ -126,6 +127,7 @@ struct FmtQ4K {
 // 8hh + is + 2j, activation block 8b + 4hh + j bytes 16is..+16.
 struct FmtQ6K {
     static constexpr uint32_t BLOCK_BYTES = 210, BLOCK_COLS = 256, UNIT_COLS = 64;
+    static constexpr uint32_t TWO_ROW_BATCH_BYTES = 0;  // 52 bytes and 11 registers per unit: one row per batch
     struct Lane {
         uint32_t hh, is;
     };
@@ -160,6 +162,7 @@ struct FmtQ6K {
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &k) {
         const uint8_t *blk = row + (size_t)(u >> 2) * BLOCK_BYTES;
+        // plain unaligned loads: re-aligning in registers (ld16_h) was measured slower here
         w.ql0 = ld16(blk + 64 * k.hh + 16 * k.is);
         w.ql1 = ld16(blk + 64 * k.hh + 32 + 16 * k.is);
         w.qh = ld16(blk + 128 + 32 * k.hh + 16 * k.is);
@@ -206,6 +209,7 @@ struct FmtQ6K {
 // Unit = one 34-byte block against the activation block of the same index.
 struct FmtQ8_0 {
     static constexpr uint32_t BLOCK_BYTES = 34, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {};
     struct Act {
         u32x4 q0, q1;
@@ -261,6 +265,7 @@ __device__ __forceinline__ void split_even_odd(const u32x4 &q0, const u32x4 &q1,
 // Unit = one 18-byte block.  sum (q-8)*a = sum q*a - 8*sum a.
 struct FmtQ4_0 {
     static constexpr uint32_t BLOCK_BYTES = 18, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {};
     struct Act {
         uint32_t ev[4], od[4];
@@ -311,6 +316,7 @@ struct FmtQ4_0 {
 // d * float((ls - 32) * sum kvalues[idx] * a) * d_a.
 struct FmtIQ4XS {
     static constexpr uint32_t BLOCK_BYTES = 136, BLOCK_COLS = 256, UNIT_COLS = 32;
+    static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {
         uint32_t i;
     };

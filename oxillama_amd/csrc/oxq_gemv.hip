@@ -63,9 +63,9 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     uint32_t ks = a.waves_per_row;
     if (ks == 0) ks = steps >= 3 ? 4 : 1;
     // Rows per batch: two while a wave's slice of a row is at most ~3.4 KB, else one
-    // (measured on MI355X: more in flight per wave does not pay beyond that).
+    // (measured on MI355X: more in flight per wave does not pay beyond that); Q6_K always one.
     uint32_t rb = a.rows_per_batch;
-    if (rb == 0) rb = row_bytes / (ks >= 4 ? 4 : 1) <= 3400 ? 2 : 1;
+    if (rb == 0) rb = row_bytes / (ks >= 4 ? 4 : 1) <= F::TWO_ROW_BATCH_BYTES ? 2 : 1;
     if (ks >= 4 && steps <= 32) {
         const uint32_t sw = (steps + 3) / 4;
         switch (sw) {
