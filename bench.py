@@ -30,6 +30,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per gate+up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
+# what the counter reads for a copy kernel of known size (2.000 and 1.000); the runs and figures are in
+# profiles/hbm_traffic_gemv_gate_up_lm_head_prefill_pmc.txt.  Algorithmic bytes are 66 179 328.
+MEASURED_TRAFFIC_GATE_UP = 66312806
 INT8_PEAK_TOPS = 5000.0
 
 Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS = 2, 8, 12, 14, 23
@@ -55,6 +59,10 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra-kernels", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="launch a 256 MiB copy kernel 3 times, then gate+up (one launch) over 8 distinct layers, "
+                         "lm_head twice and the prefill matmul twice, and exit: the workload of the rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE runs (the copy kernel scales the counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives or sharding here)",
@@ -74,6 +82,48 @@ def main():
     L = max(1, args.layers)
 
     k_q8, k_q4k, k_q6k = quant.HipKernel(Q8_0), quant.HipKernel(Q4_K), quant.HipKernel(Q6_K)
+
+    if args.traffic_probe:
+        import ctypes as C
+        kit = C.CDLL(os.path.join(ROOT, "oxillama_amd", "liboxq_benchkit.so"))
+        kit.oxq_benchkit_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint, C.c_void_p]
+        nbytes = 256 << 20
+        src = torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            kit.oxq_benchkit_copy(src.data_ptr(), dst.data_ptr(), nbytes, 2048, None)
+        torch.cuda.synchronize()
+        del src, dst
+        xq = torch.from_numpy(np.zeros(H // 32 * 34, dtype=np.uint8)).to(dev)
+        quant.quantize_q8_0_dev(torch.from_numpy(synth.normal_f32(1, H)).to(dev), xq)
+        yg = torch.zeros(F, dtype=torch.float32, device=dev)
+        yu = torch.zeros(F, dtype=torch.float32, device=dev)
+        for l in range(8):
+            g, u = (torch.from_numpy(synth.weights(Q4_K, s0 + l, F, H)).to(dev) for s0 in (2000, 3000))
+            torch.cuda.synchronize()
+            k_q4k.matvec_q8_fused_multi_dev([g, u], xq, [yg, yu], F, H, accumulate=False)
+            torch.cuda.synchronize()
+        V = 128256
+        logits = torch.zeros(V, dtype=torch.float32, device=dev)
+        for i in range(2):
+            lm = torch.from_numpy(synth.weights(Q6_K, 6000 + i, V, H)).to(dev)
+            torch.cuda.synchronize()
+            k_q6k.matvec_q8_fused_dev(lm, xq, logits, V, H, accumulate=False)
+            torch.cuda.synchronize()
+            del lm
+        M = 512
+        xsq = torch.empty(M * (H // 32 * 34), dtype=torch.uint8, device=dev)
+        quant.quantize_q8_0_dev(torch.from_numpy(synth.normal_f32(3, M * H)).to(dev), xsq)
+        ys = torch.zeros(M * F, dtype=torch.float32, device=dev)
+        ws = torch.empty(k_q4k.gemm_workspace_bytes(M, F, H), dtype=torch.uint8, device=dev)
+        for i in range(2):
+            w = torch.from_numpy(synth.weights(Q4_K, 2100 + i, F, H)).to(dev)
+            torch.cuda.synchronize()
+            k_q4k.gemm_q8_dev(w, xsq, ys, M, F, H, workspace=ws)
+            torch.cuda.synchronize()
+        print(json.dumps({"traffic_probe": "done", "copy_bytes": nbytes}), flush=True)
+        return
 
     def upload(t, seed, n_rows, n_cols):
         return torch.from_numpy(synth.weights(t, seed, n_rows, n_cols)).to(dev)
@@ -182,7 +232,7 @@ def main():
     dom = time_pair()
     roofline = {"bound": "hbm", "kernel": "gemv_q8_cached<Q4_K>, ffn_gate + ffn_up (2 x 14336x4096) in one launch",
                 "achieved": dom["algorithmic_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dom["frac_hbm_peak"],
-                "traffic": None, "us_per_call": dom["us_per_call"], "algorithmic_bytes": dom["algorithmic_bytes"]}
+                "traffic": MEASURED_TRAFFIC_GATE_UP, "us_per_call": dom["us_per_call"], "algorithmic_bytes": dom["algorithmic_bytes"]}
 
     kernels = {"q4k_gate_plus_up_one_launch": dom, "q4k_gate_up_14336x4096": time_kernel(k_q4k, Q4_K, gate_up, xq, yg, F, H)}
     if not args.no_extra_kernels:
