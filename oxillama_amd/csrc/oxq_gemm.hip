@@ -141,8 +141,8 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
 // holds row 8*(v/4) + 4*h + v%4 (token), column c (weight row).
 //
 // Everything lives in the 256 architectural VGPRs (two waves per SIMD), so MFMA results
-// are read by the VALU without accumulator-register copies.  Per super-block the work
-// group decodes its rows' 8 sub-block scales once into LDS as ready-made fp32 factors
+// are read by the VALU without accumulator-register copies.  Per super-block each wave
+// decodes its rows' 8 sub-block scales once into LDS as ready-made fp32 factors
 // (dsc, -12582912*dsc, and for Q4_K -dmin*mn); the f16 token scales of the whole k sit in
 // LDS for the life of the work group and enter the accumulate fma as f16 operands.  The
 // Q4_K min term is folded into the same accumulators by one fp32 MFMA per tile and pair
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
 // Grouped form (mixture-of-experts): blockIdx.y = expert; expert e multiplies the token
 // rows offsets[e] .. offsets[e+1]-1 by the weights at W + e * w_stride.
 template <class F, int MT, int NT, int WM, int DIST, bool DUMP>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_tile_kernel(
+__device__ __forceinline__ void gemm_tile_body(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,
     const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m, uint32_t mpad,
     uint32_t n, uint32_t k, int accumulate, uint32_t m_tiles, uint32_t n_tiles, const int32_t *__restrict__ offsets,
@@ -163,10 +163,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     constexpr int WN = 4 / WM;
     constexpr int WG_TOK = 32 * MT * WM, WG_ROWS = 32 * NT * WN, MTILES = MT * WM;
     constexpr int NP = F::HAS_MIN ? 3 : 2;
-    constexpr int TPR = 256 / WG_ROWS, SPT = 8 / TPR;  // decode: threads per row, sub-blocks per thread
-    static_assert(WG_ROWS <= 256 && (DIST == 1 || DIST == 2 || DIST == 4), "tile configuration");
+    constexpr int W_ROWS = 32 * NT;                  // weight rows of one wave
+    constexpr int LPR = 64 / W_ROWS, SPL = 8 / LPR;  // scale decode: lanes per row, sub-blocks per lane
+    static_assert(NT <= 2 && (DIST == 1 || DIST == 2 || DIST == 4), "tile configuration");
     extern __shared__ uint16_t lds_da[];            // [nsb][MTILES][2 halves][16] f16 token scales
-    __shared__ float lds_sc[2][8][NP][WG_ROWS];     // [buffer][sub-block][dsc, -MAGIC*dsc, -dmin*mn][row]
+    __shared__ float lds_sc[4][8][NP][W_ROWS];      // [wave][sub-block][dsc, -MAGIC*dsc, -dmin*mn][row of the wave]
     const uint32_t nsb = k / 32, nblk = k / 256, ngrp = nblk * 4;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
@@ -207,21 +208,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const __amdgpu_buffer_rsrc_t rs_p =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P), 0, (int)(nsb * mpad * 4), BUFFER_FLAGS);
 
-    // Scale decode: thread -> row tid % WG_ROWS, sub-blocks SPT * (tid / WG_ROWS) + 0..SPT-1.
-    const uint32_t drow = tid % WG_ROWS, ds0 = SPT * (tid / WG_ROWS);
-    const uint32_t hrow_off = (min(n_wg + drow, n - 1) - n_base) * row_bytes;
-    auto decode = [&](const u32x4 hd, uint32_t buf) {
+    // Scale decode, per wave for its own rows (no work-group barrier in the k loop): lane ->
+    // row lane % W_ROWS, sub-blocks SPL * (lane / W_ROWS) + 0..SPL-1.  The wave writes the
+    // factors of the next super-block after its last read of the current ones.
+    const uint32_t drow = lane % W_ROWS, ds0 = SPL * (lane / W_ROWS);
+    const uint32_t hrow_off = (min(n_wave + drow, n - 1) - n_base) * row_bytes;
+    auto decode = [&](const u32x4 hd) {
 #pragma unroll
-        for (int e = 0; e < SPT; e++) {
+        for (int e = 0; e < SPL; e++) {
             const uint32_t s = ds0 + e;
             float dsc, qneg;
             F::scales(hd, s, dsc, qneg);
-            lds_sc[buf][s][0][drow] = dsc;
-            lds_sc[buf][s][1][drow] = -(MAGIC_F * dsc);  // exact
-            if (F::HAS_MIN) lds_sc[buf][s][NP - 1][drow] = qneg;
+            lds_sc[wave][s][0][drow] = dsc;
+            lds_sc[wave][s][1][drow] = -(MAGIC_F * dsc);  // exact
+            if (F::HAS_MIN) lds_sc[wave][s][NP - 1][drow] = qneg;
         }
     };
-    decode(__builtin_amdgcn_raw_buffer_load_b128(rs_w, hrow_off, 0, 0), 0);
+    decode(__builtin_amdgcn_raw_buffer_load_b128(rs_w, hrow_off, 0, 0));
 
     v16f acc[MT][NT];
     v16i magic;
@@ -266,11 +269,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     // One pair of sub-blocks (2g, 2g+1): 2*MT*NT int8 MFMA tiles, each followed by its 32
     // VALU operations; the MFMA of tile t+2 is issued before the VALU work of tile t+1 so
     // that the matrix core runs ahead of the VALU.
-    auto compute = [&](const u32x4 (&qs)[NT], const Ops &o, uint32_t blk, uint32_t g, uint32_t buf) {
+    auto compute = [&](const u32x4 (&qs)[NT], const Ops &o, uint32_t blk, uint32_t g) {
         constexpr int T = 2 * MT * NT;
         v4i bop[NT][2];
         for (int nt = 0; nt < NT; nt++) F::operands(qs[nt], bop[nt]);
-        const uint32_t lrow = wn * (32 * NT) + c;
         auto mfma_tile = [&](int t) {
             const int e = t / (MT * NT), mt = (t / NT) % MT, nt = t % NT;
             v4i aop;
@@ -284,8 +286,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         for (int t = 0; t < T; t++) {
             const int e = t / (MT * NT), mt = (t / NT) % MT, nt = t % NT;
             const uint32_t s = 2 * g + e, j = blk * 8 + s;
-            const float dsc = lds_sc[buf][s][0][lrow + nt * 32];
-            const float nc2 = lds_sc[buf][s][1][lrow + nt * 32];
+            const float dsc = lds_sc[wave][s][0][nt * 32 + c];
+            const float nc2 = lds_sc[wave][s][1][nt * 32 + c];
             const u32x4 *dp = reinterpret_cast<const u32x4 *>(&lds_da[((j * MTILES + wm * MT + mt) * 2 + h) * 16]);
             const u32x4 dav[2] = {dp[0], dp[1]};
             const v16i dres = dq[t & 1];
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (F::HAS_MIN && e == 1) {
                 // min term of sub-blocks 2g (lanes h = 0) and 2g+1 (lanes h = 1):
                 // acc[token][row] += P[token][s] * (-dmin*mn)[row][s], contracted over the pair
-                const float qv = lds_sc[buf][2 * g + h][NP - 1][lrow + nt * 32];
+                const float qv = lds_sc[wave][2 * g + h][NP - 1][nt * 32 + c];
                 acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(o.pv[mt], qv, acc[mt][nt], 0, 0, 0);
             }
         }
@@ -321,7 +323,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     __syncthreads();
 
     for (uint32_t blk = 0; blk < nblk; blk++) {
-        const uint32_t buf = blk & 1;
         const uint32_t nxt = min(blk + 1, nblk - 1);  // last trip: harmless re-read
         const u32x4 hd = __builtin_amdgcn_raw_buffer_load_b128(rs_w, hrow_off, nxt * F::BLOCK_BYTES, 0);
 #pragma unroll
@@ -331,14 +332,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             fetch_w(wring[g % DIST], blk * 4 + g + DIST);  // slot consumed: refill it DIST groups ahead
             if (g & 1) {
                 fetch_a(ops0, blk * 4 + g + 1);
-                compute(qs, ops1, blk, g, buf);
+                compute(qs, ops1, blk, g);
             } else {
                 fetch_a(ops1, blk * 4 + g + 1);
-                compute(qs, ops0, blk, g, buf);
+                compute(qs, ops0, blk, g);
             }
         }
-        decode(hd, buf ^ 1);
-        __syncthreads();
+        __builtin_amdgcn_wave_barrier();  // the wave's reads of this super-block's factors come first
+        decode(hd);
+        __builtin_amdgcn_wave_barrier();
     }
 
     for (int mt = 0; mt < MT; mt++)
@@ -354,6 +356,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             }
         }
 }
+
+// The kernel proper, compiled for a fixed number of waves per SIMD (OCC = 2: up to 256 VGPRs,
+// OCC = 3: up to 168): the register budget decides how far the compiler lets loads and MFMAs
+// run ahead of their use.
+#define OXQ_TILE_KERNEL(NAME, OCC)                                                                                   \
+    template <class F, int MT, int NT, int WM, int DIST, bool DUMP>                                                 \
+    __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void NAME(                      \
+        const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,                \
+        const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m,         \
+        uint32_t mpad, uint32_t n, uint32_t k, int accumulate, uint32_t m_tiles, uint32_t n_tiles,                  \
+        const int32_t *__restrict__ offsets, size_t w_stride) {                                                     \
+        gemm_tile_body<F, MT, NT, WM, DIST, DUMP>(W, q8t, P, da16, out, sums, m, mpad, n, k, accumulate, m_tiles,   \
+                                                  n_tiles, offsets, w_stride);                                      \
+    }
+OXQ_TILE_KERNEL(gemm_tile_kernel, 2)
+OXQ_TILE_KERNEL(gemm_tile_kernel_occ3, 3)
+#undef OXQ_TILE_KERNEL
 
 // One fused matvec per activation row: every format other than Q4_K, and Q4_K shapes the
 // tile kernel does not take.
@@ -386,14 +405,14 @@ struct TilePlan {
     uint32_t mpad;
 };
 
-template <class F, int MT, int NT, int WM, int DIST, bool DUMP>
+template <class F, int MT, int NT, int WM, int DIST, bool DUMP, int OCC = 2>
 static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
     constexpr uint32_t WG_TOK = 32 * MT * WM, WG_ROWS = 32 * NT * (4 / WM);
     const uint32_t rows = a.offsets ? a.max_rows : a.m;
     const uint32_t m_tiles = (rows + WG_TOK - 1) / WG_TOK, n_tiles = (a.n + WG_ROWS - 1) / WG_ROWS;
     const dim3 grid(8 * ((n_tiles + 7) / 8) * m_tiles, a.offsets ? a.n_experts : 1);
     const size_t lds = (size_t)(a.k / 32) * WG_TOK * 2;
-    auto kern = &gemm_tile_kernel<F, MT, NT, WM, DIST, DUMP>;
+    auto kern = OCC == 3 ? &gemm_tile_kernel_occ3<F, MT, NT, WM, DIST, DUMP> : &gemm_tile_kernel<F, MT, NT, WM, DIST, DUMP>;
     if (lds > 32 * 1024) {  // beyond the default dynamic LDS limit: opt in (up to the 160 KB of a CU)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -417,6 +436,9 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     case 2: return launch_tile<F, 1, 2, 2, 1, false>(a, p, stream);
     case 3: return launch_tile<F, 2, 2, 2, 1, false>(a, p, stream);
     case 4: return launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
+    case 5: return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
+    case 6: return launch_tile<F, 1, 2, 2, 1, false, 3>(a, p, stream);
+    case 7: return launch_tile<F, 1, 1, 2, 1, false, 3>(a, p, stream);
     case 11: return launch_tile<F, 1, 2, 1, 1, false>(a, p, stream);
     case 12: return launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
     case 13: return launch_tile<F, 1, 2, 1, 4, false>(a, p, stream);
