@@ -278,10 +278,28 @@ def main():
             e1.synchronize()
             quant_us = e0.elapsed_time(e1) * 1e3 / reps
         ops = 2 * M * F * H
+        # the same shape in the other four formats (tile kernel, same workspace)
+        others = {}
+        for name, t in (("Q6_K", Q6_K), ("Q8_0", Q8_0), ("Q4_0", Q4_0), ("IQ4_XS", IQ4_XS)):
+            kt = quant.HipKernel(t)
+            wt = [upload(t, 8000 + i, F, H) for i in range(4)]
+            wst = torch.empty(max(kt.gemm_workspace_bytes(M, F, H), 256), dtype=torch.uint8, device=dev)
+            with torch.cuda.stream(stream):
+                kt.gemm_q8_dev(wt[0], xsq, ys, M, F, H, workspace=wst)
+                stream.synchronize()
+                e0.record(stream)
+                for i in range(4):
+                    kt.gemm_q8_dev(wt[i], xsq, ys, M, F, H, workspace=wst)
+                e1.record(stream)
+                e1.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / 4
+            others[name] = {"gemm_us": round(us, 2), "TOPS": round(ops / us / 1e6, 1)}
+            del wt, wst
         prefill = {"workload": "Q4_K 14336x4096 x Q8_0 acts 512x4096", "int8_ops": ops,
                    "gemm_us": round(gemm_us, 2), "quantize_us": round(quant_us, 2),
                    "TOPS": round(ops / gemm_us / 1e6, 2), "peak_TOPS": INT8_PEAK_TOPS,
-                   "frac_int8_peak": round(ops / gemm_us / 1e6 / INT8_PEAK_TOPS, 4)}
+                   "frac_int8_peak": round(ops / gemm_us / 1e6 / INT8_PEAK_TOPS, 4),
+                   "same_shape_other_formats": others}
 
     # ---- C5: Mixtral-shaped IQ4_XS expert matmuls, 64 tokens, top-2 of 8 experts ------------
     moe_out = None

@@ -184,18 +184,19 @@ int oxq_matvec_q8_fused_multi_dev(uint32_t type, size_t n_mats, const uint8_t *c
                                   size_t n_cols, int accumulate, void *stream);
 
 /* Prefill: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched form
- * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  Q4_K with
- * m >= 8 (and IQ4_XS likewise) uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()
+ * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  With m >= 8 and k a
+ * multiple of 256 every format uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()
  * bytes of 256-byte-aligned device scratch: pass it and the call is asynchronous
  * and allocation-free; pass NULL and the library uses its own scratch (the call
- * then serialises and waits for the stream).  Other formats, and shapes for which
- * the workspace size is 0, run m fused matvecs and ignore the workspace. */
+ * then serialises and waits for the stream).  Shapes for which the workspace size is 0
+ * run m fused matvecs and ignore the workspace. */
 size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k);
 int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                     float *d_out, size_t m, size_t n, size_t k, int accumulate,
                     void *d_workspace, size_t workspace_bytes, void *stream);
 /* Debug: as oxq_gemm_q8_dev (overwrite), and the exact int32 group sums of the tile
- * kernel, d_sums[(r * n + c) * (k/32) + g].  OXQ_ERR_UNSUPPORTED_SHAPE when the shape
+ * kernel, d_sums[(r * n + c) * groups + g], groups = k/32 (k/16 for Q6_K).  For Q4_0 the
+ * tile kernel multiplies the unsigned nibbles (sum q*a); the "- 8" of (q - 8) enters in fp32.  OXQ_ERR_UNSUPPORTED_SHAPE when the shape
  * has no tile kernel. */
 int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                             float *d_out, int32_t *d_sums, size_t m, size_t n, size_t k,
@@ -209,7 +210,7 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
  * expert_stride_bytes and writes the same rows of d_out [total_rows x n].  d_row_offsets is
  * device memory (n_experts + 1 ascending int32 values, last = total_rows), so the call neither
  * copies nor synchronises; max_rows_per_expert bounds any one group (0 = total_rows) and only
- * sizes the launch.  Q4_K and IQ4_XS; needs oxq_moe_gemm_q8_workspace_bytes() bytes of
+ * sizes the launch.  k must be a multiple of 256; needs oxq_moe_gemm_q8_workspace_bytes() bytes of
  * 256-byte-aligned device scratch.  d_sums (optional, else NULL): exact int32 group sums
  * [(row * n + c) * (k/32) + g] as in oxq_gemm_block_sums_dev. */
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k);

@@ -37,67 +37,254 @@ constexpr float MAGIC_F = 12582912.0f;
 constexpr int BUFFER_FLAGS = 0x00020000;  // raw buffer descriptor word 3 on gfx9: 32-bit data format, no swizzle
 
 // ---- per-format pieces of the tile kernel ------------------------------------------------
-// A 256-weight super-block is walked as 4 groups of 2 sub-blocks; for group g lane (c, h)
-// loads the 16 bytes at QS_OFF + 32*g + 16*h of its row's block.
+// 256 consecutive weights of a row (a K-quant super-block, or 8 blocks of the 32-weight
+// formats) are walked as 4 groups of 2 sub-blocks of 32 weights; sub-block s meets the
+// activation block 8*blk + s.  For each group a lane (c, h) fetches NQ 16-byte pieces of its
+// row and turns them into the B operands of the MFMAs of both sub-blocks.  A format says:
+//   sub_block(g, e)   which sub-block (0..7) the e-th of group g is
+//   fetch             the lane's NQ loads for group g (scalar offset + fixed lane offset)
+//   operands          int8 B operands from those bytes: one K = 32 operand per sub-block, or
+//                     (KSPLIT = 2, scales every 16 weights) one K = 16 operand per half
+//   load_hdr/factors  the fp32 scale factors of a row's sub-blocks: dsc per (sub-block, half)
+//                     and, HAS_MIN, the factor of the zero-point term
+//   ACT_PERM          the byte order the activations must have so that k-slots line up
 
-// Q4_K (reference/q4_k.rs:27-102): those 16 bytes carry weights 16h..16h+15 of sub-block 2g
-// in the low nibbles and of sub-block 2g+1 in the high nibbles.
+typedef long i64x1;
+
+template <int KSPLIT>
+struct BOperand;
+template <>
+struct BOperand<1> {
+    v4i k32;  // 16 bytes: k-slots 16h..16h+15 of the sub-block
+};
+template <>
+struct BOperand<2> {
+    long k16[2];  // per 16-weight half: 8 bytes, k-slots 8h..8h+7 of the half
+};
+
+__device__ __forceinline__ u32x4 buf16(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+    return __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 0);
+}
+
+// Q4_K (reference/q4_k.rs:27-102): 144 B = d, dmin, 12 B of 6-bit scales/mins, 128 B nibbles.
+// The lane's 16 bytes qs[32g + 16h ..] carry weights 16h..16h+15 of sub-block 2g in the low
+// nibbles and of sub-block 2g+1 in the high nibbles.
 struct TileQ4K {
-    static constexpr uint32_t TYPE = OXQ_TYPE_Q4_K, BLOCK_BYTES = 144, QS_OFF = 16;
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q4_K, BLOCK_BYTES = 144;
     static constexpr bool HAS_MIN = true;
-    static constexpr int ACT_PERM = 0;  // activation bytes stay in column order
-    // hd = the 16 header bytes: d | dmin<<16, scales[0..4], [4..8], [8..12] (decode_scales_mins, :27-49)
-    static __device__ __forceinline__ void scales(const u32x4 hd, uint32_t s, float &dsc, float &qneg) {
+    static constexpr int ACT_PERM = 0, NQ = 1, KSPLIT = 1;
+    struct Hdr {
+        u32x4 w;  // d | dmin<<16, scales[0..4], [4..8], [8..12]
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 16 + 32 * g);
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t,
+                                                    Hdr &hd) {
+        hd.w = buf16(rs, row_off, so_blk);
+    }
+    // decode_scales_mins, reference/q4_k.rs:27-49
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t, uint32_t s, float (&dsc)[KSPLIT], float &qneg) {
         const uint32_t sh = 8 * (s & 3);
         uint32_t sc, mn;
         if (s < 4) {
-            sc = (hd[1] >> sh) & 63;
-            mn = (hd[2] >> sh) & 63;
+            sc = (hd.w[1] >> sh) & 63;
+            mn = (hd.w[2] >> sh) & 63;
         } else {
-            sc = ((hd[3] >> sh) & 15) | (((hd[1] >> (sh + 6)) & 3) << 4);
-            mn = ((hd[3] >> (sh + 4)) & 15) | (((hd[2] >> (sh + 6)) & 3) << 4);
+            sc = ((hd.w[3] >> sh) & 15) | (((hd.w[1] >> (sh + 6)) & 3) << 4);
+            mn = ((hd.w[3] >> (sh + 4)) & 15) | (((hd.w[2] >> (sh + 6)) & 3) << 4);
         }
-        dsc = h2f(hd[0] & 0xFFFF) * (float)sc;       // reference/q4_k.rs:280, exact
-        qneg = -(h2f(hd[0] >> 16) * (float)mn);      // reference/q4_k.rs:281, exact
+        dsc[0] = h2f(hd.w[0] & 0xFFFF) * (float)sc;  // reference/q4_k.rs:280, exact
+        qneg = -(h2f(hd.w[0] >> 16) * (float)mn);    // reference/q4_k.rs:281, exact
     }
-    static __device__ __forceinline__ void operands(const u32x4 qs, v4i (&bop)[2]) {
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t, BOperand<1> (&bop)[2]) {
         for (int i = 0; i < 4; i++) {
-            bop[0][i] = (int)(qs[i] & 0x0F0F0F0Fu);
-            bop[1][i] = (int)((qs[i] >> 4) & 0x0F0F0F0Fu);
+            bop[0].k32[i] = (int)(qs[0][i] & 0x0F0F0F0Fu);
+            bop[1].k32[i] = (int)((qs[0][i] >> 4) & 0x0F0F0F0Fu);
         }
     }
 };
 
-// IQ4_XS (reference/iq4_xs.rs:47-97): the 16 bytes are the whole sub-block 2g+h, byte j =
-// codebook indices of weights 2j (low nibble) and 2j+1 (high).  The two halves of the wave
-// trade 8 bytes (v_permlane32_swap) so that lane (c, h) ends up with bytes 8h..8h+7 of
-// sub-block 2g and of sub-block 2g+1; the table lookup then yields weights
-// 16h + {0,2,4,6, 1,3,5,7, 8,10,12,14, 9,11,13,15}, and the activation bytes are stored in
-// that same order by the preparation kernel (ACT_PERM).
+// Swap so that, of two 16-byte pieces held one by each half of the wave (half h holds piece
+// h), every lane ends up with bytes 8h..8h+7 of piece 0 (x[0]) and of piece 1 (x[1]).
+__device__ __forceinline__ void halves_to_pieces(const u32x4 q, uint32_t (&x)[2][2]) {
+    const auto s02 = __builtin_amdgcn_permlane32_swap(q[0], q[2], false, false);
+    const auto s13 = __builtin_amdgcn_permlane32_swap(q[1], q[3], false, false);
+    x[0][0] = s02[0];
+    x[0][1] = s13[0];
+    x[1][0] = s02[1];
+    x[1][1] = s13[1];
+}
+
+// IQ4_XS (reference/iq4_xs.rs:47-97): 136 B = d, scales_h, scales_l, 128 B of indices.  The
+// lane's 16 bytes are the whole sub-block 2g+h, byte j = codebook indices of weights 2j (low
+// nibble) and 2j+1 (high).  After halves_to_pieces the table lookup yields weights
+// 16h + {0,2,4,6, 1,3,5,7, 8,10,12,14, 9,11,13,15}; the preparation kernel stores the
+// activation bytes in that same order (ACT_PERM = 1).
 struct TileIQ4XS {
-    static constexpr uint32_t TYPE = OXQ_TYPE_IQ4_XS, BLOCK_BYTES = 136, QS_OFF = 8;
+    static constexpr uint32_t TYPE = OXQ_TYPE_IQ4_XS, BLOCK_BYTES = 136;
     static constexpr bool HAS_MIN = false;
-    static constexpr int ACT_PERM = 1;
-    // hd = the first 16 bytes: d | scales_h<<16, scales_l, (qs...) (unpack_sub_scale, :47-53)
-    static __device__ __forceinline__ void scales(const u32x4 hd, uint32_t s, float &dsc, float &qneg) {
-        const uint32_t ls = ((hd[1] >> (4 * s)) & 15) | ((((hd[0] >> 16) >> (2 * s)) & 3) << 4);
-        dsc = h2f(hd[0] & 0xFFFF) * (float)((int)ls - 32);  // reference/iq4_xs.rs:81, exact
+    static constexpr int ACT_PERM = 1, NQ = 1, KSPLIT = 1;
+    struct Hdr {
+        u32x4 w;  // d | scales_h<<16, scales_l, (indices)
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 8 + 32 * g);
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t,
+                                                    Hdr &hd) {
+        hd.w = buf16(rs, row_off, so_blk);
+    }
+    // unpack_sub_scale, reference/iq4_xs.rs:47-53; scale = d * ls first, :81
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t, uint32_t s, float (&dsc)[KSPLIT], float &qneg) {
+        const uint32_t ls = ((hd.w[1] >> (4 * s)) & 15) | ((((hd.w[0] >> 16) >> (2 * s)) & 3) << 4);
+        dsc[0] = h2f(hd.w[0] & 0xFFFF) * (float)((int)ls - 32);  // exact
         qneg = 0.0f;
     }
-    static __device__ __forceinline__ void operands(const u32x4 qs, v4i (&bop)[2]) {
-        const auto s02 = __builtin_amdgcn_permlane32_swap(qs[0], qs[2], false, false);
-        const auto s13 = __builtin_amdgcn_permlane32_swap(qs[1], qs[3], false, false);
-        const uint32_t x[2][2] = {{s02[0], s13[0]}, {s02[1], s13[1]}};
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t, BOperand<1> (&bop)[2]) {
+        uint32_t x[2][2];
+        halves_to_pieces(qs[0], x);
         for (int e = 0; e < 2; e++)
             for (int i = 0; i < 2; i++) {
-                bop[e][2 * i] = (int)FmtIQ4XS::lut4(x[e][i] & 0x0F0F0F0Fu);
-                bop[e][2 * i + 1] = (int)FmtIQ4XS::lut4((x[e][i] >> 4) & 0x0F0F0F0Fu);
+                bop[e].k32[2 * i] = (int)FmtIQ4XS::lut4(x[e][i] & 0x0F0F0F0Fu);
+                bop[e].k32[2 * i + 1] = (int)FmtIQ4XS::lut4((x[e][i] >> 4) & 0x0F0F0F0Fu);
             }
     }
 };
 
-// One thread per (token, activation block): payload copy (optionally permuted inside each
-// 16-byte half to the order the weight lookup produces), P = da * sum(q), da.
+// Q4_0 (reference/q4_0.rs:22-49): 18 B = d, 16 B of nibbles, byte j = weights 2j (low) and
+// 2j+1 (high), each minus 8.  Eight blocks make the 256-weight step.  Same interleave as
+// IQ4_XS; the "- 8" goes through the zero-point term: sum (q-8) a = sum q a - 8 sum a.
+struct TileQ4_0 {
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q4_0, BLOCK_BYTES = 8 * 18;
+    static constexpr bool HAS_MIN = true;
+    static constexpr int ACT_PERM = 1, NQ = 1, KSPLIT = 1;
+    struct Hdr {
+        uint32_t d[8];  // f16 scale bits of the lane's sub-blocks
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 18 * h, so_blk + 36 * g + 2);  // block 2g + h, its 16 nibble bytes
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk,
+                                                    uint32_t s0, Hdr &hd) {
+#pragma unroll
+        for (int e = 0; e < SPL; e++)
+            hd.d[e] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row_off + 18 * (s0 + e), so_blk, 0);
+    }
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t e, uint32_t, float (&dsc)[KSPLIT], float &qneg) {
+        dsc[0] = h2f(hd.d[e]);
+        qneg = -(8.0f * dsc[0]);  // exact
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t, BOperand<1> (&bop)[2]) {
+        uint32_t x[2][2];
+        halves_to_pieces(qs[0], x);
+        for (int e = 0; e < 2; e++)
+            for (int i = 0; i < 2; i++) {
+                bop[e].k32[2 * i] = (int)(x[e][i] & 0x0F0F0F0Fu);
+                bop[e].k32[2 * i + 1] = (int)((x[e][i] >> 4) & 0x0F0F0F0Fu);
+            }
+    }
+};
+
+// Q8_0 weights (reference/q8_0.rs:22-47): 34 B = d, 32 int8.  Eight blocks make the
+// 256-weight step; the payload is the B operand as it is.
+struct TileQ8_0 {
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q8_0, BLOCK_BYTES = 8 * 34;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int ACT_PERM = 0, NQ = 2, KSPLIT = 1;
+    struct Hdr {
+        uint32_t d[8];
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 68 * g + 2);
+        qs[1] = buf16(rs, row_off + 16 * h, so_blk + 68 * g + 36);
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk,
+                                                    uint32_t s0, Hdr &hd) {
+#pragma unroll
+        for (int e = 0; e < SPL; e++)
+            hd.d[e] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row_off + 34 * (s0 + e), so_blk, 0);
+    }
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t e, uint32_t, float (&dsc)[KSPLIT], float &qneg) {
+        dsc[0] = h2f(hd.d[e]);
+        qneg = 0.0f;
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t, BOperand<1> (&bop)[2]) {
+        for (int e = 0; e < 2; e++)
+            for (int i = 0; i < 4; i++) bop[e].k32[i] = (int)qs[e][i];
+    }
+};
+
+// Q6_K (reference/q6_k.rs:25-75): 210 B = ql[128], qh[64], 16 int8 scales, d.  Scales change
+// every 16 weights, so each 32-weight sub-block is two K = 16 MFMAs with their own factor.
+// Group g = (half hh = g / 2, pair p = g % 2): ql[64hh + 32p + l] holds, for l = 0..31, the low
+// 4 bits of sub-block 4hh + p (low nibble) and of sub-block 4hh + p + 2 (high nibble); their
+// upper 2 bits sit in qh[32hh + l] at bit 2p and 2p + 4.  Lane (c, h) fetches ql and qh bytes
+// 16h..16h+15 (the 16-weight half h of both sub-blocks); halves_to_pieces hands every lane
+// bytes 8h..8h+7 of both halves, which is the k-slot order of the K = 16 operand and of the
+// activations as the preparation kernel stores them (ACT_PERM = 2).
+struct TileQ6K {
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q6_K, BLOCK_BYTES = 210;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int ACT_PERM = 2, NQ = 2, KSPLIT = 2;
+    struct Hdr {
+        u32x4 sc;    // 16 int8 scales
+        uint32_t d;  // f16 bits
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 4 * (g >> 1) + (g & 1) + 2 * e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 64 * (g >> 1) + 32 * (g & 1));
+        qs[1] = buf16(rs, row_off + 16 * h, so_blk + 128 + 32 * (g >> 1));
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t,
+                                                    Hdr &hd) {
+        hd.sc = buf16(rs, row_off, so_blk + 192);
+        hd.d = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row_off, so_blk + 208, 0);
+    }
+    // scale of half `is` of sub-block s: scales[2s + is] (reference/q6_k.rs:55-72: index 8hh + is + 2j)
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t, uint32_t s, float (&dsc)[KSPLIT], float &qneg) {
+        const uint32_t pair = hd.sc[s >> 1] >> (16 * (s & 1));
+        const float d = h2f(hd.d);
+        dsc[0] = d * (float)(int)(int8_t)(pair & 0xFF);         // reference/q6_k.rs:62, exact
+        dsc[1] = d * (float)(int)(int8_t)((pair >> 8) & 0xFF);
+        qneg = 0.0f;
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t g, BOperand<2> (&bop)[2]) {
+        uint32_t l[2][2], hb[2][2];
+        halves_to_pieces(qs[0], l);
+        halves_to_pieces(qs[1], hb);
+        const uint32_t p2 = 2 * (g & 1);
+        for (int e = 0; e < 2; e++)
+            for (int is = 0; is < 2; is++) {
+                uint32_t q[2];
+                for (int i = 0; i < 2; i++) {
+                    const uint32_t lo = (l[is][i] >> (4 * e)) & 0x0F0F0F0Fu;
+                    const uint32_t hi = ((hb[is][i] >> (p2 + 4 * e)) & 0x03030303u) << 4;
+                    // q - 32 per byte (0..63 -> -32..31) without carries between bytes
+                    q[i] = (((lo | hi) | 0x80808080u) - 0x20202020u) ^ 0x80808080u;
+                }
+                bop[e].k16[is] = (long)(((uint64_t)q[1] << 32) | q[0]);
+            }
+    }
+};
+
+// One thread per (token, activation block): payload copy in the byte order the format's B
+// operands have (PERM 1: even bytes then odd bytes inside each 8; PERM 2: the two 8-byte
+// halves of each 16-weight half side by side), P = da * sum(q), da.
 template <int PERM>
 __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict__ A, uint8_t *__restrict__ q8t,
                                                      float *__restrict__ P, uint16_t *__restrict__ da16, uint32_t m,
@@ -118,7 +305,12 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
         s = sdot4(q[0][i], 0x01010101u, s);
         s = sdot4(q[1][i], 0x01010101u, s);
     }
-    if (PERM) {
+    if (PERM == 2) {  // [half 0 | half 1] x [bytes 0-7 | 8-15] -> bytes 8h..8h+7 of both halves in 16-byte piece h
+        const u32x4 x0 = q[0], x1 = q[1];
+        q[0] = u32x4{x0[0], x0[1], x1[0], x1[1]};
+        q[1] = u32x4{x0[2], x0[3], x1[2], x1[3]};
+    }
+    if (PERM == 1) {
         for (int hf = 0; hf < 2; hf++) {
             const u32x4 x = q[hf];
             q[hf][0] = __builtin_amdgcn_perm(x[1], x[0], 0x06040200u);
@@ -162,12 +354,14 @@ __device__ __forceinline__ void gemm_tile_body(
     size_t w_stride) {
     constexpr int WN = 4 / WM;
     constexpr int WG_TOK = 32 * MT * WM, WG_ROWS = 32 * NT * WN, MTILES = MT * WM;
-    constexpr int NP = F::HAS_MIN ? 3 : 2;
-    constexpr int W_ROWS = 32 * NT;                  // weight rows of one wave
-    constexpr int LPR = 64 / W_ROWS, SPL = 8 / LPR;  // scale decode: lanes per row, sub-blocks per lane
+    constexpr int KS = F::KSPLIT;                     // MFMAs (and scale factors) per sub-block
+    constexpr int NP = 2 * KS + (F::HAS_MIN ? 1 : 0);  // fp32 factor planes per sub-block in LDS
+    constexpr int W_ROWS = 32 * NT;                   // weight rows of one wave
+    constexpr int LPR = 64 / W_ROWS, SPL = 8 / LPR;   // scale decode: lanes per row, sub-blocks per lane
     static_assert(NT <= 2 && (DIST == 1 || DIST == 2 || DIST == 4), "tile configuration");
     extern __shared__ uint16_t lds_da[];            // [nsb][MTILES][2 halves][16] f16 token scales
-    __shared__ float lds_sc[4][8][NP][W_ROWS];      // [wave][sub-block][dsc, -MAGIC*dsc, -dmin*mn][row of the wave]
+    // [wave][sub-block][KS x dsc, KS x -MAGIC*dsc, zero-point factor][row of the wave]
+    __shared__ float lds_sc[4][8][NP][W_ROWS];
     const uint32_t nsb = k / 32, nblk = k / 256, ngrp = nblk * 4;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
@@ -213,18 +407,25 @@ __device__ __forceinline__ void gemm_tile_body(
     // factors of the next super-block after its last read of the current ones.
     const uint32_t drow = lane % W_ROWS, ds0 = SPL * (lane / W_ROWS);
     const uint32_t hrow_off = (min(n_wave + drow, n - 1) - n_base) * row_bytes;
-    auto decode = [&](const u32x4 hd) {
+    auto decode = [&](const typename F::Hdr &hd) {
 #pragma unroll
         for (int e = 0; e < SPL; e++) {
             const uint32_t s = ds0 + e;
-            float dsc, qneg;
-            F::scales(hd, s, dsc, qneg);
-            lds_sc[wave][s][0][drow] = dsc;
-            lds_sc[wave][s][1][drow] = -(MAGIC_F * dsc);  // exact
+            float dsc[KS], qneg;
+            F::factors(hd, e, s, dsc, qneg);
+#pragma unroll
+            for (int is = 0; is < KS; is++) {
+                lds_sc[wave][s][is][drow] = dsc[is];
+                lds_sc[wave][s][KS + is][drow] = -(MAGIC_F * dsc[is]);  // exact
+            }
             if (F::HAS_MIN) lds_sc[wave][s][NP - 1][drow] = qneg;
         }
     };
-    decode(__builtin_amdgcn_raw_buffer_load_b128(rs_w, hrow_off, 0, 0));
+    {
+        typename F::Hdr hd;
+        F::template load_hdr<SPL>(rs_w, hrow_off, 0, ds0, hd);
+        decode(hd);
+    }
 
     v16f acc[MT][NT];
     v16i magic;
@@ -233,61 +434,69 @@ __device__ __forceinline__ void gemm_tile_body(
         for (int b = 0; b < NT; b++)
             for (int i = 0; i < 16; i++) acc[a][b][i] = 0.0f;
 
-    uint32_t nrow[NT], wq_off[NT];  // wq_off: the lane's 16 bytes of group 0 of its row
+    uint32_t nrow[NT], wq_off[NT];  // wq_off: byte offset of the lane's row from the descriptor base
     for (int nt = 0; nt < NT; nt++) {
         nrow[nt] = n_wave + nt * 32 + c;
-        wq_off[nt] = (min(nrow[nt], n - 1) - n_base) * row_bytes + F::QS_OFF + 16 * h;
+        wq_off[nt] = (min(nrow[nt], n - 1) - n_base) * row_bytes;
     }
     uint32_t aq_off[MT], pq_off[MT];
     for (int mt = 0; mt < MT; mt++) {
         const uint32_t tok = m_wave + mt * 32 + c;  // always < mpad
         aq_off[mt] = tok * 32 + 16 * h;             // the lane's 16 bytes of its token's activation block
-        pq_off[mt] = (h * mpad + tok) * 4;          // P of sub-block h of the pair
+        pq_off[mt] = (h * mpad + tok) * 4;          // P of the sub-block the lane's half feeds to the min term
     }
 
+    struct Wq {
+        u32x4 q[NT][F::NQ];
+    };
     struct Ops {
         u32x4 a[2][MT];  // [sub-block of the pair][token tile] 16 activation bytes
-        float pv[MT];    // P of sub-block 2g + h
+        float pv[MT];    // P of sub-block sub_block(g, h)
     };
     // group index G = 4*blk + g; groups past the end re-read the last one (result unused)
-    auto fetch_w = [&](u32x4 (&qs)[NT], uint32_t G) {
+    auto fetch_w = [&](Wq &w, uint32_t G) {
         G = min(G, ngrp - 1);
-        const uint32_t w_so = (G >> 2) * F::BLOCK_BYTES + 32 * (G & 3);
-        for (int nt = 0; nt < NT; nt++) qs[nt] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, wq_off[nt], w_so, 0);
+        for (int nt = 0; nt < NT; nt++) F::fetch(rs_w, wq_off[nt], h, (G >> 2) * F::BLOCK_BYTES, G & 3, w.q[nt]);
     };
     auto fetch_a = [&](Ops &o, uint32_t G) {
         G = min(G, ngrp - 1);
+        const uint32_t blk8 = (G >> 2) * 8, g = G & 3;
         for (int e = 0; e < 2; e++)
             for (int mt = 0; mt < MT; mt++)
-                o.a[e][mt] = __builtin_amdgcn_raw_buffer_load_b128(rs_a, aq_off[mt], (2 * G + e) * mpad * 32, 0);
+                o.a[e][mt] = buf16(rs_a, aq_off[mt], (blk8 + F::sub_block(g, e)) * mpad * 32);
         if (F::HAS_MIN)
-            for (int mt = 0; mt < MT; mt++)
-                o.pv[mt] = __builtin_bit_cast(
-                    float, __builtin_amdgcn_raw_buffer_load_b32(rs_p, pq_off[mt], 2 * G * mpad * 4, 0));
+            for (int mt = 0; mt < MT; mt++)  // sub_block(g, 0) and (g, 1) are adjacent for every format with a min term
+                o.pv[mt] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                         rs_p, pq_off[mt], (blk8 + F::sub_block(g, 0)) * mpad * 4, 0));
     };
 
-    // One pair of sub-blocks (2g, 2g+1): 2*MT*NT int8 MFMA tiles, each followed by its 32
-    // VALU operations; the MFMA of tile t+2 is issued before the VALU work of tile t+1 so
-    // that the matrix core runs ahead of the VALU.
-    auto compute = [&](const u32x4 (&qs)[NT], const Ops &o, uint32_t blk, uint32_t g) {
-        constexpr int T = 2 * MT * NT;
-        v4i bop[NT][2];
-        for (int nt = 0; nt < NT; nt++) F::operands(qs[nt], bop[nt]);
+    // One group: 2 sub-blocks x KS MFMAs x MT x NT tiles, each MFMA followed by its 32 VALU
+    // operations; the MFMA of tile t+2 is issued before the VALU work of tile t+1 so that the
+    // matrix core runs ahead of the VALU.
+    auto compute = [&](const Wq &w, const Ops &o, uint32_t blk, uint32_t g) {
+        constexpr int T = 2 * KS * MT * NT;
+        BOperand<KS> bop[NT][2];
+        for (int nt = 0; nt < NT; nt++) F::operands(w.q[nt], g, bop[nt]);
         auto mfma_tile = [&](int t) {
-            const int e = t / (MT * NT), mt = (t / NT) % MT, nt = t % NT;
-            v4i aop;
-            for (int i = 0; i < 4; i++) aop[i] = (int)o.a[e][mt][i];
-            return __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop[nt][e], magic, 0, 0, 0);
+            const int e = t / (KS * MT * NT), is = (t / (MT * NT)) % KS, mt = (t / NT) % MT, nt = t % NT;
+            if constexpr (KS == 1) {
+                v4i aop;
+                for (int i = 0; i < 4; i++) aop[i] = (int)o.a[e][mt][i];
+                return __builtin_amdgcn_mfma_i32_32x32x32_i8(aop, bop[nt][e].k32, magic, 0, 0, 0);
+            } else {
+                const long aop = (long)(((uint64_t)o.a[e][mt][2 * is + 1] << 32) | o.a[e][mt][2 * is]);
+                return __builtin_amdgcn_mfma_i32_32x32x16_i8(aop, bop[nt][e].k16[is], magic, 0, 0, 0);
+            }
         };
         v16i dq[2];
         dq[0] = mfma_tile(0);
         if (T > 1) dq[1] = mfma_tile(1);
 #pragma unroll
         for (int t = 0; t < T; t++) {
-            const int e = t / (MT * NT), mt = (t / NT) % MT, nt = t % NT;
-            const uint32_t s = 2 * g + e, j = blk * 8 + s;
-            const float dsc = lds_sc[wave][s][0][nt * 32 + c];
-            const float nc2 = lds_sc[wave][s][1][nt * 32 + c];
+            const int e = t / (KS * MT * NT), is = (t / (MT * NT)) % KS, mt = (t / NT) % MT, nt = t % NT;
+            const uint32_t s = F::sub_block(g, e), j = blk * 8 + s;
+            const float dsc = lds_sc[wave][s][is][nt * 32 + c];
+            const float nc2 = lds_sc[wave][s][KS + is][nt * 32 + c];
             const u32x4 *dp = reinterpret_cast<const u32x4 *>(&lds_da[((j * MTILES + wm * MT + mt) * 2 + h) * 16]);
             const u32x4 dav[2] = {dp[0], dp[1]};
             const v16i dres = dq[t & 1];
@@ -302,20 +511,20 @@ __device__ __forceinline__ void gemm_tile_body(
                 if (DUMP) {
                     const uint32_t row = m_wave + mt * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
                     if (row < row_end && nrow[nt] < n)
-                        sums[((size_t)row * n + nrow[nt]) * nsb + j] = (int)(dbits - MAGIC_BITS);
+                        sums[((size_t)row * n + nrow[nt]) * (nsb * KS) + j * KS + is] = (int)(dbits - MAGIC_BITS);
                 }
             }
             if (t + 2 < T) dq[t & 1] = mfma_tile(t + 2);
-            if (F::HAS_MIN && e == 1) {
-                // min term of sub-blocks 2g (lanes h = 0) and 2g+1 (lanes h = 1):
-                // acc[token][row] += P[token][s] * (-dmin*mn)[row][s], contracted over the pair
-                const float qv = lds_sc[wave][2 * g + h][NP - 1][nt * 32 + c];
+            if (F::HAS_MIN && e == 1 && is == KS - 1) {
+                // zero-point term of the group's sub-blocks (lanes h = 0: the first, h = 1: the second):
+                // acc[token][row] += P[token][s] * factor[row][s], contracted over the pair
+                const float qv = lds_sc[wave][F::sub_block(g, 0) + h][NP - 1][nt * 32 + c];
                 acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(o.pv[mt], qv, acc[mt][nt], 0, 0, 0);
             }
         }
     };
 
-    u32x4 wring[DIST][NT];
+    Wq wring[DIST];
     Ops ops0, ops1;
 #pragma unroll
     for (int d = 0; d < DIST; d++) fetch_w(wring[d], d);
@@ -324,18 +533,18 @@ __device__ __forceinline__ void gemm_tile_body(
 
     for (uint32_t blk = 0; blk < nblk; blk++) {
         const uint32_t nxt = min(blk + 1, nblk - 1);  // last trip: harmless re-read
-        const u32x4 hd = __builtin_amdgcn_raw_buffer_load_b128(rs_w, hrow_off, nxt * F::BLOCK_BYTES, 0);
+        typename F::Hdr hd;
+        F::template load_hdr<SPL>(rs_w, hrow_off, nxt * F::BLOCK_BYTES, ds0, hd);
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            u32x4 qs[NT];
-            for (int nt = 0; nt < NT; nt++) qs[nt] = wring[g % DIST][nt];
+            const Wq w = wring[g % DIST];
             fetch_w(wring[g % DIST], blk * 4 + g + DIST);  // slot consumed: refill it DIST groups ahead
             if (g & 1) {
                 fetch_a(ops0, blk * 4 + g + 1);
-                compute(qs, ops1, blk, g);
+                compute(w, ops1, blk, g);
             } else {
                 fetch_a(ops1, blk * 4 + g + 1);
-                compute(qs, ops0, blk, g);
+                compute(w, ops0, blk, g);
             }
         }
         __builtin_amdgcn_wave_barrier();  // the wave's reads of this super-block's factors come first
@@ -412,7 +621,8 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
     const uint32_t m_tiles = (rows + WG_TOK - 1) / WG_TOK, n_tiles = (a.n + WG_ROWS - 1) / WG_ROWS;
     const dim3 grid(8 * ((n_tiles + 7) / 8) * m_tiles, a.offsets ? a.n_experts : 1);
     const size_t lds = (size_t)(a.k / 32) * WG_TOK * 2;
-    auto kern = OCC == 3 ? &gemm_tile_kernel_occ3<F, MT, NT, WM, DIST, DUMP> : &gemm_tile_kernel<F, MT, NT, WM, DIST, DUMP>;
+    auto kern = &gemm_tile_kernel<F, MT, NT, WM, DIST, DUMP>;
+    if constexpr (OCC == 3) kern = &gemm_tile_kernel_occ3<F, MT, NT, WM, DIST, DUMP>;
     if (lds > 32 * 1024) {  // beyond the default dynamic LDS limit: opt in (up to the 160 KB of a CU)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -429,26 +639,23 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
 template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
     const uint32_t rows = a.offsets ? a.max_rows : a.m;
+    // formats with a scale every 16 weights keep two MFMA results per tile in flight: one row tile per wave
+    constexpr int NTB = F::KSPLIT == 2 ? 1 : 2;
     if (a.sums)
-        return rows > 32 ? launch_tile<F, 2, 2, 2, 1, true>(a, p, stream) : launch_tile<F, 1, 2, 1, 2, true>(a, p, stream);
+        return rows > 32 ? launch_tile<F, 2, NTB, 2, 1, true>(a, p, stream) : launch_tile<F, 1, NTB, 1, 2, true>(a, p, stream);
     switch (g_gemm_variant) {
     case 1: return launch_tile<F, 2, 1, 2, 1, false>(a, p, stream);
-    case 2: return launch_tile<F, 1, 2, 2, 1, false>(a, p, stream);
     case 3: return launch_tile<F, 2, 2, 2, 1, false>(a, p, stream);
     case 4: return launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
     case 5: return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
-    case 6: return launch_tile<F, 1, 2, 2, 1, false, 3>(a, p, stream);
-    case 7: return launch_tile<F, 1, 1, 2, 1, false, 3>(a, p, stream);
-    case 11: return launch_tile<F, 1, 2, 1, 1, false>(a, p, stream);
     case 12: return launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
     case 13: return launch_tile<F, 1, 2, 1, 4, false>(a, p, stream);
     case 14: return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
-    case 15: return launch_tile<F, 1, 1, 1, 4, false>(a, p, stream);
     case 16: return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
     default:
-        if (rows > 32) return launch_tile<F, 2, 2, 2, 1, false>(a, p, stream);
+        if (rows > 32) return launch_tile<F, 2, NTB, 2, 1, false>(a, p, stream);
         // few tokens: 256-row tiles unless that leaves compute units without a work group
-        if ((size_t)((a.n + 255) / 256) * (a.offsets ? a.n_experts : 1) >= device_cus())
+        if (NTB == 2 && (size_t)((a.n + 255) / 256) * (a.offsets ? a.n_experts : 1) >= device_cus())
             return launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
         return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
     }
@@ -463,7 +670,10 @@ size_t gemm_workspace_bytes(uint32_t m, uint32_t k) {
 bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t k) {
     // LDS holds the f16 token scales of up to 128 tokens for the whole k (k/32 * 256 bytes)
     // beside up to 24 KB of decoded weight scales; up to k = 8192 two work groups share a CU
-    return (type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS) && m >= 8 && (size_t)(k / 32) * 256 <= 128 * 1024 &&
+    const bool known = type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K ||
+                       type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0;
+    // the 32-weight formats are walked eight blocks at a time
+    return known && k % 256 == 0 && m >= 8 && (size_t)(k / 32) * 256 <= 128 * 1024 &&
            gemm_workspace_bytes(m, k) < 0x7FFFFFFFull;
 }
 
@@ -477,14 +687,24 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
     float *P = reinterpret_cast<float *>(q8t + (size_t)nsb * mpad * 32);
     uint16_t *da16 = reinterpret_cast<uint16_t *>(q8t + (size_t)nsb * mpad * 36);
     const dim3 pgrid((mpad * nsb + 255) / 256);
-    if (type == OXQ_TYPE_IQ4_XS)
+    const int perm = type == OXQ_TYPE_Q6_K ? TileQ6K::ACT_PERM
+                     : (type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q4_0) ? TileIQ4XS::ACT_PERM : 0;
+    if (perm == 2)
+        hipLaunchKernelGGL(gemm_prep_acts<2>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb);
+    else if (perm == 1)
         hipLaunchKernelGGL(gemm_prep_acts<1>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb);
     else
         hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const TilePlan plan = {q8t, P, da16, mpad};
-    return type == OXQ_TYPE_IQ4_XS ? launch_tiles<TileIQ4XS>(a, plan, stream) : launch_tiles<TileQ4K>(a, plan, stream);
+    switch (type) {
+    case OXQ_TYPE_Q4_K: return launch_tiles<TileQ4K>(a, plan, stream);
+    case OXQ_TYPE_IQ4_XS: return launch_tiles<TileIQ4XS>(a, plan, stream);
+    case OXQ_TYPE_Q6_K: return launch_tiles<TileQ6K>(a, plan, stream);
+    case OXQ_TYPE_Q8_0: return launch_tiles<TileQ8_0>(a, plan, stream);
+    default: return launch_tiles<TileQ4_0>(a, plan, stream);
+    }
 }
 
 }  // namespace oxq

@@ -333,6 +333,15 @@ def test_gemm_matches_oracle(hip, ref, t):
     assert_close(y, ref.gemm_q8(t, w, x, m, n, k_), "gemm")
 
 
+def _tile_zero_point(t, acts, rows, k_):
+    """The tile kernel multiplies Q4_0's unsigned nibbles and applies the "- 8" of (q - 8) in fp32
+    through the zero-point term, so its integer sums are sum q*a = sum (q-8)*a + 8 * sum a."""
+    if t != O.Q4_0:
+        return 0
+    a = acts.reshape(rows, k_ // 32, 34)[:, :, 2:].view(np.int8).astype(np.int32).sum(axis=2)
+    return (8 * a)[:, None, :]
+
+
 def _oracle_prefill(ref, t, w, acts, m, n, k_, rows=None):
     """m fused matvecs (threaded row split) on already-quantized activation rows."""
     arb = k_ // 32 * 34
@@ -342,9 +351,9 @@ def _oracle_prefill(ref, t, w, acts, m, n, k_, rows=None):
 
 @pytest.mark.parametrize("shape", [(8, 32, 256), (33, 100, 1024), (128, 160, 512), (200, 257, 1024), (64, 64, 4096),
                                    (130, 129, 2048)], ids=lambda s: "x".join(map(str, s)))
-@pytest.mark.parametrize("t", [O.Q4_K, O.IQ4_XS], ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
 def test_prefill_tile_kernel(hip, ref, shape, t):
-    """Q4_K / IQ4_XS x Q8_0 int8-MFMA tile kernel: integer sub-block sums bit-exact, fp32 within
+    """Weights of every format x Q8_0 activations on the int8-MFMA tile kernel: integer sub-block sums bit-exact, fp32 within
     1e-5, ragged tile edges in both directions, overwrite and accumulate."""
     import torch
     m, n, k_ = shape
@@ -368,13 +377,13 @@ def test_prefill_tile_kernel(hip, ref, shape, t):
     torch.cuda.synchronize()
     assert torch.equal(dy2, dy + dy)
     # exact integer sums of every (token, weight row, sub-block)
-    dsum = torch.empty((m, n, k_ // 32), dtype=torch.int32, device="cuda")
+    dsum = torch.empty((m, n, k_ // (16 if t == O.Q6_K else 32)), dtype=torch.int32, device="cuda")
     dy3 = torch.empty_like(dy)
     kern.gemm_block_sums_dev(dw, da, dy3, dsum, m, n, k_, workspace=ws)
     torch.cuda.synchronize()
     arb = k_ // 32 * 34
     want = np.stack([ref.block_sums(t, w, acts[r * arb:(r + 1) * arb], n, k_) for r in range(m)])
-    assert np.array_equal(dsum.cpu().numpy(), want)
+    assert np.array_equal(dsum.cpu().numpy() - _tile_zero_point(t, acts, m, k_), want)
     assert torch.equal(dy3, dy)
 
 
@@ -423,7 +432,7 @@ def _moe_case(ref, t, n_experts, n_tok, top_k, n, k_, seed):
     return offsets, tok, slot, weights, acts, w
 
 
-@pytest.mark.parametrize("t", [O.IQ4_XS, O.Q4_K], ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
 @pytest.mark.parametrize("cfg", [(8, 64, 2, 96, 1024), (4, 7, 2, 300, 512), (8, 200, 2, 64, 256), (3, 5, 1, 33, 2048)],
                          ids=lambda c: "e%d_t%d_k%d_n%d_k%d" % c)
 def test_moe_grouped_matmul(hip, ref, t, cfg):
@@ -441,20 +450,21 @@ def test_moe_grouped_matmul(hip, ref, t, cfg):
     dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
     doff = torch.from_numpy(offsets).cuda()
     dy = torch.full((rows + 3, n), 7.0, dtype=torch.float32, device="cuda")  # 3 guard rows
-    dsum = torch.full((rows, n, k_ // 32), -1, dtype=torch.int32, device="cuda")
+    groups = k_ // (16 if t == O.Q6_K else 32)
+    dsum = torch.full((rows, n, groups), -1, dtype=torch.int32, device="cuda")
     max_rows = int(np.diff(offsets).max())
     kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy, n, k_, ws, d_sums=dsum)
     torch.cuda.synchronize()
     y = dy.cpu().numpy()
     assert np.all(y[rows:] == 7.0)
     y_ref = np.empty((rows, n), dtype=np.float32)
-    s_ref = np.empty((rows, n, k_ // 32), dtype=np.int32)
+    s_ref = np.empty((rows, n, groups), dtype=np.int32)
     for e in range(n_experts):
         for r in range(offsets[e], offsets[e + 1]):
             y_ref[r] = canonical_ref(ref, t, w[e], acts[r], n, k_)
             s_ref[r] = ref.block_sums(t, w[e], acts[r], n, k_)
     assert_close(y[:rows], y_ref, f"moe {cfg}")
-    assert np.array_equal(dsum.cpu().numpy(), s_ref)
+    assert np.array_equal(dsum.cpu().numpy() - _tile_zero_point(t, acts.reshape(-1), rows, k_), s_ref)
     # production launch (no sums), overwrite then accumulate, max_rows = 0 (unknown)
     dy2 = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
     kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, 0, dy2, n, k_, ws)
