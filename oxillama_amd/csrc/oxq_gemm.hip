@@ -633,9 +633,9 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
     return hipGetLastError();
 }
 
-// Tile shape by use: prefill (many tokens) takes 128 x 128 work-group tiles; few tokens
-// (a mixture-of-experts group, a short prompt) take 32 tokens x 256 rows with the weight
-// bytes fetched further ahead, because that case is bound by the weight stream from HBM.
+// Tile shape by use: many tokens (prefill) take 128-token work-group tiles; few tokens (a
+// mixture-of-experts group, a short prompt, a decode batch) take 32-token tiles with the
+// weight bytes fetched further ahead, because that case is paced by the weight stream.
 template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
     const uint32_t rows = a.offsets ? a.max_rows : a.m;
@@ -653,9 +653,13 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     case 14: return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
     case 16: return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
     default:
-        if (rows > 32) return launch_tile<F, 2, NTB, 2, 1, false>(a, p, stream);
-        // few tokens: 256-row tiles unless that leaves compute units without a work group
-        if (NTB == 2 && (size_t)((a.n + 255) / 256) * (a.offsets ? a.n_experts : 1) >= device_cus())
+        // Measured on MI355X at 14336 x 4096 (Q4_K, Q6_K): up to 64 tokens one 32-token tile per work
+        // group is fastest (the weight stream paces it), up to 384 tokens 64 x 128 tiles, beyond that
+        // 128 x 64 tiles at three waves per SIMD.
+        if (rows > 384) return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
+        if (rows > 64) return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
+        // few tokens: 256-row tiles where that still gives every compute unit a work group
+        if (rows <= 32 && NTB == 2 && (size_t)((a.n + 255) / 256) * (a.offsets ? a.n_experts : 1) >= device_cus())
             return launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
         return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
     }
