@@ -346,26 +346,29 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
 //
 // Grouped form (mixture-of-experts): blockIdx.y = expert; expert e multiplies the token
 // rows offsets[e] .. offsets[e+1]-1 by the weights at W + e * w_stride.
-template <class F, int MT, int NT, int WM, int DIST, bool DUMP>
+template <class F, int MT, int NT, int WM, int DIST, bool DUMP, int ADIST>
 __device__ __forceinline__ void gemm_tile_body(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,
     const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m, uint32_t mpad,
     uint32_t n, uint32_t k, int accumulate, uint32_t m_tiles, uint32_t n_tiles, const int32_t *__restrict__ offsets,
     size_t w_stride) {
-    constexpr int WN = 4 / WM;
-    constexpr int WG_TOK = 32 * MT * WM, WG_ROWS = 32 * NT * WN, MTILES = MT * WM;
+    constexpr bool SPLITK = WM == 0;  // the four waves share one tile and each walk a quarter of k
+    constexpr int WMX = SPLITK ? 1 : WM, WN = SPLITK ? 1 : 4 / WMX;
+    constexpr int WG_TOK = 32 * MT * WMX, WG_ROWS = 32 * NT * WN, MTILES = MT * WMX;
     constexpr int KS = F::KSPLIT;                     // MFMAs (and scale factors) per sub-block
     constexpr int NP = 2 * KS + (F::HAS_MIN ? 1 : 0);  // fp32 factor planes per sub-block in LDS
     constexpr int W_ROWS = 32 * NT;                   // weight rows of one wave
     constexpr int LPR = 64 / W_ROWS, SPL = 8 / LPR;   // scale decode: lanes per row, sub-blocks per lane
-    static_assert(NT <= 2 && (DIST == 1 || DIST == 2 || DIST == 4), "tile configuration");
+    static_assert(NT <= 2 && DIST >= 1, "tile configuration");
     extern __shared__ uint16_t lds_da[];            // [nsb][MTILES][2 halves][16] f16 token scales
     // [wave][sub-block][KS x dsc, KS x -MAGIC*dsc, zero-point factor][row of the wave]
     __shared__ float lds_sc[4][8][NP][W_ROWS];
     const uint32_t nsb = k / 32, nblk = k / 256, ngrp = nblk * 4;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
-    const uint32_t wm = wave % WM, wn = wave / WM;
+    const uint32_t wm = SPLITK ? 0 : wave % WMX, wn = SPLITK ? 0 : wave / WMX;
+    // super-blocks of this wave: all of them, or its quarter
+    const uint32_t blk_begin = SPLITK ? wave * nblk / 4 : 0, blk_end = SPLITK ? (wave + 1) * nblk / 4 : nblk;
 
     const uint32_t xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
     const uint32_t n_tile = (loc / m_tiles) * 8 + xcd, m_tile = loc % m_tiles;
@@ -423,7 +426,7 @@ __device__ __forceinline__ void gemm_tile_body(
     };
     {
         typename F::Hdr hd;
-        F::template load_hdr<SPL>(rs_w, hrow_off, 0, ds0, hd);
+        F::template load_hdr<SPL>(rs_w, hrow_off, min(blk_begin, nblk - 1) * F::BLOCK_BYTES, ds0, hd);
         decode(hd);
     }
 
@@ -524,34 +527,77 @@ __device__ __forceinline__ void gemm_tile_body(
         }
     };
 
-    Wq wring[DIST];
-    Ops ops0, ops1;
+    // Weight ring.  DIST < 4: slot g % DIST is refilled DIST groups ahead as soon as it is consumed.
+    // DIST >= 4 (a multiple of 4): ring[i] holds group 4*blk + i; at the top of a super-block the four
+    // groups DIST ahead are requested into `incoming`, and the ring advances by four at its end.  The
+    // deep form is for few tokens, where the weight stream from HBM paces the kernel and a wave
+    // needs many loads in flight.
+    constexpr int RING = DIST < 4 ? DIST : DIST;
+    static_assert(DIST < 4 || DIST % 4 == 0, "deep prefetch advances by whole super-blocks");
+    Wq wring[RING];
+    // Token bytes: ring of four slots (slot = group % 4), requested ADIST (1..3) groups ahead.
+    static_assert(ADIST >= 1 && ADIST <= 3, "activation prefetch distance");
+    Ops ops[4];
 #pragma unroll
-    for (int d = 0; d < DIST; d++) fetch_w(wring[d], d);
-    fetch_a(ops0, 0);
+    for (int d = 0; d < RING; d++) fetch_w(wring[d], blk_begin * 4 + d);
+#pragma unroll
+    for (int d = 0; d < ADIST; d++) fetch_a(ops[d], blk_begin * 4 + d);
     __syncthreads();
 
-    for (uint32_t blk = 0; blk < nblk; blk++) {
+    for (uint32_t blk = blk_begin; blk < blk_end; blk++) {
         const uint32_t nxt = min(blk + 1, nblk - 1);  // last trip: harmless re-read
+        Wq incoming[DIST < 4 ? 1 : 4];
+        if constexpr (DIST >= 4) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) fetch_w(incoming[i], blk * 4 + DIST + i);
+        }
         typename F::Hdr hd;
         F::template load_hdr<SPL>(rs_w, hrow_off, nxt * F::BLOCK_BYTES, ds0, hd);
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            const Wq w = wring[g % DIST];
-            fetch_w(wring[g % DIST], blk * 4 + g + DIST);  // slot consumed: refill it DIST groups ahead
-            if (g & 1) {
-                fetch_a(ops0, blk * 4 + g + 1);
-                compute(w, ops1, blk, g);
-            } else {
-                fetch_a(ops1, blk * 4 + g + 1);
-                compute(w, ops0, blk, g);
-            }
+            const Wq w = DIST < 4 ? wring[g % (DIST < 4 ? DIST : 1)] : wring[DIST < 4 ? 0 : g];
+            if constexpr (DIST < 4) fetch_w(wring[g % DIST], blk * 4 + g + DIST);  // slot consumed: refill it
+            fetch_a(ops[(g + ADIST) % 4], blk * 4 + g + ADIST);
+            compute(w, ops[g], blk, g);
+        }
+        if constexpr (DIST >= 4) {
+#pragma unroll
+            for (int i = 0; i + 4 < DIST; i++) wring[i] = wring[i + 4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) wring[DIST - 4 + i] = incoming[i];
         }
         __builtin_amdgcn_wave_barrier();  // the wave's reads of this super-block's factors come first
         decode(hd);
         __builtin_amdgcn_wave_barrier();
     }
 
+    if constexpr (SPLITK) {
+        // The four partial tiles meet in LDS; wave w then adds registers 4w..4w+3 of every tile in
+        // the fixed order (w0 + w1) + (w2 + w3) and stores them.
+        __shared__ float lds_red[4][MT * NT][16][64];
+        for (int mt = 0; mt < MT; mt++)
+            for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) lds_red[wave][mt * NT + nt][i][lane] = acc[mt][nt][i];
+        __syncthreads();
+        for (int mt = 0; mt < MT; mt++)
+            for (int nt = 0; nt < NT; nt++) {
+                if (nrow[nt] >= n) continue;
+#pragma unroll
+                for (int ii = 0; ii < 4; ii++) {
+                    const uint32_t i = 4 * wave + ii;  // register index: rows 8*wave + 4*h + ii
+                    const uint32_t row = m_wave + mt * 32 + 8 * wave + 4 * h + ii;
+                    if (row < row_end) {
+                        const int tl = mt * NT + nt;
+                        const float y = (lds_red[0][tl][i][lane] + lds_red[1][tl][i][lane]) +
+                                        (lds_red[2][tl][i][lane] + lds_red[3][tl][i][lane]);
+                        float *o = out + (size_t)row * n + nrow[nt];
+                        *o = accumulate ? *o + y : y;
+                    }
+                }
+            }
+        return;
+    }
     for (int mt = 0; mt < MT; mt++)
         for (int nt = 0; nt < NT; nt++) {
             if (nrow[nt] >= n) continue;
@@ -570,14 +616,14 @@ __device__ __forceinline__ void gemm_tile_body(
 // OCC = 3: up to 168): the register budget decides how far the compiler lets loads and MFMAs
 // run ahead of their use.
 #define OXQ_TILE_KERNEL(NAME, OCC)                                                                                   \
-    template <class F, int MT, int NT, int WM, int DIST, bool DUMP>                                                 \
+    template <class F, int MT, int NT, int WM, int DIST, bool DUMP, int ADIST>                                      \
     __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void NAME(                      \
         const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,                \
         const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m,         \
         uint32_t mpad, uint32_t n, uint32_t k, int accumulate, uint32_t m_tiles, uint32_t n_tiles,                  \
         const int32_t *__restrict__ offsets, size_t w_stride) {                                                     \
-        gemm_tile_body<F, MT, NT, WM, DIST, DUMP>(W, q8t, P, da16, out, sums, m, mpad, n, k, accumulate, m_tiles,   \
-                                                  n_tiles, offsets, w_stride);                                      \
+        gemm_tile_body<F, MT, NT, WM, DIST, DUMP, ADIST>(W, q8t, P, da16, out, sums, m, mpad, n, k, accumulate,     \
+                                                         m_tiles, n_tiles, offsets, w_stride);                      \
     }
 OXQ_TILE_KERNEL(gemm_tile_kernel, 2)
 OXQ_TILE_KERNEL(gemm_tile_kernel_occ3, 3)
@@ -614,15 +660,15 @@ struct TilePlan {
     uint32_t mpad;
 };
 
-template <class F, int MT, int NT, int WM, int DIST, bool DUMP, int OCC = 2>
+template <class F, int MT, int NT, int WM, int DIST, bool DUMP, int OCC = 2, int ADIST = 1>
 static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
-    constexpr uint32_t WG_TOK = 32 * MT * WM, WG_ROWS = 32 * NT * (4 / WM);
+    constexpr uint32_t WG_TOK = 32 * MT * (WM ? WM : 1), WG_ROWS = 32 * NT * (WM ? 4 / WM : 1);
     const uint32_t rows = a.offsets ? a.max_rows : a.m;
     const uint32_t m_tiles = (rows + WG_TOK - 1) / WG_TOK, n_tiles = (a.n + WG_ROWS - 1) / WG_ROWS;
     const dim3 grid(8 * ((n_tiles + 7) / 8) * m_tiles, a.offsets ? a.n_experts : 1);
     const size_t lds = (size_t)(a.k / 32) * WG_TOK * 2;
-    auto kern = &gemm_tile_kernel<F, MT, NT, WM, DIST, DUMP>;
-    if constexpr (OCC == 3) kern = &gemm_tile_kernel_occ3<F, MT, NT, WM, DIST, DUMP>;
+    auto kern = &gemm_tile_kernel<F, MT, NT, WM, DIST, DUMP, ADIST>;
+    if constexpr (OCC == 3) kern = &gemm_tile_kernel_occ3<F, MT, NT, WM, DIST, DUMP, ADIST>;
     if (lds > 32 * 1024) {  // beyond the default dynamic LDS limit: opt in (up to the 160 KB of a CU)
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -639,10 +685,11 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
 template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
     const uint32_t rows = a.offsets ? a.max_rows : a.m;
-    // formats with a scale every 16 weights keep two MFMA results per tile in flight: one row tile per wave
-    constexpr int NTB = F::KSPLIT == 2 ? 1 : 2;
-    if (a.sums)
-        return rows > 32 ? launch_tile<F, 2, NTB, 2, 1, true>(a, p, stream) : launch_tile<F, 1, NTB, 1, 2, true>(a, p, stream);
+    if (a.sums)  // debug dump: the same tile layout (and fp32 summation order) as the production choice below
+        return rows > 384  ? launch_tile<F, 2, 1, 2, 1, true>(a, p, stream)
+               : rows > 64 ? launch_tile<F, 2, 1, 1, 2, true>(a, p, stream)
+               : rows > 32 ? launch_tile<F, 2, 1, 0, 2, true, 2, 2>(a, p, stream)
+                           : launch_tile<F, 1, 2, 0, 2, true, 2, 2>(a, p, stream);
     switch (g_gemm_variant) {
     case 1: return launch_tile<F, 2, 1, 2, 1, false>(a, p, stream);
     case 3: return launch_tile<F, 2, 2, 2, 1, false>(a, p, stream);
@@ -652,16 +699,18 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     case 13: return launch_tile<F, 1, 2, 1, 4, false>(a, p, stream);
     case 14: return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
     case 16: return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
+    case 21: return launch_tile<F, 1, 1, 0, 2, false, 2, 2>(a, p, stream);
+    case 22: return launch_tile<F, 1, 2, 0, 2, false, 2, 2>(a, p, stream);
+    case 23: return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
     default:
-        // Measured on MI355X at 14336 x 4096 (Q4_K, Q6_K): up to 64 tokens one 32-token tile per work
-        // group is fastest (the weight stream paces it), up to 384 tokens 64 x 128 tiles, beyond that
-        // 128 x 64 tiles at three waves per SIMD.
+        // Measured on MI355X at 14336 x 4096 (Q4_K, Q6_K) and on the 8-expert IQ4_XS shapes: up to 64
+        // tokens the four waves of a work group share one tile and split k (most work groups, shortest
+        // dependency chain per wave); up to 384 tokens 64 x 128 tiles; beyond that 128 x 64 tiles at
+        // three waves per SIMD.
         if (rows > 384) return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
         if (rows > 64) return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
-        // few tokens: 256-row tiles where that still gives every compute unit a work group
-        if (rows <= 32 && NTB == 2 && (size_t)((a.n + 255) / 256) * (a.offsets ? a.n_experts : 1) >= device_cus())
-            return launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
-        return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
+        if (rows > 32) return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
+        return launch_tile<F, 1, 2, 0, 2, false, 2, 2>(a, p, stream);
     }
 }
 

@@ -465,12 +465,18 @@ def test_moe_grouped_matmul(hip, ref, t, cfg):
             s_ref[r] = ref.block_sums(t, w[e], acts[r], n, k_)
     assert_close(y[:rows], y_ref, f"moe {cfg}")
     assert np.array_equal(dsum.cpu().numpy() - _tile_zero_point(t, acts.reshape(-1), rows, k_), s_ref)
-    # production launch (no sums), overwrite then accumulate, max_rows = 0 (unknown)
+    # production launch (no sums), overwrite then accumulate: the same bits as the dump launch
     dy2 = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
-    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, 0, dy2, n, k_, ws)
+    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy2, n, k_, ws)
     kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy2, n, k_, ws, accumulate=True)
     torch.cuda.synchronize()
     assert torch.equal(dy2, dy[:rows] + dy[:rows])
+    # max_rows = 0 (unknown) sizes the launch for the worst case: another tile shape and fp32
+    # summation order, the same values within the bar
+    dy3 = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
+    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, 0, dy3, n, k_, ws)
+    torch.cuda.synchronize()
+    assert_close(dy3.cpu().numpy(), y_ref, f"moe {cfg} max_rows=0")
 
 
 def test_moe_full_size_c5_one_projection(hip, ref):
