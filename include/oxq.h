@@ -184,7 +184,7 @@ int oxq_matvec_q8_fused_multi_dev(uint32_t type, size_t n_mats, const uint8_t *c
                                   size_t n_cols, int accumulate, void *stream);
 
 /* Prefill: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched form
- * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  With m >= 8 and k a
+ * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  With m >= 3 and k a
  * multiple of 256 every format uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()
  * bytes of 256-byte-aligned device scratch: pass it and the call is asynchronous
  * and allocation-free; pass NULL and the library uses its own scratch (the call

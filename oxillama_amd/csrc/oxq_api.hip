@@ -683,7 +683,7 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
 }
 
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k) {
-    return oxq_gemm_q8_workspace_bytes(type, total_rows < 8 ? 8 : total_rows, n, k);
+    return oxq_gemm_q8_workspace_bytes(type, total_rows < 3 ? 3 : total_rows, n, k);
 }
 
 int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
@@ -712,7 +712,7 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
     ga.out = d_out;
     ga.sums = d_sums;
     ga.workspace = (uint8_t *)d_workspace;
-    ga.m = (uint32_t)(total_rows < 8 ? 8 : total_rows);  // the tile kernel's minimum; rows past the offsets are never stored
+    ga.m = (uint32_t)(total_rows < 3 ? 3 : total_rows);  // the tile kernel's minimum; rows past the offsets are never stored
     ga.n = (uint32_t)n;
     ga.k = (uint32_t)k;
     ga.accumulate = accumulate ? 1 : 0;
