@@ -558,6 +558,9 @@ __device__ __forceinline__ void gemm_tile_body(
             const Wq w = DIST < 4 ? wring[g % (DIST < 4 ? DIST : 1)] : wring[DIST < 4 ? 0 : g];
             if constexpr (DIST < 4) fetch_w(wring[g % DIST], blk * 4 + g + DIST);  // slot consumed: refill it
             fetch_a(ops[(g + ADIST) % 4], blk * 4 + g + ADIST);
+            // keep the requests up here: the instruction scheduler otherwise sinks them to the end of
+            // the group's arithmetic (fewer live registers) and the prefetch distance is lost
+            __builtin_amdgcn_sched_barrier(0);
             compute(w, ops[g], blk, g);
         }
         if constexpr (DIST >= 4) {
