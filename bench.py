@@ -59,6 +59,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra-kernels", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--fused-quantize", action="store_true",
+                    help="decode step with the Q8_0 quantization done inside the GEMV kernels (3 launches per layer)")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch a 256 MiB copy kernel 3 times, then gate+up (one launch) over 8 distinct layers, "
                          "lm_head twice and the prefill matmul twice, and exit: the workload of the rocprofv3 --pmc "
@@ -152,15 +154,22 @@ def main():
     stream = torch.cuda.Stream()
 
     def step(i):
-        """One layer: quantize x; q_proj; ffn_gate + ffn_up in one launch (both read the same
-        Q8_0 vector); quantize h; ffn_down.  (Running q_proj on a second stream beside gate+up
-        was measured slower: the fork and join inside the graph cost more than the overlap gains.)"""
+        """One layer, five launches: quantize x; q_proj; ffn_gate + ffn_up (one launch: both read
+        the same vector); quantize h; ffn_down.  --fused-quantize lets the GEMV kernels quantize
+        their fp32 input in registers instead (three launches, bit-identical results); measured
+        slower here (42.7 vs 37.7 us per layer): every wave then reads and quantizes its slice of
+        the fp32 vector, which costs more than the two small launches it saves."""
         w = layers[i % L]
-        quant.quantize_q8_0_dev(x, xq)
-        k_q8.matvec_q8_fused_dev(w["q"], xq, yq, H, H, accumulate=False)
-        k_q4k.matvec_q8_fused_multi_dev([w["gate"], w["up"]], xq, [yg, yu], F, H, accumulate=False)
-        quant.quantize_q8_0_dev(h, hq)
-        k_q6k.matvec_q8_fused_dev(w["down"], hq, yd, H, F, accumulate=False)
+        if not args.fused_quantize:
+            quant.quantize_q8_0_dev(x, xq)
+            k_q8.matvec_q8_fused_dev(w["q"], xq, yq, H, H, accumulate=False)
+            k_q4k.matvec_q8_fused_multi_dev([w["gate"], w["up"]], xq, [yg, yu], F, H, accumulate=False)
+            quant.quantize_q8_0_dev(h, hq)
+            k_q6k.matvec_q8_fused_dev(w["down"], hq, yd, H, F, accumulate=False)
+        else:
+            k_q8.gemv_dev(w["q"], x, yq, H, H)
+            k_q4k.gemv_multi_dev([w["gate"], w["up"]], x, [yg, yu], F, H)
+            k_q6k.gemv_dev(w["down"], h, yd, H, F)
 
     def capture(fn):
         """Record fn()'s launches on `stream` into a HIP graph."""
@@ -195,6 +204,11 @@ def main():
     wall_ms = (time.perf_counter() - t_start) * 1e3
     ms_per_step = wall_ms / K
     value = step_weight_bytes / (ms_per_step * 1e-3) / 1e9
+
+    with torch.cuda.stream(stream):  # the per-kernel legs below read pre-quantized activations
+        quant.quantize_q8_0_dev(x, xq)
+        quant.quantize_q8_0_dev(h, hq)
+        stream.synchronize()
 
     # ---- per-kernel figures: back-to-back launches of one shape over rotating weights ----
     def time_kernel(kern, t, mats, acts, out, n_rows, n_cols, launches=None):
@@ -421,8 +435,10 @@ def main():
                                "ffn_gate/ffn_up 14336x4096 Q4_K, ffn_down 4096x14336 Q6_K, Q8_0 activations",
                    "weight_bytes_per_step": step_weight_bytes, "distinct_layers": L,
                    "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-                   "launch": "one HIP graph of all timed steps; per step 2 quantizations, q_proj, gate+up (one launch), "
-                             "down"},
+                   "launch": "one HIP graph of all timed steps; per step " +
+                             ("2 quantizations, q_proj, gate+up (one launch), down" if not args.fused_quantize else
+                              "q_proj, gate+up (one launch), down, each quantizing its fp32 input vector to Q8_0 in "
+                              "registers")},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "kernels": kernels,

@@ -607,6 +607,32 @@ int oxq_matvec_q8_fused_multi_dev(uint32_t type, size_t n_mats, const uint8_t *c
     return OXQ_OK;
 }
 
+int oxq_gemv_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_weights, const float *d_x,
+                       float *const *d_outs, size_t n_rows, size_t n_cols, int accumulate, void *stream) {
+    int st = check_dev_shape(type, n_rows, n_cols);
+    if (st != OXQ_OK) return st;
+    if (n_mats == 0) return OXQ_OK;
+    if (n_mats > 4) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 4, n_mats, "at most 4 matrices per call");
+    if (!d_weights || !d_outs) return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer table");
+    if (!oxq::gemv_takes_f32(type, (uint32_t)n_cols))
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, n_cols, "row too long for in-kernel activation quantization");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    oxq::GemvArgs a = gemv_args(d_weights[0], nullptr, d_outs[0], nullptr, n_rows, n_cols, accumulate ? 1 : 0);
+    a.X = d_x;
+    a.n_mats = (uint32_t)n_mats;
+    for (size_t i = 1; i < n_mats; i++) {
+        a.W_more[i - 1] = d_weights[i];
+        a.out_more[i - 1] = d_outs[i];
+    }
+    OXQ_HIP(oxq::launch_gemv_q8(type, a, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_gemv_dev(uint32_t type, const uint8_t *d_weights, const float *d_x, float *d_out, size_t n_rows,
+                 size_t n_cols, int accumulate, void *stream) {
+    return oxq_gemv_multi_dev(type, 1, &d_weights, d_x, &d_out, n_rows, n_cols, accumulate, stream);
+}
+
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, int32_t *d_sums,
                        size_t n_rows, size_t n_cols, void *stream) {
     int st = check_dev_shape(type, n_rows, n_cols);

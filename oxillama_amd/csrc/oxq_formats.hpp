@@ -33,6 +33,61 @@ constexpr uint32_t Q8_BLOCK_BYTES = 34;  // Q/traits.rs:12: f16 d + 32 x i8
 // v_mul_i32_i24: exact product of two values that fit in 24 signed bits.
 __device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
 
+// Where a wave takes its activations from.  Both sources hand out one Q8_0 block as it sits
+// in the reference's acts_q8 buffer: 32 int8 (two 16-byte halves) and the f16 scale bits.
+//  * ActQ8: the blocks were quantized beforehand (oxq_quantize_q8_0_dev) and are read.
+//  * ActF32: fp32 activations are quantized in registers, block by block, with the
+//    arithmetic of encode_q8_0_block (crates/oxillama-quant/src/quantize.rs:190-210): the
+//    same bytes, without a separate quantize launch (QuantKernel::gemv takes fp32 input,
+//    crates/oxillama-quant/src/traits.rs:39-44).  Every wave does this for its own slice.
+struct ActQ8 {
+    const uint8_t *A;
+    static __device__ __forceinline__ ActQ8 make(const void *p) { return ActQ8{static_cast<const uint8_t *>(p)}; }
+    __device__ __forceinline__ void block(uint32_t b, u32x4 &q0, u32x4 &q1, uint32_t &dbits) const {
+        const uint8_t *blk = A + (size_t)b * Q8_BLOCK_BYTES;
+        q0 = ld16(blk + 2);
+        q1 = ld16(blk + 18);
+        dbits = ld2(blk);
+    }
+};
+struct ActF32 {
+    const float *X;
+    static __device__ __forceinline__ ActF32 make(const void *p) { return ActF32{static_cast<const float *>(p)}; }
+    __device__ __forceinline__ void block(uint32_t b, u32x4 &q0, u32x4 &q1, uint32_t &dbits) const {
+        float v[32];
+        const u32x4 *px = reinterpret_cast<const u32x4 *>(X + (size_t)b * 32);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const u32x4 raw = px[j];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t bits = raw[i];  // copy out first: bit_cast must not see the vector element lvalue
+                v[4 * j + i] = __builtin_bit_cast(float, bits);
+            }
+        }
+        float m = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 32; i++) m = fmaxf(m, fabsf(v[i]));  // max is exact in any order (quantize.rs:194)
+        const float d = m / 127.0f;                               // quantize.rs:197
+        const float id = (d != 0.0f) ? 1.0f / d : 0.0f;           // quantize.rs:198
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            uint32_t packed = 0;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                int q = (int)roundf(v[4 * j + i] * id);  // quantize.rs:206 (round half away from zero)
+                q = q < -128 ? -128 : (q > 127 ? 127 : q);
+                packed |= ((uint32_t)q & 0xFFu) << (8 * i);
+            }
+            w[j] = packed;
+        }
+        q0 = u32x4{w[0], w[1], w[2], w[3]};
+        q1 = u32x4{w[4], w[5], w[6], w[7]};
+        dbits = f2h(d);  // quantize.rs:201
+    }
+};
+
 // ---------------------------------------------------------------------------
 // Q4_K, Q/reference/q4_k.rs:27-99,218-333.  144 B = d, dmin (f16), 12 B packed
 // 6-bit scales/mins, 128 B nibbles.  Unit = one 64-weight group g (0..3) of a
@@ -61,14 +116,11 @@ struct FmtQ4K {
         k.upper = k.g >= 2;
         return k;
     }
-    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
-                                                    const Lane &k) {
-        const uint8_t *blo = A + (size_t)(8 * (u >> 2) + 2 * k.g) * Q8_BLOCK_BYTES;
-        const uint8_t *bhi = blo + Q8_BLOCK_BYTES;
-        a.lo0 = ld16(blo + 2);
-        a.lo1 = ld16(blo + 18);
-        a.hi0 = ld16(bhi + 2);
-        a.hi1 = ld16(bhi + 18);
+    template <class SRC>
+    static __device__ __forceinline__ void load_act(Act &a, const SRC &src, uint32_t u, bool valid, const Lane &k) {
+        uint32_t dlo_bits, dhi_bits;
+        src.block(8 * (u >> 2) + 2 * k.g, a.lo0, a.lo1, dlo_bits);
+        src.block(8 * (u >> 2) + 2 * k.g + 1, a.hi0, a.hi1, dhi_bits);
         int slo = 0, shi = 0;
         for (int i = 0; i < 4; i++) {
             slo = sdot4(a.lo0[i], 0x01010101u, slo);
@@ -76,7 +128,7 @@ struct FmtQ4K {
             shi = sdot4(a.hi0[i], 0x01010101u, shi);
             shi = sdot4(a.hi1[i], 0x01010101u, shi);
         }
-        const float dlo = h2f(ld2(blo)), dhi = h2f(ld2(bhi));
+        const float dlo = h2f(dlo_bits), dhi = h2f(dhi_bits);
         a.a_lo = valid ? dlo : 0.0f;
         a.a_hi = valid ? dhi : 0.0f;
         a.b_lo = valid ? dlo * (float)slo : 0.0f;
@@ -147,14 +199,16 @@ struct FmtQ6K {
         k.is = lane & 1;
         return k;
     }
-    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
-                                                    const Lane &k) {
+    template <class SRC>
+    static __device__ __forceinline__ void load_act(Act &a, const SRC &src, uint32_t u, bool valid, const Lane &k) {
         const u32x4 z = {0, 0, 0, 0};
         for (int j = 0; j < 4; j++) {
-            const uint8_t *blk = A + (size_t)(8 * (u >> 2) + 4 * k.hh + j) * Q8_BLOCK_BYTES;
-            const u32x4 q = ld16(blk + 2 + 16 * k.is);
+            u32x4 q0, q1;
+            uint32_t dbits;
+            src.block(8 * (u >> 2) + 4 * k.hh + j, q0, q1, dbits);
+            const u32x4 q = k.is ? q1 : q0;
             a.q[j] = valid ? q : z;
-            a.d_a[j] = valid ? h2f(ld2(blk)) : 0.0f;
+            a.d_a[j] = valid ? h2f(dbits) : 0.0f;
             int s = 0;
             for (int i = 0; i < 4; i++) s = sdot4(a.q[j][i], 0x01010101u, s);
             a.nasum32[j] = -32 * s;
@@ -220,12 +274,11 @@ struct FmtQ8_0 {
         uint32_t d;
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t) { return Lane{}; }
-    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
-                                                    const Lane &) {
-        const uint8_t *blk = A + (size_t)u * Q8_BLOCK_BYTES;
-        a.q0 = ld16(blk + 2);
-        a.q1 = ld16(blk + 18);
-        a.d_a = valid ? h2f(ld2(blk)) : 0.0f;
+    template <class SRC>
+    static __device__ __forceinline__ void load_act(Act &a, const SRC &src, uint32_t u, bool valid, const Lane &) {
+        uint32_t dbits;
+        src.block(u, a.q0, a.q1, dbits);
+        a.d_a = valid ? h2f(dbits) : 0.0f;
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
@@ -277,10 +330,11 @@ struct FmtQ4_0 {
         uint32_t d;
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t) { return Lane{}; }
-    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
-                                                    const Lane &) {
-        const uint8_t *blk = A + (size_t)u * Q8_BLOCK_BYTES;
-        const u32x4 q0 = ld16(blk + 2), q1 = ld16(blk + 18);
+    template <class SRC>
+    static __device__ __forceinline__ void load_act(Act &a, const SRC &src, uint32_t u, bool valid, const Lane &) {
+        u32x4 q0, q1;
+        uint32_t dbits;
+        src.block(u, q0, q1, dbits);
         split_even_odd(q0, q1, a.ev, a.od);
         int s = 0;
         for (int i = 0; i < 4; i++) {
@@ -288,7 +342,7 @@ struct FmtQ4_0 {
             s = sdot4(q1[i], 0x01010101u, s);
         }
         a.nasum8 = -8 * s;
-        a.d_a = valid ? h2f(ld2(blk)) : 0.0f;
+        a.d_a = valid ? h2f(dbits) : 0.0f;
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
@@ -329,12 +383,13 @@ struct FmtIQ4XS {
         u32x2 hdr;
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t lane) { return Lane{lane & 7}; }
-    static __device__ __forceinline__ void load_act(Act &a, const uint8_t *A, uint32_t u, bool valid,
-                                                    const Lane &) {
-        const uint8_t *blk = A + (size_t)u * Q8_BLOCK_BYTES;
-        const u32x4 q0 = ld16(blk + 2), q1 = ld16(blk + 18);
+    template <class SRC>
+    static __device__ __forceinline__ void load_act(Act &a, const SRC &src, uint32_t u, bool valid, const Lane &) {
+        u32x4 q0, q1;
+        uint32_t dbits;
+        src.block(u, q0, q1, dbits);
         split_even_odd(q0, q1, a.ev, a.od);
-        a.d_a = valid ? h2f(ld2(blk)) : 0.0f;
+        a.d_a = valid ? h2f(dbits) : 0.0f;
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &k) {
         const uint8_t *blk = row + (size_t)(u >> 3) * BLOCK_BYTES;

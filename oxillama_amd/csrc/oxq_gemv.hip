@@ -15,8 +15,8 @@
 
 namespace oxq {
 
-template <class F, int STEPS, int RB, int KS, bool DUMP>
-static hipError_t launch_cached(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
+template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP>
+static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
                                 hipStream_t stream) {
     constexpr uint32_t G = 4 / KS;  // row groups per work group
     const uint32_t n_mats = a.n_mats ? a.n_mats : 1;
@@ -35,10 +35,21 @@ static hipError_t launch_cached(const GemvArgs &a, uint32_t units, uint32_t grou
     const uint32_t groups = (n_batches + passes - 1) / passes;
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
-    hipLaunchKernelGGL((gemv_q8_cached<F, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), 0, stream, w[0], w[1],
-                       w[2], w[3], o[0], o[1], o[2], o[3], a.A, a.sums, a.n_rows, units, groups_per_row, row_bytes,
-                       a.accumulate);
+    const void *acts = a.X ? static_cast<const void *>(a.X) : static_cast<const void *>(a.A);
+    hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), 0, stream, w[0],
+                       w[1], w[2], w[3], o[0], o[1], o[2], o[3], acts, a.sums, a.n_rows, units, groups_per_row,
+                       row_bytes, a.accumulate);
     return hipGetLastError();
+}
+
+// a.X set: fp32 activations, quantized to Q8_0 in registers by every wave (no dump variant).
+template <class F, int STEPS, int RB, int KS, bool DUMP>
+static hipError_t launch_cached(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
+                                hipStream_t stream) {
+    if constexpr (!DUMP) {
+        if (a.X) return launch_cached_src<F, ActF32, STEPS, RB, KS, false>(a, units, groups_per_row, row_bytes, stream);
+    }
+    return launch_cached_src<F, ActQ8, STEPS, RB, KS, DUMP>(a, units, groups_per_row, row_bytes, stream);
 }
 
 template <class F, int STEPS, int KS>
@@ -87,6 +98,7 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     case 8: return launch_steps<F, 8, 1>(a, units, groups_per_row, row_bytes, rb, stream);
     default: break;
     }
+    if (a.X) return hipErrorNotSupported;  // rows this long re-read the activations: Q8_0 blocks only
     const uint32_t max_waves = device_cus() * a.waves_per_cu;
     uint32_t waves = a.n_rows < max_waves ? a.n_rows : max_waves;
     uint32_t blocks = (waves + 3) / 4;
@@ -105,6 +117,12 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
 template <class F>
 static bool multi_in_one_launch(const GemvArgs &a) {
     return (a.n_cols / F::UNIT_COLS + 63) / 64 <= 32 && !a.sums;
+}
+
+bool gemv_takes_f32(uint32_t type, uint32_t n_cols) {
+    uint32_t unit = 32;
+    if (type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_Q6_K) unit = 64;
+    return (n_cols / unit + 63) / 64 <= 32;  // the register-cached kernel (up to 8 steps, or 4 waves x 8)
 }
 
 hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream) {

@@ -62,15 +62,16 @@ __device__ __forceinline__ float reduce_batch(const Batch<F, STEPS, RB> &b, cons
     return res;
 }
 
-template <class F, int STEPS, int RB, int KS, bool DUMP>
+template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP>
 __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
                                                      const uint8_t *__restrict__ W2, const uint8_t *__restrict__ W3,
                                                      float *__restrict__ out0, float *__restrict__ out1,
                                                      float *__restrict__ out2, float *__restrict__ out3,
-                                                     const uint8_t *__restrict__ A, int32_t *__restrict__ sums,
+                                                     const void *__restrict__ A, int32_t *__restrict__ sums,
                                                      uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
                                                      size_t row_bytes, int accumulate) {
     static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
+    const SRC src = SRC::make(A);
     // Up to four matrices of one shape and format that share the activation vector (wq/wk/wv,
     // ffn_gate/ffn_up) ride in one launch: blockIdx.y picks the matrix, and each matrix gets
     // its own gridDim.x work groups.
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
 #pragma unroll
     for (int s = 0; s < STEPS; s++) {
         const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
-        F::load_act(act[s], A, min(u, units - 1), u < units, k);  // all-zero constants past the end
+        F::load_act(act[s], src, min(u, units - 1), u < units, k);  // all-zero constants past the end
     }
     Batch<F, STEPS, RB> b0, b1;
     load_batch<F, STEPS, RB>(b0, W, out, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
@@ -174,7 +175,7 @@ __global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict
             typename F::Wt w;
             const uint32_t uc = min(u, units - 1);
             F::load_w(w, rp, uc, k);
-            F::load_act(a, A, uc, valid, k);
+            F::load_act(a, ActQ8{A}, uc, valid, k);
             acc += F::template dot<DUMP>(w, a, k, DUMP ? sums + (size_t)row * groups_per_row : nullptr, u, valid);
         }
         const float total = wave_sum(acc);

@@ -11,6 +11,7 @@ namespace oxq {
 struct GemvArgs {
     const uint8_t *W;     // raw GGUF blocks, row-major, device memory
     const uint8_t *A;     // Q8_0 activation blocks, device memory
+    const float *X = nullptr;  // instead of A: fp32 activations, quantized to Q8_0 inside the kernel
     float *out;           // n_rows floats, device memory
     int32_t *sums;        // optional: per-row integer group sums (debug), else null
     uint32_t n_rows;
@@ -30,6 +31,8 @@ struct GemvArgs {
 uint32_t device_cus();
 
 hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream);
+// True when the GEMV of this row length can quantize fp32 activations itself (GemvArgs::X).
+bool gemv_takes_f32(uint32_t type, uint32_t n_cols);
 
 // x: n floats (n % 32 == 0) -> n/32 Q8_0 blocks of 34 bytes.
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *out, hipStream_t stream);

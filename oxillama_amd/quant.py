@@ -241,6 +241,19 @@ class HipKernel:
         _check(self._lib.oxq_matvec_q8_fused_multi_dev(self.tensor_type, n, wp, d_acts.data_ptr(), op, n_rows, n_cols,
                                                        int(accumulate), self._stream()))
 
+    def gemv_dev(self, d_weights, d_x, d_out, n_rows, n_cols, accumulate=False):
+        """fp32 activations in, quantized to Q8_0 inside the kernel (one launch)."""
+        _check(self._lib.oxq_gemv_dev(self.tensor_type, d_weights.data_ptr(), d_x.data_ptr(), d_out.data_ptr(),
+                                      n_rows, n_cols, int(accumulate), self._stream()))
+
+    def gemv_multi_dev(self, d_weights, d_x, d_outs, n_rows, n_cols, accumulate=False):
+        import ctypes as C
+        n = len(d_weights)
+        wp = (C.c_void_p * n)(*[w.data_ptr() for w in d_weights])
+        op = (C.c_void_p * n)(*[o.data_ptr() for o in d_outs])
+        _check(self._lib.oxq_gemv_multi_dev(self.tensor_type, n, wp, d_x.data_ptr(), op, n_rows, n_cols,
+                                            int(accumulate), self._stream()))
+
     def gemm_workspace_bytes(self, m, n, k):
         return self._lib.oxq_gemm_q8_workspace_bytes(self.tensor_type, m, n, k)
 

@@ -219,6 +219,37 @@ def test_fused_multi_matrix_launch_is_bit_identical(hip, ref, t, n_mats):
                 assert torch.equal(y1, y2), (O.NAMES[t], n_mats, n_rows, n_cols, acc)
 
 
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_gemv_dev_quantizes_in_kernel_bit_identically(hip, ref, t):
+    """fp32 activations quantized inside the GEMV: the same bits as quantize + fused, for one and
+    for several matrices, short and long rows (1, 2, 4 steps and rows split over four waves)."""
+    import torch
+    for n_rows, n_cols in ((48, 512), (64, 4096), (33, 8192), (20, 14336)):
+        x = synth.normal_f32(820 + n_cols, n_cols)
+        x[32:64] = 0.0                      # an all-zero block (d = 0)
+        x[64:96] *= 1.0e-30                 # a block of tiny values
+        dx = torch.from_numpy(x).cuda()
+        da = torch.from_numpy(ref.quantize_q8_0(x)).cuda()
+        ws = [torch.from_numpy(synth.weights(t, 830 + i, n_rows, n_cols)).cuda() for i in range(2)]
+        kern = hip.HipKernel(t)
+        want = [torch.full((n_rows,), 2.0, dtype=torch.float32, device="cuda") for _ in range(2)]
+        got = [torch.full((n_rows,), 2.0, dtype=torch.float32, device="cuda") for _ in range(2)]
+        for acc in (False, True):
+            for w, y in zip(ws, want):
+                kern.matvec_q8_fused_dev(w, da, y, n_rows, n_cols, accumulate=acc)
+            kern.gemv_dev(ws[0], dx, got[0], n_rows, n_cols, accumulate=acc)
+            kern.gemv_dev(ws[1], dx, got[1], n_rows, n_cols, accumulate=acc)
+            torch.cuda.synchronize()
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), (O.NAMES[t], n_rows, n_cols, acc)
+        multi = [torch.zeros(n_rows, dtype=torch.float32, device="cuda") for _ in range(2)]
+        single = [torch.zeros(n_rows, dtype=torch.float32, device="cuda") for _ in range(2)]
+        kern.gemv_multi_dev(ws, dx, multi, n_rows, n_cols)
+        for w, y in zip(ws, single):
+            kern.matvec_q8_fused_dev(w, da, y, n_rows, n_cols, accumulate=False)
+        torch.cuda.synchronize()
+        assert torch.equal(multi[0], single[0]) and torch.equal(multi[1], single[1])
+
+
 def test_empty_inputs(hip):
     for t in O.ALL_TYPES:
         k = hip.HipKernel(t)
