@@ -156,9 +156,9 @@ def main():
     def step(i):
         """One layer, five launches: quantize x; q_proj; ffn_gate + ffn_up (one launch: both read
         the same vector); quantize h; ffn_down.  --fused-quantize lets the GEMV kernels quantize
-        their fp32 input in registers instead (three launches, bit-identical results); measured
-        slower here (42.7 vs 37.7 us per layer): every wave then reads and quantizes its slice of
-        the fp32 vector, which costs more than the two small launches it saves."""
+        their fp32 input themselves (three launches, bit-identical results); measured slightly
+        slower here (40.2 vs 38.5 us per layer): every work group then quantizes the whole vector
+        into LDS before its first row, which costs more than the two small launches it saves."""
         w = layers[i % L]
         if not args.fused_quantize:
             quant.quantize_q8_0_dev(x, xq)

@@ -184,11 +184,11 @@ int oxq_matvec_q8_fused_multi_dev(uint32_t type, size_t n_mats, const uint8_t *c
                                   size_t n_cols, int accumulate, void *stream);
 
 /* QuantKernel::gemv on device pointers (Q/traits.rs:39-44: fp32 input): d_out[r] (+)= W[r,:] . q8(x).
- * The kernel quantizes d_x (n_cols floats) to Q8_0 in registers with the reference encoder's
- * arithmetic, so the result is bit-identical to oxq_quantize_q8_0_dev + oxq_matvec_q8_fused_dev
+ * Every work group of the kernel first quantizes d_x (n_cols floats) to Q8_0 into LDS with the
+ * reference encoder's arithmetic, so the result is bit-identical to oxq_quantize_q8_0_dev + oxq_matvec_q8_fused_dev
  * at one launch instead of two.  oxq_gemv_multi_dev: the same for up to 4 matrices of one shape
- * and format sharing x.  Rows of more than 65536 columns (131072 for Q4_K / Q6_K), which the
- * register-cached kernel does not cover, return OXQ_ERR_UNSUPPORTED_SHAPE: quantize first. */
+ * and format sharing x.  Rows of more than 46080 columns (the quantized vector is staged in
+ * LDS) return OXQ_ERR_UNSUPPORTED_SHAPE: quantize first. */
 int oxq_gemv_dev(uint32_t type, const uint8_t *d_weights, const float *d_x, float *d_out,
                  size_t n_rows, size_t n_cols, int accumulate, void *stream);
 int oxq_gemv_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_weights,

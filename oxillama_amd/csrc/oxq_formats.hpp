@@ -36,10 +36,10 @@ __device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
 // Where a wave takes its activations from.  Both sources hand out one Q8_0 block as it sits
 // in the reference's acts_q8 buffer: 32 int8 (two 16-byte halves) and the f16 scale bits.
 //  * ActQ8: the blocks were quantized beforehand (oxq_quantize_q8_0_dev) and are read.
-//  * ActF32: fp32 activations are quantized in registers, block by block, with the
-//    arithmetic of encode_q8_0_block (crates/oxillama-quant/src/quantize.rs:190-210): the
+//  * ActF32: fp32 activations; every work group first quantizes the vector into LDS with the
+//    arithmetic of encode_q8_0_block (crates/oxillama-quant/src/quantize.rs:190-210) -- the
 //    same bytes, without a separate quantize launch (QuantKernel::gemv takes fp32 input,
-//    crates/oxillama-quant/src/traits.rs:39-44).  Every wave does this for its own slice.
+//    crates/oxillama-quant/src/traits.rs:39-44) -- and its waves read the blocks from there.
 struct ActQ8 {
     const uint8_t *A;
     static __device__ __forceinline__ ActQ8 make(const void *p) { return ActQ8{static_cast<const uint8_t *>(p)}; }
@@ -53,40 +53,54 @@ struct ActQ8 {
 struct ActF32 {
     const float *X;
     static __device__ __forceinline__ ActF32 make(const void *p) { return ActF32{static_cast<const float *>(p)}; }
+};
+// The blocks ActF32 stands for, once the work group has quantized them into LDS
+// (quantize_to_lds): 32 payload bytes per block, 32-byte aligned, and the f16 scales apart.
+struct ActLds {
+    const u32x4 *q;     // [n_blocks][2]
+    const uint16_t *d;  // [n_blocks]
     __device__ __forceinline__ void block(uint32_t b, u32x4 &q0, u32x4 &q1, uint32_t &dbits) const {
-        float v[32];
-        const u32x4 *px = reinterpret_cast<const u32x4 *>(X + (size_t)b * 32);
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            const u32x4 raw = px[j];
-#pragma unroll
+        q0 = q[2 * b];
+        q1 = q[2 * b + 1];
+        dbits = d[b];
+    }
+};
+
+// All 256 threads of a work group quantize n_blocks * 32 floats into LDS: eight lanes per
+// block, four floats per lane, exactly as quantize_q8_0_kernel does.
+__device__ __forceinline__ void quantize_to_lds(const float *__restrict__ x, uint32_t n_blocks, uint32_t *lds_q,
+                                                uint16_t *lds_d) {
+    const uint32_t j = threadIdx.x & 7;
+    for (uint32_t base = 0; base < n_blocks; base += 32) {
+        const uint32_t blk = base + (threadIdx.x >> 3);
+        const bool valid = blk < n_blocks;
+        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (valid) {
+            const u32x4 raw = *reinterpret_cast<const u32x4 *>(x + (size_t)blk * 32 + 4 * j);
             for (int i = 0; i < 4; i++) {
                 const uint32_t bits = raw[i];  // copy out first: bit_cast must not see the vector element lvalue
-                v[4 * j + i] = __builtin_bit_cast(float, bits);
+                v[i] = __builtin_bit_cast(float, bits);
             }
         }
         float m = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 32; i++) m = fmaxf(m, fabsf(v[i]));  // max is exact in any order (quantize.rs:194)
-        const float d = m / 127.0f;                               // quantize.rs:197
-        const float id = (d != 0.0f) ? 1.0f / d : 0.0f;           // quantize.rs:198
-        uint32_t w[8];
-#pragma unroll
-        for (int j = 0; j < 8; j++) {
-            uint32_t packed = 0;
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                int q = (int)roundf(v[4 * j + i] * id);  // quantize.rs:206 (round half away from zero)
-                q = q < -128 ? -128 : (q > 127 ? 127 : q);
-                packed |= ((uint32_t)q & 0xFFu) << (8 * i);
-            }
-            w[j] = packed;
+        for (int i = 0; i < 4; i++) m = fmaxf(m, fabsf(v[i]));
+        m = fmaxf(m, dpp_f<0xB1>(m));
+        m = fmaxf(m, dpp_f<0x4E>(m));
+        m = fmaxf(m, __shfl_xor(m, 4, 64));  // max is exact in any order (quantize.rs:194)
+        const float d = m / 127.0f;                      // quantize.rs:197
+        const float id = (d != 0.0f) ? 1.0f / d : 0.0f;  // quantize.rs:198
+        uint32_t packed = 0;
+        for (int i = 0; i < 4; i++) {
+            int q = (int)roundf(v[i] * id);  // quantize.rs:206 (round half away from zero)
+            q = q < -128 ? -128 : (q > 127 ? 127 : q);
+            packed |= ((uint32_t)q & 0xFFu) << (8 * i);
         }
-        q0 = u32x4{w[0], w[1], w[2], w[3]};
-        q1 = u32x4{w[4], w[5], w[6], w[7]};
-        dbits = f2h(d);  // quantize.rs:201
+        if (valid) {
+            lds_q[blk * 8 + j] = packed;
+            if (j == 0) lds_d[blk] = (uint16_t)f2h(d);  // quantize.rs:201
+        }
     }
-};
+}
 
 // ---------------------------------------------------------------------------
 // Q4_K, Q/reference/q4_k.rs:27-99,218-333.  144 B = d, dmin (f16), 12 B packed

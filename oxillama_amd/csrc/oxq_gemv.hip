@@ -36,7 +36,9 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
     const void *acts = a.X ? static_cast<const void *>(a.X) : static_cast<const void *>(a.A);
-    hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), 0, stream, w[0],
+    // fp32 source: LDS for the quantized vector (32 payload bytes + one f16 scale per block)
+    const size_t lds = std::is_same<SRC, ActF32>::value ? (size_t)(a.n_cols / 32) * 34 : 0;
+    hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), lds, stream, w[0],
                        w[1], w[2], w[3], o[0], o[1], o[2], o[3], acts, a.sums, a.n_rows, units, groups_per_row,
                        row_bytes, a.accumulate);
     return hipGetLastError();
@@ -122,7 +124,8 @@ static bool multi_in_one_launch(const GemvArgs &a) {
 bool gemv_takes_f32(uint32_t type, uint32_t n_cols) {
     uint32_t unit = 32;
     if (type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_Q6_K) unit = 64;
-    return (n_cols / unit + 63) / 64 <= 32;  // the register-cached kernel (up to 8 steps, or 4 waves x 8)
+    // the register-cached kernel (up to 8 steps, or 4 waves x 8) and the default dynamic LDS limit
+    return (n_cols / unit + 63) / 64 <= 32 && (size_t)(n_cols / 32) * 34 <= 48 * 1024;
 }
 
 hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream) {

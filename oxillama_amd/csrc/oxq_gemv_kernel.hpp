@@ -1,5 +1,7 @@
 // Kernel templates of the Q8_0-activation GEMV (see oxq_gemv.hip for the design).
 #pragma once
+#include <type_traits>
+
 #include "oxq_formats.hpp"
 
 namespace oxq {
@@ -71,7 +73,6 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
                                                      uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
                                                      size_t row_bytes, int accumulate) {
     static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
-    const SRC src = SRC::make(A);
     // Up to four matrices of one shape and format that share the activation vector (wq/wk/wv,
     // ffn_gate/ffn_up) ride in one launch: blockIdx.y picks the matrix, and each matrix gets
     // its own gridDim.x work groups.
@@ -91,19 +92,37 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
     // With KS > 1 every wave of the work group runs the same number of trips (barriers);
     // trips past the last batch re-read the last rows and store nothing.
     const uint32_t n_trips = KS == 1 ? n_batches : ((n_batches + n_groups - 1) / n_groups) * n_groups;
-    if (KS == 1 && group >= n_batches) return;
     const bool want_old = accumulate && part == 0;
-
-    // Activations first (they sit in L2 and arrive early), then the first batch of
-    // weights: the activation constants are derived while HBM is being read.
-    typename F::Act act[STEPS];
-#pragma unroll
-    for (int s = 0; s < STEPS; s++) {
-        const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
-        F::load_act(act[s], src, min(u, units - 1), u < units, k);  // all-zero constants past the end
-    }
+    constexpr bool F32 = std::is_same<SRC, ActF32>::value;
     Batch<F, STEPS, RB> b0, b1;
-    load_batch<F, STEPS, RB>(b0, W, out, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
+    typename F::Act act[STEPS];
+    extern __shared__ uint32_t lds_acts[];  // fp32 source: [n_blocks * 8] payload dwords, then n_blocks f16 scales
+    auto load_acts = [&](const auto &src) {
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
+            F::load_act(act[s], src, min(u, units - 1), u < units, k);  // all-zero constants past the end
+        }
+    };
+    if constexpr (F32) {
+        // fp32 activations: request the first weights, then the work group quantizes the vector into
+        // LDS once (every wave takes part in the barrier) and each wave picks up its slice.
+        load_batch<F, STEPS, RB>(b0, W, out, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k,
+                                 want_old);
+        const uint32_t nb = units * (F::UNIT_COLS / 32);
+        uint16_t *lds_d = reinterpret_cast<uint16_t *>(lds_acts + (size_t)nb * 8);
+        quantize_to_lds(static_cast<const float *>(A), nb, lds_acts, lds_d);
+        __syncthreads();
+        if (KS == 1 && group >= n_batches) return;
+        load_acts(ActLds{reinterpret_cast<const u32x4 *>(lds_acts), lds_d});
+    } else {
+        if (KS == 1 && group >= n_batches) return;
+        // Activations first (they sit in L2 and arrive early), then the first batch of
+        // weights: the activation constants are derived while HBM is being read.
+        load_acts(SRC::make(A));
+        load_batch<F, STEPS, RB>(b0, W, out, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k,
+                                 want_old);
+    }
 
     uint32_t trip = 0;
     auto finish = [&](float res, float old, uint32_t batch) {
