@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-matmul hot path on one MI355X.
 
-Workload (BASELINE.json configs[1]): the decode projections of one Llama-3-8B
+Workload: the decode projections of one Llama-3-8B
 layer at batch 1 -- Q8_0-quantize x[4096]; q_proj 4096x4096 Q8_0; ffn_gate and
 ffn_up 14336x4096 Q4_K; Q8_0-quantize h[14336]; ffn_down 4096x14336 Q6_K -- with
 synthetic N(0,0.02) weights and N(0,1) activations.  One step = one layer.  Steps
@@ -11,8 +11,9 @@ second over the timed steps (inputs resident in HBM, launches replayed from one
 HIP graph so the host adds no per-kernel latency).
 
 Prints ONE JSON line.  Extra objects:
-  roofline     the dominant kernel (Q4_K GEMV, 14336x4096) timed alone with HIP
-               events on the launch stream, algorithmic bytes / duration vs 8 TB/s
+  roofline     the dominant kernel (Q4_K GEMV on ffn_gate + ffn_up, 2 x 14336x4096 in one launch)
+               timed alone with HIP events on the launch stream, algorithmic bytes / duration
+               vs 8 TB/s
   kernels      the same figure for each GEMV shape, the lm_head and C1 shapes
   prefill      batch-512 Q4_K prefill matmul, int8 TOPS vs the 5.0 POPS peak
   moe          IQ4_XS grouped expert matmuls (8 experts, 64 tokens, top-2), weight GB/s
@@ -431,7 +432,7 @@ def main():
         "vs_baseline": None,
         "dtype": "int8 dot (v_dot4_i32_i8) -> int32 group sums -> f32",
         "data": "synthetic",
-        "config": {"workload": "Llama-3-8B decode projections, batch 1 (BASELINE configs[1]): q_proj 4096x4096 Q8_0, "
+        "config": {"workload": "Llama-3-8B decode projections, batch 1: q_proj 4096x4096 Q8_0, "
                                "ffn_gate/ffn_up 14336x4096 Q4_K, ffn_down 4096x14336 Q6_K, Q8_0 activations",
                    "weight_bytes_per_step": step_weight_bytes, "distinct_layers": L,
                    "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
