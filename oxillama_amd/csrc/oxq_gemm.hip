@@ -1,28 +1,28 @@
-// Batched (prefill) form of the fused matvec on gfx950:
+// Batched (prefill, decode batch, mixture-of-experts group) form of the fused matvec on gfx950:
 //   out[m x n] (+)= A_q8[m rows of Q8_0 blocks] x W[n x k]^T
 // i.e. m fused matvecs over the same weight blocks (the reference's gemm is exactly
 // that loop, crates/oxillama-quant/src/reference/q4_k.rs:186-201, with
-// matvec_q8_fused's arithmetic, :218-333).
+// matvec_q8_fused's arithmetic, :218-333), for all five formats.
 //
-// Q4_K runs on the int8 matrix cores.  One v_mfma_i32_32x32x32_i8 contracts one
-// 32-weight sub-block of 32 weight rows against the matching Q8_0 block of 32
-// tokens, so every int32 result is exactly one "group sum" I[m][n][s] of the
-// matvec.  The fp32 value is then
-//   y[m][n] = sum_s da[m][s] * (d_n*sc_ns) * I  -  sum_s (da[m][s]*S[m][s]) * (dmin_n*mn_ns)
-// (S = sum of the block's int8 activations).
+// The contraction runs on the int8 matrix cores.  One v_mfma_i32_32x32x32_i8 contracts one
+// 32-weight sub-block of 32 weight rows against the matching Q8_0 block of 32 tokens, so
+// every int32 result is exactly one "group sum" I[m][n][s] of the matvec (Q6_K, whose scales
+// change every 16 weights, uses two v_mfma_i32_32x32x16_i8 per sub-block).  The fp32 value is
+//   y[m][n] = sum_s da[m][s] * dsc[n][s] * I[m][n][s]  +  sum_s (da[m][s]*S[m][s]) * z[n][s]
+// with dsc the weight scale of the sub-block (d*sc for the K-quants), S the sum of the block's
+// int8 activations and z the zero-point factor (-dmin*mn for Q4_K, -8*d for Q4_0, else absent).
 //  * first sum: the MFMA adds into the constant 0x4B400000 (= 12582912.0f), so the
 //    int32 result read as a float is 12582912 + I exactly; one fma with the per-lane
-//    constants dsc and -12582912*dsc (exact: dsc has <= 17 significant bits) gives
+//    constants dsc and -12582912*dsc (exact: dsc has <= 19 significant bits) gives
 //    fl(dsc * I) -- the rounding of the reference's `da * dot as f32` -- without an
 //    int->float conversion, and a second fma with the token's f16 scale accumulates.
 //    Two VALU operations per (token, weight row, sub-block): that, not the matrix
 //    core, bounds this kernel.
 //  * second sum: a rank-(k/32) fp32 product, added into the same accumulators with
-//    v_mfma_f32_32x32x2_f32 on P[m][s] = da*S and -dmin*mn while the VALU works on
-//    other tiles.
+//    v_mfma_f32_32x32x2_f32 on P[m][s] = da*S and z while the VALU works on other tiles.
 // A small preparation kernel lays the activations out once per call: int8 payload
-// tiled [k/32][m][32] (so every MFMA operand load is one aligned, contiguous KB),
-// P as fp32 [k/32][m], da as f16 [k/32][m].
+// tiled [k/32][m][32] in the byte order the format's operands need (so every MFMA operand
+// load is one aligned, contiguous KB), P as fp32 [k/32][m], da as f16 [k/32][m].
 #include "oxq_gemv_kernel.hpp"
 #include "oxq_internal.hpp"
 

@@ -14,6 +14,9 @@ namespace oxq {
 // (into a second register set) before the current batch is reduced, so every
 // wave always has loads in flight.  With KS > 1 the per-wave row sums are added
 // through LDS in a fixed order (part 0, 1, ...), one barrier per batch.
+// SRC says where the activations come from: Q8_0 blocks in memory (ActQ8), or an fp32
+// vector that the work group quantizes into LDS first (ActF32).  blockIdx.y selects one
+// of up to four matrices of the same shape that share the activations.
 template <class F, int STEPS, int RB>
 struct Batch {
     typename F::Wt w[RB][STEPS];
