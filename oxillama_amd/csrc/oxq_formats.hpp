@@ -117,8 +117,9 @@ struct FmtQ4K {
     };
     struct Act {
         u32x4 lo0, lo1, hi0, hi1;
-        float a_lo, a_hi;  // d_a of the two activation blocks
-        float b_lo, b_hi;  // d_a * sum(q_a)
+        float a_lo, a_hi16;  // d_a of the low-nibble block; d_a / 16 of the high-nibble block
+        float b_lo, b_hi;    // d_a * sum(q_a)
+        int s_hi128;         // 128 * sum(q_a) of the high-nibble block
     };
     struct Wt {
         u32x4 hdr, q0, q1;
@@ -144,9 +145,10 @@ struct FmtQ4K {
         }
         const float dlo = h2f(dlo_bits), dhi = h2f(dhi_bits);
         a.a_lo = valid ? dlo : 0.0f;
-        a.a_hi = valid ? dhi : 0.0f;
+        a.a_hi16 = valid ? dhi * 0.0625f : 0.0f;  // exact
         a.b_lo = valid ? dlo * (float)slo : 0.0f;
         a.b_hi = valid ? dhi * (float)shi : 0.0f;
+        a.s_hi128 = 128 * shi;
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &k) {
         const uint8_t *blk = row + (size_t)(u >> 2) * BLOCK_BYTES;
@@ -157,16 +159,19 @@ struct FmtQ4K {
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &k, int32_t *sums,
                                                 uint32_t u, bool valid) {
-        int plo = 0, phi = 0;
+        // Low nibbles: q & 0x0F.  High nibbles stay in place: (q & 0xF0) ^ 0x80 read as a signed byte is
+        // 16 * (n - 8), so the dot product is 16 * (sum n*a - 8 * sum a); adding 128 * sum a gives
+        // 16 * phi exactly, one operation per dword instead of a shift and a mask.
+        int plo = 0, phi16 = a.s_hi128;
         for (int i = 0; i < 4; i++) {
             plo = sdot4(w.q0[i] & 0x0F0F0F0Fu, a.lo0[i], plo);
-            phi = sdot4((w.q0[i] >> 4) & 0x0F0F0F0Fu, a.hi0[i], phi);
+            phi16 = sdot4((w.q0[i] & 0xF0F0F0F0u) ^ 0x80808080u, a.hi0[i], phi16);
             plo = sdot4(w.q1[i] & 0x0F0F0F0Fu, a.lo1[i], plo);
-            phi = sdot4((w.q1[i] >> 4) & 0x0F0F0F0Fu, a.hi1[i], phi);
+            phi16 = sdot4((w.q1[i] & 0xF0F0F0F0u) ^ 0x80808080u, a.hi1[i], phi16);
         }
         if (DUMP && valid) {
             sums[2 * u] = plo;
-            sums[2 * u + 1] = phi;
+            sums[2 * u + 1] = phi16 >> 4;
         }
         // 6-bit scales / mins of sub-blocks 2g, 2g+1 as byte pairs (decode_scales_mins,
         // q4_k.rs:27-49): j < 4: sc = s[j] & 63, mn = s[j+4] & 63; j >= 4: sc = (s[j+4] & 15) |
@@ -178,7 +183,8 @@ struct FmtQ4K {
         const uint32_t mn2 = (y & m1) | ((sb >> 2) & m2);
         const float d = h2f(w.hdr[0] & 0xFFFF), dmin = h2f(w.hdr[0] >> 16);
         float su = a.a_lo * (float)mul24(plo, (int)(sc2 & 0xFF));
-        su = fmaf(a.a_hi, (float)mul24(phi, (int)((sc2 >> 8) & 0xFF)), su);
+        // |16 phi| < 2^20 fits mul24; 16 * phi * sc is a multiple of 16 below 2^26: exact in fp32
+        su = fmaf(a.a_hi16, (float)mul24(phi16, (int)((sc2 >> 8) & 0xFF)), su);
         float sv = a.b_lo * (float)(mn2 & 0xFF);
         sv = fmaf(a.b_hi, (float)((mn2 >> 8) & 0xFF), sv);
         return fmaf(d, su, -(dmin * sv));
