@@ -195,13 +195,14 @@ int oxq_gemv_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_wei
                        const float *d_x, float *const *d_outs, size_t n_rows, size_t n_cols,
                        int accumulate, void *stream);
 
-/* Prefill: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched form
- * of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  With m >= 3 and k a
- * multiple of 256 every format uses the int8-MFMA tile kernel, which needs oxq_gemm_q8_workspace_bytes()
- * bytes of 256-byte-aligned device scratch: pass it and the call is asynchronous
- * and allocation-free; pass NULL and the library uses its own scratch (the call
- * then serialises and waits for the stream).  Shapes for which the workspace size is 0
- * run m fused matvecs and ignore the workspace. */
+/* Prefill / decode batch: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched
+ * form of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  From 6 rows up
+ * (13 where n < 8192), with k a multiple of 256, every format runs on the int8-MFMA tile
+ * kernel, which needs oxq_gemm_q8_workspace_bytes() bytes of 256-byte-aligned device scratch:
+ * pass it and the call is asynchronous and allocation-free; pass NULL and the library uses
+ * its own scratch (the call then serialises and waits for the stream).  Fewer rows, and
+ * shapes for which the workspace size is 0, run GEMV launches (up to four rows per pass over
+ * the weights) and ignore the workspace. */
 size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k);
 int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                     float *d_out, size_t m, size_t n, size_t k, int accumulate,
@@ -244,6 +245,9 @@ int oxq_set_gemv_rows_per_batch(unsigned rows);
 /* Waves that share one row in the GEMV kernels (1 or 4; tuning knob; 0 restores the
  * per-shape default: 4 for rows of three or more 64-unit steps). */
 int oxq_set_gemv_waves_per_row(unsigned waves);
+/* Fewest activation rows for which oxq_gemm_q8_dev / oxq_gemm take the tile kernel; below it
+ * they run GEMV launches, two to four rows per launch (tuning knob; 0 restores the default). */
+int oxq_set_gemm_tile_min_rows(unsigned rows);
 /* Tile shape / prefetch depth of the prefill kernel (tuning knob; 0 restores the default). */
 int oxq_set_gemm_variant(int variant);
 

@@ -93,6 +93,7 @@ SIGNATURES = {
     "oxq_set_gemv_rows_per_batch": (C.c_int, [C.c_uint]),
     "oxq_set_gemv_waves_per_row": (C.c_int, [C.c_uint]),
     "oxq_set_gemm_variant": (C.c_int, [C.c_int]),
+    "oxq_set_gemm_tile_min_rows": (C.c_int, [C.c_uint]),
 }
 
 _lib = None

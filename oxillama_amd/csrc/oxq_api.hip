@@ -12,6 +12,7 @@
 
 namespace oxq {
 extern int g_gemm_variant;
+extern uint32_t g_gemm_tile_min_rows;
 hipError_t launch_dequant(uint32_t type, const uint8_t *blocks, size_t n_blocks, float *out, hipStream_t stream);
 }
 
@@ -365,6 +366,11 @@ int oxq_set_gemv_waves_per_row(unsigned waves) {
     return OXQ_OK;
 }
 
+int oxq_set_gemm_tile_min_rows(unsigned rows) {
+    oxq::g_gemm_tile_min_rows = rows;
+    return OXQ_OK;
+}
+
 int oxq_set_gemm_variant(int variant) {
     oxq::g_gemm_variant = variant;
     return OXQ_OK;
@@ -497,7 +503,7 @@ int oxq_gemm(uint32_t type, const uint8_t *data, size_t data_len, const size_t *
     ga.out = (float *)g.s_out.ptr;
     ga.sums = nullptr;
     ga.workspace = nullptr;
-    if (oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n_cols)) {
+    if (oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n_rows, (uint32_t)n_cols)) {
         if ((st = g.s_work.reserve(oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)n_cols))) != OXQ_OK) return st;
         ga.workspace = (uint8_t *)g.s_work.ptr;
     }
@@ -648,8 +654,9 @@ int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d
 }
 
 size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k) {
-    (void)n;
-    if (m > 0xFFFFFFFFull || k > 0xFFFFFFFFull || !oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)k)) return 0;
+    if (m > 0xFFFFFFFFull || n > 0xFFFFFFFFull || k > 0xFFFFFFFFull ||
+        !oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k))
+        return 0;
     return oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k);
 }
 
@@ -709,7 +716,10 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
 }
 
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k) {
-    return oxq_gemm_q8_workspace_bytes(type, total_rows < 3 ? 3 : total_rows, n, k);
+    (void)n;
+    if (total_rows > 0x7FFFFFFFull || k > 0xFFFFFFFFull || !oxq::gemm_tiles_supported(type, (uint32_t)total_rows, (uint32_t)k))
+        return 0;
+    return oxq::gemm_workspace_bytes((uint32_t)total_rows, (uint32_t)k);
 }
 
 int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
@@ -738,7 +748,7 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
     ga.out = d_out;
     ga.sums = d_sums;
     ga.workspace = (uint8_t *)d_workspace;
-    ga.m = (uint32_t)(total_rows < 3 ? 3 : total_rows);  // the tile kernel's minimum; rows past the offsets are never stored
+    ga.m = (uint32_t)total_rows;
     ga.n = (uint32_t)n;
     ga.k = (uint32_t)k;
     ga.accumulate = accumulate ? 1 : 0;

@@ -632,11 +632,30 @@ OXQ_TILE_KERNEL(gemm_tile_kernel, 2)
 OXQ_TILE_KERNEL(gemm_tile_kernel_occ3, 3)
 #undef OXQ_TILE_KERNEL
 
-// One fused matvec per activation row: every format other than Q4_K, and Q4_K shapes the
-// tile kernel does not take.
+// Without the tile kernel (very few rows, or a shape it does not take): GEMV launches, two to
+// four activation rows per pass over the weights where the row length allows.
 static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t stream) {
     const size_t act_row_bytes = (size_t)(a.k / 32) * 34;
-    for (uint32_t r = 0; r < a.m; r++) {
+    const uint32_t vecs = gemv_vecs_max(type, a.k);
+    uint32_t r = 0;
+    while (r < a.m) {
+        const uint32_t left = a.m - r;
+        if (vecs >= 2 && left >= 2) {  // 2..4 activation rows share one pass over the weights
+            GemvVecsArgs v;
+            v.W = a.W;
+            v.A = a.A + r * act_row_bytes;
+            v.a_stride = act_row_bytes;
+            v.out = a.out + (size_t)r * a.n;
+            v.out_stride = a.n;
+            v.n_vecs = left < vecs ? left : vecs;
+            v.n_rows = a.n;
+            v.n_cols = a.k;
+            v.accumulate = a.accumulate;
+            hipError_t e = launch_gemv_vecs(type, v, stream);
+            if (e != hipSuccess) return e;
+            r += v.n_vecs;
+            continue;
+        }
         GemvArgs g;
         g.W = a.W;
         g.A = a.A + r * act_row_bytes;
@@ -650,6 +669,7 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
         g.waves_per_row = 0;
         hipError_t e = launch_gemv_q8(type, g, stream);
         if (e != hipSuccess) return e;
+        r++;
     }
     return hipSuccess;
 }
@@ -723,22 +743,32 @@ size_t gemm_workspace_bytes(uint32_t m, uint32_t k) {
     return nsb * mpad * (32 + 4 + 2);
 }
 
-// Below this many activation rows one GEMV launch per row is faster than the tile kernel
-// (measured at 14336 x 4096: 9 us per row against 23 us for up to 32 rows).
-constexpr uint32_t GEMM_TILE_MIN_ROWS = 3;
+uint32_t g_gemm_tile_min_rows = 0;  // tuning: 0 = default
 
-bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t k) {
+// The tile kernel can take this format and shape at all.
+bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
     // LDS holds the f16 token scales of up to 128 tokens for the whole k (k/32 * 256 bytes)
     // beside up to 24 KB of decoded weight scales; up to k = 8192 two work groups share a CU
     const bool known = type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K ||
                        type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0;
     // the 32-weight formats are walked eight blocks at a time
-    return known && k % 256 == 0 && m >= GEMM_TILE_MIN_ROWS && (size_t)(k / 32) * 256 <= 128 * 1024 &&
+    return known && k % 256 == 0 && m >= 1 && (size_t)(k / 32) * 256 <= 128 * 1024 &&
            gemm_workspace_bytes(m, k) < 0x7FFFFFFFull;
 }
 
+// ... and is the faster way for m activation rows.  Below the threshold GEMV launches that take up
+// to four rows per pass over the weights win (measured: 14336 x 4096 Q4_K, 4 rows 15 us, 8 rows 28 us
+// against 22 us for the tile kernel; 4096-row matrices give the tile kernel too few work groups:
+// 4096 x 14336 Q6_K, 12 rows 62 us against 89 us).
+bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
+    const uint32_t min_rows = g_gemm_tile_min_rows ? g_gemm_tile_min_rows : (n >= 8192 ? 6 : 13);
+    return gemm_tiles_supported(type, m, k) && m >= min_rows;
+}
+
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) {
-    if (!gemm_uses_tiles(type, a.m, a.k) || a.workspace == nullptr) {
+    const bool tiles = a.workspace != nullptr &&
+                       (a.offsets ? gemm_tiles_supported(type, a.m, a.k) : gemm_uses_tiles(type, a.m, a.n, a.k));
+    if (!tiles) {
         if (a.offsets) return hipErrorInvalidValue;  // grouped form exists for the tile kernel only
         return gemm_by_rows(type, a, stream);
     }

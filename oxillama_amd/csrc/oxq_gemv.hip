@@ -121,6 +121,63 @@ static bool multi_in_one_launch(const GemvArgs &a) {
     return (a.n_cols / F::UNIT_COLS + 63) / 64 <= 32 && !a.sums;
 }
 
+// ---- several activation vectors per launch -------------------------------------------------
+
+template <class F, int STEPS, int KS, int NV>
+static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t row_bytes, hipStream_t stream) {
+    constexpr uint32_t G = 4 / KS;
+    const uint32_t max_groups = device_cus() * 8 / KS;
+    const uint32_t passes = (a.n_rows + max_groups - 1) / max_groups;
+    const uint32_t groups = (a.n_rows + passes - 1) / passes;
+    uint32_t blocks = (groups + G - 1) / G;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride, a.out,
+                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs);
+    return hipGetLastError();
+}
+
+// Same split of a row over steps and waves as the single-vector kernel (so the fp32 sums are
+// formed in the same order and the results are bit-identical to one launch per vector); two
+// steps per wave leave registers for two vectors only.
+template <class F>
+static hipError_t launch_vecs_f(const GemvVecsArgs &a, hipStream_t stream) {
+    const uint32_t units = a.n_cols / F::UNIT_COLS;
+    const size_t row_bytes = (size_t)(a.n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
+    const uint32_t steps = (units + 63) / 64;
+    if (steps == 1)
+        return a.n_vecs > 2 ? launch_vecs_k<F, 1, 1, 4>(a, units, row_bytes, stream)
+                            : launch_vecs_k<F, 1, 1, 2>(a, units, row_bytes, stream);
+    if (steps == 2 && a.n_vecs <= 2) return launch_vecs_k<F, 2, 1, 2>(a, units, row_bytes, stream);
+    if (steps == 3 || steps == 4)
+        return a.n_vecs > 2 ? launch_vecs_k<F, 1, 4, 4>(a, units, row_bytes, stream)
+                            : launch_vecs_k<F, 1, 4, 2>(a, units, row_bytes, stream);
+    if (steps >= 5 && steps <= 8 && a.n_vecs <= 2) return launch_vecs_k<F, 2, 4, 2>(a, units, row_bytes, stream);
+    return hipErrorNotSupported;
+}
+
+// Most activation vectors one launch takes for rows of n_cols columns (0: none).
+uint32_t gemv_vecs_max(uint32_t type, uint32_t n_cols) {
+    uint32_t unit = 32;
+    if (type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_Q6_K) unit = 64;
+    const uint32_t steps = (n_cols / unit + 63) / 64;
+    if (steps == 1 || steps == 3 || steps == 4) return 4;
+    if (steps == 2 || (steps >= 5 && steps <= 8)) return 2;
+    return 0;
+}
+
+// 2..4 activation vectors (3 run in the 4-vector kernel, which repeats the last one).
+hipError_t launch_gemv_vecs(uint32_t type, const GemvVecsArgs &a, hipStream_t stream) {
+    if (a.n_rows == 0 || a.n_cols == 0) return hipSuccess;
+    switch (type) {
+    case OXQ_TYPE_Q4_0: return launch_vecs_f<FmtQ4_0>(a, stream);
+    case OXQ_TYPE_Q8_0: return launch_vecs_f<FmtQ8_0>(a, stream);
+    case OXQ_TYPE_Q4_K: return launch_vecs_f<FmtQ4K>(a, stream);
+    case OXQ_TYPE_Q6_K: return launch_vecs_f<FmtQ6K>(a, stream);
+    case OXQ_TYPE_IQ4_XS: return launch_vecs_f<FmtIQ4XS>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 bool gemv_takes_f32(uint32_t type, uint32_t n_cols) {
     uint32_t unit = 32;
     if (type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_Q6_K) unit = 64;

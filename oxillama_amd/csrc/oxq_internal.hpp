@@ -34,6 +34,21 @@ hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream);
 // True when the GEMV of this row length can quantize fp32 activations itself (GemvArgs::X).
 bool gemv_takes_f32(uint32_t type, uint32_t n_cols);
 
+// 2..4 activation vectors against one weight matrix in one launch (a small decode batch).
+struct GemvVecsArgs {
+    const uint8_t *W;
+    const uint8_t *A;    // vector v: Q8_0 blocks at A + v * a_stride
+    size_t a_stride;     // bytes
+    float *out;          // vector v: out + v * out_stride
+    size_t out_stride;   // floats
+    uint32_t n_vecs;     // 2, 3 or 4
+    uint32_t n_rows, n_cols;
+    int accumulate;
+};
+hipError_t launch_gemv_vecs(uint32_t type, const GemvVecsArgs &a, hipStream_t stream);
+// Most activation vectors one launch takes for rows of n_cols columns (4, 2, or 0: none).
+uint32_t gemv_vecs_max(uint32_t type, uint32_t n_cols);
+
 // x: n floats (n % 32 == 0) -> n/32 Q8_0 blocks of 34 bytes.
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *out, hipStream_t stream);
 
@@ -56,6 +71,8 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
 // Device scratch the tile kernel needs for m tokens of k columns (activation re-layout).
 size_t gemm_workspace_bytes(uint32_t m, uint32_t k);
 // True when (type, m, k) is served by the int8-MFMA tile kernel.
-bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t k);
+bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k);
+// True when the tile kernel can take (type, m, k) at all (the grouped form always uses it).
+bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k);
 
 }  // namespace oxq

@@ -250,6 +250,36 @@ def test_gemv_dev_quantizes_in_kernel_bit_identically(hip, ref, t):
         assert torch.equal(multi[0], single[0]) and torch.equal(multi[1], single[1])
 
 
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_gemm_few_rows_share_one_weight_pass(hip, ref, t):
+    """2..7 activation rows without the tile kernel: GEMV launches that take up to four rows per
+    pass over the weights give the same bits as one fused matvec per row (short rows, rows split
+    over four waves, and rows too long for the shared pass)."""
+    import torch
+    from oxillama_amd import capi
+    lib = capi.load()
+    lib.oxq_set_gemm_tile_min_rows(1000)
+    try:
+        for n, k_ in ((40, 768), (24, 4096), (12, 14336), (6, 32768)):
+            w = synth.weights(t, 840 + n, n, k_)
+            dw = torch.from_numpy(w).cuda()
+            kern = hip.HipKernel(t)
+            for m in (2, 3, 4, 5, 7):
+                acts = ref.quantize_q8_0(synth.normal_f32(850 + m, m * k_))
+                da = torch.from_numpy(acts).cuda()
+                arb = k_ // 32 * 34
+                want = torch.full((m, n), 1.5, dtype=torch.float32, device="cuda")
+                got = torch.full((m, n), 1.5, dtype=torch.float32, device="cuda")
+                for acc in (False, True):
+                    for r in range(m):
+                        kern.matvec_q8_fused_dev(dw, da[r * arb:(r + 1) * arb], want[r], n, k_, accumulate=acc)
+                    kern.gemm_q8_dev(dw, da, got, m, n, k_, accumulate=acc)
+                    torch.cuda.synchronize()
+                    assert torch.equal(got, want), (O.NAMES[t], n, k_, m, acc)
+    finally:
+        lib.oxq_set_gemm_tile_min_rows(0)
+
+
 def test_empty_inputs(hip):
     for t in O.ALL_TYPES:
         k = hip.HipKernel(t)
@@ -387,8 +417,19 @@ def test_prefill_tile_kernel(hip, ref, shape, t):
     """Weights of every format x Q8_0 activations on the int8-MFMA tile kernel: integer sub-block sums bit-exact, fp32 within
     1e-5, ragged tile edges in both directions, overwrite and accumulate."""
     import torch
+    from oxillama_amd import capi
     m, n, k_ = shape
     say("prefill", O.NAMES[t], shape)
+    capi.load().oxq_set_gemm_tile_min_rows(1)  # small shapes would otherwise take the GEMV route
+    try:
+        _prefill_tile_case(hip, ref, shape, t)
+    finally:
+        capi.load().oxq_set_gemm_tile_min_rows(0)
+
+
+def _prefill_tile_case(hip, ref, shape, t):
+    import torch
+    m, n, k_ = shape
     w = synth.weights(t, 600 + m, n, k_)
     x = synth.normal_f32(700 + n, m * k_)
     acts = ref.quantize_q8_0(x)
