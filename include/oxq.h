@@ -197,7 +197,7 @@ int oxq_gemv_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_wei
 
 /* Prefill / decode batch: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched
  * form of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  From 6 rows up
- * (13 where n < 8192), with k a multiple of 256, every format runs on the int8-MFMA tile
+ * (9 where n < 8192), with k a multiple of 256, every format runs on the int8-MFMA tile
  * kernel, which needs oxq_gemm_q8_workspace_bytes() bytes of 256-byte-aligned device scratch:
  * pass it and the call is asynchronous and allocation-free; pass NULL and the library uses
  * its own scratch (the call then serialises and waits for the stream).  Fewer rows, and

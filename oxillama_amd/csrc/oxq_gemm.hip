@@ -732,6 +732,10 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
         // three waves per SIMD.
         if (rows > 384) return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
         if (rows > 64) return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
+        // split k; 64 weight rows (or 64 tokens) per work group only where that still leaves every
+        // compute unit at least one work group, else 32 x 32
+        if ((size_t)((a.n + 63) / 64) * (a.offsets ? a.n_experts : 1) < device_cus())
+            return launch_tile<F, 1, 1, 0, 2, false, 2, 2>(a, p, stream);
         if (rows > 32) return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
         return launch_tile<F, 1, 2, 0, 2, false, 2, 2>(a, p, stream);
     }
@@ -758,10 +762,10 @@ bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
 
 // ... and is the faster way for m activation rows.  Below the threshold GEMV launches that take up
 // to four rows per pass over the weights win (measured: 14336 x 4096 Q4_K, 4 rows 15 us, 8 rows 28 us
-// against 22 us for the tile kernel; 4096-row matrices give the tile kernel too few work groups:
-// 4096 x 14336 Q6_K, 12 rows 62 us against 89 us).
+// against 22 us for the tile kernel; 4096-row matrices give the tile kernel fewer work groups:
+// 4096 x 14336 Q6_K, 8 rows 41 us against 55 us, 12 rows 61 us against 55 us).
 bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
-    const uint32_t min_rows = g_gemm_tile_min_rows ? g_gemm_tile_min_rows : (n >= 8192 ? 6 : 13);
+    const uint32_t min_rows = g_gemm_tile_min_rows ? g_gemm_tile_min_rows : (n >= 8192 ? 6 : 9);
     return gemm_tiles_supported(type, m, k) && m >= min_rows;
 }
 
