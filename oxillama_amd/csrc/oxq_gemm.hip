@@ -384,11 +384,32 @@ __device__ __forceinline__ void gemm_tile_body(
 
     // Token scales of this work group's tokens, permuted so that the 16 values a lane needs
     // for one MFMA tile are 32 contiguous bytes.
-    for (uint32_t idx = tid; idx < nsb * WG_TOK; idx += 256) {
-        const uint32_t j = idx / WG_TOK, tl = idx % WG_TOK;
-        const uint32_t mt = tl >> 5, r = tl & 31;  // r = 8a + 4hh + b
-        const uint32_t a = r >> 3, hh = (r >> 2) & 1, b = r & 3;
-        lds_da[((j * MTILES + mt) * 2 + hh) * 16 + a * 4 + b] = da16[(size_t)j * mpad + m_wg + tl];
+    // One task = 8 consecutive tokens of one sub-block (16 bytes in, two 8-byte pieces out: token
+    // r = 8a + 4hh + b of a tile goes to [hh][4a + b]); four tasks per trip, loads before stores.
+    {
+        constexpr uint32_t CH = WG_TOK / 8;  // 8-token chunks per sub-block
+        const uint32_t n_tasks = nsb * CH;
+        for (uint32_t base = 0; base < n_tasks; base += 4 * 256) {
+            u32x4 v[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t task = min(base + q * 256 + tid, n_tasks - 1);
+                const uint32_t j = task / CH, ch = task % CH;
+                v[q] = ld16(reinterpret_cast<const uint8_t *>(da16 + (size_t)j * mpad + m_wg + 8 * ch));
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const uint32_t task = base + q * 256 + tid;
+                if (task < n_tasks) {
+                    const uint32_t j = task / CH, ch = task % CH;
+                    const uint32_t mt = ch >> 2, a = ch & 3;
+                    u32x2 *d0 = reinterpret_cast<u32x2 *>(&lds_da[((j * MTILES + mt) * 2 + 0) * 16 + a * 4]);
+                    u32x2 *d1 = reinterpret_cast<u32x2 *>(&lds_da[((j * MTILES + mt) * 2 + 1) * 16 + a * 4]);
+                    *d0 = u32x2{v[q][0], v[q][1]};
+                    *d1 = u32x2{v[q][2], v[q][3]};
+                }
+            }
+        }
     }
 
     // Operands come through buffer loads: a wave-uniform descriptor, a fixed 32-bit
