@@ -73,7 +73,7 @@ def main():
         sys.exit(2)
 
     import torch
-    from oxillama_amd import quant, synth
+    from oxillama_amd import linear, quant, synth
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -156,20 +156,22 @@ def main():
 
     def step(i):
         """One layer, five launches: quantize x; q_proj; ffn_gate + ffn_up (one launch: both read
-        the same vector); quantize h; ffn_down.  --fused-quantize lets the GEMV kernels quantize
-        their fp32 input themselves (three launches, bit-identical results); measured slightly
-        slower here (40.2 vs 38.5 us per layer): every work group then quantizes the whole vector
-        into LDS before its first row, which costs more than the two small launches it saves."""
+        the same vector); h = silu(gate) * up quantized to Q8_0 in the same kernel; ffn_down on h.
+        --fused-quantize lets the GEMV kernels quantize their fp32 input themselves (four
+        launches, bit-identical results); measured slightly slower here: every work group then
+        quantizes the whole vector into LDS before its first row, which costs more than the
+        small launches it saves."""
         w = layers[i % L]
         if not args.fused_quantize:
             quant.quantize_q8_0_dev(x, xq)
             k_q8.matvec_q8_fused_dev(w["q"], xq, yq, H, H, accumulate=False)
             k_q4k.matvec_q8_fused_multi_dev([w["gate"], w["up"]], xq, [yg, yu], F, H, accumulate=False)
-            quant.quantize_q8_0_dev(h, hq)
+            linear.swiglu_quantize_dev(yg, yu, None, hq)
             k_q6k.matvec_q8_fused_dev(w["down"], hq, yd, H, F, accumulate=False)
         else:
             k_q8.gemv_dev(w["q"], x, yq, H, H)
             k_q4k.gemv_multi_dev([w["gate"], w["up"]], x, [yg, yu], F, H)
+            linear.swiglu_quantize_dev(yg, yu, h, None)
             k_q6k.gemv_dev(w["down"], h, yd, H, F)
 
     def capture(fn):
@@ -382,7 +384,7 @@ def main():
         cores = min(os.cpu_count() or 1, 16)
         hw = {"q": layers[0]["q"].cpu().numpy(), "gate": layers[0]["gate"].cpu().numpy(),
               "up": layers[0]["up"].cpu().numpy(), "down": layers[0]["down"].cpu().numpy()}
-        hx, hh = x.cpu().numpy(), h.cpu().numpy()
+        hx = x.cpu().numpy()
 
         avx2 = O.load_avx2() is not None
 
@@ -394,9 +396,9 @@ def main():
         def cpu_step(threads):
             a = O.quantize_q8_0(hx)
             fused(O.Q8_0, hw["q"], a, H, H, threads)
-            fused(O.Q4_K, hw["gate"], a, F, H, threads)
-            fused(O.Q4_K, hw["up"], a, F, H, threads)
-            b = O.quantize_q8_0(hh)
+            hg = fused(O.Q4_K, hw["gate"], a, F, H, threads)
+            hu = fused(O.Q4_K, hw["up"], a, F, H, threads)
+            b = O.quantize_q8_0(O.swiglu(hg, hu))
             fused(O.Q6_K, hw["down"], b, H, F, threads)
 
         def time_cpu(threads, budget_s):
@@ -412,7 +414,7 @@ def main():
         s_mt, n_mt = time_cpu(cores, 8.0)
         s_1t, n_1t = time_cpu(1, 8.0)
         cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-               "sample": f"one layer (same 4 matrices + 2 quantizations), {n_mt} repeats, static row split over "
+               "sample": f"one layer (same 4 matrices, quantization of x, SwiGLU + quantization of h), {n_mt} repeats, static row split over "
                          f"{cores} threads; " + ("AVX2 intrinsics twin of the reference's fused rows (Q6_K body is scalar "
                          "there too)" if avx2 else "scalar C restatement of the reference's AVX2-tier fused rows"),
                "ms_per_step": round(s_mt * 1e3, 3),
@@ -437,9 +439,9 @@ def main():
                    "weight_bytes_per_step": step_weight_bytes, "distinct_layers": L,
                    "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
                    "launch": "one HIP graph of all timed steps; per step " +
-                             ("2 quantizations, q_proj, gate+up (one launch), down" if not args.fused_quantize else
-                              "q_proj, gate+up (one launch), down, each quantizing its fp32 input vector to Q8_0 in "
-                              "registers")},
+                             ("quantize x, q_proj, gate+up (one launch), SwiGLU + quantize, down" if not args.fused_quantize
+                              else "q_proj, gate+up (one launch), SwiGLU, down, each projection quantizing its fp32 "
+                                   "input vector to Q8_0 itself")},
         "roofline": roofline,
         "cpu_baseline": cpu,
         "kernels": kernels,

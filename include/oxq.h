@@ -233,6 +233,91 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
                         size_t n, size_t k, int accumulate, void *d_workspace,
                         size_t workspace_bytes, void *stream);
 
+/* ---- the callers of the kernel trait: QuantLinear, the dense SwiGLU feed-forward, RMSNorm ----
+ *
+ * LoRA adapter on device memory (LoraAdapter, crates/oxillama-quant/src/lora.rs:21-35): d_a is
+ * [rank x in_features], d_b is [out_features x rank], both row-major fp32; d_r is rank floats
+ * of device scratch that the call overwrites. */
+typedef struct oxq_lora {
+    const float *d_a;
+    const float *d_b;
+    float *d_r;
+    size_t rank;
+    float scale;
+} oxq_lora;
+
+/* LoraAdapter::apply (lora.rs:83-124): d_out += d_b (d_a d_x) * scale.  NULL or rank 0: no-op. */
+int oxq_lora_apply_dev(const oxq_lora *lora, const float *d_x, float *d_out, size_t out_features,
+                       size_t in_features, void *stream);
+
+/* QuantLinear::forward (crates/oxillama-arch/src/common/linear.rs:77-98): d_out = W . q8(x)
+ * + bias + LoRA correction, in that order.  Activations: pass d_acts_q8 (Q8_0 blocks of x,
+ * quantized once for every projection that reads x), or NULL to have the kernel quantize d_x
+ * itself (as oxq_gemv_dev).  d_x is needed for the LoRA term; d_bias and lora may be NULL.
+ * The bias rides in the matvec's epilogue (no extra launch); LoRA adds two small launches. */
+int oxq_linear_forward_dev(uint32_t type, const uint8_t *d_weights, const float *d_x,
+                           const uint8_t *d_acts_q8, const float *d_bias, const oxq_lora *lora,
+                           float *d_out, size_t out_features, size_t in_features, void *stream);
+
+/* Up to 4 QuantLinear::forward calls on the same input as one launch: wq/wk/wv, or ffn_gate/
+ * ffn_up, which the reference issues one after the other
+ * (crates/oxillama-arch/src/llama/model.rs:295-310).  The matrices share the format and
+ * in_features; each has its own out_features[i], output and optional bias (d_biases may be
+ * NULL, and so may any entry).  Results are bit-identical to separate calls. */
+int oxq_linear_forward_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_weights,
+                                 const uint8_t *d_acts_q8, const float *const *d_biases,
+                                 float *const *d_outs, const size_t *out_features,
+                                 size_t in_features, void *stream);
+
+/* QuantLinear::forward_batch (linear.rs:105-132): d_out[batch x out_features] = gemm + bias
+ * broadcast over the batch (no LoRA, as in the reference).  Workspace as oxq_gemm_q8_dev. */
+int oxq_linear_forward_batch_dev(uint32_t type, const uint8_t *d_weights,
+                                 const uint8_t *d_acts_q8, const float *d_bias, float *d_out,
+                                 size_t batch, size_t out_features, size_t in_features,
+                                 void *d_workspace, size_t workspace_bytes, void *stream);
+
+/* QuantLinear::forward on host slices, staged per call like oxq_gemv (drop-in route).  bias:
+ * NULL or bias_len floats (a short bias covers its own length, as the reference's zip does);
+ * LoRA: NULL pointers or rank 0 for none, else lora_a_len == rank * in_features and
+ * lora_b_len == out_features * rank (LoraAdapter::new, lora.rs:43-73) or
+ * OXQ_ERR_DIMENSION_MISMATCH. */
+int oxq_linear_forward(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape,
+                       size_t n_dims, const float *bias, size_t bias_len, const float *lora_a,
+                       size_t lora_a_len, const float *lora_b, size_t lora_b_len, size_t rank,
+                       float scale, const float *input, size_t input_len, float *output,
+                       size_t output_len);
+
+/* QuantLinear::forward_batch on host slices (linear.rs:105-132): gemm with n = shape[0] and
+ * k = shape[1], then the bias added to every row of the batch. */
+int oxq_linear_forward_batch(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape,
+                             size_t n_dims, const float *bias, size_t bias_len, const float *input,
+                             size_t input_len, float *output, size_t output_len, size_t batch);
+
+/* swiglu_inplace (crates/oxillama-arch/src/common/swiglu.rs:15-21) fused with the quantizer of
+ * the next projection's input: h = silu(gate) * up over n_total floats (a multiple of 32),
+ * sigmoid = 1 / (1 + exp(-g)), h = (g * sigmoid) * u.  d_h (fp32 h) and d_out_q8 (Q8_0 blocks
+ * of h, bit-exact to quantizing d_h) are each optional (NULL). */
+int oxq_swiglu_quantize_q8_0_dev(const float *d_gate, const float *d_up, size_t n_total,
+                                 float *d_h, uint8_t *d_out_q8, void *stream);
+
+/* RmsNorm::forward_to (crates/oxillama-arch/src/common/rms_norm.rs:49-66) fused with the
+ * quantizer: per row of n floats (a multiple of 32), y = (x * (1 / sqrt(mean(x^2) + eps))) *
+ * weight.  d_y (fp32) and d_out_q8 (Q8_0 blocks of y, bit-exact to quantizing d_y) are each
+ * optional (NULL).  The sum of squares is a tree sum (the reference adds in index order). */
+int oxq_rmsnorm_quantize_q8_0_dev(const float *d_x, const float *d_weight, float eps, size_t rows,
+                                  size_t n, float *d_y, uint8_t *d_out_q8, void *stream);
+
+/* Dense feed-forward block (crates/oxillama-arch/src/llama/model.rs:277-310): d_out =
+ * down(silu(gate(x)) * up(x)) for one token, from the Q8_0 blocks of the normed hidden state.
+ * Three launches when gate and up share a format (gate + up, SwiGLU + quantize, down), four
+ * otherwise.  Needs oxq_ffn_workspace_bytes() bytes of 256-byte-aligned device scratch;
+ * allocates nothing and does not synchronise. */
+size_t oxq_ffn_workspace_bytes(size_t hidden, size_t intermediate);
+int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_type,
+                       const uint8_t *d_up, uint32_t down_type, const uint8_t *d_down,
+                       const uint8_t *d_acts_q8, float *d_out, size_t hidden, size_t intermediate,
+                       void *d_workspace, size_t workspace_bytes, void *stream);
+
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                        int32_t *d_sums, size_t n_rows, size_t n_cols, void *stream);
 

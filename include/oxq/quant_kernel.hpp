@@ -8,6 +8,8 @@
 //   QuantError       crates/oxillama-quant/src/error.rs:10-71
 //   KernelDispatcher crates/oxillama-quant/src/dispatch.rs:141-243
 //   quantize_f32_to_q8_0  crates/oxillama-quant/src/quantize.rs:58-75
+//   LoraAdapter      crates/oxillama-quant/src/lora.rs:21-124
+//   QuantLinear      crates/oxillama-arch/src/common/linear.rs:20-132
 // Results come back as QuantResult (Ok / Err(QuantError)); nothing throws.
 #ifndef OXQ_QUANT_KERNEL_HPP
 #define OXQ_QUANT_KERNEL_HPP
@@ -198,6 +200,77 @@ class KernelDispatcher {
 
   private:
     int init_status_;
+};
+
+// LoraAdapter (crates/oxillama-quant/src/lora.rs:21-124): delta = B (A input) * scale, A is
+// [rank x in_features], B is [out_features x rank], both row-major.
+struct LoraAdapter {
+    std::vector<float> a, b;
+    size_t rank = 0;
+    float scale = 0.0f;
+    size_t in_features = 0, out_features = 0;
+
+    // LoraAdapter::new (lora.rs:43-73): Err(DimensionMismatch) when a matrix has the wrong size.
+    static QuantResult create(std::vector<float> a, std::vector<float> b, size_t rank, float scale, size_t in_features,
+                              size_t out_features, std::shared_ptr<LoraAdapter> &out) {
+        auto mismatch = [](size_t expected, size_t got) {
+            QuantError e;
+            e.kind = QuantError::DimensionMismatch;
+            e.expected = expected;
+            e.got = got;
+            return QuantResult(std::move(e));
+        };
+        if (a.size() != rank * in_features) return mismatch(rank * in_features, a.size());
+        if (b.size() != out_features * rank) return mismatch(out_features * rank, b.size());
+        out = std::make_shared<LoraAdapter>();
+        out->a = std::move(a);
+        out->b = std::move(b);
+        out->rank = rank;
+        out->scale = scale;
+        out->in_features = in_features;
+        out->out_features = out_features;
+        return QuantResult();
+    }
+};
+
+// QuantLinear (crates/oxillama-arch/src/common/linear.rs:20-132).
+struct QuantLinear {
+    QuantTensor weight;
+    std::vector<float> bias;  // empty = none
+    bool has_bias = false;
+    size_t out_features = 0, in_features = 0;
+    std::shared_ptr<LoraAdapter> lora;
+
+    explicit QuantLinear(QuantTensor w) : weight(std::move(w)) { dims(); }
+    QuantLinear(QuantTensor w, std::vector<float> b) : weight(std::move(w)), bias(std::move(b)), has_bias(true) { dims(); }
+    void set_lora(std::shared_ptr<LoraAdapter> l) { lora = std::move(l); }
+    void clear_lora() { lora.reset(); }
+
+    // output = weight @ input + bias [+ lora delta] (linear.rs:77-98), one call across the ABI.
+    QuantResult forward(const QuantKernel &kernel, Slice<const float> input, Slice<float> output) const {
+        (void)kernel;  // the tensor's own type selects the GPU kernel, as get_kernel(weight.tensor_type) does
+        const LoraAdapter *l = lora.get();
+        return QuantResult::from_status(oxq_linear_forward(
+            static_cast<uint32_t>(weight.tensor_type), weight.data.data(), weight.data.size(), weight.shape.data(),
+            weight.shape.size(), has_bias ? bias.data() : nullptr, has_bias ? bias.size() : 0, l ? l->a.data() : nullptr,
+            l ? l->a.size() : 0, l ? l->b.data() : nullptr, l ? l->b.size() : 0, l ? l->rank : 0, l ? l->scale : 0.0f,
+            input.ptr, input.len, output.ptr, output.len));
+    }
+    // output[batch x out_features] = gemm + bias broadcast (linear.rs:105-132).
+    QuantResult forward_batch(const QuantKernel &kernel, Slice<const float> input, Slice<float> output,
+                              size_t batch_size) const {
+        (void)kernel;
+        return QuantResult::from_status(oxq_linear_forward_batch(
+            static_cast<uint32_t>(weight.tensor_type), weight.data.data(), weight.data.size(), weight.shape.data(),
+            weight.shape.size(), has_bias ? bias.data() : nullptr, has_bias ? bias.size() : 0, input.ptr, input.len,
+            output.ptr, output.len, batch_size));
+    }
+
+  private:
+    void dims() {  // linear.rs:38-48
+        out_features = weight.shape.empty() ? 0 : weight.shape[0];
+        in_features = weight.shape.size() < 2 ? 0 : weight.shape[1];
+    }
 };
 
 // quantize_f32_to_q8_0 (quantize.rs:58-75): Ok(Vec<u8>) of data.len()/32 * 34 bytes.

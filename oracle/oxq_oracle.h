@@ -118,6 +118,27 @@ oxq_ref_status oxq_ref_matvec_q8_fused_mt(uint32_t type, int tier, const uint8_t
                                           size_t out_len, size_t n_rows, size_t n_cols,
                                           int n_threads);
 
+/* ---- the callers' glue (oxq_oracle_linear.c) ---- */
+
+/* swiglu_inplace, crates/oxillama-arch/src/common/swiglu.rs:15-21 */
+void oxq_ref_swiglu_inplace(float *gate, const float *up, size_t n);
+/* RmsNorm::forward_to, crates/oxillama-arch/src/common/rms_norm.rs:49-66 */
+void oxq_ref_rmsnorm_forward_to(const float *input, const float *weight, float eps, size_t n,
+                                float *output);
+/* LoraAdapter::new / apply, crates/oxillama-quant/src/lora.rs:43-124 */
+oxq_ref_status oxq_ref_lora_new(size_t a_len, size_t b_len, size_t rank, size_t in_features,
+                                size_t out_features);
+oxq_ref_status oxq_ref_lora_apply(const float *a, const float *b, size_t rank, float scale,
+                                  size_t in_features, size_t out_features, const float *input,
+                                  size_t input_len, float *output, size_t output_len);
+/* QuantLinear::forward, crates/oxillama-arch/src/common/linear.rs:77-98, gemv on the
+ * Q8_0-activation path; bias / lora_a / lora_b may be NULL. */
+oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w, size_t w_len,
+                                      size_t n_rows, size_t n_cols, const float *bias, size_t bias_len,
+                                      const float *lora_a, const float *lora_b, size_t rank, float scale,
+                                      const float *input, size_t input_len, float *output,
+                                      size_t output_len);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,144 @@
+/*
+ * oxq_oracle_linear.c -- TEST INFRASTRUCTURE, NOT PRODUCT CODE.
+ *
+ * Scalar C restatement of the callers' glue around the quantized matvec in the reference
+ * (/root/reference): SwiGLU, RMSNorm, the LoRA correction and QuantLinear::forward.  Same
+ * rules as oxq_oracle.c: reference operation order, -ffp-contract=off -fno-fast-math.
+ *
+ * Pinning (tests/test_oracle_linear.py):
+ *   swiglu_inplace     the reference's own values (swiglu.rs:62-77) and a float64 closed form
+ *   rmsnorm_forward_to the reference's tests (rms_norm.rs:72-127) and a float64 closed form
+ *   lora_apply         the reference's hand-computed cases (lora.rs:141-200) and its error
+ *                      cases (lora.rs:229-259); float64 recomputation on random adapters
+ *   linear_forward     the reference's QuantLinear tests (linear.rs:161-270) replayed on Q8_0
+ *                      tensors with exactly representable weights
+ */
+#include <math.h>
+#include <stdlib.h>
+
+#include "oxq_oracle.h"
+
+static oxq_ref_status st(int code, size_t a, size_t b) {
+    oxq_ref_status s = {code, a, b};
+    return s;
+}
+
+/* swiglu_inplace, crates/oxillama-arch/src/common/swiglu.rs:15-21 */
+void oxq_ref_swiglu_inplace(float *gate, const float *up, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float g = gate[i];
+        float sigmoid = 1.0f / (1.0f + expf(-g)); /* :18 */
+        gate[i] = g * sigmoid * up[i];            /* :19, (g * sigmoid) * u */
+    }
+}
+
+/* RmsNorm::forward_to, crates/oxillama-arch/src/common/rms_norm.rs:49-66 */
+void oxq_ref_rmsnorm_forward_to(const float *input, const float *weight, float eps, size_t n,
+                                float *output) {
+    if (n == 0) {
+        return;
+    }
+    float sum_sq = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        sum_sq += input[i] * input[i]; /* :56-58, index order */
+    }
+    float rms = sqrtf(sum_sq / (float)n + eps); /* :59 */
+    float inv_rms = 1.0f / rms;                 /* :60 */
+    for (size_t i = 0; i < n; i++) {
+        output[i] = input[i] * inv_rms * weight[i]; /* :63 */
+    }
+}
+
+/* LoraAdapter::new, crates/oxillama-quant/src/lora.rs:43-73: size checks only */
+oxq_ref_status oxq_ref_lora_new(size_t a_len, size_t b_len, size_t rank, size_t in_features,
+                                size_t out_features) {
+    if (a_len != rank * in_features) {
+        return st(OXQ_REF_DIMENSION_MISMATCH, rank * in_features, a_len);
+    }
+    if (b_len != out_features * rank) {
+        return st(OXQ_REF_DIMENSION_MISMATCH, out_features * rank, b_len);
+    }
+    return st(OXQ_REF_OK, 0, 0);
+}
+
+/* LoraAdapter::apply, crates/oxillama-quant/src/lora.rs:83-124.  Both sums are Rust iterator
+ * sums: a left fold from 0.0 in index order. */
+oxq_ref_status oxq_ref_lora_apply(const float *a, const float *b, size_t rank, float scale,
+                                  size_t in_features, size_t out_features, const float *input,
+                                  size_t input_len, float *output, size_t output_len) {
+    if (input_len < in_features) {
+        return st(OXQ_REF_DIMENSION_MISMATCH, in_features, input_len);
+    }
+    if (output_len < out_features) {
+        return st(OXQ_REF_DIMENSION_MISMATCH, out_features, output_len);
+    }
+    float *r_vec = (float *)calloc(rank ? rank : 1, sizeof(float));
+    if (!r_vec) {
+        return st(OXQ_REF_INTERNAL, 0, 0);
+    }
+    for (size_t i = 0; i < rank; i++) {
+        const float *row = a + i * in_features;
+        float s = 0.0f;
+        for (size_t j = 0; j < in_features; j++) {
+            s += row[j] * input[j];
+        }
+        r_vec[i] = s;
+    }
+    for (size_t i = 0; i < out_features; i++) {
+        const float *row = b + i * rank;
+        float s = 0.0f;
+        for (size_t j = 0; j < rank; j++) {
+            s += row[j] * r_vec[j];
+        }
+        float delta = s * scale; /* :114-119 */
+        output[i] += delta;      /* :120 */
+    }
+    free(r_vec);
+    return st(OXQ_REF_OK, 0, 0);
+}
+
+/* QuantLinear::forward, crates/oxillama-arch/src/common/linear.rs:77-98, with `gemv` taken on
+ * the Q8_0-activation path this build accelerates (quantize the input, fused matvec into a
+ * zeroed output), then bias (zip: the shorter of the two lengths), then LoRA. */
+oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w, size_t w_len,
+                                      size_t n_rows, size_t n_cols, const float *bias, size_t bias_len,
+                                      const float *lora_a, const float *lora_b, size_t rank, float scale,
+                                      const float *input, size_t input_len, float *output,
+                                      size_t output_len) {
+    if (input_len < n_cols) {
+        return st(OXQ_REF_DIMENSION_MISMATCH, n_cols, input_len); /* gemv's checks, q4_k.rs:117-128 */
+    }
+    if (output_len < n_rows) {
+        return st(OXQ_REF_DIMENSION_MISMATCH, n_rows, output_len);
+    }
+    if (n_cols % 32 != 0) {
+        return st(OXQ_REF_KERNEL_ERROR, n_cols, 32);
+    }
+    size_t acts_len = n_cols / 32 * 34;
+    uint8_t *acts = (uint8_t *)malloc(acts_len ? acts_len : 1);
+    if (!acts) {
+        return st(OXQ_REF_INTERNAL, 0, 0);
+    }
+    oxq_ref_status s = oxq_ref_quantize_f32_to_q8_0(input, n_cols, acts);
+    if (s.code == OXQ_REF_OK) {
+        for (size_t r = 0; r < n_rows; r++) {
+            output[r] = 0.0f; /* gemv overwrites */
+        }
+        s = oxq_ref_matvec_q8_fused(type, tier, w, w_len, acts, acts_len, output, output_len, n_rows, n_cols);
+    }
+    free(acts);
+    if (s.code != OXQ_REF_OK) {
+        return s;
+    }
+    if (bias) {
+        size_t nb = bias_len < n_rows ? bias_len : n_rows; /* :87-89 */
+        for (size_t i = 0; i < nb; i++) {
+            output[i] += bias[i];
+        }
+    }
+    if (lora_a && lora_b && rank) {
+        return oxq_ref_lora_apply(lora_a, lora_b, rank, scale, n_cols, n_rows, input, input_len, output,
+                                  output_len); /* :93-95 */
+    }
+    return st(OXQ_REF_OK, 0, 0);
+}

@@ -87,6 +87,29 @@ SIGNATURES = {
     "oxq_moe_gemm_q8_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p,
                                       C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int,
                                       C.c_void_p, C.c_size_t, C.c_void_p]),
+    "oxq_lora_apply_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]),
+    "oxq_linear_forward_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                         C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p]),
+    "oxq_linear_forward_multi_dev": (C.c_int, [C.c_uint32, C.c_size_t, C.POINTER(C.c_void_p), C.c_void_p,
+                                               C.POINTER(C.c_void_p), C.POINTER(C.c_void_p),
+                                               C.POINTER(C.c_size_t), C.c_size_t, C.c_void_p]),
+    "oxq_linear_forward_batch_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                               C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t,
+                                               C.c_void_p]),
+    "oxq_linear_forward": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t), C.c_size_t,
+                                     C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                     C.c_size_t, C.c_float, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t]),
+    "oxq_linear_forward_batch": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.POINTER(C.c_size_t), C.c_size_t,
+                                           C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t,
+                                           C.c_size_t]),
+    "oxq_swiglu_quantize_q8_0_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p,
+                                               C.c_void_p]),
+    "oxq_rmsnorm_quantize_q8_0_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_float, C.c_size_t, C.c_size_t,
+                                                C.c_void_p, C.c_void_p, C.c_void_p]),
+    "oxq_ffn_workspace_bytes": (C.c_size_t, [C.c_size_t, C.c_size_t]),
+    "oxq_ffn_swiglu_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p,
+                                     C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t,
+                                     C.c_void_p]),
     "oxq_block_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                      C.c_size_t, C.c_void_p]),
     "oxq_set_gemv_waves_per_cu": (C.c_int, [C.c_uint]),

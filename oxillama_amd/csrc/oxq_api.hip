@@ -99,7 +99,7 @@ struct State {
     uint32_t waves_per_row = 0;   // 0 = chosen per shape
     bool cache_enabled = false;
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
-    Scratch s_weights, s_acts, s_x, s_out, s_sums, s_work;
+    Scratch s_weights, s_acts, s_x, s_out, s_sums, s_work, s_bias, s_lora_a, s_lora_b, s_lora_r;
 };
 State g;
 
@@ -264,6 +264,10 @@ int oxq_shutdown(void) {
     g.s_out.release();
     g.s_sums.release();
     g.s_work.release();
+    g.s_bias.release();
+    g.s_lora_a.release();
+    g.s_lora_b.release();
+    g.s_lora_r.release();
     g.initialised = false;
     g.device = -1;
     return OXQ_OK;
@@ -465,8 +469,9 @@ int oxq_block_sums(uint32_t type, const uint8_t *weights, size_t weights_len, co
     return OXQ_OK;
 }
 
-int oxq_gemm(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
-             const float *input, size_t input_len, float *output, size_t output_len, size_t m, size_t n, size_t k) {
+static int gemm_host(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
+                     const float *bias, size_t bias_len, const float *input, size_t input_len, float *output,
+                     size_t output_len, size_t m, size_t n, size_t k) {
     size_t n_rows = 0, n_cols = 0;
     int st = tensor_dims(type, data_len, shape, n_dims, &n_rows, &n_cols);
     if (st != OXQ_OK) return st;
@@ -511,10 +516,34 @@ int oxq_gemm(uint32_t type, const uint8_t *data, size_t data_len, const size_t *
     ga.n = (uint32_t)n_rows;
     ga.k = (uint32_t)n_cols;
     ga.accumulate = 0;
+    if (bias && bias_len) {
+        // the reference adds bias[j] for every j the bias holds (linear.rs:123-128)
+        if ((st = g.s_bias.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+        const size_t nb = bias_len < n_rows ? bias_len : n_rows;
+        OXQ_HIP(hipMemset(g.s_bias.ptr, 0, n_rows * sizeof(float)));
+        OXQ_HIP(hipMemcpy(g.s_bias.ptr, bias, nb * sizeof(float), hipMemcpyHostToDevice));
+        ga.bias = (const float *)g.s_bias.ptr;
+    }
     OXQ_HIP(oxq::launch_gemm_q8(type, ga, nullptr));
     OXQ_HIP(hipMemcpy2D(output, n * sizeof(float), g.s_out.ptr, n_rows * sizeof(float), n_rows * sizeof(float), m,
                         hipMemcpyDeviceToHost));
     return OXQ_OK;
+}
+
+int oxq_gemm(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
+             const float *input, size_t input_len, float *output, size_t output_len, size_t m, size_t n, size_t k) {
+    return gemm_host(type, data, data_len, shape, n_dims, nullptr, 0, input, input_len, output, output_len, m, n, k);
+}
+
+int oxq_linear_forward_batch(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
+                             const float *bias, size_t bias_len, const float *input, size_t input_len, float *output,
+                             size_t output_len, size_t batch) {
+    // QuantLinear::forward_batch: gemm with n = out_features = shape[0], k = in_features = shape[1]
+    // (linear.rs:112-119), then the bias broadcast over the batch.
+    const size_t out_features = (shape && n_dims > 0) ? shape[0] : 0;
+    const size_t in_features = (shape && n_dims > 1) ? shape[1] : 0;
+    return gemm_host(type, data, data_len, shape, n_dims, bias, bias_len, input, input_len, output, output_len, batch,
+                     out_features, in_features);
 }
 
 int oxq_gemv(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
@@ -661,8 +690,8 @@ size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k) 
 }
 
 static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, int32_t *d_sums,
-                    size_t m, size_t n, size_t k, int accumulate, void *d_workspace, size_t workspace_bytes,
-                    void *stream) {
+                    size_t m, size_t n, size_t k, int accumulate, const float *d_bias, void *d_workspace,
+                    size_t workspace_bytes, void *stream) {
     int st = check_dev_shape(type, n, k);
     if (st != OXQ_OK) return st;
     if (m > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, m, "dimension exceeds 2^32-1");
@@ -678,6 +707,7 @@ static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
     ga.n = (uint32_t)n;
     ga.k = (uint32_t)k;
     ga.accumulate = accumulate ? 1 : 0;
+    ga.bias = d_bias;
     const size_t need = oxq_gemm_q8_workspace_bytes(type, m, n, k);
     if (need && d_workspace) {
         if (workspace_bytes < need) return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, workspace_bytes, "workspace too small");
@@ -703,7 +733,8 @@ static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
 
 int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, size_t m,
                     size_t n, size_t k, int accumulate, void *d_workspace, size_t workspace_bytes, void *stream) {
-    return gemm_dev(type, d_weights, d_acts_q8, d_out, nullptr, m, n, k, accumulate, d_workspace, workspace_bytes, stream);
+    return gemm_dev(type, d_weights, d_acts_q8, d_out, nullptr, m, n, k, accumulate, nullptr, d_workspace, workspace_bytes,
+                    stream);
 }
 
 int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out,
@@ -712,7 +743,7 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
     if (!d_sums) return fail(OXQ_ERR_INTERNAL, 0, 0, "null sums");
     if (oxq_gemm_q8_workspace_bytes(type, m, n, k) == 0)
         return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, m, "no tile kernel for this type/shape");
-    return gemm_dev(type, d_weights, d_acts_q8, d_out, d_sums, m, n, k, 0, d_workspace, workspace_bytes, stream);
+    return gemm_dev(type, d_weights, d_acts_q8, d_out, d_sums, m, n, k, 0, nullptr, d_workspace, workspace_bytes, stream);
 }
 
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k) {
@@ -758,6 +789,204 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
                                                  : total_rows);
     ga.w_stride = expert_stride_bytes;
     OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+// ---- the callers' side: QuantLinear, SwiGLU feed-forward, RMSNorm ------------------------
+
+static int check_lora(const oxq_lora *lora) {
+    if (!lora || lora->rank == 0) return OXQ_OK;
+    if (!lora->d_a || !lora->d_b || !lora->d_r) return fail(OXQ_ERR_INTERNAL, 0, 0, "LoRA adapter with a null pointer");
+    if (lora->rank > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, lora->rank, "rank exceeds 2^32-1");
+    return OXQ_OK;
+}
+
+int oxq_lora_apply_dev(const oxq_lora *lora, const float *d_x, float *d_out, size_t out_features, size_t in_features,
+                       void *stream) {
+    int st = check_lora(lora);
+    if (st != OXQ_OK) return st;
+    if (!lora || lora->rank == 0) return OXQ_OK;
+    if (out_features > 0xFFFFFFFFull || in_features > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, out_features, "dimension exceeds 2^32-1");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_lora_apply(lora->d_a, lora->d_b, lora->d_r, (uint32_t)lora->rank, lora->scale, d_x, d_out,
+                                   (uint32_t)out_features, (uint32_t)in_features, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_linear_forward_dev(uint32_t type, const uint8_t *d_weights, const float *d_x, const uint8_t *d_acts_q8,
+                           const float *d_bias, const oxq_lora *lora, float *d_out, size_t out_features,
+                           size_t in_features, void *stream) {
+    int st = check_dev_shape(type, out_features, in_features);
+    if (st != OXQ_OK) return st;
+    if ((st = check_lora(lora)) != OXQ_OK) return st;
+    const bool has_lora = lora && lora->rank;
+    if (!d_acts_q8 && !d_x) return fail(OXQ_ERR_INTERNAL, 0, 0, "neither fp32 nor Q8_0 activations given");
+    if (has_lora && !d_x) return fail(OXQ_ERR_INTERNAL, 0, 0, "LoRA needs the fp32 input");
+    if (!d_acts_q8 && !oxq::gemv_takes_f32(type, (uint32_t)in_features))
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, in_features, "row too long for in-kernel activation quantization");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (out_features == 0 || in_features == 0) return OXQ_OK;
+    oxq::GemvArgs a = gemv_args(d_weights, d_acts_q8, d_out, nullptr, out_features, in_features, 0);
+    if (!d_acts_q8) a.X = d_x;
+    a.bias = d_bias;
+    OXQ_HIP(oxq::launch_gemv_q8(type, a, (hipStream_t)stream));
+    if (has_lora) return oxq_lora_apply_dev(lora, d_x, d_out, out_features, in_features, stream);
+    return OXQ_OK;
+}
+
+int oxq_linear_forward_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_weights,
+                                 const uint8_t *d_acts_q8, const float *const *d_biases, float *const *d_outs,
+                                 const size_t *out_features, size_t in_features, void *stream) {
+    if (n_mats == 0) return OXQ_OK;
+    if (n_mats > 4) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 4, n_mats, "at most 4 matrices per call");
+    if (!d_weights || !d_outs || !out_features) return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer table");
+    int st;
+    for (size_t i = 0; i < n_mats; i++) {
+        if ((st = check_dev_shape(type, out_features[i], in_features)) != OXQ_OK) return st;
+        if (out_features[i] == 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 1, 0, "a matrix of the call has no rows");
+    }
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (in_features == 0) return OXQ_OK;
+    oxq::GemvArgs a = gemv_args(d_weights[0], d_acts_q8, d_outs[0], nullptr, out_features[0], in_features, 0);
+    a.bias = d_biases ? d_biases[0] : nullptr;
+    a.n_mats = (uint32_t)n_mats;
+    for (size_t i = 1; i < n_mats; i++) {
+        a.W_more[i - 1] = d_weights[i];
+        a.out_more[i - 1] = d_outs[i];
+        a.bias_more[i - 1] = d_biases ? d_biases[i] : nullptr;
+        a.n_rows_more[i - 1] = (uint32_t)out_features[i];
+    }
+    OXQ_HIP(oxq::launch_gemv_q8(type, a, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_linear_forward_batch_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
+                                 const float *d_bias, float *d_out, size_t batch, size_t out_features,
+                                 size_t in_features, void *d_workspace, size_t workspace_bytes, void *stream) {
+    return gemm_dev(type, d_weights, d_acts_q8, d_out, nullptr, batch, out_features, in_features, 0, d_bias,
+                    d_workspace, workspace_bytes, stream);
+}
+
+int oxq_swiglu_quantize_q8_0_dev(const float *d_gate, const float *d_up, size_t n_total, float *d_h,
+                                 uint8_t *d_out_q8, void *stream) {
+    if (n_total % 32 != 0)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, (n_total / 32 + 1) * 32, n_total, "length is not a multiple of 32");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_swiglu_quantize(d_gate, d_up, n_total, d_h, d_out_q8, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_rmsnorm_quantize_q8_0_dev(const float *d_x, const float *d_weight, float eps, size_t rows, size_t n,
+                                  float *d_y, uint8_t *d_out_q8, void *stream) {
+    if (n % 32 != 0) return fail(OXQ_ERR_DIMENSION_MISMATCH, (n / 32 + 1) * 32, n, "row length is not a multiple of 32");
+    if (n > 0xFFFFFFFFull || rows > 0x7FFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n, "dimension exceeds the launch limits");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_rmsnorm_quantize(d_x, d_weight, eps, rows, (uint32_t)n, d_y, d_out_q8, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+size_t oxq_ffn_workspace_bytes(size_t hidden, size_t intermediate) {
+    (void)hidden;
+    // gate fp32 | up fp32 | Q8_0 blocks of silu(gate) * up, each piece 256-byte aligned
+    const size_t f = (intermediate * sizeof(float) + 255) & ~(size_t)255;
+    return 2 * f + ((intermediate / 32 * 34 + 255) & ~(size_t)255);
+}
+
+int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_type, const uint8_t *d_up,
+                       uint32_t down_type, const uint8_t *d_down, const uint8_t *d_acts_q8, float *d_out, size_t hidden,
+                       size_t intermediate, void *d_workspace, size_t workspace_bytes, void *stream) {
+    int st;
+    if ((st = check_dev_shape(gate_type, intermediate, hidden)) != OXQ_OK) return st;
+    if ((st = check_dev_shape(up_type, intermediate, hidden)) != OXQ_OK) return st;
+    if ((st = check_dev_shape(down_type, hidden, intermediate)) != OXQ_OK) return st;
+    if (intermediate % 32 != 0)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 32, intermediate, "intermediate size is not a multiple of 32");
+    const size_t need = oxq_ffn_workspace_bytes(hidden, intermediate);
+    if (!d_workspace || workspace_bytes < need)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, d_workspace ? workspace_bytes : 0, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
+        return fail(OXQ_ERR_KERNEL, 256, reinterpret_cast<uintptr_t>(d_workspace) & 255, "workspace must be 256-byte aligned");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (hidden == 0 || intermediate == 0) return OXQ_OK;
+    const size_t f = (intermediate * sizeof(float) + 255) & ~(size_t)255;
+    float *gate = (float *)d_workspace, *up = (float *)((uint8_t *)d_workspace + f);
+    uint8_t *hq = (uint8_t *)d_workspace + 2 * f;
+    hipStream_t s = (hipStream_t)stream;
+    if (gate_type == up_type) {  // one pass of the launch machinery over both matrices
+        oxq::GemvArgs a = gemv_args(d_gate, d_acts_q8, gate, nullptr, intermediate, hidden, 0);
+        a.n_mats = 2;
+        a.W_more[0] = d_up;
+        a.out_more[0] = up;
+        OXQ_HIP(oxq::launch_gemv_q8(gate_type, a, s));
+    } else {
+        OXQ_HIP(oxq::launch_gemv_q8(gate_type, gemv_args(d_gate, d_acts_q8, gate, nullptr, intermediate, hidden, 0), s));
+        OXQ_HIP(oxq::launch_gemv_q8(up_type, gemv_args(d_up, d_acts_q8, up, nullptr, intermediate, hidden, 0), s));
+    }
+    OXQ_HIP(oxq::launch_swiglu_quantize(gate, up, intermediate, nullptr, hq, s));
+    OXQ_HIP(oxq::launch_gemv_q8(down_type, gemv_args(d_down, hq, d_out, nullptr, hidden, intermediate, 0), s));
+    return OXQ_OK;
+}
+
+// QuantLinear::forward on host slices (drop-in route: everything is staged per call).
+int oxq_linear_forward(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
+                       const float *bias, size_t bias_len, const float *lora_a, size_t lora_a_len, const float *lora_b,
+                       size_t lora_b_len, size_t rank, float scale, const float *input, size_t input_len, float *output,
+                       size_t output_len) {
+    size_t n_rows = 0, n_cols = 0;
+    int st = tensor_dims(type, data_len, shape, n_dims, &n_rows, &n_cols);
+    if (st != OXQ_OK) return st;
+    // gemv's checks first (reference/q4_k.rs:117-128), then the adapter's (lora.rs:84-95)
+    if (input_len < n_cols) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_cols, input_len, "input shorter than n_cols");
+    if (output_len < n_rows) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_rows, output_len, "output shorter than n_rows");
+    const bool has_lora = lora_a && lora_b && rank;
+    if (has_lora) {
+        if (lora_a_len != rank * n_cols) return fail(OXQ_ERR_DIMENSION_MISMATCH, rank * n_cols, lora_a_len, "LoRA A has the wrong size");
+        if (lora_b_len != n_rows * rank) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_rows * rank, lora_b_len, "LoRA B has the wrong size");
+    }
+    const size_t bs = oxq_block_size(type), bb = oxq_block_bytes(type);
+    const size_t row_bytes = (n_cols + bs - 1) / bs * bb;
+    if (data_len < n_rows * row_bytes)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * row_bytes, data_len, "tensor data too small");
+    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
+    if (n_rows == 0 || n_cols == 0) return OXQ_OK;
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows, "dimension exceeds 2^32-1");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    std::lock_guard<std::mutex> lock(g.mu);
+    const uint8_t *dW = nullptr;
+    if ((st = stage_weights(type, data, n_rows * row_bytes, &dW)) != OXQ_OK) return st;
+    if ((st = g.s_x.reserve(n_cols * sizeof(float))) != OXQ_OK) return st;
+    if ((st = g.s_acts.reserve(n_cols / 32 * 34)) != OXQ_OK) return st;
+    if ((st = g.s_out.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+    OXQ_HIP(hipMemcpy(g.s_x.ptr, input, n_cols * sizeof(float), hipMemcpyHostToDevice));
+    OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, n_cols, (uint8_t *)g.s_acts.ptr, nullptr));
+    const float *d_bias = nullptr;
+    if (bias && bias_len) {
+        // the reference zips output with bias (linear.rs:87-89): a short bias covers its own length only
+        if ((st = g.s_bias.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+        const size_t nb = bias_len < n_rows ? bias_len : n_rows;
+        OXQ_HIP(hipMemset(g.s_bias.ptr, 0, n_rows * sizeof(float)));
+        OXQ_HIP(hipMemcpy(g.s_bias.ptr, bias, nb * sizeof(float), hipMemcpyHostToDevice));
+        d_bias = (const float *)g.s_bias.ptr;
+    }
+    oxq::GemvArgs a = gemv_args(dW, (const uint8_t *)g.s_acts.ptr, (float *)g.s_out.ptr, nullptr, n_rows, n_cols, 0);
+    a.bias = d_bias;
+    OXQ_HIP(oxq::launch_gemv_q8(type, a, nullptr));
+    if (has_lora) {
+        if ((st = g.s_lora_a.reserve(lora_a_len * sizeof(float))) != OXQ_OK) return st;
+        if ((st = g.s_lora_b.reserve(lora_b_len * sizeof(float))) != OXQ_OK) return st;
+        if ((st = g.s_lora_r.reserve(rank * sizeof(float))) != OXQ_OK) return st;
+        OXQ_HIP(hipMemcpy(g.s_lora_a.ptr, lora_a, lora_a_len * sizeof(float), hipMemcpyHostToDevice));
+        OXQ_HIP(hipMemcpy(g.s_lora_b.ptr, lora_b, lora_b_len * sizeof(float), hipMemcpyHostToDevice));
+        OXQ_HIP(oxq::launch_lora_apply((const float *)g.s_lora_a.ptr, (const float *)g.s_lora_b.ptr,
+                                       (float *)g.s_lora_r.ptr, (uint32_t)rank, scale, (const float *)g.s_x.ptr,
+                                       (float *)g.s_out.ptr, (uint32_t)n_rows, (uint32_t)n_cols, nullptr));
+    }
+    OXQ_HIP(hipMemcpy(output, g.s_out.ptr, n_rows * sizeof(float), hipMemcpyDeviceToHost));
     return OXQ_OK;
 }
 

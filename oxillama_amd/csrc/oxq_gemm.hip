@@ -350,7 +350,8 @@ template <class F, int MT, int NT, int WM, int DIST, bool DUMP, int ADIST>
 __device__ __forceinline__ void gemm_tile_body(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,
     const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m, uint32_t mpad,
-    uint32_t n, uint32_t k, int accumulate, uint32_t m_tiles, uint32_t n_tiles, const int32_t *__restrict__ offsets,
+    uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, uint32_t m_tiles, uint32_t n_tiles,
+    const int32_t *__restrict__ offsets,
     size_t w_stride) {
     constexpr bool SPLITK = WM == 0;  // the four waves share one tile and each walk a quarter of k
     constexpr int WMX = SPLITK ? 1 : WM, WN = SPLITK ? 1 : 4 / WMX;
@@ -616,7 +617,7 @@ __device__ __forceinline__ void gemm_tile_body(
                         const float y = (lds_red[0][tl][i][lane] + lds_red[1][tl][i][lane]) +
                                         (lds_red[2][tl][i][lane] + lds_red[3][tl][i][lane]);
                         float *o = out + (size_t)row * n + nrow[nt];
-                        *o = accumulate ? *o + y : y;
+                        *o = accumulate ? *o + y : bias ? y + bias[nrow[nt]] : y;
                     }
                 }
             }
@@ -630,7 +631,7 @@ __device__ __forceinline__ void gemm_tile_body(
                 const uint32_t row = m_wave + mt * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
                 if (row < row_end) {
                     float *o = out + (size_t)row * n + nrow[nt];
-                    *o = accumulate ? *o + acc[mt][nt][i] : acc[mt][nt][i];
+                    *o = accumulate ? *o + acc[mt][nt][i] : bias ? acc[mt][nt][i] + bias[nrow[nt]] : acc[mt][nt][i];
                 }
             }
         }
@@ -644,10 +645,10 @@ __device__ __forceinline__ void gemm_tile_body(
     __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(OCC, OCC))) void NAME(                      \
         const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,                \
         const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m,         \
-        uint32_t mpad, uint32_t n, uint32_t k, int accumulate, uint32_t m_tiles, uint32_t n_tiles,                  \
-        const int32_t *__restrict__ offsets, size_t w_stride) {                                                     \
+        uint32_t mpad, uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, uint32_t m_tiles,   \
+        uint32_t n_tiles, const int32_t *__restrict__ offsets, size_t w_stride) {                                   \
         gemm_tile_body<F, MT, NT, WM, DIST, DUMP, ADIST>(W, q8t, P, da16, out, sums, m, mpad, n, k, accumulate,     \
-                                                         m_tiles, n_tiles, offsets, w_stride);                      \
+                                                         bias, m_tiles, n_tiles, offsets, w_stride);                \
     }
 OXQ_TILE_KERNEL(gemm_tile_kernel, 2)
 OXQ_TILE_KERNEL(gemm_tile_kernel_occ3, 3)
@@ -672,6 +673,7 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
             v.n_rows = a.n;
             v.n_cols = a.k;
             v.accumulate = a.accumulate;
+            v.bias = a.bias;
             hipError_t e = launch_gemv_vecs(type, v, stream);
             if (e != hipSuccess) return e;
             r += v.n_vecs;
@@ -685,6 +687,7 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
         g.n_rows = a.n;
         g.n_cols = a.k;
         g.accumulate = a.accumulate;
+        g.bias = a.bias;
         g.waves_per_cu = 8;
         g.rows_per_batch = 0;
         g.waves_per_row = 0;
@@ -719,7 +722,7 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
         if (e != hipSuccess) return e;
     }
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a.W, p.q8t, p.P, p.da16, a.out, a.sums, a.m, p.mpad, a.n,
-                       a.k, a.accumulate, m_tiles, n_tiles, a.offsets, a.w_stride);
+                       a.k, a.accumulate, a.bias, m_tiles, n_tiles, a.offsets, a.w_stride);
     return hipGetLastError();
 }
 

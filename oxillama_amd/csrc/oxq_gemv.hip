@@ -22,13 +22,23 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     const uint32_t n_mats = a.n_mats ? a.n_mats : 1;
     const uint8_t *w[4];
     float *o[4];
+    const float *old[4];  // what a row's sum is added to: the output (accumulate), a bias, or nothing
+    uint32_t rows[4];
+    uint32_t max_rows = a.n_rows;
     for (uint32_t i = 0; i < 4; i++) {
-        w[i] = i > 0 && i < n_mats ? a.W_more[i - 1] : a.W;
-        o[i] = i > 0 && i < n_mats ? a.out_more[i - 1] : a.out;
+        const bool more = i > 0 && i < n_mats;
+        w[i] = more ? a.W_more[i - 1] : a.W;
+        o[i] = more ? a.out_more[i - 1] : a.out;
+        old[i] = a.accumulate ? o[i] : more ? a.bias_more[i - 1] : a.bias;
+        rows[i] = more && a.n_rows_more[i - 1] ? a.n_rows_more[i - 1] : a.n_rows;
+        if (rows[i] > max_rows) max_rows = rows[i];
     }
-    const uint32_t n_batches = (a.n_rows + RB - 1) / RB;
+    const uint32_t n_batches = (max_rows + RB - 1) / RB;
     // the launch width is shared by the matrices of the call
-    uint32_t max_groups = device_cus() * a.waves_per_cu / KS / n_mats;
+    uint64_t total_rows = 0;
+    for (uint32_t i = 0; i < n_mats; i++) total_rows += rows[i];
+    // each matrix gets gridDim.x work groups, sized so that the whole launch fills the chip once
+    uint32_t max_groups = (uint32_t)((uint64_t)(device_cus() * a.waves_per_cu / KS) * max_rows / (total_rows ? total_rows : 1));
     if (max_groups == 0) max_groups = 1;
     // Equal share per group: ceil(n_batches / passes) groups, each doing `passes` batches.
     const uint32_t passes = (n_batches + max_groups - 1) / max_groups;
@@ -39,8 +49,8 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     // fp32 source: LDS for the quantized vector (32 payload bytes + one f16 scale per block)
     const size_t lds = std::is_same<SRC, ActF32>::value ? (size_t)(a.n_cols / 32) * 34 : 0;
     hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), lds, stream, w[0],
-                       w[1], w[2], w[3], o[0], o[1], o[2], o[3], acts, a.sums, a.n_rows, units, groups_per_row,
-                       row_bytes, a.accumulate);
+                       w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums, rows[0],
+                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes);
     return hipGetLastError();
 }
 
@@ -107,10 +117,10 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     if (blocks == 0) blocks = 1;
     if (a.sums)
         hipLaunchKernelGGL((gemv_q8_generic<F, true>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.out, a.sums,
-                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate);
+                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias);
     else
         hipLaunchKernelGGL((gemv_q8_generic<F, false>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.out, a.sums,
-                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate);
+                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias);
     return hipGetLastError();
 }
 
@@ -132,7 +142,7 @@ static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t ro
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
     hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride, a.out,
-                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs);
+                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias);
     return hipGetLastError();
 }
 
@@ -204,6 +214,8 @@ hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream) 
                 if (i) {
                     s.W = a.W_more[i - 1];
                     s.out = a.out_more[i - 1];
+                    s.bias = a.bias_more[i - 1];
+                    if (a.n_rows_more[i - 1]) s.n_rows = a.n_rows_more[i - 1];
                 }
                 hipError_t e = launch_gemv_q8(type, s, stream);
                 if (e != hipSuccess) return e;

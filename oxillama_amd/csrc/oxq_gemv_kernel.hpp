@@ -25,12 +25,12 @@ struct Batch {
 
 template <class F, int STEPS, int RB>
 __device__ __forceinline__ void load_batch(Batch<F, STEPS, RB> &b, const uint8_t *__restrict__ W,
-                                           const float *__restrict__ out, uint32_t batch, uint32_t n_rows,
+                                           const float *__restrict__ old, uint32_t batch, uint32_t n_rows,
                                            size_t row_bytes, uint32_t units, uint32_t unit0, uint32_t lane,
                                            const typename F::Lane &k, bool want_old) {
     const uint32_t row0 = batch * RB;
     b.old = 0.0f;
-    if (want_old && lane < RB && row0 + lane < n_rows) b.old = out[row0 + lane];
+    if (want_old && lane < RB && row0 + lane < n_rows) b.old = old[row0 + lane];
 #pragma unroll
     for (int r = 0; r < RB; r++) {
         const uint32_t row = min(row0 + r, n_rows - 1);  // past the last row: re-read it, result unused
@@ -72,16 +72,22 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
                                                      const uint8_t *__restrict__ W2, const uint8_t *__restrict__ W3,
                                                      float *__restrict__ out0, float *__restrict__ out1,
                                                      float *__restrict__ out2, float *__restrict__ out3,
+                                                     const float *__restrict__ old0, const float *__restrict__ old1,
+                                                     const float *__restrict__ old2, const float *__restrict__ old3,
                                                      const void *__restrict__ A, int32_t *__restrict__ sums,
-                                                     uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
-                                                     size_t row_bytes, int accumulate) {
+                                                     uint32_t n_rows0, uint32_t n_rows1, uint32_t n_rows2,
+                                                     uint32_t n_rows3, uint32_t units, uint32_t groups_per_row,
+                                                     size_t row_bytes) {
     static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
-    // Up to four matrices of one shape and format that share the activation vector (wq/wk/wv,
+    // Up to four matrices of one format and row length that share the activation vector (wq/wk/wv,
     // ffn_gate/ffn_up) ride in one launch: blockIdx.y picks the matrix, and each matrix gets
-    // its own gridDim.x work groups.
+    // its own gridDim.x work groups (sized for the one with the most rows).  old = the vector a
+    // row's sum is added to (the output itself when accumulating, a bias vector), or null.
     const uint32_t mat = blockIdx.y;
     const uint8_t *__restrict__ W = mat == 0 ? W0 : mat == 1 ? W1 : mat == 2 ? W2 : W3;
     float *__restrict__ out = mat == 0 ? out0 : mat == 1 ? out1 : mat == 2 ? out2 : out3;
+    const float *__restrict__ old = mat == 0 ? old0 : mat == 1 ? old1 : mat == 2 ? old2 : old3;
+    const uint32_t n_rows = mat == 0 ? n_rows0 : mat == 1 ? n_rows1 : mat == 2 ? n_rows2 : n_rows3;
     constexpr uint32_t G = 4 / KS;  // row groups per work group
     __shared__ float part_sums[2][4][4];
     const uint32_t lane = threadIdx.x & 63;
@@ -95,7 +101,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
     // With KS > 1 every wave of the work group runs the same number of trips (barriers);
     // trips past the last batch re-read the last rows and store nothing.
     const uint32_t n_trips = KS == 1 ? n_batches : ((n_batches + n_groups - 1) / n_groups) * n_groups;
-    const bool want_old = accumulate && part == 0;
+    const bool want_old = old != nullptr && part == 0;
     constexpr bool F32 = std::is_same<SRC, ActF32>::value;
     Batch<F, STEPS, RB> b0, b1;
     typename F::Act act[STEPS];
@@ -110,7 +116,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
     if constexpr (F32) {
         // fp32 activations: request the first weights, then the work group quantizes the vector into
         // LDS once (every wave takes part in the barrier) and each wave picks up its slice.
-        load_batch<F, STEPS, RB>(b0, W, out, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k,
+        load_batch<F, STEPS, RB>(b0, W, old, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k,
                                  want_old);
         const uint32_t nb = units * (F::UNIT_COLS / 32);
         uint16_t *lds_d = reinterpret_cast<uint16_t *>(lds_acts + (size_t)nb * 8);
@@ -123,7 +129,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
         // Activations first (they sit in L2 and arrive early), then the first batch of
         // weights: the activation constants are derived while HBM is being read.
         load_acts(SRC::make(A));
-        load_batch<F, STEPS, RB>(b0, W, out, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k,
+        load_batch<F, STEPS, RB>(b0, W, old, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k,
                                  want_old);
     }
 
@@ -156,7 +162,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
             finish(r0, b0.old, batch);
             break;
         }
-        load_batch<F, STEPS, RB>(b1, W, out, min(next, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
+        load_batch<F, STEPS, RB>(b1, W, old, min(next, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
         const float r0 = reduce_batch<F, STEPS, RB, DUMP>(b0, act, sums, min(batch, n_batches - 1), n_rows, units, unit0,
                                                           groups_per_row, lane, k);
         finish(r0, b0.old, batch);
@@ -167,7 +173,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
             finish(r1, b1.old, next);
             break;
         }
-        load_batch<F, STEPS, RB>(b0, W, out, min(next2, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
+        load_batch<F, STEPS, RB>(b0, W, old, min(next2, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
         const float r1 = reduce_batch<F, STEPS, RB, DUMP>(b1, act, sums, min(next, n_batches - 1), n_rows, units, unit0,
                                                           groups_per_row, lane, k);
         finish(r1, b1.old, next);
@@ -183,7 +189,7 @@ template <class F, int STEPS, int KS, int NV>
 __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ W, const uint8_t *__restrict__ A,
                                                    size_t a_stride, float *__restrict__ out, size_t out_stride,
                                                    uint32_t n_rows, uint32_t units, size_t row_bytes,
-                                                   int accumulate, uint32_t n_vecs) {
+                                                   int accumulate, uint32_t n_vecs, const float *__restrict__ bias) {
     static_assert((KS == 1 || KS == 4) && NV >= 2 && NV <= 4, "configuration");
     // n_vecs <= NV: the surplus slots repeat the last vector (same loads, same stored values)
     constexpr uint32_t G = 4 / KS;
@@ -230,7 +236,7 @@ __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ 
         if (KS == 1) {
             if (lane < NV && row < n_rows) {
                 float *o = out + (size_t)min(lane, n_vecs - 1) * out_stride + row;
-                *o = accumulate ? *o + res : res;
+                *o = (accumulate ? *o : bias ? bias[row] : 0.0f) + res;
             }
         } else {
             if (lane < NV) part_sums[trip & 1][wave_in_wg][lane] = res;
@@ -240,7 +246,7 @@ __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ 
 #pragma unroll
                 for (int p = 1; p < KS; p++) t += part_sums[trip & 1][grp * KS + p][lane];
                 float *o = out + (size_t)min(lane, n_vecs - 1) * out_stride + row;
-                *o = accumulate ? *o + t : t;
+                *o = (accumulate ? *o : bias ? bias[row] : 0.0f) + t;
             }
             trip++;
         }
@@ -274,7 +280,7 @@ __global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict
                                                       const uint8_t *__restrict__ A,
                                                       float *__restrict__ out, int32_t *__restrict__ sums,
                                                       uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
-                                                      size_t row_bytes, int accumulate) {
+                                                      size_t row_bytes, const float *__restrict__ old) {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
     const uint32_t n_waves = (gridDim.x * blockDim.x) >> 6;
@@ -294,7 +300,7 @@ __global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict
             acc += F::template dot<DUMP>(w, a, k, DUMP ? sums + (size_t)row * groups_per_row : nullptr, u, valid);
         }
         const float total = wave_sum(acc);
-        if (lane == 0) out[row] = (accumulate ? out[row] : 0.0f) + total;
+        if (lane == 0) out[row] = (old ? old[row] : 0.0f) + total;
     }
 }
 

@@ -17,14 +17,17 @@ struct GemvArgs {
     uint32_t n_rows;
     uint32_t n_cols;      // multiple of the format's block size
     int accumulate;       // 1: out[r] += y (matvec_q8_fused), 0: out[r] = y (gemv)
+    const float *bias = nullptr;  // with accumulate == 0: out[r] = y + bias[r] (QuantLinear::forward)
     uint32_t waves_per_cu;  // launch width: resident waves per compute unit
     uint32_t rows_per_batch;  // rows a wave loads at once (1, 2 or 4); 0 = chosen from the row size
     uint32_t waves_per_row;   // 1 or 4 waves share a row; 0 = chosen from the row length
-    // Further matrices of the same shape and format sharing A (q/k/v, gate/up): n_mats - 1
-    // entries; each has n_rows rows and its own output vector.
+    // Further matrices of the same format and row length sharing A (q/k/v, gate/up): n_mats - 1
+    // entries, each with its own output vector, bias and row count (0 = n_rows).
     uint32_t n_mats = 1;
     const uint8_t *W_more[3] = {nullptr, nullptr, nullptr};
     float *out_more[3] = {nullptr, nullptr, nullptr};
+    const float *bias_more[3] = {nullptr, nullptr, nullptr};
+    uint32_t n_rows_more[3] = {0, 0, 0};
 };
 
 // Number of compute units of the current device (cached per device).
@@ -44,6 +47,7 @@ struct GemvVecsArgs {
     uint32_t n_vecs;     // 2, 3 or 4
     uint32_t n_rows, n_cols;
     int accumulate;
+    const float *bias = nullptr;  // with accumulate == 0: added to every vector's result
 };
 hipError_t launch_gemv_vecs(uint32_t type, const GemvVecsArgs &a, hipStream_t stream);
 // Most activation vectors one launch takes for rows of n_cols columns (4, 2, or 0: none).
@@ -51,6 +55,16 @@ uint32_t gemv_vecs_max(uint32_t type, uint32_t n_cols);
 
 // x: n floats (n % 32 == 0) -> n/32 Q8_0 blocks of 34 bytes.
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *out, hipStream_t stream);
+
+// h = silu(gate) * up over n floats (n % 32 == 0); h (fp32) and/or out (Q8_0 blocks) may be null.
+hipError_t launch_swiglu_quantize(const float *gate, const float *up, size_t n, float *h, uint8_t *out,
+                                  hipStream_t stream);
+// RMSNorm of `rows` rows of n floats (n % 32 == 0); y (fp32) and/or out (Q8_0 blocks) may be null.
+hipError_t launch_rmsnorm_quantize(const float *x, const float *weight, float eps, size_t rows, uint32_t n, float *y,
+                                   uint8_t *out, hipStream_t stream);
+// out += b (a x) * scale; r = rank floats of scratch.
+hipError_t launch_lora_apply(const float *a, const float *b, float *r, uint32_t rank, float scale, const float *x,
+                             float *out, uint32_t out_features, uint32_t in_features, hipStream_t stream);
 
 struct GemmArgs {
     const uint8_t *W;   // raw GGUF blocks [n x k]
@@ -60,6 +74,7 @@ struct GemmArgs {
     uint8_t *workspace; // gemm_workspace_bytes(m, k) bytes, 256-byte aligned; null: row-by-row matvecs
     uint32_t m, n, k;   // m = all token rows (of all experts in the grouped form)
     int accumulate;
+    const float *bias = nullptr;  // with accumulate == 0: out[t][r] = y + bias[r] (QuantLinear::forward_batch)
     // Grouped (mixture-of-experts) form: expert e multiplies token rows offsets[e] ..
     // offsets[e+1]-1 by the weights at W + e * w_stride.  offsets == null: plain matmul.
     const int32_t *offsets = nullptr;  // device memory, n_experts + 1 entries

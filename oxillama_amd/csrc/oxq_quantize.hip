@@ -9,6 +9,7 @@
 // (reference/{q4_0,q8_0,q4_k,q6_k,iq4_xs}.rs), same fp32 operation order.
 #include "oxq_device.hpp"
 #include "oxq_internal.hpp"
+#include "oxq_q8_encode.hpp"
 
 namespace oxq {
 
@@ -20,31 +21,8 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(const float *__restr
     const uint32_t j = (uint32_t)(t & 7);
     const bool valid = blk < n_blocks;
     float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (valid) {
-        const u32x4 raw = ld16(reinterpret_cast<const uint8_t *>(x + blk * 32 + 4 * j));
-        for (int i = 0; i < 4; i++) {
-            const uint32_t bits = raw[i];  // copy out first: bit_cast must not see the vector element lvalue
-            v[i] = __builtin_bit_cast(float, bits);
-        }
-    }
-    float m = 0.0f;
-    for (int i = 0; i < 4; i++) m = fmaxf(m, fabsf(v[i]));
-    m = fmaxf(m, dpp_f<0xB1>(m));
-    m = fmaxf(m, dpp_f<0x4E>(m));
-    m = fmaxf(m, __shfl_xor(m, 4, 64));  // max is exact: any order gives the fold of quantize.rs:194
-    const float d = m / 127.0f;                        // quantize.rs:197
-    const float id = (d != 0.0f) ? 1.0f / d : 0.0f;    // quantize.rs:198
-    uint32_t packed = 0;
-    for (int i = 0; i < 4; i++) {
-        int q = (int)roundf(v[i] * id);  // quantize.rs:206 (round half away from zero)
-        q = q < -128 ? -128 : (q > 127 ? 127 : q);
-        packed |= ((uint32_t)q & 0xFFu) << (8 * i);
-    }
-    if (valid) {
-        uint8_t *ob = out + blk * 34;
-        if (j == 0) st2(ob, f2h(d));  // quantize.rs:201
-        reinterpret_cast<PackedU1 *>(ob + 2 + 4 * j)->v = packed;
-    }
+    if (valid) load4(v, x + blk * 32 + 4 * j);
+    encode_q8_0_lanes(v, valid, out + blk * 34, j);
 }
 
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *out, hipStream_t stream) {

@@ -1,0 +1,143 @@
+"""Python mirror of the callers of the kernel trait, over liboxq_hip.so.
+
+  LoraAdapter      crates/oxillama-quant/src/lora.rs:21-124
+  QuantLinear      crates/oxillama-arch/src/common/linear.rs:20-132
+  swiglu / rmsnorm crates/oxillama-arch/src/common/swiglu.rs:15-21, rms_norm.rs:49-66
+  dense FFN        crates/oxillama-arch/src/llama/model.rs:277-310
+
+`QuantLinear.forward` crosses the C ABI with numpy host buffers (everything staged per call);
+the `*_dev` functions take torch CUDA tensors and enqueue on torch's current stream.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import capi
+from .quant import DimensionMismatch, HipKernel, QuantTensor, _check, _ptr, _u8
+
+
+class LoraAdapter:
+    """delta = B @ (A @ input) * scale; A is [rank x in_features], B is [out_features x rank]."""
+
+    def __init__(self, a, b, rank, scale, in_features, out_features):
+        a = np.ascontiguousarray(a, dtype=np.float32).ravel()
+        b = np.ascontiguousarray(b, dtype=np.float32).ravel()
+        if a.size != rank * in_features:  # lora.rs:51-57
+            raise DimensionMismatch(rank * in_features, a.size)
+        if b.size != out_features * rank:  # lora.rs:58-64
+            raise DimensionMismatch(out_features * rank, b.size)
+        self.a, self.b, self.rank, self.scale = a, b, rank, float(scale)
+        self.in_features, self.out_features = in_features, out_features
+
+
+class QuantLinear:
+    """weight: QuantTensor [out_features, in_features]; optional fp32 bias; optional LoRA."""
+
+    def __init__(self, weight: QuantTensor, bias=None):
+        self.weight = weight
+        self.bias = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32).ravel()
+        self.out_features = weight.shape[0] if len(weight.shape) > 0 else 0  # linear.rs:38-48
+        self.in_features = weight.shape[1] if len(weight.shape) > 1 else 0
+        self.lora = None
+
+    def set_lora(self, lora):
+        self.lora = lora
+
+    def clear_lora(self):
+        self.lora = None
+
+    def forward(self, kernel: HipKernel, input, output):
+        """output = weight @ input + bias [+ lora delta] (linear.rs:77-98); output is filled in place."""
+        lib = capi.load()
+        w = _u8(self.weight.data)
+        shape = (C.c_size_t * len(self.weight.shape))(*self.weight.shape)
+        x = np.ascontiguousarray(input, dtype=np.float32).ravel()
+        bias_p, bias_n = (_ptr(self.bias), self.bias.size) if self.bias is not None else (None, 0)
+        if self.lora is not None:
+            la, lb = self.lora.a, self.lora.b
+            lora_args = (_ptr(la), la.size, _ptr(lb), lb.size, self.lora.rank, self.lora.scale)
+        else:
+            lora_args = (None, 0, None, 0, 0, 0.0)
+        _check(lib.oxq_linear_forward(kernel.tensor_type, _ptr(w), w.size, shape, len(self.weight.shape), bias_p,
+                                      bias_n, *lora_args, _ptr(x), x.size, _ptr(output), output.size))
+
+    def forward_batch(self, kernel: HipKernel, input, output, batch_size):
+        """output[batch x out] = gemm + bias broadcast (linear.rs:105-132; no LoRA in batch mode)."""
+        lib = capi.load()
+        w = _u8(self.weight.data)
+        shape = (C.c_size_t * len(self.weight.shape))(*self.weight.shape)
+        x = np.ascontiguousarray(input, dtype=np.float32).ravel()
+        bias_p, bias_n = (_ptr(self.bias), self.bias.size) if self.bias is not None else (None, 0)
+        _check(lib.oxq_linear_forward_batch(kernel.tensor_type, _ptr(w), w.size, shape, len(self.weight.shape),
+                                            bias_p, bias_n, _ptr(x), x.size, _ptr(output), output.size, batch_size))
+
+
+# ---- device route -------------------------------------------------------------------------
+
+
+class LoraStruct(C.Structure):
+    _fields_ = [("d_a", C.c_void_p), ("d_b", C.c_void_p), ("d_r", C.c_void_p), ("rank", C.c_size_t),
+                ("scale", C.c_float)]
+
+
+def _stream():
+    return HipKernel._stream()
+
+
+def _opt(t):
+    return t.data_ptr() if t is not None else None
+
+
+def lora_struct(d_a, d_b, d_r, rank, scale):
+    return LoraStruct(d_a.data_ptr(), d_b.data_ptr(), d_r.data_ptr(), rank, scale)
+
+
+def lora_apply_dev(lora, d_x, d_out, out_features, in_features):
+    _check(capi.load().oxq_lora_apply_dev(C.byref(lora), d_x.data_ptr(), d_out.data_ptr(), out_features, in_features,
+                                          _stream()))
+
+
+def linear_forward_dev(tensor_type, d_weights, d_out, out_features, in_features, d_x=None, d_acts=None, d_bias=None,
+                       lora=None):
+    _check(capi.load().oxq_linear_forward_dev(int(tensor_type), d_weights.data_ptr(), _opt(d_x), _opt(d_acts),
+                                              _opt(d_bias), C.byref(lora) if lora is not None else None,
+                                              d_out.data_ptr(), out_features, in_features, _stream()))
+
+
+def linear_forward_multi_dev(tensor_type, d_weights, d_acts, d_outs, out_features, in_features, d_biases=None):
+    n = len(d_weights)
+    wp = (C.c_void_p * n)(*[w.data_ptr() for w in d_weights])
+    op = (C.c_void_p * n)(*[o.data_ptr() for o in d_outs])
+    bp = (C.c_void_p * n)(*[_opt(b) for b in d_biases]) if d_biases is not None else None
+    of = (C.c_size_t * n)(*out_features)
+    _check(capi.load().oxq_linear_forward_multi_dev(int(tensor_type), n, wp, d_acts.data_ptr(), bp, op, of,
+                                                    in_features, _stream()))
+
+
+def linear_forward_batch_dev(tensor_type, d_weights, d_acts, d_out, batch, out_features, in_features, d_bias=None,
+                             workspace=None):
+    _check(capi.load().oxq_linear_forward_batch_dev(int(tensor_type), d_weights.data_ptr(), d_acts.data_ptr(),
+                                                    _opt(d_bias), d_out.data_ptr(), batch, out_features, in_features,
+                                                    _opt(workspace), workspace.numel() if workspace is not None else 0,
+                                                    _stream()))
+
+
+def swiglu_quantize_dev(d_gate, d_up, d_h=None, d_out_q8=None):
+    _check(capi.load().oxq_swiglu_quantize_q8_0_dev(d_gate.data_ptr(), d_up.data_ptr(), d_gate.numel(), _opt(d_h),
+                                                    _opt(d_out_q8), _stream()))
+
+
+def rmsnorm_quantize_dev(d_x, d_weight, eps, rows, n, d_y=None, d_out_q8=None):
+    _check(capi.load().oxq_rmsnorm_quantize_q8_0_dev(d_x.data_ptr(), d_weight.data_ptr(), float(eps), rows, n,
+                                                     _opt(d_y), _opt(d_out_q8), _stream()))
+
+
+def ffn_workspace_bytes(hidden, intermediate):
+    return capi.load().oxq_ffn_workspace_bytes(hidden, intermediate)
+
+
+def ffn_swiglu_dev(gate, up, down, d_acts, d_out, hidden, intermediate, workspace):
+    """gate/up/down: (tensor_type, device weights).  d_out = down(silu(gate x) * up x)."""
+    _check(capi.load().oxq_ffn_swiglu_dev(int(gate[0]), gate[1].data_ptr(), int(up[0]), up[1].data_ptr(),
+                                          int(down[0]), down[1].data_ptr(), d_acts.data_ptr(), d_out.data_ptr(),
+                                          hidden, intermediate, workspace.data_ptr(), workspace.numel(), _stream()))

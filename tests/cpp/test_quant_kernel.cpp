@@ -218,6 +218,36 @@ static void host_tests() {
         CHECK(r.error().kind == QuantError::BufferTooSmall);
         CHECK(r.error().expected == 256 && r.error().got == 255);
     });
+
+    run("lora new: dimension mismatches (lora.rs:203-227)", [&] {
+        std::shared_ptr<LoraAdapter> l;
+        QuantResult r = LoraAdapter::create({1.0f}, {1.0f, 0.0f, 0.0f, 1.0f}, 2, 1.0f, 1, 2, l);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 2 && r.error().got == 1);
+        r = LoraAdapter::create({1.0f, 0.0f}, {1.0f}, 1, 1.0f, 2, 2, l);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 2 && r.error().got == 1);
+        CHECK(LoraAdapter::create({1, 0, 0, 1}, {1, 0, 0, 1}, 2, 1.0f, 2, 2, l).is_ok() && l && l->rank == 2);
+    });
+
+    run("quant linear: new has no lora; short input / output are dimension errors (linear.rs:265-270, q4_k.rs:117-128)", [&] {
+        std::vector<uint8_t> w;
+        for (int r = 0; r < 32; ++r) {
+            std::vector<int> q(32, 0);
+            q[r] = 1;
+            append(w, q8_0_block(1.0f, q));
+        }
+        QuantLinear lin(QuantTensor(w, {32, 32}, GgufTensorType::Q8_0));
+        CHECK(!lin.lora && lin.out_features == 32 && lin.in_features == 32);
+        HipKernel k(GgufTensorType::Q8_0);
+        std::vector<float> x(31, 0.0f), y(32, 0.0f);
+        QuantResult r = lin.forward(k, x, y);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch && r.error().expected == 32 && r.error().got == 31);
+        x.resize(32);
+        y.resize(31);
+        r = lin.forward(k, x, y);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch && r.error().expected == 32 && r.error().got == 31);
+    });
 }
 
 // ======================================================================================
@@ -420,6 +450,112 @@ static void gpu_tests() {
         CHECK(quantize_f32_to_q8_0(x, a).is_ok());
         CHECK(k->matvec_q8_fused(w, a, z, 3, 256).is_ok());
         for (int r = 0; r < 3; ++r) CHECK(y[r] == z[r]);
+    });
+
+    // QuantLinear tests of crates/oxillama-arch/src/common/linear.rs:161-270.  The reference runs them on
+    // an F32 tensor; here the weight is the same matrix as Q8_0 blocks (d = 1, q in {0, 1, 2, 3}: exact) and
+    // the inputs have one magnitude per block, so the activation quantization only adds the f16 rounding of
+    // its scale (tolerance 2e-3 instead of 1e-5).
+    auto diag_q8 = [&](const std::vector<int> &diag) {
+        std::vector<uint8_t> w;
+        for (size_t r = 0; r < 32; ++r) {
+            std::vector<int> q(32, 0);
+            if (r < diag.size()) q[r] = diag[r];
+            append(w, q8_0_block(1.0f, q));
+        }
+        return QuantTensor(w, {32, 32}, GgufTensorType::Q8_0);
+    };
+    auto eye32 = [] {
+        std::vector<float> m(32 * 32, 0.0f);
+        for (int i = 0; i < 32; ++i) m[i * 32 + i] = 1.0f;
+        return m;
+    };
+
+    run("linear forward_no_lora (linear.rs:161-177)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        QuantLinear lin(diag_q8({2, 3}));  // [[2, 0], [0, 3]]
+        std::vector<float> x(32, 0.0f), y(32, -1.0f);
+        x[0] = 4.0f;
+        x[1] = -4.0f;  // one magnitude per block: q = +-127
+        CHECK(lin.forward(*k, x, y).is_ok());
+        CHECK_NEAR(y[0], 8.0, 8e-3);
+        CHECK_NEAR(y[1], -12.0, 12e-3);
+        CHECK(y[2] == 0.0f);
+    });
+
+    run("linear forward_with_lora_identity (linear.rs:184-204)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        QuantLinear lin(diag_q8(std::vector<int>(32, 1)));  // identity
+        std::shared_ptr<LoraAdapter> l;
+        CHECK(LoraAdapter::create(eye32(), eye32(), 32, 1.0f, 32, 32, l).is_ok());
+        lin.set_lora(l);
+        std::vector<float> x(32, 0.0f), y(32, 0.0f);
+        x[0] = 2.0f;
+        x[1] = -2.0f;
+        CHECK(lin.forward(*k, x, y).is_ok());
+        CHECK_NEAR(y[0], 4.0, 4e-3);  // W x + delta = x + x
+        CHECK_NEAR(y[1], -4.0, 4e-3);
+    });
+
+    run("linear clear_lora (linear.rs:207-233)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        QuantLinear lin(diag_q8(std::vector<int>(32, 1)));
+        std::shared_ptr<LoraAdapter> l;
+        CHECK(LoraAdapter::create(eye32(), eye32(), 32, 1.0f, 32, 32, l).is_ok());
+        lin.set_lora(l);
+        lin.clear_lora();
+        std::vector<float> x(32, 0.0f), y(32, 0.0f);
+        x[0] = 7.0f;
+        x[1] = -7.0f;
+        CHECK(lin.forward(*k, x, y).is_ok());
+        CHECK_NEAR(y[0], 7.0, 7e-3);
+        CHECK_NEAR(y[1], -7.0, 7e-3);
+    });
+
+    run("linear lora_applied_after_bias (linear.rs:236-262)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        QuantLinear lin(diag_q8(std::vector<int>(32, 1)), std::vector<float>(32, 10.0f));
+        std::shared_ptr<LoraAdapter> l;
+        CHECK(LoraAdapter::create(eye32(), eye32(), 32, 1.0f, 32, 32, l).is_ok());
+        lin.set_lora(l);
+        std::vector<float> x(32, 0.0f), y(32, 0.0f);
+        x[0] = 3.0f;
+        x[1] = -3.0f;
+        CHECK(lin.forward(*k, x, y).is_ok());
+        CHECK_NEAR(y[0], 3.0 + 10.0 + 3.0, 6e-3);
+        CHECK_NEAR(y[1], -3.0 + 10.0 - 3.0, 6e-3);
+        CHECK(y[5] == 10.0f);
+    });
+
+    run("lora apply: scale and accumulation onto the base output (lora.rs:141-200)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        // base output = bias (weights all zero), delta = B (A x) * scale
+        QuantLinear lin(diag_q8({}), std::vector<float>(32, 10.0f));
+        std::vector<float> a(32, 0.0f), b(32, 0.0f);  // rank 1: A = e0^T, B = e0
+        a[0] = 1.0f;
+        b[0] = 1.0f;
+        std::shared_ptr<LoraAdapter> l;
+        CHECK(LoraAdapter::create(a, b, 1, 0.5f, 32, 32, l).is_ok());
+        lin.set_lora(l);
+        std::vector<float> x(32, 0.0f), y(32, 0.0f);
+        x[0] = 4.0f;
+        CHECK(lin.forward(*k, x, y).is_ok());
+        CHECK_NEAR(y[0], 12.0, 1e-6);  // 10 + 1 * (1 * 4) * 0.5
+        CHECK(y[1] == 10.0f);
+    });
+
+    run("linear forward_batch: gemm + bias broadcast (linear.rs:105-132)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        std::vector<float> bias(32);
+        for (int i = 0; i < 32; ++i) bias[i] = (float)i;
+        QuantLinear lin(diag_q8(std::vector<int>(32, 2)), bias);
+        std::vector<float> x(3 * 32, 0.0f), y(3 * 32, -1.0f);
+        for (int r = 0; r < 3; ++r) x[r * 32 + r] = (float)(r + 1);
+        CHECK(lin.forward_batch(*k, x, y, 3).is_ok());
+        for (int r = 0; r < 3; ++r) {
+            CHECK_NEAR(y[r * 32 + r], 2.0 * (r + 1) + r, 8e-3);
+            CHECK(y[r * 32 + 31] == 31.0f);
+        }
     });
 }
 

@@ -104,10 +104,17 @@ def load():
         "oxq_ref_block_sums": [u32, vp, sz, vp, sz, vp, sz, sz],
         "oxq_ref_gemm_q8": [u32, C.c_int, vp, sz, vp, vp, sz, sz, sz],
         "oxq_ref_matvec_q8_fused_mt": [u32, C.c_int, vp, sz, vp, sz, vp, sz, sz, sz, C.c_int],
+        "oxq_ref_lora_new": [sz, sz, sz, sz, sz],
+        "oxq_ref_lora_apply": [vp, vp, sz, C.c_float, sz, sz, vp, sz, vp, sz],
+        "oxq_ref_linear_forward": [u32, C.c_int, vp, sz, sz, sz, vp, sz, vp, vp, sz, C.c_float, vp, sz, vp, sz],
     }.items():
         fn = getattr(lib, name)
         fn.restype = Status
         fn.argtypes = args
+    lib.oxq_ref_swiglu_inplace.restype = None
+    lib.oxq_ref_swiglu_inplace.argtypes = [vp, vp, sz]
+    lib.oxq_ref_rmsnorm_forward_to.restype = None
+    lib.oxq_ref_rmsnorm_forward_to.argtypes = [vp, vp, C.c_float, sz, vp]
     _lib = lib
     return lib
 
@@ -271,3 +278,57 @@ def make_iq4_xs_block(scale, sub_scales, nibbles):  # Q/reference/iq4_xs.rs:211-
         scales_l[i // 2] |= low if i % 2 == 0 else (low << 4)
         scales_h |= high << (2 * i)
     return f16_bytes(scale) + bytes([scales_h & 0xFF, scales_h >> 8]) + bytes(scales_l) + bytes(nibbles)
+
+
+# ---- the callers' glue (oracle/oxq_oracle_linear.c) ----
+
+def swiglu(gate, up):
+    """silu(gate) * up as swiglu_inplace computes it; returns a new array."""
+    g = np.array(gate, dtype=np.float32).ravel().copy()
+    u = np.ascontiguousarray(up, dtype=np.float32).ravel()
+    assert g.size == u.size
+    load().oxq_ref_swiglu_inplace(_p(g), _p(u), g.size)
+    return g
+
+
+def rmsnorm(x, weight, eps):
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    w = np.ascontiguousarray(weight, dtype=np.float32).ravel()
+    out = np.zeros(x.size, dtype=np.float32)
+    load().oxq_ref_rmsnorm_forward_to(_p(x), _p(w), float(eps), x.size, _p(out))
+    return out
+
+
+def lora_new(a_len, b_len, rank, in_features, out_features):
+    _chk(load().oxq_ref_lora_new(a_len, b_len, rank, in_features, out_features))
+
+
+def lora_apply(a, b, rank, scale, in_features, out_features, x, out):
+    """out += b (a x) * scale in place (LoraAdapter::apply); out is a float32 array."""
+    a = np.ascontiguousarray(a, dtype=np.float32).ravel()
+    b = np.ascontiguousarray(b, dtype=np.float32).ravel()
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    assert out.dtype == np.float32 and out.flags.c_contiguous
+    _chk(load().oxq_ref_lora_apply(_p(a), _p(b), rank, float(scale), in_features, out_features, _p(x), x.size,
+                                   _p(out), out.size))
+    return out
+
+
+def linear_forward(t, w, n_rows, n_cols, x, bias=None, lora=None, tier=TIER_AVX2, out_len=None):
+    """QuantLinear::forward on the Q8_0-activation path; lora = (a, b, rank, scale) or None."""
+    w = _u8(w)
+    x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.full(n_rows if out_len is None else out_len, np.float32(7.0), dtype=np.float32)  # overwritten
+    bp, bl = (None, 0)
+    if bias is not None:
+        bias = np.ascontiguousarray(bias, dtype=np.float32).ravel()
+        bp, bl = _p(bias), bias.size
+    ap = bq = None
+    rank, scale = 0, 0.0
+    if lora is not None:
+        la = np.ascontiguousarray(lora[0], dtype=np.float32).ravel()
+        lb = np.ascontiguousarray(lora[1], dtype=np.float32).ravel()
+        ap, bq, rank, scale = _p(la), _p(lb), int(lora[2]), float(lora[3])
+    _chk(load().oxq_ref_linear_forward(t, tier, _p(w), w.size, n_rows, n_cols, bp, bl, ap, bq, rank, scale, _p(x),
+                                       x.size, _p(out), out.size))
+    return out

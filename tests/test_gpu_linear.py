@@ -1,0 +1,345 @@
+"""Parity of the callers' side of the HIP library (QuantLinear::forward / forward_batch, LoRA,
+SwiGLU + quantize, RMSNorm + quantize, the dense feed-forward block, several projections of
+different heights in one launch) against the CPU oracle, through the C ABI.
+
+Bars: Q8_0 bytes bit-exact given the same fp32 values; matvec results bit-identical between the
+fused entry points and the plain ones; fp32 within 1e-5 * |y_ref|_inf of the oracle (SwiGLU's
+exp and RMSNorm's tree sum differ from libm / index order in the last place)."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from oxillama_amd import linear as L
+from oxillama_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+FP32_REL_TOL = 1e-5
+DEV = "cuda:0"
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def assert_close(y, y_ref, what, tol=FP32_REL_TOL):
+    scale = float(np.abs(y_ref).max())
+    err = float(np.abs(y.astype(np.float64) - y_ref.astype(np.float64)).max())
+    assert err <= tol * scale + 1e-30, f"{what}: max err {err:.3e} > {tol} * {scale:.3e}"
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def q8_identity(n, scale=1.0):
+    rows = []
+    for r in range(n):
+        for b in range(n // 32):
+            qs = [0] * 32
+            if r // 32 == b:
+                qs[r % 32] = 1
+            rows.append(O.make_q8_0_block(scale, qs))
+    return np.frombuffer(b"".join(rows), dtype=np.uint8)
+
+
+# ---- SwiGLU + quantize -----------------------------------------------------------------------
+
+def test_swiglu_quantize(hip, ref):
+    for seed, n in ((1, 14336), (2, 32), (3, 64 * 14336)):
+        say("swiglu seed", seed, "n", n)
+        g = synth.normal_f32(seed, n, 3.0)
+        u = synth.normal_f32(seed + 100, n, 1.0)
+        g[:6] = [0.0, -0.0, 88.0, -88.0, -100.0, -1000.0]
+        d_h = torch.empty(n, dtype=torch.float32, device=DEV)
+        d_q = torch.empty(n // 32 * 34, dtype=torch.uint8, device=DEV)
+        L.swiglu_quantize_dev(dev(g), dev(u), d_h, d_q)
+        h, q = host(d_h), host(d_q)
+        want = ref.swiglu(g, u)
+        assert np.all(np.isfinite(h))
+        # elementwise: a few ulp from expf
+        assert np.all(np.abs(h - want) <= 4e-7 * np.abs(want) + 1e-37), "swiglu fp32"
+        # the bytes are the quantizer's bytes for the values the kernel itself produced
+        assert np.array_equal(q, ref.quantize_q8_0(h))
+        # each output alone gives the same result
+        d_q2 = torch.empty_like(d_q)
+        L.swiglu_quantize_dev(dev(g), dev(u), None, d_q2)
+        assert np.array_equal(host(d_q2), q)
+
+
+def test_swiglu_reference_values(hip):
+    # crates/oxillama-arch/src/common/swiglu.rs:62-77, padded to one block
+    g = np.zeros(32, dtype=np.float32); g[:3] = [1.0, -1.0, 0.0]
+    u = np.zeros(32, dtype=np.float32); u[:3] = [2.0, 3.0, 4.0]
+    d_h = torch.empty(32, dtype=torch.float32, device=DEV)
+    L.swiglu_quantize_dev(dev(g), dev(u), d_h, None)
+    h = host(d_h)
+    assert abs(h[0] - 1.4621) < 0.01 and abs(h[2]) < 1e-6
+
+
+def test_swiglu_rejects_ragged_length(hip):
+    g = torch.zeros(33, dtype=torch.float32, device=DEV)
+    with pytest.raises(hip.DimensionMismatch) as e:
+        L.swiglu_quantize_dev(g, g, g, None)
+    assert (e.value.expected, e.value.got) == (64, 33)
+
+
+# ---- RMSNorm + quantize ----------------------------------------------------------------------
+
+def test_rmsnorm_quantize(hip, ref):
+    for seed, rows, n in ((1, 1, 4096), (2, 5, 4096), (3, 3, 14336), (4, 2, 32), (5, 512, 4096)):
+        say("rmsnorm seed", seed, rows, "x", n)
+        x = synth.normal_f32(seed, rows * n, 2.0)
+        w = (1.0 + 0.1 * synth.normal_f32(seed + 50, n, 1.0)).astype(np.float32)
+        d_y = torch.empty(rows * n, dtype=torch.float32, device=DEV)
+        d_q = torch.empty(rows * n // 32 * 34, dtype=torch.uint8, device=DEV)
+        L.rmsnorm_quantize_dev(dev(x), dev(w), 1e-5, rows, n, d_y, d_q)
+        y, q = host(d_y), host(d_q)
+        want = np.concatenate([ref.rmsnorm(x[r * n:(r + 1) * n], w, 1e-5) for r in range(rows)])
+        assert_close(y, want, f"rmsnorm {rows}x{n}", tol=2e-6)
+        assert np.array_equal(q, ref.quantize_q8_0(y))
+        d_q2 = torch.empty_like(d_q)
+        L.rmsnorm_quantize_dev(dev(x), dev(w), 1e-5, rows, n, None, d_q2)
+        assert np.array_equal(host(d_q2), q)
+
+
+def test_rmsnorm_reference_values(hip):
+    # crates/oxillama-arch/src/common/rms_norm.rs:72-88, padded with zeros to 32 (same sum of squares,
+    # mean over 32 instead of 4)
+    x = np.zeros(32, dtype=np.float32); x[:4] = [1, 2, 3, 4]
+    d_y = torch.empty(32, dtype=torch.float32, device=DEV)
+    L.rmsnorm_quantize_dev(dev(x), dev(np.ones(32, dtype=np.float32)), 1e-5, 1, 32, d_y, None)
+    y = host(d_y)
+    rms = np.sqrt(np.float32(30.0) / np.float32(32.0) + np.float32(1e-5))
+    assert np.all(np.abs(y[:4] - x[:4] / rms) < 1e-5) and np.all(y[4:] == 0)
+    # all-zero row: zeros, not NaN
+    L.rmsnorm_quantize_dev(dev(np.zeros(32, dtype=np.float32)), dev(np.ones(32, dtype=np.float32)), 1e-5, 1, 32, d_y,
+                           None)
+    assert np.all(host(d_y) == 0.0)
+
+
+# ---- LoRA ------------------------------------------------------------------------------------
+
+def test_lora_apply(hip, ref):
+    for seed, rank, n_in, n_out in ((1, 16, 4096, 4096), (2, 4, 4096, 14336), (3, 64, 14336, 4096), (4, 1, 32, 8)):
+        say("lora seed", seed, rank, n_in, n_out)
+        a = synth.normal_f32(seed, rank * n_in, 0.05)
+        b = synth.normal_f32(seed + 10, n_out * rank, 0.05)
+        x = synth.normal_f32(seed + 20, n_in, 1.0)
+        base = synth.normal_f32(seed + 30, n_out, 1.0)
+        d_out = dev(base)
+        d_r = torch.empty(rank, dtype=torch.float32, device=DEV)
+        d_a, d_b = dev(a), dev(b)
+        lora = L.lora_struct(d_a, d_b, d_r, rank, 0.25)
+        L.lora_apply_dev(lora, dev(x), d_out, n_out, n_in)
+        want = base.copy()
+        ref.lora_apply(a, b, rank, 0.25, n_in, n_out, x, want)
+        assert_close(host(d_out), want, "lora")
+        # the up-projection is in the reference's order: exact given the kernel's own r
+        r = host(d_r)
+        exact = base.copy()
+        s = np.zeros(n_out, dtype=np.float32)
+        bm = b.reshape(n_out, rank)
+        for j in range(rank):
+            s = (s + (bm[:, j] * r[j]).astype(np.float32)).astype(np.float32)
+        exact = (exact + (s * np.float32(0.25)).astype(np.float32)).astype(np.float32)
+        assert np.array_equal(host(d_out), exact)
+
+
+# ---- QuantLinear::forward --------------------------------------------------------------------
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_linear_forward_dev(hip, ref, t):
+    for seed, n_rows, n_cols in ((1, 96, 512), (2, 4096, 4096), (3, 1024, 14336)):
+        say("linear", O.NAMES[t], n_rows, n_cols)
+        w = synth.weights(t, seed, n_rows, n_cols)
+        x = synth.normal_f32(seed + 1, n_cols)
+        bias = synth.normal_f32(seed + 2, n_rows)
+        rank = 8
+        a = synth.normal_f32(seed + 3, rank * n_cols, 0.05)
+        b = synth.normal_f32(seed + 4, n_rows * rank, 0.05)
+        d_w, d_x, d_bias = dev(w), dev(x), dev(bias)
+        d_acts = torch.empty(n_cols // 32 * 34, dtype=torch.uint8, device=DEV)
+        hip.quantize_q8_0_dev(d_x, d_acts)
+        k = hip.HipKernel(t)
+        plain = torch.zeros(n_rows, dtype=torch.float32, device=DEV)
+        k.matvec_q8_fused_dev(d_w, d_acts, plain, n_rows, n_cols, accumulate=False)
+        y0 = host(plain)
+        # no bias, no LoRA: the plain matvec, bit for bit (linear.rs:161-177)
+        d_out = torch.full((n_rows,), 7.0, dtype=torch.float32, device=DEV)
+        L.linear_forward_dev(t, d_w, d_out, n_rows, n_cols, d_acts=d_acts)
+        assert np.array_equal(host(d_out), y0)
+        # bias in the epilogue == matvec, then + bias
+        L.linear_forward_dev(t, d_w, d_out, n_rows, n_cols, d_acts=d_acts, d_bias=d_bias)
+        assert np.array_equal(host(d_out), (y0 + bias).astype(np.float32))
+        # in-kernel quantization of x gives the same
+        if n_cols <= 46080:  # the quantized vector is staged in LDS
+            L.linear_forward_dev(t, d_w, d_out, n_rows, n_cols, d_x=d_x, d_bias=d_bias)
+            assert np.array_equal(host(d_out), (y0 + bias).astype(np.float32))
+        # bias, then LoRA, against the oracle (linear.rs:236-262)
+        d_r = torch.empty(rank, dtype=torch.float32, device=DEV)
+        d_a, d_b = dev(a), dev(b)
+        lora = L.lora_struct(d_a, d_b, d_r, rank, 0.5)
+        L.linear_forward_dev(t, d_w, d_out, n_rows, n_cols, d_x=d_x, d_acts=d_acts, d_bias=d_bias, lora=lora)
+        want = ref.linear_forward(t, w, n_rows, n_cols, x, bias=bias, lora=(a, b, rank, 0.5))
+        assert_close(host(d_out), want, "linear forward")
+
+
+def test_linear_forward_host_reference_cases(hip, ref):
+    """The QuantLinear tests of linear.rs:161-270 on a Q8_0 identity, through the host-slice route."""
+    n = 32
+    w = q8_identity(n)
+    lin = L.QuantLinear(hip.QuantTensor(w, [n, n], O.Q8_0))
+    assert lin.lora is None and (lin.out_features, lin.in_features) == (n, n)  # linear.rs:265-270
+    k = hip.HipKernel(O.Q8_0)
+    x = np.zeros(n, dtype=np.float32); x[3], x[7] = 2.0, -2.0
+    out = np.zeros(n, dtype=np.float32)
+    lin.forward(k, x, out)
+    assert np.array_equal(out, ref.linear_forward(O.Q8_0, w, n, n, x))
+    assert abs(out[3] - 2.0) < 2e-3 and abs(out[7] + 2.0) < 2e-3
+    eye = np.eye(n, dtype=np.float32)
+    lin.set_lora(L.LoraAdapter(eye, eye, n, 1.0, n, n))
+    lin.bias = np.full(n, 10.0, dtype=np.float32)
+    lin.forward(k, x, out)  # linear.rs:236-262: W x + bias + delta
+    assert abs(out[3] - 14.0) < 2e-3 and abs(out[7] - 6.0) < 2e-3 and out[0] == 10.0
+    assert_close(out, ref.linear_forward(O.Q8_0, w, n, n, x, bias=lin.bias, lora=(eye, eye, n, 1.0)), "host lora")
+    lin.clear_lora()  # linear.rs:207-233
+    lin.bias = None
+    lin.forward(k, x, out)
+    assert np.array_equal(out, ref.linear_forward(O.Q8_0, w, n, n, x))
+    # a short bias covers its own length (zip semantics)
+    lin.bias = np.full(4, 10.0, dtype=np.float32)
+    lin.forward(k, x, out)
+    assert np.array_equal(out, ref.linear_forward(O.Q8_0, w, n, n, x, bias=lin.bias))
+    # errors: gemv's checks, then the adapter's
+    with pytest.raises(hip.DimensionMismatch) as e:
+        lin.forward(k, x[:31], out)
+    assert (e.value.expected, e.value.got) == (32, 31)
+    with pytest.raises(hip.DimensionMismatch) as e:
+        lin.forward(k, x, out[:31])
+    assert (e.value.expected, e.value.got) == (32, 31)
+    with pytest.raises(hip.DimensionMismatch):
+        L.LoraAdapter([1.0], [1, 0, 0, 1], 2, 1.0, 1, 2)  # lora.rs:203-214
+
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_linear_forward_batch(hip, ref, t):
+    n, kk = 512, 1024
+    w = synth.weights(t, 9, n, kk)
+    bias = synth.normal_f32(10, n)
+    k = hip.HipKernel(t)
+    lin = L.QuantLinear(hip.QuantTensor(w, [n, kk], t), bias)
+    for m in (1, 3, 40):  # single GEMV, several vectors per pass, tile kernel
+        say("forward_batch", O.NAMES[t], m)
+        x = synth.normal_f32(11 + m, m * kk)
+        out = np.zeros(m * n, dtype=np.float32)
+        lin.forward_batch(k, x, out, m)
+        plain = np.zeros(m * n, dtype=np.float32)
+        k.gemm(lin.weight, x, plain, m, n, kk)
+        assert np.array_equal(out, (plain.reshape(m, n) + bias[None, :]).astype(np.float32).ravel())
+        want = ref.gemm_q8(t, w, x, m, n, kk).reshape(m, n) + bias[None, :]
+        assert_close(out, want.astype(np.float32).ravel(), "forward_batch")
+        # device route with a caller workspace
+        d_x = dev(x)
+        d_acts = torch.empty(m * (kk // 32 * 34), dtype=torch.uint8, device=DEV)
+        hip.quantize_q8_0_dev(d_x, d_acts)
+        ws_bytes = k.gemm_workspace_bytes(m, n, kk)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=DEV)
+        d_out = torch.empty(m * n, dtype=torch.float32, device=DEV)
+        L.linear_forward_batch_dev(t, dev(w), d_acts, d_out, m, n, kk, d_bias=dev(bias),
+                                   workspace=ws if ws_bytes else None)
+        assert np.array_equal(host(d_out), out)
+
+
+# ---- several projections of different heights in one launch ------------------------------------
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_linear_forward_multi_unequal_rows(hip, ref, t):
+    for n_cols, heights in ((4096, (4096, 1024, 1024)), (512, (96, 8, 40, 2)), (14336, (256, 4096))):
+        say("multi", O.NAMES[t], n_cols, heights)
+        x = synth.normal_f32(3, n_cols)
+        d_x = dev(x)
+        d_acts = torch.empty(n_cols // 32 * 34, dtype=torch.uint8, device=DEV)
+        hip.quantize_q8_0_dev(d_x, d_acts)
+        ws_, bs_, outs, singles = [], [], [], []
+        k = hip.HipKernel(t)
+        for i, h in enumerate(heights):
+            w = dev(synth.weights(t, 20 + i, h, n_cols))
+            b = dev(synth.normal_f32(30 + i, h)) if i != 1 else None
+            ws_.append(w); bs_.append(b)
+            outs.append(torch.full((h + 3,), -5.0, dtype=torch.float32, device=DEV))  # 3 guard floats
+            one = torch.empty(h, dtype=torch.float32, device=DEV)
+            L.linear_forward_dev(t, w, one, h, n_cols, d_acts=d_acts, d_bias=b)
+            singles.append(host(one))
+        L.linear_forward_multi_dev(t, ws_, d_acts, outs, heights, n_cols, d_biases=bs_)
+        for i, h in enumerate(heights):
+            got = host(outs[i])
+            assert np.array_equal(got[:h], singles[i]), f"matrix {i}"
+            assert np.all(got[h:] == -5.0), "wrote past the matrix's rows"
+        # and against the oracle
+        w0 = host(ws_[0])
+        want = ref.linear_forward(t, w0, heights[0], n_cols, x, bias=host(bs_[0]))
+        assert_close(host(outs[0])[:heights[0]], want, "multi vs oracle")
+
+
+# ---- the dense feed-forward block ---------------------------------------------------------------
+
+@pytest.mark.parametrize("types", [(O.Q4_K, O.Q4_K, O.Q6_K), (O.Q4_0, O.Q4_0, O.Q4_0), (O.Q8_0, O.Q4_K, O.IQ4_XS)],
+                         ids=["q4k_q4k_q6k", "q4_0", "mixed"])
+def test_ffn_swiglu(hip, ref, types):
+    for hidden, inter in ((512, 1024), (4096, 14336)):
+        say("ffn", types, hidden, inter)
+        tg, tu, td = types
+        wg, wu = synth.weights(tg, 1, inter, hidden), synth.weights(tu, 2, inter, hidden)
+        wd = synth.weights(td, 3, hidden, inter)
+        x = synth.normal_f32(4, hidden)
+        d_acts = torch.empty(hidden // 32 * 34, dtype=torch.uint8, device=DEV)
+        hip.quantize_q8_0_dev(dev(x), d_acts)
+        ws = torch.empty(L.ffn_workspace_bytes(hidden, inter), dtype=torch.uint8, device=DEV)
+        d_out = torch.empty(hidden, dtype=torch.float32, device=DEV)
+        d_wg, d_wu, d_wd = dev(wg), dev(wu), dev(wd)
+        L.ffn_swiglu_dev((tg, d_wg), (tu, d_wu), (td, d_wd), d_acts, d_out, hidden, inter, ws)
+        got = host(d_out)
+        # step by step with the plain entry points: bit-identical
+        g = torch.empty(inter, dtype=torch.float32, device=DEV)
+        u = torch.empty(inter, dtype=torch.float32, device=DEV)
+        hip.HipKernel(tg).matvec_q8_fused_dev(d_wg, d_acts, g, inter, hidden, accumulate=False)
+        hip.HipKernel(tu).matvec_q8_fused_dev(d_wu, d_acts, u, inter, hidden, accumulate=False)
+        hq = torch.empty(inter // 32 * 34, dtype=torch.uint8, device=DEV)
+        L.swiglu_quantize_dev(g, u, None, hq)
+        step = torch.empty(hidden, dtype=torch.float32, device=DEV)
+        hip.HipKernel(td).matvec_q8_fused_dev(d_wd, hq, step, hidden, inter, accumulate=False)
+        assert np.array_equal(got, host(step))
+        # against the oracle end to end: gate/up within 1e-5, then the oracle's SwiGLU and down on
+        # the oracle's own h; Q8_0 re-quantization of h amplifies last-place differences of gate/up,
+        # so the end-to-end bar is the quantization step of h (1/127 of a block's range) carried
+        # through down -- checked instead on the GPU's own h, which isolates each stage exactly.
+        acts = host(d_acts)
+        g_ref = ref.matvec_q8_fused_mt(tg, wg, acts, inter, hidden, 8)
+        u_ref = ref.matvec_q8_fused_mt(tu, wu, acts, inter, hidden, 8)
+        assert_close(host(g), g_ref, "gate")
+        assert_close(host(u), u_ref, "up")
+        h_gpu = ref.swiglu(host(g), host(u))
+        hq_ref = ref.quantize_q8_0(h_gpu)
+        same = np.mean(host(hq) == hq_ref)
+        assert same > 0.999, f"only {same:.5f} of the h bytes match the oracle's SwiGLU of the same gate/up"
+        down_ref = ref.matvec_q8_fused_mt(td, wd, host(hq), hidden, inter, 8)
+        assert_close(got, down_ref, "down")
+
+
+def test_ffn_swiglu_errors(hip):
+    z = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+    with pytest.raises(hip.BufferTooSmall) as e:
+        L.ffn_swiglu_dev((O.Q4_K, z), (O.Q4_K, z), (O.Q6_K, z), z, z, 256, 512, z[:64])
+    assert e.value.needed == L.ffn_workspace_bytes(256, 512)
+    with pytest.raises(hip.UnsupportedShape):
+        L.ffn_swiglu_dev((O.Q4_K, z), (O.Q4_K, z), (O.Q6_K, z), z, z, 100, 512, z)
