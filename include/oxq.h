@@ -36,6 +36,15 @@ extern "C" {
 #define OXQ_TYPE_Q4_K 12u
 #define OXQ_TYPE_Q6_K 14u
 #define OXQ_TYPE_IQ4_XS 23u
+/* GEMV, dequant_block and the batched form by rows (no int8-MFMA tile kernel yet): */
+#define OXQ_TYPE_Q4_1 3u
+#define OXQ_TYPE_Q5_0 6u
+#define OXQ_TYPE_Q5_1 7u
+#define OXQ_TYPE_Q8_1 9u
+#define OXQ_TYPE_Q2_K 10u
+#define OXQ_TYPE_Q3_K 11u
+#define OXQ_TYPE_Q5_K 13u
+#define OXQ_TYPE_IQ4_NL 20u
 
 /* Status codes: 1..7 are the QuantError variants of Q/error.rs:10-71 in order;
  * the (expected, got) / (needed, available) pair of the failing check is kept per

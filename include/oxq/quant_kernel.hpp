@@ -38,7 +38,10 @@ struct Slice {
 };
 
 // GgufTensorType discriminants (crates/oxillama-gguf/src/types.rs:72-150).
-enum class GgufTensorType : uint32_t { Q4_0 = 2, Q8_0 = 8, Q4K = 12, Q6K = 14, Iq4Xs = 23 };
+enum class GgufTensorType : uint32_t {
+    Q4_0 = 2, Q4_1 = 3, Q5_0 = 6, Q5_1 = 7, Q8_0 = 8, Q8_1 = 9, Q2K = 10, Q3K = 11, Q4K = 12, Q5K = 13, Q6K = 14,
+    Iq4Nl = 20, Iq4Xs = 23
+};
 
 struct QuantError {
     enum Kind {

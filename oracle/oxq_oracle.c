@@ -5,6 +5,7 @@
  * order.  Q/ = /root/reference/crates/oxillama-quant/src.
  */
 #include "oxq_oracle.h"
+#include "oxq_oracle_more.h"
 
 #include <math.h>
 #include <stdlib.h>
@@ -32,7 +33,7 @@ size_t oxq_ref_block_size(uint32_t type) {
     case OXQ_REF_IQ4_XS:
         return 256;
     default:
-        return 0;
+        return oxq_more_block_size(type);
     }
 }
 
@@ -50,7 +51,7 @@ size_t oxq_ref_block_bytes(uint32_t type) {
     case OXQ_REF_IQ4_XS:
         return 136;
     default:
-        return 0;
+        return oxq_more_block_bytes(type);
     }
 }
 
@@ -352,6 +353,9 @@ static void dequant_any(uint32_t type, const uint8_t *block, float *out) {
     case OXQ_REF_IQ4_XS:
         dequant_iq4_xs(block, out);
         break;
+    default:
+        oxq_more_dequant(type, block, out);
+        break;
     }
 }
 
@@ -513,6 +517,9 @@ static float gemv_row_iq4_xs(const uint8_t *row, size_t bpr, size_t n_cols, cons
 
 static float gemv_row(uint32_t type, const uint8_t *row, size_t bpr, size_t n_cols,
                       const float *x) {
+    if (oxq_more_known(type)) {
+        return oxq_more_gemv_row(type, row, bpr, n_cols, x);
+    }
     switch (type) {
     case OXQ_REF_Q4_0:
         return gemv_row_q4_0(row, bpr, n_cols, x);
@@ -839,6 +846,10 @@ static float fused_row_q6_k(const uint8_t *row, size_t bpr, size_t n_cols, const
 
 static void block_sums_row(uint32_t type, const uint8_t *row, size_t bpr, const uint8_t *acts,
                            int32_t *sums) {
+    if (oxq_more_known(type)) {
+        oxq_more_block_sums_row(type, row, bpr, acts, sums);
+        return;
+    }
     switch (type) {
     case OXQ_REF_Q4_0:
         for (size_t blk = 0; blk < bpr; blk++) {
@@ -918,6 +929,9 @@ static void block_sums_row(uint32_t type, const uint8_t *row, size_t bpr, const 
 }
 
 static size_t groups_per_block(uint32_t type) {
+    if (oxq_more_known(type)) {
+        return oxq_more_groups_per_block(type);
+    }
     switch (type) {
     case OXQ_REF_Q6_K:
         return 16;
@@ -939,6 +953,9 @@ static size_t groups_per_block(uint32_t type) {
  */
 static float intdot_row(uint32_t type, const uint8_t *row, size_t bpr, size_t n_cols,
                         const uint8_t *acts, int32_t *scratch) {
+    if (oxq_more_known(type)) {
+        return oxq_more_intdot_row(type, row, bpr, acts, scratch);
+    }
     switch (type) {
     case OXQ_REF_Q4_0:
         return fused_row_q4_0_avx2(row, bpr, n_cols, acts);
@@ -1004,6 +1021,9 @@ static oxq_ref_status fused_validate(uint32_t type, size_t w_len, size_t acts_le
 
 static float fused_row(uint32_t type, int tier, const uint8_t *row, size_t bpr, size_t n_cols,
                        const uint8_t *acts, int32_t *scratch) {
+    if (oxq_more_known(type)) { /* one tier: the *Ref kernels of Q/reference */
+        return oxq_more_fused_row(type, row, bpr, n_cols, acts);
+    }
     switch (type) {
     case OXQ_REF_Q4_0:
         if (tier == OXQ_REF_TIER_AVX2) return fused_row_q4_0_avx2(row, bpr, n_cols, acts);
@@ -1055,8 +1075,9 @@ oxq_ref_status oxq_ref_matvec_q8_intdot(uint32_t type, const uint8_t *w, size_t 
     if (s.code != OXQ_REF_OK) {
         return s;
     }
-    if ((type == OXQ_REF_IQ4_XS || type == OXQ_REF_Q6_K) && n_cols % 256 != 0) {
-        return err(OXQ_REF_KERNEL_ERROR, n_cols, 256);
+    if ((type == OXQ_REF_IQ4_XS || type == OXQ_REF_Q6_K || oxq_more_known(type)) &&
+        n_cols % oxq_ref_block_size(type) != 0) {
+        return err(OXQ_REF_KERNEL_ERROR, n_cols, oxq_ref_block_size(type));
     }
     size_t row_bytes = bpr * oxq_ref_block_bytes(type);
     int32_t *scratch = (int32_t *)malloc(sizeof(int32_t) * (bpr * 16 + 16));

@@ -41,7 +41,16 @@ enum {
     OXQ_REF_Q8_0 = 8,
     OXQ_REF_Q4_K = 12,
     OXQ_REF_Q6_K = 14,
-    OXQ_REF_IQ4_XS = 23
+    OXQ_REF_IQ4_XS = 23,
+    /* restated in oxq_oracle_more.c */
+    OXQ_REF_Q4_1 = 3,
+    OXQ_REF_Q5_0 = 6,
+    OXQ_REF_Q5_1 = 7,
+    OXQ_REF_Q8_1 = 9,
+    OXQ_REF_Q2_K = 10,
+    OXQ_REF_Q3_K = 11,
+    OXQ_REF_Q5_K = 13,
+    OXQ_REF_IQ4_NL = 20
 };
 
 /* QuantError variants, Q/error.rs:10-71 */

@@ -13,7 +13,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-HIP_SOURCES = ["oxq_api.hip", "oxq_gemv.hip", "oxq_gemm.hip", "oxq_quantize.hip", "oxq_linear.hip"]
+HIP_SOURCES = ["oxq_api.hip", "oxq_gemv.hip", "oxq_gemv_more.hip", "oxq_gemm.hip", "oxq_quantize.hip", "oxq_linear.hip"]
 HIP_LIB = os.path.join(HERE, "liboxq_hip.so")
 SYNTH_LIB = os.path.join(HERE, "liboxq_synth.so")
 BENCHKIT_LIB = os.path.join(HERE, "liboxq_benchkit.so")
@@ -35,11 +35,11 @@ def run(cmd):
 
 def build_hip(extra=()):
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    objs = []
-    for src in HIP_SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-        run([hipcc, *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj])
-        objs.append(obj)
+    from concurrent.futures import ThreadPoolExecutor
+    objs = [os.path.join(CSRC, src.replace(".hip", ".o")) for src in HIP_SOURCES]
+    with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES), 6)) as pool:  # one hipcc per translation unit
+        list(pool.map(lambda so: run([hipcc, *HIPCC_FLAGS, *extra, "-c", os.path.join(CSRC, so[0]), "-o", so[1]]),
+                      zip(HIP_SOURCES, objs)))
     run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB, *objs])
     return HIP_LIB
 

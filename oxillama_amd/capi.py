@@ -21,6 +21,8 @@ ERR_UNSUPPORTED_SHAPE = 8
 ERR_NO_DEVICE = 9
 
 TYPE_Q4_0, TYPE_Q8_0, TYPE_Q4_K, TYPE_Q6_K, TYPE_IQ4_XS = 2, 8, 12, 14, 23
+TYPE_Q4_1, TYPE_Q5_0, TYPE_Q5_1, TYPE_Q8_1, TYPE_Q2_K, TYPE_Q3_K, TYPE_Q5_K, TYPE_IQ4_NL = 3, 6, 7, 9, 10, 11, 13, 20
+GROUPS_OF_16 = (TYPE_Q6_K, TYPE_Q2_K, TYPE_Q3_K)  # formats whose exact integer sums cover 16 weights
 
 # Every symbol include/oxq.h declares, with its signature.
 _u8p = C.POINTER(C.c_uint8)

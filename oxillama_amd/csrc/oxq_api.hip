@@ -317,10 +317,18 @@ const char *oxq_status_name(int status) {
 size_t oxq_block_size(uint32_t type) {
     switch (type) {
     case OXQ_TYPE_Q4_0:
-    case OXQ_TYPE_Q8_0: return 32;
+    case OXQ_TYPE_Q8_0:
+    case OXQ_TYPE_Q4_1:
+    case OXQ_TYPE_Q5_0:
+    case OXQ_TYPE_Q5_1:
+    case OXQ_TYPE_Q8_1:
+    case OXQ_TYPE_IQ4_NL: return 32;
     case OXQ_TYPE_Q4_K:
     case OXQ_TYPE_Q6_K:
-    case OXQ_TYPE_IQ4_XS: return 256;
+    case OXQ_TYPE_IQ4_XS:
+    case OXQ_TYPE_Q2_K:
+    case OXQ_TYPE_Q3_K:
+    case OXQ_TYPE_Q5_K: return 256;
     default: return 0;
     }
 }
@@ -332,6 +340,14 @@ size_t oxq_block_bytes(uint32_t type) {
     case OXQ_TYPE_Q4_K: return 144;
     case OXQ_TYPE_Q6_K: return 210;
     case OXQ_TYPE_IQ4_XS: return 136;
+    case OXQ_TYPE_Q4_1: return 20;
+    case OXQ_TYPE_Q5_0: return 22;
+    case OXQ_TYPE_Q5_1: return 24;
+    case OXQ_TYPE_Q8_1: return 36;
+    case OXQ_TYPE_IQ4_NL: return 18;
+    case OXQ_TYPE_Q2_K: return 84;
+    case OXQ_TYPE_Q3_K: return 110;
+    case OXQ_TYPE_Q5_K: return 176;
     default: return 0;
     }
 }
@@ -343,6 +359,14 @@ const char *oxq_type_name(uint32_t type) {
     case OXQ_TYPE_Q4_K: return "Q4_K";
     case OXQ_TYPE_Q6_K: return "Q6_K";
     case OXQ_TYPE_IQ4_XS: return "IQ4_XS";
+    case OXQ_TYPE_Q4_1: return "Q4_1";
+    case OXQ_TYPE_Q5_0: return "Q5_0";
+    case OXQ_TYPE_Q5_1: return "Q5_1";
+    case OXQ_TYPE_Q8_1: return "Q8_1";
+    case OXQ_TYPE_IQ4_NL: return "IQ4_NL";
+    case OXQ_TYPE_Q2_K: return "Q2_K";
+    case OXQ_TYPE_Q3_K: return "Q3_K";
+    case OXQ_TYPE_Q5_K: return "Q5_K";
     default: return nullptr;
     }
 }
@@ -452,7 +476,7 @@ int oxq_block_sums(uint32_t type, const uint8_t *weights, size_t weights_len, co
     FusedShape fs;
     int st = validate_fused(type, weights_len, acts_len, n_rows, n_rows, n_cols, &fs);
     if (st != OXQ_OK) return st;
-    const size_t groups = n_cols / (type == OXQ_TYPE_Q6_K ? 16 : 32);
+    const size_t groups = n_cols / oxq::gemv_group_cols(type);
     if (sums_len < n_rows * groups) return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * groups, sums_len, "sums buffer too small");
     if (n_rows == 0 || n_cols == 0) return OXQ_OK;
     if ((st = ensure_init()) != OXQ_OK) return st;

@@ -1,0 +1,181 @@
+// Launch policy of the GEMV kernels, as templates over the format policy: shared by the
+// translation units that instantiate them for their formats.
+#pragma once
+#include "oxq_gemv_kernel.hpp"
+#include "oxq_internal.hpp"
+
+namespace oxq {
+
+template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP>
+static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
+                                hipStream_t stream) {
+    constexpr uint32_t G = 4 / KS;  // row groups per work group
+    const uint32_t n_mats = a.n_mats ? a.n_mats : 1;
+    const uint8_t *w[4];
+    float *o[4];
+    const float *old[4];  // what a row's sum is added to: the output (accumulate), a bias, or nothing
+    uint32_t rows[4];
+    uint32_t max_rows = a.n_rows;
+    for (uint32_t i = 0; i < 4; i++) {
+        const bool more = i > 0 && i < n_mats;
+        w[i] = more ? a.W_more[i - 1] : a.W;
+        o[i] = more ? a.out_more[i - 1] : a.out;
+        old[i] = a.accumulate ? o[i] : more ? a.bias_more[i - 1] : a.bias;
+        rows[i] = more && a.n_rows_more[i - 1] ? a.n_rows_more[i - 1] : a.n_rows;
+        if (rows[i] > max_rows) max_rows = rows[i];
+    }
+    const uint32_t n_batches = (max_rows + RB - 1) / RB;
+    // the launch width is shared by the matrices of the call
+    uint64_t total_rows = 0;
+    for (uint32_t i = 0; i < n_mats; i++) total_rows += rows[i];
+    // each matrix gets gridDim.x work groups, sized so that the whole launch fills the chip once
+    uint32_t max_groups = (uint32_t)((uint64_t)(device_cus() * a.waves_per_cu / KS) * max_rows / (total_rows ? total_rows : 1));
+    if (max_groups == 0) max_groups = 1;
+    // Equal share per group: ceil(n_batches / passes) groups, each doing `passes` batches.
+    const uint32_t passes = (n_batches + max_groups - 1) / max_groups;
+    const uint32_t groups = (n_batches + passes - 1) / passes;
+    uint32_t blocks = (groups + G - 1) / G;
+    if (blocks == 0) blocks = 1;
+    const void *acts = a.X ? static_cast<const void *>(a.X) : static_cast<const void *>(a.A);
+    // fp32 source: LDS for the quantized vector (32 payload bytes + one f16 scale per block)
+    const size_t lds = std::is_same<SRC, ActF32>::value ? (size_t)(a.n_cols / 32) * 34 : 0;
+    hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), lds, stream, w[0],
+                       w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums, rows[0],
+                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes);
+    return hipGetLastError();
+}
+
+// a.X set: fp32 activations, quantized to Q8_0 in registers by every wave (no dump variant).
+template <class F, int STEPS, int RB, int KS, bool DUMP>
+static hipError_t launch_cached(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
+                                hipStream_t stream) {
+    if constexpr (!DUMP) {
+        if (a.X) return launch_cached_src<F, ActF32, STEPS, RB, KS, false>(a, units, groups_per_row, row_bytes, stream);
+    }
+    return launch_cached_src<F, ActQ8, STEPS, RB, KS, DUMP>(a, units, groups_per_row, row_bytes, stream);
+}
+
+template <class F, int STEPS, int KS>
+static hipError_t launch_steps(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
+                               uint32_t rb, hipStream_t stream) {
+    if (a.sums) return launch_cached<F, STEPS, 1, KS, true>(a, units, groups_per_row, row_bytes, stream);
+    if constexpr (STEPS <= 2) {
+        if (rb >= 4) return launch_cached<F, STEPS, 4, KS, false>(a, units, groups_per_row, row_bytes, stream);
+        if (rb >= 2) return launch_cached<F, STEPS, 2, KS, false>(a, units, groups_per_row, row_bytes, stream);
+    }
+    return launch_cached<F, STEPS, 1, KS, false>(a, units, groups_per_row, row_bytes, stream);
+}
+
+template <class F>
+static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStream_t stream) {
+    const uint32_t units = a.n_cols / F::UNIT_COLS;
+    const uint32_t groups_per_row = a.n_cols / group_cols;
+    const size_t row_bytes = (size_t)(a.n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
+    const uint32_t steps = (units + 63) / 64;
+    // Long rows are split over the four waves of a work group (fewer registers per wave,
+    // more waves per SIMD); short ones keep one wave per row and need no barrier.
+    uint32_t ks = a.waves_per_row;
+    if (ks == 0) ks = steps >= 3 ? 4 : 1;
+    // Rows per batch: two while a wave's slice of a row is at most ~3.4 KB, else one
+    // (measured on MI355X: more in flight per wave does not pay beyond that); Q6_K always one.
+    uint32_t rb = a.rows_per_batch;
+    if (rb == 0) rb = row_bytes / (ks >= 4 ? 4 : 1) <= F::TWO_ROW_BATCH_BYTES ? 2 : 1;
+    if (ks >= 4 && steps <= 32) {
+        const uint32_t sw = (steps + 3) / 4;
+        switch (sw) {
+        case 1: return launch_steps<F, 1, 4>(a, units, groups_per_row, row_bytes, rb, stream);
+        case 2: return launch_steps<F, 2, 4>(a, units, groups_per_row, row_bytes, rb, stream);
+        case 3:
+        case 4: return launch_steps<F, 4, 4>(a, units, groups_per_row, row_bytes, rb, stream);
+        default: return launch_steps<F, 8, 4>(a, units, groups_per_row, row_bytes, rb, stream);
+        }
+    }
+    switch (steps) {
+    case 1: return launch_steps<F, 1, 1>(a, units, groups_per_row, row_bytes, rb, stream);
+    case 2: return launch_steps<F, 2, 1>(a, units, groups_per_row, row_bytes, rb, stream);
+    case 3:
+    case 4: return launch_steps<F, 4, 1>(a, units, groups_per_row, row_bytes, rb, stream);
+    case 5:
+    case 6:
+    case 7:
+    case 8: return launch_steps<F, 8, 1>(a, units, groups_per_row, row_bytes, rb, stream);
+    default: break;
+    }
+    if (a.X) return hipErrorNotSupported;  // rows this long re-read the activations: Q8_0 blocks only
+    const uint32_t max_waves = device_cus() * a.waves_per_cu;
+    uint32_t waves = a.n_rows < max_waves ? a.n_rows : max_waves;
+    uint32_t blocks = (waves + 3) / 4;
+    if (blocks == 0) blocks = 1;
+    if (a.sums)
+        hipLaunchKernelGGL((gemv_q8_generic<F, true>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.out, a.sums,
+                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias);
+    else
+        hipLaunchKernelGGL((gemv_q8_generic<F, false>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.out, a.sums,
+                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias);
+    return hipGetLastError();
+}
+
+// True when one launch can take the n_mats matrices of `a` (the register-cached kernel, whole
+// batches per matrix); otherwise the caller gets one launch per matrix.
+template <class F>
+static bool multi_in_one_launch(const GemvArgs &a) {
+    return (a.n_cols / F::UNIT_COLS + 63) / 64 <= 32 && !a.sums;
+}
+
+// ---- several activation vectors per launch -------------------------------------------------
+
+template <class F, int STEPS, int KS, int NV>
+static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t row_bytes, hipStream_t stream) {
+    constexpr uint32_t G = 4 / KS;
+    const uint32_t max_groups = device_cus() * 8 / KS;
+    const uint32_t passes = (a.n_rows + max_groups - 1) / max_groups;
+    const uint32_t groups = (a.n_rows + passes - 1) / passes;
+    uint32_t blocks = (groups + G - 1) / G;
+    if (blocks == 0) blocks = 1;
+    hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride, a.out,
+                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias);
+    return hipGetLastError();
+}
+
+// Same split of a row over steps and waves as the single-vector kernel (so the fp32 sums are
+// formed in the same order and the results are bit-identical to one launch per vector); two
+// steps per wave leave registers for two vectors only.
+template <class F>
+static hipError_t launch_vecs_f(const GemvVecsArgs &a, hipStream_t stream) {
+    const uint32_t units = a.n_cols / F::UNIT_COLS;
+    const size_t row_bytes = (size_t)(a.n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
+    const uint32_t steps = (units + 63) / 64;
+    if (steps == 1)
+        return a.n_vecs > 2 ? launch_vecs_k<F, 1, 1, 4>(a, units, row_bytes, stream)
+                            : launch_vecs_k<F, 1, 1, 2>(a, units, row_bytes, stream);
+    if (steps == 2 && a.n_vecs <= 2) return launch_vecs_k<F, 2, 1, 2>(a, units, row_bytes, stream);
+    if (steps == 3 || steps == 4)
+        return a.n_vecs > 2 ? launch_vecs_k<F, 1, 4, 4>(a, units, row_bytes, stream)
+                            : launch_vecs_k<F, 1, 4, 2>(a, units, row_bytes, stream);
+    if (steps >= 5 && steps <= 8 && a.n_vecs <= 2) return launch_vecs_k<F, 2, 4, 2>(a, units, row_bytes, stream);
+    return hipErrorNotSupported;
+}
+
+// One matrix set (GemvArgs::n_mats) of format F: one launch when the register-cached kernel
+// takes it, else one launch per matrix.
+template <class F>
+static hipError_t launch_gemv_format(const GemvArgs &a, uint32_t group_cols, hipStream_t stream) {
+    if (a.n_mats > 1 && !multi_in_one_launch<F>(a)) {
+        for (uint32_t i = 0; i < a.n_mats; i++) {
+            GemvArgs s = a;
+            s.n_mats = 1;
+            if (i) {
+                s.W = a.W_more[i - 1];
+                s.out = a.out_more[i - 1];
+                s.bias = a.bias_more[i - 1];
+                if (a.n_rows_more[i - 1]) s.n_rows = a.n_rows_more[i - 1];
+            }
+            hipError_t e = launch_format<F>(s, group_cols, stream);
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
+    return launch_format<F>(a, group_cols, stream);
+}
+
+}  // namespace oxq

@@ -52,6 +52,12 @@ struct GemvVecsArgs {
 hipError_t launch_gemv_vecs(uint32_t type, const GemvVecsArgs &a, hipStream_t stream);
 // Most activation vectors one launch takes for rows of n_cols columns (4, 2, or 0: none).
 uint32_t gemv_vecs_max(uint32_t type, uint32_t n_cols);
+// Columns of one lane's unit (32 or 64; 0: unknown type) and weights per exact integer group sum.
+uint32_t gemv_unit_cols(uint32_t type);
+uint32_t gemv_group_cols(uint32_t type);
+// The formats beyond the first five live in a translation unit of their own.
+hipError_t launch_gemv_q8_more(uint32_t type, const GemvArgs &a, hipStream_t stream);
+hipError_t launch_gemv_vecs_more(uint32_t type, const GemvVecsArgs &a, hipStream_t stream);
 
 // x: n floats (n % 32 == 0) -> n/32 Q8_0 blocks of 34 bytes.
 hipError_t launch_quantize_q8_0(const float *x, size_t n, uint8_t *out, hipStream_t stream);

@@ -89,6 +89,83 @@ __device__ __forceinline__ float dq_iq4_xs(const uint8_t *b, uint32_t i) {
     return scale * (float)kv[idx];  // reference/iq4_xs.rs:91-92
 }
 
+// ---- the formats beyond the first five: element decoders in the reference's operation order ----
+
+__device__ __forceinline__ float dq_q4_1(const uint8_t *b, uint32_t i) {
+    const uint32_t byte = b[4 + (i >> 1)];
+    const float q = (float)((i & 1) ? (byte >> 4) : (byte & 0x0F));
+    return h2f(ld2(b)) * q + h2f(ld2(b + 2));  // reference/q4_1.rs:44-45
+}
+
+// q5 of Q5_0 / Q5_1: nibbles at qs, fifth bits in the u32 at qh (reference/q5_0.rs:43-51)
+__device__ __forceinline__ uint32_t q5_of(const uint8_t *qh, const uint8_t *qs, uint32_t i) {
+    const uint32_t bits = ld4(qh), byte = qs[i & 15];
+    const uint32_t nib = i < 16 ? (byte & 0x0F) : (byte >> 4);
+    return nib | (((bits >> i) & 1) << 4);
+}
+
+__device__ __forceinline__ float dq_q5_0(const uint8_t *b, uint32_t i) {
+    return h2f(ld2(b)) * (float)((int)q5_of(b + 2, b + 6, i) - 16);  // reference/q5_0.rs:50-54
+}
+
+__device__ __forceinline__ float dq_q5_1(const uint8_t *b, uint32_t i) {
+    return h2f(ld2(b)) * (float)q5_of(b + 4, b + 8, i) + h2f(ld2(b + 2));  // reference/q5_1.rs:51-55
+}
+
+__device__ __forceinline__ float dq_q8_1(const uint8_t *b, uint32_t i) {
+    return h2f(ld2(b)) * (float)(int8_t)b[4 + i];  // reference/q8_1.rs:40-42
+}
+
+__device__ __forceinline__ float dq_iq4_nl(const uint8_t *b, uint32_t i) {
+    const int8_t kv[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+    const uint32_t byte = b[2 + (i >> 1)];
+    return h2f(ld2(b)) * (float)kv[(i & 1) ? (byte >> 4) : (byte & 0x0F)];  // reference/iq4_nl.rs:45-50
+}
+
+// column i of a Q2_K / Q3_K super-block: group n, shift 2j, half hf, lane l
+__device__ __forceinline__ float dq_q2_k(const uint8_t *b, uint32_t i) {
+    const uint32_t is = i >> 4, n = i >> 7, j = (i >> 5) & 3, l = i & 31;
+    const uint32_t q = (b[16 + 32 * n + l] >> (2 * j)) & 3;
+    const float dl = h2f(ld2(b + 80)) * (float)(b[is] & 0x0F);  // reference/q2_k.rs:56-57
+    const float ml = h2f(ld2(b + 82)) * (float)(b[is] >> 4);
+    return dl * (float)q - ml;  // reference/q2_k.rs:62
+}
+
+__device__ __forceinline__ float dq_q3_k(const uint8_t *b, uint32_t i) {
+    const uint32_t is = i >> 4, n = i >> 7, j = (i >> 5) & 3, l = i & 31;
+    const uint8_t *s = b + 96;
+    uint32_t sc;  // decode_scales, reference/q3_k.rs:30-59
+    if (is < 8) {
+        sc = s[is] & 0x3F;
+    } else if (is < 12) {
+        sc = (s[is] & 0x0F) | ((uint32_t)(s[is - 8] >> 6) << 4);
+    } else {
+        sc = (s[is - 4] >> 4) | ((uint32_t)(s[is - 8] >> 6) << 4);
+    }
+    const int q_lo = (int)((b[32 + 32 * n + l] >> (2 * j)) & 3);
+    const int sub = (b[l] >> (4 * n + j)) & 1 ? 0 : 4;  // reference/q3_k.rs:108-111
+    const float dl = h2f(ld2(b + 108)) * (float)((int)sc - 32);
+    return dl * (float)(q_lo - sub);
+}
+
+__device__ __forceinline__ float dq_q5_k(const uint8_t *b, uint32_t i) {
+    const float d = h2f(ld2(b)), dmin = h2f(ld2(b + 2));
+    const uint8_t *s = b + 4;
+    const uint32_t j = i >> 5, l = i & 31, g = j >> 1;
+    uint32_t sc, mn;  // reference/q5_k.rs:27-49
+    if (j < 4) {
+        sc = s[j] & 0x3F;
+        mn = s[j + 4] & 0x3F;
+    } else {
+        sc = (s[j + 4] & 0x0F) | ((uint32_t)(s[j - 4] >> 6) << 4);
+        mn = (s[j + 4] >> 4) | ((uint32_t)(s[j] >> 6) << 4);
+    }
+    const uint32_t byte = b[48 + 32 * g + l];
+    const uint32_t nib = (j & 1) ? (byte >> 4) : (byte & 0x0F);
+    const uint32_t q = nib | (((b[16 + l] >> (g + 4 * (j & 1))) & 1) << 4);  // reference/q5_k.rs:84-95
+    return d * (float)sc * (float)q - dmin * (float)mn;
+}
+
 __global__ __launch_bounds__(256) void dequant_kernel(uint32_t type, const uint8_t *__restrict__ blocks,
                                                      float *__restrict__ out, size_t n_elems,
                                                      uint32_t block_cols, uint32_t block_bytes) {
@@ -102,7 +179,15 @@ __global__ __launch_bounds__(256) void dequant_kernel(uint32_t type, const uint8
     case OXQ_TYPE_Q8_0: v = dq_q8_0(b, i); break;
     case OXQ_TYPE_Q4_K: v = dq_q4_k(b, i); break;
     case OXQ_TYPE_Q6_K: v = dq_q6_k(b, i); break;
-    default: v = dq_iq4_xs(b, i); break;
+    case OXQ_TYPE_IQ4_XS: v = dq_iq4_xs(b, i); break;
+    case OXQ_TYPE_Q4_1: v = dq_q4_1(b, i); break;
+    case OXQ_TYPE_Q5_0: v = dq_q5_0(b, i); break;
+    case OXQ_TYPE_Q5_1: v = dq_q5_1(b, i); break;
+    case OXQ_TYPE_Q8_1: v = dq_q8_1(b, i); break;
+    case OXQ_TYPE_IQ4_NL: v = dq_iq4_nl(b, i); break;
+    case OXQ_TYPE_Q2_K: v = dq_q2_k(b, i); break;
+    case OXQ_TYPE_Q3_K: v = dq_q3_k(b, i); break;
+    default: v = dq_q5_k(b, i); break;
     }
     out[e] = v;
 }

@@ -112,15 +112,26 @@ class GgufTensorType(enum.IntEnum):
     Q4K = 12
     Q6K = 14
     Iq4Xs = 23
+    Q4_1 = 3
+    Q5_0 = 6
+    Q5_1 = 7
+    Q8_1 = 9
+    Q2K = 10
+    Q3K = 11
+    Q5K = 13
+    Iq4Nl = 20
 
     def block_size(self):
-        return {2: 32, 8: 32, 12: 256, 14: 256, 23: 256}[int(self)]
+        return {2: 32, 8: 32, 12: 256, 14: 256, 23: 256, 3: 32, 6: 32, 7: 32, 9: 32, 10: 256, 11: 256, 13: 256,
+                20: 32}[int(self)]
 
     def block_bytes(self):
-        return {2: 18, 8: 34, 12: 144, 14: 210, 23: 136}[int(self)]
+        return {2: 18, 8: 34, 12: 144, 14: 210, 23: 136, 3: 20, 6: 22, 7: 24, 9: 36, 10: 84, 11: 110, 13: 176,
+                20: 18}[int(self)]
 
     def type_name(self):
-        return {2: "Q4_0", 8: "Q8_0", 12: "Q4_K", 14: "Q6_K", 23: "IQ4_XS"}[int(self)]
+        return {2: "Q4_0", 8: "Q8_0", 12: "Q4_K", 14: "Q6_K", 23: "IQ4_XS", 3: "Q4_1", 6: "Q5_0", 7: "Q5_1", 9: "Q8_1",
+                10: "Q2_K", 11: "Q3_K", 13: "Q5_K", 20: "IQ4_NL"}[int(self)]
 
 
 class QuantTensor:
@@ -215,7 +226,7 @@ class HipKernel:
 
     def block_sums(self, weights, acts_q8, n_rows, n_cols):
         w, a = _u8(weights), _u8(acts_q8)
-        groups = n_cols // (16 if self.tensor_type == capi.TYPE_Q6_K else 32)
+        groups = n_cols // (16 if self.tensor_type in capi.GROUPS_OF_16 else 32)
         sums = np.zeros(n_rows * groups, dtype=np.int32)
         _check(self._lib.oxq_block_sums(self.tensor_type, _ptr(w), w.size, _ptr(a), a.size,
                                         _ptr(sums), sums.size, n_rows, n_cols))

@@ -16,6 +16,16 @@ ALL_TYPES = [Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS]
 BLOCK = {Q4_0: (32, 18), Q8_0: (32, 34), Q4_K: (256, 144), Q6_K: (256, 210), IQ4_XS: (256, 136)}
 NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", IQ4_XS: "IQ4_XS"}
 
+# formats beyond the first five (oracle/oxq_oracle_more.c); integer groups of 16 for Q2_K / Q3_K
+Q4_1, Q5_0, Q5_1, Q8_1, Q2_K, Q3_K, Q5_K, IQ4_NL = 3, 6, 7, 9, 10, 11, 13, 20
+MORE_TYPES = [Q4_1, Q5_0, Q5_1, Q8_1, Q2_K, Q3_K, Q5_K, IQ4_NL]
+BLOCK.update({Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q8_1: (32, 36), Q2_K: (256, 84), Q3_K: (256, 110),
+              Q5_K: (256, 176), IQ4_NL: (32, 18)})
+NAMES.update({Q4_1: "Q4_1", Q5_0: "Q5_0", Q5_1: "Q5_1", Q8_1: "Q8_1", Q2_K: "Q2_K", Q3_K: "Q3_K", Q5_K: "Q5_K",
+              IQ4_NL: "IQ4_NL"})
+GROUP_COLS = {t: 32 for t in BLOCK}
+GROUP_COLS.update({Q6_K: 16, Q2_K: 16, Q3_K: 16})
+
 TIER_SCALAR, TIER_AVX2, TIER_Q4_0_STANDALONE = 0, 1, 2
 OK, UNSUPPORTED_TYPE, DIMENSION_MISMATCH, KERNEL_ERROR, BUFFER_TOO_SMALL = 0, 1, 3, 4, 6
 
@@ -133,7 +143,7 @@ def _u8(a):
 
 
 def groups_per_row(t, n_cols):
-    return n_cols // (16 if t == Q6_K else 32)
+    return n_cols // GROUP_COLS[t]
 
 
 def row_bytes(t, n_cols):
@@ -332,3 +342,57 @@ def linear_forward(t, w, n_rows, n_cols, x, bias=None, lora=None, tier=TIER_AVX2
     _chk(load().oxq_ref_linear_forward(t, tier, _p(w), w.size, n_rows, n_cols, bp, bl, ap, bq, rank, scale, _p(x),
                                        x.size, _p(out), out.size))
     return out
+
+
+# ---- builders for the other formats' blocks, mirroring the make_*_block helpers of the reference's tests ----
+
+def make_q4_1_block(d, m, qs):  # Q/reference/q4_1.rs tests
+    return f16_bytes(d) + f16_bytes(m) + bytes(qs)
+
+
+def make_q5_0_block(d, qh, qs):  # Q/reference/q5_0.rs:248-254
+    return f16_bytes(d) + int(qh).to_bytes(4, "little") + bytes(qs)
+
+
+def make_q5_1_block(d, m, qh, qs):  # Q/reference/q5_1.rs tests
+    return f16_bytes(d) + f16_bytes(m) + int(qh).to_bytes(4, "little") + bytes(qs)
+
+
+def make_q8_1_block(d, qs):  # Q/reference/q8_1.rs tests: s = d * sum(qs) as f16
+    return f16_bytes(d) + f16_bytes(float(d) * float(sum(qs))) + bytes(int(q) & 0xFF for q in qs)
+
+
+def make_iq4_nl_block(scale, nibble_bytes):  # Q/reference/iq4_nl.rs tests
+    return f16_bytes(scale) + bytes(nibble_bytes)
+
+
+def make_q2_k_block(d, dmin, scales, qs):  # Q/reference/q2_k.rs tests
+    return bytes(scales) + bytes(qs) + f16_bytes(d) + f16_bytes(dmin)
+
+
+def make_q3_k_block(d, scales, hmask, qs):  # Q/reference/q3_k.rs tests
+    return bytes(hmask) + bytes(qs) + bytes(scales) + f16_bytes(d)
+
+
+def make_q5_k_block(d, dmin, scales, qh, qs):  # Q/reference/q5_k.rs:362-377
+    return f16_bytes(d) + f16_bytes(dmin) + bytes(scales) + bytes(qh) + bytes(qs)
+
+
+# byte offsets of the f16 fields of each format's block
+F16_FIELDS = {Q4_0: (0,), Q8_0: (0,), Q4_K: (0, 2), Q6_K: (208,), IQ4_XS: (0,), Q4_1: (0, 2), Q5_0: (0,), Q5_1: (0, 2),
+              Q8_1: (0, 2), Q2_K: (80, 82), Q3_K: (108,), Q5_K: (0, 2), IQ4_NL: (0,)}
+
+
+def random_blocks(t, seed, n_rows, n_cols, scale=0.02):
+    """Valid blocks with every payload bit random: uniform random bytes, f16 fields drawn from
+    +-[scale/4, scale] (finite, normal).  Any bytes are a legal block of these formats."""
+    rng = np.random.default_rng(seed)
+    bs, bb = BLOCK[t]
+    n_blocks = n_rows * (n_cols // bs)
+    w = rng.integers(0, 256, size=(n_blocks, bb), dtype=np.uint8)
+    for off in F16_FIELDS[t]:
+        v = (rng.uniform(scale / 4, scale, n_blocks) * rng.choice([-1.0, 1.0], n_blocks)).astype(np.float16)
+        if off in (2, 82) and t in (Q4_K, Q5_K, Q2_K):
+            v = np.abs(v)  # dmin is a magnitude in real files
+        w[:, off:off + 2] = v.view(np.uint8).reshape(n_blocks, 2)
+    return w.reshape(-1)

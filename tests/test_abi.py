@@ -33,15 +33,17 @@ def test_format_metadata_matches_reference_tables():
     # crates/oxillama-gguf/src/types.rs:199-262
     lib = capi.load()
     table = {2: (32, 18, b"Q4_0"), 8: (32, 34, b"Q8_0"), 12: (256, 144, b"Q4_K"), 14: (256, 210, b"Q6_K"),
-             23: (256, 136, b"IQ4_XS")}
+             23: (256, 136, b"IQ4_XS"), 3: (32, 20, b"Q4_1"), 6: (32, 22, b"Q5_0"), 7: (32, 24, b"Q5_1"),
+             9: (32, 36, b"Q8_1"), 10: (256, 84, b"Q2_K"), 11: (256, 110, b"Q3_K"), 13: (256, 176, b"Q5_K"),
+             20: (32, 18, b"IQ4_NL")}
     for t, (bs, bb, name) in table.items():
         assert lib.oxq_block_size(t) == bs and lib.oxq_block_bytes(t) == bb and lib.oxq_type_name(t) == name
         assert lib.oxq_get_kernel(t) == capi.OK
-    for t in (0, 1, 3, 13, 15, 39):  # formats this library has no kernel for
+    for t in (0, 1, 15, 16, 24, 39):  # formats this library has no kernel for
         assert lib.oxq_block_size(t) == 0 and lib.oxq_type_name(t) is None
         assert lib.oxq_get_kernel(t) == capi.ERR_UNSUPPORTED_TYPE
     with pytest.raises(quant.UnsupportedType):
-        quant.KernelDispatcher().get_kernel(13)
+        quant.KernelDispatcher().get_kernel(15)
 
 
 def test_status_names_follow_quant_error_variants():
@@ -58,7 +60,7 @@ def test_quantize_rejects_unaligned_length_before_touching_the_gpu():
     assert (e.value.expected, e.value.got) == (32, 31)
 
 
-@pytest.mark.parametrize("t", [2, 8, 12, 14, 23])
+@pytest.mark.parametrize("t", [2, 8, 12, 14, 23, 3, 6, 7, 9, 10, 11, 13, 20])
 def test_fused_validation_order_before_touching_the_gpu(t):
     # Q/reference/q4_k.rs:226-250: out, then weights, then activations
     k = quant.HipKernel(t)
@@ -80,7 +82,7 @@ def test_fused_validation_order_before_touching_the_gpu(t):
         k.matvec_q8_fused(w, a, np.zeros(3, dtype=np.float32), n_rows, n_cols - 1)
 
 
-@pytest.mark.parametrize("t", [2, 8, 12, 14, 23])
+@pytest.mark.parametrize("t", [2, 8, 12, 14, 23, 3, 6, 7, 9, 10, 11, 13, 20])
 def test_dequant_and_gemv_argument_errors(t):
     k = quant.HipKernel(t)
     bs, bb = k.block_size(), k.block_bytes()

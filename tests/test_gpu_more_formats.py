@@ -1,0 +1,197 @@
+"""Parity of the HIP path for the formats beyond the first five (Q4_1, Q5_0, Q5_1, Q8_1, IQ4_NL,
+Q2_K, Q3_K, Q5_K) against the CPU oracle, through the C ABI: dequant_block and integer group
+sums bit-exact, fp32 within 1e-5 * |y_ref|_inf of the reference's *Ref kernels
+(crates/oxillama-quant/src/reference/*.rs).  Weights are random bytes with finite f16 scale
+fields, so every bit pattern of the payload is exercised."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+from oxillama_amd import linear as L
+from oxillama_amd import synth
+
+pytestmark = pytest.mark.gpu
+FP32_REL_TOL = 1e-5
+DEV = "cuda:0"
+TYPES = O.MORE_TYPES
+ids = lambda t: O.NAMES[t]
+
+
+def say(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def assert_close(y, y_ref, what, tol=FP32_REL_TOL):
+    scale = float(np.abs(y_ref).max())
+    err = float(np.abs(y.astype(np.float64) - y_ref.astype(np.float64)).max())
+    assert err <= tol * scale + 1e-30, f"{what}: max err {err:.3e} > {tol} * {scale:.3e}"
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+KAT_BLOCKS = {
+    O.Q4_1: [O.make_q4_1_block(1.0, 2.0, [0x88] * 16), O.make_q4_1_block(0.0, 5.0, [0] * 16)],
+    O.Q5_0: [O.make_q5_0_block(1.0, 0xFFFFFFFF, [0xFF] * 16), O.make_q5_0_block(2.0, 0, [0] * 16),
+             O.make_q5_0_block(0.5, 0xA5A5A5A5, [(i * 11 + 5) & 0xFF for i in range(16)])],
+    O.Q5_1: [O.make_q5_1_block(1.0, 0.0, 0xFFFFFFFF, [0xFF] * 16), O.make_q5_1_block(0.0, 3.0, 0, [0] * 16)],
+    O.Q8_1: [O.make_q8_1_block(0.5, [10] * 32), O.make_q8_1_block(2.0, [-5] * 32)],
+    O.IQ4_NL: [O.make_iq4_nl_block(1.0, [0x50] + [0] * 15), O.make_iq4_nl_block(1.0, [0xFF] * 16)],
+    O.Q2_K: [O.make_q2_k_block(1.0, 0.0, [0x01] * 16, [0xFF] * 64), O.make_q2_k_block(2.0, 1.0, [0x11] * 16, [0] * 64)],
+    O.Q3_K: [O.make_q3_k_block(1.0, [0xA1] * 8 + [0x11] * 4, [0] * 32, [0] * 64),
+             O.make_q3_k_block(1.0, [0xA1] * 8 + [0x11] * 4, [0xFF] * 32, [0xFF] * 64)],
+    O.Q5_K: [O.make_q5_k_block(1.0, 0.0, [1] * 4 + [0] * 4 + [1] * 4, [0] * 32, [0x88] * 128),
+             O.make_q5_k_block(1.0, 0.0, [1] * 4 + [0] * 4 + [1] * 4, [0xFF] * 32, [0] * 128)],
+}
+KAT_VALUES = {O.Q4_1: [10.0, 5.0], O.Q5_0: [15.0, -32.0, None], O.Q5_1: [31.0, 3.0], O.Q8_1: [5.0, -10.0],
+              O.IQ4_NL: [None, 113.0], O.Q2_K: [3.0, -1.0], O.Q3_K: [-4.0, 3.0], O.Q5_K: [8.0, 16.0]}
+
+
+@pytest.mark.parametrize("t", TYPES, ids=ids)
+def test_metadata_and_dispatch(hip, t):
+    k = hip.KernelDispatcher().get_kernel(t)
+    assert (k.block_size(), k.block_bytes(), k.name()) == (*O.BLOCK[t], O.NAMES[t])
+    assert k.gemm_workspace_bytes(64, 4096, 4096) == 0  # no tile kernel: the batched form runs by rows
+
+
+def test_unknown_types_still_rejected(hip):
+    for t in (0, 1, 15, 16, 24, 30, 99):  # F32, F16, Q8_K, IQ2_XXS, I8, BF16, nonsense
+        with pytest.raises(hip.UnsupportedType):
+            hip.HipKernel(t)
+
+
+@pytest.mark.parametrize("t", TYPES, ids=ids)
+def test_dequant_block(hip, ref, t):
+    bs, bb = O.BLOCK[t]
+    k = hip.HipKernel(t)
+    for blk, val in zip(KAT_BLOCKS[t], KAT_VALUES[t]):  # the reference's hand-built blocks
+        out = np.zeros(bs, dtype=np.float32)
+        k.dequant_block(np.frombuffer(blk, dtype=np.uint8), out)
+        if val is not None:
+            assert np.all(out == val)
+        assert np.array_equal(out, ref.dequant_block(t, np.frombuffer(blk, dtype=np.uint8)))
+    w = O.random_blocks(t, 200 + t, 12, bs)
+    for i in range(12):
+        out = np.zeros(bs, dtype=np.float32)
+        k.dequant_block(w[i * bb:(i + 1) * bb], out)
+        assert np.array_equal(out, ref.dequant_block(t, w[i * bb:(i + 1) * bb])), f"block {i}"
+    with pytest.raises(hip.BufferTooSmall) as e:
+        k.dequant_block(w[:bb - 1], np.zeros(bs, dtype=np.float32))
+    assert (e.value.needed, e.value.available) == (bb, bb - 1)
+
+
+SHAPES = ((5, 256), (96, 512), (64, 4096), (33, 14336), (9, 2 * 32768 + 256))
+
+
+@pytest.mark.parametrize("t", TYPES, ids=ids)
+def test_fused_matvec_sums_and_fp32(hip, ref, t):
+    k = hip.HipKernel(t)
+    for seed, (n_rows, n_cols) in enumerate(SHAPES):
+        say("fused", O.NAMES[t], n_rows, n_cols)
+        w = O.random_blocks(t, 300 + 10 * t + seed, n_rows, n_cols)
+        x = synth.normal_f32(400 + seed, n_cols)
+        a = ref.quantize_q8_0(x)
+        sums = k.block_sums(w, a, n_rows, n_cols)
+        assert np.array_equal(sums, ref.block_sums(t, w, a, n_rows, n_cols)), "integer group sums"
+        out = np.full(n_rows, 42.0, dtype=np.float32)  # accumulate semantics (traits.rs:169)
+        k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+        want = ref.matvec_q8_fused(t, w, a, n_rows, n_cols, out=np.full(n_rows, 42.0, dtype=np.float32))
+        # Rows of 65 792 columns (the kernel without cached activations): the reference adds every element
+        # into one fp32 accumulator, whose own rounding noise there is about sqrt(n) * 2^-24 * |partial sums|,
+        # i.e. 1e-5 of |y|; the bar is widened for that shape only.
+        assert_close(out - 42.0, want - 42.0, f"fused {O.NAMES[t]} {n_rows}x{n_cols}",
+                     tol=FP32_REL_TOL if n_cols <= 32768 else 5e-5)
+        # zero activations contribute nothing (q4_0.rs:382-392 applied to every format)
+        zero = ref.quantize_q8_0(np.zeros(n_cols, dtype=np.float32))
+        out = np.full(n_rows, 77.0, dtype=np.float32)
+        k.matvec_q8_fused(w, zero, out, n_rows, n_cols)
+        assert np.all(out == 77.0)
+
+
+@pytest.mark.parametrize("t", TYPES, ids=ids)
+def test_gemv_gemm_host_route(hip, ref, t):
+    n, kk = 160, 1024
+    w = O.random_blocks(t, 500 + t, n, kk)
+    k = hip.HipKernel(t)
+    qt = hip.QuantTensor(w, [n, kk], t)
+    x = synth.normal_f32(3, kk)
+    y = np.full(n, -1.0, dtype=np.float32)
+    k.gemv(qt, x, y)
+    z = np.zeros(n, dtype=np.float32)
+    k.matvec_q8_fused(w, ref.quantize_q8_0(x), z, n, kk)
+    assert np.array_equal(y, z)  # gemv = quantize + fused into zeros
+    # against the reference's fp32-activation gemv: equal up to the Q8_0 rounding of x (about 1/127 per element)
+    y_f32 = ref.gemv(t, w, n, kk, x)
+    assert np.abs(y - y_f32).max() <= 0.02 * np.abs(y_f32).max()
+    for m in (2, 5, 13):  # several vectors per pass, chunks of four, more rows than the tile threshold
+        xs = synth.normal_f32(10 + m, m * kk)
+        ys = np.zeros(m * n, dtype=np.float32)
+        k.gemm(qt, xs, ys, m, n, kk)
+        for r in range(m):
+            yr = np.zeros(n, dtype=np.float32)
+            k.gemv(qt, xs[r * kk:(r + 1) * kk], yr)
+            assert np.array_equal(ys[r * n:(r + 1) * n], yr), f"gemm row {r} of {m}"
+        assert_close(ys, ref.gemm_q8(t, w, xs, m, n, kk).ravel(), f"gemm {m}")
+    with pytest.raises(hip.DimensionMismatch) as e:
+        k.gemv(qt, x[:-1], y)
+    assert (e.value.expected, e.value.got) == (kk, kk - 1)
+
+
+@pytest.mark.parametrize("t", TYPES, ids=ids)
+def test_device_route_forms(hip, ref, t):
+    """fp32 activations quantized in the kernel, bias epilogue, several matrices of different heights in one
+    launch, several vectors per pass: each bit-identical to the plain fused launch."""
+    k = hip.HipKernel(t)
+    for n_cols, heights in ((4096, (1024, 256, 512)), (14336, (96, 200))):
+        say("device forms", O.NAMES[t], n_cols, heights)
+        x = synth.normal_f32(5, n_cols)
+        d_x = dev(x)
+        d_acts = torch.empty(n_cols // 32 * 34, dtype=torch.uint8, device=DEV)
+        hip.quantize_q8_0_dev(d_x, d_acts)
+        ws, bs_, singles = [], [], []
+        for i, h in enumerate(heights):
+            w = dev(O.random_blocks(t, 600 + 10 * t + i, h, n_cols))
+            b = dev(synth.normal_f32(40 + i, h))
+            one = torch.zeros(h, dtype=torch.float32, device=DEV)
+            k.matvec_q8_fused_dev(w, d_acts, one, h, n_cols, accumulate=False)
+            ws.append(w); bs_.append(b); singles.append(host(one))
+            f32 = torch.empty(h, dtype=torch.float32, device=DEV)
+            k.gemv_dev(w, d_x, f32, h, n_cols)
+            assert np.array_equal(host(f32), singles[i]), "in-kernel quantization"
+        outs = [torch.empty(h, dtype=torch.float32, device=DEV) for h in heights]
+        L.linear_forward_multi_dev(t, ws, d_acts, outs, heights, n_cols, d_biases=bs_)
+        for i, h in enumerate(heights):
+            assert np.array_equal(host(outs[i]), (singles[i] + host(bs_[i])).astype(np.float32)), f"matrix {i}"
+        # against the oracle
+        want = ref.matvec_q8_fused_mt(t, host(ws[0]), host(d_acts), heights[0], n_cols, 8)
+        assert_close(singles[0], want, "device fused")
+        # a small batch through the batched entry point (GEMV launches of up to four vectors)
+        m = 4
+        xs = synth.normal_f32(77, m * n_cols)
+        d_as = torch.empty(m * (n_cols // 32 * 34), dtype=torch.uint8, device=DEV)
+        hip.quantize_q8_0_dev(dev(xs), d_as)
+        d_y = torch.empty(m * heights[0], dtype=torch.float32, device=DEV)
+        k.gemm_q8_dev(ws[0], d_as, d_y, m, heights[0], n_cols)
+        ys = host(d_y).reshape(m, heights[0])
+        for r in range(m):
+            one = torch.zeros(heights[0], dtype=torch.float32, device=DEV)
+            k.matvec_q8_fused_dev(ws[0], d_as[r * (n_cols // 32 * 34):], one, heights[0], n_cols, accumulate=False)
+            assert np.array_equal(ys[r], host(one)), f"batch row {r}"
+
+
+def test_grouped_form_reports_unsupported(hip):
+    z = torch.zeros(4096, dtype=torch.uint8, device=DEV)
+    k = hip.HipKernel(O.Q5_K)
+    assert k.moe_gemm_workspace_bytes(64, 256, 256) == 0
+    with pytest.raises(hip.UnsupportedShape):
+        k.moe_gemm_q8_dev(z, 256 * 176, 1, z, z, 4, 4, z, 256, 256, z)
