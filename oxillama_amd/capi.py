@@ -44,6 +44,37 @@ class DeviceProps(C.Structure):
     ]
 
 
+class GgufSummary(C.Structure):
+    _fields_ = [("version", C.c_uint32), ("tensor_count", C.c_uint64), ("metadata_kv_count", C.c_uint64),
+                ("n_tensors", C.c_uint64), ("n_metadata", C.c_uint64), ("alignment", C.c_uint64),
+                ("data_offset", C.c_uint64), ("file_size", C.c_uint64)]
+
+
+class GgufTensor(C.Structure):
+    _fields_ = [("name", C.c_char_p), ("n_dims", C.c_uint32), ("dims", C.c_uint64 * 4), ("type", C.c_uint32),
+                ("offset", C.c_uint64), ("n_elements", C.c_uint64), ("data_size", C.c_uint64)]
+
+
+class GgufValue(C.Structure):
+    _fields_ = [("type", C.c_uint32), ("u", C.c_uint64), ("i", C.c_int64), ("f", C.c_double), ("str", C.c_void_p),
+                ("str_len", C.c_size_t), ("elem_type", C.c_uint32), ("count", C.c_uint64)]
+
+
+# include/oxq_gguf.h
+GGUF_SIGNATURES = {
+    "oxq_gguf_open": (C.c_int, [C.c_char_p, C.POINTER(C.c_void_p)]),
+    "oxq_gguf_open_bytes": (C.c_int, [C.c_void_p, C.c_size_t, C.POINTER(C.c_void_p)]),
+    "oxq_gguf_close": (C.c_int, [C.c_void_p]),
+    "oxq_gguf_get_summary": (C.c_int, [C.c_void_p, C.POINTER(GgufSummary)]),
+    "oxq_gguf_tensor_at": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(GgufTensor)]),
+    "oxq_gguf_find_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(GgufTensor)]),
+    "oxq_gguf_tensor_data": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]),
+    "oxq_gguf_meta_find": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(GgufValue)]),
+    "oxq_gguf_meta_at": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_char_p), C.POINTER(GgufValue)]),
+    "oxq_gguf_load_weights": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]),
+    "oxq_gguf_upload_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]),
+}
+
 SIGNATURES = {
     "oxq_init": (C.c_int, [C.c_int]),
     "oxq_shutdown": (C.c_int, []),
@@ -134,7 +165,7 @@ def load():
             f"{LIB_PATH} is missing: build it with `python -m oxillama_amd.build` "
             "(there is no CPU fallback for the HIP path)")
     lib = C.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in SIGNATURES.items():
+    for name, (restype, argtypes) in {**SIGNATURES, **GGUF_SIGNATURES}.items():
         fn = getattr(lib, name)  # AttributeError if the ABI lost a symbol
         fn.restype = restype
         fn.argtypes = argtypes

@@ -16,12 +16,6 @@ extern uint32_t g_gemm_tile_min_rows;
 hipError_t launch_dequant(uint32_t type, const uint8_t *blocks, size_t n_blocks, float *out, hipStream_t stream);
 }
 
-struct oxq_weights {
-    uint32_t type;
-    size_t n_rows, n_cols, nbytes;
-    uint8_t *dev;
-};
-
 namespace {
 
 struct ErrorDetail {
@@ -225,6 +219,8 @@ int tensor_dims(uint32_t type, size_t data_len, const size_t *shape, size_t n_di
 
 namespace oxq {
 uint32_t device_cus() { return g.cus ? g.cus : 256; }
+int set_error(int status, size_t a, size_t b, const char *msg) { return fail(status, a, b, msg); }
+int ensure_device() { return ensure_init(); }
 }  // namespace oxq
 
 extern "C" {
@@ -268,6 +264,7 @@ int oxq_shutdown(void) {
     g.s_lora_a.release();
     g.s_lora_b.release();
     g.s_lora_r.release();
+    oxq::gguf_release_staging();
     g.initialised = false;
     g.device = -1;
     return OXQ_OK;
@@ -310,6 +307,14 @@ const char *oxq_status_name(int status) {
     case OXQ_ERR_INTERNAL: return "Internal";
     case OXQ_ERR_UNSUPPORTED_SHAPE: return "UnsupportedShape";
     case OXQ_ERR_NO_DEVICE: return "NoDevice";
+    case 10: return "GgufInvalidMagic";
+    case 11: return "GgufUnsupportedVersion";
+    case 12: return "GgufUnexpectedEof";
+    case 13: return "GgufInvalidMetadata";
+    case 14: return "GgufUnsupportedQuantType";
+    case 15: return "GgufTensorNotFound";
+    case 16: return "GgufInvalidString";
+    case 17: return "GgufIo";
     default: return "Unknown";
     }
 }

@@ -6,7 +6,21 @@
 
 #include "../../include/oxq.h"
 
+// A weight matrix resident in HBM (oxq_weights_t): raw GGUF blocks, row-major.
+struct oxq_weights {
+    uint32_t type;
+    size_t n_rows, n_cols, nbytes;
+    uint8_t *dev;
+};
+
 namespace oxq {
+
+// Record the calling thread's error detail (what oxq_last_error reports) and return `status`.
+int set_error(int status, size_t a, size_t b, const char *msg);
+// oxq_init(0) unless a device is already initialised.
+int ensure_device();
+// GGUF loader: pinned staging buffers, released at shutdown.
+void gguf_release_staging();
 
 struct GemvArgs {
     const uint8_t *W;     // raw GGUF blocks, row-major, device memory

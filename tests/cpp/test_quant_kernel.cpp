@@ -16,6 +16,7 @@
 #include <string>
 #include <vector>
 
+#include "oxq/gguf_model.hpp"
 #include "oxq/quant_kernel.hpp"
 
 using namespace oxq;
@@ -247,6 +248,52 @@ static void host_tests() {
         y.resize(31);
         r = lin.forward(k, x, y);
         CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch && r.error().expected == 32 && r.error().got == 31);
+    });
+
+    // ---- GGUF reader: the file images of crates/oxillama-gguf/src/parser.rs tests, byte for byte ----
+    auto put32 = [](std::vector<uint8_t> &b, uint32_t v) { for (int i = 0; i < 4; ++i) b.push_back((uint8_t)(v >> (8 * i))); };
+    auto put64 = [](std::vector<uint8_t> &b, uint64_t v) { for (int i = 0; i < 8; ++i) b.push_back((uint8_t)(v >> (8 * i))); };
+    auto put_str = [&](std::vector<uint8_t> &b, const std::string &s) { put64(b, s.size()); b.insert(b.end(), s.begin(), s.end()); };
+    auto build_test_gguf = [&] {  // parser.rs:232-270
+        std::vector<uint8_t> d;
+        put32(d, 0x46554747u); put32(d, 3); put64(d, 1); put64(d, 2);
+        put_str(d, "general.architecture"); put32(d, 8); put_str(d, "llama");
+        put_str(d, "llama.block_count"); put32(d, 4); put32(d, 32);
+        put_str(d, "output.weight"); put32(d, 2); put64(d, 32); put64(d, 32); put32(d, 2); put64(d, 0);
+        d.resize((d.size() + 31) / 32 * 32, 0);
+        d.resize(d.size() + 1024, 0xAB);
+        return d;
+    };
+
+    run("gguf parse_full_gguf, tensor_data_access, missing_tensor (parser.rs:277-307)", [&] {
+        GgufModel m;
+        CHECK(m.from_bytes(build_test_gguf()) == OXQ_OK);
+        CHECK(m.header().version == 3 && m.header().tensor_count == 1 && m.header().metadata_kv_count == 2);
+        std::string arch;
+        uint64_t blocks = 0;
+        CHECK(m.architecture(arch) == OXQ_OK && arch == "llama");
+        CHECK(m.get_u64("llama.block_count", blocks) == OXQ_OK && blocks == 32);
+        TensorInfo t;
+        CHECK(m.tensor("output.weight", t) == OXQ_OK);
+        CHECK(t.n_dims == 2 && t.dimensions == std::vector<uint64_t>({32, 32}) && t.tensor_type == 2);
+        CHECK(t.n_elements() == 1024 && t.data_size() == 576);
+        const uint8_t *p = nullptr;
+        size_t n = 0;
+        CHECK(m.tensor_data("output.weight", p, n) == OXQ_OK && n == 576 && p[0] == 0xAB && p[575] == 0xAB);
+        CHECK(m.tensor_data("nonexistent", p, n) == OXQ_ERR_GGUF_TENSOR_NOT_FOUND);
+    });
+
+    run("gguf header errors: magic, version, truncation (header.rs:121-167, loader.rs tests)", [&] {
+        GgufModel m;
+        size_t a = 0, b = 0;
+        CHECK(m.from_bytes({0, 0, 0, 0, 3, 0, 0, 0}) == OXQ_ERR_GGUF_INVALID_MAGIC);
+        oxq_last_error(&a, &b, nullptr, 0);
+        CHECK(a == 0);
+        std::vector<uint8_t> v0;
+        put32(v0, 0x46554747u); put32(v0, 0); put32(v0, 0); put32(v0, 0);
+        CHECK(m.from_bytes(v0) == OXQ_ERR_GGUF_UNSUPPORTED_VERSION);
+        CHECK(m.from_bytes({'G', 'G', 'U', 'F'}) == OXQ_ERR_GGUF_UNEXPECTED_EOF);
+        CHECK(m.load("/nonexistent/path/does_not_exist.gguf") == OXQ_ERR_GGUF_IO);
     });
 }
 
@@ -556,6 +603,37 @@ static void gpu_tests() {
             CHECK_NEAR(y[r * 32 + r], 2.0 * (r + 1) + r, 8e-3);
             CHECK(y[r * 32 + 31] == 31.0f);
         }
+    });
+
+    run("gguf load_quant_linear: the tensor loads into HBM with its stored shape and size (llama/model.rs:805-822)", [&] {
+        auto k = kernel(GgufTensorType::Q8_0);
+        // one Q8_0 tensor [2, 32]: row 0 = d 1.0, q = 1..32; row 1 = d 0.5, q = -16..15
+        std::vector<int> q0(32), q1(32);
+        for (int i = 0; i < 32; ++i) { q0[i] = i + 1; q1[i] = i - 16; }
+        std::vector<uint8_t> w = q8_0_block(1.0f, q0);
+        append(w, q8_0_block(0.5f, q1));
+        std::vector<uint8_t> d;
+        auto put32 = [&](uint32_t v) { for (int i = 0; i < 4; ++i) d.push_back((uint8_t)(v >> (8 * i))); };
+        auto put64 = [&](uint64_t v) { for (int i = 0; i < 8; ++i) d.push_back((uint8_t)(v >> (8 * i))); };
+        auto put_str = [&](const std::string &s) { put64(s.size()); d.insert(d.end(), s.begin(), s.end()); };
+        put32(0x46554747u); put32(3); put64(1); put64(0);
+        put_str("blk.0.attn_q.weight"); put32(2); put64(2); put64(32); put32(8); put64(0);
+        d.resize((d.size() + 31) / 32 * 32, 0);
+        append(d, w);
+        GgufModel m;
+        CHECK(m.from_bytes(d) == OXQ_OK);
+        DeviceWeights dw;
+        CHECK(m.load_quant_linear("blk.0.attn_q.weight", dw) == OXQ_OK);
+        CHECK(dw.shape == std::vector<size_t>({2, 32}) && dw.tensor_type == 8 && dw.nbytes() == 68);
+        // the same bytes through the host-slice trait method
+        std::vector<float> x(32, 1.0f), y_host(2, 0.0f);
+        std::vector<uint8_t> acts;
+        CHECK(quantize_f32_to_q8_0(x, acts).is_ok());
+        CHECK(k->matvec_q8_fused(w, acts, y_host, 2, 32).is_ok());
+        CHECK_NEAR(y_host[0], 528.0, 0.3);  // 1 + 2 + ... + 32, ones quantize to 127 * (1/127 in f16)
+        CHECK_NEAR(y_host[1], -8.0, 0.01);
+        DeviceWeights missing;
+        CHECK(m.load_quant_linear("blk.1.attn_q.weight", missing) == OXQ_ERR_GGUF_TENSOR_NOT_FOUND);
     });
 }
 

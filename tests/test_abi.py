@@ -13,19 +13,20 @@ from oxillama_amd import capi, quant
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "oxq.h")).read()
+def declared_symbols(header="oxq.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(oxq_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_header_and_binding_list_the_same_symbols():
     assert declared_symbols() == sorted(capi.SIGNATURES)
+    assert declared_symbols("oxq_gguf.h") == sorted(capi.GGUF_SIGNATURES)
 
 
 def test_library_exports_every_declared_symbol():
     lib = C.CDLL(capi.LIB_PATH)
-    for name in declared_symbols():
+    for name in declared_symbols() + declared_symbols("oxq_gguf.h"):
         assert hasattr(lib, name), name
 
 
