@@ -327,6 +327,17 @@ int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_ty
                        const uint8_t *d_acts_q8, float *d_out, size_t hidden, size_t intermediate,
                        void *d_workspace, size_t workspace_bytes, void *stream);
 
+/* The sampler's candidate list on the device: the k largest of n fp32 values (logits or
+ * probabilities), largest first, with their indices -- what the reference builds by sorting
+ * (index, value) pairs and truncating to top_k (crates/oxillama-runtime/src/sampling/mod.rs:
+ * 500-509); k = 1 is its argmax (mod.rs:652-662: the first of equal maxima).  Exactly equal values
+ * come out lower index first (the reference's unstable sort leaves that open); NaNs rank last.
+ * 1 <= k <= 256, k <= n <= 2^20.  Needs oxq_topk_workspace_bytes() bytes of 8-byte-aligned device
+ * scratch; two launches, no allocation, no synchronisation. */
+size_t oxq_topk_workspace_bytes(size_t n, size_t k);
+int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
+                 uint32_t *d_out_indices, void *d_workspace, size_t workspace_bytes, void *stream);
+
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                        int32_t *d_sums, size_t n_rows, size_t n_cols, void *stream);
 

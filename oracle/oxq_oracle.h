@@ -148,6 +148,11 @@ oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w,
                                       const float *input, size_t input_len, float *output,
                                       size_t output_len);
 
+/* argmax and the truncated, sorted candidate list of the sampler,
+ * crates/oxillama-runtime/src/sampling/mod.rs:500-509,652-662 */
+uint32_t oxq_ref_argmax(const float *values, size_t n);
+void oxq_ref_topk(const float *values, size_t n, size_t k, float *out_vals, uint32_t *out_idx);
+
 #ifdef __cplusplus
 }
 #endif

@@ -142,3 +142,45 @@ oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w,
     }
     return st(OXQ_REF_OK, 0, 0);
 }
+
+/* argmax, crates/oxillama-runtime/src/sampling/mod.rs:652-662: strict '>' from -inf, so the first of
+ * equal maxima wins (and index 0 when nothing exceeds -inf). */
+uint32_t oxq_ref_argmax(const float *values, size_t n) {
+    uint32_t max_idx = 0;
+    float max_val = -INFINITY;
+    for (size_t i = 0; i < n; i++) {
+        if (values[i] > max_val) {
+            max_val = values[i];
+            max_idx = (uint32_t)i;
+        }
+    }
+    return max_idx;
+}
+
+/* The sampler's candidate list, mod.rs:500-509: (index, value) pairs sorted by value, largest first,
+ * truncated to k.  The reference's sort_unstable_by leaves the order of equal values open; this
+ * restatement fixes it (lower index first) and ranks NaN last.  O(n k) selection, small inputs only. */
+void oxq_ref_topk(const float *values, size_t n, size_t k, float *out_vals, uint32_t *out_idx) {
+    unsigned char *taken = (unsigned char *)calloc(n ? n : 1, 1);
+    for (size_t r = 0; r < k && r < n; r++) {
+        size_t best = n;
+        for (size_t i = 0; i < n; i++) {
+            if (taken[i]) {
+                continue;
+            }
+            if (best == n) {
+                best = i;
+                continue;
+            }
+            float a = values[i], b = values[best];
+            int a_nan = a != a, b_nan = b != b;
+            if ((b_nan && !a_nan) || (!a_nan && !b_nan && a > b)) {
+                best = i;
+            }
+        }
+        taken[best] = 1;
+        out_vals[r] = values[best];
+        out_idx[r] = (uint32_t)best;
+    }
+    free(taken);
+}

@@ -960,6 +960,24 @@ int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_ty
     return OXQ_OK;
 }
 
+size_t oxq_topk_workspace_bytes(size_t n, size_t k) { return oxq::topk_workspace_bytes(n, k); }
+
+int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values, uint32_t *d_out_indices,
+                 void *d_workspace, size_t workspace_bytes, void *stream) {
+    if (k == 0 || k > n) return fail(OXQ_ERR_DIMENSION_MISMATCH, n, k, "k must be between 1 and the vector length");
+    const size_t need = oxq::topk_workspace_bytes(n, k);
+    if (need == 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, k, "k above 256 or more than 2^20 values");
+    if (!d_workspace || workspace_bytes < need)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, d_workspace ? workspace_bytes : 0, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(d_workspace) & 7)
+        return fail(OXQ_ERR_KERNEL, 8, reinterpret_cast<uintptr_t>(d_workspace) & 7, "workspace must be 8-byte aligned");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_topk(d_values, (uint32_t)n, (uint32_t)k, d_out_values, d_out_indices, d_workspace,
+                             (hipStream_t)stream));
+    return OXQ_OK;
+}
+
 // QuantLinear::forward on host slices (drop-in route: everything is staged per call).
 int oxq_linear_forward(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
                        const float *bias, size_t bias_len, const float *lora_a, size_t lora_a_len, const float *lora_b,

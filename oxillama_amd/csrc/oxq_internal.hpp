@@ -86,6 +86,11 @@ hipError_t launch_rmsnorm_quantize(const float *x, const float *weight, float ep
 hipError_t launch_lora_apply(const float *a, const float *b, float *r, uint32_t rank, float scale, const float *x,
                              float *out, uint32_t out_features, uint32_t in_features, hipStream_t stream);
 
+// Exact top-k (k <= 256, n <= 2^20) of an fp32 vector; workspace of topk_workspace_bytes(n, k) bytes (0: unsupported).
+size_t topk_workspace_bytes(size_t n, size_t k);
+hipError_t launch_topk(const float *x, uint32_t n, uint32_t k, float *out_vals, uint32_t *out_idx, void *workspace,
+                       hipStream_t stream);
+
 struct GemmArgs {
     const uint8_t *W;   // raw GGUF blocks [n x k]
     const uint8_t *A;   // Q8_0 blocks of the m activation rows, row-major, k/32 blocks per row

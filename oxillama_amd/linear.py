@@ -141,3 +141,14 @@ def ffn_swiglu_dev(gate, up, down, d_acts, d_out, hidden, intermediate, workspac
     _check(capi.load().oxq_ffn_swiglu_dev(int(gate[0]), gate[1].data_ptr(), int(up[0]), up[1].data_ptr(),
                                           int(down[0]), down[1].data_ptr(), d_acts.data_ptr(), d_out.data_ptr(),
                                           hidden, intermediate, workspace.data_ptr(), workspace.numel(), _stream()))
+
+
+def topk_dev(d_values, k, d_out_values, d_out_indices, workspace):
+    """The k largest of a float32 CUDA tensor, largest first, with their indices (uint32 viewed as int32)."""
+    lib = capi.load()
+    _check(lib.oxq_topk_dev(d_values.data_ptr(), d_values.numel(), k, d_out_values.data_ptr(), d_out_indices.data_ptr(),
+                            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream()))
+
+
+def topk_workspace_bytes(n, k):
+    return capi.load().oxq_topk_workspace_bytes(n, k)

@@ -123,6 +123,10 @@ def load():
         fn.argtypes = args
     lib.oxq_ref_swiglu_inplace.restype = None
     lib.oxq_ref_swiglu_inplace.argtypes = [vp, vp, sz]
+    lib.oxq_ref_argmax.restype = C.c_uint32
+    lib.oxq_ref_argmax.argtypes = [vp, sz]
+    lib.oxq_ref_topk.restype = None
+    lib.oxq_ref_topk.argtypes = [vp, sz, sz, vp, vp]
     lib.oxq_ref_rmsnorm_forward_to.restype = None
     lib.oxq_ref_rmsnorm_forward_to.argtypes = [vp, vp, C.c_float, sz, vp]
     _lib = lib
@@ -396,3 +400,15 @@ def random_blocks(t, seed, n_rows, n_cols, scale=0.02):
             v = np.abs(v)  # dmin is a magnitude in real files
         w[:, off:off + 2] = v.view(np.uint8).reshape(n_blocks, 2)
     return w.reshape(-1)
+
+
+def argmax(values):
+    v = np.ascontiguousarray(values, dtype=np.float32).ravel()
+    return int(load().oxq_ref_argmax(_p(v), v.size))
+
+
+def topk(values, k):
+    v = np.ascontiguousarray(values, dtype=np.float32).ravel()
+    vals, idx = np.zeros(k, dtype=np.float32), np.zeros(k, dtype=np.uint32)
+    load().oxq_ref_topk(_p(v), v.size, k, _p(vals), _p(idx))
+    return vals, idx

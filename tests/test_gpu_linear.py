@@ -343,3 +343,54 @@ def test_ffn_swiglu_errors(hip):
     assert e.value.needed == L.ffn_workspace_bytes(256, 512)
     with pytest.raises(hip.UnsupportedShape):
         L.ffn_swiglu_dev((O.Q4_K, z), (O.Q4_K, z), (O.Q6_K, z), z, z, 100, 512, z)
+
+
+# ---- top-k / argmax of the logits ------------------------------------------------------------------
+
+def test_topk_matches_oracle(hip, ref):
+    rng = np.random.default_rng(21)
+    for n, ks in ((128256, (1, 40, 256)), (1000, (1, 7, 256)), (5, (1, 5)), (300000, (2, 50)), (1 << 20, (1, 64))):
+        v = (rng.standard_normal(n) * 3).astype(np.float32)
+        if n > 2000:
+            v[1000:1010] = v[17]          # exact ties across and inside slices
+            v[5] = v.max()                # two equal maxima: the lower index wins
+            v[n - 1] = np.float32(np.inf)
+            v[n // 2] = np.float32(-np.inf)
+            v[123] = np.float32(np.nan)   # NaN ranks last
+        d_v = dev(v)
+        for k in ks:
+            say("topk n", n, "k", k)
+            ws = torch.empty(L.topk_workspace_bytes(n, k) // 8, dtype=torch.int64, device=DEV)
+            d_vals = torch.empty(k, dtype=torch.float32, device=DEV)
+            d_idx = torch.empty(k, dtype=torch.int32, device=DEV)
+            L.topk_dev(d_v, k, d_vals, d_idx, ws)
+            vals, idx = host(d_vals), host(d_idx).view(np.uint32)
+            if n <= 130000:  # the oracle's selection is O(n k)
+                want_vals, want_idx = ref.topk(v, k)
+            else:
+                key = np.where(np.isnan(v), -np.inf, v.astype(np.float64))
+                order = np.argsort(-key, kind="stable")[:k]
+                want_vals, want_idx = v[order], order.astype(np.uint32)
+            assert np.array_equal(idx, want_idx), f"indices differ at {np.nonzero(idx != want_idx)[0][:5]}"
+            assert np.array_equal(vals.view(np.uint32), want_vals.view(np.uint32))
+        v2 = np.where(np.isnan(v), np.float32(-np.inf), v)
+        ws = torch.empty(L.topk_workspace_bytes(n, 1) // 8, dtype=torch.int64, device=DEV)
+        d_vals, d_idx = torch.empty(1, dtype=torch.float32, device=DEV), torch.empty(1, dtype=torch.int32, device=DEV)
+        L.topk_dev(dev(v2), 1, d_vals, d_idx, ws)
+        assert int(host(d_idx)[0]) == ref.argmax(v2)  # k = 1 is the reference's argmax
+
+
+def test_topk_argument_errors(hip):
+    v = torch.zeros(64, dtype=torch.float32, device=DEV)
+    ws = torch.empty(4096, dtype=torch.int64, device=DEV)
+    out_v, out_i = torch.empty(300, dtype=torch.float32, device=DEV), torch.empty(300, dtype=torch.int32, device=DEV)
+    with pytest.raises(hip.DimensionMismatch):
+        L.topk_dev(v, 0, out_v, out_i, ws)
+    with pytest.raises(hip.DimensionMismatch):
+        L.topk_dev(v, 65, out_v, out_i, ws)
+    big = torch.zeros(1024, dtype=torch.float32, device=DEV)
+    with pytest.raises(hip.UnsupportedShape):
+        L.topk_dev(big, 257, out_v, out_i, ws)
+    with pytest.raises(hip.BufferTooSmall):
+        L.topk_dev(big, 16, out_v, out_i, ws[:1])
+    assert L.topk_workspace_bytes((1 << 20) + 1, 4) == 0

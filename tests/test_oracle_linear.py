@@ -156,3 +156,22 @@ def test_linear_forward_errors(ref):
     with pytest.raises(O.OracleError) as e:
         ref.linear_forward(O.Q8_0, w, 32, 32, np.zeros(32, dtype=np.float32), out_len=31)
     assert (e.value.code, e.value.a, e.value.b) == (O.DIMENSION_MISMATCH, 32, 31)
+
+
+def test_argmax_and_topk(ref):
+    # crates/oxillama-runtime/src/sampling/mod.rs:652-662: first of equal maxima; nothing above -inf -> 0
+    assert ref.argmax([1.0, 5.0, 5.0, 2.0]) == 1
+    assert ref.argmax([-np.inf, -np.inf]) == 0 and ref.argmax([]) == 0
+    assert ref.argmax([np.nan, 3.0, np.nan]) == 1  # comparisons with NaN are false
+    rng = np.random.default_rng(3)
+    v = rng.standard_normal(5000).astype(np.float32)
+    v[100:110] = v[7]  # exact ties
+    for k in (1, 2, 40, 256):
+        vals, idx = ref.topk(v, k)
+        order = np.argsort(-v.astype(np.float64), kind="stable")[:k]  # stable: lower index first among equals
+        assert np.array_equal(idx, order.astype(np.uint32)) and np.array_equal(vals, v[order])
+        assert np.all(vals[:-1] >= vals[1:])
+    assert ref.topk(v, 1)[1][0] == ref.argmax(v)
+    # mod.rs:500-509 on a hand-made list: sorted by value, truncated
+    vals, idx = ref.topk([0.1, 0.7, 0.05, 0.15], 2)
+    assert list(idx) == [1, 3] and list(vals) == [np.float32(0.7), np.float32(0.15)]
