@@ -34,7 +34,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per gate+up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # what the counter reads for a copy kernel of known size (2.000 and 1.000); the runs and figures are in
 # profiles/hbm_traffic_gemv_gate_up_lm_head_prefill_pmc.txt.  Algorithmic bytes are 66 179 328.
-MEASURED_TRAFFIC_GATE_UP = 66312806
+MEASURED_TRAFFIC_GATE_UP = 66318438
 INT8_PEAK_TOPS = 5000.0
 
 Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS = 2, 8, 12, 14, 23
