@@ -611,3 +611,53 @@ def test_registered_weights_and_cache(hip, ref):
     finally:
         lib.oxq_weight_cache_enable(0)
         lib.oxq_weight_cache_clear()
+
+
+# ---- concurrency and lifecycle ------------------------------------------------------------------
+
+def test_concurrent_host_calls_from_threads(hip, ref):
+    """The header promises thread safety: host-slice calls from several threads serialise on the library's
+    lock (they share its staging buffers) and each gets its own result."""
+    import threading
+    jobs = []
+    for i, t in enumerate((O.Q4_K, O.Q6_K, O.Q8_0, O.Q4_0, O.IQ4_XS, O.Q4_K)):
+        n_rows, n_cols = 64 + 32 * i, 1024
+        w = synth.weights(t, 700 + i, n_rows, n_cols)
+        x = synth.normal_f32(800 + i, n_cols)
+        jobs.append((t, w, x, n_rows, n_cols, ref.matvec_q8_fused(t, w, ref.quantize_q8_0(x), n_rows, n_cols)))
+    errors = []
+
+    def work(job):
+        t, w, x, n_rows, n_cols, want = job
+        try:
+            k = hip.HipKernel(t)
+            for _ in range(20):
+                y = np.zeros(n_rows, dtype=np.float32)
+                k.gemv(hip.QuantTensor(w, [n_rows, n_cols], t), x, y)
+                if np.abs(y - want).max() > FP32_REL_TOL * np.abs(want).max():
+                    errors.append((O.NAMES[t], float(np.abs(y - want).max())))
+                    return
+        except Exception as e:  # noqa: BLE001 - report any failure of a worker
+            errors.append((O.NAMES[t], repr(e)))
+
+    threads = [threading.Thread(target=work, args=(j,)) for j in jobs]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
+
+
+def test_shutdown_and_reinitialise(hip, ref):
+    lib = hip.capi.load()
+    w = synth.weights(O.Q4_K, 1, 32, 512)
+    x = synth.normal_f32(2, 512)
+    want = ref.matvec_q8_fused(O.Q4_K, w, ref.quantize_q8_0(x), 32, 512)
+    k = hip.HipKernel(O.Q4_K)
+    y = np.zeros(32, dtype=np.float32)
+    k.gemv(hip.QuantTensor(w, [32, 512], O.Q4_K), x, y)
+    assert lib.oxq_shutdown() == 0 and lib.oxq_shutdown() == 0  # idempotent; scratch and caches are released
+    y2 = np.zeros(32, dtype=np.float32)
+    k.gemv(hip.QuantTensor(w, [32, 512], O.Q4_K), x, y2)  # the next call initialises the device again
+    assert np.array_equal(y, y2) and np.abs(y - want).max() <= FP32_REL_TOL * np.abs(want).max()
+    hip.init(0)
