@@ -36,7 +36,8 @@ extern "C" {
 #define OXQ_TYPE_Q4_K 12u
 #define OXQ_TYPE_Q6_K 14u
 #define OXQ_TYPE_IQ4_XS 23u
-/* GEMV, dequant_block and the batched form by rows (no int8-MFMA tile kernel yet): */
+/* Further formats: GEMV and dequant_block for all of them; the int8-MFMA tile kernel (prefill, expert
+ * groups) for Q4_1, Q5_0, Q5_1, Q8_1, Q5_K, IQ4_NL; Q2_K and Q3_K run the batched form by rows. */
 #define OXQ_TYPE_Q4_1 3u
 #define OXQ_TYPE_Q5_0 6u
 #define OXQ_TYPE_Q5_1 7u
@@ -206,7 +207,7 @@ int oxq_gemv_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_wei
 
 /* Prefill / decode batch: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched
  * form of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  From 6 rows up
- * (9 where n < 8192), with k a multiple of 256, every format runs on the int8-MFMA tile
+ * (9 where n < 8192), with k a multiple of 256, every format but Q2_K / Q3_K runs on the int8-MFMA tile
  * kernel, which needs oxq_gemm_q8_workspace_bytes() bytes of 256-byte-aligned device scratch:
  * pass it and the call is asynchronous and allocation-free; pass NULL and the library uses
  * its own scratch (the call then serialises and waits for the stream).  Fewer rows, and
@@ -218,8 +219,8 @@ int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
                     void *d_workspace, size_t workspace_bytes, void *stream);
 /* Debug: as oxq_gemm_q8_dev (overwrite), and the exact int32 group sums of the tile
  * kernel, d_sums[(r * n + c) * groups + g], groups = k/32 (k/16 for Q6_K).  For Q4_0 the
- * tile kernel multiplies the unsigned nibbles (sum q*a); the "- 8" of (q - 8) enters in fp32.  OXQ_ERR_UNSUPPORTED_SHAPE when the shape
- * has no tile kernel. */
+ * (and Q5_0) the tile kernel multiplies the unsigned values (sum q*a); the "- 8" ("- 16") enters in
+ * fp32.  OXQ_ERR_UNSUPPORTED_SHAPE when the shape has no tile kernel. */
 int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                             float *d_out, int32_t *d_sums, size_t m, size_t n, size_t k,
                             void *d_workspace, size_t workspace_bytes, void *stream);

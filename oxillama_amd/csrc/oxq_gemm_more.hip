@@ -1,0 +1,191 @@
+// The int8-MFMA tile kernel (oxq_gemm_tile.hpp) instantiated for further formats: Q5_K, Q4_1, Q5_0,
+// Q5_1, Q8_1, IQ4_NL.  Each is a small policy (which bytes a lane fetches per group of two
+// sub-blocks, how they become int8 B operands, how the scale factors are decoded, which byte
+// order the activations need); kernel body, tile shapes and launch policy are shared.  A
+// translation unit of its own so that the two sets compile side by side; only the default tile
+// shapes are instantiated here.
+#define OXQ_TILE_DEFAULT_SHAPES_ONLY
+#include "oxq_formats_more.hpp"
+#include "oxq_gemm_tile.hpp"
+
+namespace oxq {
+
+// Q5_K (reference/q5_k.rs:27-102): 176 B = d, dmin, 12 B of 6-bit scales/mins, 32 B qh, 128 B
+// nibbles.  As Q4_K: the lane's 16 bytes qs[32g + 16h ..] carry weights 16h..16h+15 of sub-block 2g
+// (low nibbles) and 2g+1 (high); their fifth bits are bits g and g+4 of qh[16h ..].
+struct TileQ5K {
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q5_K, BLOCK_BYTES = 176;
+    static constexpr bool HAS_MIN = true;
+    static constexpr int ACT_PERM = 0, NQ = 2, KSPLIT = 1;
+    using Hdr = TileQ4K::Hdr;
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 48 + 32 * g);
+        qs[1] = buf16(rs, row_off + 16 * h, so_blk + 16);
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t s0,
+                                                    Hdr &hd) {
+        TileQ4K::load_hdr<SPL>(rs, row_off, so_blk, s0, hd);
+    }
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t e, uint32_t s, float (&dsc)[KSPLIT], float &qneg) {
+        TileQ4K::factors(hd, e, s, dsc, qneg);  // same header layout (reference/q5_k.rs:27-49)
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t g, BOperand<1> (&bop)[2]) {
+        for (int i = 0; i < 4; i++) {
+            const uint32_t hb = qs[1][i] >> g;
+            bop[0].k32[i] = (int)((qs[0][i] & 0x0F0F0F0Fu) | ((hb & 0x01010101u) << 4));
+            bop[1].k32[i] = (int)(((qs[0][i] >> 4) & 0x0F0F0F0Fu) | (hb & 0x10101010u));
+        }
+    }
+};
+
+// 32-weight blocks of interleaved nibbles (byte j = weights 2j, 2j+1), eight blocks per 256-weight
+// step: Q4_1 (reference/q4_1.rs:37-46: 20 B = d, m, 16 B; w = d * q + m, the "+ m" through the
+// zero-point term) and IQ4_NL (reference/iq4_nl.rs:43-51: 18 B = d, 16 B of codebook indices).
+template <uint32_t TYPE_ID, uint32_t STRIDE, uint32_t PAYLOAD, bool LUT, bool WITH_M>
+struct TileNibbles32 {
+    static constexpr uint32_t TYPE = TYPE_ID, BLOCK_BYTES = 8 * STRIDE;
+    static constexpr bool HAS_MIN = WITH_M;
+    static constexpr int ACT_PERM = 1, NQ = 1, KSPLIT = 1;
+    struct Hdr {
+        uint32_t d[8], m[8];  // f16 bits of the lane's sub-blocks
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        if constexpr ((STRIDE + 2) % 4 == 0 && PAYLOAD % 4 == 2)  // half 0 starts 2 past a dword boundary, half 1 on one
+            qs[0] = buf16_shift(rs, row_off + (STRIDE + 2) * h, so_blk + 2 * STRIDE * g + PAYLOAD - 2, h ? 0u : 16u);
+        else
+            qs[0] = buf16(rs, row_off + STRIDE * h, so_blk + 2 * STRIDE * g + PAYLOAD);  // block 2g + h
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t s0,
+                                                    Hdr &hd) {
+#pragma unroll
+        for (int e = 0; e < SPL; e++) {
+            hd.d[e] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row_off + STRIDE * (s0 + e), so_blk, 0);
+            if (WITH_M)
+                hd.m[e] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row_off + STRIDE * (s0 + e) + 2, so_blk, 0);
+        }
+    }
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t e, uint32_t, float (&dsc)[KSPLIT], float &qneg) {
+        dsc[0] = h2f(hd.d[e]);
+        qneg = WITH_M ? h2f(hd.m[e]) : 0.0f;
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t, BOperand<1> (&bop)[2]) {
+        uint32_t x[2][2];
+        halves_to_pieces(qs[0], x);
+        for (int e = 0; e < 2; e++)
+            for (int i = 0; i < 2; i++) {
+                const uint32_t lo = x[e][i] & 0x0F0F0F0Fu, hi = (x[e][i] >> 4) & 0x0F0F0F0Fu;
+                bop[e].k32[2 * i] = (int)(LUT ? FmtIQ4XS::lut4(lo) : lo);
+                bop[e].k32[2 * i + 1] = (int)(LUT ? FmtIQ4XS::lut4(hi) : hi);
+            }
+    }
+};
+using TileQ4_1 = TileNibbles32<OXQ_TYPE_Q4_1, 20, 4, false, true>;
+using TileIQ4NL = TileNibbles32<OXQ_TYPE_IQ4_NL, 18, 2, true, false>;
+
+// Q8_1 (reference/q8_1.rs:36-42): 36 B = d, s (unused), 32 int8; the payload is the B operand.
+struct TileQ8_1 {
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q8_1, BLOCK_BYTES = 8 * 36;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int ACT_PERM = 0, NQ = 2, KSPLIT = 1;
+    using Hdr = TileQ8_0::Hdr;
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 72 * g + 4);
+        qs[1] = buf16(rs, row_off + 16 * h, so_blk + 72 * g + 40);
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t s0,
+                                                    Hdr &hd) {
+#pragma unroll
+        for (int e = 0; e < SPL; e++)
+            hd.d[e] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row_off + 36 * (s0 + e), so_blk, 0);
+    }
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t e, uint32_t, float (&dsc)[KSPLIT], float &qneg) {
+        dsc[0] = h2f(hd.d[e]);
+        qneg = 0.0f;
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t, BOperand<1> (&bop)[2]) {
+        for (int e = 0; e < 2; e++)
+            for (int i = 0; i < 4; i++) bop[e].k32[i] = (int)qs[e][i];
+    }
+};
+
+// Q5_0 / Q5_1 (reference/q5_0.rs:39-55, q5_1.rs:38-56): d [, m], u32 qh, 16 B of nibbles; byte j holds
+// the low four bits of weights j (low nibble) and j + 16 (high nibble), bit j / j + 16 of qh the
+// fifth.  Lane half h fetches block 2g + h whole; after the exchange every lane holds bytes
+// 8h..8h+7 of both blocks, i.e. weights {8h..8h+7, 16+8h..23+8h}: the k-slot order the preparation
+// kernel stores under ACT_PERM = 2.  Q5_0's "- 16" and Q5_1's "+ m" go through the zero-point term.
+template <uint32_t TYPE_ID, uint32_t STRIDE, bool WITH_M>
+struct TileQ5x {
+    static constexpr uint32_t TYPE = TYPE_ID, BLOCK_BYTES = 8 * STRIDE;
+    static constexpr uint32_t QH = WITH_M ? 4 : 2, PAYLOAD = QH + 4;
+    static constexpr bool HAS_MIN = true;
+    static constexpr int ACT_PERM = 2, NQ = 2, KSPLIT = 1;
+    using Hdr = typename TileNibbles32<TYPE_ID, STRIDE, PAYLOAD, false, WITH_M>::Hdr;
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        if constexpr ((STRIDE + 2) % 4 == 0 && PAYLOAD % 4 == 2)  // Q5_0: half 0 starts 2 past a dword boundary, half 1 on one
+            qs[0] = buf16_shift(rs, row_off + (STRIDE + 2) * h, so_blk + 2 * STRIDE * g + PAYLOAD - 2, h ? 0u : 16u);
+        else
+            qs[0] = buf16(rs, row_off + STRIDE * h, so_blk + 2 * STRIDE * g + PAYLOAD);  // block 2g + h: nibbles
+        qs[1] = u32x4{(uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, row_off + STRIDE * h, so_blk + 2 * STRIDE * g + QH, 0),
+                      0, 0, 0};                                                          // and its qh
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t s0,
+                                                    Hdr &hd) {
+        TileNibbles32<TYPE_ID, STRIDE, PAYLOAD, false, WITH_M>::template load_hdr<SPL>(rs, row_off, so_blk, s0, hd);
+    }
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t e, uint32_t, float (&dsc)[KSPLIT], float &qneg) {
+        dsc[0] = h2f(hd.d[e]);
+        qneg = WITH_M ? h2f(hd.m[e]) : -(16.0f * dsc[0]);  // exact
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t, BOperand<1> (&bop)[2]) {
+        uint32_t x[2][2];
+        halves_to_pieces(qs[0], x);
+        // qh of block 2g in every lane (s[0]) and of block 2g + 1 (s[1])
+        const auto s = __builtin_amdgcn_permlane32_swap(qs[1][0], qs[1][0], false, false);
+        const uint32_t hsel = (__lane_id() >> 5) * 8;  // this half's byte of the low / high 16 fifth bits
+        for (int e = 0; e < 2; e++) {
+            const uint32_t lo8 = ((uint32_t)s[e] >> hsel) & 0xFFu, hi8 = ((uint32_t)s[e] >> (16 + hsel)) & 0xFFu;
+            bop[e].k32[0] = (int)((x[e][0] & 0x0F0F0F0Fu) | (spread4(lo8 & 0xFu) << 4));
+            bop[e].k32[1] = (int)((x[e][1] & 0x0F0F0F0Fu) | (spread4(lo8 >> 4) << 4));
+            bop[e].k32[2] = (int)(((x[e][0] >> 4) & 0x0F0F0F0Fu) | (spread4(hi8 & 0xFu) << 4));
+            bop[e].k32[3] = (int)(((x[e][1] >> 4) & 0x0F0F0F0Fu) | (spread4(hi8 >> 4) << 4));
+        }
+    }
+};
+using TileQ5_0 = TileQ5x<OXQ_TYPE_Q5_0, 22, false>;
+using TileQ5_1 = TileQ5x<OXQ_TYPE_Q5_1, 24, true>;
+
+int tile_act_perm_more(uint32_t type) {
+    switch (type) {
+    case OXQ_TYPE_Q4_1:
+    case OXQ_TYPE_IQ4_NL: return 1;
+    case OXQ_TYPE_Q5_0:
+    case OXQ_TYPE_Q5_1: return 2;
+    default: return 0;
+    }
+}
+
+hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream) {
+    switch (type) {
+    case OXQ_TYPE_Q5_K: return launch_tiles<TileQ5K>(a, plan, stream);
+    case OXQ_TYPE_Q4_1: return launch_tiles<TileQ4_1>(a, plan, stream);
+    case OXQ_TYPE_IQ4_NL: return launch_tiles<TileIQ4NL>(a, plan, stream);
+    case OXQ_TYPE_Q8_1: return launch_tiles<TileQ8_1>(a, plan, stream);
+    case OXQ_TYPE_Q5_0: return launch_tiles<TileQ5_0>(a, plan, stream);
+    case OXQ_TYPE_Q5_1: return launch_tiles<TileQ5_1>(a, plan, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace oxq

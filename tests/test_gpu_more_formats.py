@@ -17,6 +17,7 @@ pytestmark = pytest.mark.gpu
 FP32_REL_TOL = 1e-5
 DEV = "cuda:0"
 TYPES = O.MORE_TYPES
+TILE_TYPES = [O.Q5_K, O.Q4_1, O.Q5_0, O.Q5_1, O.Q8_1, O.IQ4_NL]
 ids = lambda t: O.NAMES[t]
 
 
@@ -61,7 +62,8 @@ KAT_VALUES = {O.Q4_1: [10.0, 5.0], O.Q5_0: [15.0, -32.0, None], O.Q5_1: [31.0, 3
 def test_metadata_and_dispatch(hip, t):
     k = hip.KernelDispatcher().get_kernel(t)
     assert (k.block_size(), k.block_bytes(), k.name()) == (*O.BLOCK[t], O.NAMES[t])
-    assert k.gemm_workspace_bytes(64, 4096, 4096) == 0  # no tile kernel: the batched form runs by rows
+    # the int8-MFMA tile kernel takes six of them; Q2_K and Q3_K run the batched form by rows
+    assert (k.gemm_workspace_bytes(64, 4096, 4096) > 0) == (t in TILE_TYPES)
 
 
 def test_unknown_types_still_rejected(hip):
@@ -140,7 +142,10 @@ def test_gemv_gemm_host_route(hip, ref, t):
         for r in range(m):
             yr = np.zeros(n, dtype=np.float32)
             k.gemv(qt, xs[r * kk:(r + 1) * kk], yr)
-            assert np.array_equal(ys[r * n:(r + 1) * n], yr), f"gemm row {r} of {m}"
+            if m >= 9 and t in TILE_TYPES:  # the tile kernel adds the groups in another order
+                assert_close(ys[r * n:(r + 1) * n], yr, f"gemm row {r} of {m}")
+            else:
+                assert np.array_equal(ys[r * n:(r + 1) * n], yr), f"gemm row {r} of {m}"
         assert_close(ys, ref.gemm_q8(t, w, xs, m, n, kk).ravel(), f"gemm {m}")
     with pytest.raises(hip.DimensionMismatch) as e:
         k.gemv(qt, x[:-1], y)
@@ -191,7 +196,78 @@ def test_device_route_forms(hip, ref, t):
 
 def test_grouped_form_reports_unsupported(hip):
     z = torch.zeros(4096, dtype=torch.uint8, device=DEV)
-    k = hip.HipKernel(O.Q5_K)
+    k = hip.HipKernel(O.Q2_K)
     assert k.moe_gemm_workspace_bytes(64, 256, 256) == 0
     with pytest.raises(hip.UnsupportedShape):
-        k.moe_gemm_q8_dev(z, 256 * 176, 1, z, z, 4, 4, z, 256, 256, z)
+        k.moe_gemm_q8_dev(z, 256 * 84, 1, z, z, 4, 4, z, 256, 256, z)
+
+
+def _tile_zero_point(t, acts, rows, k_):
+    """Q5_0's tile policy multiplies the unsigned 5-bit values and applies the "- 16" in fp32 through the
+    zero-point term, so its integer sums are sum q5*a = sum (q5 - 16)*a + 16 * sum a."""
+    if t != O.Q5_0:
+        return 0
+    a = acts.reshape(rows, k_ // 32, 34)[:, :, 2:].view(np.int8).astype(np.int32).sum(axis=2)
+    return (16 * a)[:, None, :]
+
+
+@pytest.mark.parametrize("shape", [(8, 32, 256), (40, 100, 1024), (130, 129, 2048), (200, 257, 1024), (512, 160, 512)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("t", TILE_TYPES, ids=ids)
+def test_prefill_tile_kernel(hip, ref, shape, t):
+    """The int8-MFMA tile kernel on the added formats: integer sub-block sums bit-exact, fp32 within 1e-5 of
+    the reference's fused kernel, every tile shape (split k, 64 x 128, 128 x 64), ragged edges, accumulate."""
+    from oxillama_amd import capi
+    m, n, k_ = shape
+    say("prefill", O.NAMES[t], shape)
+    capi.load().oxq_set_gemm_tile_min_rows(1)
+    try:
+        w = O.random_blocks(t, 900 + m, n, k_)
+        x = synth.normal_f32(950 + n, m * k_)
+        acts = ref.quantize_q8_0(x)
+        kern = hip.HipKernel(t)
+        ws_bytes = kern.gemm_workspace_bytes(m, n, k_)
+        assert ws_bytes > 0
+        dw, da = dev(w), dev(acts)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=DEV)
+        dy = torch.full((m, n), 7.0, dtype=torch.float32, device=DEV)
+        kern.gemm_q8_dev(dw, da, dy, m, n, k_, accumulate=False, workspace=ws)
+        arb = k_ // 32 * 34
+        y_ref = np.stack([ref.matvec_q8_fused_mt(t, w, acts[r * arb:(r + 1) * arb], n, k_, 16) for r in range(m)])
+        assert_close(host(dy), y_ref, f"prefill {O.NAMES[t]} {shape}")
+        dy2 = dy.clone()
+        kern.gemm_q8_dev(dw, da, dy2, m, n, k_, accumulate=True, workspace=None)
+        torch.cuda.synchronize()
+        assert torch.equal(dy2, dy + dy)
+        dsum = torch.empty((m, n, k_ // 32), dtype=torch.int32, device=DEV)
+        dy3 = torch.empty_like(dy)
+        kern.gemm_block_sums_dev(dw, da, dy3, dsum, m, n, k_, workspace=ws)
+        want = np.stack([ref.block_sums(t, w, acts[r * arb:(r + 1) * arb], n, k_) for r in range(m)])
+        assert np.array_equal(host(dsum) - _tile_zero_point(t, acts, m, k_), want), "integer sub-block sums"
+        assert torch.equal(dy3, dy)
+    finally:
+        capi.load().oxq_set_gemm_tile_min_rows(0)
+
+
+@pytest.mark.parametrize("t", [O.Q5_K, O.Q5_0, O.IQ4_NL], ids=ids)
+def test_grouped_expert_matmul(hip, ref, t):
+    """Grouped (mixture-of-experts) form on added formats: each expert's rows against its own weights."""
+    n_exp, n, k_ = 4, 96, 512
+    rows = [5, 0, 33, 17]
+    total = sum(rows)
+    offsets = np.concatenate([[0], np.cumsum(rows)]).astype(np.int32)
+    bs, bb = O.BLOCK[t]
+    stride = n * (k_ // bs) * bb
+    w = O.random_blocks(t, 77, n_exp * n, k_)
+    x = synth.normal_f32(78, total * k_)
+    acts = ref.quantize_q8_0(x)
+    kern = hip.HipKernel(t)
+    ws = torch.empty(kern.moe_gemm_workspace_bytes(total, n, k_), dtype=torch.uint8, device=DEV)
+    dy = torch.zeros((total, n), dtype=torch.float32, device=DEV)
+    kern.moe_gemm_q8_dev(dev(w), stride, n_exp, dev(acts), dev(offsets), total, max(rows), dy, n, k_, ws)
+    got = host(dy)
+    arb = k_ // 32 * 34
+    for e in range(n_exp):
+        for r in range(offsets[e], offsets[e + 1]):
+            want = ref.matvec_q8_fused(t, w[e * stride:(e + 1) * stride], acts[r * arb:(r + 1) * arb], n, k_)
+            assert_close(got[r], want, f"expert {e} row {r}")
