@@ -328,6 +328,53 @@ int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_ty
                        const uint8_t *d_acts_q8, float *d_out, size_t hidden, size_t intermediate,
                        void *d_workspace, size_t workspace_bytes, void *stream);
 
+/* MoeFfn::forward (crates/oxillama-arch/src/common/moe.rs:184-258) for n_tokens tokens at once, the
+ * experts' gate / up / down matrices in quantized formats (one format per projection, as in
+ * oxq_ffn_swiglu_dev).
+ *
+ * oxq_moe_route_dev: steps 1-4 (moe.rs:189-250) for every token and the grouping of the (token,
+ * expert) pairs by expert.  Logits of the fp32 router [n_experts x hidden] against d_x [n_tokens
+ * x hidden], stable softmax, the k = min(top_k, n_experts) experts of largest weight in
+ * descending order (the lower index first among equal weights, which the reference's
+ * sort_unstable_by leaves open), weights renormalised over the selected ones.  Outputs:
+ * d_experts, d_weights [n_tokens x k]; d_row_offsets [n_experts + 1] (grouped rows of expert e:
+ * offsets[e] .. offsets[e+1]-1); d_pair_token [n_tokens * k] (the token of grouped row r);
+ * d_token_rows [n_tokens x k] (the grouped row of each token's j-th choice).  Rows of an expert
+ * are in ascending (token, choice) order: the tables do not depend on scheduling.  top_k == 0
+ * is KernelError (the reference's InvalidConfig, moe.rs:168-172).
+ *
+ * oxq_moe_gather_quantize_q8_0_dev: grouped activation row r = the Q8_0 blocks of
+ * d_x[d_pair_token[r]] (every selected expert reads the token's own input, moe.rs:252).
+ *
+ * oxq_moe_combine_dev: d_out[t] = sum over j < top_k, in that order from 0.0, of d_weights[t][j]
+ * * d_y_pairs[d_token_rows[t][j]] (moe.rs:240-256: product and sum rounded separately).
+ *
+ * oxq_moe_ffn_dev: the whole layer after routing -- gather + quantize, grouped gate and up
+ * matmuls (oxq_moe_gemm_q8_dev), SwiGLU + quantize, grouped down matmul, combine.  top_k is the
+ * width of the tables (the clamped k); max_rows_per_expert as in oxq_moe_gemm_q8_dev (0:
+ * unknown, e.g. tables made on the device).  Expert e's matrices sit at d_gate + e *
+ * gate_stride_bytes, etc.  No allocation, no synchronisation; needs
+ * oxq_moe_ffn_workspace_bytes() bytes of 256-byte-aligned scratch (0: no grouped kernel for a
+ * type / shape). */
+int oxq_moe_route_dev(const float *d_router, const float *d_x, size_t n_tokens, size_t n_experts,
+                      size_t hidden, size_t top_k, int32_t *d_experts, float *d_weights,
+                      int32_t *d_row_offsets, int32_t *d_pair_token, int32_t *d_token_rows,
+                      void *stream);
+int oxq_moe_gather_quantize_q8_0_dev(const float *d_x, const int32_t *d_pair_token, size_t n_pairs,
+                                     size_t hidden, uint8_t *d_out_q8, void *stream);
+int oxq_moe_combine_dev(const float *d_y_pairs, const int32_t *d_token_rows, const float *d_weights,
+                        size_t n_tokens, size_t top_k, size_t hidden, float *d_out, void *stream);
+size_t oxq_moe_ffn_workspace_bytes(uint32_t gate_type, uint32_t up_type, uint32_t down_type,
+                                   size_t n_pairs, size_t hidden, size_t intermediate);
+int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_bytes,
+                    uint32_t up_type, const uint8_t *d_up, size_t up_stride_bytes,
+                    uint32_t down_type, const uint8_t *d_down, size_t down_stride_bytes,
+                    size_t n_experts, const float *d_x, size_t n_tokens, size_t top_k,
+                    const int32_t *d_row_offsets, const int32_t *d_pair_token,
+                    const int32_t *d_token_rows, const float *d_weights,
+                    size_t max_rows_per_expert, float *d_out, size_t hidden, size_t intermediate,
+                    void *d_workspace, size_t workspace_bytes, void *stream);
+
 /* The sampler's candidate list on the device: the k largest of n fp32 values (logits or
  * probabilities), largest first, with their indices -- what the reference builds by sorting
  * (index, value) pairs and truncating to top_k (crates/oxillama-runtime/src/sampling/mod.rs:

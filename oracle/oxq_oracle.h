@@ -153,6 +153,31 @@ oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w,
 uint32_t oxq_ref_argmax(const float *values, size_t n);
 void oxq_ref_topk(const float *values, size_t n, size_t k, float *out_vals, uint32_t *out_idx);
 
+/* ---- mixture-of-experts feed-forward (oxq_oracle_moe.c), crates/oxillama-arch/src/common/moe.rs ---- */
+
+/* Expert::forward, moe.rs:75-127 (dense fp32) */
+oxq_ref_status oxq_ref_expert_forward(const float *gate, size_t gate_len, const float *up, size_t up_len,
+                                      const float *down, size_t down_len, size_t hidden, size_t inter,
+                                      const float *input, float *output);
+/* routing of MoeFfn::forward, moe.rs:189-250; outputs hold min(top_k, n_exp) entries */
+oxq_ref_status oxq_ref_moe_route(const float *router, size_t router_len, size_t n_exp, size_t hidden,
+                                 size_t top_k, const float *input, uint32_t *experts_out, float *weights_out,
+                                 size_t *k_out);
+/* output[i] += weight * expert_out[i], moe.rs:254-256 */
+void oxq_ref_moe_accumulate(float *output, const float *expert_out, float weight, size_t n);
+/* MoeFfn::forward, moe.rs:184-258, dense experts stored back to back */
+oxq_ref_status oxq_ref_moe_forward(const float *router, size_t router_len, const float *gate_all,
+                                   const float *up_all, const float *down_all, size_t n_exp, size_t hidden,
+                                   size_t inter, size_t top_k, const float *input, float *output);
+/* the same with the experts' projections in a block format, through matvec_q8_fused */
+oxq_ref_status oxq_ref_expert_forward_q(uint32_t type, int tier, const uint8_t *gate, const uint8_t *up,
+                                        const uint8_t *down, size_t hidden, size_t inter,
+                                        const uint8_t *input_q8, float *output);
+oxq_ref_status oxq_ref_moe_forward_q(uint32_t type, int tier, const float *router, size_t router_len,
+                                     const uint8_t *gate_all, const uint8_t *up_all, const uint8_t *down_all,
+                                     size_t n_exp, size_t hidden, size_t inter, size_t top_k, const float *input,
+                                     float *output, uint32_t *sel_out, float *wt_out);
+
 #ifdef __cplusplus
 }
 #endif

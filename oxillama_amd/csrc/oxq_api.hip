@@ -960,6 +960,129 @@ int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_ty
     return OXQ_OK;
 }
 
+// ---- MoeFfn::forward on the device, experts in a quantized format ----
+
+namespace {
+struct MoeFfnLayout {
+    size_t acts, gate, up, hq, y, gemm, total;
+};
+size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+bool moe_ffn_layout(uint32_t gate_type, uint32_t up_type, uint32_t down_type, size_t pairs, size_t hidden, size_t inter,
+                    MoeFfnLayout *l) {
+    const size_t g1 = oxq_moe_gemm_q8_workspace_bytes(gate_type, pairs, inter, hidden);
+    const size_t g2 = oxq_moe_gemm_q8_workspace_bytes(up_type, pairs, inter, hidden);
+    const size_t g3 = oxq_moe_gemm_q8_workspace_bytes(down_type, pairs, hidden, inter);
+    if (g1 == 0 || g2 == 0 || g3 == 0 || hidden % 32 || inter % 32) return false;
+    size_t off = 0;
+    l->acts = off; off += align256(pairs * (hidden / 32) * 34);
+    l->gate = off; off += align256(pairs * inter * sizeof(float));
+    l->up = off; off += align256(pairs * inter * sizeof(float));
+    l->hq = off; off += align256(pairs * (inter / 32) * 34);
+    l->y = off; off += align256(pairs * hidden * sizeof(float));
+    l->gemm = off; off += align256(g1 > g2 ? (g1 > g3 ? g1 : g3) : (g2 > g3 ? g2 : g3));
+    l->total = off;
+    return true;
+}
+}  // namespace
+
+int oxq_moe_route_dev(const float *d_router, const float *d_x, size_t n_tokens, size_t n_experts, size_t hidden,
+                      size_t top_k, int32_t *d_experts, float *d_weights, int32_t *d_row_offsets,
+                      int32_t *d_pair_token, int32_t *d_token_rows, void *stream) {
+    if (top_k == 0) return fail(OXQ_ERR_KERNEL, 1, 0, "MoeFfn top_k must be >= 1");  // moe.rs:168-172
+    if (n_experts > 4096) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 4096, n_experts, "at most 4096 experts");
+    const size_t k = top_k < n_experts ? top_k : n_experts;  // moe.rs:233
+    if (n_tokens * k > 0x7FFFFFFFull || hidden > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0x7FFFFFFFull, n_tokens * k, "too many (token, expert) pairs");
+    int st;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (n_tokens == 0 || n_experts == 0) return OXQ_OK;
+    if (!d_router || !d_x || !d_experts || !d_weights || !d_row_offsets || !d_pair_token || !d_token_rows)
+        return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer");
+    OXQ_HIP(oxq::launch_moe_route(d_router, d_x, d_experts, d_weights, (uint32_t)n_tokens, (uint32_t)n_experts,
+                                  (uint32_t)hidden, (uint32_t)k, d_row_offsets, d_pair_token, d_token_rows,
+                                  (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_moe_gather_quantize_q8_0_dev(const float *d_x, const int32_t *d_pair_token, size_t n_pairs, size_t hidden,
+                                     uint8_t *d_out_q8, void *stream) {
+    if (hidden % 32) return fail(OXQ_ERR_DIMENSION_MISMATCH, 32, hidden, "row length must be a multiple of 32");
+    if (n_pairs > 0x7FFFFFFFull || hidden > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0x7FFFFFFFull, n_pairs, "too many rows");
+    int st;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (n_pairs == 0 || hidden == 0) return OXQ_OK;
+    OXQ_HIP(oxq::launch_moe_gather_quantize(d_x, d_pair_token, d_out_q8, n_pairs, (uint32_t)hidden, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_moe_combine_dev(const float *d_y_pairs, const int32_t *d_token_rows, const float *d_weights, size_t n_tokens,
+                        size_t top_k, size_t hidden, float *d_out, void *stream) {
+    if (n_tokens * top_k > 0x7FFFFFFFull || hidden > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0x7FFFFFFFull, n_tokens * top_k, "too many rows");
+    int st;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (n_tokens == 0 || hidden == 0) return OXQ_OK;
+    OXQ_HIP(oxq::launch_moe_combine(d_y_pairs, d_token_rows, d_weights, d_out, (uint32_t)n_tokens, (uint32_t)top_k,
+                                    (uint32_t)hidden, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+size_t oxq_moe_ffn_workspace_bytes(uint32_t gate_type, uint32_t up_type, uint32_t down_type, size_t n_pairs,
+                                   size_t hidden, size_t intermediate) {
+    MoeFfnLayout l;
+    return moe_ffn_layout(gate_type, up_type, down_type, n_pairs, hidden, intermediate, &l) ? l.total : 0;
+}
+
+int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_bytes, uint32_t up_type,
+                    const uint8_t *d_up, size_t up_stride_bytes, uint32_t down_type, const uint8_t *d_down,
+                    size_t down_stride_bytes, size_t n_experts, const float *d_x, size_t n_tokens, size_t top_k,
+                    const int32_t *d_row_offsets, const int32_t *d_pair_token, const int32_t *d_token_rows,
+                    const float *d_weights, size_t max_rows_per_expert, float *d_out, size_t hidden,
+                    size_t intermediate, void *d_workspace, size_t workspace_bytes, void *stream) {
+    int st;
+    if ((st = check_dev_shape(gate_type, intermediate, hidden)) != OXQ_OK) return st;
+    if ((st = check_dev_shape(up_type, intermediate, hidden)) != OXQ_OK) return st;
+    if ((st = check_dev_shape(down_type, hidden, intermediate)) != OXQ_OK) return st;
+    if (top_k == 0) return fail(OXQ_ERR_KERNEL, 1, 0, "MoeFfn top_k must be >= 1");  // moe.rs:168-172
+    const size_t pairs = n_tokens * top_k;
+    if (pairs > 0x7FFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0x7FFFFFFFull, pairs, "too many rows");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (pairs == 0 || n_experts == 0 || hidden == 0 || intermediate == 0) return OXQ_OK;
+    if (!d_row_offsets || !d_pair_token || !d_token_rows || !d_weights)
+        return fail(OXQ_ERR_INTERNAL, 0, 0, "null routing table");
+    MoeFfnLayout l;
+    if (!moe_ffn_layout(gate_type, up_type, down_type, pairs, hidden, intermediate, &l))
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, hidden, "no grouped kernel for this type/shape");
+    if (!d_workspace || workspace_bytes < l.total)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, l.total, d_workspace ? workspace_bytes : 0, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
+        return fail(OXQ_ERR_KERNEL, 256, reinterpret_cast<uintptr_t>(d_workspace) & 255,
+                    "workspace must be 256-byte aligned");
+    uint8_t *ws = (uint8_t *)d_workspace;
+    uint8_t *acts = ws + l.acts, *hq = ws + l.hq;
+    float *gate = (float *)(ws + l.gate), *up = (float *)(ws + l.up), *y = (float *)(ws + l.y);
+    hipStream_t s = (hipStream_t)stream;
+    OXQ_HIP(oxq::launch_moe_gather_quantize(d_x, d_pair_token, acts, pairs, (uint32_t)hidden, s));
+    const size_t gws = workspace_bytes - l.gemm;
+    if ((st = oxq_moe_gemm_q8_dev(gate_type, d_gate, gate_stride_bytes, n_experts, acts, d_row_offsets, pairs,
+                                  max_rows_per_expert, gate, nullptr, intermediate, hidden, 0, ws + l.gemm, gws,
+                                  stream)) != OXQ_OK)
+        return st;
+    if ((st = oxq_moe_gemm_q8_dev(up_type, d_up, up_stride_bytes, n_experts, acts, d_row_offsets, pairs,
+                                  max_rows_per_expert, up, nullptr, intermediate, hidden, 0, ws + l.gemm, gws,
+                                  stream)) != OXQ_OK)
+        return st;
+    OXQ_HIP(oxq::launch_swiglu_quantize(gate, up, pairs * intermediate, nullptr, hq, s));
+    if ((st = oxq_moe_gemm_q8_dev(down_type, d_down, down_stride_bytes, n_experts, hq, d_row_offsets, pairs,
+                                  max_rows_per_expert, y, nullptr, hidden, intermediate, 0, ws + l.gemm, gws,
+                                  stream)) != OXQ_OK)
+        return st;
+    OXQ_HIP(oxq::launch_moe_combine(y, d_token_rows, d_weights, d_out, (uint32_t)n_tokens, (uint32_t)top_k,
+                                    (uint32_t)hidden, s));
+    return OXQ_OK;
+}
+
 size_t oxq_topk_workspace_bytes(size_t n, size_t k) { return oxq::topk_workspace_bytes(n, k); }
 
 int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values, uint32_t *d_out_indices,

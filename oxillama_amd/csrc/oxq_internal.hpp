@@ -86,6 +86,18 @@ hipError_t launch_rmsnorm_quantize(const float *x, const float *weight, float ep
 hipError_t launch_lora_apply(const float *a, const float *b, float *r, uint32_t rank, float scale, const float *x,
                              float *out, uint32_t out_features, uint32_t in_features, hipStream_t stream);
 
+// Mixture-of-experts glue: grouped activation rows from the tokens' fp32 inputs; weighted combine of the
+// selected experts' outputs per token, in selection order.
+hipError_t launch_moe_gather_quantize(const float *x, const int32_t *pair_token, uint8_t *out, size_t n_pairs,
+                                      uint32_t hidden, hipStream_t stream);
+hipError_t launch_moe_combine(const float *y_pairs, const int32_t *token_rows, const float *weights, float *out,
+                              uint32_t n_tokens, uint32_t top_k, uint32_t hidden, hipStream_t stream);
+
+// Router of the mixture-of-experts layer and the grouping of its (token, expert) pairs; k <= n_exp.
+hipError_t launch_moe_route(const float *router, const float *x, int32_t *experts, float *weights, uint32_t n_tokens,
+                            uint32_t n_exp, uint32_t hidden, uint32_t k, int32_t *offsets, int32_t *pair_token,
+                            int32_t *token_rows, hipStream_t stream);
+
 // Exact top-k (k <= 256, n <= 2^20) of an fp32 vector; workspace of topk_workspace_bytes(n, k) bytes (0: unsupported).
 size_t topk_workspace_bytes(size_t n, size_t k);
 hipError_t launch_topk(const float *x, uint32_t n, uint32_t k, float *out_vals, uint32_t *out_idx, void *workspace,

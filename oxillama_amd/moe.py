@@ -38,3 +38,55 @@ def group_by_expert(experts, n_experts):
     offsets = np.zeros(n_experts + 1, dtype=np.int32)
     offsets[1:] = np.cumsum(counts)
     return offsets, (order // k).astype(np.int32), (order % k).astype(np.int32)
+
+
+def token_rows(offsets, token, slot, n_tokens, k):
+    """Inverse of the grouping: int32 [n_tokens, k], the grouped row of each token's j-th choice."""
+    rows = np.zeros((n_tokens, k), dtype=np.int32)
+    rows[token, slot] = np.arange(token.size, dtype=np.int32)
+    return rows
+
+
+def route_dev(d_router, d_x, n_tokens, n_experts, hidden, top_k, d_experts, d_weights, d_offsets, d_pair_token,
+              d_token_rows):
+    """Steps 1-4 of MoeFfn::forward (moe.rs:189-250) and the grouping, on torch CUDA tensors."""
+    from . import capi
+    from .quant import HipKernel, _check
+    _check(capi.load().oxq_moe_route_dev(d_router.data_ptr(), d_x.data_ptr(), n_tokens, n_experts, hidden, top_k,
+                                         d_experts.data_ptr(), d_weights.data_ptr(), d_offsets.data_ptr(),
+                                         d_pair_token.data_ptr(), d_token_rows.data_ptr(), HipKernel._stream()))
+
+
+def gather_quantize_dev(d_x, d_pair_token, n_pairs, hidden, d_out_q8):
+    from . import capi
+    from .quant import HipKernel, _check
+    _check(capi.load().oxq_moe_gather_quantize_q8_0_dev(d_x.data_ptr(), d_pair_token.data_ptr(), n_pairs, hidden,
+                                                        d_out_q8.data_ptr(), HipKernel._stream()))
+
+
+def combine_dev(d_y_pairs, d_token_rows, d_weights, n_tokens, top_k, hidden, d_out):
+    from . import capi
+    from .quant import HipKernel, _check
+    _check(capi.load().oxq_moe_combine_dev(d_y_pairs.data_ptr(), d_token_rows.data_ptr(), d_weights.data_ptr(),
+                                           n_tokens, top_k, hidden, d_out.data_ptr(), HipKernel._stream()))
+
+
+def moe_ffn_workspace_bytes(types, n_pairs, hidden, intermediate):
+    from . import capi
+    tg, tu, td = (int(t) for t in types)
+    return capi.load().oxq_moe_ffn_workspace_bytes(tg, tu, td, n_pairs, hidden, intermediate)
+
+
+def moe_ffn_dev(gate, up, down, n_experts, d_x, n_tokens, top_k, d_offsets, d_pair_token, d_token_rows, d_weights,
+                max_rows, d_out, hidden, intermediate, workspace):
+    """MoeFfn::forward (moe.rs:184-258) after routing, for n_tokens tokens on torch CUDA tensors, current
+    stream.  gate / up / down: (tensor_type, device tensor of all experts, bytes per expert)."""
+    from . import capi
+    from .quant import HipKernel, _check
+    args = []
+    for t, d_w, stride in (gate, up, down):
+        args += [int(t), d_w.data_ptr(), stride]
+    _check(capi.load().oxq_moe_ffn_dev(*args, n_experts, d_x.data_ptr(), n_tokens, top_k, d_offsets.data_ptr(),
+                                       d_pair_token.data_ptr(), d_token_rows.data_ptr(), d_weights.data_ptr(),
+                                       max_rows, d_out.data_ptr(), hidden, intermediate, workspace.data_ptr(),
+                                       workspace.numel(), HipKernel._stream()))

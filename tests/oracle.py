@@ -117,12 +117,19 @@ def load():
         "oxq_ref_lora_new": [sz, sz, sz, sz, sz],
         "oxq_ref_lora_apply": [vp, vp, sz, C.c_float, sz, sz, vp, sz, vp, sz],
         "oxq_ref_linear_forward": [u32, C.c_int, vp, sz, sz, sz, vp, sz, vp, vp, sz, C.c_float, vp, sz, vp, sz],
+        "oxq_ref_expert_forward": [vp, sz, vp, sz, vp, sz, sz, sz, vp, vp],
+        "oxq_ref_moe_route": [vp, sz, sz, sz, sz, vp, vp, vp, vp],
+        "oxq_ref_moe_forward": [vp, sz, vp, vp, vp, sz, sz, sz, sz, vp, vp],
+        "oxq_ref_expert_forward_q": [u32, C.c_int, vp, vp, vp, sz, sz, vp, vp],
+        "oxq_ref_moe_forward_q": [u32, C.c_int, vp, sz, vp, vp, vp, sz, sz, sz, sz, vp, vp, vp, vp],
     }.items():
         fn = getattr(lib, name)
         fn.restype = Status
         fn.argtypes = args
     lib.oxq_ref_swiglu_inplace.restype = None
     lib.oxq_ref_swiglu_inplace.argtypes = [vp, vp, sz]
+    lib.oxq_ref_moe_accumulate.restype = None
+    lib.oxq_ref_moe_accumulate.argtypes = [vp, vp, C.c_float, sz]
     lib.oxq_ref_argmax.restype = C.c_uint32
     lib.oxq_ref_argmax.argtypes = [vp, sz]
     lib.oxq_ref_topk.restype = None
@@ -412,3 +419,60 @@ def topk(values, k):
     vals, idx = np.zeros(k, dtype=np.float32), np.zeros(k, dtype=np.uint32)
     load().oxq_ref_topk(_p(v), v.size, k, _p(vals), _p(idx))
     return vals, idx
+
+
+# ---- mixture-of-experts feed-forward (oracle/oxq_oracle_moe.c) ----
+
+def _f32(a):
+    return np.ascontiguousarray(a, dtype=np.float32).ravel()
+
+
+def expert_forward(gate, up, down, hidden, inter, x):
+    gate, up, down, x = _f32(gate), _f32(up), _f32(down), _f32(x)
+    out = np.zeros(hidden, dtype=np.float32)
+    _chk(load().oxq_ref_expert_forward(_p(gate), gate.size, _p(up), up.size, _p(down), down.size, hidden, inter,
+                                       _p(x), _p(out)))
+    return out
+
+
+def moe_route(router, n_exp, hidden, top_k, x):
+    """-> (experts uint32 [k], weights float32 [k]) with k = min(top_k, n_exp)."""
+    router, x = _f32(router), _f32(x)
+    sel = np.zeros(max(n_exp, 1), dtype=np.uint32)
+    wt = np.zeros(max(n_exp, 1), dtype=np.float32)
+    k = C.c_size_t(0)
+    _chk(load().oxq_ref_moe_route(_p(router), router.size, n_exp, hidden, top_k, _p(x), _p(sel), _p(wt),
+                                  C.cast(C.byref(k), C.c_void_p)))
+    return sel[:k.value].copy(), wt[:k.value].copy()
+
+
+def moe_forward(router, gate_all, up_all, down_all, n_exp, hidden, inter, top_k, x):
+    router, x = _f32(router), _f32(x)
+    g, u, d = _f32(gate_all), _f32(up_all), _f32(down_all)
+    assert g.size == u.size == d.size == n_exp * hidden * inter
+    out = np.zeros(hidden, dtype=np.float32)
+    _chk(load().oxq_ref_moe_forward(_p(router), router.size, _p(g), _p(u), _p(d), n_exp, hidden, inter, top_k,
+                                    _p(x), _p(out)))
+    return out
+
+
+def expert_forward_q(t, gate, up, down, hidden, inter, x_q8, tier=TIER_AVX2):
+    gate, up, down, x_q8 = _u8(gate), _u8(up), _u8(down), _u8(x_q8)
+    assert gate.size == up.size == row_bytes(t, hidden) * inter and down.size == row_bytes(t, inter) * hidden
+    out = np.zeros(hidden, dtype=np.float32)
+    _chk(load().oxq_ref_expert_forward_q(t, tier, _p(gate), _p(up), _p(down), hidden, inter, _p(x_q8), _p(out)))
+    return out
+
+
+def moe_forward_q(t, router, gate_all, up_all, down_all, n_exp, hidden, inter, top_k, x, tier=TIER_AVX2):
+    """-> (output float32 [hidden], experts uint32 [k], weights float32 [k])."""
+    router, x = _f32(router), _f32(x)
+    g, u, d = _u8(gate_all), _u8(up_all), _u8(down_all)
+    assert g.size == u.size == n_exp * row_bytes(t, hidden) * inter and d.size == n_exp * row_bytes(t, inter) * hidden
+    out = np.zeros(hidden, dtype=np.float32)
+    k = min(top_k, n_exp)
+    sel = np.zeros(max(k, 1), dtype=np.uint32)
+    wt = np.zeros(max(k, 1), dtype=np.float32)
+    _chk(load().oxq_ref_moe_forward_q(t, tier, _p(router), router.size, _p(g), _p(u), _p(d), n_exp, hidden, inter,
+                                      top_k, _p(x), _p(out), _p(sel), _p(wt)))
+    return out, sel[:k], wt[:k]
