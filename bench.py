@@ -323,38 +323,32 @@ def main():
     if not args.no_moe:
         from oxillama_amd import moe
         E, NTOK, TOPK = 8, 64, 2
-        k_iq = quant.HipKernel(IQ4_XS)
-        rng = np.random.default_rng(5)
-        experts, _ = moe.route_top_k(rng.random((NTOK, E), dtype=np.float32), TOPK)
-        offsets, tok, _slot = moe.group_by_expert(experts, E)
-        rows, max_rows = int(offsets[-1]), int(np.diff(offsets).max())
 
         def expert_set(seed, n_rows, n_cols):
             return torch.from_numpy(np.stack([synth.weights(IQ4_XS, seed + e, n_rows, n_cols) for e in range(E)])).to(dev)
         wg, wu, wd = expert_set(7000, F, H), expert_set(7100, F, H), expert_set(7200, H, F)
         stride = wg[0].numel()
-        xt = torch.from_numpy(synth.normal_f32(7, NTOK * H)).to(dev).reshape(NTOK, H)
-        xp = xt[torch.from_numpy(tok.astype(np.int64)).to(dev)].contiguous()      # one row per (token, expert) pair
-        hp = torch.from_numpy(synth.normal_f32(8, rows * F)).to(dev)
-        xpq = torch.empty(rows * (H // 32 * 34), dtype=torch.uint8, device=dev)
-        hpq = torch.empty(rows * (F // 32 * 34), dtype=torch.uint8, device=dev)
-        doff = torch.from_numpy(offsets).to(dev)
-        og = torch.zeros(rows * F, dtype=torch.float32, device=dev)
-        ou = torch.zeros(rows * F, dtype=torch.float32, device=dev)
-        od = torch.zeros(rows * H, dtype=torch.float32, device=dev)
-        wsm = torch.empty(max(k_iq.moe_gemm_workspace_bytes(rows, F, H), k_iq.moe_gemm_workspace_bytes(rows, H, F)),
-                          dtype=torch.uint8, device=dev)
+        xt = torch.from_numpy(synth.normal_f32(7, NTOK * H)).to(dev)
+        router = torch.from_numpy(synth.normal_f32(9, E * H, 0.05)).to(dev)
+        rows = NTOK * TOPK
+        d_exp = torch.empty(rows, dtype=torch.int32, device=dev)
+        d_wt = torch.empty(rows, dtype=torch.float32, device=dev)
+        d_off = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        d_tok = torch.empty(rows, dtype=torch.int32, device=dev)
+        d_rows = torch.empty(rows, dtype=torch.int32, device=dev)
+        d_y = torch.empty(NTOK * H, dtype=torch.float32, device=dev)
+        types3 = (IQ4_XS, IQ4_XS, IQ4_XS)
+        wsm = torch.empty(moe.moe_ffn_workspace_bytes(types3, rows, H, F), dtype=torch.uint8, device=dev)
 
         def moe_step():
-            quant.quantize_q8_0_dev(xp, xpq)
-            k_iq.moe_gemm_q8_dev(wg, stride, E, xpq, doff, rows, max_rows, og, F, H, wsm)
-            k_iq.moe_gemm_q8_dev(wu, stride, E, xpq, doff, rows, max_rows, ou, F, H, wsm)
-            quant.quantize_q8_0_dev(hp, hpq)
-            k_iq.moe_gemm_q8_dev(wd, stride, E, hpq, doff, rows, max_rows, od, H, F, wsm)
+            moe.route_dev(router, xt, NTOK, E, H, TOPK, d_exp, d_wt, d_off, d_tok, d_rows)
+            moe.moe_ffn_dev((IQ4_XS, wg, stride), (IQ4_XS, wu, stride), (IQ4_XS, wd, stride), E, xt, NTOK, TOPK, d_off,
+                            d_tok, d_rows, d_wt, 0, d_y, H, F, wsm)
 
         with torch.cuda.stream(stream):
             moe_step()
             stream.synchronize()
+            offsets = d_off.cpu().numpy()
             reps = 6
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
@@ -366,13 +360,14 @@ def main():
         moe_bytes = 3 * E * stride
         moe_ops = 2 * rows * 3 * F * H
         moe_out = {"workload": "IQ4_XS, 8 experts x (gate, up 14336x4096; down 4096x14336), 64 tokens, top-2 "
-                               "(seeded uniform logits), pairs grouped per expert",
+                               "(seeded fp32 router), pairs grouped per expert on the device",
                    "pairs": rows, "rows_per_expert": np.diff(offsets).tolist(), "us_per_step": round(moe_us, 1),
                    "weight_bytes": moe_bytes, "weight_GBps": round(moe_bytes / moe_us / 1e3, 1),
                    "frac_hbm_peak": round(moe_bytes / moe_us / 1e3 / HBM_PEAK_GBPS, 4),
                    "int8_TOPS": round(moe_ops / moe_us / 1e6, 1),
-                   "timed": "2 activation quantizations + 3 grouped int8-MFMA matmuls (the 749 MB of expert weights "
-                            "exceed the 256 MB Infinity Cache, so every step streams them from HBM)"}
+                   "timed": "the whole layer: router + softmax + top-2 + grouping, gather + quantize, 3 grouped int8-MFMA "
+                            "matmuls, SwiGLU + quantize, weighted combine (the 749 MB of expert weights exceed the "
+                            "256 MB Infinity Cache, so every step streams them from HBM)"}
         del wg, wu, wd
 
     # ---- CPU baseline: the reference's fused rows restated in C, same layer -------------

@@ -816,6 +816,13 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
     ga.n_experts = (uint32_t)n_experts;
     ga.max_rows = (uint32_t)(max_rows_per_expert ? (max_rows_per_expert < total_rows ? max_rows_per_expert : total_rows)
                                                  : total_rows);
+    ga.shape_rows = ga.max_rows;
+    if (!max_rows_per_expert) {
+        // Row counts known only on the device: the grid covers the worst case (one expert takes every
+        // row; tiles past an expert's rows exit at once), the tile shape is chosen for twice the mean.
+        const size_t mean = (total_rows + n_experts - 1) / n_experts;
+        ga.shape_rows = (uint32_t)(2 * mean < total_rows ? 2 * mean : total_rows);
+    }
     ga.w_stride = expert_stride_bytes;
     OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
     return OXQ_OK;

@@ -403,9 +403,14 @@ __device__ __forceinline__ void gemm_tile_body(
     const uint32_t blk_begin = SPLITK ? wave * nblk / 4 : 0, blk_end = SPLITK ? (wave + 1) * nblk / 4 : nblk;
 
     const uint32_t xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
-    const uint32_t n_tile = (loc / m_tiles) * 8 + xcd, m_tile = loc % m_tiles;
+    uint32_t n_tile = (loc / m_tiles) * 8 + xcd, m_tile = loc % m_tiles;
     uint32_t row0 = 0, row_end = m;
     if (offsets) {
+        // expert groups: token tiles outermost, so that the tiles past an expert's rows (the grid is
+        // sized for the largest group) form one run at the end instead of sitting between live ones
+        const uint32_t n_groups = (n_tiles + 7) / 8;
+        m_tile = loc / n_groups;
+        n_tile = (loc % n_groups) * 8 + xcd;
         row0 = (uint32_t)offsets[blockIdx.y];
         row_end = (uint32_t)offsets[blockIdx.y + 1];
         W += (size_t)blockIdx.y * w_stride;
@@ -719,7 +724,7 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
 // weight bytes fetched further ahead, because that case is paced by the weight stream.
 template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
-    const uint32_t rows = a.offsets ? a.max_rows : a.m;
+    const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
     if (a.sums)  // debug dump: the same tile layout (and fp32 summation order) as the production choice below
         return rows > 384  ? launch_tile<F, 2, 1, 2, 1, true>(a, p, stream)
                : rows > 64 ? launch_tile<F, 2, 1, 1, 2, true>(a, p, stream)

@@ -116,7 +116,8 @@ struct GemmArgs {
     // offsets[e+1]-1 by the weights at W + e * w_stride.  offsets == null: plain matmul.
     const int32_t *offsets = nullptr;  // device memory, n_experts + 1 entries
     uint32_t n_experts = 0;
-    uint32_t max_rows = 0;             // upper bound of the rows of any one expert
+    uint32_t max_rows = 0;             // upper bound of the rows of any one expert (sizes the grid)
+    uint32_t shape_rows = 0;           // rows per expert the tile shape is chosen for (<= max_rows)
     size_t w_stride = 0;
 };
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);

@@ -13,68 +13,89 @@
 
 namespace oxq {
 
-// One work group per token.  Wave w forms the logits of experts w, w+4, ... (lane-strided dot
-// product, wave sum); lane 0 of wave 0 then runs the softmax and the selection serially in the
-// reference's order (moe.rs:201-250): max, exp(l - max), sum in ascending expert order, divide;
-// k times the largest remaining weight, the lower index on ties; weights divided by the sum of
-// the selected ones (1/k when that sum is <= 1e-9).  n_exp floats of dynamic LDS.
+// One work group per token.  The 256 lanes form the logits together (16-byte loads, lane, wave and
+// work-group sums); wave 0 then runs the softmax and the selection (moe.rs:201-250): max,
+// exp(l - max), sum, divide; k rounds of "largest remaining weight, lower index on ties" as one
+// 64-bit wave maximum over keys (weight bits, complemented index); weights divided by the sum of
+// the selected ones in selection order (1/k when that sum is <= 1e-9).  Lane l owns experts l,
+// l + 64, ... in LDS.  5 * n_exp floats of dynamic LDS.
 __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict__ router, const float *__restrict__ x,
                                                        int32_t *__restrict__ experts, float *__restrict__ weights,
                                                        uint32_t n_exp, uint32_t hidden, uint32_t k) {
-    extern __shared__ float probs[];
+    extern __shared__ float lds[];
+    float *probs = lds, *part = lds + n_exp;
     const uint32_t t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const float *xr = x + (size_t)t * hidden;
-    for (uint32_t e = wave; e < n_exp; e += 4) {
-        const float *rr = router + (size_t)e * hidden;
-        float acc = 0.0f;
-        for (uint32_t c = lane; c < hidden; c += 64) acc += rr[c] * xr[c];
-        acc = wave_sum(acc);
-        if (lane == 0) probs[e] = acc;
+    const uint32_t n4 = (hidden & 3) == 0 ? hidden / 4 : 0;
+    for (uint32_t e0 = 0; e0 < n_exp; e0 += 4) {  // four experts per pass: their loads are in flight together
+        const float *rr[4];
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int q = 0; q < 4; q++) rr[q] = router + (size_t)min(e0 + q, n_exp - 1) * hidden;
+        if (n4) {
+            for (uint32_t c = threadIdx.x; c < n4; c += 256) {
+                float xv[4], rv[4][4];
+                load4(xv, xr + 4 * c);
+#pragma unroll
+                for (int q = 0; q < 4; q++) load4(rv[q], rr[q] + 4 * c);
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+                    for (int i = 0; i < 4; i++) acc[q] += rv[q][i] * xv[i];
+            }
+        } else {
+            for (uint32_t c = threadIdx.x; c < hidden; c += 256)
+                for (int q = 0; q < 4; q++) acc[q] += rr[q][c] * xr[c];
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const float v = wave_sum(acc[q]);
+            if (lane == 0 && e0 + q < n_exp) part[4 * (e0 + q) + wave] = v;
+        }
     }
     __syncthreads();
-    if (threadIdx.x != 0) return;
-    float max_logit = -INFINITY;
-    for (uint32_t e = 0; e < n_exp; e++) max_logit = fmaxf(max_logit, probs[e]);
-    float exp_sum = 0.0f;
-    for (uint32_t e = 0; e < n_exp; e++) {
+    for (uint32_t e = threadIdx.x; e < n_exp; e += 256)
+        probs[e] = (part[4 * e] + part[4 * e + 1]) + (part[4 * e + 2] + part[4 * e + 3]);
+    __syncthreads();
+    if (wave != 0) return;
+
+    float m = -INFINITY;
+    for (uint32_t e = lane; e < n_exp; e += 64) m = fmaxf(m, probs[e]);
+    m = fmaxf(m, dpp_f<0xB1>(m));
+    m = fmaxf(m, dpp_f<0x4E>(m));
+    m = fmaxf(m, dpp_f<0x124>(m));
+    m = fmaxf(m, dpp_f<0x128>(m));
+    const float max_logit = fmaxf(fmaxf(readlane_f(m, 0), readlane_f(m, 16)), fmaxf(readlane_f(m, 32), readlane_f(m, 48)));
+    float s = 0.0f;
+    for (uint32_t e = lane; e < n_exp; e += 64) {
         const float v = expf(probs[e] - max_logit);
         probs[e] = v;
-        exp_sum += v;
+        s += v;
     }
-    if (exp_sum > 0.0f) {
-        for (uint32_t e = 0; e < n_exp; e++) probs[e] /= exp_sum;
-    } else {
-        const float uniform = 1.0f / (float)n_exp;
-        for (uint32_t e = 0; e < n_exp; e++) probs[e] = uniform;
-    }
+    const float exp_sum = wave_sum(s);
+    const float uniform = 1.0f / (float)n_exp;
+    for (uint32_t e = lane; e < n_exp; e += 64) probs[e] = exp_sum > 0.0f ? probs[e] / exp_sum : uniform;
+
     int32_t *sel = experts + (size_t)t * k;
     float *wt = weights + (size_t)t * k;
     float selected_sum = 0.0f;
     for (uint32_t r = 0; r < k; r++) {
-        uint32_t best = 0;
-        float best_v = -1.0f;  // weights are >= 0; taken entries are marked -2
-        for (uint32_t e = 0; e < n_exp; e++) {
-            const float v = probs[e];
-            if (v > best_v) {
-                best_v = v;
-                best = e;
-            }
+        uint64_t best = 0;
+        for (uint32_t e = lane; e < n_exp; e += 64) {
+            const float v = probs[e];  // >= 0 (or NaN, which ranks first and is taken once); taken entries are -1
+            const uint64_t key = v < 0.0f ? 0 : ((uint64_t)__builtin_bit_cast(uint32_t, v) << 32) | (0xFFFFFFFFu - e);
+            best = max_u64(best, key);
         }
-        // NaN weights (a NaN logit) never compare greater: fall back to the first untaken expert
-        if (best_v < 0.0f) {
-            for (uint32_t e = 0; e < n_exp; e++)
-                if (probs[e] != -2.0f) {
-                    best = e;
-                    best_v = probs[e];
-                    break;
-                }
+        best = wave_max_u64(best);
+        const uint32_t e = 0xFFFFFFFFu - (uint32_t)best;
+        const float v = __builtin_bit_cast(float, (uint32_t)(best >> 32));
+        if ((e & 63) == lane) probs[e] = -1.0f;  // the owner lane is the only one that reads it again
+        selected_sum += v;
+        if (lane == 0) {
+            sel[r] = (int32_t)e;
+            wt[r] = v;
         }
-        probs[best] = -2.0f;
-        sel[r] = (int32_t)best;
-        wt[r] = best_v;
-        selected_sum += best_v;
     }
-    for (uint32_t r = 0; r < k; r++) wt[r] = selected_sum > 1e-9f ? wt[r] / selected_sum : 1.0f / (float)k;
+    if (lane == 0)
+        for (uint32_t r = 0; r < k; r++) wt[r] = selected_sum > 1e-9f ? wt[r] / selected_sum : 1.0f / (float)k;
 }
 
 // One work group per expert e.  Pass 1 counts the pairs routed to experts below e (the first
@@ -181,7 +202,7 @@ hipError_t launch_moe_route(const float *router, const float *x, int32_t *expert
                             uint32_t n_exp, uint32_t hidden, uint32_t k, int32_t *offsets, int32_t *pair_token,
                             int32_t *token_rows, hipStream_t stream) {
     if (n_tokens == 0 || n_exp == 0) return hipSuccess;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(256), n_exp * sizeof(float), stream, router, x, experts,
+    hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(256), 5 * n_exp * sizeof(float), stream, router, x, experts,
                        weights, n_exp, hidden, k);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
