@@ -375,6 +375,20 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
                     size_t max_rows_per_expert, float *d_out, size_t hidden, size_t intermediate,
                     void *d_workspace, size_t workspace_bytes, void *stream);
 
+/* MoeFfn::forward on host slices, for n_tokens input vectors at once (n_tokens = 1 is the
+ * reference's call): experts' matrices as raw blocks, expert after expert (gate_len = n_experts *
+ * bytes of one [intermediate x hidden] matrix, etc.), fp32 router [n_experts x hidden].  Checks
+ * in the reference's order (moe.rs:151-173: router size, top_k; moe.rs:33-58: gate, up, down
+ * sizes) as DimensionMismatch {expected, got} / KernelError; hidden and intermediate must be
+ * multiples of 256 (UnsupportedShape otherwise).  Stages everything to the device (weights
+ * through the weight cache when it is on), runs oxq_moe_route_dev + oxq_moe_ffn_dev, copies the
+ * output back. */
+int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, uint32_t up_type,
+                    const uint8_t *up, size_t up_len, uint32_t down_type, const uint8_t *down,
+                    size_t down_len, const float *router, size_t router_len, size_t n_experts,
+                    size_t hidden, size_t intermediate, size_t top_k, const float *input,
+                    size_t input_len, float *output, size_t output_len, size_t n_tokens);
+
 /* The sampler's candidate list on the device: the k largest of n fp32 values (logits or
  * probabilities), largest first, with their indices -- what the reference builds by sorting
  * (index, value) pairs and truncating to top_k (crates/oxillama-runtime/src/sampling/mod.rs:

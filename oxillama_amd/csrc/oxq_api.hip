@@ -94,6 +94,7 @@ struct State {
     bool cache_enabled = false;
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
     Scratch s_weights, s_acts, s_x, s_out, s_sums, s_work, s_bias, s_lora_a, s_lora_b, s_lora_r;
+    Scratch s_moe_up, s_moe_down, s_moe_tables;
 };
 State g;
 
@@ -264,6 +265,9 @@ int oxq_shutdown(void) {
     g.s_lora_a.release();
     g.s_lora_b.release();
     g.s_lora_r.release();
+    g.s_moe_up.release();
+    g.s_moe_down.release();
+    g.s_moe_tables.release();
     oxq::gguf_release_staging();
     g.initialised = false;
     g.device = -1;
@@ -1087,6 +1091,85 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
         return st;
     OXQ_HIP(oxq::launch_moe_combine(y, d_token_rows, d_weights, d_out, (uint32_t)n_tokens, (uint32_t)top_k,
                                     (uint32_t)hidden, s));
+    return OXQ_OK;
+}
+
+// MoeFfn::forward on host slices (the drop-in route): everything is staged to the device, the layer
+// runs there, the output comes back.  Validation in the reference's order (moe.rs:151-173, 33-58).
+int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, uint32_t up_type, const uint8_t *up,
+                    size_t up_len, uint32_t down_type, const uint8_t *down, size_t down_len, const float *router,
+                    size_t router_len, size_t n_experts, size_t hidden, size_t intermediate, size_t top_k,
+                    const float *input, size_t input_len, float *output, size_t output_len, size_t n_tokens) {
+    if (!known_type(gate_type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, gate_type, 0, "unsupported quantization type");
+    if (!known_type(up_type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, up_type, 0, "unsupported quantization type");
+    if (!known_type(down_type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, down_type, 0, "unsupported quantization type");
+    if (router_len != n_experts * hidden)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, n_experts * hidden, router_len, "moe.router has the wrong size");
+    if (top_k == 0) return fail(OXQ_ERR_KERNEL, 1, 0, "MoeFfn top_k must be >= 1");
+    auto mat_bytes = [](uint32_t t, size_t rows, size_t cols) {
+        const size_t bs = oxq_block_size(t);
+        return rows * ((cols + bs - 1) / bs) * oxq_block_bytes(t);
+    };
+    const size_t g_one = mat_bytes(gate_type, intermediate, hidden), u_one = mat_bytes(up_type, intermediate, hidden);
+    const size_t d_one = mat_bytes(down_type, hidden, intermediate);
+    if (gate_len != n_experts * g_one)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, n_experts * g_one, gate_len, "expert.gate has the wrong size");
+    if (up_len != n_experts * u_one)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, n_experts * u_one, up_len, "expert.up has the wrong size");
+    if (down_len != n_experts * d_one)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, n_experts * d_one, down_len, "expert.down has the wrong size");
+    if (input_len < n_tokens * hidden)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, n_tokens * hidden, input_len, "input shorter than n_tokens * hidden");
+    if (output_len < n_tokens * hidden)
+        return fail(OXQ_ERR_DIMENSION_MISMATCH, n_tokens * hidden, output_len, "output shorter than n_tokens * hidden");
+    if (n_tokens == 0 || hidden == 0) return OXQ_OK;
+    if (n_experts == 0 || intermediate == 0) {  // no expert to add: the zeroed output (moe.rs:240-242)
+        std::memset(output, 0, n_tokens * hidden * sizeof(float));
+        return OXQ_OK;
+    }
+    const size_t k = top_k < n_experts ? top_k : n_experts, pairs = n_tokens * k;
+    const size_t ws_bytes = oxq_moe_ffn_workspace_bytes(gate_type, up_type, down_type, pairs, hidden, intermediate);
+    if (ws_bytes == 0)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, hidden % 256 ? hidden : intermediate,
+                    "no grouped kernel for this type/shape (dimensions must be multiples of 256)");
+    int st;
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    std::lock_guard<std::mutex> lock(g.mu);
+    const uint8_t *dg = nullptr, *du = nullptr, *dd = nullptr;
+    auto stage = [&](Scratch &slot, uint32_t t, const uint8_t *host, size_t len, const uint8_t **dev) -> int {
+        if (g.cache_enabled) return stage_weights(t, host, len, dev);
+        int r = slot.reserve(len);
+        if (r != OXQ_OK) return r;
+        OXQ_HIP(hipMemcpy(slot.ptr, host, len, hipMemcpyHostToDevice));
+        *dev = (const uint8_t *)slot.ptr;
+        return OXQ_OK;
+    };
+    if ((st = stage(g.s_weights, gate_type, gate, gate_len, &dg)) != OXQ_OK) return st;
+    if ((st = stage(g.s_moe_up, up_type, up, up_len, &du)) != OXQ_OK) return st;
+    if ((st = stage(g.s_moe_down, down_type, down, down_len, &dd)) != OXQ_OK) return st;
+    // tables: router | experts | weights | offsets | pair_token | token_rows, each 256-byte aligned
+    size_t off = 0;
+    auto take = [&](size_t bytes) { const size_t at = off; off += align256(bytes); return at; };
+    const size_t o_router = take(router_len * sizeof(float)), o_exp = take(pairs * 4), o_wt = take(pairs * 4);
+    const size_t o_off = take((n_experts + 1) * 4), o_tok = take(pairs * 4), o_rows = take(pairs * 4);
+    if ((st = g.s_moe_tables.reserve(off)) != OXQ_OK) return st;
+    if ((st = g.s_x.reserve(n_tokens * hidden * sizeof(float))) != OXQ_OK) return st;
+    if ((st = g.s_out.reserve(n_tokens * hidden * sizeof(float))) != OXQ_OK) return st;
+    if ((st = g.s_work.reserve(ws_bytes + 256)) != OXQ_OK) return st;
+    uint8_t *tb = (uint8_t *)g.s_moe_tables.ptr;
+    uint8_t *ws = (uint8_t *)((reinterpret_cast<uintptr_t>(g.s_work.ptr) + 255) & ~(uintptr_t)255);
+    OXQ_HIP(hipMemcpy(tb + o_router, router, router_len * sizeof(float), hipMemcpyHostToDevice));
+    OXQ_HIP(hipMemcpy(g.s_x.ptr, input, n_tokens * hidden * sizeof(float), hipMemcpyHostToDevice));
+    if ((st = oxq_moe_route_dev((const float *)(tb + o_router), (const float *)g.s_x.ptr, n_tokens, n_experts, hidden,
+                                top_k, (int32_t *)(tb + o_exp), (float *)(tb + o_wt), (int32_t *)(tb + o_off),
+                                (int32_t *)(tb + o_tok), (int32_t *)(tb + o_rows), nullptr)) != OXQ_OK)
+        return st;
+    if ((st = oxq_moe_ffn_dev(gate_type, dg, g_one, up_type, du, u_one, down_type, dd, d_one, n_experts,
+                              (const float *)g.s_x.ptr, n_tokens, k, (const int32_t *)(tb + o_off),
+                              (const int32_t *)(tb + o_tok), (const int32_t *)(tb + o_rows), (const float *)(tb + o_wt), 0,
+                              (float *)g.s_out.ptr, hidden, intermediate, ws, ws_bytes, nullptr)) != OXQ_OK)
+        return st;
+    OXQ_HIP(hipMemcpy(output, g.s_out.ptr, n_tokens * hidden * sizeof(float), hipMemcpyDeviceToHost));
     return OXQ_OK;
 }
 

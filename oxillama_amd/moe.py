@@ -90,3 +90,37 @@ def moe_ffn_dev(gate, up, down, n_experts, d_x, n_tokens, top_k, d_offsets, d_pa
                                        d_pair_token.data_ptr(), d_token_rows.data_ptr(), d_weights.data_ptr(),
                                        max_rows, d_out.data_ptr(), hidden, intermediate, workspace.data_ptr(),
                                        workspace.numel(), HipKernel._stream()))
+
+
+class MoeFfn:
+    """MoeFfn of the reference (moe.rs:129-258) with the experts' projections as GGUF blocks.
+
+    gate / up / down: (tensor_type, uint8 array holding the matrices of all experts back to back).
+    forward() takes one input vector like the reference's; forward_batch() takes n_tokens of them.
+    Errors are the QuantError classes of oxillama_amd.quant (InvalidShape -> DimensionMismatch,
+    InvalidConfig -> KernelError)."""
+
+    def __init__(self, router, gate, up, down, top_k, num_experts, hidden_size, intermediate_size):
+        self.router = np.ascontiguousarray(router, dtype=np.float32).ravel()
+        self.gate, self.up, self.down = ((int(t), np.ascontiguousarray(w).view(np.uint8).ravel())
+                                         for t, w in (gate, up, down))
+        self.top_k, self.num_experts = top_k, num_experts
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+
+    def forward(self, x, out=None):
+        return self.forward_batch(x, 1, out)
+
+    def forward_batch(self, x, n_tokens, out=None):
+        import ctypes as C
+        from . import capi
+        from .quant import _check
+        x = np.ascontiguousarray(x, dtype=np.float32).ravel()
+        if out is None:
+            out = np.zeros(n_tokens * self.hidden_size, dtype=np.float32)
+        vp = lambda a: a.ctypes.data_as(C.c_void_p)
+        (tg, g), (tu, u), (td, d) = self.gate, self.up, self.down
+        _check(capi.load().oxq_moe_forward(tg, vp(g), g.size, tu, vp(u), u.size, td, vp(d), d.size, vp(self.router),
+                                           self.router.size, self.num_experts, self.hidden_size,
+                                           self.intermediate_size, self.top_k, vp(x), x.size, vp(out), out.size,
+                                           n_tokens))
+        return out

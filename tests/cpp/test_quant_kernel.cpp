@@ -17,6 +17,7 @@
 #include <vector>
 
 #include "oxq/gguf_model.hpp"
+#include "oxq/moe_ffn.hpp"
 #include "oxq/quant_kernel.hpp"
 
 using namespace oxq;
@@ -123,6 +124,24 @@ static const std::vector<int> Q8_ALT16 = {1, -2, 3, -4, 5, -6, 7, -8, 9, -10, 11
                                           -1, 2, -3, 4, -5, 6, -7, 8, -9, 10, -11, 12, -13, 14, -15, 16};
 static const std::vector<uint8_t> NIB_A = {0x5A, 0xF0, 0x13, 0x7E, 0xC2, 0x48, 0x9D, 0x6B,
                                            0xA3, 0x2F, 0x71, 0xE4, 0x0C, 0x58, 0xB6, 0xD9};
+
+// All-ones experts as the reference's make_expert (moe.rs:266-274), held as Q8_0 blocks (d = 1, q = 1).
+static MoeFfn ones_moe(size_t h, size_t n, size_t n_exp, size_t top_k, float router_fill = 1.0f) {
+    auto ones = [](size_t rows, size_t cols) {
+        std::vector<uint8_t> w;
+        const std::vector<uint8_t> blk = q8_0_block(1.0f, std::vector<int>(32, 1));
+        for (size_t i = 0; i < rows * cols / 32; ++i) append(w, blk);
+        return QuantTensor(std::move(w), {rows, cols}, GgufTensorType::Q8_0);
+    };
+    MoeFfn moe;
+    moe.router.assign(n_exp * h, router_fill);
+    for (size_t e = 0; e < n_exp; ++e) moe.experts.push_back(QuantExpert{ones(n, h), ones(n, h), ones(h, n)});
+    moe.top_k = top_k;
+    moe.num_experts = n_exp;
+    moe.hidden_size = h;
+    moe.intermediate_size = n;
+    return moe;
+}
 
 // ======================================================================================
 //  host-only cases
@@ -294,6 +313,32 @@ static void host_tests() {
         CHECK(m.from_bytes(v0) == OXQ_ERR_GGUF_UNSUPPORTED_VERSION);
         CHECK(m.from_bytes({'G', 'G', 'U', 'F'}) == OXQ_ERR_GGUF_UNEXPECTED_EOF);
         CHECK(m.load("/nonexistent/path/does_not_exist.gguf") == OXQ_ERR_GGUF_IO);
+    });
+
+    // ---- MoeFfn (crates/oxillama-arch/src/common/moe.rs tests) -------------------------------
+    run("moe top_k = 0 is an error (moe.rs:403-424); router and expert sizes are checked first (moe.rs:426-450, 307-322)", [&] {
+        MoeFfn moe = ones_moe(256, 256, 2, 0);
+        std::vector<float> x(256, 1.0f), y(256, 0.0f);
+        QuantResult r = moe.forward(x, y);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::KernelError);
+        moe.top_k = 1;
+        moe.router.resize(5);  // wrong router size
+        r = moe.forward(x, y);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 512 && r.error().got == 5);
+        moe = ones_moe(256, 256, 2, 1);
+        moe.experts.pop_back();  // experts.len() != num_experts
+        r = moe.forward(x, y);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch && r.error().expected == 2 && r.error().got == 1);
+        moe = ones_moe(256, 256, 2, 1);
+        moe.experts[1].gate.data.resize(3);  // expert.gate of the wrong size
+        r = moe.forward(x, y);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch);
+        CHECK(r.error().expected == 2 * 256 * 8 * 34 && r.error().got == 256 * 8 * 34 + 3);
+        moe = ones_moe(256, 256, 2, 1);
+        std::vector<float> short_x(100, 1.0f);
+        r = moe.forward(short_x, y);
+        CHECK(!r.is_ok() && r.error().kind == QuantError::DimensionMismatch && r.error().expected == 256 && r.error().got == 100);
     });
 }
 
@@ -634,6 +679,32 @@ static void gpu_tests() {
         CHECK_NEAR(y_host[1], -8.0, 0.01);
         DeviceWeights missing;
         CHECK(m.load_quant_linear("blk.1.attn_q.weight", missing) == OXQ_ERR_GGUF_TENSOR_NOT_FOUND);
+    });
+
+    run("moe top-1 / top-2 / clamped top-k on all-ones experts (moe.rs:324-401): the expert's own output", [&] {
+        // x = 127/128 everywhere: exact under Q8_0 (d = 2^-7, q = 127).  gate = up = 256 * x = 254, silu(254) = 254
+        // in fp32, h = 254^2 = 64516 (d = 508, q = 127: exact), down = 256 * 64516 = 16516096 < 2^24.
+        std::vector<float> x(256, 0.9921875f), y(256, -1.0f);
+        for (size_t top_k : {(size_t)1, (size_t)2, (size_t)10}) {
+            MoeFfn moe = ones_moe(256, 256, 4, top_k);
+            std::fill(y.begin(), y.end(), -1.0f);
+            QuantResult r = moe.forward(x, y);
+            CHECK(r.is_ok());
+            for (float v : y) CHECK_NEAR(v, 16516096.0, 16516096.0 * 1e-6);
+        }
+        // one-hot router: expert 0 alone at top-1 (its down matrix doubled tells it apart)
+        MoeFfn moe = ones_moe(256, 256, 4, 1, 0.0f);
+        moe.router[0] = 1.0f;
+        for (size_t b = 0; b < moe.experts[0].down.data.size(); b += 34) put_f16(moe.experts[0].down.data, b, 2.0f);
+        CHECK(moe.forward(x, y).is_ok());
+        for (float v : y) CHECK_NEAR(v, 2 * 16516096.0, 2 * 16516096.0 * 1e-6);
+        // three tokens at once; a zero token gives a zero row (moe.rs:291-305)
+        std::vector<float> xb(3 * 256, 0.9921875f), yb(3 * 256, -1.0f);
+        std::fill(xb.begin() + 256, xb.begin() + 512, 0.0f);
+        CHECK(moe.forward_batch(xb, yb, 3).is_ok());
+        CHECK_NEAR(yb[0], 2 * 16516096.0, 40.0);
+        CHECK(yb[256] == 0.0f && yb[511] == 0.0f);
+        CHECK_NEAR(yb[767], 2 * 16516096.0, 40.0);
     });
 }
 

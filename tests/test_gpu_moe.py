@@ -240,3 +240,72 @@ def test_moe_ffn_with_host_tables_and_errors(hip, ref):
     assert moe.moe_ffn_workspace_bytes((O.Q2_K, t, t), n_tok * k, hidden, inter) == 0
     with pytest.raises(hip.KernelError):  # top_k = 0, moe.rs:168-172
         moe.moe_ffn_dev(*args[:6], 0, *args[7:], ws)
+
+
+def test_moe_forward_host_slices(hip, ref):
+    """MoeFfn::forward through the host-slice entry point (the drop-in route), one token and a batch."""
+    n_exp, k, hidden, inter = 4, 2, 256, 512
+    t = O.Q4_K
+    wg, wu, wd = (expert_weights(t, s, n_exp, inter, hidden) for s in (11, 12, 13))
+    wd = expert_weights(O.Q6_K, 13, n_exp, hidden, inter)
+    router = synth.normal_f32(14, n_exp * hidden, 0.05)
+    layer = moe.MoeFfn(router, (t, wg), (t, wu), (O.Q6_K, wd), k, n_exp, hidden, inter)
+    x = synth.normal_f32(15, 5 * hidden)
+    sg, sd = wg.size // n_exp, wd.size // n_exp
+
+    def want(xt):
+        sel, wt = ref.moe_route(router, n_exp, hidden, k, xt)
+        xq = ref.quantize_q8_0(xt)
+        acc = np.zeros(hidden, np.float32)
+        for e, w in zip(sel, wt):
+            g = ref.matvec_q8_fused(t, wg[e * sg:(e + 1) * sg], xq, inter, hidden)
+            u = ref.matvec_q8_fused(t, wu[e * sg:(e + 1) * sg], xq, inter, hidden)
+            hq = ref.quantize_q8_0(ref.swiglu(g, u))
+            eo = ref.matvec_q8_fused(O.Q6_K, wd[e * sd:(e + 1) * sd], hq, hidden, inter)
+            acc = acc + np.float32(w) * eo
+        return acc
+
+    from oxillama_amd import capi
+    lib = capi.load()
+    for cache in (0, 1):
+        lib.oxq_weight_cache_enable(cache)
+        one = layer.forward(x[:hidden])
+        assert_close(one, want(x[:hidden]), "one token", tol=2e-3)
+        many = layer.forward_batch(x, 5).reshape(5, hidden)
+        assert np.array_equal(many[0].view(np.uint32), one.view(np.uint32))  # a row does not depend on the batch
+        for i in range(5):
+            assert_close(many[i], want(x[i * hidden:(i + 1) * hidden]), f"token {i}", tol=2e-3)
+    lib.oxq_weight_cache_enable(0)
+    lib.oxq_weight_cache_clear()
+    # the reference's error cases (moe.rs:403-450, 307-322) after a working call
+    layer.top_k = 0
+    with pytest.raises(hip.KernelError):
+        layer.forward(x[:hidden])
+    layer.top_k = 10  # clamps to the expert count (moe.rs:381-401)
+    assert_close(layer.forward(x[:hidden]), want_all(ref, layer, router, wg, wu, wd, x[:hidden]), "top_k clamp", tol=2e-3)
+    bad = moe.MoeFfn(router[:-1], (t, wg), (t, wu), (O.Q6_K, wd), k, n_exp, hidden, inter)
+    with pytest.raises(hip.DimensionMismatch) as e:
+        bad.forward(x[:hidden])
+    assert (e.value.expected, e.value.got) == (n_exp * hidden, n_exp * hidden - 1)
+    bad = moe.MoeFfn(router, (t, wg[:-1]), (t, wu), (O.Q6_K, wd), k, n_exp, hidden, inter)
+    with pytest.raises(hip.DimensionMismatch) as e:
+        bad.forward(x[:hidden])
+    assert (e.value.expected, e.value.got) == (wg.size, wg.size - 1)
+    bad = moe.MoeFfn(router[:n_exp * 100], (t, wg), (t, wu), (O.Q6_K, wd), k, n_exp, 100, inter)
+    with pytest.raises(hip.DimensionMismatch):  # sizes no longer fit hidden = 100
+        bad.forward(x[:100])
+
+
+def want_all(ref, layer, router, wg, wu, wd, xt):
+    """All experts selected (top_k >= num_experts): weights are the plain softmax."""
+    n_exp, hidden, inter = layer.num_experts, layer.hidden_size, layer.intermediate_size
+    sel, wt = ref.moe_route(router, n_exp, hidden, layer.top_k, xt)
+    assert len(sel) == n_exp
+    xq = ref.quantize_q8_0(xt)
+    sg, sd = wg.size // n_exp, wd.size // n_exp
+    acc = np.zeros(hidden, np.float32)
+    for e, w in zip(sel, wt):
+        eo_in = ref.quantize_q8_0(ref.swiglu(ref.matvec_q8_fused(layer.gate[0], wg[e * sg:(e + 1) * sg], xq, inter, hidden),
+                                             ref.matvec_q8_fused(layer.up[0], wu[e * sg:(e + 1) * sg], xq, inter, hidden)))
+        acc = acc + np.float32(w) * ref.matvec_q8_fused(layer.down[0], wd[e * sd:(e + 1) * sd], eo_in, hidden, inter)
+    return acc
