@@ -393,8 +393,12 @@ __device__ __forceinline__ void gemm_tile_body(
     constexpr int LPR = 64 / W_ROWS, SPL = 8 / LPR;   // scale decode: lanes per row, sub-blocks per lane
     static_assert(NT <= 2 && DIST >= 1, "tile configuration");
     extern __shared__ uint16_t lds_da[];            // [nsb][MTILES][2 halves][16] f16 token scales
-    // [wave][sub-block][KS x dsc, KS x -MAGIC*dsc, zero-point factor][row of the wave]
-    __shared__ float lds_sc[4][8][NP][W_ROWS];
+    // [wave][sub-block][KS x dsc, KS x -MAGIC*dsc, zero-point factor][row of the wave]; the split-k
+    // reduction at the end reuses the same memory (after a barrier), so that it does not cost occupancy
+    constexpr size_t SC_BYTES = sizeof(float) * 4 * 8 * NP * W_ROWS;
+    constexpr size_t RED_BYTES = SPLITK ? sizeof(float) * 4 * MT * NT * 16 * 64 : 0;
+    __shared__ __align__(16) uint8_t lds_static[SC_BYTES > RED_BYTES ? SC_BYTES : RED_BYTES];
+    float (*lds_sc)[8][NP][W_ROWS] = reinterpret_cast<float (*)[8][NP][W_ROWS]>(lds_static);
     const uint32_t nsb = k / 32, nblk = k / 256, ngrp = nblk * 4;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
@@ -635,7 +639,8 @@ __device__ __forceinline__ void gemm_tile_body(
     if constexpr (SPLITK) {
         // The four partial tiles meet in LDS; wave w then adds registers 4w..4w+3 of every tile in
         // the fixed order (w0 + w1) + (w2 + w3) and stores them.
-        __shared__ float lds_red[4][MT * NT][16][64];
+        float (*lds_red)[MT * NT][16][64] = reinterpret_cast<float (*)[MT * NT][16][64]>(lds_static);
+        __syncthreads();  // every wave is done with its scale factors
         for (int mt = 0; mt < MT; mt++)
             for (int nt = 0; nt < NT; nt++)
 #pragma unroll
