@@ -54,7 +54,7 @@ int g_gemm_variant = 0;  // tuning: 0 = default
 size_t gemm_workspace_bytes(uint32_t m, uint32_t k) {
     // token rows are padded so that a 128-token tile starting at any row stays inside
     const size_t mpad = ((size_t)m + 127) / 128 * 128 + 128, nsb = k / 32;
-    return nsb * mpad * (32 + 4 + 2);
+    return nsb * mpad * (32 + 4 + 2 + 8);  // activation bytes, P, f16 scales, the two half-block planes of P
 }
 
 uint32_t g_gemm_tile_min_rows = 0;  // tuning: 0 = default
@@ -65,7 +65,8 @@ bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
     // beside up to 24 KB of decoded weight scales; up to k = 8192 two work groups share a CU
     const bool known = type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K ||
                        type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q5_K || type == OXQ_TYPE_Q4_1 ||
-                       type == OXQ_TYPE_IQ4_NL || type == OXQ_TYPE_Q8_1 || type == OXQ_TYPE_Q5_0 || type == OXQ_TYPE_Q5_1;
+                       type == OXQ_TYPE_IQ4_NL || type == OXQ_TYPE_Q8_1 || type == OXQ_TYPE_Q5_0 || type == OXQ_TYPE_Q5_1 ||
+                       type == OXQ_TYPE_Q3_K || type == OXQ_TYPE_Q2_K;
     // the 32-weight formats are walked eight blocks at a time
     return known && k % 256 == 0 && m >= 1 && (size_t)(k / 32) * 256 <= 128 * 1024 &&
            gemm_workspace_bytes(m, k) < 0x7FFFFFFFull;
@@ -95,12 +96,16 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
     const int perm = type == OXQ_TYPE_Q6_K ? TileQ6K::ACT_PERM
                      : (type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q4_0) ? TileIQ4XS::ACT_PERM
                      : (type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_Q8_0) ? 0 : tile_act_perm_more(type);
+    // formats with a 16-weight zero-point term also need P per half block
+    float *p16 = tile_needs_p16_more(type)
+                     ? reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(P) + tile_p16_offset(nsb, mpad))
+                     : nullptr;
     if (perm == 2)
-        hipLaunchKernelGGL(gemm_prep_acts<2>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb);
+        hipLaunchKernelGGL(gemm_prep_acts<2>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
     else if (perm == 1)
-        hipLaunchKernelGGL(gemm_prep_acts<1>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb);
+        hipLaunchKernelGGL(gemm_prep_acts<1>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
     else
-        hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb);
+        hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const TilePlan plan = {q8t, P, da16, mpad};

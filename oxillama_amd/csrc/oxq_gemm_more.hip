@@ -166,15 +166,123 @@ struct TileQ5x {
 using TileQ5_0 = TileQ5x<OXQ_TYPE_Q5_0, 22, false>;
 using TileQ5_1 = TileQ5x<OXQ_TYPE_Q5_1, 24, true>;
 
+// Q3_K (reference/q3_k.rs:30-109): 110 B = 32 B hmask, 64 B of 2-bit fields, 12 B of 6-bit scales
+// (one per 16 weights, minus 32), d.  Sub-block s = 4n + j (32 weights) takes bits 2j..2j+1 of
+// qs[32n + l] and bit s of hmask[l], l = 0..31; weight = (q2 | hbit << 2) - 4.  As Q6_K: lane (c, h)
+// fetches bytes 16h..16h+15 (the 16-weight half h, which has its own scale), halves_to_pieces
+// hands every lane bytes 8h..8h+7 of both halves -- the k-slot order of the K = 16 operands and
+// of the activations (ACT_PERM = 2).  Group g = sub-blocks 2g and 2g+1 (n = g / 2).
+struct TileQ3K {
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q3_K, BLOCK_BYTES = 110;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int ACT_PERM = 2, NQ = 2, KSPLIT = 2;
+    struct Hdr {
+        uint32_t s[3];  // the 12 scale bytes
+        uint32_t d;     // f16 bits
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 32 + 32 * (g >> 1));
+        qs[1] = buf16(rs, row_off + 16 * h, so_blk);
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t,
+                                                    Hdr &hd) {
+        for (int i = 0; i < 3; i++) hd.s[i] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, row_off, so_blk + 96 + 4 * i, 0);
+        hd.d = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rs, row_off, so_blk + 108, 0);
+    }
+    // decode_scales (reference/q3_k.rs:30-59) for index 2s + is = 8n + kk: n = 0: s[kk] & 63;
+    // n = 1: nibble (kk >> 2) of s[8 + (kk & 3)] | (s[kk] >> 6) << 4; each minus 32.
+    static __device__ __forceinline__ void factors(const Hdr &hd, uint32_t, uint32_t s, float (&dsc)[KSPLIT], float &qneg) {
+        const float d = h2f(hd.d);
+        for (int is = 0; is < 2; is++) {
+            const uint32_t idx = 2 * s + is, kk = idx & 7;
+            const uint32_t byte = ((kk < 4 ? hd.s[0] : hd.s[1]) >> (8 * (kk & 3))) & 0xFF;
+            const uint32_t hi = ((hd.s[2] >> (8 * (kk & 3) + 4 * (kk >> 2))) & 0x0F) | ((byte >> 6) << 4);
+            dsc[is] = d * (float)((int)(idx < 8 ? (byte & 0x3F) : hi) - 32);  // exact
+        }
+        qneg = 0.0f;
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t g, BOperand<2> (&bop)[2]) {
+        uint32_t l[2][2], hb[2][2];
+        halves_to_pieces(qs[0], l);
+        halves_to_pieces(qs[1], hb);
+        for (int e = 0; e < 2; e++) {
+            const uint32_t j = 2 * (g & 1) + e, s = 2 * g + e;
+            for (int is = 0; is < 2; is++) {
+                uint32_t q[2];
+                for (int i = 0; i < 2; i++) {
+                    const uint32_t v = ((l[is][i] >> (2 * j)) & 0x03030303u) | (((hb[is][i] >> s) & 0x01010101u) << 2);
+                    // v - 4 per byte (0..7 -> -4..3) without carries between bytes
+                    q[i] = ((v | 0x80808080u) - 0x04040404u) ^ 0x80808080u;
+                }
+                bop[e].k16[is] = (long)(((uint64_t)q[1] << 32) | q[0]);
+            }
+        }
+    }
+};
+
+// Q2_K (reference/q2_k.rs:31-105): 84 B = 16 scale bytes (low nibble: scale, high nibble: min, one
+// per 16 weights), 64 B of 2-bit fields, d, dmin.  Same walk as Q3_K without the high bit; weight =
+// d * sc * q2 - dmin * mn, the second part through the zero-point term with one factor per
+// 16-weight half (MIN_PLANES = 2).
+struct TileQ2K {
+    static constexpr uint32_t TYPE = OXQ_TYPE_Q2_K, BLOCK_BYTES = 84;
+    static constexpr bool HAS_MIN = true;
+    static constexpr int ACT_PERM = 2, NQ = 1, KSPLIT = 2, MIN_PLANES = 2;
+    struct Hdr {
+        u32x4 sc;     // the 16 scale bytes
+        uint32_t dd;  // d | dmin << 16 (f16 bits)
+    };
+    static __device__ __forceinline__ uint32_t sub_block(uint32_t g, uint32_t e) { return 2 * g + e; }
+    static __device__ __forceinline__ void fetch(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t h, uint32_t so_blk,
+                                                 uint32_t g, u32x4 (&qs)[NQ]) {
+        qs[0] = buf16(rs, row_off + 16 * h, so_blk + 16 + 32 * (g >> 1));
+    }
+    template <int SPL>
+    static __device__ __forceinline__ void load_hdr(__amdgpu_buffer_rsrc_t rs, uint32_t row_off, uint32_t so_blk, uint32_t,
+                                                    Hdr &hd) {
+        hd.sc = buf16(rs, row_off, so_blk);
+        hd.dd = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rs, row_off, so_blk + 80, 0);
+    }
+    // scales[2s + is]: low nibble the scale, high nibble the min (reference/q2_k.rs:60-75)
+    static __device__ __forceinline__ void factors2(const Hdr &hd, uint32_t, uint32_t s, float (&dsc)[KSPLIT],
+                                                    float (&qneg)[2]) {
+        const uint32_t pair = hd.sc[s >> 1] >> (16 * (s & 1));
+        const float d = h2f(hd.dd & 0xFFFF), dmin = h2f(hd.dd >> 16);
+        for (int is = 0; is < 2; is++) {
+            const uint32_t byte = (pair >> (8 * is)) & 0xFF;
+            dsc[is] = d * (float)(byte & 0x0F);        // exact
+            qneg[is] = -(dmin * (float)(byte >> 4));   // exact
+        }
+    }
+    static __device__ __forceinline__ void operands(const u32x4 (&qs)[NQ], uint32_t g, BOperand<2> (&bop)[2]) {
+        uint32_t l[2][2];
+        halves_to_pieces(qs[0], l);
+        for (int e = 0; e < 2; e++) {
+            const uint32_t j = 2 * (g & 1) + e;
+            for (int is = 0; is < 2; is++) {
+                const uint32_t q0 = (l[is][0] >> (2 * j)) & 0x03030303u, q1 = (l[is][1] >> (2 * j)) & 0x03030303u;
+                bop[e].k16[is] = (long)(((uint64_t)q1 << 32) | q0);
+            }
+        }
+    }
+};
+
 int tile_act_perm_more(uint32_t type) {
     switch (type) {
     case OXQ_TYPE_Q4_1:
     case OXQ_TYPE_IQ4_NL: return 1;
     case OXQ_TYPE_Q5_0:
-    case OXQ_TYPE_Q5_1: return 2;
+    case OXQ_TYPE_Q5_1:
+    case OXQ_TYPE_Q3_K:
+    case OXQ_TYPE_Q2_K: return 2;
     default: return 0;
     }
 }
+
+bool tile_needs_p16_more(uint32_t type) { return type == OXQ_TYPE_Q2_K; }
 
 hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream) {
     switch (type) {
@@ -184,6 +292,8 @@ hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &p
     case OXQ_TYPE_Q8_1: return launch_tiles<TileQ8_1>(a, plan, stream);
     case OXQ_TYPE_Q5_0: return launch_tiles<TileQ5_0>(a, plan, stream);
     case OXQ_TYPE_Q5_1: return launch_tiles<TileQ5_1>(a, plan, stream);
+    case OXQ_TYPE_Q3_K: return launch_tiles<TileQ3K>(a, plan, stream);
+    case OXQ_TYPE_Q2_K: return launch_tiles<TileQ2K>(a, plan, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -27,6 +27,7 @@
 // tiled [k/32][m][32] in the byte order the format's operands need (so every MFMA operand
 // load is one aligned, contiguous KB), P as fp32 [k/32][m], da as f16 [k/32][m].
 #pragma once
+#include <type_traits>
 #include "oxq_gemv_kernel.hpp"
 #include "oxq_internal.hpp"
 
@@ -316,10 +317,12 @@ struct TileQ6K {
 // One thread per (token, activation block): payload copy in the byte order the format's B
 // operands have (PERM 1: even bytes then odd bytes inside each 8; PERM 2: the two 8-byte
 // halves of each 16-weight half side by side), P = da * sum(q), da.
+// p16 (optional): two more planes, da * sum(q) over the first and the second 16 weights of the
+// block, for formats whose zero-point term has 16-weight granularity.
 template <int PERM>
 __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict__ A, uint8_t *__restrict__ q8t,
                                                      float *__restrict__ P, uint16_t *__restrict__ da16, uint32_t m,
-                                                     uint32_t mpad, uint32_t nsb) {
+                                                     uint32_t mpad, uint32_t nsb, float *__restrict__ p16) {
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= mpad * nsb) return;
     const uint32_t j = idx / mpad, t = idx % mpad;
@@ -331,11 +334,12 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
         q[0] = ld16(blk + 2);
         q[1] = ld16(blk + 18);
     }
-    int s = 0;
+    int s0 = 0, s1 = 0;
     for (int i = 0; i < 4; i++) {
-        s = sdot4(q[0][i], 0x01010101u, s);
-        s = sdot4(q[1][i], 0x01010101u, s);
+        s0 = sdot4(q[0][i], 0x01010101u, s0);
+        s1 = sdot4(q[1][i], 0x01010101u, s1);
     }
+    const int s = s0 + s1;
     if (PERM == 2) {  // [half 0 | half 1] x [bytes 0-7 | 8-15] -> bytes 8h..8h+7 of both halves in 16-byte piece h
         const u32x4 x0 = q[0], x1 = q[1];
         q[0] = u32x4{x0[0], x0[1], x1[0], x1[1]};
@@ -354,8 +358,22 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
     dst[0] = q[0];
     dst[1] = q[1];
     P[(size_t)j * mpad + t] = h2f(dbits) * (float)s;
+    if (p16) {
+        p16[(size_t)j * mpad + t] = h2f(dbits) * (float)s0;
+        p16[((size_t)nsb + j) * mpad + t] = h2f(dbits) * (float)s1;
+    }
     da16[(size_t)j * mpad + t] = (uint16_t)dbits;
 }
+
+// Zero-point planes of a format: 1 (one factor per 32-weight sub-block, F::factors) unless the policy
+// says MIN_PLANES = 2 (one per 16-weight half, F::factors2).
+template <class F, class = void> struct tile_min_planes { static constexpr int value = 1; };
+template <class F> struct tile_min_planes<F, std::void_t<decltype(F::MIN_PLANES)>> {
+    static constexpr int value = F::MIN_PLANES;
+};
+// Byte offset, from the start of the P plane, of the two half-block planes (the workspace holds the
+// activation bytes, P, the f16 scales, then the half planes: 32 + 4 + 2 bytes per token block before them).
+__host__ __device__ __forceinline__ size_t tile_p16_offset(size_t nsb, size_t mpad) { return nsb * mpad * 6; }
 
 // Work group = 4 waves as WM (tokens) x WN (weight rows); each wave owns MT x NT MFMA tiles
 // of 32 x 32: a (32*MT*WM)-token x (32*NT*WN)-row tile per work group.  Lane l: c = l % 32
@@ -388,7 +406,8 @@ __device__ __forceinline__ void gemm_tile_body(
     constexpr int WMX = SPLITK ? 1 : WM, WN = SPLITK ? 1 : 4 / WMX;
     constexpr int WG_TOK = 32 * MT * WMX, WG_ROWS = 32 * NT * WN, MTILES = MT * WMX;
     constexpr int KS = F::KSPLIT;                     // MFMAs (and scale factors) per sub-block
-    constexpr int NP = 2 * KS + (F::HAS_MIN ? 1 : 0);  // fp32 factor planes per sub-block in LDS
+    constexpr int MINP = tile_min_planes<F>::value;    // zero-point factors per sub-block
+    constexpr int NP = 2 * KS + (F::HAS_MIN ? MINP : 0);  // fp32 factor planes per sub-block in LDS
     constexpr int W_ROWS = 32 * NT;                   // weight rows of one wave
     constexpr int LPR = 64 / W_ROWS, SPL = 8 / LPR;   // scale decode: lanes per row, sub-blocks per lane
     static_assert(NT <= 2 && DIST >= 1, "tile configuration");
@@ -464,8 +483,9 @@ __device__ __forceinline__ void gemm_tile_body(
         const_cast<uint8_t *>(W + (size_t)n_base * row_bytes), 0, (int)min(w_left, (size_t)0x7FFFFFFF), BUFFER_FLAGS);
     const __amdgpu_buffer_rsrc_t rs_a =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(q8t), 0, (int)(nsb * mpad * 32), BUFFER_FLAGS);
-    const __amdgpu_buffer_rsrc_t rs_p =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(P), 0, (int)(nsb * mpad * 4), BUFFER_FLAGS);
+    const __amdgpu_buffer_rsrc_t rs_p = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(P), 0, (int)(MINP == 2 ? tile_p16_offset(nsb, mpad) + nsb * mpad * 8 : nsb * mpad * 4),
+        BUFFER_FLAGS);
 
     // Scale decode, per wave for its own rows (no work-group barrier in the k loop): lane ->
     // row lane % W_ROWS, sub-blocks SPL * (lane / W_ROWS) + 0..SPL-1.  The wave writes the
@@ -476,14 +496,18 @@ __device__ __forceinline__ void gemm_tile_body(
 #pragma unroll
         for (int e = 0; e < SPL; e++) {
             const uint32_t s = ds0 + e;
-            float dsc[KS], qneg;
-            F::factors(hd, e, s, dsc, qneg);
+            float dsc[KS], qneg[MINP];
+            if constexpr (MINP == 2)
+                F::factors2(hd, e, s, dsc, qneg);
+            else
+                F::factors(hd, e, s, dsc, qneg[0]);
 #pragma unroll
             for (int is = 0; is < KS; is++) {
                 lds_sc[wave][s][is][drow] = dsc[is];
                 lds_sc[wave][s][KS + is][drow] = -(MAGIC_F * dsc[is]);  // exact
             }
-            if (F::HAS_MIN) lds_sc[wave][s][NP - 1][drow] = qneg;
+            if (F::HAS_MIN)
+                for (int ip = 0; ip < MINP; ip++) lds_sc[wave][s][2 * KS + ip][drow] = qneg[ip];
         }
     };
     {
@@ -516,7 +540,7 @@ __device__ __forceinline__ void gemm_tile_body(
     };
     struct Ops {
         u32x4 a[2][MT];  // [sub-block of the pair][token tile] 16 activation bytes
-        float pv[MT];    // P of sub-block sub_block(g, h)
+        float pv[MT][MINP];  // P of sub-block sub_block(g, h) (MINP = 2: of its two halves)
     };
     // group index G = 4*blk + g; groups past the end re-read the last one (result unused)
     auto fetch_w = [&](Wq &w, uint32_t G) {
@@ -531,8 +555,12 @@ __device__ __forceinline__ void gemm_tile_body(
                 o.a[e][mt] = buf16(rs_a, aq_off[mt], (blk8 + F::sub_block(g, e)) * mpad * 32);
         if (F::HAS_MIN)
             for (int mt = 0; mt < MT; mt++)  // sub_block(g, 0) and (g, 1) are adjacent for every format with a min term
-                o.pv[mt] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                                         rs_p, pq_off[mt], (blk8 + F::sub_block(g, 0)) * mpad * 4, 0));
+                for (int ip = 0; ip < MINP; ip++) {
+                    const uint32_t plane = MINP == 2 ? (uint32_t)tile_p16_offset(nsb, mpad) + ip * nsb * mpad * 4 : 0u;
+                    o.pv[mt][ip] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(rs_p, pq_off[mt],
+                                                                    plane + (blk8 + F::sub_block(g, 0)) * mpad * 4, 0));
+                }
     };
 
     // One group: 2 sub-blocks x KS MFMAs x MT x NT tiles, each MFMA followed by its 32 VALU
@@ -583,8 +611,10 @@ __device__ __forceinline__ void gemm_tile_body(
             if (F::HAS_MIN && e == 1 && is == KS - 1) {
                 // zero-point term of the group's sub-blocks (lanes h = 0: the first, h = 1: the second):
                 // acc[token][row] += P[token][s] * factor[row][s], contracted over the pair
-                const float qv = lds_sc[wave][F::sub_block(g, 0) + h][NP - 1][nt * 32 + c];
-                acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(o.pv[mt], qv, acc[mt][nt], 0, 0, 0);
+                for (int ip = 0; ip < MINP; ip++) {
+                    const float qv = lds_sc[wave][F::sub_block(g, 0) + h][2 * KS + ip][nt * 32 + c];
+                    acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(o.pv[mt][ip], qv, acc[mt][nt], 0, 0, 0);
+                }
             }
         }
     };
@@ -704,6 +734,7 @@ struct TilePlan {
 // The formats instantiated in the second translation unit, and the activation byte order they need.
 hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream);
 int tile_act_perm_more(uint32_t type);
+bool tile_needs_p16_more(uint32_t type);
 
 template <class F, int MT, int NT, int WM, int DIST, bool DUMP, int OCC = 2, int ADIST = 1>
 static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {

@@ -235,9 +235,10 @@ def test_moe_ffn_with_host_tables_and_errors(hip, ref):
     with pytest.raises(hip.BufferTooSmall) as e:
         moe.moe_ffn_dev(*args, ws[:256])
     assert e.value.needed == ws.numel()
-    with pytest.raises(hip.UnsupportedShape):  # no grouped kernel for Q2_K
-        moe.moe_ffn_dev((O.Q2_K, args[0][1], stride), *args[1:], ws)
-    assert moe.moe_ffn_workspace_bytes((O.Q2_K, t, t), n_tok * k, hidden, inter) == 0
+    with pytest.raises(hip.UnsupportedShape):  # the grouped kernel walks 256 columns at a time
+        moe.moe_ffn_dev((O.Q8_0, args[0][1], stride), (O.Q8_0, args[1][1], stride), (O.Q8_0, args[2][1], stride),
+                        *args[3:-2], 288, inter, ws)
+    assert moe.moe_ffn_workspace_bytes((O.Q8_0, O.Q8_0, O.Q8_0), n_tok * k, 288, inter) == 0
     with pytest.raises(hip.KernelError):  # top_k = 0, moe.rs:168-172
         moe.moe_ffn_dev(*args[:6], 0, *args[7:], ws)
 

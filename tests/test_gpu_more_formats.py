@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 FP32_REL_TOL = 1e-5
 DEV = "cuda:0"
 TYPES = O.MORE_TYPES
-TILE_TYPES = [O.Q5_K, O.Q4_1, O.Q5_0, O.Q5_1, O.Q8_1, O.IQ4_NL]
+TILE_TYPES = [O.Q5_K, O.Q4_1, O.Q5_0, O.Q5_1, O.Q8_1, O.IQ4_NL, O.Q3_K, O.Q2_K]
 ids = lambda t: O.NAMES[t]
 
 
@@ -62,7 +62,7 @@ KAT_VALUES = {O.Q4_1: [10.0, 5.0], O.Q5_0: [15.0, -32.0, None], O.Q5_1: [31.0, 3
 def test_metadata_and_dispatch(hip, t):
     k = hip.KernelDispatcher().get_kernel(t)
     assert (k.block_size(), k.block_bytes(), k.name()) == (*O.BLOCK[t], O.NAMES[t])
-    # the int8-MFMA tile kernel takes six of them; Q2_K and Q3_K run the batched form by rows
+    # the int8-MFMA tile kernel takes all of them
     assert (k.gemm_workspace_bytes(64, 4096, 4096) > 0) == (t in TILE_TYPES)
 
 
@@ -196,10 +196,10 @@ def test_device_route_forms(hip, ref, t):
 
 def test_grouped_form_reports_unsupported(hip):
     z = torch.zeros(4096, dtype=torch.uint8, device=DEV)
-    k = hip.HipKernel(O.Q2_K)
-    assert k.moe_gemm_workspace_bytes(64, 256, 256) == 0
+    k = hip.HipKernel(O.Q5_0)  # the tile kernel walks 256 columns at a time
+    assert k.moe_gemm_workspace_bytes(64, 256, 288) == 0
     with pytest.raises(hip.UnsupportedShape):
-        k.moe_gemm_q8_dev(z, 256 * 84, 1, z, z, 4, 4, z, 256, 256, z)
+        k.moe_gemm_q8_dev(z, 256 * 9 * 22, 1, z, z, 4, 4, z, 256, 288, z)
 
 
 def _tile_zero_point(t, acts, rows, k_):
@@ -239,7 +239,7 @@ def test_prefill_tile_kernel(hip, ref, shape, t):
         kern.gemm_q8_dev(dw, da, dy2, m, n, k_, accumulate=True, workspace=None)
         torch.cuda.synchronize()
         assert torch.equal(dy2, dy + dy)
-        dsum = torch.empty((m, n, k_ // 32), dtype=torch.int32, device=DEV)
+        dsum = torch.empty((m, n, k_ // O.GROUP_COLS[t]), dtype=torch.int32, device=DEV)  # Q2_K, Q3_K: 16-weight groups
         dy3 = torch.empty_like(dy)
         kern.gemm_block_sums_dev(dw, da, dy3, dsum, m, n, k_, workspace=ws)
         want = np.stack([ref.block_sums(t, w, acts[r * arb:(r + 1) * arb], n, k_) for r in range(m)])
@@ -249,7 +249,7 @@ def test_prefill_tile_kernel(hip, ref, shape, t):
         capi.load().oxq_set_gemm_tile_min_rows(0)
 
 
-@pytest.mark.parametrize("t", [O.Q5_K, O.Q5_0, O.IQ4_NL], ids=ids)
+@pytest.mark.parametrize("t", [O.Q5_K, O.Q5_0, O.IQ4_NL, O.Q3_K, O.Q2_K], ids=ids)
 def test_grouped_expert_matmul(hip, ref, t):
     """Grouped (mixture-of-experts) form on added formats: each expert's rows against its own weights."""
     n_exp, n, k_ = 4, 96, 512
