@@ -312,10 +312,27 @@ def main():
             us = e0.elapsed_time(e1) * 1e3 / 4
             others[name] = {"gemm_us": round(us, 2), "TOPS": round(ops / us / 1e6, 1)}
             del wt, wst
+        # what the matrix cores deliver on a kernel of nothing but int8 MFMAs (register operands)
+        import ctypes as C
+        kit = C.CDLL(os.path.join(ROOT, "oxillama_amd", "liboxq_benchkit.so"))
+        kit.oxq_benchkit_mfma_i8.argtypes = [C.c_void_p, C.c_uint, C.c_int, C.c_void_p]
+        mf_blocks, mf_iters = 4096, 1024
+        mf_out = torch.empty(mf_blocks * 256, dtype=torch.int32, device=dev)
+        with torch.cuda.stream(stream):
+            kit.oxq_benchkit_mfma_i8(mf_out.data_ptr(), mf_blocks, mf_iters, quant.HipKernel._stream())
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            kit.oxq_benchkit_mfma_i8(mf_out.data_ptr(), mf_blocks, mf_iters, quant.HipKernel._stream())
+            e1.record(stream)
+            e1.synchronize()
+        mfma_only_tops = mf_blocks * 4 * mf_iters * 4 * 2 * 32 ** 3 / (e0.elapsed_time(e1) * 1e3) / 1e6
         prefill = {"workload": "Q4_K 14336x4096 x Q8_0 acts 512x4096", "int8_ops": ops,
                    "gemm_us": round(gemm_us, 2), "quantize_us": round(quant_us, 2),
                    "TOPS": round(ops / gemm_us / 1e6, 2), "peak_TOPS": INT8_PEAK_TOPS,
                    "frac_int8_peak": round(ops / gemm_us / 1e6 / INT8_PEAK_TOPS, 4),
+                   "mfma_only_TOPS": round(mfma_only_tops, 1),
+                   "frac_of_mfma_only": round(ops / gemm_us / 1e6 / mfma_only_tops, 4),
                    "same_shape_other_formats": others}
 
     # ---- C5: Mixtral-shaped IQ4_XS expert matmuls, 64 tokens, top-2 of 8 experts ------------

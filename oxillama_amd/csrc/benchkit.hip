@@ -1,7 +1,8 @@
 // Measurement helpers (not part of the quantized-matmul ABI): a plain copy kernel of
-// known size, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters, and a
+// known size, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters, a
 // streaming read kernel that marks the practical HBM read ceiling for a given
-// footprint and launch shape.
+// footprint and launch shape, and a kernel of nothing but int8 MFMAs on register
+// operands, which marks what the matrix cores deliver when nothing else is in the way.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -33,7 +34,33 @@ __global__ __launch_bounds__(256) void benchkit_read_kernel(const u32x4 *__restr
     if (r == 0x9E3779B9u) out[blockIdx.x] = r;  // practically never: keeps the loads alive
 }
 
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// Four independent accumulator chains of v_mfma_i32_32x32x32_i8 per wave, `iters` rounds.
+__global__ __launch_bounds__(256) void benchkit_mfma_i8_kernel(int *__restrict__ out, int iters) {
+    const int lane = threadIdx.x;
+    v4i a = {lane, lane * 3, lane * 5, lane * 7}, b = {lane ^ 21, lane * 11, lane * 13, lane * 17};
+    v16i acc[4];
+    for (int c = 0; c < 4; c++)
+        for (int i = 0; i < 16; i++) acc[c][i] = 0;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, acc[c], 0, 0, 0);
+    }
+    int r = 0;
+    for (int c = 0; c < 4; c++)
+        for (int i = 0; i < 16; i++) r ^= acc[c][i];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
+}
+
 extern "C" {
+
+// blocks x 4 waves x iters x 4 MFMAs of 2 * 32 * 32 * 32 int8 operations; out: blocks * 256 ints.
+int oxq_benchkit_mfma_i8(void *out, unsigned blocks, int iters, void *stream) {
+    hipLaunchKernelGGL(benchkit_mfma_i8_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (int *)out, iters);
+    return (int)hipGetLastError();
+}
 
 int oxq_benchkit_copy(const void *src, void *dst, size_t bytes, unsigned blocks, void *stream) {
     hipLaunchKernelGGL(benchkit_copy_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4 *)src,
