@@ -389,6 +389,7 @@ def main():
 
     # ---- CPU baseline: the reference's fused rows restated in C, same layer -------------
     cpu = None
+    parity = None
     if not args.no_cpu_baseline:
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         import oracle as O
@@ -423,6 +424,35 @@ def main():
                 if el > budget_s or n >= 50:
                     return el / n, n
 
+        # Parity gate beside the timing: the timed step once more on layer 0, each stage against the
+        # oracle on the device's own input to that stage (activation bytes ==, fp32 within 1e-5 * |y|_inf).
+        with torch.cuda.stream(stream):
+            step(0)
+            stream.synchronize()
+        g_xq, g_hq = xq.cpu().numpy(), hq.cpu().numpy()
+        g_y = {"q": yq.cpu().numpy(), "gate": yg.cpu().numpy(), "up": yu.cpu().numpy(), "down": yd.cpu().numpy()}
+
+        def rel_err(got, want):
+            return float(np.abs(got.astype(np.float64) - want).max() / max(float(np.abs(want).max()), 1e-30))
+
+        if args.fused_quantize:
+            parity = None  # this variant keeps no Q8_0 buffers to compare stage by stage
+        else:
+            a_ref = O.quantize_q8_0(hx)
+            h_ref = O.quantize_q8_0(O.swiglu(g_y["gate"], g_y["up"]))
+            errs = {"q_proj": rel_err(g_y["q"], O.matvec_q8_fused_mt(O.Q8_0, hw["q"], g_xq, H, H, cores)),
+                    "ffn_gate": rel_err(g_y["gate"], O.matvec_q8_fused_mt(O.Q4_K, hw["gate"], g_xq, F, H, cores)),
+                    "ffn_up": rel_err(g_y["up"], O.matvec_q8_fused_mt(O.Q4_K, hw["up"], g_xq, F, H, cores)),
+                    "ffn_down": rel_err(g_y["down"], O.matvec_q8_fused_mt(O.Q6_K, hw["down"], g_hq, H, F, cores))}
+            parity = {"acts_q8_bytes_equal": bool(np.array_equal(g_xq, a_ref)),
+                      "h_q8_bytes_equal_fraction": round(float(np.mean(g_hq == h_ref)), 6),
+                      "fp32_max_err_over_ymax": {k: float(f"{v:.3e}") for k, v in errs.items()},
+                      "tolerance": 1e-5,
+                      "pass": bool(np.array_equal(g_xq, a_ref) and max(errs.values()) <= 1e-5),
+                      "checked_against": "scalar C restatement of the reference's fused rows, layer 0 of the timed step"}
+            if not parity["pass"]:
+                print("bench.py: PARITY GATE FAILED: " + json.dumps(parity), file=sys.stderr, flush=True)
+
         s_mt, n_mt = time_cpu(cores, 8.0)
         s_1t, n_1t = time_cpu(1, 8.0)
         cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
@@ -456,6 +486,7 @@ def main():
                                    "input vector to Q8_0 itself")},
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "parity": parity,
         "kernels": kernels,
         "prefill": prefill,
         "moe": moe_out,
@@ -463,6 +494,8 @@ def main():
                    "clock_mhz": info["clock_khz"] / 1000.0, "weight_generation_s": round(gen_s, 1)},
     }
     print(json.dumps(out), flush=True)
+    if parity is not None and not parity["pass"]:
+        sys.exit(3)  # the line above is still printed; a fast kernel with wrong results is not a result
 
 
 if __name__ == "__main__":

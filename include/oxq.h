@@ -341,7 +341,7 @@ int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_ty
  * offsets[e] .. offsets[e+1]-1); d_pair_token [n_tokens * k] (the token of grouped row r);
  * d_token_rows [n_tokens x k] (the grouped row of each token's j-th choice).  Rows of an expert
  * are in ascending (token, choice) order: the tables do not depend on scheduling.  top_k == 0
- * is KernelError (the reference's InvalidConfig, moe.rs:168-172).
+ * is KernelError (the reference's InvalidConfig, moe.rs:168-172); at most 1024 experts.
  *
  * oxq_moe_gather_quantize_q8_0_dev: grouped activation row r = the Q8_0 blocks of
  * d_x[d_pair_token[r]] (every selected expert reads the token's own input, moe.rs:252).

@@ -1000,7 +1000,7 @@ int oxq_moe_route_dev(const float *d_router, const float *d_x, size_t n_tokens, 
                       size_t top_k, int32_t *d_experts, float *d_weights, int32_t *d_row_offsets,
                       int32_t *d_pair_token, int32_t *d_token_rows, void *stream) {
     if (top_k == 0) return fail(OXQ_ERR_KERNEL, 1, 0, "MoeFfn top_k must be >= 1");  // moe.rs:168-172
-    if (n_experts > 4096) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 4096, n_experts, "at most 4096 experts");
+    if (n_experts > 1024) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 1024, n_experts, "at most 1024 experts");
     const size_t k = top_k < n_experts ? top_k : n_experts;  // moe.rs:233
     if (n_tokens * k > 0x7FFFFFFFull || hidden > 0xFFFFFFFFull)
         return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0x7FFFFFFFull, n_tokens * k, "too many (token, expert) pairs");
