@@ -107,3 +107,47 @@ def test_quant_tensor_bookkeeping():
     t = quant.QuantTensor(np.zeros(144 * 6, dtype=np.uint8), [3, 512], 12)
     assert t.n_elements() == 1536 and t.n_blocks() == 6 and t.expected_data_size() == 864
     assert quant.QuantTensor(b"", [], 12).n_elements() == 0
+
+
+def test_moe_forward_argument_errors_before_touching_the_gpu():
+    # MoeFfn::validate / Expert::validate, crates/oxillama-arch/src/common/moe.rs:151-173, 33-58: router size,
+    # top_k, then the experts' gate / up / down sizes; all of it is checked before any device work
+    from oxillama_amd import moe
+    n_exp, hidden, inter, t = 2, 256, 256, 12
+    one = inter * (hidden // 256) * 144
+    w = np.zeros(n_exp * one, dtype=np.uint8)
+    router = np.zeros(n_exp * hidden, dtype=np.float32)
+    x = np.zeros(hidden, dtype=np.float32)
+
+    def layer(**kw):
+        a = dict(router=router, gate=(t, w), up=(t, w), down=(t, w), top_k=1, num_experts=n_exp, hidden_size=hidden,
+                 intermediate_size=inter)
+        a.update(kw)
+        return moe.MoeFfn(**a)
+
+    with pytest.raises(quant.DimensionMismatch) as e:  # moe.rs:426-450
+        layer(router=router[:-3]).forward(x)
+    assert (e.value.expected, e.value.got) == (n_exp * hidden, n_exp * hidden - 3)
+    with pytest.raises(quant.KernelError):  # moe.rs:403-424; comes before the experts' sizes
+        layer(top_k=0, gate=(t, w[:-1])).forward(x)
+    for name in ("gate", "up", "down"):  # moe.rs:307-322
+        with pytest.raises(quant.DimensionMismatch) as e:
+            layer(**{name: (t, w[:-1])}).forward(x)
+        assert (e.value.expected, e.value.got) == (w.size, w.size - 1)
+    with pytest.raises(quant.DimensionMismatch) as e:
+        layer().forward(x[:100])
+    assert (e.value.expected, e.value.got) == (hidden, 100)
+    with pytest.raises(quant.DimensionMismatch) as e:
+        layer().forward_batch(x, 1, out=np.zeros(5, dtype=np.float32))
+    assert (e.value.expected, e.value.got) == (hidden, 5)
+    with pytest.raises(quant.UnsupportedType):
+        layer(gate=(15, w)).forward(x)
+    # a layer without experts leaves the zeroed output (moe.rs:240-242)
+    empty = moe.MoeFfn(np.zeros(0, np.float32), (t, w[:0]), (t, w[:0]), (t, w[:0]), 1, 0, hidden, inter)
+    out = empty.forward_batch(np.ones(2 * hidden, np.float32), 2, out=np.full(2 * hidden, 7.0, np.float32))
+    assert np.all(out == 0)
+    lib = capi.load()
+    assert lib.oxq_moe_route_dev(None, None, 1, 2, 4, 0, None, None, None, None, None, None) == capi.ERR_KERNEL
+    assert lib.oxq_moe_route_dev(None, None, 1, 2000, 4, 1, None, None, None, None, None, None) == capi.ERR_UNSUPPORTED_SHAPE
+    assert lib.oxq_moe_ffn_workspace_bytes(t, t, t, 8, 288, 256) == 0  # the grouped kernel walks 256 columns at a time
+    assert lib.oxq_moe_ffn_workspace_bytes(t, t, t, 8, 256, 512) > 0
