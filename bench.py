@@ -11,7 +11,8 @@ second over the timed steps (inputs resident in HBM, launches replayed from one
 HIP graph so the host adds no per-kernel latency).
 
 Prints ONE JSON line.  Extra objects:
-  roofline     the dominant kernel (Q4_K GEMV on ffn_gate + ffn_up, 2 x 14336x4096 in one launch)
+  roofline     the dominant kernel of the timed step (Q4_K ffn_gate + ffn_up, 2 x 14336x4096, with SwiGLU and the
+               quantizer of h in the same launch; --unfused-swiglu: the plain gate + up launch)
                timed alone with HIP events on the launch stream, algorithmic bytes / duration
                vs 8 TB/s
   kernels      the same figure for each GEMV shape, the lm_head and C1 shapes
@@ -33,8 +34,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per gate+up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
 # what the counter reads for a copy kernel of known size (2.000 and 1.000); the runs and figures are in
-# profiles/hbm_traffic_gemv_gate_up_lm_head_prefill_pmc.txt.  Algorithmic bytes are 66 179 328.
+# profiles/hbm_traffic_gemv_gate_up_lm_head_prefill_pmc.txt.  Algorithmic bytes are 66 179 328 for the plain
+# gate + up launch and 66 079 872 for the launch that also forms and quantizes h.
 MEASURED_TRAFFIC_GATE_UP = 66318438
+MEASURED_TRAFFIC_GATE_UP_SWIGLU = 66301133
 INT8_PEAK_TOPS = 5000.0
 
 Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS = 2, 8, 12, 14, 23
@@ -60,6 +63,8 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra-kernels", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--unfused-swiglu", action="store_true",
+                    help="gate + up in one launch, SwiGLU + quantize in a second (default: all of it in one launch)")
     ap.add_argument("--fused-quantize", action="store_true",
                     help="decode step with the Q8_0 quantization done inside the GEMV kernels (3 launches per layer)")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -102,10 +107,13 @@ def main():
         quant.quantize_q8_0_dev(torch.from_numpy(synth.normal_f32(1, H)).to(dev), xq)
         yg = torch.zeros(F, dtype=torch.float32, device=dev)
         yu = torch.zeros(F, dtype=torch.float32, device=dev)
+        hq_probe = torch.zeros(F // 32 * 34, dtype=torch.uint8, device=dev)
         for l in range(8):
             g, u = (torch.from_numpy(synth.weights(Q4_K, s0 + l, F, H)).to(dev) for s0 in (2000, 3000))
             torch.cuda.synchronize()
             k_q4k.matvec_q8_fused_multi_dev([g, u], xq, [yg, yu], F, H, accumulate=False)
+            torch.cuda.synchronize()
+            linear.gate_up_swiglu_dev(Q4_K, g, u, xq, None, hq_probe, F, H)
             torch.cuda.synchronize()
         V = 128256
         logits = torch.zeros(V, dtype=torch.float32, device=dev)
@@ -155,8 +163,9 @@ def main():
     stream = torch.cuda.Stream()
 
     def step(i):
-        """One layer, five launches: quantize x; q_proj; ffn_gate + ffn_up (one launch: both read
-        the same vector); h = silu(gate) * up quantized to Q8_0 in the same kernel; ffn_down on h.
+        """One layer, four launches: quantize x; q_proj; ffn_gate + ffn_up + h = silu(gate) * up quantized
+        to Q8_0 (one launch: a work group owns 32 rows of both matrices, one block of h); ffn_down on h.
+        --unfused-swiglu: gate + up in one launch, SwiGLU + quantize in another (five launches).
         --fused-quantize lets the GEMV kernels quantize their fp32 input themselves (four
         launches, bit-identical results); measured slightly slower here: every work group then
         quantizes the whole vector into LDS before its first row, which costs more than the
@@ -165,8 +174,11 @@ def main():
         if not args.fused_quantize:
             quant.quantize_q8_0_dev(x, xq)
             k_q8.matvec_q8_fused_dev(w["q"], xq, yq, H, H, accumulate=False)
-            k_q4k.matvec_q8_fused_multi_dev([w["gate"], w["up"]], xq, [yg, yu], F, H, accumulate=False)
-            linear.swiglu_quantize_dev(yg, yu, None, hq)
+            if args.unfused_swiglu:
+                k_q4k.matvec_q8_fused_multi_dev([w["gate"], w["up"]], xq, [yg, yu], F, H, accumulate=False)
+                linear.swiglu_quantize_dev(yg, yu, None, hq)
+            else:
+                linear.gate_up_swiglu_dev(Q4_K, w["gate"], w["up"], xq, None, hq, F, H)
             k_q6k.matvec_q8_fused_dev(w["down"], hq, yd, H, F, accumulate=False)
         else:
             k_q8.gemv_dev(w["q"], x, yq, H, H)
@@ -245,13 +257,39 @@ def main():
                 "algorithmic_GBps": round(ab / us / 1e3, 1), "frac_hbm_peak": round(ab / us / 1e3 / HBM_PEAK_GBPS, 4),
                 "algorithmic_bytes": ab}
 
-    gate_up = [w["gate"] for w in layers] + [w["up"] for w in layers]
-    dom = time_pair()
-    roofline = {"bound": "hbm", "kernel": "gemv_q8_cached<Q4_K>, ffn_gate + ffn_up (2 x 14336x4096) in one launch",
-                "achieved": dom["algorithmic_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dom["frac_hbm_peak"],
-                "traffic": MEASURED_TRAFFIC_GATE_UP, "us_per_call": dom["us_per_call"], "algorithmic_bytes": dom["algorithmic_bytes"]}
+    def time_pair_swiglu():
+        """ffn_gate + ffn_up + SwiGLU + the Q8_0 quantizer of h in one launch, over all layers."""
+        def body():
+            for w in layers:
+                linear.gate_up_swiglu_dev(Q4_K, w["gate"], w["up"], xq, None, hq, F, H)
+        g = capture(body)
+        timed_replay(g)
+        us = min(timed_replay(g) for _ in range(3)) * 1e3 / L
+        ab = 2 * F * row_bytes(Q4_K, H) + H // 32 * 34 + F // 32 * 34
+        return {"us_per_call": round(us, 3), "launches": L, "distinct_weight_sets": L,
+                "weight_GBps": round(2 * F * row_bytes(Q4_K, H) / us / 1e3, 1),
+                "algorithmic_GBps": round(ab / us / 1e3, 1), "frac_hbm_peak": round(ab / us / 1e3 / HBM_PEAK_GBPS, 4),
+                "algorithmic_bytes": ab}
 
-    kernels = {"q4k_gate_plus_up_one_launch": dom, "q4k_gate_up_14336x4096": time_kernel(k_q4k, Q4_K, gate_up, xq, yg, F, H)}
+    gate_up = [w["gate"] for w in layers] + [w["up"] for w in layers]
+    pair = time_pair()
+    pair_swiglu = time_pair_swiglu()
+    with torch.cuda.stream(stream):  # the legs below read the quantized synthetic h again
+        quant.quantize_q8_0_dev(h, hq)
+        stream.synchronize()
+    # the dominant kernel of the timed step
+    if args.unfused_swiglu or args.fused_quantize:
+        dom, dom_name, dom_traffic = pair, "gemv_q8_cached<Q4_K>, ffn_gate + ffn_up (2 x 14336x4096) in one launch", \
+            MEASURED_TRAFFIC_GATE_UP
+    else:
+        dom, dom_name, dom_traffic = pair_swiglu, "gemv_q8_gate_up_swiglu<Q4_K>, ffn_gate + ffn_up (2 x 14336x4096) + " \
+            "SwiGLU + Q8_0 quantizer of h in one launch", MEASURED_TRAFFIC_GATE_UP_SWIGLU
+    roofline = {"bound": "hbm", "kernel": dom_name,
+                "achieved": dom["algorithmic_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dom["frac_hbm_peak"],
+                "traffic": dom_traffic, "us_per_call": dom["us_per_call"], "algorithmic_bytes": dom["algorithmic_bytes"]}
+
+    kernels = {"q4k_gate_plus_up_one_launch": pair, "q4k_gate_up_swiglu_one_launch": pair_swiglu,
+               "q4k_gate_up_14336x4096": time_kernel(k_q4k, Q4_K, gate_up, xq, yg, F, H)}
     if not args.no_extra_kernels:
         kernels["q6k_down_4096x14336"] = time_kernel(k_q6k, Q6_K, [w["down"] for w in layers], hq, yd, H, F)
         kernels["q8_0_q_proj_4096x4096"] = time_kernel(k_q8, Q8_0, [w["q"] for w in layers], xq, yq, H, H)
@@ -439,11 +477,23 @@ def main():
             parity = None  # this variant keeps no Q8_0 buffers to compare stage by stage
         else:
             a_ref = O.quantize_q8_0(hx)
-            h_ref = O.quantize_q8_0(O.swiglu(g_y["gate"], g_y["up"]))
+            g_ref = O.matvec_q8_fused_mt(O.Q4_K, hw["gate"], g_xq, F, H, cores)
+            u_ref = O.matvec_q8_fused_mt(O.Q4_K, hw["up"], g_xq, F, H, cores)
             errs = {"q_proj": rel_err(g_y["q"], O.matvec_q8_fused_mt(O.Q8_0, hw["q"], g_xq, H, H, cores)),
-                    "ffn_gate": rel_err(g_y["gate"], O.matvec_q8_fused_mt(O.Q4_K, hw["gate"], g_xq, F, H, cores)),
-                    "ffn_up": rel_err(g_y["up"], O.matvec_q8_fused_mt(O.Q4_K, hw["up"], g_xq, F, H, cores)),
                     "ffn_down": rel_err(g_y["down"], O.matvec_q8_fused_mt(O.Q6_K, hw["down"], g_hq, H, F, cores))}
+            if args.unfused_swiglu:
+                errs["ffn_gate"], errs["ffn_up"] = rel_err(g_y["gate"], g_ref), rel_err(g_y["up"], u_ref)
+                h_ref = O.quantize_q8_0(O.swiglu(g_y["gate"], g_y["up"]))
+            else:  # the fused launch keeps gate / up in registers: compare h = silu(gate) * up instead
+                h_f32 = torch.empty(F, dtype=torch.float32, device=dev)
+                hq2 = torch.empty_like(hq)
+                with torch.cuda.stream(stream):
+                    linear.gate_up_swiglu_dev(Q4_K, layers[0]["gate"], layers[0]["up"], xq, h_f32, hq2, F, H)
+                    stream.synchronize()
+                g_h = h_f32.cpu().numpy()
+                errs["ffn_gate_up_swiglu_h"] = rel_err(g_h, O.swiglu(g_ref, u_ref))
+                h_ref = O.quantize_q8_0(g_h)
+                assert np.array_equal(hq2.cpu().numpy(), g_hq)
             parity = {"acts_q8_bytes_equal": bool(np.array_equal(g_xq, a_ref)),
                       "h_q8_bytes_equal_fraction": round(float(np.mean(g_hq == h_ref)), 6),
                       "fp32_max_err_over_ymax": {k: float(f"{v:.3e}") for k, v in errs.items()},
@@ -481,7 +531,8 @@ def main():
                    "weight_bytes_per_step": step_weight_bytes, "distinct_layers": L,
                    "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
                    "launch": "one HIP graph of all timed steps; per step " +
-                             ("quantize x, q_proj, gate+up (one launch), SwiGLU + quantize, down" if not args.fused_quantize
+                             ("quantize x, q_proj, gate+up+SwiGLU+quantize (one launch), down" if not (args.fused_quantize or args.unfused_swiglu)
+                              else "quantize x, q_proj, gate+up (one launch), SwiGLU + quantize, down" if not args.fused_quantize
                               else "q_proj, gate+up (one launch), SwiGLU, down, each projection quantizing its fp32 "
                                    "input vector to Q8_0 itself")},
         "roofline": roofline,

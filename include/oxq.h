@@ -322,6 +322,18 @@ int oxq_rmsnorm_quantize_q8_0_dev(const float *d_x, const float *d_weight, float
  * Three launches when gate and up share a format (gate + up, SwiGLU + quantize, down), four
  * otherwise.  Needs oxq_ffn_workspace_bytes() bytes of 256-byte-aligned device scratch;
  * allocates nothing and does not synchronise. */
+/* ffn_gate and ffn_up (both of `type`, [intermediate x hidden]) on one Q8_0 input, SwiGLU and the
+ * Q8_0 quantizer of the down projection's input in ONE launch: a work group owns 32 rows of both
+ * matrices, i.e. one block of h.  d_out_q8: intermediate / 32 * 34 bytes; d_h (optional): h in
+ * fp32.  The sums are those of oxq_matvec_q8_fused_dev bit for bit, so the bytes equal those of
+ * the separate calls.  UnsupportedShape when the type / row length has no such kernel (rows
+ * longer than 128 units, Q8_1 / IQ4_NL / Q2_K / Q3_K): use the separate calls.
+ * oxq_ffn_swiglu_dev takes this route by itself when gate and up share a type;
+ * oxq_set_ffn_fusion(0) switches that off (measurement only). */
+int oxq_ffn_gate_up_swiglu_q8_dev(uint32_t type, const uint8_t *d_gate, const uint8_t *d_up,
+                                  const uint8_t *d_acts_q8, float *d_h, uint8_t *d_out_q8,
+                                  size_t intermediate, size_t hidden, void *stream);
+int oxq_set_ffn_fusion(int enabled);
 size_t oxq_ffn_workspace_bytes(size_t hidden, size_t intermediate);
 int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_type,
                        const uint8_t *d_up, uint32_t down_type, const uint8_t *d_down,

@@ -139,6 +139,9 @@ SIGNATURES = {
                                                C.c_void_p]),
     "oxq_rmsnorm_quantize_q8_0_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_float, C.c_size_t, C.c_size_t,
                                                 C.c_void_p, C.c_void_p, C.c_void_p]),
+    "oxq_ffn_gate_up_swiglu_q8_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                                C.c_size_t, C.c_size_t, C.c_void_p]),
+    "oxq_set_ffn_fusion": (C.c_int, [C.c_int]),
     "oxq_ffn_workspace_bytes": (C.c_size_t, [C.c_size_t, C.c_size_t]),
     "oxq_ffn_swiglu_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p,
                                      C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t,

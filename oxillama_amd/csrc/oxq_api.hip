@@ -95,6 +95,7 @@ struct State {
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
     Scratch s_weights, s_acts, s_x, s_out, s_sums, s_work, s_bias, s_lora_a, s_lora_b, s_lora_r;
     Scratch s_moe_up, s_moe_down, s_moe_tables;
+    bool fuse_swiglu = true;  // oxq_ffn_swiglu_dev: gate, up, SwiGLU and the quantizer of h in one launch where possible
 };
 State g;
 
@@ -936,6 +937,29 @@ size_t oxq_ffn_workspace_bytes(size_t hidden, size_t intermediate) {
     return 2 * f + ((intermediate / 32 * 34 + 255) & ~(size_t)255);
 }
 
+int oxq_ffn_gate_up_swiglu_q8_dev(uint32_t type, const uint8_t *d_gate, const uint8_t *d_up, const uint8_t *d_acts_q8,
+                                  float *d_h, uint8_t *d_out_q8, size_t intermediate, size_t hidden, void *stream) {
+    int st;
+    if ((st = check_dev_shape(type, intermediate, hidden)) != OXQ_OK) return st;
+    if (intermediate % 32 != 0)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 32, intermediate, "intermediate size is not a multiple of 32");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (hidden == 0 || intermediate == 0) return OXQ_OK;
+    hipError_t e = oxq::launch_gate_up_swiglu(type, d_gate, d_up, d_acts_q8, d_out_q8, d_h, (uint32_t)intermediate,
+                                              (uint32_t)hidden, (hipStream_t)stream);
+    if (e == hipErrorNotSupported) {
+        (void)hipGetLastError();
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, hidden, "no fused gate/up kernel for this type and row length");
+    }
+    OXQ_HIP(e);
+    return OXQ_OK;
+}
+
+int oxq_set_ffn_fusion(int enabled) {
+    g.fuse_swiglu = enabled != 0;
+    return OXQ_OK;
+}
+
 int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_type, const uint8_t *d_up,
                        uint32_t down_type, const uint8_t *d_down, const uint8_t *d_acts_q8, float *d_out, size_t hidden,
                        size_t intermediate, void *d_workspace, size_t workspace_bytes, void *stream) {
@@ -956,6 +980,16 @@ int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_ty
     float *gate = (float *)d_workspace, *up = (float *)((uint8_t *)d_workspace + f);
     uint8_t *hq = (uint8_t *)d_workspace + 2 * f;
     hipStream_t s = (hipStream_t)stream;
+    if (gate_type == up_type && g.fuse_swiglu) {  // both projections, SwiGLU and the quantizer of h in one launch
+        hipError_t e = oxq::launch_gate_up_swiglu(gate_type, d_gate, d_up, d_acts_q8, hq, nullptr, (uint32_t)intermediate,
+                                                  (uint32_t)hidden, s);
+        if (e == hipSuccess) {
+            OXQ_HIP(oxq::launch_gemv_q8(down_type, gemv_args(d_down, hq, d_out, nullptr, hidden, intermediate, 0), s));
+            return OXQ_OK;
+        }
+        if (e != hipErrorNotSupported) return fail_hip(e, "launch_gate_up_swiglu");
+        (void)hipGetLastError();
+    }
     if (gate_type == up_type) {  // one pass of the launch machinery over both matrices
         oxq::GemvArgs a = gemv_args(d_gate, d_acts_q8, gate, nullptr, intermediate, hidden, 0);
         a.n_mats = 2;

@@ -68,6 +68,18 @@ bool gemv_takes_f32(uint32_t type, uint32_t n_cols) {
     return unit != 0 && (n_cols / unit + 63) / 64 <= 32 && (size_t)(n_cols / 32) * 34 <= 48 * 1024;
 }
 
+hipError_t launch_gate_up_swiglu(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts, uint8_t *hq,
+                                 float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream) {
+    switch (type) {
+    case OXQ_TYPE_Q4_0: return launch_gate_up_swiglu_format<FmtQ4_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    case OXQ_TYPE_Q8_0: return launch_gate_up_swiglu_format<FmtQ8_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    case OXQ_TYPE_Q4_K: return launch_gate_up_swiglu_format<FmtQ4K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    case OXQ_TYPE_Q6_K: return launch_gate_up_swiglu_format<FmtQ6K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    case OXQ_TYPE_IQ4_XS: return launch_gate_up_swiglu_format<FmtIQ4XS>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    default: return launch_gate_up_swiglu_more(type, Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    }
+}
+
 hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream) {
     if (a.n_rows == 0 || a.n_cols == 0) return hipSuccess;
     switch (type) {

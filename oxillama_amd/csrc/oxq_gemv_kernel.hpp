@@ -3,6 +3,7 @@
 #include <type_traits>
 
 #include "oxq_formats.hpp"
+#include "oxq_q8_encode.hpp"
 
 namespace oxq {
 
@@ -179,6 +180,62 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
         finish(r1, b1.old, next);
         batch = next2;
     }
+}
+
+// ffn_gate and ffn_up of the dense feed-forward block (crates/oxillama-arch/src/llama/model.rs:295-310)
+// with SwiGLU (swiglu.rs:15-21) and the Q8_0 quantizer of the down projection's input
+// (quantize.rs:58) in the same kernel.  A work group owns rows 32b..32b+31 of BOTH matrices -- one
+// Q8_0 block of h -- so nothing crosses work groups: wave w streams rows 8w..8w+7 of gate, then of
+// up (RB rows per batch, the next batch's loads in flight while one is reduced; one wave per row,
+// so the sums are those of gemv_q8_cached with KS = 1, bit for bit), the 64 sums meet in LDS and
+// eight lanes encode the block.  h_out (optional) receives h in fp32.
+template <class F, int STEPS, int RB, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8_t *__restrict__ Wg,
+                                                             const uint8_t *__restrict__ Wu,
+                                                             const void *__restrict__ A, uint8_t *__restrict__ hq,
+                                                             float *__restrict__ h_out, uint32_t n_rows, uint32_t units,
+                                                             size_t row_bytes) {
+    static_assert((RB == 1 || RB == 2) && (WAVES == 4 || WAVES == 8), "configuration");
+    constexpr int RPW = 32 / WAVES;  // rows of each matrix per wave
+    constexpr int NB = RPW / RB;     // batches per matrix and wave
+    __shared__ float row_sums[2][32];
+    const uint32_t lane = threadIdx.x & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const typename F::Lane k = F::lane_consts(lane);
+    typename F::Act act[STEPS];
+    {
+        const auto src = ActQ8::make(A);
+#pragma unroll
+        for (int s = 0; s < STEPS; s++) {
+            const uint32_t u = (uint32_t)(s * 64) + lane;
+            F::load_act(act[s], src, min(u, units - 1), u < units, k);
+        }
+    }
+    const uint32_t batch0 = (blockIdx.x * 32 + wave * RPW) / RB;
+    Batch<F, STEPS, RB> b[2];
+    load_batch<F, STEPS, RB>(b[0], Wg, nullptr, batch0, n_rows, row_bytes, units, 0, lane, k, false);
+#pragma unroll
+    for (int i = 0; i < 2 * NB; i++) {
+        if (i + 1 < 2 * NB)
+            load_batch<F, STEPS, RB>(b[(i + 1) & 1], i + 1 < NB ? Wg : Wu, nullptr, batch0 + (i + 1) % NB, n_rows, row_bytes,
+                                     units, 0, lane, k, false);
+        const float r = reduce_batch<F, STEPS, RB, false>(b[i & 1], act, nullptr, batch0 + i % NB, n_rows, units, 0, 0,
+                                                          lane, k);
+        if (lane < RB) row_sums[i / NB][wave * RPW + (i % NB) * RB + lane] = r;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    const uint32_t j = lane & 7;
+    float v[4];
+    for (int i = 0; i < 4; i++) {
+        const float g = row_sums[0][4 * j + i], u = row_sums[1][4 * j + i];
+        const float sigmoid = 1.0f / (1.0f + expf(-g));  // swiglu.rs:18
+        v[i] = g * sigmoid * u;                          // swiglu.rs:19
+    }
+    const bool writer = lane < 8;
+    if (writer && h_out)
+        for (int i = 0; i < 4; i++) h_out[(size_t)blockIdx.x * 32 + 4 * j + i] = v[i];
+    encode_q8_0_lanes(v, writer, hq + (size_t)blockIdx.x * 34, j);
 }
 
 // Several activation vectors against one weight stream (a small decode batch): NV vectors'

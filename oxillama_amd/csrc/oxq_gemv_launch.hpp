@@ -115,6 +115,29 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     return hipGetLastError();
 }
 
+// gate + up + SwiGLU + quantize in one launch: rows short enough for one wave per row (the
+// configurations launch_format gives KS = 1 and at most two steps), a whole number of 32-row blocks.
+template <class F>
+static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts, uint8_t *hq,
+                                               float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream) {
+    const uint32_t units = n_cols / F::UNIT_COLS;
+    const size_t row_bytes = (size_t)(n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
+    const uint32_t steps = (units + 63) / 64;
+    if (steps > 2 || n_rows % 32 != 0 || n_rows == 0) return hipErrorNotSupported;
+    const bool two = row_bytes <= F::TWO_ROW_BATCH_BYTES;
+    const dim3 grid(n_rows / 32);
+#define OXQ_LAUNCH(ST, RBV)                                                                                          \
+    hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4>), grid, dim3(256), 0, stream, Wg, Wu, acts, hq, h,     \
+                       n_rows, units, row_bytes)
+    if (steps == 1) {
+        if (two) OXQ_LAUNCH(1, 2); else OXQ_LAUNCH(1, 1);
+    } else {
+        if (two) OXQ_LAUNCH(2, 2); else OXQ_LAUNCH(2, 1);
+    }
+#undef OXQ_LAUNCH
+    return hipGetLastError();
+}
+
 // True when one launch can take the n_mats matrices of `a` (the register-cached kernel, whole
 // batches per matrix); otherwise the caller gets one launch per matrix.
 template <class F>

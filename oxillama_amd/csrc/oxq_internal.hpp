@@ -71,6 +71,12 @@ uint32_t gemv_unit_cols(uint32_t type);
 uint32_t gemv_group_cols(uint32_t type);
 // The formats beyond the first five live in a translation unit of their own.
 hipError_t launch_gemv_q8_more(uint32_t type, const GemvArgs &a, hipStream_t stream);
+// ffn_gate, ffn_up, SwiGLU and the Q8_0 quantizer of h in one launch (both matrices of `type`, n_rows a
+// multiple of 32).  hipErrorNotSupported: no such kernel for this type / row length.
+hipError_t launch_gate_up_swiglu(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts, uint8_t *hq,
+                                 float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream);
+hipError_t launch_gate_up_swiglu_more(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts,
+                                      uint8_t *hq, float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream);
 hipError_t launch_gemv_vecs_more(uint32_t type, const GemvVecsArgs &a, hipStream_t stream);
 
 // x: n floats (n % 32 == 0) -> n/32 Q8_0 blocks of 34 bytes.

@@ -132,6 +132,13 @@ def rmsnorm_quantize_dev(d_x, d_weight, eps, rows, n, d_y=None, d_out_q8=None):
                                                      _opt(d_y), _opt(d_out_q8), _stream()))
 
 
+def gate_up_swiglu_dev(tensor_type, d_gate, d_up, d_acts_q8, d_h, d_out_q8, intermediate, hidden):
+    """ffn_gate + ffn_up + SwiGLU + Q8_0 quantizer of h in one launch (d_h optional)."""
+    _check(capi.load().oxq_ffn_gate_up_swiglu_q8_dev(int(tensor_type), d_gate.data_ptr(), d_up.data_ptr(),
+                                                     d_acts_q8.data_ptr(), d_h.data_ptr() if d_h is not None else None,
+                                                     d_out_q8.data_ptr(), intermediate, hidden, HipKernel._stream()))
+
+
 def ffn_workspace_bytes(hidden, intermediate):
     return capi.load().oxq_ffn_workspace_bytes(hidden, intermediate)
 

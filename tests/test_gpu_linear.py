@@ -309,6 +309,14 @@ def test_ffn_swiglu(hip, ref, types):
         d_wg, d_wu, d_wd = dev(wg), dev(wu), dev(wd)
         L.ffn_swiglu_dev((tg, d_wg), (tu, d_wu), (td, d_wd), d_acts, d_out, hidden, inter, ws)
         got = host(d_out)
+        from oxillama_amd import capi
+        capi.load().oxq_set_ffn_fusion(0)  # gate + up, SwiGLU, down as three launches: the same bits
+        try:
+            d_out3 = torch.empty_like(d_out)
+            L.ffn_swiglu_dev((tg, d_wg), (tu, d_wu), (td, d_wd), d_acts, d_out3, hidden, inter, ws)
+            assert np.array_equal(got.view(np.uint32), host(d_out3).view(np.uint32))
+        finally:
+            capi.load().oxq_set_ffn_fusion(1)
         # step by step with the plain entry points: bit-identical
         g = torch.empty(inter, dtype=torch.float32, device=DEV)
         u = torch.empty(inter, dtype=torch.float32, device=DEV)
@@ -334,6 +342,51 @@ def test_ffn_swiglu(hip, ref, types):
         assert same > 0.999, f"only {same:.5f} of the h bytes match the oracle's SwiGLU of the same gate/up"
         down_ref = ref.matvec_q8_fused_mt(td, wd, host(hq), hidden, inter, 8)
         assert_close(got, down_ref, "down")
+
+
+@pytest.mark.parametrize("t", [O.Q4_K, O.Q6_K, O.Q8_0, O.Q4_0, O.IQ4_XS, O.Q5_K, O.Q4_1, O.Q5_0, O.Q5_1], ids=lambda t: O.NAMES[t])
+def test_gate_up_swiglu_one_launch(hip, ref, t):
+    """gate + up + SwiGLU + quantize in one launch: the bytes (and h) of the separate calls, bit for bit."""
+    for hidden, inter in ((256, 64), (4096, 14336), (2048, 5632)):
+        say("gate_up_swiglu", O.NAMES[t], hidden, inter)
+        if t in (O.Q4_K, O.Q6_K, O.Q8_0, O.Q4_0, O.IQ4_XS):
+            wg, wu = synth.weights(t, 21, inter, hidden), synth.weights(t, 22, inter, hidden)
+        else:
+            wg, wu = O.random_blocks(t, 21, inter, hidden), O.random_blocks(t, 22, inter, hidden)
+        x = synth.normal_f32(23, hidden)
+        d_acts = torch.empty(hidden // 32 * 34, dtype=torch.uint8, device=DEV)
+        hip.quantize_q8_0_dev(dev(x), d_acts)
+        d_wg, d_wu = dev(wg), dev(wu)
+        hq = torch.zeros(inter // 32 * 34, dtype=torch.uint8, device=DEV)
+        h = torch.zeros(inter, dtype=torch.float32, device=DEV)
+        L.gate_up_swiglu_dev(t, d_wg, d_wu, d_acts, h, hq, inter, hidden)
+        g = torch.empty(inter, dtype=torch.float32, device=DEV)
+        u = torch.empty(inter, dtype=torch.float32, device=DEV)
+        hip.HipKernel(t).matvec_q8_fused_dev(d_wg, d_acts, g, inter, hidden, accumulate=False)
+        hip.HipKernel(t).matvec_q8_fused_dev(d_wu, d_acts, u, inter, hidden, accumulate=False)
+        hq2 = torch.zeros_like(hq)
+        h2 = torch.zeros_like(h)
+        L.swiglu_quantize_dev(g, u, h2, hq2)
+        assert np.array_equal(host(hq), host(hq2))
+        assert np.array_equal(host(h).view(np.uint32), host(h2).view(np.uint32))
+        # and against the oracle: the SwiGLU of the oracle's own gate / up sums, within the fp32 bar
+        acts = host(d_acts)
+        h_ref = ref.swiglu(ref.matvec_q8_fused_mt(t, wg, acts, inter, hidden, 8),
+                           ref.matvec_q8_fused_mt(t, wu, acts, inter, hidden, 8))
+        assert_close(host(h), h_ref, "h")
+        hq3 = torch.zeros_like(hq)  # without the fp32 copy of h
+        L.gate_up_swiglu_dev(t, d_wg, d_wu, d_acts, None, hq3, inter, hidden)
+        assert np.array_equal(host(hq3), host(hq2))
+
+
+def test_gate_up_swiglu_unsupported(hip):
+    z = torch.zeros(1 << 20, dtype=torch.uint8, device=DEV)
+    with pytest.raises(hip.UnsupportedShape):  # rows of 16384 columns take four waves per row
+        L.gate_up_swiglu_dev(O.Q4_K, z, z, z, None, z, 32, 16384)
+    with pytest.raises(hip.UnsupportedShape):  # a format without the fused kernel
+        L.gate_up_swiglu_dev(O.Q2_K, z, z, z, None, z, 32, 256)
+    with pytest.raises(hip.UnsupportedShape):  # not whole Q8_0 blocks of h
+        L.gate_up_swiglu_dev(O.Q4_K, z, z, z, None, z, 48, 256)
 
 
 def test_ffn_swiglu_errors(hip):
