@@ -212,15 +212,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
         }
     }
     const uint32_t batch0 = (blockIdx.x * 32 + wave * RPW) / RB;
-    Batch<F, STEPS, RB> b[2];
-    load_batch<F, STEPS, RB>(b[0], Wg, nullptr, batch0, n_rows, row_bytes, units, 0, lane, k, false);
+    constexpr int AHEAD = 2;  // batches requested ahead of the one being reduced
+    Batch<F, STEPS, RB> b[AHEAD + 1];
+#pragma unroll
+    for (int i = 0; i < AHEAD; i++)
+        load_batch<F, STEPS, RB>(b[i], i < NB ? Wg : Wu, nullptr, batch0 + i % NB, n_rows, row_bytes, units, 0, lane, k, false);
 #pragma unroll
     for (int i = 0; i < 2 * NB; i++) {
-        if (i + 1 < 2 * NB)
-            load_batch<F, STEPS, RB>(b[(i + 1) & 1], i + 1 < NB ? Wg : Wu, nullptr, batch0 + (i + 1) % NB, n_rows, row_bytes,
-                                     units, 0, lane, k, false);
-        const float r = reduce_batch<F, STEPS, RB, false>(b[i & 1], act, nullptr, batch0 + i % NB, n_rows, units, 0, 0,
-                                                          lane, k);
+        if (i + AHEAD < 2 * NB)
+            load_batch<F, STEPS, RB>(b[(i + AHEAD) % (AHEAD + 1)], i + AHEAD < NB ? Wg : Wu, nullptr,
+                                     batch0 + (i + AHEAD) % NB, n_rows, row_bytes, units, 0, lane, k, false);
+        const float r = reduce_batch<F, STEPS, RB, false>(b[i % (AHEAD + 1)], act, nullptr, batch0 + i % NB, n_rows, units,
+                                                          0, 0, lane, k);
         if (lane < RB) row_sums[i / NB][wave * RPW + (i % NB) * RB + lane] = r;
     }
     __syncthreads();
