@@ -419,7 +419,12 @@ __device__ __forceinline__ void gemm_tile_body(
     __shared__ __align__(16) uint8_t lds_static[SC_BYTES > RED_BYTES ? SC_BYTES : RED_BYTES];
     float (*lds_sc)[8][NP][W_ROWS] = reinterpret_cast<float (*)[8][NP][W_ROWS]>(lds_static);
     const uint32_t nsb = k / 32, nblk = k / 256, ngrp = nblk * 4;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    // split k: the wave index as a scalar -- everything derived from it (the wave's k range, hence the scalar
+    // offsets of its buffer loads) must be known to be wave-uniform, or every load is wrapped in a waterfall
+    // loop.  The other shapes only form lane offsets from it and keep the plain value (measured: the prefill
+    // shapes lose a few per cent with the scalar form).
+    const uint32_t wave = SPLITK ? (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6)) : tid >> 6;
     const uint32_t c = lane & 31, h = lane >> 5;
     const uint32_t wm = SPLITK ? 0 : wave % WMX, wn = SPLITK ? 0 : wave / WMX;
     // super-blocks of this wave: all of them, or its quarter
@@ -791,7 +796,12 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
         if (rows > 64) return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
         // split k; 64 weight rows (or 64 tokens) per work group only where that still leaves every
         // compute unit at least one work group, else 32 x 32
-        if ((size_t)((a.n + 63) / 64) * (a.offsets ? a.n_experts : 1) < device_cus())
+        const size_t groups = a.offsets ? a.n_experts : 1;
+        // 33..64 tokens: one 64-token tile where 32-row tiles still give every compute unit a work group
+        // (14336 x 4096, 64 rows: 26.6 us against 31.1 with 32 x 32 tiles; 4096 rows: 61 against 50)
+        if (rows > 32 && (size_t)((a.n + 31) / 32) * groups >= device_cus())
+            return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
+        if ((size_t)((a.n + 63) / 64) * groups < device_cus())
             return launch_tile<F, 1, 1, 0, 2, false, 2, 2>(a, p, stream);
         if (rows > 32) return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
         return launch_tile<F, 1, 2, 0, 2, false, 2, 2>(a, p, stream);
