@@ -787,10 +787,11 @@ size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t 
     return oxq::gemm_workspace_bytes((uint32_t)total_rows, (uint32_t)k);
 }
 
-int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
-                        const uint8_t *d_acts_q8, const int32_t *d_row_offsets, size_t total_rows,
-                        size_t max_rows_per_expert, float *d_out, int32_t *d_sums, size_t n, size_t k, int accumulate,
-                        void *d_workspace, size_t workspace_bytes, void *stream) {
+// prepared_for: format id of an immediately preceding call on the same activations and workspace (0: none).
+static int moe_gemm_impl(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
+                         const uint8_t *d_acts_q8, const int32_t *d_row_offsets, size_t total_rows,
+                         size_t max_rows_per_expert, float *d_out, int32_t *d_sums, size_t n, size_t k, int accumulate,
+                         void *d_workspace, size_t workspace_bytes, void *stream, uint32_t prepared_for) {
     int st = check_dev_shape(type, n, k);
     if (st != OXQ_OK) return st;
     if (total_rows > 0x7FFFFFFFull || n_experts > 65535)
@@ -829,8 +830,17 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
         ga.shape_rows = (uint32_t)(2 * mean < total_rows ? 2 * mean : total_rows);
     }
     ga.w_stride = expert_stride_bytes;
+    ga.prepared_for = prepared_for;
     OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
     return OXQ_OK;
+}
+
+int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
+                        const uint8_t *d_acts_q8, const int32_t *d_row_offsets, size_t total_rows,
+                        size_t max_rows_per_expert, float *d_out, int32_t *d_sums, size_t n, size_t k, int accumulate,
+                        void *d_workspace, size_t workspace_bytes, void *stream) {
+    return moe_gemm_impl(type, d_weights, expert_stride_bytes, n_experts, d_acts_q8, d_row_offsets, total_rows,
+                         max_rows_per_expert, d_out, d_sums, n, k, accumulate, d_workspace, workspace_bytes, stream, 0);
 }
 
 // ---- the callers' side: QuantLinear, SwiGLU feed-forward, RMSNorm ------------------------
@@ -1114,9 +1124,9 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
                                   max_rows_per_expert, gate, nullptr, intermediate, hidden, 0, ws + l.gemm, gws,
                                   stream)) != OXQ_OK)
         return st;
-    if ((st = oxq_moe_gemm_q8_dev(up_type, d_up, up_stride_bytes, n_experts, acts, d_row_offsets, pairs,
-                                  max_rows_per_expert, up, nullptr, intermediate, hidden, 0, ws + l.gemm, gws,
-                                  stream)) != OXQ_OK)
+    // up reads the activations gate just re-laid out in the workspace
+    if ((st = moe_gemm_impl(up_type, d_up, up_stride_bytes, n_experts, acts, d_row_offsets, pairs, max_rows_per_expert, up,
+                            nullptr, intermediate, hidden, 0, ws + l.gemm, gws, stream, gate_type)) != OXQ_OK)
         return st;
     OXQ_HIP(oxq::launch_swiglu_quantize(gate, up, pairs * intermediate, nullptr, hq, s));
     if ((st = oxq_moe_gemm_q8_dev(down_type, d_down, down_stride_bytes, n_experts, hq, d_row_offsets, pairs,

@@ -93,22 +93,31 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
     float *P = reinterpret_cast<float *>(q8t + (size_t)nsb * mpad * 32);
     uint16_t *da16 = reinterpret_cast<uint16_t *>(q8t + (size_t)nsb * mpad * 36);
     const dim3 pgrid((mpad * nsb + 255) / 256);
-    const int perm = type == OXQ_TYPE_Q6_K ? TileQ6K::ACT_PERM
-                     : (type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q4_0) ? TileIQ4XS::ACT_PERM
-                     : (type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_Q8_0) ? 0 : tile_act_perm_more(type);
-    // formats with a 16-weight zero-point term also need P per half block
-    float *p16 = tile_needs_p16_more(type)
-                     ? reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(P) + tile_p16_offset(nsb, mpad))
-                     : nullptr;
-    if (perm == 2)
-        hipLaunchKernelGGL(gemm_prep_acts<2>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
-    else if (perm == 1)
-        hipLaunchKernelGGL(gemm_prep_acts<1>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
-    else
-        hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    auto act_perm = [](uint32_t t) {
+        return t == OXQ_TYPE_Q6_K ? TileQ6K::ACT_PERM
+               : (t == OXQ_TYPE_IQ4_XS || t == OXQ_TYPE_Q4_0) ? TileIQ4XS::ACT_PERM
+               : (t == OXQ_TYPE_Q4_K || t == OXQ_TYPE_Q8_0) ? 0 : tile_act_perm_more(t);
+    };
+    const int perm = act_perm(type);
     const TilePlan plan = {q8t, P, da16, mpad};
+    // the previous call left the same activations in the same byte order (and the half-block planes if this
+    // format needs them): go straight to the tile kernel
+    const bool prepared = a.prepared_for != 0 && act_perm(a.prepared_for) == perm &&
+                          (!tile_needs_p16_more(type) || tile_needs_p16_more(a.prepared_for));
+    if (!prepared) {
+        // formats with a 16-weight zero-point term also need P per half block
+        float *p16 = tile_needs_p16_more(type)
+                         ? reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(P) + tile_p16_offset(nsb, mpad))
+                         : nullptr;
+        if (perm == 2)
+            hipLaunchKernelGGL(gemm_prep_acts<2>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
+        else if (perm == 1)
+            hipLaunchKernelGGL(gemm_prep_acts<1>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
+        else
+            hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     switch (type) {
     case OXQ_TYPE_Q4_K: return launch_tiles<TileQ4K>(a, plan, stream);
     case OXQ_TYPE_IQ4_XS: return launch_tiles<TileIQ4XS>(a, plan, stream);

@@ -124,6 +124,8 @@ struct GemmArgs {
     uint32_t n_experts = 0;
     uint32_t max_rows = 0;             // upper bound of the rows of any one expert (sizes the grid)
     uint32_t shape_rows = 0;           // rows per expert the tile shape is chosen for (<= max_rows)
+    uint32_t prepared_for = 0;         // tile kernel: the workspace already holds these activations, re-laid out for
+                                       // this format id by the previous call (0: none); same layout -> no second pass
     size_t w_stride = 0;
 };
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
