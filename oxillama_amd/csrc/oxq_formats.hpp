@@ -423,7 +423,11 @@ struct FmtIQ4XS {
         const uint32_t sel = idx & 0x07070707u;
         const uint32_t lo = __builtin_amdgcn_perm(T1, T0, sel);
         const uint32_t hi = __builtin_amdgcn_perm(T3, T2, sel);
-        return __builtin_amdgcn_perm(hi, lo, 0x03020100u | ((idx >> 1) & 0x04040404u));
+        // the identity selector in a vector register: (x >> 1 & mask) | base is then one v_and_or_b32 (an
+        // instruction takes a single scalar operand, and both constants would be scalars otherwise)
+        uint32_t base;
+        asm("v_mov_b32 %0, 0x03020100" : "=v"(base));
+        return __builtin_amdgcn_perm(hi, lo, ((idx >> 1) & 0x04040404u) | base);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &k, int32_t *sums,
