@@ -310,3 +310,44 @@ def want_all(ref, layer, router, wg, wu, wd, xt):
                                              ref.matvec_q8_fused(layer.up[0], wu[e * sg:(e + 1) * sg], xq, inter, hidden)))
         acc = acc + np.float32(w) * ref.matvec_q8_fused(layer.down[0], wd[e * sd:(e + 1) * sd], eo_in, hidden, inter)
     return acc
+
+
+def test_moe_layer_full_size_c5(hip, ref):
+    """The whole layer at the C5 size (IQ4_XS, 8 experts of 14336 x 4096 / 4096 x 14336, 64 tokens, top-2): routing
+    exact for every token; for three tokens the layer's output against the oracle's MoeFfn::forward on quantized
+    experts (end-to-end bar), and the size-independent property that the weights of a token sum to one."""
+    n_exp, top_k, n_tok, hidden, inter = 8, 2, 64, 4096, 14336
+    t = O.IQ4_XS
+    say("moe layer C5 full size: generating 749 MB of expert weights")
+    wg = np.concatenate([synth.weights(t, 7000 + e, inter, hidden) for e in range(n_exp)])
+    wu = np.concatenate([synth.weights(t, 7100 + e, inter, hidden) for e in range(n_exp)])
+    wd = np.concatenate([synth.weights(t, 7200 + e, hidden, inter) for e in range(n_exp)])
+    stride = wg.size // n_exp
+    router = synth.normal_f32(9, n_exp * hidden, 0.05)
+    x = synth.normal_f32(7, n_tok * hidden)
+    d, k = route_on_device(router, x, n_tok, n_exp, hidden, top_k)
+    experts, weights = host(d["experts"]), host(d["weights"])
+    for tk in range(n_tok):
+        sel, wt = ref.moe_route(router, n_exp, hidden, top_k, x[tk * hidden:(tk + 1) * hidden])
+        assert experts[tk].tolist() == sel.tolist() and np.max(np.abs(weights[tk] - wt)) <= 1e-5
+    assert np.all(np.abs(weights.sum(axis=1) - 1) < 1e-5)
+    ws = torch.empty(moe.moe_ffn_workspace_bytes((t, t, t), n_tok * k, hidden, inter), dtype=torch.uint8, device=DEV)
+    d_out = torch.empty(n_tok * hidden, dtype=torch.float32, device=DEV)
+    d_wg, d_wu, d_wd = dev(wg), dev(wu), dev(wd)
+    say("moe layer C5 full size: device run")
+    moe.moe_ffn_dev((t, d_wg, stride), (t, d_wu, stride), (t, d_wd, stride), n_exp, dev(x), n_tok, k, d["offsets"],
+                    d["pair_token"], d["token_rows"], d["weights"], 0, d_out, hidden, inter, ws)
+    got = host(d_out).reshape(n_tok, hidden)
+    assert np.all(np.isfinite(got))
+    for tk in (0, 31, 63):
+        say("moe layer C5 full size: oracle token", tk)
+        xt = x[tk * hidden:(tk + 1) * hidden]
+        xq = ref.quantize_q8_0(xt)
+        acc = np.zeros(hidden, np.float32)
+        for j, e in enumerate(experts[tk]):
+            g = ref.matvec_q8_fused_mt(t, wg[e * stride:(e + 1) * stride], xq, inter, hidden, 16)
+            u = ref.matvec_q8_fused_mt(t, wu[e * stride:(e + 1) * stride], xq, inter, hidden, 16)
+            hq = ref.quantize_q8_0(ref.swiglu(g, u))
+            eo = ref.matvec_q8_fused_mt(t, wd[e * stride:(e + 1) * stride], hq, hidden, inter, 16)
+            acc = acc + weights[tk, j] * eo
+        assert_close(got[tk], acc, f"token {tk}", tol=2e-3)
