@@ -13,9 +13,15 @@
  * ceil(n_cols / block_size) * block_bytes (Q/reference/q4_k.rs:130-131).  They go
  * to HBM unchanged; nothing is repacked.
  *
- * Supported formats: Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS.  Shapes whose n_cols is not
- * a multiple of the format's block size return OXQ_ERR_UNSUPPORTED_SHAPE so the
- * caller can fall back to its CPU kernel.
+ * Rows that end inside a block (n_cols not a multiple of the block size): the
+ * matvec, gemv and gemm entry points, on host slices and on device pointers, skip
+ * the columns past n_cols as the reference's kernels do (Q/reference/q4_k.rs:307-321,
+ * Q/traits.rs:150-166) -- whole blocks are stored and read, whole Q8_0 activation
+ * blocks are expected (their bytes past n_cols are ignored).  The fused layers
+ * (feed-forward, mixture of experts, QuantLinear on device pointers), the grouped
+ * matmul, the GGUF loader and the debug dumps of the group sums take whole blocks
+ * only and return OXQ_ERR_UNSUPPORTED_SHAPE otherwise, so that the caller can fall
+ * back to its CPU kernel.
  *
  * Thread safety: every function may be called from several host threads; calls
  * taking host slices serialise on an internal lock.
@@ -130,7 +136,9 @@ int oxq_matvec_q8_fused(uint32_t type, const uint8_t *weights, size_t weights_le
  * The activation vector is quantized to Q8_0 on the GPU and fed to the fused
  * kernel: results equal oxq_quantize_f32_to_q8_0 + oxq_matvec_q8_fused into
  * zeros, and differ from the reference's f32-activation gemv by the Q8_0
- * rounding of the input.  n_cols must be a multiple of 32. */
+ * rounding of the input.  Where n_cols is not a multiple of the block size the
+ * input is taken as zero-padded to whole blocks (the reference's gemv skips those
+ * columns, Q/reference/q4_k.rs:161,168). */
 int oxq_gemv(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape,
              size_t n_dims, const float *input, size_t input_len, float *output,
              size_t output_len);

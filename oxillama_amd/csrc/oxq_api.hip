@@ -163,8 +163,10 @@ struct FusedShape {
 
 // Validation order of the reference's matvec_q8_fused
 // (crates/oxillama-quant/src/reference/q4_k.rs:226-250, traits.rs:99-130).
+// whole_blocks: refuse rows that end inside a block (the debug dump of the group sums needs whole groups);
+// the matvec itself takes them as the reference does, skipping the columns past n_cols.
 int validate_fused(uint32_t type, size_t weights_len, size_t acts_len, size_t out_len, size_t n_rows,
-                   size_t n_cols, FusedShape *fs) {
+                   size_t n_cols, FusedShape *fs, bool whole_blocks) {
     if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
     if (out_len < n_rows) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_rows, out_len, "out shorter than n_rows");
     const size_t bs = oxq_block_size(type), bb = oxq_block_bytes(type);
@@ -175,10 +177,10 @@ int validate_fused(uint32_t type, size_t weights_len, size_t acts_len, size_t ou
         return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * fs->row_bytes, weights_len, "weights buffer too small");
     if (acts_len < fs->acts_needed)
         return fail(OXQ_ERR_BUFFER_TOO_SMALL, fs->acts_needed, acts_len, "activation buffer too small");
-    if (n_cols % bs != 0)
+    if (whole_blocks && n_cols % bs != 0)
         return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
-    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull)
-        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows > n_cols ? n_rows : n_cols, "dimension exceeds 2^32-1");
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFF00ull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFF00ull, n_rows > n_cols ? n_rows : n_cols, "dimension exceeds 2^32-257");
     return OXQ_OK;
 }
 
@@ -464,7 +466,7 @@ int oxq_quantize_f32_to_q8_0(const float *data, size_t n, uint8_t *out, size_t o
 int oxq_matvec_q8_fused(uint32_t type, const uint8_t *weights, size_t weights_len, const uint8_t *acts_q8,
                         size_t acts_len, float *out, size_t out_len, size_t n_rows, size_t n_cols) {
     FusedShape fs;
-    int st = validate_fused(type, weights_len, acts_len, out_len, n_rows, n_cols, &fs);
+    int st = validate_fused(type, weights_len, acts_len, out_len, n_rows, n_cols, &fs, false);
     if (st != OXQ_OK) return st;
     if (n_rows == 0 || n_cols == 0) return OXQ_OK;
     if ((st = ensure_init()) != OXQ_OK) return st;
@@ -484,7 +486,7 @@ int oxq_matvec_q8_fused(uint32_t type, const uint8_t *weights, size_t weights_le
 int oxq_block_sums(uint32_t type, const uint8_t *weights, size_t weights_len, const uint8_t *acts_q8,
                    size_t acts_len, int32_t *sums, size_t sums_len, size_t n_rows, size_t n_cols) {
     FusedShape fs;
-    int st = validate_fused(type, weights_len, acts_len, n_rows, n_rows, n_cols, &fs);
+    int st = validate_fused(type, weights_len, acts_len, n_rows, n_rows, n_cols, &fs, true);
     if (st != OXQ_OK) return st;
     const size_t groups = n_cols / oxq::gemv_group_cols(type);
     if (sums_len < n_rows * groups) return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * groups, sums_len, "sums buffer too small");
@@ -520,22 +522,25 @@ static int gemm_host(uint32_t type, const uint8_t *data, size_t data_len, const 
     const size_t bpr = (n_cols + bs - 1) / bs, row_bytes = bpr * bb;
     if (data_len < n_rows * row_bytes)
         return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * row_bytes, data_len, "tensor data too small");
-    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
     if (n_rows == 0 || n_cols == 0) return OXQ_OK;
-    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull || m > 0xFFFFFFFFull)
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFF00ull || m > 0xFFFFFFFFull)
         return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows, "dimension exceeds 2^32-1");
     if ((st = ensure_init()) != OXQ_OK) return st;
     std::lock_guard<std::mutex> lock(g.mu);
     const uint8_t *dW = nullptr;
     if ((st = stage_weights(type, data, n_rows * row_bytes, &dW)) != OXQ_OK) return st;
-    const size_t act_row_bytes = n_cols / 32 * 34;
-    if ((st = g.s_x.reserve(m * n_cols * sizeof(float))) != OXQ_OK) return st;
+    // A row that ends inside a block (the reference's gemv skips the columns past n_cols,
+    // reference/q4_k.rs:161,168): the input rows are staged zero-padded to whole blocks, so the padding
+    // quantizes to zero bytes and the kernels mask it besides.
+    const size_t k_pad = bpr * bs, act_row_bytes = k_pad / 32 * 34;
+    if ((st = g.s_x.reserve(m * k_pad * sizeof(float))) != OXQ_OK) return st;
     if ((st = g.s_acts.reserve(m * act_row_bytes)) != OXQ_OK) return st;
     if ((st = g.s_out.reserve(m * n_rows * sizeof(float))) != OXQ_OK) return st;
     // Gather the first n_cols floats of each input row (k may exceed n_cols).
-    OXQ_HIP(hipMemcpy2D(g.s_x.ptr, n_cols * sizeof(float), input, k * sizeof(float), n_cols * sizeof(float), m,
+    if (k_pad != n_cols) OXQ_HIP(hipMemset(g.s_x.ptr, 0, m * k_pad * sizeof(float)));
+    OXQ_HIP(hipMemcpy2D(g.s_x.ptr, k_pad * sizeof(float), input, k * sizeof(float), n_cols * sizeof(float), m,
                         hipMemcpyHostToDevice));
-    OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, m * n_cols, (uint8_t *)g.s_acts.ptr, nullptr));
+    OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, m * k_pad, (uint8_t *)g.s_acts.ptr, nullptr));
     oxq::GemmArgs ga;
     ga.W = dW;
     ga.A = (const uint8_t *)g.s_acts.ptr;
@@ -601,7 +606,6 @@ int oxq_weights_register(uint32_t type, size_t n_rows, size_t n_cols, const uint
     const size_t bs = oxq_block_size(type), bb = oxq_block_bytes(type);
     const size_t need = n_rows * ((n_cols + bs - 1) / bs) * bb;
     if (len < need) return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, len, "weights buffer too small");
-    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
     int st = ensure_init();
     if (st != OXQ_OK) return st;
     oxq_weights *w = new (std::nothrow) oxq_weights{type, n_rows, n_cols, need, nullptr};
@@ -638,18 +642,21 @@ int oxq_quantize_q8_0_dev(const float *d_x, size_t n_total, uint8_t *d_out, void
     return OXQ_OK;
 }
 
-static int check_dev_shape(uint32_t type, size_t n_rows, size_t n_cols) {
+// ragged_ok: the entry point takes rows that end inside a block (the plain matvec / gemv / gemm, which skip the
+// columns past n_cols as the reference does); the fused layers and the debug dumps want whole blocks.
+static int check_dev_shape(uint32_t type, size_t n_rows, size_t n_cols, bool ragged_ok = false) {
     if (!known_type(type)) return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "unsupported quantization type");
     const size_t bs = oxq_block_size(type);
-    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
-    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull)
-        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows, "dimension exceeds 2^32-1");
+    if (!ragged_ok && n_cols % bs != 0)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFF00ull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFF00ull, n_rows, "dimension exceeds 2^32-257");
     return OXQ_OK;
 }
 
 int oxq_matvec_q8_fused_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out,
                             size_t n_rows, size_t n_cols, int accumulate, void *stream) {
-    int st = check_dev_shape(type, n_rows, n_cols);
+    int st = check_dev_shape(type, n_rows, n_cols, true);
     if (st != OXQ_OK) return st;
     if ((st = ensure_init()) != OXQ_OK) return st;
     OXQ_HIP(oxq::launch_gemv_q8(type, gemv_args(d_weights, d_acts_q8, d_out, nullptr, n_rows, n_cols, accumulate ? 1 : 0),
@@ -660,7 +667,7 @@ int oxq_matvec_q8_fused_dev(uint32_t type, const uint8_t *d_weights, const uint8
 int oxq_matvec_q8_fused_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_weights,
                                   const uint8_t *d_acts_q8, float *const *d_outs, size_t n_rows, size_t n_cols,
                                   int accumulate, void *stream) {
-    int st = check_dev_shape(type, n_rows, n_cols);
+    int st = check_dev_shape(type, n_rows, n_cols, true);
     if (st != OXQ_OK) return st;
     if (n_mats == 0) return OXQ_OK;
     if (n_mats > 4) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 4, n_mats, "at most 4 matrices per call");
@@ -678,7 +685,7 @@ int oxq_matvec_q8_fused_multi_dev(uint32_t type, size_t n_mats, const uint8_t *c
 
 int oxq_gemv_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_weights, const float *d_x,
                        float *const *d_outs, size_t n_rows, size_t n_cols, int accumulate, void *stream) {
-    int st = check_dev_shape(type, n_rows, n_cols);
+    int st = check_dev_shape(type, n_rows, n_cols, true);
     if (st != OXQ_OK) return st;
     if (n_mats == 0) return OXQ_OK;
     if (n_mats > 4) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 4, n_mats, "at most 4 matrices per call");
@@ -726,7 +733,7 @@ size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k) 
 static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, int32_t *d_sums,
                     size_t m, size_t n, size_t k, int accumulate, const float *d_bias, void *d_workspace,
                     size_t workspace_bytes, void *stream) {
-    int st = check_dev_shape(type, n, k);
+    int st = check_dev_shape(type, n, k, true);
     if (st != OXQ_OK) return st;
     if (m > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, m, "dimension exceeds 2^32-1");
     if ((st = ensure_init()) != OXQ_OK) return st;

@@ -42,17 +42,35 @@ __device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
 //    crates/oxillama-quant/src/traits.rs:39-44) -- and its waves read the blocks from there.
 struct ActQ8 {
     const uint8_t *A;
-    static __device__ __forceinline__ ActQ8 make(const void *p) { return ActQ8{static_cast<const uint8_t *>(p)}; }
+    uint32_t n_cols;  // columns that exist: the payload bytes of columns past them read as zero
+    static __device__ __forceinline__ ActQ8 make(const void *p, uint32_t n_cols) {
+        return ActQ8{static_cast<const uint8_t *>(p), n_cols};
+    }
+    // Bytes off..off+3 of a block of which only the first `rem` columns exist.
+    static __device__ __forceinline__ uint32_t tail_mask(uint32_t rem, uint32_t off) {
+        const uint32_t keep = rem > off ? min(rem - off, 4u) : 0u;
+        return keep >= 4 ? 0xFFFFFFFFu : (1u << (8 * keep)) - 1u;
+    }
     __device__ __forceinline__ void block(uint32_t b, u32x4 &q0, u32x4 &q1, uint32_t &dbits) const {
         const uint8_t *blk = A + (size_t)b * Q8_BLOCK_BYTES;
         q0 = ld16(blk + 2);
         q1 = ld16(blk + 18);
         dbits = ld2(blk);
+        // A row that ends inside a block: the reference skips the columns past n_cols
+        // (crates/oxillama-quant/src/reference/q4_k.rs:307-321, traits.rs:150-166), which is a dot
+        // product with zero activations there.  Never taken when n_cols is a whole number of blocks.
+        if (32 * b + 32 > n_cols) {
+            const uint32_t rem = n_cols > 32 * b ? n_cols - 32 * b : 0;
+            for (int i = 0; i < 4; i++) {
+                q0[i] &= tail_mask(rem, 4 * i);
+                q1[i] &= tail_mask(rem, 16 + 4 * i);
+            }
+        }
     }
 };
 struct ActF32 {
     const float *X;
-    static __device__ __forceinline__ ActF32 make(const void *p) { return ActF32{static_cast<const float *>(p)}; }
+    static __device__ __forceinline__ ActF32 make(const void *p, uint32_t) { return ActF32{static_cast<const float *>(p)}; }
 };
 // The blocks ActF32 stands for, once the work group has quantized them into LDS
 // (quantize_to_lds): 32 payload bytes per block, 32-byte aligned, and the f16 scales apart.
@@ -68,19 +86,23 @@ struct ActLds {
 
 // All 256 threads of a work group quantize n_blocks * 32 floats into LDS: eight lanes per
 // block, four floats per lane, exactly as quantize_q8_0_kernel does.
-__device__ __forceinline__ void quantize_to_lds(const float *__restrict__ x, uint32_t n_blocks, uint32_t *lds_q,
-                                                uint16_t *lds_d) {
+__device__ __forceinline__ void quantize_to_lds(const float *__restrict__ x, uint32_t n_blocks, uint32_t n_cols,
+                                                uint32_t *lds_q, uint16_t *lds_d) {
     const uint32_t j = threadIdx.x & 7;
     for (uint32_t base = 0; base < n_blocks; base += 32) {
         const uint32_t blk = base + (threadIdx.x >> 3);
         const bool valid = blk < n_blocks;
         float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (valid) {
-            const u32x4 raw = *reinterpret_cast<const u32x4 *>(x + (size_t)blk * 32 + 4 * j);
+        const uint32_t col = blk * 32 + 4 * j;
+        if (valid && col + 4 <= n_cols) {
+            const u32x4 raw = *reinterpret_cast<const u32x4 *>(x + col);
             for (int i = 0; i < 4; i++) {
                 const uint32_t bits = raw[i];  // copy out first: bit_cast must not see the vector element lvalue
                 v[i] = __builtin_bit_cast(float, bits);
             }
+        } else if (valid) {  // the row ends inside these four: the columns past it count as 0.0
+            for (int i = 0; i < 4; i++)
+                if (col + i < n_cols) v[i] = x[col + i];
         }
         float m = 0.0f;
         for (int i = 0; i < 4; i++) m = fmaxf(m, fabsf(v[i]));

@@ -8,7 +8,9 @@ namespace oxq {
 // Without the tile kernel (very few rows, or a shape it does not take): GEMV launches, two to
 // four activation rows per pass over the weights where the row length allows.
 static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t stream) {
-    const size_t act_row_bytes = (size_t)(a.k / 32) * 34;
+    // Q8_0 blocks per activation row: whole weight blocks' worth, also where a row ends inside one
+    const size_t bs = oxq_block_size(type);
+    const size_t act_row_bytes = ((size_t)a.k + bs - 1) / bs * (bs / 32) * 34;
     const uint32_t vecs = gemv_vecs_max(type, a.k);
     uint32_t r = 0;
     while (r < a.m) {

@@ -43,7 +43,8 @@ uint32_t gemv_group_cols(uint32_t type) {
 uint32_t gemv_vecs_max(uint32_t type, uint32_t n_cols) {
     const uint32_t unit = gemv_unit_cols(type);
     if (unit == 0) return 0;
-    const uint32_t steps = (n_cols / unit + 63) / 64;
+    const uint32_t bs = (uint32_t)oxq_block_size(type);
+    const uint32_t steps = ((n_cols + bs - 1) / bs * (bs / unit) + 63) / 64;
     if (steps == 1 || steps == 3 || steps == 4) return 4;
     if (steps == 2 || (steps >= 5 && steps <= 8)) return 2;
     return 0;
@@ -65,7 +66,9 @@ hipError_t launch_gemv_vecs(uint32_t type, const GemvVecsArgs &a, hipStream_t st
 bool gemv_takes_f32(uint32_t type, uint32_t n_cols) {
     const uint32_t unit = gemv_unit_cols(type);
     // the register-cached kernel (up to 8 steps, or 4 waves x 8) and the default dynamic LDS limit
-    return unit != 0 && (n_cols / unit + 63) / 64 <= 32 && (size_t)(n_cols / 32) * 34 <= 48 * 1024;
+    if (unit == 0) return false;
+    const uint32_t bs = (uint32_t)oxq_block_size(type), units = (n_cols + bs - 1) / bs * (bs / unit);
+    return (units + 63) / 64 <= 32 && (size_t)units * (unit / 32) * 34 <= 48 * 1024;
 }
 
 hipError_t launch_gate_up_swiglu(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts, uint8_t *hq,

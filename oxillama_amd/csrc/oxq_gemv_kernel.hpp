@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
                                                      const void *__restrict__ A, int32_t *__restrict__ sums,
                                                      uint32_t n_rows0, uint32_t n_rows1, uint32_t n_rows2,
                                                      uint32_t n_rows3, uint32_t units, uint32_t groups_per_row,
-                                                     size_t row_bytes) {
+                                                     size_t row_bytes, uint32_t n_cols) {
     static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
     // Up to four matrices of one format and row length that share the activation vector (wq/wk/wv,
     // ffn_gate/ffn_up) ride in one launch: blockIdx.y picks the matrix, and each matrix gets
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
                                  want_old);
         const uint32_t nb = units * (F::UNIT_COLS / 32);
         uint16_t *lds_d = reinterpret_cast<uint16_t *>(lds_acts + (size_t)nb * 8);
-        quantize_to_lds(static_cast<const float *>(A), nb, lds_acts, lds_d);
+        quantize_to_lds(static_cast<const float *>(A), nb, n_cols, lds_acts, lds_d);
         __syncthreads();
         if (KS == 1 && group >= n_batches) return;
         load_acts(ActLds{reinterpret_cast<const u32x4 *>(lds_acts), lds_d});
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
         if (KS == 1 && group >= n_batches) return;
         // Activations first (they sit in L2 and arrive early), then the first batch of
         // weights: the activation constants are derived while HBM is being read.
-        load_acts(SRC::make(A));
+        load_acts(SRC::make(A, n_cols));
         load_batch<F, STEPS, RB>(b0, W, old, min(group, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k,
                                  want_old);
     }
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
                                                              const uint8_t *__restrict__ Wu,
                                                              const void *__restrict__ A, uint8_t *__restrict__ hq,
                                                              float *__restrict__ h_out, uint32_t n_rows, uint32_t units,
-                                                             size_t row_bytes) {
+                                                             size_t row_bytes, uint32_t n_cols) {
     static_assert((RB == 1 || RB == 2) && (WAVES == 4 || WAVES == 8), "configuration");
     constexpr int RPW = 32 / WAVES;  // rows of each matrix per wave
     constexpr int NB = RPW / RB;     // batches per matrix and wave
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
     const typename F::Lane k = F::lane_consts(lane);
     typename F::Act act[STEPS];
     {
-        const auto src = ActQ8::make(A);
+        const auto src = ActQ8::make(A, n_cols);
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
             const uint32_t u = (uint32_t)(s * 64) + lane;
@@ -249,7 +249,8 @@ template <class F, int STEPS, int KS, int NV>
 __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ W, const uint8_t *__restrict__ A,
                                                    size_t a_stride, float *__restrict__ out, size_t out_stride,
                                                    uint32_t n_rows, uint32_t units, size_t row_bytes,
-                                                   int accumulate, uint32_t n_vecs, const float *__restrict__ bias) {
+                                                   int accumulate, uint32_t n_vecs, const float *__restrict__ bias,
+                                                   uint32_t n_cols) {
     static_assert((KS == 1 || KS == 4) && NV >= 2 && NV <= 4, "configuration");
     // n_vecs <= NV: the surplus slots repeat the last vector (same loads, same stored values)
     constexpr uint32_t G = 4 / KS;
@@ -270,7 +271,7 @@ __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ 
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
             const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
-            F::load_act(act[v][s], ActQ8{A + (size_t)min((uint32_t)v, n_vecs - 1) * a_stride}, min(u, units - 1),
+            F::load_act(act[v][s], ActQ8{A + (size_t)min((uint32_t)v, n_vecs - 1) * a_stride, n_cols}, min(u, units - 1),
                         u < units, k);
         }
     auto load_row = [&](typename F::Wt (&w)[STEPS], uint32_t row) {
@@ -340,7 +341,7 @@ __global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict
                                                       const uint8_t *__restrict__ A,
                                                       float *__restrict__ out, int32_t *__restrict__ sums,
                                                       uint32_t n_rows, uint32_t units, uint32_t groups_per_row,
-                                                      size_t row_bytes, const float *__restrict__ old) {
+                                                      size_t row_bytes, const float *__restrict__ old, uint32_t n_cols) {
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
     const uint32_t n_waves = (gridDim.x * blockDim.x) >> 6;
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict
             typename F::Wt w;
             const uint32_t uc = min(u, units - 1);
             F::load_w(w, rp, uc, k);
-            F::load_act(a, ActQ8{A}, uc, valid, k);
+            F::load_act(a, ActQ8{A, n_cols}, uc, valid, k);
             acc += F::template dot<DUMP>(w, a, k, DUMP ? sums + (size_t)row * groups_per_row : nullptr, u, valid);
         }
         const float total = wave_sum(acc);

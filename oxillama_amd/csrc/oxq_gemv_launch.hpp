@@ -38,10 +38,10 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     if (blocks == 0) blocks = 1;
     const void *acts = a.X ? static_cast<const void *>(a.X) : static_cast<const void *>(a.A);
     // fp32 source: LDS for the quantized vector (32 payload bytes + one f16 scale per block)
-    const size_t lds = std::is_same<SRC, ActF32>::value ? (size_t)(a.n_cols / 32) * 34 : 0;
+    const size_t lds = std::is_same<SRC, ActF32>::value ? (size_t)units * (F::UNIT_COLS / 32) * 34 : 0;
     hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), lds, stream, w[0],
                        w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums, rows[0],
-                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes);
+                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols);
     return hipGetLastError();
 }
 
@@ -68,9 +68,12 @@ static hipError_t launch_steps(const GemvArgs &a, uint32_t units, uint32_t group
 
 template <class F>
 static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStream_t stream) {
-    const uint32_t units = a.n_cols / F::UNIT_COLS;
+    // a row may end inside a block (the reference skips the columns past n_cols): whole blocks are
+    // stored and streamed (a unit's weights need not be consecutive columns), and the activation
+    // source hands out zero bytes for the columns that do not exist
+    const uint32_t units = (a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS * (F::BLOCK_COLS / F::UNIT_COLS);
     const uint32_t groups_per_row = a.n_cols / group_cols;
-    const size_t row_bytes = (size_t)(a.n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
+    const size_t row_bytes = (size_t)((a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS) * F::BLOCK_BYTES;
     const uint32_t steps = (units + 63) / 64;
     // Long rows are split over the four waves of a work group (fewer registers per wave,
     // more waves per SIMD); short ones keep one wave per row and need no barrier.
@@ -108,10 +111,10 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     if (blocks == 0) blocks = 1;
     if (a.sums)
         hipLaunchKernelGGL((gemv_q8_generic<F, true>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.out, a.sums,
-                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias);
+                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias, a.n_cols);
     else
         hipLaunchKernelGGL((gemv_q8_generic<F, false>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.out, a.sums,
-                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias);
+                           a.n_rows, units, groups_per_row, row_bytes, a.accumulate ? a.out : a.bias, a.n_cols);
     return hipGetLastError();
 }
 
@@ -128,7 +131,7 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
     const dim3 grid(n_rows / 32);
 #define OXQ_LAUNCH(ST, RBV)                                                                                          \
     hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4>), grid, dim3(256), 0, stream, Wg, Wu, acts, hq, h,     \
-                       n_rows, units, row_bytes)
+                       n_rows, units, row_bytes, n_cols)
     if (steps == 1) {
         if (two) OXQ_LAUNCH(1, 2); else OXQ_LAUNCH(1, 1);
     } else {
@@ -142,7 +145,7 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
 // batches per matrix); otherwise the caller gets one launch per matrix.
 template <class F>
 static bool multi_in_one_launch(const GemvArgs &a) {
-    return (a.n_cols / F::UNIT_COLS + 63) / 64 <= 32 && !a.sums;
+    return ((a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS * (F::BLOCK_COLS / F::UNIT_COLS) + 63) / 64 <= 32 && !a.sums;
 }
 
 // ---- several activation vectors per launch -------------------------------------------------
@@ -156,7 +159,7 @@ static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t ro
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
     hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride, a.out,
-                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias);
+                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias, a.n_cols);
     return hipGetLastError();
 }
 
@@ -165,8 +168,8 @@ static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t ro
 // steps per wave leave registers for two vectors only.
 template <class F>
 static hipError_t launch_vecs_f(const GemvVecsArgs &a, hipStream_t stream) {
-    const uint32_t units = a.n_cols / F::UNIT_COLS;
-    const size_t row_bytes = (size_t)(a.n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
+    const uint32_t units = (a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS * (F::BLOCK_COLS / F::UNIT_COLS);
+    const size_t row_bytes = (size_t)((a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS) * F::BLOCK_BYTES;
     const uint32_t steps = (units + 63) / 64;
     if (steps == 1)
         return a.n_vecs > 2 ? launch_vecs_k<F, 1, 1, 4>(a, units, row_bytes, stream)

@@ -121,6 +121,46 @@ def test_fused_matvec_sums_and_fp32(hip, ref, t):
 
 
 @pytest.mark.parametrize("t", TYPES, ids=ids)
+def test_rows_that_end_inside_a_block(hip, ref, t):
+    """n_cols that is not a whole number of blocks: the reference's fused rows skip the columns past it
+    (traits.rs:150-166 for the 32-weight formats; q2_k.rs:224-292, q3_k.rs:258-322, q5_k.rs:270-345).  The
+    activation blocks past n_cols hold non-zero bytes, so a kernel that did not skip them fails."""
+    k = hip.HipKernel(t)
+    bs = O.BLOCK[t][0]
+    for i, n_cols in enumerate((20, 45, 1000, 4101) if bs == 32 else (200, 300, 1000, 4097, 14336 - 100)):
+        n_rows = (33, 64, 40, 35, 48)[i]
+        full = -(-n_cols // bs) * bs
+        say("ragged", O.NAMES[t], n_rows, n_cols, "of", full)
+        w = O.random_blocks(t, 900 + 10 * t + i, n_rows, full)
+        x = synth.normal_f32(950 + i, full)
+        a = ref.quantize_q8_0(x)
+        want = ref.matvec_q8_fused(t, w, a, n_rows, n_cols)
+        out = np.zeros(n_rows, dtype=np.float32)
+        k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+        assert_close(out, want, f"fused {O.NAMES[t]} {n_rows}x{n_cols}")
+        y = torch.full((n_rows,), 2.0, dtype=torch.float32, device=DEV)
+        k.matvec_q8_fused_dev(dev(w), dev(a), y, n_rows, n_cols, accumulate=True)
+        assert np.array_equal(host(y), np.float32(2.0) + out)
+        # fp32 activations, exactly n_cols of them: quantize (zero-padded) + fused
+        xz = x.copy()
+        xz[n_cols:] = 0.0
+        want_q = ref.matvec_q8_fused(t, w, ref.quantize_q8_0(xz), n_rows, n_cols)
+        yg = torch.zeros(n_rows, dtype=torch.float32, device=DEV)
+        k.gemv_dev(dev(w), dev(x[:n_cols].copy()), yg, n_rows, n_cols)
+        assert_close(host(yg), want_q, "gemv_dev ragged")
+        yh = np.full(n_rows, 7.0, dtype=np.float32)
+        k.gemv(hip.QuantTensor(w, [n_rows, n_cols], t), x[:n_cols], yh)
+        assert np.array_equal(yh, host(yg))
+        xs = synth.normal_f32(970 + i, 7 * n_cols).reshape(7, n_cols)
+        ym = np.zeros((7, n_rows), dtype=np.float32)
+        k.gemm(hip.QuantTensor(w, [n_rows, n_cols], t), xs, ym, 7, n_rows, n_cols)
+        for r in range(7):
+            xr = np.zeros(full, dtype=np.float32)
+            xr[:n_cols] = xs[r]
+            assert_close(ym[r], ref.matvec_q8_fused(t, w, ref.quantize_q8_0(xr), n_rows, n_cols), f"gemm ragged row {r}")
+
+
+@pytest.mark.parametrize("t", TYPES, ids=ids)
 def test_gemv_gemm_host_route(hip, ref, t):
     n, kk = 160, 1024
     w = O.random_blocks(t, 500 + t, n, kk)

@@ -280,6 +280,96 @@ def test_gemm_few_rows_share_one_weight_pass(hip, ref, t):
         lib.oxq_set_gemm_tile_min_rows(0)
 
 
+def _ragged_cols(t):
+    bs = O.BLOCK[t][0]
+    return (20, 33, 1000, 4097, 8200 - 13) if bs == 32 else (200, 300, 1000, 4097, 14336 - 100, 17000)
+
+
+def _ragged_ref(ref, t, w, a, n_rows, n_cols):
+    """Rows that end inside a block: the reference skips the columns past n_cols
+    (Q/reference/q4_k.rs:307-321, Q/simd/avx2/q4_0.rs:266-287, q8_0.rs:244-252, Q/reference/q6_k.rs:327).
+    IQ4_XS has no working fused kernel in the reference; its integer form is this build's and takes whole
+    blocks, so the columns past n_cols are given zero activation bytes, which is what skipping them means."""
+    bs = O.BLOCK[t][0]
+    if t != O.IQ4_XS:
+        return ref.matvec_q8_fused(t, w, a, n_rows, n_cols, tier=O.TIER_AVX2)
+    full = -(-n_cols // bs) * bs
+    am = a.copy().reshape(-1, 34)
+    for b in range(am.shape[0]):
+        keep = min(max(n_cols - 32 * b, 0), 32)
+        am[b, 2 + keep:] = 0
+    return ref.matvec_q8_fused(t, w, am.ravel(), n_rows, full, tier=O.TIER_AVX2)
+
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_rows_that_end_inside_a_block(hip, ref, t):
+    """n_cols that is not a whole number of blocks (the reference's partial-block cases,
+    Q/simd/avx2/q4_0.rs:557-580 with 20 columns, Q/simd/avx2/q4_k.rs:837-864 with 200): host slices,
+    device pointers, several matrices per launch, fp32 activations quantized in the kernel, and gemm.
+    The activation blocks past n_cols hold non-zero bytes, so a kernel that did not skip them fails."""
+    import torch
+    k = hip.HipKernel(t)
+    bs = O.BLOCK[t][0]
+    for i, n_cols in enumerate(_ragged_cols(t)):
+        n_rows = (33, 64, 40, 35, 48, 37)[i]
+        full = -(-n_cols // bs) * bs
+        say(O.NAMES[t], "n_rows", n_rows, "n_cols", n_cols, "of", full)
+        w = synth.weights(t, 1700 + i, n_rows, full)
+        x = synth.normal_f32(1800 + i, full)
+        a = ref.quantize_q8_0(x)
+        y_ref = _ragged_ref(ref, t, w, a, n_rows, n_cols)
+        out = np.zeros(n_rows, dtype=np.float32)
+        k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+        assert_close(out, y_ref, f"{O.NAMES[t]} fused {n_rows}x{n_cols}")
+        # the same as whole blocks with the activations past n_cols set to zero
+        xz = x.copy()
+        xz[n_cols:] = 0.0
+        az = a.copy().reshape(-1, 34)
+        for b in range(az.shape[0]):
+            az[b, 2 + min(max(n_cols - 32 * b, 0), 32):] = 0
+        outz = np.zeros(n_rows, dtype=np.float32)
+        k.matvec_q8_fused(w, az.ravel(), outz, n_rows, full)
+        assert_close(out, outz, "ragged against zeroed activations")
+        # device pointers: accumulate, two matrices per launch
+        dw = torch.from_numpy(w).cuda()
+        dw2 = torch.from_numpy(synth.weights(t, 1750 + i, n_rows, full)).cuda()
+        da = torch.from_numpy(a).cuda()
+        y1 = torch.full((n_rows,), 3.0, dtype=torch.float32, device="cuda")
+        k.matvec_q8_fused_dev(dw, da, y1, n_rows, n_cols, accumulate=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(y1.cpu().numpy(), np.float32(3.0) + out)
+        m1 = [torch.zeros(n_rows, dtype=torch.float32, device="cuda") for _ in range(2)]
+        s2 = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+        k.matvec_q8_fused_multi_dev([dw, dw2], da, m1, n_rows, n_cols, accumulate=False)
+        k.matvec_q8_fused_dev(dw2, da, s2, n_rows, n_cols, accumulate=False)
+        torch.cuda.synchronize()
+        assert np.array_equal(m1[0].cpu().numpy(), out) and torch.equal(m1[1], s2)
+        # fp32 activations, exactly n_cols of them: quantize (zero-padded) + fused
+        xq = ref.quantize_q8_0(xz)
+        y_q = _ragged_ref(ref, t, w, xq, n_rows, n_cols)
+        dx = torch.from_numpy(x[:n_cols].copy()).cuda()
+        yg = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+        k.gemv_dev(dw, dx, yg, n_rows, n_cols)
+        torch.cuda.synchronize()
+        assert_close(yg.cpu().numpy(), y_q, "gemv_dev ragged")
+        yh = np.full(n_rows, 7.0, dtype=np.float32)
+        k.gemv(hip.QuantTensor(w, [n_rows, n_cols], t), x[:n_cols], yh)
+        assert_close(yh, y_q, "gemv ragged")
+        assert np.array_equal(yh, yg.cpu().numpy())
+        # gemm on host slices: rows of n_cols floats, few rows and more rows than the tile threshold
+        for m in (3, 11):
+            xs = synth.normal_f32(1900 + i + m, m * n_cols).reshape(m, n_cols)
+            ym = np.zeros((m, n_rows), dtype=np.float32)
+            k.gemm(hip.QuantTensor(w, [n_rows, n_cols], t), xs, ym, m, n_rows, n_cols)
+            for r in range(m):
+                xr = np.zeros(full, dtype=np.float32)
+                xr[:n_cols] = xs[r]
+                assert_close(ym[r], _ragged_ref(ref, t, w, ref.quantize_q8_0(xr), n_rows, n_cols), f"gemm ragged row {r}")
+    # the debug dump of the group sums wants whole blocks
+    with pytest.raises(hip.UnsupportedShape):
+        k.block_sums(synth.weights(t, 1, 2, bs), ref.quantize_q8_0(synth.normal_f32(2, bs)), 2, bs - 3)
+
+
 def test_empty_inputs(hip):
     for t in O.ALL_TYPES:
         k = hip.HipKernel(t)
@@ -382,6 +472,16 @@ def test_gemv_known_answers(hip):
     w = np.frombuffer(O.make_q8_0_block(2.0, q), dtype=np.uint8)
     hip.HipKernel(O.Q8_0).gemv(hip.QuantTensor(w, [1, 32], O.Q8_0), x, y)
     assert abs(y[0] - 6.0) < 0.1
+    # partial blocks, Q/simd/avx2/q4_k.rs:837-864 (200 of 256 columns, all weights 1 -> 200) and
+    # Q/simd/avx2/q4_0.rs:557-580 (20 of 32 columns, all weights 0 -> 0), at the reference's tolerances
+    # (plus the Q8_0 rounding of the all-ones input, 127 * f16(1/127) = 0.99994)
+    w = np.frombuffer(O.make_q4_k_block(1.0, 0.0, FX.Q4K_SCALES_ONES, [0x11] * 128), dtype=np.uint8)
+    hip.HipKernel(O.Q4_K).gemv(hip.QuantTensor(w, [1, 200], O.Q4_K), np.ones(200, dtype=np.float32), y)
+    assert abs(y[0] - 200.0) < 0.1
+    w = np.frombuffer(O.make_q4_0_block(1.0, [0x88] * 16), dtype=np.uint8)
+    y[0] = 5.0
+    hip.HipKernel(O.Q4_0).gemv(hip.QuantTensor(w, [1, 20], O.Q4_0), np.ones(20, dtype=np.float32), y)
+    assert abs(y[0]) < 1e-4
 
 
 @pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
