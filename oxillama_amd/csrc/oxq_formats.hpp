@@ -42,23 +42,27 @@ __device__ __forceinline__ int mul24(int a, int b) { return __mul24(a, b); }
 //    crates/oxillama-quant/src/traits.rs:39-44) -- and its waves read the blocks from there.
 struct ActQ8 {
     const uint8_t *A;
-    uint32_t n_cols;  // columns that exist: the payload bytes of columns past them read as zero
-    static __device__ __forceinline__ ActQ8 make(const void *p, uint32_t n_cols) {
-        return ActQ8{static_cast<const uint8_t *>(p), n_cols};
+    static __device__ __forceinline__ ActQ8 make(const void *p, uint32_t) { return ActQ8{static_cast<const uint8_t *>(p)}; }
+    __device__ __forceinline__ void block(uint32_t b, u32x4 &q0, u32x4 &q1, uint32_t &dbits) const {
+        const uint8_t *blk = A + (size_t)b * Q8_BLOCK_BYTES;
+        q0 = ld16(blk + 2);
+        q1 = ld16(blk + 18);
+        dbits = ld2(blk);
     }
+};
+// The same blocks for a row that ends inside a block: the reference skips the columns past n_cols
+// (crates/oxillama-quant/src/reference/q4_k.rs:307-321, traits.rs:150-166), which is a dot product
+// with zero activations there, so the payload bytes of those columns read as zero.
+struct ActQ8Tail {
+    const uint8_t *A;
+    uint32_t n_cols;
     // Bytes off..off+3 of a block of which only the first `rem` columns exist.
     static __device__ __forceinline__ uint32_t tail_mask(uint32_t rem, uint32_t off) {
         const uint32_t keep = rem > off ? min(rem - off, 4u) : 0u;
         return keep >= 4 ? 0xFFFFFFFFu : (1u << (8 * keep)) - 1u;
     }
     __device__ __forceinline__ void block(uint32_t b, u32x4 &q0, u32x4 &q1, uint32_t &dbits) const {
-        const uint8_t *blk = A + (size_t)b * Q8_BLOCK_BYTES;
-        q0 = ld16(blk + 2);
-        q1 = ld16(blk + 18);
-        dbits = ld2(blk);
-        // A row that ends inside a block: the reference skips the columns past n_cols
-        // (crates/oxillama-quant/src/reference/q4_k.rs:307-321, traits.rs:150-166), which is a dot
-        // product with zero activations there.  Never taken when n_cols is a whole number of blocks.
+        ActQ8{A}.block(b, q0, q1, dbits);
         if (32 * b + 32 > n_cols) {
             const uint32_t rem = n_cols > 32 * b ? n_cols - 32 * b : 0;
             for (int i = 0; i < 4; i++) {

@@ -43,8 +43,8 @@ uint32_t gemv_group_cols(uint32_t type) {
 uint32_t gemv_vecs_max(uint32_t type, uint32_t n_cols) {
     const uint32_t unit = gemv_unit_cols(type);
     if (unit == 0) return 0;
-    const uint32_t bs = (uint32_t)oxq_block_size(type);
-    const uint32_t steps = ((n_cols + bs - 1) / bs * (bs / unit) + 63) / 64;
+    if (n_cols % (uint32_t)oxq_block_size(type) != 0) return 0;  // rows that end inside a block: one vector per launch
+    const uint32_t steps = (n_cols / unit + 63) / 64;
     if (steps == 1 || steps == 3 || steps == 4) return 4;
     if (steps == 2 || (steps >= 5 && steps <= 8)) return 2;
     return 0;

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
                                                              const uint8_t *__restrict__ Wu,
                                                              const void *__restrict__ A, uint8_t *__restrict__ hq,
                                                              float *__restrict__ h_out, uint32_t n_rows, uint32_t units,
-                                                             size_t row_bytes, uint32_t n_cols) {
+                                                             size_t row_bytes) {
     static_assert((RB == 1 || RB == 2) && (WAVES == 4 || WAVES == 8), "configuration");
     constexpr int RPW = 32 / WAVES;  // rows of each matrix per wave
     constexpr int NB = RPW / RB;     // batches per matrix and wave
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
     const typename F::Lane k = F::lane_consts(lane);
     typename F::Act act[STEPS];
     {
-        const auto src = ActQ8::make(A, n_cols);
+        const auto src = ActQ8{static_cast<const uint8_t *>(A)};
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
             const uint32_t u = (uint32_t)(s * 64) + lane;
@@ -249,8 +249,7 @@ template <class F, int STEPS, int KS, int NV>
 __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ W, const uint8_t *__restrict__ A,
                                                    size_t a_stride, float *__restrict__ out, size_t out_stride,
                                                    uint32_t n_rows, uint32_t units, size_t row_bytes,
-                                                   int accumulate, uint32_t n_vecs, const float *__restrict__ bias,
-                                                   uint32_t n_cols) {
+                                                   int accumulate, uint32_t n_vecs, const float *__restrict__ bias) {
     static_assert((KS == 1 || KS == 4) && NV >= 2 && NV <= 4, "configuration");
     // n_vecs <= NV: the surplus slots repeat the last vector (same loads, same stored values)
     constexpr uint32_t G = 4 / KS;
@@ -271,7 +270,7 @@ __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ 
 #pragma unroll
         for (int s = 0; s < STEPS; s++) {
             const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
-            F::load_act(act[v][s], ActQ8{A + (size_t)min((uint32_t)v, n_vecs - 1) * a_stride, n_cols}, min(u, units - 1),
+            F::load_act(act[v][s], ActQ8{A + (size_t)min((uint32_t)v, n_vecs - 1) * a_stride}, min(u, units - 1),
                         u < units, k);
         }
     auto load_row = [&](typename F::Wt (&w)[STEPS], uint32_t row) {
@@ -335,7 +334,8 @@ __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ 
     }
 }
 
-// Any number of steps: activations re-read (from L2) for every row.
+// Any number of steps: activations re-read (from L2) for every row.  Also the kernel of rows that end
+// inside a block (n_cols not a whole number of blocks): the columns past n_cols are skipped.
 template <class F, bool DUMP>
 __global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict__ W,
                                                       const uint8_t *__restrict__ A,
@@ -357,7 +357,7 @@ __global__ __launch_bounds__(256) void gemv_q8_generic(const uint8_t *__restrict
             typename F::Wt w;
             const uint32_t uc = min(u, units - 1);
             F::load_w(w, rp, uc, k);
-            F::load_act(a, ActQ8{A, n_cols}, uc, valid, k);
+            F::load_act(a, ActQ8Tail{A, n_cols}, uc, valid, k);
             acc += F::template dot<DUMP>(w, a, k, DUMP ? sums + (size_t)row * groups_per_row : nullptr, u, valid);
         }
         const float total = wave_sum(acc);

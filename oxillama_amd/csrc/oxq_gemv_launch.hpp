@@ -83,7 +83,9 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     // (measured on MI355X: more in flight per wave does not pay beyond that); Q6_K always one.
     uint32_t rb = a.rows_per_batch;
     if (rb == 0) rb = row_bytes / (ks >= 4 ? 4 : 1) <= F::TWO_ROW_BATCH_BYTES ? 2 : 1;
-    if (ks >= 4 && steps <= 32) {
+    // Q8_0 activations and a row that ends inside a block: the kernel that masks the activations
+    const bool ragged_q8 = a.n_cols % F::BLOCK_COLS != 0 && !a.X;
+    if (ks >= 4 && steps <= 32 && !ragged_q8) {
         const uint32_t sw = (steps + 3) / 4;
         switch (sw) {
         case 1: return launch_steps<F, 1, 4>(a, units, groups_per_row, row_bytes, rb, stream);
@@ -93,7 +95,7 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
         default: return launch_steps<F, 8, 4>(a, units, groups_per_row, row_bytes, rb, stream);
         }
     }
-    switch (steps) {
+    switch (ragged_q8 ? 0 : steps) {
     case 1: return launch_steps<F, 1, 1>(a, units, groups_per_row, row_bytes, rb, stream);
     case 2: return launch_steps<F, 2, 1>(a, units, groups_per_row, row_bytes, rb, stream);
     case 3:
@@ -131,7 +133,7 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
     const dim3 grid(n_rows / 32);
 #define OXQ_LAUNCH(ST, RBV)                                                                                          \
     hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4>), grid, dim3(256), 0, stream, Wg, Wu, acts, hq, h,     \
-                       n_rows, units, row_bytes, n_cols)
+                       n_rows, units, row_bytes)
     if (steps == 1) {
         if (two) OXQ_LAUNCH(1, 2); else OXQ_LAUNCH(1, 1);
     } else {
@@ -145,7 +147,7 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
 // batches per matrix); otherwise the caller gets one launch per matrix.
 template <class F>
 static bool multi_in_one_launch(const GemvArgs &a) {
-    return ((a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS * (F::BLOCK_COLS / F::UNIT_COLS) + 63) / 64 <= 32 && !a.sums;
+    return (a.n_cols / F::UNIT_COLS + 63) / 64 <= 32 && !a.sums && (a.n_cols % F::BLOCK_COLS == 0 || a.X);
 }
 
 // ---- several activation vectors per launch -------------------------------------------------
@@ -159,7 +161,7 @@ static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t ro
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
     hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride, a.out,
-                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias, a.n_cols);
+                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias);
     return hipGetLastError();
 }
 
@@ -168,8 +170,9 @@ static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t ro
 // steps per wave leave registers for two vectors only.
 template <class F>
 static hipError_t launch_vecs_f(const GemvVecsArgs &a, hipStream_t stream) {
-    const uint32_t units = (a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS * (F::BLOCK_COLS / F::UNIT_COLS);
-    const size_t row_bytes = (size_t)((a.n_cols + F::BLOCK_COLS - 1) / F::BLOCK_COLS) * F::BLOCK_BYTES;
+    if (a.n_cols % F::BLOCK_COLS != 0) return hipErrorNotSupported;  // gemv_vecs_max says so beforehand
+    const uint32_t units = a.n_cols / F::UNIT_COLS;
+    const size_t row_bytes = (size_t)(a.n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
     const uint32_t steps = (units + 63) / 64;
     if (steps == 1)
         return a.n_vecs > 2 ? launch_vecs_k<F, 1, 1, 4>(a, units, row_bytes, stream)

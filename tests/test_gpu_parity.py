@@ -355,7 +355,6 @@ def test_rows_that_end_inside_a_block(hip, ref, t):
         yh = np.full(n_rows, 7.0, dtype=np.float32)
         k.gemv(hip.QuantTensor(w, [n_rows, n_cols], t), x[:n_cols], yh)
         assert_close(yh, y_q, "gemv ragged")
-        assert np.array_equal(yh, yg.cpu().numpy())
         # gemm on host slices: rows of n_cols floats, few rows and more rows than the tile threshold
         for m in (3, 11):
             xs = synth.normal_f32(1900 + i + m, m * n_cols).reshape(m, n_cols)
