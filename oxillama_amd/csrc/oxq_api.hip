@@ -99,7 +99,6 @@ struct State {
 };
 State g;
 
-constexpr uint32_t DEFAULT_WAVES_PER_CU = 8;
 
 // FNV-1a over up to 64 samples of 64 bytes spread across the buffer, plus its length.
 uint64_t fingerprint(const uint8_t *p, size_t len) {
@@ -194,7 +193,7 @@ oxq::GemvArgs gemv_args(const uint8_t *W, const uint8_t *A, float *out, int32_t 
     a.n_rows = (uint32_t)n_rows;
     a.n_cols = (uint32_t)n_cols;
     a.accumulate = accumulate;
-    a.waves_per_cu = g.waves_per_cu ? g.waves_per_cu : DEFAULT_WAVES_PER_CU;
+    a.waves_per_cu = g.waves_per_cu;
     a.rows_per_batch = g.rows_per_batch;
     a.waves_per_row = g.waves_per_row;
     return a;

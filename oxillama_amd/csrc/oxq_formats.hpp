@@ -225,7 +225,10 @@ struct FmtQ4K {
 // 8hh + is + 2j, activation block 8b + 4hh + j bytes 16is..+16.
 struct FmtQ6K {
     static constexpr uint32_t BLOCK_BYTES = 210, BLOCK_COLS = 256, UNIT_COLS = 64;
-    static constexpr uint32_t TWO_ROW_BATCH_BYTES = 0;  // 52 bytes and 11 registers per unit: one row per batch
+    // Measured on MI355X (4096 x 14336 and 128256 x 4096): four waves per compute unit with two rows per
+    // batch beat eight waves with one (11.4 against 11.8 us, 73.6 against 76.6 us).
+    static constexpr uint32_t TWO_ROW_BATCH_BYTES = 4000;
+    static constexpr uint32_t WAVES_PER_CU = 4;
     struct Lane {
         uint32_t hh, is;
     };
@@ -235,15 +238,27 @@ struct FmtQ6K {
         int nasum32[4];  // -32 * sum of the 16 activation bytes
     };
     struct Wt {
-        u32x4 ql0, ql1, qh;
+        u32x4 ql0, ql1, qh;  // as loaded from the dword-aligned address at or below the lane's bytes
         u32x2 sc;
+        uint32_t sc2;        // the dword after sc (needed when the block sits off a dword boundary)
         uint32_t d;
+        uint32_t sh;         // bits by which the loaded dwords are off: 8 * (block address % 4)
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t lane) {
         Lane k;
         k.hh = (lane >> 1) & 1;
         k.is = lane & 1;
         return k;
+    }
+    template <int CTRL> static __device__ __forceinline__ uint32_t qp(uint32_t v) { return (uint32_t)dpp_i<CTRL>((int)v); }
+    // 16 bytes that start `sh` bits into x: x holds the 16 bytes at the aligned address below, `next` the dword after
+    static __device__ __forceinline__ u32x4 realign(const u32x4 x, uint32_t next, uint32_t sh) {
+        u32x4 r;
+        r[0] = __builtin_amdgcn_alignbit(x[1], x[0], sh);
+        r[1] = __builtin_amdgcn_alignbit(x[2], x[1], sh);
+        r[2] = __builtin_amdgcn_alignbit(x[3], x[2], sh);
+        r[3] = __builtin_amdgcn_alignbit(next, x[3], sh);
+        return r;
     }
     template <class SRC>
     static __device__ __forceinline__ void load_act(Act &a, const SRC &src, uint32_t u, bool valid, const Lane &k) {
@@ -262,11 +277,19 @@ struct FmtQ6K {
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &k) {
         const uint8_t *blk = row + (size_t)(u >> 2) * BLOCK_BYTES;
-        // plain unaligned loads: re-aligning in registers (ld16_h) was measured slower here
-        w.ql0 = ld16(blk + 64 * k.hh + 16 * k.is);
-        w.ql1 = ld16(blk + 64 * k.hh + 32 + 16 * k.is);
-        w.qh = ld16(blk + 128 + 32 * k.hh + 16 * k.is);
-        w.sc = ld8(blk + 192 + 8 * k.hh);
+        // A block is 210 bytes, so every other block sits two bytes off a dword boundary, and 16-byte loads
+        // from such addresses cost a large part of the load bandwidth.  All loads therefore go to the
+        // dword-aligned address at or below; the missing last bytes of a lane's piece are the first bytes of
+        // the neighbouring lane's load (the pieces of a block are consecutive), fetched in dot() with DPP.
+        // W is dword-aligned (checked by the host), so the two bytes below a block are inside the matrix.
+        const uint32_t off = (uint32_t)(reinterpret_cast<uintptr_t>(blk) & 3);
+        const uint8_t *base = blk - off;
+        w.sh = 8 * off;
+        w.ql0 = *reinterpret_cast<const u32x4 *>(base + 64 * k.hh + 16 * k.is);
+        w.ql1 = *reinterpret_cast<const u32x4 *>(base + 64 * k.hh + 32 + 16 * k.is);
+        w.qh = *reinterpret_cast<const u32x4 *>(base + 128 + 32 * k.hh + 16 * k.is);
+        w.sc = *reinterpret_cast<const u32x2 *>(base + 192 + 8 * k.hh);
+        w.sc2 = *reinterpret_cast<const uint32_t *>(base + 192 + 8 * k.hh + (off ? 8 : 4));  // aligned block: re-read
         w.d = ld2(blk + 208);
     }
     template <bool DUMP>
@@ -274,8 +297,17 @@ struct FmtQ6K {
                                                 uint32_t u, bool valid) {
         // sum (q - 32) a = sum q a - 32 sum a: the accumulators start at -32 sum a
         int p0 = a.nasum32[0], p1 = a.nasum32[1], p2 = a.nasum32[2], p3 = a.nasum32[3];
+        // The dword after each of the lane's pieces.  The 16-byte pieces of a block in address order: ql 0..7
+        // (lane (hh, is) holds 4hh + is in ql0 and 4hh + 2 + is in ql1), qh 8..11 (8 + 2hh + is), scales 12.
+        // Lanes of a block are a quad: position 2hh + is.
+        const uint32_t x_ql0 = qp<0xB1>(w.ql0[0]), x_ql1 = qp<0xB1>(w.ql1[0]), x_qh = qp<0xB1>(w.qh[0]);
+        const uint32_t p2_ql0 = qp<0xAA>(w.ql0[0]), p2_qh = qp<0xAA>(w.qh[0]);  // quad position 2: (hh 1, is 0)
+        const uint32_t p0_qh = qp<0x00>(w.qh[0]), p0_sc = qp<0x00>(w.sc[0]);     // quad position 0: (hh 0, is 0)
+        const u32x4 ql0 = realign(w.ql0, k.is ? x_ql1 : x_ql0, w.sh);
+        const u32x4 ql1 = realign(w.ql1, k.is ? (k.hh ? p0_qh : p2_ql0) : x_ql1, w.sh);
+        const u32x4 qh = realign(w.qh, k.is ? (k.hh ? p0_sc : p2_qh) : x_qh, w.sh);
         for (int i = 0; i < 4; i++) {
-            const uint32_t l0 = w.ql0[i], l1 = w.ql1[i], h = w.qh[i];
+            const uint32_t l0 = ql0[i], l1 = ql1[i], h = qh[i];
             // q6_k.rs:55-60, four bytes at a time.  hm holds the 2-bit fields of q1 (bits 0-1)
             // and q3 (bits 4-5) of every byte, hn those of q2 and q4; a bitfield insert under
             // the low-nibble mask joins them with the ql nibbles.
@@ -291,7 +323,8 @@ struct FmtQ6K {
         }
         const int isum[4] = {p0, p1, p2, p3};
         // scales[8hh + is + 2j]: bytes is, is+2 of sc[0], then of sc[1]
-        const uint32_t s0 = w.sc[0] >> (8 * k.is), s1 = w.sc[1] >> (8 * k.is);
+        const uint32_t s0 = __builtin_amdgcn_alignbit(w.sc[1], w.sc[0], w.sh) >> (8 * k.is);
+        const uint32_t s1 = __builtin_amdgcn_alignbit(w.sc2, w.sc[1], w.sh) >> (8 * k.is);
         const int scv[4] = {(int)(int8_t)(s0 & 0xFF), (int)(int8_t)((s0 >> 16) & 0xFF),
                             (int)(int8_t)(s1 & 0xFF), (int)(int8_t)((s1 >> 16) & 0xFF)};
         float t = 0.0f;

@@ -41,7 +41,7 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
         g.n_cols = a.k;
         g.accumulate = a.accumulate;
         g.bias = a.bias;
-        g.waves_per_cu = 8;
+        g.waves_per_cu = 0;
         g.rows_per_batch = 0;
         g.waves_per_row = 0;
         hipError_t e = launch_gemv_q8(type, g, stream);

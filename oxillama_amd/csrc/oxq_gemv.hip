@@ -50,6 +50,10 @@ uint32_t gemv_vecs_max(uint32_t type, uint32_t n_cols) {
     return 0;
 }
 
+// The Q6_K lane policy loads from the dword-aligned address at or below its bytes, which for the first
+// block of a matrix must not lie before the matrix.
+static bool misaligned(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 3) != 0; }
+
 // 2..4 activation vectors (3 run in the 4-vector kernel, which repeats the last one).
 hipError_t launch_gemv_vecs(uint32_t type, const GemvVecsArgs &a, hipStream_t stream) {
     if (a.n_rows == 0 || a.n_cols == 0) return hipSuccess;
@@ -57,7 +61,7 @@ hipError_t launch_gemv_vecs(uint32_t type, const GemvVecsArgs &a, hipStream_t st
     case OXQ_TYPE_Q4_0: return launch_vecs_f<FmtQ4_0>(a, stream);
     case OXQ_TYPE_Q8_0: return launch_vecs_f<FmtQ8_0>(a, stream);
     case OXQ_TYPE_Q4_K: return launch_vecs_f<FmtQ4K>(a, stream);
-    case OXQ_TYPE_Q6_K: return launch_vecs_f<FmtQ6K>(a, stream);
+    case OXQ_TYPE_Q6_K: return misaligned(a.W) ? hipErrorInvalidDevicePointer : launch_vecs_f<FmtQ6K>(a, stream);
     case OXQ_TYPE_IQ4_XS: return launch_vecs_f<FmtIQ4XS>(a, stream);
     default: return launch_gemv_vecs_more(type, a, stream);
     }
@@ -77,7 +81,9 @@ hipError_t launch_gate_up_swiglu(uint32_t type, const uint8_t *Wg, const uint8_t
     case OXQ_TYPE_Q4_0: return launch_gate_up_swiglu_format<FmtQ4_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
     case OXQ_TYPE_Q8_0: return launch_gate_up_swiglu_format<FmtQ8_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
     case OXQ_TYPE_Q4_K: return launch_gate_up_swiglu_format<FmtQ4K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    case OXQ_TYPE_Q6_K: return launch_gate_up_swiglu_format<FmtQ6K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    case OXQ_TYPE_Q6_K:
+        if (misaligned(Wg) || misaligned(Wu)) return hipErrorInvalidDevicePointer;
+        return launch_gate_up_swiglu_format<FmtQ6K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
     case OXQ_TYPE_IQ4_XS: return launch_gate_up_swiglu_format<FmtIQ4XS>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
     default: return launch_gate_up_swiglu_more(type, Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
     }
@@ -89,7 +95,11 @@ hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream) 
     case OXQ_TYPE_Q4_0: return launch_gemv_format<FmtQ4_0>(a, 32, stream);
     case OXQ_TYPE_Q8_0: return launch_gemv_format<FmtQ8_0>(a, 32, stream);
     case OXQ_TYPE_Q4_K: return launch_gemv_format<FmtQ4K>(a, 32, stream);
-    case OXQ_TYPE_Q6_K: return launch_gemv_format<FmtQ6K>(a, 16, stream);
+    case OXQ_TYPE_Q6_K:
+        if (misaligned(a.W)) return hipErrorInvalidDevicePointer;
+        for (uint32_t i = 1; i < a.n_mats; i++)
+            if (misaligned(a.W_more[i - 1])) return hipErrorInvalidDevicePointer;
+        return launch_gemv_format<FmtQ6K>(a, 16, stream);
     case OXQ_TYPE_IQ4_XS: return launch_gemv_format<FmtIQ4XS>(a, 32, stream);
     default: return launch_gemv_q8_more(type, a, stream);
     }

@@ -6,6 +6,17 @@
 
 namespace oxq {
 
+// Launch width when the caller names none: 8 resident waves per compute unit unless the format's
+// policy says otherwise (WAVES_PER_CU).
+template <class F, class = void> struct format_waves_per_cu { static constexpr uint32_t value = 8; };
+template <class F> struct format_waves_per_cu<F, std::void_t<decltype(F::WAVES_PER_CU)>> {
+    static constexpr uint32_t value = F::WAVES_PER_CU;
+};
+template <class F>
+static uint32_t launch_width(const GemvArgs &a) {
+    return a.waves_per_cu ? a.waves_per_cu : format_waves_per_cu<F>::value;
+}
+
 template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP>
 static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
                                 hipStream_t stream) {
@@ -29,7 +40,7 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     uint64_t total_rows = 0;
     for (uint32_t i = 0; i < n_mats; i++) total_rows += rows[i];
     // each matrix gets gridDim.x work groups, sized so that the whole launch fills the chip once
-    uint32_t max_groups = (uint32_t)((uint64_t)(device_cus() * a.waves_per_cu / KS) * max_rows / (total_rows ? total_rows : 1));
+    uint32_t max_groups = (uint32_t)((uint64_t)(device_cus() * launch_width<F>(a) / KS) * max_rows / (total_rows ? total_rows : 1));
     if (max_groups == 0) max_groups = 1;
     // Equal share per group: ceil(n_batches / passes) groups, each doing `passes` batches.
     const uint32_t passes = (n_batches + max_groups - 1) / max_groups;
@@ -107,7 +118,7 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     default: break;
     }
     if (a.X) return hipErrorNotSupported;  // rows this long re-read the activations: Q8_0 blocks only
-    const uint32_t max_waves = device_cus() * a.waves_per_cu;
+    const uint32_t max_waves = device_cus() * launch_width<F>(a);
     uint32_t waves = a.n_rows < max_waves ? a.n_rows : max_waves;
     uint32_t blocks = (waves + 3) / 4;
     if (blocks == 0) blocks = 1;

@@ -32,7 +32,7 @@ struct GemvArgs {
     uint32_t n_cols;      // multiple of the format's block size
     int accumulate;       // 1: out[r] += y (matvec_q8_fused), 0: out[r] = y (gemv)
     const float *bias = nullptr;  // with accumulate == 0: out[r] = y + bias[r] (QuantLinear::forward)
-    uint32_t waves_per_cu;  // launch width: resident waves per compute unit
+    uint32_t waves_per_cu;  // launch width: resident waves per compute unit; 0 = the format's default
     uint32_t rows_per_batch;  // rows a wave loads at once (1, 2 or 4); 0 = chosen from the row size
     uint32_t waves_per_row;   // 1 or 4 waves share a row; 0 = chosen from the row length
     // Further matrices of the same format and row length sharing A (q/k/v, gate/up): n_mats - 1
