@@ -181,7 +181,9 @@ size_t oxq_weights_nbytes(oxq_weights_t handle);
 /* ---- device-pointer entry points (no copies, asynchronous) ------------- */
 /* All pointers are device memory; `stream` is a hipStream_t (NULL = default
  * stream).  Shapes are validated as above (lengths are the caller's promise);
- * kernels are enqueued and the call returns. */
+ * kernels are enqueued and the call returns.  Q6_K weight matrices must start on
+ * a 4-byte boundary (device allocations and GGUF tensor data do); OXQ_ERR_KERNEL
+ * otherwise. */
 
 /* quantize_f32_to_q8_0 over `rows` rows of n floats each (rows*n contiguous). */
 int oxq_quantize_q8_0_dev(const float *d_x, size_t n_total, uint8_t *d_out, void *stream);

@@ -369,6 +369,28 @@ def test_rows_that_end_inside_a_block(hip, ref, t):
         k.block_sums(synth.weights(t, 1, 2, bs), ref.quantize_q8_0(synth.normal_f32(2, bs)), 2, bs - 3)
 
 
+def test_q6_k_weights_off_a_dword_boundary_are_refused(hip, ref):
+    """The Q6_K kernel reads from the dword-aligned address at or below a block, so the matrix has to start
+    on one (device allocations and GGUF tensor data do); two bytes off, the call fails and launches nothing."""
+    import torch
+    n_rows, n_cols = 8, 512
+    w = synth.weights(O.Q6_K, 77, n_rows, n_cols)
+    buf = torch.zeros(w.size + 4, dtype=torch.uint8, device="cuda")
+    buf[2:2 + w.size] = torch.from_numpy(w).cuda()
+    da = torch.from_numpy(ref.quantize_q8_0(synth.normal_f32(78, n_cols))).cuda()
+    y = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+    with pytest.raises(hip.KernelError):
+        hip.HipKernel(O.Q6_K).matvec_q8_fused_dev(buf[2:], da, y, n_rows, n_cols)
+    # four bytes off is fine
+    buf2 = torch.zeros(w.size + 4, dtype=torch.uint8, device="cuda")
+    buf2[4:] = torch.from_numpy(w).cuda()
+    hip.HipKernel(O.Q6_K).matvec_q8_fused_dev(buf2[4:], da, y, n_rows, n_cols, accumulate=False)
+    torch.cuda.synchronize()
+    want = np.zeros(n_rows, dtype=np.float32)
+    hip.HipKernel(O.Q6_K).matvec_q8_fused(w, da.cpu().numpy(), want, n_rows, n_cols)
+    assert np.array_equal(y.cpu().numpy(), want)
+
+
 def test_empty_inputs(hip):
     for t in O.ALL_TYPES:
         k = hip.HipKernel(t)
