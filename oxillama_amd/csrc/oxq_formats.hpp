@@ -348,9 +348,15 @@ struct FmtQ8_0 {
         u32x4 q0, q1;
         float d_a;
     };
+    // A block is 34 bytes, so every other one starts two bytes off a dword boundary.  Each lane issues
+    // two dword-aligned 16-byte loads and one 2-byte load that together cover its 34 bytes exactly:
+    //   block on a dword boundary: bytes 0..31 (d, payload 0..29) + the 2 bytes 32..33 (payload 30..31);
+    //   block two bytes off:       bytes 2..33 (the payload, aligned as it is) + the 2 bytes 0..1 (d).
+    // dot() shifts the first form into place (v_alignbit by 16; by 0 for the second form).
     struct Wt {
         u32x4 q0, q1;
-        uint32_t d;
+        uint32_t x;    // the 2-byte load
+        uint32_t off;  // 0: first form, else second
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t) { return Lane{}; }
     template <class SRC>
@@ -361,20 +367,25 @@ struct FmtQ8_0 {
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
-        w.q0 = ld16_h(blk + 2);
-        w.q1 = ld16_h(blk + 18);
-        w.d = ld2(blk);
+        w.off = (uint32_t)(reinterpret_cast<uintptr_t>(blk) & 2);  // blocks start on even addresses
+        const uint8_t *base = blk + w.off;
+        w.q0 = *reinterpret_cast<const u32x4 *>(base);
+        w.q1 = *reinterpret_cast<const u32x4 *>(base + 16);
+        w.x = ld2(w.off ? blk : blk + 32);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &, int32_t *sums,
                                                 uint32_t u, bool valid) {
+        const uint32_t sh = w.off ? 0u : 16u;
+        const uint32_t dw[9] = {w.q0[0], w.q0[1], w.q0[2], w.q0[3], w.q1[0], w.q1[1], w.q1[2], w.q1[3], w.x};
         int p = 0;
         for (int i = 0; i < 4; i++) {
-            p = sdot4(w.q0[i], a.q0[i], p);
-            p = sdot4(w.q1[i], a.q1[i], p);
+            p = sdot4(__builtin_amdgcn_alignbit(dw[i + 1], dw[i], sh), a.q0[i], p);
+            p = sdot4(__builtin_amdgcn_alignbit(dw[i + 5], dw[i + 4], sh), a.q1[i], p);
         }
         if (DUMP && valid) sums[u] = p;
-        const float scale = h2f(w.d) * a.d_a;  // avx2/q8_0.rs:205
+        const uint32_t dbits = w.off ? w.x : (w.q0[0] & 0xFFFFu);
+        const float scale = h2f(dbits) * a.d_a;  // avx2/q8_0.rs:205
         return scale * (float)p;               // avx2/q8_0.rs:242
     }
 };
@@ -404,9 +415,11 @@ struct FmtQ4_0 {
         float d_a;
         int nasum8;  // -8 * sum of the 32 activation bytes
     };
+    // 18-byte blocks, loaded as FmtQ8_0 loads its 34: one dword-aligned 16-byte load (bytes 0..15 of a
+    // block on a dword boundary, bytes 2..17 of one two bytes off) and one 2-byte load for the rest.
     struct Wt {
         u32x4 q;
-        uint32_t d;
+        uint32_t x, off;
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t) { return Lane{}; }
     template <class SRC>
@@ -425,19 +438,23 @@ struct FmtQ4_0 {
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
-        w.q = ld16_h(blk + 2);
-        w.d = ld2(blk);
+        w.off = (uint32_t)(reinterpret_cast<uintptr_t>(blk) & 2);
+        w.q = *reinterpret_cast<const u32x4 *>(blk + w.off);
+        w.x = ld2(w.off ? blk : blk + 16);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &, int32_t *sums,
                                                 uint32_t u, bool valid) {
+        const uint32_t sh = w.off ? 0u : 16u;
+        const uint32_t dw[5] = {w.q[0], w.q[1], w.q[2], w.q[3], w.x};
         int p = a.nasum8;
         for (int i = 0; i < 4; i++) {
-            p = sdot4(w.q[i] & 0x0F0F0F0Fu, a.ev[i], p);
-            p = sdot4((w.q[i] >> 4) & 0x0F0F0F0Fu, a.od[i], p);
+            const uint32_t q = __builtin_amdgcn_alignbit(dw[i + 1], dw[i], sh);
+            p = sdot4(q & 0x0F0F0F0Fu, a.ev[i], p);
+            p = sdot4((q >> 4) & 0x0F0F0F0Fu, a.od[i], p);
         }
         if (DUMP && valid) sums[u] = p;
-        const float scale = h2f(w.d) * a.d_a;  // avx2/q4_0.rs:211
+        const float scale = h2f(w.off ? w.x : (w.q[0] & 0xFFFFu)) * a.d_a;  // avx2/q4_0.rs:211
         return scale * (float)p;               // avx2/q4_0.rs:265
     }
 };
