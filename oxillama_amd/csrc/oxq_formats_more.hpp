@@ -84,9 +84,11 @@ struct FmtQ5_0 {
         float d_a;
         int nasum16;  // -16 * sum(q_a)
     };
+    // 22-byte blocks: three aligned loads cover a block exactly.  On a dword boundary: bytes 0..15, 16..19,
+    // 20..21; two bytes off: bytes 2..17, 18..21 and the 2 bytes 0..1 (d).  dot() shifts the first form by 16 bits.
     struct Wt {
         u32x4 q;
-        uint32_t qh, d;
+        uint32_t q4, x, off;
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t) { return Lane{}; }
     template <class SRC>
@@ -98,9 +100,11 @@ struct FmtQ5_0 {
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
-        w.d = ld2(blk);
-        w.qh = ld4(blk + 2);
-        w.q = ld16_h(blk + 6);
+        w.off = (uint32_t)(reinterpret_cast<uintptr_t>(blk) & 2);
+        const uint8_t *base = blk + w.off;
+        w.q = *reinterpret_cast<const u32x4 *>(base);
+        w.q4 = *reinterpret_cast<const uint32_t *>(base + 16);
+        w.x = ld2(w.off ? blk : blk + 20);
     }
     // Exact sum of q5 * a over the block, q5 in 0..31, starting from `start`.
     static __device__ __forceinline__ int dot5(const u32x4 &q, uint32_t qh, const u32x4 &a0, const u32x4 &a1, int start) {
@@ -116,9 +120,14 @@ struct FmtQ5_0 {
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &, int32_t *sums, uint32_t u,
                                                 bool valid) {
-        const int p = dot5(w.q, w.qh, a.q0, a.q1, a.nasum16);
+        const uint32_t sh = w.off ? 0u : 16u;
+        const uint32_t dw[6] = {w.q[0], w.q[1], w.q[2], w.q[3], w.q4, w.x};
+        const uint32_t qh = __builtin_amdgcn_alignbit(dw[1], dw[0], sh);
+        u32x4 q;
+        for (int i = 0; i < 4; i++) q[i] = __builtin_amdgcn_alignbit(dw[i + 2], dw[i + 1], sh);
+        const int p = dot5(q, qh, a.q0, a.q1, a.nasum16);
         if (DUMP && valid) sums[u] = p;
-        return (h2f(w.d) * a.d_a) * (float)p;
+        return (h2f(w.off ? w.x : (w.q[0] & 0xFFFFu)) * a.d_a) * (float)p;
     }
 };
 
@@ -210,9 +219,11 @@ struct FmtIQ4NL {
         uint32_t ev[4], od[4];
         float d_a;
     };
+    // loaded as FmtQ4_0's blocks: one dword-aligned 16-byte load (bytes 0..15 of a block on a dword
+    // boundary, bytes 2..17 of one two bytes off) and one 2-byte load for the rest
     struct Wt {
         u32x4 q;
-        uint32_t d;
+        uint32_t x, off;
     };
     static __device__ __forceinline__ Lane lane_consts(uint32_t) { return Lane{}; }
     template <class SRC>
@@ -225,19 +236,23 @@ struct FmtIQ4NL {
     }
     static __device__ __forceinline__ void load_w(Wt &w, const uint8_t *row, uint32_t u, const Lane &) {
         const uint8_t *blk = row + (size_t)u * BLOCK_BYTES;
-        w.q = ld16_h(blk + 2);
-        w.d = ld2(blk);
+        w.off = (uint32_t)(reinterpret_cast<uintptr_t>(blk) & 2);
+        w.q = *reinterpret_cast<const u32x4 *>(blk + w.off);
+        w.x = ld2(w.off ? blk : blk + 16);
     }
     template <bool DUMP>
     static __device__ __forceinline__ float dot(const Wt &w, const Act &a, const Lane &, int32_t *sums, uint32_t u,
                                                 bool valid) {
+        const uint32_t sh = w.off ? 0u : 16u;
+        const uint32_t dw[5] = {w.q[0], w.q[1], w.q[2], w.q[3], w.x};
         int p = 0;
         for (int i = 0; i < 4; i++) {
-            p = sdot4(FmtIQ4XS::lut4(w.q[i] & 0x0F0F0F0Fu), a.ev[i], p);
-            p = sdot4(FmtIQ4XS::lut4((w.q[i] >> 4) & 0x0F0F0F0Fu), a.od[i], p);
+            const uint32_t q = __builtin_amdgcn_alignbit(dw[i + 1], dw[i], sh);
+            p = sdot4(FmtIQ4XS::lut4(q & 0x0F0F0F0Fu), a.ev[i], p);
+            p = sdot4(FmtIQ4XS::lut4((q >> 4) & 0x0F0F0F0Fu), a.od[i], p);
         }
         if (DUMP && valid) sums[u] = p;
-        return (h2f(w.d) * a.d_a) * (float)p;
+        return (h2f(w.off ? w.x : (w.q[0] & 0xFFFFu)) * a.d_a) * (float)p;
     }
 };
 
