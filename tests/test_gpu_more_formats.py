@@ -160,6 +160,24 @@ def test_rows_that_end_inside_a_block(hip, ref, t):
             assert_close(ym[r], ref.matvec_q8_fused(t, w, ref.quantize_q8_0(xr), n_rows, n_cols), f"gemm ragged row {r}")
 
 
+@pytest.mark.parametrize("t", [O.IQ4_NL, O.Q5_0], ids=ids)
+def test_weights_two_bytes_off_a_dword_boundary(hip, ref, t):
+    """The 18- and 22-byte formats pick one of two load forms per block from the block's address; a matrix
+    that starts two bytes off a dword boundary swaps the forms of all its blocks and must give the same bits."""
+    for n_rows, n_cols in ((40, 4096), (16, 14336)):
+        w = O.random_blocks(t, 990 + t, n_rows, n_cols)
+        da = dev(ref.quantize_q8_0(synth.normal_f32(991, n_cols)))
+        aligned = dev(w)
+        buf = torch.zeros(w.size + 8, dtype=torch.uint8, device=DEV)
+        buf[2:2 + w.size] = aligned
+        y0 = torch.zeros(n_rows, dtype=torch.float32, device=DEV)
+        y2 = torch.zeros(n_rows, dtype=torch.float32, device=DEV)
+        k = hip.HipKernel(t)
+        k.matvec_q8_fused_dev(aligned, da, y0, n_rows, n_cols, accumulate=False)
+        k.matvec_q8_fused_dev(buf[2:], da, y2, n_rows, n_cols, accumulate=False)
+        assert np.array_equal(host(y0), host(y2)), (O.NAMES[t], n_rows, n_cols)
+
+
 @pytest.mark.parametrize("t", TYPES, ids=ids)
 def test_gemv_gemm_host_route(hip, ref, t):
     n, kk = 160, 1024

@@ -369,6 +369,26 @@ def test_rows_that_end_inside_a_block(hip, ref, t):
         k.block_sums(synth.weights(t, 1, 2, bs), ref.quantize_q8_0(synth.normal_f32(2, bs)), 2, bs - 3)
 
 
+@pytest.mark.parametrize("t", [O.Q8_0, O.Q4_0], ids=lambda t: O.NAMES[t])
+def test_weights_two_bytes_off_a_dword_boundary(hip, ref, t):
+    """The 34- and 18-byte formats pick one of two load forms per block from the block's address; a matrix
+    that starts two bytes off a dword boundary swaps the forms of all its blocks and must give the same bits."""
+    import torch
+    for n_rows, n_cols in ((40, 4096), (33, 8192), (16, 14336)):
+        w = synth.weights(t, 91, n_rows, n_cols)
+        da = torch.from_numpy(ref.quantize_q8_0(synth.normal_f32(92, n_cols))).cuda()
+        aligned = torch.from_numpy(w).cuda()
+        buf = torch.zeros(w.size + 8, dtype=torch.uint8, device="cuda")
+        buf[2:2 + w.size] = aligned
+        y0 = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+        y2 = torch.zeros(n_rows, dtype=torch.float32, device="cuda")
+        k = hip.HipKernel(t)
+        k.matvec_q8_fused_dev(aligned, da, y0, n_rows, n_cols, accumulate=False)
+        k.matvec_q8_fused_dev(buf[2:], da, y2, n_rows, n_cols, accumulate=False)
+        torch.cuda.synchronize()
+        assert torch.equal(y0, y2), (O.NAMES[t], n_rows, n_cols)
+
+
 def test_q6_k_weights_off_a_dword_boundary_are_refused(hip, ref):
     """The Q6_K kernel reads from the dword-aligned address at or below a block, so the matrix has to start
     on one (device allocations and GGUF tensor data do); two bytes off, the call fails and launches nothing."""
