@@ -243,17 +243,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
 
 // Several activation vectors against one weight stream (a small decode batch): NV vectors'
 // constants live in registers, every weight row is loaded once and dotted with each of them.
-// One row per trip (double-buffered like the kernel above), KS waves per row.  Vector v reads
-// its Q8_0 blocks at A + v * a_stride and writes out[v * out_stride + row].
-template <class F, int STEPS, int KS, int NV>
+// RB rows per trip (double-buffered like the kernel above: the next trip's rows are requested
+// before this trip's are reduced), KS waves per row.  Vector v reads its Q8_0 blocks at
+// A + v * a_stride and writes out[v * out_stride + row].
+template <class F, int STEPS, int KS, int NV, int RB>
 __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ W, const uint8_t *__restrict__ A,
                                                    size_t a_stride, float *__restrict__ out, size_t out_stride,
                                                    uint32_t n_rows, uint32_t units, size_t row_bytes,
                                                    int accumulate, uint32_t n_vecs, const float *__restrict__ bias) {
-    static_assert((KS == 1 || KS == 4) && NV >= 2 && NV <= 4, "configuration");
+    static_assert((KS == 1 || KS == 4) && NV >= 2 && NV <= 4 && (RB == 1 || RB == 2), "configuration");
     // n_vecs <= NV: the surplus slots repeat the last vector (same loads, same stored values)
     constexpr uint32_t G = 4 / KS;
-    __shared__ float part_sums[2][4][4];
+    __shared__ float part_sums[2][4][RB * 4];
     const uint32_t lane = threadIdx.x & 63;
     const uint32_t wave_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const uint32_t part = wave_in_wg % KS, grp = wave_in_wg / KS;
@@ -261,8 +262,9 @@ __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ 
     const uint32_t n_groups = gridDim.x * G;
     const uint32_t unit0 = part * STEPS * 64;
     const typename F::Lane k = F::lane_consts(lane);
-    const uint32_t n_trips = KS == 1 ? n_rows : ((n_rows + n_groups - 1) / n_groups) * n_groups;
-    if (KS == 1 && group >= n_rows) return;
+    const uint32_t n_batches = (n_rows + RB - 1) / RB;
+    const uint32_t n_trips = KS == 1 ? n_batches : ((n_batches + n_groups - 1) / n_groups) * n_groups;
+    if (KS == 1 && group >= n_batches) return;
 
     typename F::Act act[NV][STEPS];
 #pragma unroll
@@ -273,64 +275,72 @@ __global__ __launch_bounds__(256) void gemv_q8_vecs(const uint8_t *__restrict__ 
             F::load_act(act[v][s], ActQ8{A + (size_t)min((uint32_t)v, n_vecs - 1) * a_stride}, min(u, units - 1),
                         u < units, k);
         }
-    auto load_row = [&](typename F::Wt (&w)[STEPS], uint32_t row) {
-        const uint8_t *rp = W + (size_t)min(row, n_rows - 1) * row_bytes;  // past the end: re-read the last row
+    auto load_rows = [&](typename F::Wt (&w)[RB][STEPS], uint32_t batch) {
 #pragma unroll
-        for (int s = 0; s < STEPS; s++)
-            F::load_w(w[s], rp, min(unit0 + (uint32_t)(s * 64) + lane, units - 1), k);
+        for (int r = 0; r < RB; r++) {
+            // past the end: re-read the last row
+            const uint8_t *rp = W + (size_t)min(batch * RB + (uint32_t)r, n_rows - 1) * row_bytes;
+#pragma unroll
+            for (int s = 0; s < STEPS; s++)
+                F::load_w(w[r][s], rp, min(unit0 + (uint32_t)(s * 64) + lane, units - 1), k);
+        }
     };
     uint32_t trip = 0;
-    auto reduce_row = [&](const typename F::Wt (&w)[STEPS], uint32_t row) {
+    // lane r * NV + v ends up with the sum of row r of the batch against vector v
+    auto reduce_rows = [&](const typename F::Wt (&w)[RB][STEPS], uint32_t batch) {
         float res = 0.0f;
 #pragma unroll
-        for (int v = 0; v < NV; v++) {
-            float acc = 0.0f;
+        for (int r = 0; r < RB; r++)
 #pragma unroll
-            for (int s = 0; s < STEPS; s++) {
-                const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
-                acc += F::template dot<false>(w[s], act[v][s], k, nullptr, u, u < units);
+            for (int v = 0; v < NV; v++) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int s = 0; s < STEPS; s++) {
+                    const uint32_t u = unit0 + (uint32_t)(s * 64) + lane;
+                    acc += F::template dot<false>(w[r][s], act[v][s], k, nullptr, u, u < units);
+                }
+                const float total = wave_sum(acc);
+                if (lane == (uint32_t)(r * NV + v)) res = total;
             }
-            const float total = wave_sum(acc);
-            if (lane == (uint32_t)v) res = total;
-        }
+        const uint32_t row = batch * RB + lane / NV, vec = min(lane % NV, n_vecs - 1);
         if (KS == 1) {
-            if (lane < NV && row < n_rows) {
-                float *o = out + (size_t)min(lane, n_vecs - 1) * out_stride + row;
+            if (lane < RB * NV && row < n_rows) {
+                float *o = out + (size_t)vec * out_stride + row;
                 *o = (accumulate ? *o : bias ? bias[row] : 0.0f) + res;
             }
         } else {
-            if (lane < NV) part_sums[trip & 1][wave_in_wg][lane] = res;
+            if (lane < RB * NV) part_sums[trip & 1][wave_in_wg][lane] = res;
             __syncthreads();
-            if (part == 0 && lane < NV && row < n_rows) {
+            if (part == 0 && lane < RB * NV && batch < n_batches && row < n_rows) {
                 float t = part_sums[trip & 1][grp * KS][lane];
 #pragma unroll
                 for (int p = 1; p < KS; p++) t += part_sums[trip & 1][grp * KS + p][lane];
-                float *o = out + (size_t)min(lane, n_vecs - 1) * out_stride + row;
+                float *o = out + (size_t)vec * out_stride + row;
                 *o = (accumulate ? *o : bias ? bias[row] : 0.0f) + t;
             }
             trip++;
         }
     };
 
-    typename F::Wt w0[STEPS], w1[STEPS];
-    load_row(w0, group);
-    uint32_t row = group;
+    typename F::Wt w0[RB][STEPS], w1[RB][STEPS];
+    load_rows(w0, min(group, n_batches - 1));
+    uint32_t batch = group;
     while (true) {
-        const uint32_t next = row + n_groups;
+        const uint32_t next = batch + n_groups;
         if (next >= n_trips) {
-            reduce_row(w0, row);
+            reduce_rows(w0, batch);
             break;
         }
-        load_row(w1, next);
-        reduce_row(w0, row);
+        load_rows(w1, min(next, n_batches - 1));
+        reduce_rows(w0, batch);
         const uint32_t next2 = next + n_groups;
         if (next2 >= n_trips) {
-            reduce_row(w1, next);
+            reduce_rows(w1, next);
             break;
         }
-        load_row(w0, next2);
-        reduce_row(w1, next);
-        row = next2;
+        load_rows(w0, min(next2, n_batches - 1));
+        reduce_rows(w1, next);
+        batch = next2;
     }
 }
 

@@ -166,13 +166,17 @@ static bool multi_in_one_launch(const GemvArgs &a) {
 template <class F, int STEPS, int KS, int NV>
 static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t row_bytes, hipStream_t stream) {
     constexpr uint32_t G = 4 / KS;
+    // Two rows per trip where a wave's slice of a row is one step (measured on 14336 x 4096 and 4096 x 14336:
+    // one row per trip leaves too few bytes in flight per wave)
+    constexpr int RB = STEPS == 1 ? 2 : 1;
+    const uint32_t n_batches = (a.n_rows + RB - 1) / RB;
     const uint32_t max_groups = device_cus() * 8 / KS;
-    const uint32_t passes = (a.n_rows + max_groups - 1) / max_groups;
-    const uint32_t groups = (a.n_rows + passes - 1) / passes;
+    const uint32_t passes = (n_batches + max_groups - 1) / max_groups;
+    const uint32_t groups = (n_batches + passes - 1) / passes;
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
-    hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride, a.out,
-                       a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias);
+    hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV, RB>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride,
+                       a.out, a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias);
     return hipGetLastError();
 }
 
