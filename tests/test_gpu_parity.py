@@ -288,7 +288,7 @@ def _ragged_cols(t):
 def _ragged_ref(ref, t, w, a, n_rows, n_cols):
     """Rows that end inside a block: the reference skips the columns past n_cols
     (Q/reference/q4_k.rs:307-321, Q/simd/avx2/q4_0.rs:266-287, q8_0.rs:244-252, Q/reference/q6_k.rs:327).
-    IQ4_XS has no working fused kernel in the reference; its integer form is this build's and takes whole
+    IQ4_XS has no working fused kernel in the reference; its integer form is defined by this library and takes whole
     blocks, so the columns past n_cols are given zero activation bytes, which is what skipping them means."""
     bs = O.BLOCK[t][0]
     if t != O.IQ4_XS:
