@@ -15,6 +15,7 @@
  */
 #include <math.h>
 #include <stdlib.h>
+#include <string.h>
 
 #include "oxq_oracle.h"
 
@@ -111,15 +112,24 @@ oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w,
     if (output_len < n_rows) {
         return st(OXQ_REF_DIMENSION_MISMATCH, n_rows, output_len);
     }
-    if (n_cols % 32 != 0) {
-        return st(OXQ_REF_KERNEL_ERROR, n_cols, 32);
+    /* A row that ends inside a block: the reference's gemv skips the columns past n_cols
+     * (q4_k.rs:161,168); with Q8_0 activations that is the input zero-padded to whole blocks. */
+    size_t bs = oxq_ref_block_size(type);
+    if (bs == 0) {
+        return st(OXQ_REF_UNSUPPORTED_TYPE, type, 0);
     }
-    size_t acts_len = n_cols / 32 * 34;
+    size_t k_pad = (n_cols + bs - 1) / bs * bs;
+    size_t acts_len = k_pad / 32 * 34;
     uint8_t *acts = (uint8_t *)malloc(acts_len ? acts_len : 1);
-    if (!acts) {
+    float *padded = (float *)calloc(k_pad ? k_pad : 1, sizeof(float));
+    if (!acts || !padded) {
+        free(acts);
+        free(padded);
         return st(OXQ_REF_INTERNAL, 0, 0);
     }
-    oxq_ref_status s = oxq_ref_quantize_f32_to_q8_0(input, n_cols, acts);
+    memcpy(padded, input, n_cols * sizeof(float));
+    oxq_ref_status s = oxq_ref_quantize_f32_to_q8_0(padded, k_pad, acts);
+    free(padded);
     if (s.code == OXQ_REF_OK) {
         for (size_t r = 0; r < n_rows; r++) {
             output[r] = 0.0f; /* gemv overwrites */

@@ -1261,19 +1261,21 @@ int oxq_linear_forward(uint32_t type, const uint8_t *data, size_t data_len, cons
     const size_t row_bytes = (n_cols + bs - 1) / bs * bb;
     if (data_len < n_rows * row_bytes)
         return fail(OXQ_ERR_BUFFER_TOO_SMALL, n_rows * row_bytes, data_len, "tensor data too small");
-    if (n_cols % bs != 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, bs, n_cols, "n_cols is not a multiple of the block size");
     if (n_rows == 0 || n_cols == 0) return OXQ_OK;
-    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull)
-        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_rows, "dimension exceeds 2^32-1");
+    if (n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFF00ull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFF00ull, n_rows, "dimension exceeds 2^32-257");
     if ((st = ensure_init()) != OXQ_OK) return st;
     std::lock_guard<std::mutex> lock(g.mu);
     const uint8_t *dW = nullptr;
     if ((st = stage_weights(type, data, n_rows * row_bytes, &dW)) != OXQ_OK) return st;
-    if ((st = g.s_x.reserve(n_cols * sizeof(float))) != OXQ_OK) return st;
-    if ((st = g.s_acts.reserve(n_cols / 32 * 34)) != OXQ_OK) return st;
+    // a row that ends inside a block: the input is staged zero-padded to whole blocks (gemv skips those columns)
+    const size_t k_pad = (n_cols + bs - 1) / bs * bs;
+    if ((st = g.s_x.reserve(k_pad * sizeof(float))) != OXQ_OK) return st;
+    if ((st = g.s_acts.reserve(k_pad / 32 * 34)) != OXQ_OK) return st;
     if ((st = g.s_out.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+    if (k_pad != n_cols) OXQ_HIP(hipMemset(g.s_x.ptr, 0, k_pad * sizeof(float)));
     OXQ_HIP(hipMemcpy(g.s_x.ptr, input, n_cols * sizeof(float), hipMemcpyHostToDevice));
-    OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, n_cols, (uint8_t *)g.s_acts.ptr, nullptr));
+    OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, k_pad, (uint8_t *)g.s_acts.ptr, nullptr));
     const float *d_bias = nullptr;
     if (bias && bias_len) {
         // the reference zips output with bias (linear.rs:87-89): a short bias covers its own length only

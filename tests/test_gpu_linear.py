@@ -231,6 +231,27 @@ def test_linear_forward_host_reference_cases(hip, ref):
         L.LoraAdapter([1.0], [1, 0, 0, 1], 2, 1.0, 1, 2)  # lora.rs:203-214
 
 
+@pytest.mark.parametrize("t", [O.Q4_0, O.Q8_0, O.Q4_K, O.Q6_K], ids=lambda t: O.NAMES[t])
+def test_linear_forward_host_rows_that_end_inside_a_block(hip, ref, t):
+    """in_features that is not a whole number of blocks: QuantLinear::forward goes through gemv, which skips the
+    columns past n_cols (Q/reference/q4_k.rs:161,168); bias and LoRA see the n_cols inputs as they are."""
+    bs = O.BLOCK[t][0]
+    for n_rows, n_cols in ((33, bs + 20), (40, 5 * bs - 7)):
+        full = -(-n_cols // bs) * bs
+        w = synth.weights(t, 1200 + n_cols, n_rows, full)
+        x = synth.normal_f32(1201, n_cols)
+        bias = synth.normal_f32(1202, n_rows)
+        rank = 3
+        a = synth.normal_f32(1203, rank * n_cols) * np.float32(0.1)
+        b = synth.normal_f32(1204, n_rows * rank) * np.float32(0.1)
+        lin = L.QuantLinear(hip.QuantTensor(w, [n_rows, n_cols], t), bias=bias)
+        lin.set_lora(L.LoraAdapter(a, b, rank, 0.5, n_cols, n_rows))
+        out = np.zeros(n_rows, dtype=np.float32)
+        lin.forward(hip.HipKernel(t), x, out)
+        want = ref.linear_forward(t, w, n_rows, n_cols, x, bias=bias, lora=(a, b, rank, 0.5))
+        assert_close(out, want, f"ragged linear {O.NAMES[t]} {n_rows}x{n_cols}")
+
+
 @pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
 def test_linear_forward_batch(hip, ref, t):
     n, kk = 512, 1024
