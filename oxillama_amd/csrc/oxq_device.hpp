@@ -83,23 +83,23 @@ __device__ __forceinline__ float wave_sum(float v) {
 }
 
 __device__ __forceinline__ uint64_t max_u64(uint64_t a, uint64_t b) { return a > b ? a : b; }
-template <int CTRL> __device__ __forceinline__ uint64_t dpp_u64(uint64_t v) {
-    const uint32_t lo = (uint32_t)dpp_i<CTRL>((int)(uint32_t)v), hi = (uint32_t)dpp_i<CTRL>((int)(uint32_t)(v >> 32));
-    return ((uint64_t)hi << 32) | lo;
-}
 // Maximum over the 64 lanes of a wave, the same value in every lane; no LDS, no barrier.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = max(v, (uint32_t)dpp_i<0xB1>((int)v));   // quad_perm [1,0,3,2]
+    v = max(v, (uint32_t)dpp_i<0x4E>((int)v));   // quad_perm [2,3,0,1]
+    v = max(v, (uint32_t)dpp_i<0x124>((int)v));  // row_ror:4
+    v = max(v, (uint32_t)dpp_i<0x128>((int)v));  // row_ror:8
+    const uint32_t r0 = (uint32_t)__builtin_amdgcn_readlane((int)v, 0), r1 = (uint32_t)__builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t r2 = (uint32_t)__builtin_amdgcn_readlane((int)v, 32), r3 = (uint32_t)__builtin_amdgcn_readlane((int)v, 48);
+    return max(max(r0, r1), max(r2, r3));
+}
+// The same for 64-bit keys, as two 32-bit maxima: the largest upper half, then the largest lower half among
+// the lanes that hold it (fewer instructions than carrying 64-bit compares through the DPP steps).
 __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
-    v = max_u64(v, dpp_u64<0xB1>(v));   // quad_perm [1,0,3,2]
-    v = max_u64(v, dpp_u64<0x4E>(v));   // quad_perm [2,3,0,1]
-    v = max_u64(v, dpp_u64<0x124>(v));  // row_ror:4
-    v = max_u64(v, dpp_u64<0x128>(v));  // row_ror:8
-    uint64_t r[4];
-    for (int i = 0; i < 4; i++) {
-        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 16 * i);
-        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 16 * i);
-        r[i] = ((uint64_t)hi << 32) | lo;
-    }
-    return max_u64(max_u64(r[0], r[1]), max_u64(r[2], r[3]));
+    const uint32_t hi = (uint32_t)(v >> 32), lo = (uint32_t)v;
+    const uint32_t mh = wave_max_u32(hi);
+    const uint32_t ml = wave_max_u32(hi == mh ? lo : 0u);
+    return ((uint64_t)mh << 32) | ml;
 }
 
 }  // namespace oxq
