@@ -24,7 +24,14 @@
  * back to its CPU kernel.
  *
  * Thread safety: every function may be called from several host threads; calls
- * taking host slices serialise on an internal lock.
+ * taking host slices serialise on an internal lock.  Calls on device pointers are
+ * asynchronous on the caller's stream, with two documented exceptions that
+ * synchronise that stream and therefore cannot be recorded into a HIP graph: the
+ * forms of oxq_gemm_q8_dev and oxq_block_sums_dev that are given no workspace.
+ *
+ * Every entry point below cites the reference interface it stands in for.  The
+ * launch-shape knobs used for measurement live in oxq_tuning.h and are not part of
+ * what the reference-side shim binds.
  */
 #ifndef OXQ_H
 #define OXQ_H
@@ -159,13 +166,27 @@ int oxq_block_sums(uint32_t type, const uint8_t *weights, size_t weights_len,
                    const uint8_t *acts_q8, size_t acts_len, int32_t *sums, size_t sums_len,
                    size_t n_rows, size_t n_cols);
 
-/* When enabled, host-slice calls keep a device copy of each weight buffer keyed
- * by (pointer, length, type) plus a fingerprint of sampled bytes, so repeated
- * calls with the same QuantTensor do not cross PCIe again.  Off by default: the
- * caller must not mutate cached buffers.  Stands in for the ownership the
- * reference gets for free from host slices (Q/types.rs:11-18). */
-int oxq_weight_cache_enable(int enabled);
+/* Host-slice calls can keep a device copy of each weight buffer, keyed by (pointer,
+ * length, type), so that repeated calls with the same QuantTensor do not cross PCIe
+ * again.  Stands in for the ownership the reference gets for free from host slices
+ * (Q/types.rs:11-18: QuantTensor.data is an owned, immutable Vec<u8> after load).
+ * Off by default.  The contract of mode 1: while a buffer is cached the caller does
+ * not change its bytes and does not free it -- or calls oxq_weight_cache_invalidate
+ * with its address first (a freed address that the allocator hands out again with
+ * other weights would otherwise hit the old copy).  Mode 1 guards that contract only
+ * loosely, with a fingerprint of 64 sampled 64-byte pieces; mode 2 hashes every byte
+ * of the buffer on every call, so that any change is seen and the buffer uploaded
+ * again (slower than the upload it saves on PCIe 5: for checking a caller against the
+ * contract, not for production).  Resident handles (oxq_weights_register) are the
+ * route without any of this.  The cache holds at most oxq_weight_cache_set_limit
+ * bytes (default 16 GiB; least recently used copies are freed first; a buffer larger
+ * than the limit is staged per call as if the cache were off). */
+int oxq_weight_cache_enable(int mode); /* 0 off, 1 on, 2 on and verified */
 int oxq_weight_cache_clear(void);
+int oxq_weight_cache_invalidate(const void *host_ptr);
+int oxq_weight_cache_set_limit(size_t max_bytes);
+/* entries, bytes held, hits and uploads since the library was loaded (any may be null). */
+int oxq_weight_cache_stats(size_t *entries, size_t *bytes, uint64_t *hits, uint64_t *uploads);
 
 /* ---- weights resident in HBM ------------------------------------------- */
 
@@ -338,12 +359,10 @@ int oxq_rmsnorm_quantize_q8_0_dev(const float *d_x, const float *d_weight, float
  * fp32.  The sums are those of oxq_matvec_q8_fused_dev bit for bit, so the bytes equal those of
  * the separate calls.  UnsupportedShape when the type / row length has no such kernel (rows
  * longer than 128 units, Q8_1 / IQ4_NL / Q2_K / Q3_K): use the separate calls.
- * oxq_ffn_swiglu_dev takes this route by itself when gate and up share a type;
- * oxq_set_ffn_fusion(0) switches that off (measurement only). */
+ * oxq_ffn_swiglu_dev takes this route by itself when gate and up share a type. */
 int oxq_ffn_gate_up_swiglu_q8_dev(uint32_t type, const uint8_t *d_gate, const uint8_t *d_up,
                                   const uint8_t *d_acts_q8, float *d_h, uint8_t *d_out_q8,
                                   size_t intermediate, size_t hidden, void *stream);
-int oxq_set_ffn_fusion(int enabled);
 size_t oxq_ffn_workspace_bytes(size_t hidden, size_t intermediate);
 int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_type,
                        const uint8_t *d_up, uint32_t down_type, const uint8_t *d_down,
@@ -424,21 +443,6 @@ int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
 
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                        int32_t *d_sums, size_t n_rows, size_t n_cols, void *stream);
-
-/* Launch width of the GEMV kernels: resident waves per compute unit (tuning
- * knob for benchmarks; 0 restores the default). */
-int oxq_set_gemv_waves_per_cu(unsigned waves);
-/* Rows a wave loads per batch in the GEMV kernels (1, 2 or 4; tuning knob; 0 restores
- * the per-shape default). */
-int oxq_set_gemv_rows_per_batch(unsigned rows);
-/* Waves that share one row in the GEMV kernels (1 or 4; tuning knob; 0 restores the
- * per-shape default: 4 for rows of three or more 64-unit steps). */
-int oxq_set_gemv_waves_per_row(unsigned waves);
-/* Fewest activation rows for which oxq_gemm_q8_dev / oxq_gemm take the tile kernel; below it
- * they run GEMV launches, two to four rows per launch (tuning knob; 0 restores the default). */
-int oxq_set_gemm_tile_min_rows(unsigned rows);
-/* Tile shape / prefetch depth of the prefill kernel (tuning knob; 0 restores the default). */
-int oxq_set_gemm_variant(int variant);
 
 #ifdef __cplusplus
 }

@@ -72,7 +72,9 @@ int oxq_gguf_get_summary(oxq_gguf_t g, oxq_gguf_summary *out);
 typedef struct oxq_gguf_tensor {
     const char *name;
     uint32_t n_dims;
-    uint64_t dims[4];     /* dimensions as stored (the reference takes dims[0] as rows, dims[1] as columns) */
+    uint64_t dims[4];     /* dimensions as stored (the reference takes dims[0] as rows, dims[1] as columns);
+                           * a tensor of more than four dimensions parses as in the reference and shows its
+                           * first four here (n_dims, n_elements and data_size cover all of them) */
     uint32_t type;        /* GgufTensorType id */
     uint64_t offset;      /* relative to the data section */
     uint64_t n_elements;  /* product of the dimensions; 0 when there are none */
@@ -99,10 +101,18 @@ typedef struct oxq_gguf_value {
     size_t str_len;
     uint32_t elem_type; /* arrays */
     uint64_t count;     /* arrays */
+    /* arrays: the encoded elements (fixed-width values back to back; strings as length + bytes, the
+     * length u64 in version 3, u32 before) occupy array_bytes bytes at this offset of the
+     * file image; oxq_gguf_meta_array_data hands out the pointer. */
+    uint64_t array_offset;
+    uint64_t array_bytes;
 } oxq_gguf_value;
 /* OXQ_ERR_GGUF_INVALID_METADATA when the key is missing (as MetadataStore::get_string does). */
 int oxq_gguf_meta_find(oxq_gguf_t g, const char *key, oxq_gguf_value *out);
 int oxq_gguf_meta_at(oxq_gguf_t g, uint64_t index, const char **key, oxq_gguf_value *out);
+/* The encoded elements of an array value (tokenizer.ggml.tokens, scores, merges ...), valid until
+ * oxq_gguf_close; INVALID_METADATA when the key is missing or not an array. */
+int oxq_gguf_meta_array_data(oxq_gguf_t g, const char *key, const uint8_t **data, size_t *len);
 
 /* load_quant_linear (llama/model.rs:805-822) with the QuantTensor in HBM: shape = the stored
  * dimensions (rows = dims[0], columns = dims[1]), bytes copied unchanged, mmap -> pinned staging ->

@@ -1,0 +1,41 @@
+/*
+ * oxq_tuning.h -- launch-shape knobs of liboxq_hip.so for benchmarks and tests.
+ *
+ * Not part of the drop-in boundary: nothing here has a counterpart in the reference,
+ * and the reference-side shim binds none of it.  Every knob is process-global, is
+ * stored atomically and is read once per launch, so flipping one while other threads
+ * are launching is safe; it changes which launch shape later calls take, never their
+ * results (all shapes give the same integer sums; fp32 results differ only where the
+ * summation order over a row differs, within the documented tolerance).  A value of 0
+ * restores the built-in choice.
+ */
+#ifndef OXQ_TUNING_H
+#define OXQ_TUNING_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Launch width of the GEMV kernels: resident waves per compute unit (tuning
+ * knob for benchmarks; 0 restores the default). */
+int oxq_set_gemv_waves_per_cu(unsigned waves);
+/* Rows a wave loads per batch in the GEMV kernels (1, 2 or 4; tuning knob; 0 restores
+ * the per-shape default). */
+int oxq_set_gemv_rows_per_batch(unsigned rows);
+/* Waves that share one row in the GEMV kernels (1 or 4; tuning knob; 0 restores the
+ * per-shape default: 4 for rows of three or more 64-unit steps). */
+int oxq_set_gemv_waves_per_row(unsigned waves);
+/* Fewest activation rows for which oxq_gemm_q8_dev / oxq_gemm take the tile kernel; below it
+ * they run GEMV launches, two to four rows per launch (tuning knob; 0 restores the default). */
+int oxq_set_gemm_tile_min_rows(unsigned rows);
+/* Tile shape / prefetch depth of the prefill kernel (tuning knob; 0 restores the default). */
+int oxq_set_gemm_variant(int variant);
+/* oxq_ffn_swiglu_dev: 1 (default) = gate, up, SwiGLU and the quantizer of h in one launch where a kernel
+ * exists for the type and row length; 0 = the separate launches (same bits). */
+int oxq_set_ffn_fusion(int enabled);
+
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OXQ_TUNING_H */

@@ -57,7 +57,8 @@ class GgufTensor(C.Structure):
 
 class GgufValue(C.Structure):
     _fields_ = [("type", C.c_uint32), ("u", C.c_uint64), ("i", C.c_int64), ("f", C.c_double), ("str", C.c_void_p),
-                ("str_len", C.c_size_t), ("elem_type", C.c_uint32), ("count", C.c_uint64)]
+                ("str_len", C.c_size_t), ("elem_type", C.c_uint32), ("count", C.c_uint64), ("array_offset", C.c_uint64),
+                ("array_bytes", C.c_uint64)]
 
 
 # include/oxq_gguf.h
@@ -71,6 +72,7 @@ GGUF_SIGNATURES = {
     "oxq_gguf_tensor_data": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]),
     "oxq_gguf_meta_find": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(GgufValue)]),
     "oxq_gguf_meta_at": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_char_p), C.POINTER(GgufValue)]),
+    "oxq_gguf_meta_array_data": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p), C.POINTER(C.c_size_t)]),
     "oxq_gguf_load_weights": (C.c_int, [C.c_void_p, C.c_char_p, C.POINTER(C.c_void_p)]),
     "oxq_gguf_upload_tensor": (C.c_int, [C.c_void_p, C.c_char_p, C.c_void_p, C.c_size_t]),
 }
@@ -97,6 +99,9 @@ SIGNATURES = {
                                  C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t]),
     "oxq_weight_cache_enable": (C.c_int, [C.c_int]),
     "oxq_weight_cache_clear": (C.c_int, []),
+    "oxq_weight_cache_invalidate": (C.c_int, [C.c_void_p]),
+    "oxq_weight_cache_set_limit": (C.c_int, [C.c_size_t]),
+    "oxq_weight_cache_stats": (C.c_int, [_szp, _szp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "oxq_weights_register": (C.c_int, [C.c_uint32, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t,
                                        C.POINTER(C.c_void_p)]),
     "oxq_weights_release": (C.c_int, [C.c_void_p]),
@@ -141,7 +146,6 @@ SIGNATURES = {
                                                 C.c_void_p, C.c_void_p, C.c_void_p]),
     "oxq_ffn_gate_up_swiglu_q8_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
                                                 C.c_size_t, C.c_size_t, C.c_void_p]),
-    "oxq_set_ffn_fusion": (C.c_int, [C.c_int]),
     "oxq_ffn_workspace_bytes": (C.c_size_t, [C.c_size_t, C.c_size_t]),
     "oxq_ffn_swiglu_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p,
                                      C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t,
@@ -166,11 +170,16 @@ SIGNATURES = {
                                C.c_void_p]),
     "oxq_block_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                      C.c_size_t, C.c_void_p]),
+}
+
+# include/oxq_tuning.h: launch-shape knobs for benchmarks and tests, outside the drop-in boundary.
+TUNING_SIGNATURES = {
     "oxq_set_gemv_waves_per_cu": (C.c_int, [C.c_uint]),
     "oxq_set_gemv_rows_per_batch": (C.c_int, [C.c_uint]),
     "oxq_set_gemv_waves_per_row": (C.c_int, [C.c_uint]),
     "oxq_set_gemm_variant": (C.c_int, [C.c_int]),
     "oxq_set_gemm_tile_min_rows": (C.c_int, [C.c_uint]),
+    "oxq_set_ffn_fusion": (C.c_int, [C.c_int]),
 }
 
 _lib = None
@@ -186,7 +195,7 @@ def load():
             f"{LIB_PATH} is missing: build it with `python -m oxillama_amd.build` "
             "(there is no CPU fallback for the HIP path)")
     lib = C.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in {**SIGNATURES, **GGUF_SIGNATURES}.items():
+    for name, (restype, argtypes) in {**SIGNATURES, **GGUF_SIGNATURES, **TUNING_SIGNATURES}.items():
         fn = getattr(lib, name)  # AttributeError if the ABI lost a symbol
         fn.restype = restype
         fn.argtypes = argtypes

@@ -1,6 +1,7 @@
 // C ABI of liboxq_hip.so (see include/oxq.h): argument validation in the
 // reference's order, HBM residency of weights, scratch buffers for the
 // host-slice route, and kernel launches.  No exception or abort crosses the ABI.
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -11,8 +12,6 @@
 #include "oxq_internal.hpp"
 
 namespace oxq {
-extern int g_gemm_variant;
-extern uint32_t g_gemm_tile_min_rows;
 hipError_t launch_dequant(uint32_t type, const uint8_t *blocks, size_t n_blocks, float *out, hipStream_t stream);
 }
 
@@ -81,29 +80,49 @@ struct CacheKeyHash {
 struct CacheEntry {
     uint8_t *dev;
     uint64_t fingerprint;
+    uint64_t last_use;  // tick of the last hit (least recently used goes first when the byte cap is reached)
 };
 
 struct State {
     std::mutex mu;
-    bool initialised = false;
+    std::atomic<bool> initialised{false};
     int device = -1;
     uint32_t cus = 0;
-    uint32_t waves_per_cu = 0;  // 0 = default
-    uint32_t rows_per_batch = 0;  // 0 = chosen per shape
-    uint32_t waves_per_row = 0;   // 0 = chosen per shape
-    bool cache_enabled = false;
+    // launch-shape knobs (oxq_tuning.h): written by the setters, read once per launch, no lock needed
+    std::atomic<uint32_t> waves_per_cu{0};    // 0 = default
+    std::atomic<uint32_t> rows_per_batch{0};  // 0 = chosen per shape
+    std::atomic<uint32_t> waves_per_row{0};   // 0 = chosen per shape
+    int cache_mode = 0;  // 0 off, 1 on (sampled fingerprint), 2 on and verified (every byte hashed on every call)
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
+    size_t cache_bytes = 0, cache_limit = (size_t)16 << 30;
+    uint64_t cache_tick = 0, cache_hits = 0, cache_uploads = 0;
     Scratch s_weights, s_acts, s_x, s_out, s_sums, s_work, s_bias, s_lora_a, s_lora_b, s_lora_r;
     Scratch s_moe_up, s_moe_down, s_moe_tables;
-    bool fuse_swiglu = true;  // oxq_ffn_swiglu_dev: gate, up, SwiGLU and the quantizer of h in one launch where possible
+    std::atomic<bool> fuse_swiglu{true};  // oxq_ffn_swiglu_dev: gate, up, SwiGLU and the quantizer of h in one launch where possible
 };
 State g;
 
 
-// FNV-1a over up to 64 samples of 64 bytes spread across the buffer, plus its length.
-uint64_t fingerprint(const uint8_t *p, size_t len) {
+// FNV-1a over up to 64 samples of 64 bytes spread across the buffer, plus its length; `whole`: over
+// every byte, eight at a time (the verified mode: any changed byte changes the value).
+uint64_t fingerprint(const uint8_t *p, size_t len, bool whole) {
     uint64_t h = 1469598103934665603ull ^ len;
     const size_t chunk = 64, samples = 64;
+    if (whole) {
+        uint64_t lanes[4] = {h, h ^ 0x9E3779B97F4A7C15ull, h ^ 0xC2B2AE3D27D4EB4Full, h ^ 0x165667B19E3779F9ull};
+        size_t i = 0;
+        for (; i + 32 <= len; i += 32) {
+            uint64_t w[4];
+            std::memcpy(w, p + i, 32);
+            for (int l = 0; l < 4; l++) {
+                lanes[l] = (lanes[l] ^ w[l]) * 0x100000001B3ull;
+                lanes[l] ^= lanes[l] >> 29;
+            }
+        }
+        for (; i < len; i++) lanes[i & 3] = (lanes[i & 3] ^ p[i]) * 0x100000001B3ull;
+        for (int l = 0; l < 4; l++) h = (h ^ lanes[l]) * 1099511628211ull;
+        return h;
+    }
     if (len <= chunk * samples) {
         for (size_t i = 0; i < len; i++) h = (h ^ p[i]) * 1099511628211ull;
         return h;
@@ -119,24 +138,35 @@ uint64_t fingerprint(const uint8_t *p, size_t len) {
 bool known_type(uint32_t type) { return oxq_block_size(type) != 0; }
 
 int ensure_init() {
-    if (g.initialised) return OXQ_OK;
+    if (g.initialised.load(std::memory_order_acquire)) return OXQ_OK;
     return oxq_init(0);
 }
 
 // Device copy of a host weight buffer: cached when the cache is on, else staged
 // in scratch.  Caller holds g.mu.
 int stage_weights(uint32_t type, const uint8_t *host, size_t len, const uint8_t **dev) {
-    if (g.cache_enabled) {
+    if (g.cache_mode != 0 && len <= g.cache_limit) {
         CacheKey key{host, len, type};
-        const uint64_t fp = fingerprint(host, len);
+        const uint64_t fp = fingerprint(host, len, g.cache_mode == 2);
         auto it = g.cache.find(key);
         if (it != g.cache.end() && it->second.fingerprint == fp) {
+            it->second.last_use = ++g.cache_tick;
+            g.cache_hits++;
             *dev = it->second.dev;
             return OXQ_OK;
         }
-        if (it != g.cache.end()) {
+        if (it != g.cache.end()) {  // same address, different content: the device copy is stale
             (void)hipFree(it->second.dev);
+            g.cache_bytes -= it->first.len;
             g.cache.erase(it);
+        }
+        while (!g.cache.empty() && g.cache_bytes + len > g.cache_limit) {  // byte cap: least recently used first
+            auto lru = g.cache.begin();
+            for (auto jt = g.cache.begin(); jt != g.cache.end(); ++jt)
+                if (jt->second.last_use < lru->second.last_use) lru = jt;
+            (void)hipFree(lru->second.dev);
+            g.cache_bytes -= lru->first.len;
+            g.cache.erase(lru);
         }
         uint8_t *d = nullptr;
         OXQ_HIP(hipMalloc((void **)&d, len ? len : 1));
@@ -145,7 +175,9 @@ int stage_weights(uint32_t type, const uint8_t *host, size_t len, const uint8_t 
             (void)hipFree(d);
             return fail_hip(e, "hipMemcpy(weights)");
         }
-        g.cache.emplace(key, CacheEntry{d, fp});
+        g.cache.emplace(key, CacheEntry{d, fp, ++g.cache_tick});
+        g.cache_bytes += len;
+        g.cache_uploads++;
         *dev = d;
         return OXQ_OK;
     }
@@ -193,9 +225,9 @@ oxq::GemvArgs gemv_args(const uint8_t *W, const uint8_t *A, float *out, int32_t 
     a.n_rows = (uint32_t)n_rows;
     a.n_cols = (uint32_t)n_cols;
     a.accumulate = accumulate;
-    a.waves_per_cu = g.waves_per_cu;
-    a.rows_per_batch = g.rows_per_batch;
-    a.waves_per_row = g.waves_per_row;
+    a.waves_per_cu = g.waves_per_cu.load(std::memory_order_relaxed);
+    a.rows_per_batch = g.rows_per_batch.load(std::memory_order_relaxed);
+    a.waves_per_row = g.waves_per_row.load(std::memory_order_relaxed);
     return a;
 }
 
@@ -257,6 +289,7 @@ int oxq_shutdown(void) {
     if (!g.initialised) return OXQ_OK;
     for (auto &kv : g.cache) (void)hipFree(kv.second.dev);
     g.cache.clear();
+    g.cache_bytes = 0;
     g.s_weights.release();
     g.s_acts.release();
     g.s_x.release();
@@ -388,36 +421,33 @@ int oxq_get_kernel(uint32_t type) {
 }
 
 int oxq_set_gemv_waves_per_cu(unsigned waves) {
-    std::lock_guard<std::mutex> lock(g.mu);
     g.waves_per_cu = waves > 64 ? 64 : waves;
     return OXQ_OK;
 }
 
 int oxq_set_gemv_rows_per_batch(unsigned rows) {
-    std::lock_guard<std::mutex> lock(g.mu);
     g.rows_per_batch = rows > 4 ? 4 : rows;
     return OXQ_OK;
 }
 
 int oxq_set_gemv_waves_per_row(unsigned waves) {
-    std::lock_guard<std::mutex> lock(g.mu);
     g.waves_per_row = waves >= 4 ? 4 : (waves ? 1 : 0);
     return OXQ_OK;
 }
 
 int oxq_set_gemm_tile_min_rows(unsigned rows) {
-    oxq::g_gemm_tile_min_rows = rows;
+    oxq::g_gemm_tile_min_rows.store(rows, std::memory_order_relaxed);
     return OXQ_OK;
 }
 
 int oxq_set_gemm_variant(int variant) {
-    oxq::g_gemm_variant = variant;
+    oxq::g_gemm_variant.store(variant, std::memory_order_relaxed);
     return OXQ_OK;
 }
 
-int oxq_weight_cache_enable(int enabled) {
+int oxq_weight_cache_enable(int mode) {
     std::lock_guard<std::mutex> lock(g.mu);
-    g.cache_enabled = enabled != 0;
+    g.cache_mode = mode == 2 ? 2 : (mode != 0 ? 1 : 0);
     return OXQ_OK;
 }
 
@@ -425,6 +455,44 @@ int oxq_weight_cache_clear(void) {
     std::lock_guard<std::mutex> lock(g.mu);
     for (auto &kv : g.cache) (void)hipFree(kv.second.dev);
     g.cache.clear();
+    g.cache_bytes = 0;
+    return OXQ_OK;
+}
+
+int oxq_weight_cache_invalidate(const void *host_ptr) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    for (auto it = g.cache.begin(); it != g.cache.end();) {
+        if (it->first.ptr == host_ptr) {
+            (void)hipFree(it->second.dev);
+            g.cache_bytes -= it->first.len;
+            it = g.cache.erase(it);
+        } else {
+            ++it;
+        }
+    }
+    return OXQ_OK;
+}
+
+int oxq_weight_cache_set_limit(size_t max_bytes) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    g.cache_limit = max_bytes;
+    while (!g.cache.empty() && g.cache_bytes > g.cache_limit) {
+        auto lru = g.cache.begin();
+        for (auto jt = g.cache.begin(); jt != g.cache.end(); ++jt)
+            if (jt->second.last_use < lru->second.last_use) lru = jt;
+        (void)hipFree(lru->second.dev);
+        g.cache_bytes -= lru->first.len;
+        g.cache.erase(lru);
+    }
+    return OXQ_OK;
+}
+
+int oxq_weight_cache_stats(size_t *entries, size_t *bytes, uint64_t *hits, uint64_t *uploads) {
+    std::lock_guard<std::mutex> lock(g.mu);
+    if (entries) *entries = g.cache.size();
+    if (bytes) *bytes = g.cache_bytes;
+    if (hits) *hits = g.cache_hits;
+    if (uploads) *uploads = g.cache_uploads;
     return OXQ_OK;
 }
 
@@ -722,9 +790,11 @@ int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d
     return OXQ_OK;
 }
 
+// The size depends on the shape alone, never on a tuning knob: a caller that sized its workspace once stays
+// right whichever launch shape a later call takes.
 size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k) {
     if (m > 0xFFFFFFFFull || n > 0xFFFFFFFFull || k > 0xFFFFFFFFull ||
-        !oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k))
+        !oxq::gemm_tiles_supported(type, (uint32_t)m, (uint32_t)k))
         return 0;
     return oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k);
 }
@@ -748,7 +818,10 @@ static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
     ga.k = (uint32_t)k;
     ga.accumulate = accumulate ? 1 : 0;
     ga.bias = d_bias;
-    const size_t need = oxq_gemm_q8_workspace_bytes(type, m, n, k);
+    // one reading of the tuning knobs per call: tile kernel, or GEMV launches (which need no workspace)
+    const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k);
+    ga.by_rows = !tiles;
+    const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k) : 0;
     if (need && d_workspace) {
         if (workspace_bytes < need) return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, workspace_bytes, "workspace too small");
         if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
@@ -781,7 +854,8 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
                             int32_t *d_sums, size_t m, size_t n, size_t k, void *d_workspace, size_t workspace_bytes,
                             void *stream) {
     if (!d_sums) return fail(OXQ_ERR_INTERNAL, 0, 0, "null sums");
-    if (oxq_gemm_q8_workspace_bytes(type, m, n, k) == 0)
+    if (m > 0xFFFFFFFFull || n > 0xFFFFFFFFull || k > 0xFFFFFFFFull ||
+        !oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k))
         return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, m, "no tile kernel for this type/shape");
     return gemm_dev(type, d_weights, d_acts_q8, d_out, d_sums, m, n, k, 0, nullptr, d_workspace, workspace_bytes, stream);
 }
@@ -972,7 +1046,7 @@ int oxq_ffn_gate_up_swiglu_q8_dev(uint32_t type, const uint8_t *d_gate, const ui
 }
 
 int oxq_set_ffn_fusion(int enabled) {
-    g.fuse_swiglu = enabled != 0;
+    g.fuse_swiglu.store(enabled != 0, std::memory_order_relaxed);
     return OXQ_OK;
 }
 
@@ -996,7 +1070,7 @@ int oxq_ffn_swiglu_dev(uint32_t gate_type, const uint8_t *d_gate, uint32_t up_ty
     float *gate = (float *)d_workspace, *up = (float *)((uint8_t *)d_workspace + f);
     uint8_t *hq = (uint8_t *)d_workspace + 2 * f;
     hipStream_t s = (hipStream_t)stream;
-    if (gate_type == up_type && g.fuse_swiglu) {  // both projections, SwiGLU and the quantizer of h in one launch
+    if (gate_type == up_type && g.fuse_swiglu.load(std::memory_order_relaxed)) {  // both projections, SwiGLU and the quantizer of h in one launch
         hipError_t e = oxq::launch_gate_up_swiglu(gate_type, d_gate, d_up, d_acts_q8, hq, nullptr, (uint32_t)intermediate,
                                                   (uint32_t)hidden, s);
         if (e == hipSuccess) {
@@ -1187,7 +1261,7 @@ int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, ui
     std::lock_guard<std::mutex> lock(g.mu);
     const uint8_t *dg = nullptr, *du = nullptr, *dd = nullptr;
     auto stage = [&](Scratch &slot, uint32_t t, const uint8_t *host, size_t len, const uint8_t **dev) -> int {
-        if (g.cache_enabled) return stage_weights(t, host, len, dev);
+        if (g.cache_mode != 0 && len <= g.cache_limit) return stage_weights(t, host, len, dev);
         int r = slot.reserve(len);
         if (r != OXQ_OK) return r;
         OXQ_HIP(hipMemcpy(slot.ptr, host, len, hipMemcpyHostToDevice));

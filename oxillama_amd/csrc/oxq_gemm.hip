@@ -51,7 +51,7 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
     return hipSuccess;
 }
 
-int g_gemm_variant = 0;  // tuning: 0 = default
+std::atomic<int> g_gemm_variant{0};  // tuning: 0 = default
 
 size_t gemm_workspace_bytes(uint32_t m, uint32_t k) {
     // token rows are padded so that a 128-token tile starting at any row stays inside
@@ -59,7 +59,7 @@ size_t gemm_workspace_bytes(uint32_t m, uint32_t k) {
     return nsb * mpad * (32 + 4 + 2 + 8);  // activation bytes, P, f16 scales, the two half-block planes of P
 }
 
-uint32_t g_gemm_tile_min_rows = 0;  // tuning: 0 = default
+std::atomic<uint32_t> g_gemm_tile_min_rows{0};  // tuning: 0 = default
 
 // The tile kernel can take this format and shape at all.
 bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
@@ -79,13 +79,13 @@ bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
 // against 22 us for the tile kernel; 4096-row matrices give the tile kernel fewer work groups:
 // 4096 x 14336 Q6_K, 8 rows 41 us against 55 us, 12 rows 61 us against 55 us).
 bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
-    const uint32_t min_rows = g_gemm_tile_min_rows ? g_gemm_tile_min_rows : (n >= 8192 ? 6 : 9);
+    const uint32_t knob = g_gemm_tile_min_rows.load(std::memory_order_relaxed);
+    const uint32_t min_rows = knob ? knob : (n >= 8192 ? 6 : 9);
     return gemm_tiles_supported(type, m, k) && m >= min_rows;
 }
 
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) {
-    const bool tiles = a.workspace != nullptr &&
-                       (a.offsets ? gemm_tiles_supported(type, a.m, a.k) : gemm_uses_tiles(type, a.m, a.n, a.k));
+    const bool tiles = a.workspace != nullptr && gemm_tiles_supported(type, a.m, a.k) && (a.offsets || !a.by_rows);
     if (!tiles) {
         if (a.offsets) return hipErrorInvalidValue;  // grouped form exists for the tile kernel only
         return gemm_by_rows(type, a, stream);

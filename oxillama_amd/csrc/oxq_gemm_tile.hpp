@@ -33,7 +33,6 @@
 
 namespace oxq {
 
-extern int g_gemm_variant;  // tuning: 0 = default
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -772,7 +771,7 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
                : rows > 32 ? launch_tile<F, 2, 1, 0, 2, true, 2, 2>(a, p, stream)
                            : launch_tile<F, 1, 2, 0, 2, true, 2, 2>(a, p, stream);
 #ifndef OXQ_TILE_DEFAULT_SHAPES_ONLY
-    switch (g_gemm_variant) {
+    switch (g_gemm_variant.load(std::memory_order_relaxed)) {
     case 1: return launch_tile<F, 2, 1, 2, 1, false>(a, p, stream);
     case 3: return launch_tile<F, 2, 2, 2, 1, false>(a, p, stream);
     case 4: return launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);

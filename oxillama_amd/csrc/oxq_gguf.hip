@@ -32,6 +32,7 @@ struct Value {
     std::string str;
     uint32_t elem_type = 0;
     uint64_t count = 0;
+    uint64_t array_offset = 0, array_bytes = 0;  // arrays: where the encoded elements sit in the file image
 };
 
 struct Tensor {
@@ -193,12 +194,16 @@ bool read_value(Reader &r, uint32_t version, uint32_t type, Value *v, int depth)
         }
         v->elem_type = et;
         v->count = count;
+        v->array_offset = r.pos;
         Value e;
         for (uint64_t k = 0; k < count; k++)
             if (!read_value(r, version, et, &e, depth + 1)) return false;
+        v->array_bytes = r.pos - v->array_offset;
         return true;
     }
-    default: return false;
+    default:
+        r.status = oxq::set_error(OXQ_ERR_GGUF_INVALID_METADATA, type, 0, "unknown value type");
+        return false;
     }
 }
 
@@ -298,6 +303,8 @@ void fill_value(const Value &v, oxq_gguf_value *out) {
     out->str_len = v.type == OXQ_GGUF_STRING ? v.str.size() : 0;
     out->elem_type = v.elem_type;
     out->count = v.count;
+    out->array_offset = v.array_offset;
+    out->array_bytes = v.array_bytes;
 }
 
 const Tensor *find(const oxq_gguf *g, const char *name) {
@@ -370,7 +377,14 @@ int staged_upload(void *d_dst, const uint8_t *src, size_t n) {
 }
 
 int open_common(oxq_gguf *g, oxq_gguf_t *out) {
-    const int st = parse(g);
+    int st;
+    try {  // strings, vectors and maps allocate: no exception may cross the C ABI
+        st = parse(g);
+    } catch (const std::bad_alloc &) {
+        st = oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "out of host memory while parsing");
+    } catch (...) {
+        st = oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "unexpected exception while parsing");
+    }
     if (st != OXQ_OK) {
         if (g->map) munmap(g->map, g->len);
         delete g;
@@ -378,6 +392,18 @@ int open_common(oxq_gguf *g, oxq_gguf_t *out) {
     }
     *out = g;
     return OXQ_OK;
+}
+
+// Runs an entry point's body; name lookups build std::string keys, which may throw.
+template <class Body>
+int guarded(Body body) {
+    try {
+        return body();
+    } catch (const std::bad_alloc &) {
+        return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "out of host memory");
+    } catch (...) {
+        return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "unexpected exception");
+    }
 }
 
 }  // namespace
@@ -436,7 +462,12 @@ int oxq_gguf_open_bytes(const uint8_t *data, size_t len, oxq_gguf_t *out) {
     *out = nullptr;
     oxq_gguf *g = new (std::nothrow) oxq_gguf;
     if (!g) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "out of host memory");
-    if (len) g->owned.assign(data, data + len);
+    try {
+        if (len) g->owned.assign(data, data + len);
+    } catch (...) {
+        delete g;
+        return oxq::set_error(OXQ_ERR_INTERNAL, len, 0, "out of host memory");
+    }
     g->data = g->owned.data();
     g->len = len;
     return open_common(g, out);
@@ -470,30 +501,36 @@ int oxq_gguf_tensor_at(oxq_gguf_t g, uint64_t index, oxq_gguf_tensor *out) {
 }
 
 int oxq_gguf_find_tensor(oxq_gguf_t g, const char *name, oxq_gguf_tensor *out) {
-    if (!g || !out) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
-    const Tensor *t = find(g, name);
-    if (!t) return not_found(name);
-    fill(g, *t, out);
-    return OXQ_OK;
+    return guarded([&]() -> int {
+        if (!g || !out) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
+        const Tensor *t = find(g, name);
+        if (!t) return not_found(name);
+        fill(g, *t, out);
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_tensor_data(oxq_gguf_t g, const char *name, const uint8_t **data, size_t *len) {
-    if (!g || !data || !len) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
-    const Tensor *t = find(g, name);
-    if (!t) return not_found(name);
-    return locate(g, *t, data, len);
+    return guarded([&]() -> int {
+        if (!g || !data || !len) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
+        const Tensor *t = find(g, name);
+        if (!t) return not_found(name);
+        return locate(g, *t, data, len);
+    });
 }
 
 int oxq_gguf_meta_find(oxq_gguf_t g, const char *key, oxq_gguf_value *out) {
-    if (!g || !key || !out) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
-    auto it = g->meta_by_key.find(key);
-    if (it == g->meta_by_key.end()) {
-        char msg[200];
-        std::snprintf(msg, sizeof(msg), "%.150s: key not present", key);
-        return oxq::set_error(OXQ_ERR_GGUF_INVALID_METADATA, 0, 0, msg);
-    }
-    fill_value(g->meta[it->second].second, out);
-    return OXQ_OK;
+    return guarded([&]() -> int {
+        if (!g || !key || !out) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
+        auto it = g->meta_by_key.find(key);
+        if (it == g->meta_by_key.end()) {
+            char msg[200];
+            std::snprintf(msg, sizeof(msg), "%.150s: key not present", key);
+            return oxq::set_error(OXQ_ERR_GGUF_INVALID_METADATA, 0, 0, msg);
+        }
+        fill_value(g->meta[it->second].second, out);
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_meta_at(oxq_gguf_t g, uint64_t index, const char **key, oxq_gguf_value *out) {
@@ -504,56 +541,76 @@ int oxq_gguf_meta_at(oxq_gguf_t g, uint64_t index, const char **key, oxq_gguf_va
     return OXQ_OK;
 }
 
+int oxq_gguf_meta_array_data(oxq_gguf_t g, const char *key, const uint8_t **data, size_t *len) {
+    return guarded([&]() -> int {
+        if (!g || !key || !data || !len) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
+        auto it = g->meta_by_key.find(key);
+        if (it == g->meta_by_key.end() || g->meta[it->second].second.type != OXQ_GGUF_ARRAY) {
+            char msg[200];
+            std::snprintf(msg, sizeof(msg), "%.150s: no such array", key);
+            return oxq::set_error(OXQ_ERR_GGUF_INVALID_METADATA, 0, 0, msg);
+        }
+        const Value &v = g->meta[it->second].second;
+        *data = g->data + v.array_offset;
+        *len = (size_t)v.array_bytes;
+        return OXQ_OK;
+    });
+}
+
 int oxq_gguf_load_weights(oxq_gguf_t g, const char *name, oxq_weights_t *handle) {
-    if (!handle) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null handle pointer");
-    *handle = nullptr;
-    if (!g) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null file handle");
-    const Tensor *t = find(g, name);
-    if (!t) return not_found(name);
-    const size_t bs = oxq_block_size(t->type);
-    if (bs == 0) return oxq::set_error(OXQ_ERR_UNSUPPORTED_TYPE, t->type, 0, "no kernel for this tensor's format");
-    if (t->dims.size() != 2)
-        return oxq::set_error(OXQ_ERR_UNSUPPORTED_SHAPE, 2, t->dims.size(), "weight tensor is not two-dimensional");
-    const uint64_t n_rows = t->dims[0], n_cols = t->dims[1];  // model.rs:816: shape = the stored dimensions
-    if (n_cols % bs != 0)
-        return oxq::set_error(OXQ_ERR_UNSUPPORTED_SHAPE, bs, (size_t)n_cols, "columns are not a multiple of the block size");
-    const uint8_t *src = nullptr;
-    size_t n = 0;
-    int st = locate(g, *t, &src, &n);
-    if (st != OXQ_OK) return st;
-    if ((st = oxq::ensure_device()) != OXQ_OK) return st;
-    oxq_weights *w = new (std::nothrow) oxq_weights{t->type, (size_t)n_rows, (size_t)n_cols, n, nullptr};
-    if (!w) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "out of host memory");
-    hipError_t e = hipMalloc((void **)&w->dev, n ? n : 1);
-    if (e != hipSuccess) {
-        delete w;
-        return hip_fail(e, "hipMalloc(weights)");
-    }
-    {
-        std::lock_guard<std::mutex> lock(g_stage.mu);
-        st = staged_upload(w->dev, src, n);
-    }
-    if (st != OXQ_OK) {
-        (void)hipFree(w->dev);
-        delete w;
-        return st;
-    }
-    *handle = w;
-    return OXQ_OK;
+    return guarded([&]() -> int {
+        if (!handle) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null handle pointer");
+        *handle = nullptr;
+        if (!g) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null file handle");
+        const Tensor *t = find(g, name);
+        if (!t) return not_found(name);
+        const size_t bs = oxq_block_size(t->type);
+        if (bs == 0) return oxq::set_error(OXQ_ERR_UNSUPPORTED_TYPE, t->type, 0, "no kernel for this tensor's format");
+        if (t->dims.size() != 2)
+            return oxq::set_error(OXQ_ERR_UNSUPPORTED_SHAPE, 2, t->dims.size(), "weight tensor is not two-dimensional");
+        const uint64_t n_rows = t->dims[0], n_cols = t->dims[1];  // model.rs:816: shape = the stored dimensions
+        if (n_cols % bs != 0)
+            return oxq::set_error(OXQ_ERR_UNSUPPORTED_SHAPE, bs, (size_t)n_cols, "columns are not a multiple of the block size");
+        const uint8_t *src = nullptr;
+        size_t n = 0;
+        int st = locate(g, *t, &src, &n);
+        if (st != OXQ_OK) return st;
+        if ((st = oxq::ensure_device()) != OXQ_OK) return st;
+        oxq_weights *w = new (std::nothrow) oxq_weights{t->type, (size_t)n_rows, (size_t)n_cols, n, nullptr};
+        if (!w) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "out of host memory");
+        hipError_t e = hipMalloc((void **)&w->dev, n ? n : 1);
+        if (e != hipSuccess) {
+            delete w;
+            return hip_fail(e, "hipMalloc(weights)");
+        }
+        {
+            std::lock_guard<std::mutex> lock(g_stage.mu);
+            st = staged_upload(w->dev, src, n);
+        }
+        if (st != OXQ_OK) {
+            (void)hipFree(w->dev);
+            delete w;
+            return st;
+        }
+        *handle = w;
+        return OXQ_OK;
+    });
 }
 
 int oxq_gguf_upload_tensor(oxq_gguf_t g, const char *name, void *d_dst, size_t dst_len) {
-    if (!g || !d_dst) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
-    const Tensor *t = find(g, name);
-    if (!t) return not_found(name);
-    const uint8_t *src = nullptr;
-    size_t n = 0;
-    int st = locate(g, *t, &src, &n);
-    if (st != OXQ_OK) return st;
-    if (dst_len < n) return oxq::set_error(OXQ_ERR_BUFFER_TOO_SMALL, n, dst_len, "device buffer smaller than the tensor");
-    if ((st = oxq::ensure_device()) != OXQ_OK) return st;
-    std::lock_guard<std::mutex> lock(g_stage.mu);
-    return staged_upload(d_dst, src, n);
+    return guarded([&]() -> int {
+        if (!g || !d_dst) return oxq::set_error(OXQ_ERR_INTERNAL, 0, 0, "null argument");
+        const Tensor *t = find(g, name);
+        if (!t) return not_found(name);
+        const uint8_t *src = nullptr;
+        size_t n = 0;
+        int st = locate(g, *t, &src, &n);
+        if (st != OXQ_OK) return st;
+        if (dst_len < n) return oxq::set_error(OXQ_ERR_BUFFER_TOO_SMALL, n, dst_len, "device buffer smaller than the tensor");
+        if ((st = oxq::ensure_device()) != OXQ_OK) return st;
+        std::lock_guard<std::mutex> lock(g_stage.mu);
+        return staged_upload(d_dst, src, n);
+    });
 }
 
 }  // extern "C"

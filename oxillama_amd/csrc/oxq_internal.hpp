@@ -1,10 +1,12 @@
 // Host-side declarations shared by the kernel translation units and the C ABI.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <stddef.h>
 #include <stdint.h>
 
 #include "../../include/oxq.h"
+#include "../../include/oxq_tuning.h"
 
 // A weight matrix resident in HBM (oxq_weights_t): raw GGUF blocks, row-major.
 struct oxq_weights {
@@ -115,6 +117,8 @@ struct GemmArgs {
     float *out;         // [m x n] row-major
     int32_t *sums;      // optional debug dump [m][n][k/32]
     uint8_t *workspace; // gemm_workspace_bytes(m, k) bytes, 256-byte aligned; null: row-by-row matvecs
+    bool by_rows = false;  // plain matmul: take the GEMV launches even though a workspace is there (the caller's
+                           // snapshot of gemm_uses_tiles, so that one call reads the tuning knobs once)
     uint32_t m, n, k;   // m = all token rows (of all experts in the grouped form)
     int accumulate;
     const float *bias = nullptr;  // with accumulate == 0: out[t][r] = y + bias[r] (QuantLinear::forward_batch)
@@ -131,6 +135,9 @@ struct GemmArgs {
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
 // Device scratch the tile kernel needs for m tokens of k columns (activation re-layout).
 size_t gemm_workspace_bytes(uint32_t m, uint32_t k);
+// Tuning knobs (oxq_tuning.h), read once per call.
+extern std::atomic<int> g_gemm_variant;              // 0 = default tile shape
+extern std::atomic<uint32_t> g_gemm_tile_min_rows;   // 0 = default threshold
 // True when (type, m, k) is served by the int8-MFMA tile kernel.
 bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k);
 // True when the tile kernel can take (type, m, k) at all (the grouped form always uses it).

@@ -180,6 +180,31 @@ class GgufModel:
         _check(self._lib.oxq_gguf_meta_find(self._h, key.encode(), C.byref(v)))
         return _value(v)
 
+    def metadata_array(self, key):
+        """The elements of an array value: numbers, booleans or strings (tokenizer.ggml.tokens, scores,
+        merges ...), decoded from the encoded bytes the library points at."""
+        import struct
+        v = capi.GgufValue()
+        _check(self._lib.oxq_gguf_meta_find(self._h, key.encode(), C.byref(v)))
+        p, n = C.c_void_p(), C.c_size_t()
+        _check(self._lib.oxq_gguf_meta_array_data(self._h, key.encode(), C.byref(p), C.byref(n)))
+        raw = C.string_at(p, n.value)
+        fixed = {0: "<B", 1: "<b", 2: "<H", 3: "<h", 4: "<I", 5: "<i", 6: "<f", 7: "<B", 10: "<Q", 11: "<q", 12: "<d"}
+        et, count = v.elem_type, int(v.count)
+        if et in fixed:
+            vals = [x[0] for x in struct.iter_unpack(fixed[et], raw)]
+            assert len(vals) == count
+            return [bool(x) for x in vals] if et == 7 else vals
+        if et != 8:
+            raise InvalidMetadata(f"{key}: arrays of arrays are not decoded")
+        lfmt, lsz = ("<Q", 8) if self.version >= 3 else ("<I", 4)
+        out, pos = [], 0
+        for _ in range(count):
+            (ln,) = struct.unpack_from(lfmt, raw, pos)
+            out.append(raw[pos + lsz:pos + lsz + ln].decode("utf-8"))
+            pos += lsz + ln
+        return out
+
     def metadata_items(self):
         out = []
         for i in range(self.n_metadata):

@@ -21,6 +21,23 @@ def ref():
     return oracle
 
 
+@pytest.fixture
+def tuning():
+    """Setter for the launch-shape knobs of oxq_tuning.h; every knob a test touched is back at its
+    default (0; fusion: 1) when the test ends, pass or fail."""
+    from oxillama_amd import capi
+    lib = capi.load()
+    touched = set()
+
+    def set_knob(name, value):
+        touched.add(name)
+        assert getattr(lib, "oxq_set_" + name)(value) == capi.OK
+
+    yield set_knob
+    for name in touched:
+        getattr(lib, "oxq_set_" + name)(1 if name == "ffn_fusion" else 0)
+
+
 @pytest.fixture(scope="session")
 def hip():
     """The HIP library through its Python binding; fails loudly if it is not built."""

@@ -22,11 +22,17 @@ def declared_symbols(header="oxq.h"):
 def test_header_and_binding_list_the_same_symbols():
     assert declared_symbols() == sorted(capi.SIGNATURES)
     assert declared_symbols("oxq_gguf.h") == sorted(capi.GGUF_SIGNATURES)
+    assert declared_symbols("oxq_tuning.h") == sorted(capi.TUNING_SIGNATURES)
+
+
+def test_boundary_header_holds_no_tuning_knob():
+    # the reference-side shim binds oxq.h only: nothing there may be a launch-shape setter
+    assert not [s for s in declared_symbols() if s.startswith("oxq_set_")]
 
 
 def test_library_exports_every_declared_symbol():
     lib = C.CDLL(capi.LIB_PATH)
-    for name in declared_symbols() + declared_symbols("oxq_gguf.h"):
+    for name in declared_symbols() + declared_symbols("oxq_gguf.h") + declared_symbols("oxq_tuning.h"):
         assert hasattr(lib, name), name
 
 

@@ -100,6 +100,12 @@ def test_all_scalar_value_types_and_arrays():  # parser.rs:406-497, 683-707
         assert got["k.arr"] == ("array", B.U32, 3) and got["k.sarr"] == ("array", B.STRING, 3)
         assert got["k.nested"] == ("array", B.ARRAY, 2)
         assert [k for k, _ in g.metadata_items()] == [k for k, _, _ in kvs]  # file order
+        # array payloads stay readable (tokenizer lists live in such arrays)
+        assert g.metadata_array("k.arr") == [1, 2, 3] and g.metadata_array("k.sarr") == ["a", "bc", ""]
+        with pytest.raises(gguf.InvalidMetadata):
+            g.metadata_array("k.u8")
+        with pytest.raises(gguf.InvalidMetadata):
+            g.metadata_array("k.nested")
     with pytest.raises(gguf.InvalidMetadata):  # a missing key (MetadataStore::get_string, metadata.rs:162-169)
         g.metadata("absent")
 
@@ -122,6 +128,21 @@ def test_metadata_errors():
     many = struct.pack("<IIQQ", B.MAGIC, 3, 2 ** 40, 0)
     with pytest.raises(gguf.UnexpectedEof):  # tensor_count far beyond the file
         gguf.GgufModel.from_bytes(many)
+
+
+def test_more_than_four_dimensions_parse_and_show_the_first_four():
+    g = gguf.GgufModel.from_bytes(B.build(3, [], [("t5", [2, 3, 4, 5, 6], F32, 0)], b"\0" * (720 * 4)))
+    t = g.tensor("t5")
+    assert t.n_dims == 5 and t.dimensions == [2, 3, 4, 5] and t.n_elements() == 720 and t.data_size() == 2880
+    assert len(g.tensor_data("t5")) == 2880
+
+
+def test_array_element_of_unknown_type_is_an_error_not_a_half_parsed_file():
+    # an array whose element type id is past the last known one (parser.rs:118-169)
+    img = struct.pack("<IIQQ", B.MAGIC, 3, 0, 1) + B.string(3, "k") + struct.pack("<I", B.ARRAY) + \
+        struct.pack("<I", 13) + struct.pack("<Q", 1) + b"\0" * 8
+    with pytest.raises(gguf.InvalidMetadata):
+        gguf.GgufModel.from_bytes(img)
 
 
 def test_tensor_errors():

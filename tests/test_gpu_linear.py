@@ -316,7 +316,7 @@ def test_linear_forward_multi_unequal_rows(hip, ref, t):
 
 @pytest.mark.parametrize("types", [(O.Q4_K, O.Q4_K, O.Q6_K), (O.Q4_0, O.Q4_0, O.Q4_0), (O.Q8_0, O.Q4_K, O.IQ4_XS)],
                          ids=["q4k_q4k_q6k", "q4_0", "mixed"])
-def test_ffn_swiglu(hip, ref, types):
+def test_ffn_swiglu(hip, ref, tuning, types):
     for hidden, inter in ((512, 1024), (4096, 14336)):
         say("ffn", types, hidden, inter)
         tg, tu, td = types
@@ -330,14 +330,11 @@ def test_ffn_swiglu(hip, ref, types):
         d_wg, d_wu, d_wd = dev(wg), dev(wu), dev(wd)
         L.ffn_swiglu_dev((tg, d_wg), (tu, d_wu), (td, d_wd), d_acts, d_out, hidden, inter, ws)
         got = host(d_out)
-        from oxillama_amd import capi
-        capi.load().oxq_set_ffn_fusion(0)  # gate + up, SwiGLU, down as three launches: the same bits
-        try:
-            d_out3 = torch.empty_like(d_out)
-            L.ffn_swiglu_dev((tg, d_wg), (tu, d_wu), (td, d_wd), d_acts, d_out3, hidden, inter, ws)
-            assert np.array_equal(got.view(np.uint32), host(d_out3).view(np.uint32))
-        finally:
-            capi.load().oxq_set_ffn_fusion(1)
+        tuning("ffn_fusion", 0)  # gate + up, SwiGLU, down as three launches: the same bits
+        d_out3 = torch.empty_like(d_out)
+        L.ffn_swiglu_dev((tg, d_wg), (tu, d_wu), (td, d_wd), d_acts, d_out3, hidden, inter, ws)
+        assert np.array_equal(got.view(np.uint32), host(d_out3).view(np.uint32))
+        tuning("ffn_fusion", 1)
         # step by step with the plain entry points: bit-identical
         g = torch.empty(inter, dtype=torch.float32, device=DEV)
         u = torch.empty(inter, dtype=torch.float32, device=DEV)

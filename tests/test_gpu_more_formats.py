@@ -272,14 +272,13 @@ def _tile_zero_point(t, acts, rows, k_):
 @pytest.mark.parametrize("shape", [(8, 32, 256), (40, 100, 1024), (130, 129, 2048), (200, 257, 1024), (512, 160, 512)],
                          ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("t", TILE_TYPES, ids=ids)
-def test_prefill_tile_kernel(hip, ref, shape, t):
+def test_prefill_tile_kernel(hip, ref, tuning, shape, t):
     """The int8-MFMA tile kernel on the added formats: integer sub-block sums bit-exact, fp32 within 1e-5 of
     the reference's fused kernel, every tile shape (split k, 64 x 128, 128 x 64), ragged edges, accumulate."""
-    from oxillama_amd import capi
     m, n, k_ = shape
     say("prefill", O.NAMES[t], shape)
-    capi.load().oxq_set_gemm_tile_min_rows(1)
-    try:
+    tuning("gemm_tile_min_rows", 1)
+    if True:
         w = O.random_blocks(t, 900 + m, n, k_)
         x = synth.normal_f32(950 + n, m * k_)
         acts = ref.quantize_q8_0(x)
@@ -303,8 +302,6 @@ def test_prefill_tile_kernel(hip, ref, shape, t):
         want = np.stack([ref.block_sums(t, w, acts[r * arb:(r + 1) * arb], n, k_) for r in range(m)])
         assert np.array_equal(host(dsum) - _tile_zero_point(t, acts, m, k_), want), "integer sub-block sums"
         assert torch.equal(dy3, dy)
-    finally:
-        capi.load().oxq_set_gemm_tile_min_rows(0)
 
 
 @pytest.mark.parametrize("t", [O.Q5_K, O.Q5_0, O.IQ4_NL, O.Q3_K, O.Q2_K], ids=ids)

@@ -251,15 +251,13 @@ def test_gemv_dev_quantizes_in_kernel_bit_identically(hip, ref, t):
 
 
 @pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
-def test_gemm_few_rows_share_one_weight_pass(hip, ref, t):
+def test_gemm_few_rows_share_one_weight_pass(hip, ref, tuning, t):
     """2..7 activation rows without the tile kernel: GEMV launches that take up to four rows per
     pass over the weights give the same bits as one fused matvec per row (short rows, rows split
     over four waves, and rows too long for the shared pass)."""
     import torch
-    from oxillama_amd import capi
-    lib = capi.load()
-    lib.oxq_set_gemm_tile_min_rows(1000)
-    try:
+    tuning("gemm_tile_min_rows", 1000)
+    if True:
         for n, k_ in ((40, 768), (24, 4096), (12, 14336), (6, 32768)):
             w = synth.weights(t, 840 + n, n, k_)
             dw = torch.from_numpy(w).cuda()
@@ -276,8 +274,6 @@ def test_gemm_few_rows_share_one_weight_pass(hip, ref, t):
                     kern.gemm_q8_dev(dw, da, got, m, n, k_, accumulate=acc)
                     torch.cuda.synchronize()
                     assert torch.equal(got, want), (O.NAMES[t], n, k_, m, acc)
-    finally:
-        lib.oxq_set_gemm_tile_min_rows(0)
 
 
 def _ragged_cols(t):
@@ -554,18 +550,15 @@ def _oracle_prefill(ref, t, w, acts, m, n, k_, rows=None):
 @pytest.mark.parametrize("shape", [(8, 32, 256), (33, 100, 1024), (128, 160, 512), (200, 257, 1024), (64, 64, 4096),
                                    (130, 129, 2048)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
-def test_prefill_tile_kernel(hip, ref, shape, t):
+def test_prefill_tile_kernel(hip, ref, tuning, shape, t):
     """Weights of every format x Q8_0 activations on the int8-MFMA tile kernel: integer sub-block sums bit-exact, fp32 within
     1e-5, ragged tile edges in both directions, overwrite and accumulate."""
     import torch
     from oxillama_amd import capi
     m, n, k_ = shape
     say("prefill", O.NAMES[t], shape)
-    capi.load().oxq_set_gemm_tile_min_rows(1)  # small shapes would otherwise take the GEMV route
-    try:
-        _prefill_tile_case(hip, ref, shape, t)
-    finally:
-        capi.load().oxq_set_gemm_tile_min_rows(0)
+    tuning("gemm_tile_min_rows", 1)  # small shapes would otherwise take the GEMV route
+    _prefill_tile_case(hip, ref, shape, t)
 
 
 def _prefill_tile_case(hip, ref, shape, t):
@@ -737,21 +730,68 @@ def test_registered_weights_and_cache(hip, ref):
     assert_close(dy.cpu().numpy(), y_ref, "registered")
     assert lib.oxq_weights_release(h) == capi.OK
     # host-slice route with the cache on: same answer, and a changed buffer is noticed
+    import ctypes as C
+
+    def stats():
+        e, b, h, u = C.c_size_t(), C.c_size_t(), C.c_uint64(), C.c_uint64()
+        assert lib.oxq_weight_cache_stats(C.byref(e), C.byref(b), C.byref(h), C.byref(u)) == capi.OK
+        return e.value, b.value, h.value, u.value
+
     lib.oxq_weight_cache_enable(1)
     try:
         k = hip.HipKernel(t)
+        _, _, hits0, ups0 = stats()
         for _ in range(2):
             out = np.zeros(n_rows, dtype=np.float32)
             k.matvec_q8_fused(w, a, out, n_rows, n_cols)
             assert_close(out, y_ref, "cached")
+        assert stats() == (1, w.nbytes, hits0 + 1, ups0 + 1)
         w2 = synth.weights(t, 503, n_rows, n_cols)
         w[:] = w2
         out = np.zeros(n_rows, dtype=np.float32)
         k.matvec_q8_fused(w, a, out, n_rows, n_cols)
         assert_close(out, canonical_ref(ref, t, w2, a, n_rows, n_cols), "cache refreshed")
+        # the contract of mode 1: a caller that changes bytes in place says so
+        w[5] ^= 0xFF
+        assert lib.oxq_weight_cache_invalidate(w.ctypes.data) == capi.OK
+        assert stats()[0] == 0
+        out = np.zeros(n_rows, dtype=np.float32)
+        k.matvec_q8_fused(w, a, out, n_rows, n_cols)
+        assert_close(out, canonical_ref(ref, t, w, a, n_rows, n_cols), "invalidated")
+        # mode 2 hashes every byte: a change between the sampled pieces is seen without being told
+        lib.oxq_weight_cache_enable(2)
+        big_rows = 256
+        wb = synth.weights(t, 504, big_rows, n_cols)  # larger than the 4096 sampled bytes
+        assert wb.nbytes > 64 * 64 * 2
+        for flip in (None, 64 + 3, wb.nbytes // 2 + 1):
+            if flip is not None:
+                wb[flip] ^= 0x10
+            before = stats()[3]
+            out = np.zeros(big_rows, dtype=np.float32)
+            k.matvec_q8_fused(wb, a, out, big_rows, n_cols)
+            assert stats()[3] == before + 1, "a changed byte must cause a new upload"
+            assert_close(out, canonical_ref(ref, t, wb, a, big_rows, n_cols), f"verified cache, flip {flip}")
+        # byte cap: the least recently used copy goes first
+        lib.oxq_weight_cache_enable(1)
+        lib.oxq_weight_cache_clear()
+        bufs = [synth.weights(t, 510 + i, n_rows, n_cols) for i in range(3)]
+        lib.oxq_weight_cache_set_limit(2 * bufs[0].nbytes)
+        for wi in bufs:
+            k.matvec_q8_fused(wi, a, np.zeros(n_rows, dtype=np.float32), n_rows, n_cols)
+        assert stats()[:2] == (2, 2 * bufs[0].nbytes)
+        hits = stats()[2]
+        k.matvec_q8_fused(bufs[2], a, np.zeros(n_rows, dtype=np.float32), n_rows, n_cols)
+        k.matvec_q8_fused(bufs[1], a, np.zeros(n_rows, dtype=np.float32), n_rows, n_cols)
+        assert stats()[2] == hits + 2
+        ups = stats()[3]
+        out = np.zeros(n_rows, dtype=np.float32)
+        k.matvec_q8_fused(bufs[0], a, out, n_rows, n_cols)  # evicted earlier: uploaded again
+        assert stats()[3] == ups + 1
+        assert_close(out, canonical_ref(ref, t, bufs[0], a, n_rows, n_cols), "after eviction")
     finally:
         lib.oxq_weight_cache_enable(0)
         lib.oxq_weight_cache_clear()
+        lib.oxq_weight_cache_set_limit(16 << 30)
 
 
 # ---- concurrency and lifecycle ------------------------------------------------------------------
