@@ -248,6 +248,19 @@ size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k);
 int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                     float *d_out, size_t m, size_t n, size_t k, int accumulate,
                     void *d_workspace, size_t workspace_bytes, void *stream);
+/* oxq_gemm_q8_dev for callers that cannot allocate device memory and have no workspace to pass
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  The tile kernel's workspace is a static array in device
+ * memory that the library holds on each GPU it was initialised on (8 MiB:
+ * oxq_gemm_q8_static_max_workspace_bytes()); the call allocates nothing, synchronises nothing and
+ * gives the bits of oxq_gemm_q8_dev.  Shapes whose oxq_gemm_q8_workspace_bytes exceeds the
+ * array return OXQ_ERR_BUFFER_TOO_SMALL (needed, available); oxq_init must have run (the call
+ * does not initialise lazily: OXQ_ERR_NO_DEVICE).  All calls on one GPU share the array: calls
+ * that overlap in time on one GPU (different streams or threads) race on it. */
+size_t oxq_gemm_q8_static_max_workspace_bytes(void);
+int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
+                           float *d_out, size_t m, size_t n, size_t k, int accumulate,
+                           void *stream);
 /* Debug: as oxq_gemm_q8_dev (overwrite), and the exact int32 group sums of the tile
  * kernel, d_sums[(r * n + c) * groups + g], groups = k/32 (k/16 for Q6_K).  For Q4_0 the
  * (and Q5_0) the tile kernel multiplies the unsigned values (sum q*a); the "- 8" ("- 16") enters in

@@ -117,6 +117,9 @@ SIGNATURES = {
     "oxq_gemv_multi_dev": (C.c_int, [C.c_uint32, C.c_size_t, C.POINTER(C.c_void_p), C.c_void_p,
                                      C.POINTER(C.c_void_p), C.c_size_t, C.c_size_t, C.c_int, C.c_void_p]),
     "oxq_gemm_q8_workspace_bytes": (C.c_size_t, [C.c_uint32, C.c_size_t, C.c_size_t, C.c_size_t]),
+    "oxq_gemm_q8_static_max_workspace_bytes": (C.c_size_t, []),
+    "oxq_gemm_q8_static_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                         C.c_size_t, C.c_int, C.c_void_p]),
     "oxq_gemm_q8_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                   C.c_size_t, C.c_size_t, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "oxq_gemm_block_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,

@@ -15,7 +15,17 @@ namespace oxq {
 hipError_t launch_dequant(uint32_t type, const uint8_t *blocks, size_t n_blocks, float *out, hipStream_t stream);
 }
 
+// Workspace of oxq_gemm_q8_static_dev: the tile kernel's re-laid-out activations (int8 payload, fp32 block sums,
+// f16 scales) live here instead of in a caller's or the library's allocation.  Every GPU the library runs on holds
+// its own copy at its own address until the process ends; host code reaches it only through the address that
+// hipGetSymbolAddress returned for that device (static_scratch_ptr), never through this name.
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)8 << 20;
+static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int MAX_DEVICES = 64;
+uint8_t *static_scratch_ptr[MAX_DEVICES] = {nullptr};  // per device, filled by oxq_init with that device current
 
 struct ErrorDetail {
     int status = OXQ_OK;
@@ -277,6 +287,11 @@ int oxq_init(int device) {
         char msg[200];
         std::snprintf(msg, sizeof(msg), "device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
         return fail(OXQ_ERR_NO_DEVICE, 0, 0, msg);
+    }
+    if (device < MAX_DEVICES && !static_scratch_ptr[device]) {
+        uint8_t *p = nullptr;
+        OXQ_HIP(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+        static_scratch_ptr[device] = p;
     }
     g.device = device;
     g.cus = (uint32_t)prop.multiProcessorCount;
@@ -848,6 +863,38 @@ int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
                     size_t n, size_t k, int accumulate, void *d_workspace, size_t workspace_bytes, void *stream) {
     return gemm_dev(type, d_weights, d_acts_q8, d_out, nullptr, m, n, k, accumulate, nullptr, d_workspace, workspace_bytes,
                     stream);
+}
+
+size_t oxq_gemm_q8_static_max_workspace_bytes(void) { return STATIC_SCRATCH_BYTES; }
+
+int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, size_t m,
+                           size_t n, size_t k, int accumulate, void *stream) {
+    int st = check_dev_shape(type, n, k, true);
+    if (st != OXQ_OK) return st;
+    if (m > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, m, "dimension exceeds 2^32-1");
+    // no lazy initialisation here: that would be the one path of this call that allocates
+    if (!g.initialised.load(std::memory_order_acquire) || g.device < 0 || g.device >= MAX_DEVICES ||
+        !static_scratch_ptr[g.device])
+        return fail(OXQ_ERR_NO_DEVICE, 0, 0, "call oxq_init first: this entry point sets nothing up by itself");
+    if (m == 0 || n == 0 || k == 0) return OXQ_OK;
+    const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k);
+    const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k) : 0;
+    if (need > STATIC_SCRATCH_BYTES)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, STATIC_SCRATCH_BYTES,
+                    "shape needs more workspace than the static scratch holds: use oxq_gemm_q8_dev with a workspace");
+    oxq::GemmArgs ga;
+    ga.W = d_weights;
+    ga.A = d_acts_q8;
+    ga.out = d_out;
+    ga.sums = nullptr;
+    ga.workspace = tiles ? static_scratch_ptr[g.device] : nullptr;  // every byte the tile kernel reads is written
+    ga.by_rows = !tiles;                                            // by the preparation kernel of this same call
+    ga.m = (uint32_t)m;
+    ga.n = (uint32_t)n;
+    ga.k = (uint32_t)k;
+    ga.accumulate = accumulate ? 1 : 0;
+    OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
+    return OXQ_OK;
 }
 
 int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out,

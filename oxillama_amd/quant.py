@@ -275,6 +275,11 @@ class HipKernel:
         _check(self._lib.oxq_gemm_q8_dev(self.tensor_type, d_weights.data_ptr(), d_acts.data_ptr(),
                                          d_out.data_ptr(), m, n, k, int(accumulate), ws_ptr, ws_len, self._stream()))
 
+    def gemm_q8_static_dev(self, d_weights, d_acts, d_out, m, n, k, accumulate=False):
+        """gemm_q8_dev on the library's static device scratch: allocates nothing (shapes up to the scratch size)."""
+        _check(self._lib.oxq_gemm_q8_static_dev(self.tensor_type, d_weights.data_ptr(), d_acts.data_ptr(),
+                                                d_out.data_ptr(), m, n, k, int(accumulate), self._stream()))
+
     def gemm_block_sums_dev(self, d_weights, d_acts, d_out, d_sums, m, n, k, workspace=None):
         ws_ptr = workspace.data_ptr() if workspace is not None else None
         ws_len = workspace.numel() if workspace is not None else 0
