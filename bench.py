@@ -32,12 +32,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per gate+up launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by
-# what the counter reads for a copy kernel of known size (2.000 and 1.000); the runs and figures are in
-# profiles/hbm_traffic_gemv_gate_up_lm_head_prefill_pmc.txt.  Algorithmic bytes are 66 179 328 for the plain
-# gate + up launch and 66 079 872 for the launch that also forms and quantizes h.
-MEASURED_TRAFFIC_GATE_UP = 66318438
-MEASURED_TRAFFIC_GATE_UP_SWIGLU = 66301133
+# HBM bytes per launch come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --traffic-probe`, each
+# counter scaled by what it reads for a copy kernel of known size; the summary of those runs carries one
+# `traffic-record:` line per kernel, keyed by the launch it was measured on (kernel instantiation, grid).  This
+# run asks the library which launch it timed and reports the record only if the two agree.
+TRAFFIC_SUMMARY = os.path.join("profiles", "hbm_traffic_gemv_gate_up_lm_head_prefill_pmc.txt")
 INT8_PEAK_TOPS = 5000.0
 
 Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS = 2, 8, 12, 14, 23
@@ -53,12 +52,36 @@ def algorithmic_bytes(t, n_rows, n_cols):
     return n_rows * row_bytes(t, n_cols) + n_cols // 32 * 34 + n_rows * 4
 
 
+def last_launch():
+    """What the library launched last on this thread: 'kernel<type,params> grid XxY block B'."""
+    import ctypes as C
+    from oxillama_amd import capi
+    buf = C.create_string_buffer(256)
+    capi.load().oxq_last_launch(buf, 256)
+    return buf.value.decode()
+
+
+def measured_traffic(launch):
+    """HBM bytes per launch of `launch` from the tracked counter summary, or (None, reason)."""
+    path = os.path.join(ROOT, TRAFFIC_SUMMARY)
+    try:
+        lines = [l for l in open(path) if l.startswith("traffic-record:")]
+    except OSError:
+        return None, f"{TRAFFIC_SUMMARY} is missing"
+    for l in lines:
+        fields = dict(kv.split("=", 1) for kv in l[len("traffic-record:"):].strip().split("; "))
+        if fields.get("launch") == launch:
+            return int(fields["hbm_bytes"]), f"{TRAFFIC_SUMMARY} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, copy-kernel scaled)"
+    return None, f"no counter record for '{launch}' in {TRAFFIC_SUMMARY}: the launch changed since the counters were read"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=32)
     ap.add_argument("--layers", type=int, default=32, help="distinct weight sets the steps rotate over")
+    ap.add_argument("--replays", type=int, default=7, help="times the K timed steps are replayed; the median is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra-kernels", action="store_true")
@@ -113,8 +136,10 @@ def main():
             torch.cuda.synchronize()
             k_q4k.matvec_q8_fused_multi_dev([g, u], xq, [yg, yu], F, H, accumulate=False)
             torch.cuda.synchronize()
+            launches = {"gate_up": last_launch()}
             linear.gate_up_swiglu_dev(Q4_K, g, u, xq, None, hq_probe, F, H)
             torch.cuda.synchronize()
+            launches["gate_up_swiglu"] = last_launch()
         V = 128256
         logits = torch.zeros(V, dtype=torch.float32, device=dev)
         for i in range(2):
@@ -122,6 +147,7 @@ def main():
             torch.cuda.synchronize()
             k_q6k.matvec_q8_fused_dev(lm, xq, logits, V, H, accumulate=False)
             torch.cuda.synchronize()
+            launches["lm_head"] = last_launch()
             del lm
         M = 512
         xsq = torch.empty(M * (H // 32 * 34), dtype=torch.uint8, device=dev)
@@ -133,7 +159,8 @@ def main():
             torch.cuda.synchronize()
             k_q4k.gemm_q8_dev(w, xsq, ys, M, F, H, workspace=ws)
             torch.cuda.synchronize()
-        print(json.dumps({"traffic_probe": "done", "copy_bytes": nbytes}), flush=True)
+            launches["prefill"] = last_launch()
+        print(json.dumps({"traffic_probe": "done", "copy_bytes": nbytes, "launches": launches}), flush=True)
         return
 
     def upload(t, seed, n_rows, n_cols):
@@ -210,15 +237,26 @@ def main():
     g_warm = capture(lambda: [step(i) for i in range(W)]) if W > 0 else None
     g_main = capture(lambda: [step(W + i) for i in range(K)])
     if g_warm is not None:
-        g_warm.replay()
+        with torch.cuda.stream(stream):
+            g_warm.replay()
     torch.cuda.synchronize()
-    t_start = time.perf_counter()
-    with torch.cuda.stream(stream):
-        g_main.replay()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t_start) * 1e3
-    ms_per_step = wall_ms / K
+    # exactly K steps per replay, bracketed by synchronisation on both sides; the replay is repeated and the
+    # MEDIAN is the reported figure (one replay of few steps is a sub-millisecond sample)
+    R = max(1, args.replays)
+    wall_ms, event_ms = [], []
+    for _ in range(R):
+        torch.cuda.synchronize()
+        t_start = time.perf_counter()
+        ev = timed_replay(g_main)  # HIP events on the launch stream, waits for the second one
+        torch.cuda.synchronize()
+        wall_ms.append((time.perf_counter() - t_start) * 1e3)
+        event_ms.append(ev)
+    ms_per_step = float(np.median(wall_ms)) / K
     value = step_weight_bytes / (ms_per_step * 1e-3) / 1e9
+    timing = {"replays": R, "steps_per_replay": K, "reported": "median of the replays' host wall time / K",
+              "ms_per_step_median": round(ms_per_step, 5), "ms_per_step_min": round(min(wall_ms) / K, 5),
+              "ms_per_step_max": round(max(wall_ms) / K, 5),
+              "ms_per_step_hip_events_median": round(float(np.median(event_ms)) / K, 5)}
 
     with torch.cuda.stream(stream):  # the per-kernel legs below read pre-quantized activations
         quant.quantize_q8_0_dev(x, xq)
@@ -277,16 +315,22 @@ def main():
     with torch.cuda.stream(stream):  # the legs below read the quantized synthetic h again
         quant.quantize_q8_0_dev(h, hq)
         stream.synchronize()
-    # the dominant kernel of the timed step
-    if args.unfused_swiglu or args.fused_quantize:
-        dom, dom_name, dom_traffic = pair, "gemv_q8_cached<Q4_K>, ffn_gate + ffn_up (2 x 14336x4096) in one launch", \
-            MEASURED_TRAFFIC_GATE_UP
-    else:
-        dom, dom_name, dom_traffic = pair_swiglu, "gemv_q8_gate_up_swiglu<Q4_K>, ffn_gate + ffn_up (2 x 14336x4096) + " \
-            "SwiGLU + Q8_0 quantizer of h in one launch", MEASURED_TRAFFIC_GATE_UP_SWIGLU
-    roofline = {"bound": "hbm", "kernel": dom_name,
+    # the dominant kernel of the timed step, named by the launch the library actually makes for it
+    with torch.cuda.stream(stream):
+        if args.unfused_swiglu or args.fused_quantize:
+            k_q4k.matvec_q8_fused_multi_dev([layers[0]["gate"], layers[0]["up"]], xq, [yg, yu], F, H, accumulate=False)
+            dom, dom_name = pair, "ffn_gate + ffn_up (2 x 14336x4096 Q4_K) in one launch"
+        else:
+            linear.gate_up_swiglu_dev(Q4_K, layers[0]["gate"], layers[0]["up"], xq, None, hq, F, H)
+            dom, dom_name = pair_swiglu, "ffn_gate + ffn_up (2 x 14336x4096 Q4_K) + SwiGLU + Q8_0 quantizer of h in one launch"
+        dom_launch = last_launch()
+        quant.quantize_q8_0_dev(h, hq)
+        stream.synchronize()
+    dom_traffic, traffic_source = measured_traffic(dom_launch)
+    roofline = {"bound": "hbm", "kernel": dom_launch + ": " + dom_name,
                 "achieved": dom["algorithmic_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": dom["frac_hbm_peak"],
-                "traffic": dom_traffic, "us_per_call": dom["us_per_call"], "algorithmic_bytes": dom["algorithmic_bytes"]}
+                "traffic": dom_traffic, "traffic_source": traffic_source, "us_per_call": dom["us_per_call"],
+                "algorithmic_bytes": dom["algorithmic_bytes"]}
 
     kernels = {"q4k_gate_plus_up_one_launch": pair, "q4k_gate_up_swiglu_one_launch": pair_swiglu,
                "q4k_gate_up_14336x4096": time_kernel(k_q4k, Q4_K, gate_up, xq, yg, F, H)}
@@ -432,7 +476,8 @@ def main():
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         import oracle as O
         O.load()
-        cores = min(os.cpu_count() or 1, 16)
+        host_cores = os.cpu_count() or 1
+        cores = min(host_cores, 16)  # threads actually used (the GPU box's CPU share)
         hw = {"q": layers[0]["q"].cpu().numpy(), "gate": layers[0]["gate"].cpu().numpy(),
               "up": layers[0]["up"].cpu().numpy(), "down": layers[0]["down"].cpu().numpy()}
         hx = x.cpu().numpy()
@@ -505,7 +550,8 @@ def main():
 
         s_mt, n_mt = time_cpu(cores, 8.0)
         s_1t, n_1t = time_cpu(1, 8.0)
-        cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
+        cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "host_cores": host_cores,
+               "kind": "port",
                "sample": f"one layer (same 4 matrices, quantization of x, SwiGLU + quantization of h), {n_mt} repeats, static row split over "
                          f"{cores} threads; " + ("AVX2 intrinsics twin of the reference's fused rows (Q6_K body is scalar "
                          "there too)" if avx2 else "scalar C restatement of the reference's AVX2-tier fused rows"),
@@ -521,6 +567,7 @@ def main():
         "steps": K,
         "warmup": W,
         "ms_per_step": round(ms_per_step, 5),
+        "timing": timing,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

@@ -30,6 +30,10 @@ int oxq_set_gemv_waves_per_row(unsigned waves);
 int oxq_set_gemm_tile_min_rows(unsigned rows);
 /* Tile shape / prefetch depth of the prefill kernel (tuning knob; 0 restores the default). */
 int oxq_set_gemm_variant(int variant);
+/* Which kernel instantiation and launch shape the calling thread's last GEMV / fused gate+up / tile-kernel
+ * launch used, as "name<type,p0,p1,p2,p3> grid XxY block B" (template parameters in the kernel's own order):
+ * lets a measurement name what it timed and notice when a launch policy has changed under it. */
+int oxq_last_launch(char *out, size_t out_len);
 /* oxq_ffn_swiglu_dev: 1 (default) = gate, up, SwiGLU and the quantizer of h in one launch where a kernel
  * exists for the type and row length; 0 = the separate launches (same bits). */
 int oxq_set_ffn_fusion(int enabled);

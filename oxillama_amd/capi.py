@@ -183,6 +183,7 @@ TUNING_SIGNATURES = {
     "oxq_set_gemm_variant": (C.c_int, [C.c_int]),
     "oxq_set_gemm_tile_min_rows": (C.c_int, [C.c_uint]),
     "oxq_set_ffn_fusion": (C.c_int, [C.c_int]),
+    "oxq_last_launch": (C.c_int, [C.c_char_p, C.c_size_t]),
 }
 
 _lib = None

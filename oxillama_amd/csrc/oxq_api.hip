@@ -263,6 +263,7 @@ int tensor_dims(uint32_t type, size_t data_len, const size_t *shape, size_t n_di
 }  // namespace
 
 namespace oxq {
+thread_local LaunchNote g_last_launch;
 uint32_t device_cus() { return g.cus ? g.cus : 256; }
 int set_error(int status, size_t a, size_t b, const char *msg) { return fail(status, a, b, msg); }
 int ensure_device() { return ensure_init(); }
@@ -447,6 +448,15 @@ int oxq_set_gemv_rows_per_batch(unsigned rows) {
 
 int oxq_set_gemv_waves_per_row(unsigned waves) {
     g.waves_per_row = waves >= 4 ? 4 : (waves ? 1 : 0);
+    return OXQ_OK;
+}
+
+int oxq_last_launch(char *out, size_t out_len) {
+    if (!out || out_len == 0) return fail(OXQ_ERR_INTERNAL, 0, 0, "null output");
+    const oxq::LaunchNote &n = oxq::g_last_launch;
+    const char *tn = oxq_type_name(n.type);
+    std::snprintf(out, out_len, "%s<%s,%d,%d,%d,%d> grid %ux%u block %u", n.kernel, tn ? tn : "-", n.p[0], n.p[1], n.p[2],
+                  n.p[3], n.grid_x, n.grid_y, n.block);
     return OXQ_OK;
 }
 

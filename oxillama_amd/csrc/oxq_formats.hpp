@@ -24,6 +24,7 @@
 // multiply-adds before the cross-lane sum; only the accumulation order and the
 // placement of roundings differ from the reference, within the 1e-5*|y|inf bar.
 #pragma once
+#include "../../include/oxq.h"
 #include "oxq_device.hpp"
 
 namespace oxq {
@@ -136,6 +137,7 @@ __device__ __forceinline__ void quantize_to_lds(const float *__restrict__ x, uin
 // super-block; the 16-byte header is read by each of them (same cache line).
 struct FmtQ4K {
     static constexpr uint32_t BLOCK_BYTES = 144, BLOCK_COLS = 256, UNIT_COLS = 64;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q4_K;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {
         uint32_t g, sh;
@@ -225,6 +227,7 @@ struct FmtQ4K {
 // 8hh + is + 2j, activation block 8b + 4hh + j bytes 16is..+16.
 struct FmtQ6K {
     static constexpr uint32_t BLOCK_BYTES = 210, BLOCK_COLS = 256, UNIT_COLS = 64;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q6_K;
     // Measured on MI355X (4096 x 14336 and 128256 x 4096): four waves per compute unit with two rows per
     // batch beat eight waves with one (11.4 against 11.8 us, 73.6 against 76.6 us).
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 4000;
@@ -342,6 +345,7 @@ struct FmtQ6K {
 // Unit = one 34-byte block against the activation block of the same index.
 struct FmtQ8_0 {
     static constexpr uint32_t BLOCK_BYTES = 34, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q8_0;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {};
     struct Act {
@@ -408,6 +412,7 @@ __device__ __forceinline__ void split_even_odd(const u32x4 &q0, const u32x4 &q1,
 // Unit = one 18-byte block.  sum (q-8)*a = sum q*a - 8*sum a.
 struct FmtQ4_0 {
     static constexpr uint32_t BLOCK_BYTES = 18, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q4_0;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {};
     struct Act {
@@ -466,6 +471,7 @@ struct FmtQ4_0 {
 // d * float((ls - 32) * sum kvalues[idx] * a) * d_a.
 struct FmtIQ4XS {
     static constexpr uint32_t BLOCK_BYTES = 136, BLOCK_COLS = 256, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_IQ4_XS;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;  // two rows per batch up to this slice of a row per wave
     struct Lane {
         uint32_t i;

@@ -33,6 +33,7 @@ __device__ __forceinline__ uint32_t spread4(uint32_t x) {
 // (low) and 2i+1 (high); w = d * nibble + m.  sum w a = d * sum(nibble a) + m * sum a.
 struct FmtQ4_1 {
     static constexpr uint32_t BLOCK_BYTES = 20, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q4_1;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;
     struct Lane {};
     struct Act {
@@ -77,6 +78,7 @@ struct FmtQ4_1 {
 // w = d * (q5 - 16).  The fifth bits are spread to one per byte and merged into the nibble dword.
 struct FmtQ5_0 {
     static constexpr uint32_t BLOCK_BYTES = 22, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q5_0;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;
     struct Lane {};
     struct Act {
@@ -136,6 +138,7 @@ struct FmtQ5_0 {
 // w = d * q5 + m.
 struct FmtQ5_1 {
     static constexpr uint32_t BLOCK_BYTES = 24, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q5_1;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;
     struct Lane {};
     struct Act {
@@ -172,6 +175,7 @@ struct FmtQ5_1 {
 // Q8_1, Q/reference/q8_1.rs:36-42.  36 B = f16 d, f16 s (d * sum q, unused), 32 x i8; w = d * q.
 struct FmtQ8_1 {
     static constexpr uint32_t BLOCK_BYTES = 36, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q8_1;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;
     struct Lane {};
     struct Act {
@@ -213,6 +217,7 @@ struct FmtQ8_1 {
 // (Q/reference/iq_shared.rs:16-18); byte i holds weights 2i (low) and 2i+1 (high); w = d * kv[idx].
 struct FmtIQ4NL {
     static constexpr uint32_t BLOCK_BYTES = 18, BLOCK_COLS = 32, UNIT_COLS = 32;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_IQ4_NL;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 3400;
     struct Lane {};
     struct Act {
@@ -263,6 +268,7 @@ struct FmtIQ4NL {
 // (high) of qh[l].  Term per sub-block: (d*sc*sum(q5 a) - dmin*mn*sum a) * d_a.
 struct FmtQ5K {
     static constexpr uint32_t BLOCK_BYTES = 176, BLOCK_COLS = 256, UNIT_COLS = 64;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q5_K;
     // measured: two rows per batch beat one at both 14336 x 4096 and 4096 x 14336 (11.1 -> 10.4-10.8 us)
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 4000;
     using Lane = FmtQ4K::Lane;
@@ -355,6 +361,7 @@ __device__ __forceinline__ void load_act16x4(Act16x4 &a, const SRC &src, uint32_
 // of qs[32n + 16hf + l]; term (d*sc*sum(q a) - dmin*mn*sum a) * d_a per 16 weights.
 struct FmtQ2K {
     static constexpr uint32_t BLOCK_BYTES = 84, BLOCK_COLS = 256, UNIT_COLS = 64;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q2_K;
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 4000;  // measured: 9.5-9.9 -> 8.4-8.8 us with two rows per batch
     struct Lane {
         uint32_t n, hf;
@@ -402,6 +409,7 @@ struct FmtQ2K {
 // >> 2j & 3) - (hmask[16hf + l] bit (4n + j) ? 0 : 4); term d * (sc - 32) * sum(q3 a) * d_a.
 struct FmtQ3K {
     static constexpr uint32_t BLOCK_BYTES = 110, BLOCK_COLS = 256, UNIT_COLS = 64;
+    static constexpr uint32_t TYPE_ID = OXQ_TYPE_Q3_K;
     // measured: 11.9-12.3 -> 10.8-11.0 us with two rows per batch and four waves per compute unit
     static constexpr uint32_t TWO_ROW_BATCH_BYTES = 4000;
     static constexpr uint32_t WAVES_PER_CU = 4;

@@ -754,6 +754,7 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return e;
     }
+    note_launch(OCC == 3 ? "gemm_tile_kernel_occ3" : "gemm_tile_kernel", F::TYPE, MT, NT, WM, DIST, grid.x, grid.y, 256);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a.W, p.q8t, p.P, p.da16, a.out, a.sums, a.m, p.mpad, a.n,
                        a.k, a.accumulate, a.bias, m_tiles, n_tiles, a.offsets, a.w_stride);
     return hipGetLastError();

@@ -50,6 +50,8 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     const void *acts = a.X ? static_cast<const void *>(a.X) : static_cast<const void *>(a.A);
     // fp32 source: LDS for the quantized vector (32 payload bytes + one f16 scale per block)
     const size_t lds = std::is_same<SRC, ActF32>::value ? (size_t)units * (F::UNIT_COLS / 32) * 34 : 0;
+    note_launch(std::is_same<SRC, ActF32>::value ? "gemv_q8_cached_f32" : "gemv_q8_cached", F::TYPE_ID, STEPS, RB, KS, DUMP,
+                blocks, n_mats, 256);
     hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), lds, stream, w[0],
                        w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums, rows[0],
                        rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols);
@@ -143,12 +145,13 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
     const bool two = row_bytes <= F::TWO_ROW_BATCH_BYTES;
     const dim3 grid(n_rows / 32);
 #define OXQ_LAUNCH(ST, RBV)                                                                                          \
+    note_launch("gemv_q8_gate_up_swiglu", F::TYPE_ID, ST, RBV, 4, 0, grid.x, 1, 256);                                \
     hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4>), grid, dim3(256), 0, stream, Wg, Wu, acts, hq, h,     \
                        n_rows, units, row_bytes)
     if (steps == 1) {
-        if (two) OXQ_LAUNCH(1, 2); else OXQ_LAUNCH(1, 1);
+        if (two) { OXQ_LAUNCH(1, 2); } else { OXQ_LAUNCH(1, 1); }
     } else {
-        if (two) OXQ_LAUNCH(2, 2); else OXQ_LAUNCH(2, 1);
+        if (two) { OXQ_LAUNCH(2, 2); } else { OXQ_LAUNCH(2, 1); }
     }
 #undef OXQ_LAUNCH
     return hipGetLastError();

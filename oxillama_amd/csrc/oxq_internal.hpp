@@ -46,6 +46,20 @@ struct GemvArgs {
     uint32_t n_rows_more[3] = {0, 0, 0};
 };
 
+// What the calling thread launched last (kernel template, its integer parameters, grid): kept as plain fields,
+// formatted only when oxq_last_launch asks.  Lets a measurement say which instantiation it timed.
+struct LaunchNote {
+    const char *kernel = "";
+    uint32_t type = 0;
+    int p[4] = {0, 0, 0, 0};
+    uint32_t grid_x = 0, grid_y = 0, block = 0;
+};
+extern thread_local LaunchNote g_last_launch;
+inline void note_launch(const char *kernel, uint32_t type, int p0, int p1, int p2, int p3, uint32_t gx, uint32_t gy,
+                        uint32_t block) {
+    g_last_launch = LaunchNote{kernel, type, {p0, p1, p2, p3}, gx, gy, block};
+}
+
 // Number of compute units of the current device (cached per device).
 uint32_t device_cus();
 
