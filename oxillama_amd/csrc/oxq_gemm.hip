@@ -1,7 +1,7 @@
 // The batched form of the fused matvec (prefill, decode batch, mixture-of-experts group): host
 // side, and the tile kernel instantiated for Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS.  Kernel and launch
 // templates: oxq_gemm_tile.hpp; further formats: oxq_gemm_more.hip.
-#include "oxq_gemm_tile.hpp"
+#include "oxq_gemm_stream.hpp"
 
 namespace oxq {
 

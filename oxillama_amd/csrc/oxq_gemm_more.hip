@@ -6,7 +6,7 @@
 // shapes are instantiated here.
 #define OXQ_TILE_DEFAULT_SHAPES_ONLY
 #include "oxq_formats_more.hpp"
-#include "oxq_gemm_tile.hpp"
+#include "oxq_gemm_stream.hpp"
 
 namespace oxq {
 
