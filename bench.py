@@ -75,6 +75,134 @@ def measured_traffic(launch):
     return None, f"no counter record for '{launch}' in {TRAFFIC_SUMMARY}: the launch changed since the counters were read"
 
 
+def launch_phases(torch, dev, quant, linear, upload, synth):
+    """Where the time of one decode GEMV launch goes: every wave of the kernel stamps the 100 MHz wall clock at
+    kernel entry, after its first row batch is stored and after its last (the timestamping instantiation of the
+    same kernels, oxq_set_gemv_phase_probe).  One launch at a time, a device synchronisation between launches,
+    each launch on a weight set that no earlier launch touched (so HBM, not the Infinity Cache)."""
+    import ctypes as C
+    from oxillama_amd import capi
+    lib = capi.load()
+    H, F = 4096, 14336
+    cap = 1 << 20
+    buf = torch.zeros(cap // 8, dtype=torch.int64, device=dev)
+    xq = torch.empty(H // 32 * 34, dtype=torch.uint8, device=dev)
+    hq = torch.empty(F // 32 * 34, dtype=torch.uint8, device=dev)
+    quant.quantize_q8_0_dev(torch.from_numpy(synth.normal_f32(1, H)).to(dev), xq)
+    quant.quantize_q8_0_dev(torch.from_numpy(synth.normal_f32(2, F)).to(dev), hq)
+    yH = torch.zeros(H, dtype=torch.float32, device=dev)
+    yF, yF2 = torch.zeros(F, dtype=torch.float32, device=dev), torch.zeros(F, dtype=torch.float32, device=dev)
+    hq_out = torch.empty(F // 32 * 34, dtype=torch.uint8, device=dev)
+    k = {t: quant.HipKernel(t) for t in (Q4_0, Q8_0, Q4_K, Q6_K)}
+    n_sets = 16
+    gates = [upload(Q4_K, 2000 + i, F, H) for i in range(n_sets)]
+    ups = [upload(Q4_K, 3000 + i, F, H) for i in range(n_sets)]
+    downs = [upload(Q6_K, 4000 + i, H, F) for i in range(n_sets)]
+    qs = [upload(Q8_0, 1000 + i, H, H) for i in range(n_sets)]
+    c1 = [upload(Q4_0, 5000 + i, H, H) for i in range(n_sets)]
+    cases = [
+        ("gate + up + SwiGLU + quantize, one launch (2 x 14336x4096 Q4_K)", 2 * F * row_bytes(Q4_K, H),
+         lambda i: linear.gate_up_swiglu_dev(Q4_K, gates[i], ups[i], xq, None, hq_out, F, H)),
+        ("gate + up, one launch (2 x 14336x4096 Q4_K)", 2 * F * row_bytes(Q4_K, H),
+         lambda i: k[Q4_K].matvec_q8_fused_multi_dev([gates[i], ups[i]], xq, [yF, yF2], F, H, accumulate=False)),
+        ("gate alone (14336x4096 Q4_K)", F * row_bytes(Q4_K, H),
+         lambda i: k[Q4_K].matvec_q8_fused_dev(gates[i], xq, yF, F, H, accumulate=False)),
+        ("down (4096x14336 Q6_K)", H * row_bytes(Q6_K, F),
+         lambda i: k[Q6_K].matvec_q8_fused_dev(downs[i], hq, yH, H, F, accumulate=False)),
+        ("q_proj (4096x4096 Q8_0)", H * row_bytes(Q8_0, H),
+         lambda i: k[Q8_0].matvec_q8_fused_dev(qs[i], xq, yH, H, H, accumulate=False)),
+        ("C1 (4096x4096 Q4_0)", H * row_bytes(Q4_0, H),
+         lambda i: k[Q4_0].matvec_q8_fused_dev(c1[i], xq, yH, H, H, accumulate=False)),
+    ]
+    kit = C.CDLL(os.path.join(ROOT, "oxillama_amd", "liboxq_benchkit.so"))
+    kit.oxq_benchkit_read.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint, C.c_int, C.c_void_p]
+    big = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+    sink = torch.zeros(1 << 16, dtype=torch.int32, device=dev)
+    side = torch.cuda.Stream()
+
+    def read_only(nbytes):
+        """us per launch of the read-only kernel over nbytes, for three launch shapes (work groups x loads per lane and trip)."""
+        nbytes = nbytes // 4096 * 4096
+        nbuf, out = big.numel() // nbytes, []
+        for blocks, unroll in ((512, 4), (2048, 2), (8192, 1)):
+            def body():
+                for i in range(32):
+                    kit.oxq_benchkit_read(big.data_ptr() + (i % nbuf) * nbytes, sink.data_ptr(), nbytes, blocks, unroll,
+                                          side.cuda_stream)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                body()
+                side.synchronize()
+                with torch.cuda.graph(g, stream=side):
+                    body()
+                best = 1e9
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(side)
+                    g.replay()
+                    e1.record(side)
+                    e1.synchronize()
+                    best = min(best, e0.elapsed_time(e1))
+            out.append((blocks, unroll, best * 1e3 / 32))
+        return out
+
+    print("Launch phases of the decode GEMV kernels on MI355X: python bench.py --launch-phases")
+    print("Every wave stamps the 100 MHz wall clock (10 ns steps) at kernel entry (t0), when its first row batch is stored (t1)")
+    print("and when its last is (t2).  One launch at a time (device synchronised before each), %d launches per shape, each on" % n_sets)
+    print("a weight set of its own (touched once before, %d sets = more than the 256 MB Infinity Cache for all but the two" % n_sets)
+    print("4096x4096 shapes); times in us after the earliest t0 of the launch, median over the launches.")
+    print("  entry: when waves enter the kernel (the dispatcher fills the chip);  first: first rows stored;  last: a wave's end.")
+    print("  steady: sum over waves of (bytes the wave streams after its first batch) / (t2 - t1): the rate the waves sustain")
+    print("  between ramp and tail;  span: last t2 - first t0;  whole: weight bytes / span.")
+    for name, wbytes, fn in cases:
+        rows, by_load = [], []
+        for i in range(n_sets):  # first touch of a buffer pays for its page-table walks (66 MB: 17 us against 13)
+            fn(i)
+        torch.cuda.synchronize()
+        for i in range(n_sets):
+            buf.zero_()
+            torch.cuda.synchronize()
+            lib.oxq_set_gemv_phase_probe(buf.data_ptr(), cap)
+            fn(i)
+            lib.oxq_set_gemv_phase_probe(None, 0)
+            torch.cuda.synchronize()
+            launch = last_launch()
+            raw = buf.cpu().numpy().reshape(-1, 4)
+            raw = raw[raw[:, 0] != 0]
+            t = raw[:, :3].astype(np.float64) / 100.0  # us
+            # the compute unit a wave ran on: XCC_ID (bits 3:0 of the high word), shader engine / array / CU of HW_ID
+            hw, xcc = raw[:, 3] & 0xFFFFFFFF, (raw[:, 3] >> 32) & 0xF
+            cu_id = (xcc << 12) | (((hw >> 13) & 7) << 8) | (((hw >> 12) & 1) << 4) | ((hw >> 8) & 0xF)
+            _, inv, cnt = np.unique(cu_id, return_inverse=True, return_counts=True)
+            load = cnt[inv]  # waves of this launch on the wave's compute unit
+            base = t[:, 0].min()
+            t -= base
+            dur = np.maximum(t[:, 2] - t[:, 1], 0.01)
+            n_w = len(t)
+            # a wave's bytes after its first batch: its share of the matrix minus one batch (shares are equal)
+            share = wbytes / n_w
+            first_share = share * (t[:, 1] - t[:, 0]).clip(0) / np.maximum(t[:, 2] - t[:, 0], 0.01)
+            steady = float(((share - first_share) / dur).sum()) / 1e3  # GB/s
+            rows.append([np.percentile(t[:, 0], 50), t[:, 0].max(), t[:, 1].min(), np.percentile(t[:, 1], 50),
+                         np.percentile(t[:, 2], 10), np.percentile(t[:, 2], 50), t[:, 2].max(), steady, n_w])
+            by_load.append({int(c): (int((load == c).sum()), float(np.median(t[load == c, 2])), float(t[load == c, 2].max()))
+                            for c in np.unique(load)})
+        r = np.median(np.array(rows), axis=0)
+        span = r[6]
+        print(f"\n{name}: {launch}, {int(r[8])} waves")
+        print(f"  entry  median {r[0]:5.2f}  last {r[1]:5.2f}   first  earliest {r[2]:5.2f}  median {r[3]:5.2f}   "
+              f"last  p10 {r[4]:5.2f}  median {r[5]:5.2f}  latest {r[6]:5.2f}")
+        print(f"  steady {r[7]:7.0f} GB/s ({r[7] / 80:4.1f} % of 8 TB/s)   span {span:5.2f} us   whole {wbytes / span / 1e3:6.0f} GB/s "
+              f"({wbytes / span / 1e3 / 80:4.1f} %)   ramp (median first) {r[3]:4.2f} us   tail (latest - median last) {r[6] - r[5]:4.2f} us")
+        loads = sorted(set().union(*[d.keys() for d in by_load]))
+        print("  by waves of the launch on the wave's compute unit: " + ";  ".join(
+            "%d waves/CU: %d waves, last median %.2f latest %.2f" % (
+                c, int(np.median([d[c][0] for d in by_load if c in d])), np.median([d[c][1] for d in by_load if c in d]),
+                np.median([d[c][2] for d in by_load if c in d])) for c in loads))
+        print(f"  the same bytes with a kernel that only reads (16 bytes per lane, coalesced; graph of 32 launches over "
+              f"distinct buffers): " + ", ".join(f"{b_}x{u_}: {us_:.2f} us" for b_, u_, us_ in read_only(wbytes)))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -90,6 +218,9 @@ def main():
                     help="gate + up in one launch, SwiGLU + quantize in a second (default: all of it in one launch)")
     ap.add_argument("--fused-quantize", action="store_true",
                     help="decode step with the Q8_0 quantization done inside the GEMV kernels (3 launches per layer)")
+    ap.add_argument("--launch-phases", action="store_true",
+                    help="per-wave timestamps (kernel entry, first rows stored, last rows stored) of the decode GEMV "
+                         "launches over distinct weight sets; prints the summary kept as profiles/gemv_launch_phases.txt")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="launch a 256 MiB copy kernel 3 times, then gate+up (one launch) over 8 distinct layers, "
                          "lm_head twice and the prefill matmul twice, and exit: the workload of the rocprofv3 --pmc "
@@ -165,6 +296,10 @@ def main():
 
     def upload(t, seed, n_rows, n_cols):
         return torch.from_numpy(synth.weights(t, seed, n_rows, n_cols)).to(dev)
+
+    if args.launch_phases:
+        launch_phases(torch, dev, quant, linear, upload, synth)
+        return
 
     t0 = time.time()
     layers = []

@@ -30,6 +30,12 @@ int oxq_set_gemv_waves_per_row(unsigned waves);
 int oxq_set_gemm_tile_min_rows(unsigned rows);
 /* Tile shape / prefetch depth of the prefill kernel (tuning knob; 0 restores the default). */
 int oxq_set_gemm_variant(int variant);
+/* Launch-phase probe of the decode GEMV (Q4_0, Q8_0, Q4_K, Q6_K rows of at most two 64-unit steps, and the
+ * fused gate + up launch): while d_buffer is set, those launches run an instantiation of the same kernel in
+ * which every wave writes four uint64 words to d_buffer[(block * 4 + wave) * 4 ...]: three 100 MHz wall-clock
+ * timestamps -- kernel entry, its first row batch stored, its last -- and where it ran (XCC_ID register in the
+ * high half, HW_ID register in the low half).  Blocks of a multi-matrix launch are numbered matrix-major.  A launch that would not fit `bytes` runs unprobed.  NULL switches the probe off. */
+int oxq_set_gemv_phase_probe(void *d_buffer, size_t bytes);
 /* Which kernel instantiation and launch shape the calling thread's last GEMV / fused gate+up / tile-kernel
  * launch used, as "name<type,p0,p1,p2,p3> grid XxY block B" (template parameters in the kernel's own order):
  * lets a measurement name what it timed and notice when a launch policy has changed under it. */

@@ -184,6 +184,7 @@ TUNING_SIGNATURES = {
     "oxq_set_gemm_tile_min_rows": (C.c_int, [C.c_uint]),
     "oxq_set_ffn_fusion": (C.c_int, [C.c_int]),
     "oxq_last_launch": (C.c_int, [C.c_char_p, C.c_size_t]),
+    "oxq_set_gemv_phase_probe": (C.c_int, [C.c_void_p, C.c_size_t]),
 }
 
 _lib = None

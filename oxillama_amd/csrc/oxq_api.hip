@@ -264,6 +264,8 @@ int tensor_dims(uint32_t type, size_t data_len, const size_t *shape, size_t n_di
 
 namespace oxq {
 thread_local LaunchNote g_last_launch;
+std::atomic<uint64_t *> g_phase_buf{nullptr};
+std::atomic<size_t> g_phase_cap{0};
 uint32_t device_cus() { return g.cus ? g.cus : 256; }
 int set_error(int status, size_t a, size_t b, const char *msg) { return fail(status, a, b, msg); }
 int ensure_device() { return ensure_init(); }
@@ -457,6 +459,12 @@ int oxq_last_launch(char *out, size_t out_len) {
     const char *tn = oxq_type_name(n.type);
     std::snprintf(out, out_len, "%s<%s,%d,%d,%d,%d> grid %ux%u block %u", n.kernel, tn ? tn : "-", n.p[0], n.p[1], n.p[2],
                   n.p[3], n.grid_x, n.grid_y, n.block);
+    return OXQ_OK;
+}
+
+int oxq_set_gemv_phase_probe(void *d_buffer, size_t bytes) {
+    oxq::g_phase_cap.store(d_buffer ? bytes : 0, std::memory_order_relaxed);
+    oxq::g_phase_buf.store((uint64_t *)d_buffer, std::memory_order_relaxed);
     return OXQ_OK;
 }
 

@@ -68,7 +68,15 @@ __device__ __forceinline__ float reduce_batch(const Batch<F, STEPS, RB> &b, cons
     return res;
 }
 
-template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP>
+// PH (measurement only): every wave writes three timestamps of the 100 MHz wall clock to `phases` --
+// kernel entry, its first row batch stored, its last -- and where it ran (phase_where) at
+// [(blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave][4].
+// Where a wave runs: XCC_ID register in the high word, HW_ID (wave, SIMD, CU, shader array, shader engine) in the low.
+__device__ __forceinline__ uint64_t phase_where() {
+    const uint32_t hw = __builtin_amdgcn_s_getreg((31 << 11) | 4), xcc = __builtin_amdgcn_s_getreg((31 << 11) | 20);
+    return ((uint64_t)xcc << 32) | hw;
+}
+template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP, bool PH = false>
 __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict__ W0, const uint8_t *__restrict__ W1,
                                                      const uint8_t *__restrict__ W2, const uint8_t *__restrict__ W3,
                                                      float *__restrict__ out0, float *__restrict__ out1,
@@ -78,8 +86,10 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
                                                      const void *__restrict__ A, int32_t *__restrict__ sums,
                                                      uint32_t n_rows0, uint32_t n_rows1, uint32_t n_rows2,
                                                      uint32_t n_rows3, uint32_t units, uint32_t groups_per_row,
-                                                     size_t row_bytes, uint32_t n_cols) {
+                                                     size_t row_bytes, uint32_t n_cols, uint64_t *__restrict__ phases) {
     static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
+    uint64_t ph_t0 = 0, ph_t1 = 0;
+    if constexpr (PH) ph_t0 = wall_clock64();
     // Up to four matrices of one format and row length that share the activation vector (wq/wk/wv,
     // ffn_gate/ffn_up) ride in one launch: blockIdx.y picks the matrix, and each matrix gets
     // its own gridDim.x work groups (sized for the one with the most rows).  old = the vector a
@@ -135,6 +145,17 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
     }
 
     uint32_t trip = 0;
+    auto ph_done = [&]() {
+        if constexpr (PH) {
+            if (lane == 0) {
+                uint64_t *p = phases + ((size_t)(blockIdx.y * gridDim.x + blockIdx.x) * 4 + wave_in_wg) * 4;
+                p[0] = ph_t0;
+                p[1] = ph_t1;
+                p[2] = wall_clock64();
+                p[3] = phase_where();
+            }
+        }
+    };
     auto finish = [&](float res, float old, uint32_t batch) {
         const uint32_t row = batch * RB + lane;
         if (KS == 1) {
@@ -150,6 +171,9 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
             }
             trip++;
         }
+        if constexpr (PH) {
+            if (ph_t1 == 0) ph_t1 = wall_clock64();
+        }
     };
 
     // Each reduce_batch call site has a fixed set of loads in flight behind it, so the
@@ -161,6 +185,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
             const float r0 = reduce_batch<F, STEPS, RB, DUMP>(b0, act, sums, min(batch, n_batches - 1), n_rows, units,
                                                               unit0, groups_per_row, lane, k);
             finish(r0, b0.old, batch);
+            ph_done();
             break;
         }
         load_batch<F, STEPS, RB>(b1, W, old, min(next, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
@@ -172,6 +197,7 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
             const float r1 = reduce_batch<F, STEPS, RB, DUMP>(b1, act, sums, min(next, n_batches - 1), n_rows, units,
                                                               unit0, groups_per_row, lane, k);
             finish(r1, b1.old, next);
+            ph_done();
             break;
         }
         load_batch<F, STEPS, RB>(b0, W, old, min(next2, n_batches - 1), n_rows, row_bytes, units, unit0, lane, k, want_old);
@@ -189,13 +215,15 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
 // up (RB rows per batch, the next batch's loads in flight while one is reduced; one wave per row,
 // so the sums are those of gemv_q8_cached with KS = 1, bit for bit), the 64 sums meet in LDS and
 // eight lanes encode the block.  h_out (optional) receives h in fp32.
-template <class F, int STEPS, int RB, int WAVES>
+template <class F, int STEPS, int RB, int WAVES, bool PH = false>
 __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8_t *__restrict__ Wg,
                                                              const uint8_t *__restrict__ Wu,
                                                              const void *__restrict__ A, uint8_t *__restrict__ hq,
                                                              float *__restrict__ h_out, uint32_t n_rows, uint32_t units,
-                                                             size_t row_bytes) {
+                                                             size_t row_bytes, uint64_t *__restrict__ phases) {
     static_assert((RB == 1 || RB == 2) && (WAVES == 4 || WAVES == 8), "configuration");
+    uint64_t ph_t0 = 0, ph_t1 = 0;
+    if constexpr (PH) ph_t0 = wall_clock64();
     constexpr int RPW = 32 / WAVES;  // rows of each matrix per wave
     constexpr int NB = RPW / RB;     // batches per matrix and wave
     __shared__ float row_sums[2][32];
@@ -225,6 +253,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
         const float r = reduce_batch<F, STEPS, RB, false>(b[i % (AHEAD + 1)], act, nullptr, batch0 + i % NB, n_rows, units,
                                                           0, 0, lane, k);
         if (lane < RB) row_sums[i / NB][wave * RPW + (i % NB) * RB + lane] = r;
+        if constexpr (PH) {
+            if (i == 0) ph_t1 = wall_clock64();
+        }
+    }
+    if constexpr (PH) {
+        if (lane == 0) {  // the wave's rows are summed: what follows is the block's SwiGLU and encode
+            uint64_t *p = phases + ((size_t)blockIdx.x * WAVES + wave) * 4;
+            p[0] = ph_t0;
+            p[1] = ph_t1;
+            p[2] = wall_clock64();
+            p[3] = phase_where();
+        }
     }
     __syncthreads();
     if (wave != 0) return;

@@ -12,6 +12,12 @@ template <class F, class = void> struct format_waves_per_cu { static constexpr u
 template <class F> struct format_waves_per_cu<F, std::void_t<decltype(F::WAVES_PER_CU)>> {
     static constexpr uint32_t value = F::WAVES_PER_CU;
 };
+// Formats whose GEMV kernels also exist in the timestamping instantiation (the BASELINE decode shapes).
+template <class F> struct phase_probe_format {
+    static constexpr bool value = F::TYPE_ID == OXQ_TYPE_Q4_K || F::TYPE_ID == OXQ_TYPE_Q6_K || F::TYPE_ID == OXQ_TYPE_Q8_0 ||
+                                  F::TYPE_ID == OXQ_TYPE_Q4_0;
+};
+
 template <class F>
 static uint32_t launch_width(const GemvArgs &a) {
     return a.waves_per_cu ? a.waves_per_cu : format_waves_per_cu<F>::value;
@@ -48,13 +54,24 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
     const void *acts = a.X ? static_cast<const void *>(a.X) : static_cast<const void *>(a.A);
+    if constexpr (phase_probe_format<F>::value && std::is_same<SRC, ActQ8>::value && !DUMP && STEPS <= 2) {
+        // measurement: the same kernel with three timestamps per wave (oxq_set_gemv_phase_probe)
+        uint64_t *ph = g_phase_buf.load(std::memory_order_relaxed);
+        if (ph && (size_t)blocks * n_mats * 4 * 4 * 8 <= g_phase_cap.load(std::memory_order_relaxed)) {
+            hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP, true>), dim3(blocks, n_mats), dim3(256), 0, stream,
+                               w[0], w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums,
+                               rows[0], rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols, ph);
+            note_launch("gemv_q8_cached_phases", F::TYPE_ID, STEPS, RB, KS, DUMP, blocks, n_mats, 256);
+            return hipGetLastError();
+        }
+    }
     // fp32 source: LDS for the quantized vector (32 payload bytes + one f16 scale per block)
     const size_t lds = std::is_same<SRC, ActF32>::value ? (size_t)units * (F::UNIT_COLS / 32) * 34 : 0;
     note_launch(std::is_same<SRC, ActF32>::value ? "gemv_q8_cached_f32" : "gemv_q8_cached", F::TYPE_ID, STEPS, RB, KS, DUMP,
                 blocks, n_mats, 256);
     hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), lds, stream, w[0],
                        w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums, rows[0],
-                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols);
+                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols, (uint64_t *)nullptr);
     return hipGetLastError();
 }
 
@@ -144,10 +161,22 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
     if (steps > 2 || n_rows % 32 != 0 || n_rows == 0) return hipErrorNotSupported;
     const bool two = row_bytes <= F::TWO_ROW_BATCH_BYTES;
     const dim3 grid(n_rows / 32);
+    uint64_t *ph = nullptr;
+    if constexpr (phase_probe_format<F>::value) {
+        ph = g_phase_buf.load(std::memory_order_relaxed);
+        if (ph && (size_t)grid.x * 8 * 4 * 8 > g_phase_cap.load(std::memory_order_relaxed)) ph = nullptr;
+    }
 #define OXQ_LAUNCH(ST, RBV)                                                                                          \
     note_launch("gemv_q8_gate_up_swiglu", F::TYPE_ID, ST, RBV, 4, 0, grid.x, 1, 256);                                \
+    if constexpr (phase_probe_format<F>::value) {                                                                    \
+        if (ph) {                                                                                                    \
+            hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4, true>), grid, dim3(256), 0, stream, Wg, Wu,    \
+                               acts, hq, h, n_rows, units, row_bytes, ph);                                           \
+            return hipGetLastError();                                                                                \
+        }                                                                                                            \
+    }                                                                                                                \
     hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4>), grid, dim3(256), 0, stream, Wg, Wu, acts, hq, h,     \
-                       n_rows, units, row_bytes)
+                       n_rows, units, row_bytes, (uint64_t *)nullptr)
     if (steps == 1) {
         if (two) { OXQ_LAUNCH(1, 2); } else { OXQ_LAUNCH(1, 1); }
     } else {

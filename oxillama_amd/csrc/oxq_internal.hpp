@@ -60,6 +60,10 @@ inline void note_launch(const char *kernel, uint32_t type, int p0, int p1, int p
     g_last_launch = LaunchNote{kernel, type, {p0, p1, p2, p3}, gx, gy, block};
 }
 
+// Measurement: device buffer (and its size in bytes) that the timestamping GEMV instantiations write to; null = off.
+extern std::atomic<uint64_t *> g_phase_buf;
+extern std::atomic<size_t> g_phase_cap;
+
 // Number of compute units of the current device (cached per device).
 uint32_t device_cus();
 
