@@ -477,6 +477,23 @@ def main():
         k_q40 = quant.HipKernel(Q4_0)
         c1 = [upload(Q4_0, 5000 + i, H, H) for i in range(64)]
         kernels["c1_q4_0_4096x4096"] = time_kernel(k_q40, Q4_0, c1, xq, yq, H, H)
+        # QuantKernel::gemv with the reference's own numerics (fp32 activations, oxq_gemv_f32_dev), same shapes
+        def time_f32(kern, t, mats, xv, out, n_rows, n_cols):
+            n = max(len(mats), 32)
+
+            def body():
+                for i in range(n):
+                    kern.gemv_f32_dev(mats[i % len(mats)], xv, out, n_rows, n_cols)
+            g = capture(body)
+            timed_replay(g)
+            us = min(timed_replay(g) for _ in range(3)) * 1e3 / n
+            wb = n_rows * row_bytes(t, n_cols)
+            return {"us_per_call": round(us, 3), "launches": n, "distinct_weight_sets": len(mats),
+                    "weight_GBps": round(wb / us / 1e3, 1), "frac_hbm_peak": round((wb + 4 * n_cols + 4 * n_rows) / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        kernels["f32_route_q4k_gate_14336x4096"] = time_f32(k_q4k, Q4_K, [w["gate"] for w in layers], x, yg, F, H)
+        kernels["f32_route_q6k_down_4096x14336"] = time_f32(k_q6k, Q6_K, [w["down"] for w in layers], h, yd, H, F)
+        kernels["f32_route_q8_0_q_proj_4096x4096"] = time_f32(k_q8, Q8_0, [w["q"] for w in layers], x, yq, H, H)
+        kernels["f32_route_c1_q4_0_4096x4096"] = time_f32(k_q40, Q4_0, c1, x, yq, H, H)
         del c1
         V = 128256
         lm = [upload(Q6_K, 6000 + i, V, H) for i in range(2)]

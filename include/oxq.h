@@ -236,6 +236,31 @@ int oxq_gemv_multi_dev(uint32_t type, size_t n_mats, const uint8_t *const *d_wei
                        const float *d_x, float *const *d_outs, size_t n_rows, size_t n_cols,
                        int accumulate, void *stream);
 
+/* QuantKernel::gemv with the reference's own numerics (Q/traits.rs:39-44; rows: Q/reference/q4_0.rs:82-102,
+ * q8_0.rs:77-92, q4_k.rs:135-178, q6_k.rs:108-166, iq4_xs.rs:130-163; what QuantLinear::forward calls,
+ * crates/oxillama-arch/src/common/linear.rs:77-98): the fp32 activations are NOT quantized; every weight is
+ * dequantized in registers and every term is formed by the reference's scalar expression, in its column order
+ * inside a block; the reference's running sum over the row becomes a tree over lanes and waves, which moves the
+ * result by rounding only (within 1e-5 of |y|inf of the reference gemv).  d_out[r] = W[r,:] . x (+ d_bias[r] when
+ * d_bias is given; + d_out[r] when accumulate is set; not both).  n_cols need not be a block multiple (columns
+ * past it are skipped, as in the reference).  Formats: Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS; others return
+ * OXQ_ERR_UNSUPPORTED_TYPE.  About twice the time of the Q8_0-activation route at decode shapes. */
+int oxq_gemv_f32_dev(uint32_t type, const uint8_t *d_weights, const float *d_x, const float *d_bias,
+                     float *d_out, size_t n_rows, size_t n_cols, int accumulate, void *stream);
+
+/* Which arithmetic the entry points that take fp32 input and mirror QuantKernel::gemv / gemm and
+ * QuantLinear::forward / forward_batch use (oxq_gemv, oxq_gemm, oxq_linear_forward, oxq_linear_forward_batch,
+ * and oxq_linear_forward_dev when it is given no Q8_0 activations):
+ *   OXQ_ROUTE_Q8  (default) x is quantized to Q8_0 and the fused kernels run -- the reference's
+ *                 matvec_q8_fused arithmetic, the fast route;
+ *   OXQ_ROUTE_F32 the reference's gemv arithmetic (oxq_gemv_f32_dev); formats without such a kernel
+ *                 then return OXQ_ERR_UNSUPPORTED_TYPE instead of changing arithmetic silently.
+ * Process-wide, atomic; takes effect for calls that start afterwards. */
+#define OXQ_ROUTE_Q8 0
+#define OXQ_ROUTE_F32 1
+int oxq_select_activation_route(int route);
+int oxq_activation_route(void);
+
 /* Prefill / decode batch: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched
  * form of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  From 6 rows up
  * (9 where n < 8192), with k a multiple of 256, every format but Q2_K / Q3_K runs on the int8-MFMA tile

@@ -114,6 +114,10 @@ SIGNATURES = {
                                                 C.POINTER(C.c_void_p), C.c_size_t, C.c_size_t, C.c_int, C.c_void_p]),
     "oxq_gemv_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int,
                                C.c_void_p]),
+    "oxq_gemv_f32_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t,
+                                   C.c_int, C.c_void_p]),
+    "oxq_select_activation_route": (C.c_int, [C.c_int]),
+    "oxq_activation_route": (C.c_int, []),
     "oxq_gemv_multi_dev": (C.c_int, [C.c_uint32, C.c_size_t, C.POINTER(C.c_void_p), C.c_void_p,
                                      C.POINTER(C.c_void_p), C.c_size_t, C.c_size_t, C.c_int, C.c_void_p]),
     "oxq_gemm_q8_workspace_bytes": (C.c_size_t, [C.c_uint32, C.c_size_t, C.c_size_t, C.c_size_t]),

@@ -102,6 +102,7 @@ struct State {
     std::atomic<uint32_t> waves_per_cu{0};    // 0 = default
     std::atomic<uint32_t> rows_per_batch{0};  // 0 = chosen per shape
     std::atomic<uint32_t> waves_per_row{0};   // 0 = chosen per shape
+    std::atomic<int> act_route{OXQ_ROUTE_Q8};  // how the fp32-input entry points treat their activations
     int cache_mode = 0;  // 0 off, 1 on (sampled fingerprint), 2 on and verified (every byte hashed on every call)
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
     size_t cache_bytes = 0, cache_limit = (size_t)16 << 30;
@@ -640,6 +641,25 @@ static int gemm_host(uint32_t type, const uint8_t *data, size_t data_len, const 
     if (k_pad != n_cols) OXQ_HIP(hipMemset(g.s_x.ptr, 0, m * k_pad * sizeof(float)));
     OXQ_HIP(hipMemcpy2D(g.s_x.ptr, k_pad * sizeof(float), input, k * sizeof(float), n_cols * sizeof(float), m,
                         hipMemcpyHostToDevice));
+    const float *d_bias_f32 = nullptr;
+    if (g.act_route.load(std::memory_order_relaxed) == OXQ_ROUTE_F32) {
+        // the reference's own gemm: m gemvs on the fp32 rows (reference/q4_k.rs:186-201), bias per row (linear.rs:123-128)
+        if (!oxq::gemv_f32_supported(type))
+            return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "no fp32-activation kernel for this type (OXQ_ROUTE_F32)");
+        if (bias && bias_len) {
+            if ((st = g.s_bias.reserve(n_rows * sizeof(float))) != OXQ_OK) return st;
+            const size_t nb = bias_len < n_rows ? bias_len : n_rows;
+            OXQ_HIP(hipMemset(g.s_bias.ptr, 0, n_rows * sizeof(float)));
+            OXQ_HIP(hipMemcpy(g.s_bias.ptr, bias, nb * sizeof(float), hipMemcpyHostToDevice));
+            d_bias_f32 = (const float *)g.s_bias.ptr;
+        }
+        for (size_t r = 0; r < m; r++)
+            OXQ_HIP(oxq::launch_gemv_f32(type, dW, (const float *)g.s_x.ptr + r * k_pad, (float *)g.s_out.ptr + r * n_rows,
+                                         d_bias_f32, (uint32_t)n_rows, (uint32_t)n_cols, nullptr));
+        OXQ_HIP(hipMemcpy2D(output, n * sizeof(float), g.s_out.ptr, n_rows * sizeof(float), n_rows * sizeof(float), m,
+                            hipMemcpyDeviceToHost));
+        return OXQ_OK;
+    }
     OXQ_HIP(oxq::launch_quantize_q8_0((const float *)g.s_x.ptr, m * k_pad, (uint8_t *)g.s_acts.ptr, nullptr));
     oxq::GemmArgs ga;
     ga.W = dW;
@@ -808,6 +828,27 @@ int oxq_gemv_dev(uint32_t type, const uint8_t *d_weights, const float *d_x, floa
                  size_t n_cols, int accumulate, void *stream) {
     return oxq_gemv_multi_dev(type, 1, &d_weights, d_x, &d_out, n_rows, n_cols, accumulate, stream);
 }
+
+int oxq_gemv_f32_dev(uint32_t type, const uint8_t *d_weights, const float *d_x, const float *d_bias, float *d_out,
+                     size_t n_rows, size_t n_cols, int accumulate, void *stream) {
+    int st = check_dev_shape(type, n_rows, n_cols, true);
+    if (st != OXQ_OK) return st;
+    if (!oxq::gemv_f32_supported(type))
+        return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "no fp32-activation kernel for this type");
+    if (accumulate && d_bias) return fail(OXQ_ERR_INTERNAL, 0, 0, "accumulate and bias exclude each other");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_gemv_f32(type, d_weights, d_x, d_out, accumulate ? d_out : d_bias, (uint32_t)n_rows,
+                                 (uint32_t)n_cols, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
+int oxq_select_activation_route(int route) {
+    if (route != OXQ_ROUTE_Q8 && route != OXQ_ROUTE_F32) return fail(OXQ_ERR_INTERNAL, 0, (size_t)route, "unknown route");
+    g.act_route.store(route, std::memory_order_relaxed);
+    return OXQ_OK;
+}
+
+int oxq_activation_route(void) { return g.act_route.load(std::memory_order_relaxed); }
 
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, int32_t *d_sums,
                        size_t n_rows, size_t n_cols, void *stream) {
@@ -1019,6 +1060,16 @@ int oxq_linear_forward_dev(uint32_t type, const uint8_t *d_weights, const float 
     const bool has_lora = lora && lora->rank;
     if (!d_acts_q8 && !d_x) return fail(OXQ_ERR_INTERNAL, 0, 0, "neither fp32 nor Q8_0 activations given");
     if (has_lora && !d_x) return fail(OXQ_ERR_INTERNAL, 0, 0, "LoRA needs the fp32 input");
+    if (!d_acts_q8 && g.act_route.load(std::memory_order_relaxed) == OXQ_ROUTE_F32) {
+        // QuantLinear::forward as the reference computes it: gemv on the fp32 input, then bias, then LoRA
+        if (!oxq::gemv_f32_supported(type))
+            return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "no fp32-activation kernel for this type (OXQ_ROUTE_F32)");
+        if ((st = ensure_init()) != OXQ_OK) return st;
+        OXQ_HIP(oxq::launch_gemv_f32(type, d_weights, d_x, d_out, d_bias, (uint32_t)out_features, (uint32_t)in_features,
+                                     (hipStream_t)stream));
+        if (has_lora) return oxq_lora_apply_dev(lora, d_x, d_out, out_features, in_features, stream);
+        return OXQ_OK;
+    }
     if (!d_acts_q8 && !oxq::gemv_takes_f32(type, (uint32_t)in_features))
         return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, in_features, "row too long for in-kernel activation quantization");
     if ((st = ensure_init()) != OXQ_OK) return st;
@@ -1424,9 +1475,16 @@ int oxq_linear_forward(uint32_t type, const uint8_t *data, size_t data_len, cons
         OXQ_HIP(hipMemcpy(g.s_bias.ptr, bias, nb * sizeof(float), hipMemcpyHostToDevice));
         d_bias = (const float *)g.s_bias.ptr;
     }
-    oxq::GemvArgs a = gemv_args(dW, (const uint8_t *)g.s_acts.ptr, (float *)g.s_out.ptr, nullptr, n_rows, n_cols, 0);
-    a.bias = d_bias;
-    OXQ_HIP(oxq::launch_gemv_q8(type, a, nullptr));
+    if (g.act_route.load(std::memory_order_relaxed) == OXQ_ROUTE_F32) {
+        if (!oxq::gemv_f32_supported(type))
+            return fail(OXQ_ERR_UNSUPPORTED_TYPE, type, 0, "no fp32-activation kernel for this type (OXQ_ROUTE_F32)");
+        OXQ_HIP(oxq::launch_gemv_f32(type, dW, (const float *)g.s_x.ptr, (float *)g.s_out.ptr, d_bias, (uint32_t)n_rows,
+                                     (uint32_t)n_cols, nullptr));
+    } else {
+        oxq::GemvArgs a = gemv_args(dW, (const uint8_t *)g.s_acts.ptr, (float *)g.s_out.ptr, nullptr, n_rows, n_cols, 0);
+        a.bias = d_bias;
+        OXQ_HIP(oxq::launch_gemv_q8(type, a, nullptr));
+    }
     if (has_lora) {
         if ((st = g.s_lora_a.reserve(lora_a_len * sizeof(float))) != OXQ_OK) return st;
         if ((st = g.s_lora_b.reserve(lora_b_len * sizeof(float))) != OXQ_OK) return st;

@@ -68,6 +68,11 @@ extern std::atomic<size_t> g_phase_cap;
 uint32_t device_cus();
 
 hipError_t launch_gemv_q8(uint32_t type, const GemvArgs &a, hipStream_t stream);
+// QuantKernel::gemv as the reference computes it (fp32 activations, weights dequantized in registers):
+// out[r] = (old ? old[r] : 0) + W[r, :] . x.  hipErrorNotSupported: no such kernel for this format.
+hipError_t launch_gemv_f32(uint32_t type, const uint8_t *W, const float *x, float *out, const float *old,
+                           uint32_t n_rows, uint32_t n_cols, hipStream_t stream);
+bool gemv_f32_supported(uint32_t type);
 // True when the GEMV of this row length can quantize fp32 activations itself (GemvArgs::X).
 bool gemv_takes_f32(uint32_t type, uint32_t n_cols);
 

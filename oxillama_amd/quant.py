@@ -257,6 +257,13 @@ class HipKernel:
         _check(self._lib.oxq_gemv_dev(self.tensor_type, d_weights.data_ptr(), d_x.data_ptr(), d_out.data_ptr(),
                                       n_rows, n_cols, int(accumulate), self._stream()))
 
+    def gemv_f32_dev(self, d_weights, d_x, d_out, n_rows, n_cols, accumulate=False, d_bias=None):
+        """QuantKernel::gemv with the reference's numerics: fp32 activations against weights dequantized in
+        registers (oxq_gemv_f32_dev)."""
+        _check(self._lib.oxq_gemv_f32_dev(self.tensor_type, d_weights.data_ptr(), d_x.data_ptr(),
+                                          d_bias.data_ptr() if d_bias is not None else None, d_out.data_ptr(),
+                                          n_rows, n_cols, int(accumulate), self._stream()))
+
     def gemv_multi_dev(self, d_weights, d_x, d_outs, n_rows, n_cols, accumulate=False):
         import ctypes as C
         n = len(d_weights)
@@ -315,6 +322,20 @@ class KernelDispatcher:
 
     def get_kernel(self, tensor_type):
         return HipKernel(tensor_type)
+
+
+ROUTE_Q8, ROUTE_F32 = 0, 1
+
+
+def select_activation_route(route):
+    """How the fp32-input entry points (gemv, gemm, QuantLinear forward on host slices, linear forward on device
+    without Q8_0 activations) treat their input: ROUTE_Q8 quantizes it to Q8_0 (the fused kernels), ROUTE_F32 runs
+    the reference's gemv arithmetic (oxq_select_activation_route)."""
+    _check(capi.load().oxq_select_activation_route(int(route)))
+
+
+def activation_route():
+    return capi.load().oxq_activation_route()
 
 
 def init(device=0):
