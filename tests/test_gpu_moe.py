@@ -175,6 +175,7 @@ def test_moe_ffn_layer(hip, ref, types, shape):
     q8, gh, uh, hqh, yh = host(d_q8), host(g), host(u), host(hq), host(y).reshape(pairs, hidden)
     a_row, h_row = hidden // 32 * 34, inter // 32 * 34
     sample = sorted(set([0, n_tok - 1, n_tok // 2] + list(range(0, n_tok, 17))))
+    flipped_h = bytes_h = flipped_chain = scales_chain = 0
     for t in sample:
         xt = x[t * hidden:(t + 1) * hidden]
         sel, wt = ref.moe_route(router, n_exp, hidden, top_k, xt)
@@ -190,8 +191,25 @@ def test_moe_ffn_layer(hip, ref, types, shape):
             assert_close(uh[r * inter:(r + 1) * inter], u_ref, f"up t{t} e{e}")
             hq_ref = ref.quantize_q8_0(ref.swiglu(gh[r * inter:(r + 1) * inter], uh[r * inter:(r + 1) * inter]))
             mine = hqh[r * h_row:(r + 1) * h_row]
-            bad = int(np.sum(mine != hq_ref))  # device expf vs libm: a rounding boundary crossed now and then
-            assert bad <= max(2, mine.size // 200), f"h bytes t{t} e{e}: {bad} of {mine.size} differ"
+            # device expf vs libm: h differs in the last place now and then, and a few of those differences cross a
+            # rounding boundary of the Q8_0 encoder -- one step of one weight each, never a scale
+            mb, rb_ = mine.reshape(-1, 34), hq_ref.reshape(-1, 34)
+            assert np.array_equal(mb[:, :2], rb_[:, :2]), f"h scales t{t} e{e}"
+            step = mb[:, 2:].view(np.int8).astype(np.int32) - rb_[:, 2:].view(np.int8).astype(np.int32)
+            assert np.abs(step).max() <= 1, f"h bytes t{t} e{e}: a byte moved by more than one step"
+            flipped_h += int(np.count_nonzero(step))
+            bytes_h += mine.size
+            # against the oracle's own chain (its gate / up, within 1e-5 of the device's, then libm): the same kind
+            # of difference, counted over everything that feeds the down projection
+            chain = ref.quantize_q8_0(ref.swiglu(g_ref, u_ref)).reshape(-1, 34)
+            chain_step = mb[:, 2:].view(np.int8).astype(np.int32) - chain[:, 2:].view(np.int8).astype(np.int32)
+            d_mine = mb[:, :2].copy().view(np.uint16).astype(np.int32).ravel()
+            d_chain = chain[:, :2].copy().view(np.uint16).astype(np.int32).ravel()
+            assert np.abs(d_mine - d_chain).max() <= 1, "a block scale of h moved by more than one f16 step"
+            same_scale = d_mine == d_chain
+            assert np.abs(chain_step[same_scale]).max(initial=0) <= 1
+            flipped_chain += int(np.count_nonzero(chain_step[same_scale]))
+            scales_chain += int(np.count_nonzero(~same_scale))
             e_ref = ref.matvec_q8_fused(td, wd[e * sd:(e + 1) * sd], mine, hidden, inter)
             assert_close(yh[r], e_ref, f"down t{t} e{e}")
             ref.load().oxq_ref_moe_accumulate(O._p(acc), O._p(np.ascontiguousarray(yh[r])), float(weights[t, j]),
@@ -202,6 +220,12 @@ def test_moe_ffn_layer(hip, ref, types, shape):
             if tg == tu == td else (None, None, None)
         if want is not None:
             assert_close(got[t], want, f"end to end t{t}", tol=2e-3)
+    # the flipped bytes are what separates the 2e-3 end-to-end bar from the 1e-5 per-stage bar: far below 0.1 % of h
+    say(f"h bytes one step off the oracle's: {flipped_h} of {bytes_h} (same gate/up); oracle's gate/up: {flipped_chain} bytes, "
+        f"{scales_chain} of {bytes_h // 34} block scales one f16 step off")
+    assert flipped_h <= max(1, bytes_h // 1000), f"{flipped_h} of {bytes_h} Q8_0 bytes of h differ"
+    assert flipped_chain <= max(2, bytes_h // 1000), f"{flipped_chain} of {bytes_h} Q8_0 bytes of h differ from the oracle's chain"
+    assert scales_chain <= max(2, bytes_h // 34 // 100), f"{scales_chain} of {bytes_h // 34} block scales of h differ"
 
 
 def test_moe_ffn_with_host_tables_and_errors(hip, ref):

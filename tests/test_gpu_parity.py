@@ -594,7 +594,8 @@ def _prefill_tile_case(hip, ref, shape, t):
 
 
 def test_prefill_full_size_c4(hip, ref):
-    """C4: 512 tokens x Q4_K 14336 x 4096.  Oracle on every 16th token (all 14336 outputs each)."""
+    """C4: 512 tokens x Q4_K 14336 x 4096.  Oracle on every 16th token (all 14336 outputs each), on all tokens for two
+    512-row slabs of W, and bit-exact integer sums on those slabs."""
     import torch
     m, n, k_, t = 512, 14336, 4096, O.Q4_K
     w = synth.weights(t, 31, n, k_)
@@ -612,9 +613,27 @@ def test_prefill_full_size_c4(hip, ref):
     rows = list(range(0, m, 16)) + [m - 1]
     y_ref = _oracle_prefill(ref, t, w, acts, m, n, k_, rows=rows)
     assert_close(dy.cpu().numpy()[rows], y_ref, "C4 prefill")
+    # two 512-row slabs of W (one that straddles tile boundaries in the middle, and the last rows): the oracle
+    # on ALL 512 tokens, and the exact integer sums of every (token, weight row, 32-weight group) of the slab
+    arb, rb = k_ // 32 * 34, O.row_bytes(t, k_)
+    for r0 in (4000, n - 512):
+        w_slab = w[r0 * rb:(r0 + 512) * rb]
+        y_slab = _oracle_prefill(ref, t, w_slab, acts, m, 512, k_)
+        assert_close(dy[:, r0:r0 + 512].cpu().numpy(), y_slab, f"C4 prefill, rows {r0}..{r0 + 511}, all tokens")
+        dw_slab = dw[r0 * rb:(r0 + 512) * rb]
+        dsum = torch.empty((m, 512, k_ // 32), dtype=torch.int32, device="cuda")
+        dy_slab = torch.empty((m, 512), dtype=torch.float32, device="cuda")
+        ws_slab = torch.empty(kern.gemm_workspace_bytes(m, 512, k_), dtype=torch.uint8, device="cuda")
+        kern.gemm_block_sums_dev(dw_slab, da, dy_slab, dsum, m, 512, k_, workspace=ws_slab)
+        torch.cuda.synchronize()
+        got = dsum.cpu().numpy()
+        for r in range(m):
+            assert np.array_equal(got[r], ref.block_sums(t, w_slab, acts[r * arb:(r + 1) * arb], 512, k_)), (r0, r)
+        # the slab on its own goes through the same tile arithmetic as inside the full matrix
+        assert_close(dy_slab.cpu().numpy(), y_slab, f"C4 slab launch, rows {r0}")
+        del dsum, got
     # every token row also equals the batch-1 fused matvec of the same activations, to fp32 order
     yv = torch.zeros(n, dtype=torch.float32, device="cuda")
-    arb = k_ // 32 * 34
     for r in (1, 255, 510):
         yv.zero_()
         kern.matvec_q8_fused_dev(dw, da[r * arb:(r + 1) * arb], yv, n, k_, accumulate=False)
