@@ -800,7 +800,14 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
         // tokens the four waves of a work group share one tile and split k (most work groups, shortest
         // dependency chain per wave); up to 384 tokens 64 x 128 tiles; beyond that 128 x 64 tiles at
         // three waves per SIMD.
-        if (rows > 384) return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
+        if (rows > 384) {
+            // 128 x 128 tiles (two waves per SIMD, weight bytes fetched two steps ahead) where they still give the
+            // chip one and a half work groups per compute unit: 14336 x 4096, 512 tokens 123 us against 125 us,
+            // 2048 tokens 383 us against 422 us; 4096 x 14336 has too few such tiles (214 us against 140 us)
+            const size_t wgs = (size_t)((rows + 127) / 128) * ((a.n + 127) / 128) * (a.offsets ? a.n_experts : 1);
+            if (2 * wgs >= 3 * (size_t)device_cus()) return launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
+            return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
+        }
         if (rows > 64) return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
         // split k; 64 weight rows (or 64 tokens) per work group only where that still leaves every
         // compute unit at least one work group, else 32 x 32
