@@ -75,10 +75,218 @@ __global__ __launch_bounds__(64) void topk_merge_kernel(const uint64_t *__restri
     }
 }
 
+// ---- larger k: one work group, a filter by group maxima, then a radix select in LDS -----------------------
+// 1. Every thread takes the maximum of its share of the keys (no atomics).  The k-th largest of these 1024
+//    maxima, T1, is a lower bound of the k-th largest key overall: k different threads each hold a key >= T1.
+// 2. A second pass copies every key >= T1 to LDS.  For logits that is barely more than k keys (k = 256 of
+//    128256: about 300); at most SEL_CAP fit.
+// 3. The k-th largest of the survivors, T, is found digit by digit from the top (8-bit digits: histogram of the
+//    digit over the keys that match the digits found so far, suffix scan from the top bin; the bin in which the
+//    count crosses what is still wanted is T's next digit), until the keys at or above the prefix are exactly k.
+//    They are ranked among themselves by counting and written in order.
+// If step 2 overflows (the large values all sit in a few threads' shares, which takes an adversarial layout) the
+// same digit search runs over the keys in memory with 12-bit digits instead: exact as well, several passes slower.
+// Keys are unique (they carry the index), so every count is exact and ties come out lower index first, as in
+// the two-stage kernels above.
+constexpr uint32_t SEL_CAP = 8192, SEL_THREADS = 1024;
+
+// Suffix scan over the bins from the top: the digit d with count(bins > d) < want <= count(bins >= d), and
+// those two counts.  All threads call; nb <= 4 * SEL_THREADS bins; result broadcast through `res`.
+__device__ __forceinline__ void select_digit(const uint32_t *hist, uint32_t nb, uint32_t want, uint32_t *wave_tot,
+                                             uint32_t *res, uint32_t &digit, uint32_t &above, uint32_t &equal) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint32_t p = 0;
+    if (4 * tid < nb) p = hist[4 * tid] + hist[4 * tid + 1] + hist[4 * tid + 2] + hist[4 * tid + 3];
+    uint32_t v = p;  // sum over the lanes at or above this one
+    for (uint32_t off = 1; off < 64; off <<= 1) {
+        const uint32_t y = __shfl_down(v, off, 64);
+        if (lane + off < 64) v += y;
+    }
+    if (lane == 0) wave_tot[wave] = v;
+    __syncthreads();
+    uint32_t higher = 0;
+    for (uint32_t w = wave + 1; w < SEL_THREADS / 64; w++) higher += wave_tot[w];
+    const uint32_t incl = v + higher, excl = incl - p;
+    if (excl < want && incl >= want) {  // exactly one thread: the crossing is inside its four bins
+        uint32_t run = excl;
+        for (int b = 3; b >= 0; b--) {
+            const uint32_t c = hist[4 * tid + b];
+            if (run + c >= want) {
+                res[0] = 4 * tid + b;
+                res[1] = run;
+                res[2] = c;
+                break;
+            }
+            run += c;
+        }
+    }
+    __syncthreads();
+    digit = res[0];
+    above = res[1];
+    equal = res[2];
+    __syncthreads();  // res and wave_tot may be rewritten by the next call
+}
+
+// One count for the bin of `d`; lanes of a wave that share the first active lane's bin go in as one addition
+// (same-address LDS atomics serialise, and masked logits put tens of thousands of -inf into one bin).
+__device__ __forceinline__ void hist_add(uint32_t *hist, uint32_t d, bool valid) {
+    const uint64_t active = __ballot(valid);
+    if (active == 0) return;
+    const uint32_t leader = (uint32_t)__builtin_ctzll(active);
+    const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)d, (int)leader);
+    const uint64_t same = __ballot(valid && d == d0);
+    if (__builtin_popcountll(same) >= 8) {
+        if ((threadIdx.x & 63) == leader) atomicAdd(&hist[d0], (uint32_t)__builtin_popcountll(same));
+        if (valid && d != d0) atomicAdd(&hist[d], 1u);
+    } else if (valid) {
+        atomicAdd(&hist[d], 1u);
+    }
+}
+
+struct SelectShared {
+    uint32_t hist[4096];
+    uint32_t wave_tot[SEL_THREADS / 64], res[3], counter;
+};
+
+// The smallest threshold t (low bits zero) such that exactly `want` of the keys `each` visits are >= t, found
+// W bits at a time from the top.  `each(fn)` calls fn(key, valid) for every key, the same number of times in every
+// thread of a wave; all threads of the work group call this function.
+template <int W, class Each>
+__device__ __forceinline__ uint64_t kth_threshold(Each &&each, uint32_t want, SelectShared &sh) {
+    const uint32_t tid = threadIdx.x;
+    uint64_t prefix = 0;  // the digits found so far
+    uint32_t done = 0;    // how many bits that is
+    while (true) {
+        const uint32_t w = min((uint32_t)W, 64u - done), nb = 1u << w;
+        for (uint32_t b = tid; b < (nb < 4 ? 4 : nb); b += SEL_THREADS) sh.hist[b] = 0;
+        __syncthreads();
+        const uint32_t shift = 64 - done - w;
+        each([&](uint64_t key, bool valid) {
+            const bool match = valid && (done == 0 || (key >> (64 - done)) == prefix);
+            hist_add(sh.hist, (uint32_t)(key >> shift) & (nb - 1), match);
+        });
+        __syncthreads();
+        uint32_t digit, above, equal;
+        select_digit(sh.hist, nb, want, sh.wave_tot, sh.res, digit, above, equal);
+        prefix = (prefix << w) | digit;
+        done += w;
+        want -= above;  // the threshold is the want-th largest of the keys that match the prefix
+        if (equal == want || done == 64) return done == 64 ? prefix : prefix << (64 - done);
+    }
+}
+
+__global__ __launch_bounds__(SEL_THREADS) void topk_select_kernel(const float *__restrict__ x, uint32_t n, uint32_t k,
+                                                                 float *__restrict__ out_vals,
+                                                                 uint32_t *__restrict__ out_idx) {
+    __shared__ SelectShared sh;
+    __shared__ uint64_t cand[SEL_CAP];
+    __shared__ uint64_t sel[256];
+    const uint32_t tid = threadIdx.x;
+    const bool vec4 = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    // every key of the vector: 16-byte loads, four in flight per thread (16 keys per thread and trip), when the
+    // vector starts on a 16-byte boundary
+    auto each_in_memory = [&](auto &&fn) {
+        if (vec4) {
+            for (uint32_t i0 = 0; i0 < n; i0 += 16 * SEL_THREADS) {
+                u32x4 v[4];
+                uint32_t idx[4];
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    idx[u] = i0 + 4 * (u * SEL_THREADS + tid);
+                    v[u] = idx[u] + 4 <= n ? *reinterpret_cast<const u32x4 *>(x + idx[u]) : u32x4{0, 0, 0, 0};
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t bits = v[u][e];
+                        fn(topk_key(__builtin_bit_cast(float, bits), idx[u] + e), idx[u] + 4 <= n);
+                    }
+            }
+            if ((n & 3u) && tid < 64) {  // the last n % 4 keys, by the first wave
+                const uint32_t i = (n & ~3u) + tid;
+                fn(i < n ? topk_key(x[i], i) : 0, i < n);
+            }
+            return;
+        }
+        for (uint32_t i0 = 0; i0 < n; i0 += 4 * SEL_THREADS) {
+            float v[4];
+            uint32_t idx[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                idx[u] = i0 + u * SEL_THREADS + tid;
+                v[u] = idx[u] < n ? x[idx[u]] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) fn(topk_key(v[u], idx[u]), idx[u] < n);
+        }
+    };
+    uint32_t n_cand = 0;
+    auto each_in_lds = [&](auto &&fn) {
+        for (uint32_t j0 = 0; j0 < n_cand; j0 += SEL_THREADS) {
+            const uint32_t j = j0 + tid;
+            fn(j < n_cand ? cand[j] : 0, j < n_cand);
+        }
+    };
+    // 1. the k-th largest of the threads' maxima
+    uint64_t best = 0;
+    each_in_memory([&](uint64_t key, bool valid) { best = valid ? max_u64(best, key) : best; });
+    cand[tid] = best;  // a thread without keys holds 0, which is below every key
+    n_cand = SEL_THREADS;
+    __syncthreads();
+    const uint64_t t1 = kth_threshold<8>(each_in_lds, k, sh);
+    // 2. the keys at or above it, to LDS
+    if (tid == 0) sh.counter = 0;
+    __syncthreads();
+    each_in_memory([&](uint64_t key, bool valid) {
+        if (valid && key >= t1) {
+            const uint32_t pos = atomicAdd(&sh.counter, 1u);
+            if (pos < SEL_CAP) cand[pos] = key;
+        }
+    });
+    __syncthreads();
+    n_cand = sh.counter;
+    __syncthreads();
+    // 3. the k-th largest key
+    uint64_t t;
+    if (n_cand <= SEL_CAP) {
+        t = kth_threshold<8>(each_in_lds, k, sh);
+    } else {
+        t = kth_threshold<12>(each_in_memory, k, sh);
+        if (tid == 0) sh.counter = 0;
+        __syncthreads();
+        each_in_memory([&](uint64_t key, bool valid) {
+            if (valid && key >= t) cand[atomicAdd(&sh.counter, 1u)] = key;  // exactly k of them
+        });
+        __syncthreads();
+        n_cand = sh.counter;
+        __syncthreads();
+    }
+    // the k keys, then each one's rank among them
+    if (tid == 0) sh.counter = 0;
+    __syncthreads();
+    for (uint32_t j = tid; j < n_cand; j += SEL_THREADS) {
+        const uint64_t key = cand[j];
+        if (key >= t) sel[atomicAdd(&sh.counter, 1u)] = key;
+    }
+    __syncthreads();
+    if (tid < k) {
+        const uint64_t mine = sel[tid];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < k; j++) rank += sel[j] > mine ? 1u : 0u;
+        out_vals[rank] = topk_value(mine);
+        out_idx[rank] = 0xFFFFFFFFu - (uint32_t)mine;
+    }
+}
+
 uint32_t topk_items(size_t n) {  // elements per lane in stage 1 so that at most 256 slices (of 64 lanes) result
     const size_t per = (n + 16383) / 16384;
     return per <= 8 ? 8 : per <= 16 ? 16 : per <= 32 ? 32 : per <= 64 ? 64 : 0;
 }
+
+// From this k on the radix select is the faster of the two (128256 logits: 31-39 us whatever k, against 13 us at
+// k = 8, 26 us at 32, 36 us at 48, 47 us at 64, 173 us at 256 for the two-stage kernels).
+constexpr uint32_t TOPK_SELECT_MIN_K = 40;
 
 size_t topk_workspace_bytes(size_t n, size_t k) {
     const uint32_t items = topk_items(n);
@@ -89,6 +297,10 @@ size_t topk_workspace_bytes(size_t n, size_t k) {
 
 hipError_t launch_topk(const float *x, uint32_t n, uint32_t k, float *out_vals, uint32_t *out_idx, void *workspace,
                        hipStream_t stream) {
+    if (k >= TOPK_SELECT_MIN_K) {  // radix select by one work group; needs no workspace
+        hipLaunchKernelGGL(topk_select_kernel, dim3(1), dim3(SEL_THREADS), 0, stream, x, n, k, out_vals, out_idx);
+        return hipGetLastError();
+    }
     const uint32_t items = topk_items(n);
     const uint32_t slices = (n + 64 * items - 1) / (64 * items);
     const dim3 grid((slices + 3) / 4);

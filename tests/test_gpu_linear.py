@@ -451,6 +451,54 @@ def test_topk_matches_oracle(hip, ref):
         assert int(host(d_idx)[0]) == ref.argmax(v2)  # k = 1 is the reference's argmax
 
 
+def _topk_check(v, k, offset=0):
+    """offset: the vector starts that many floats into its allocation (not on a 16-byte boundary)."""
+    d_all = dev(v)
+    v = v[offset:]
+    n = v.size
+    ws = torch.empty(max(L.topk_workspace_bytes(n, k) // 8, 1), dtype=torch.int64, device=DEV)
+    d_vals = torch.empty(k, dtype=torch.float32, device=DEV)
+    d_idx = torch.empty(k, dtype=torch.int32, device=DEV)
+    L.topk_dev(d_all[offset:], k, d_vals, d_idx, ws)
+    vals, idx = host(d_vals), host(d_idx).view(np.uint32)
+    key = np.where(np.isnan(v), -np.inf, v.astype(np.float64))
+    order = np.argsort(-key, kind="stable")[:k]  # value descending, lower index first among equals
+    assert np.array_equal(idx, order.astype(np.uint32)), f"indices differ at {np.nonzero(idx != order)[0][:5]}"
+    assert np.array_equal(vals.view(np.uint32), v[order].view(np.uint32))
+
+
+@pytest.mark.parametrize("k", [8, 39, 40, 64, 65, 100, 200, 256])
+def test_topk_radix_select_cases(hip, k):
+    """The one-work-group radix select (k >= 8): distributions that stress each of its stages."""
+    rng = np.random.default_rng(100 + k)
+    n = 128256
+    say("topk select k", k)
+    _topk_check((rng.standard_normal(n) * 3).astype(np.float32), k)               # logits-like
+    _topk_check(np.full(n, 1.25, dtype=np.float32), k)                               # all equal: decided by index alone
+    masked = (rng.standard_normal(n) * 3).astype(np.float32)
+    masked[rng.random(n) < 0.9] = -np.inf                                            # 90 % masked out
+    _topk_check(masked, k)
+    few = np.full(n, -np.inf, dtype=np.float32)                                      # fewer finite values than k
+    few[rng.choice(n, k // 2, replace=False)] = rng.standard_normal(k // 2).astype(np.float32)
+    _topk_check(few, k)
+    close = (1.0 + rng.integers(0, 3, n) * np.float32(2.0 ** -23)).astype(np.float32)  # three adjacent floats, many ties
+    _topk_check(close, k)
+    _topk_check(rng.integers(-3, 4, n).astype(np.float32), k)                        # seven distinct values incl. +-0
+    wide = (rng.standard_normal(n) * np.exp(rng.uniform(-30, 30, n))).astype(np.float32)
+    _topk_check(wide, k)
+    _topk_check(rng.standard_normal(k).astype(np.float32), k)                        # n == k
+    _topk_check(rng.standard_normal(20000).astype(np.float32), k)
+    _topk_check(np.sort(rng.standard_normal(300000).astype(np.float32)), k)         # ascending: winners at the end
+    # the layout that defeats the filter by thread maxima: all large values in the shares of 200 of the 1024 threads
+    # (thread of index i: (i % 16384) // 4 % 1024), so that more keys pass the filter than LDS holds
+    adv = (rng.standard_normal(n) * 0.01).astype(np.float32)
+    owner = (np.arange(n) % 16384) // 4 % 1024
+    adv[owner < 200] += 100.0
+    _topk_check(adv, k)
+    for off, n2 in ((1, 128255), (3, 70001), (0, 70002), (0, 70003)):                 # unaligned start; n % 4 = 1, 2, 3
+        _topk_check((rng.standard_normal(n2 + off) * 3).astype(np.float32), k, offset=off)
+
+
 def test_topk_argument_errors(hip):
     v = torch.zeros(64, dtype=torch.float32, device=DEV)
     ws = torch.empty(4096, dtype=torch.int64, device=DEV)
