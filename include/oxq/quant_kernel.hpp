@@ -178,12 +178,21 @@ class HipKernel final : public QuantKernel {
     uint32_t type_;
 };
 
+// Which arithmetic gemv / gemm / QuantLinear::forward use for their fp32 input (process-wide, oxq.h):
+// Q8 = quantize to Q8_0 and run the fused kernels (the default, the reference's matvec_q8_fused arithmetic);
+// F32 = the reference's own gemv arithmetic (Q/reference/q4_k.rs:135-178 and siblings), five formats.
+enum class ActivationRoute : int { Q8 = OXQ_ROUTE_Q8, F32 = OXQ_ROUTE_F32 };
+
 // KernelDispatcher (dispatch.rs:141-243) with a single tier: the GPU.
 class KernelDispatcher {
   public:
     // Probes the device once (SimdCapabilities::detect, dispatch.rs:42).
     explicit KernelDispatcher(int device = 0) : init_status_(oxq_init(device)) {}
     bool has_device() const { return init_status_ == OXQ_OK; }
+    static QuantResult select_activation_route(ActivationRoute r) {
+        return QuantResult::from_status(oxq_select_activation_route(static_cast<int>(r)));
+    }
+    static ActivationRoute activation_route() { return static_cast<ActivationRoute>(oxq_activation_route()); }
 
     // Ok(Box<dyn QuantKernel>) or Err(UnsupportedType{quant_type}).
     QuantResult get_kernel(uint32_t tensor_type, std::unique_ptr<QuantKernel> &out) const {

@@ -530,6 +530,38 @@ static void gpu_tests() {
         for (int i = 0; i < 34; ++i) CHECK(out[34 + i] == 0);  // all-zero block: d = 0, q = 0
     });
 
+    // The reference's own gemv / gemm known answers at the reference's own exactness: OXQ_ROUTE_F32 runs its fp32
+    // arithmetic, so the closed forms hold exactly (every term is exactly representable in these cases).
+    run("route F32: q8_0 gemv_simple == 6.0, gemm rows == +-6.0, q4_k ones == 256.0, exactly", [&] {
+        CHECK(KernelDispatcher::select_activation_route(ActivationRoute::F32).is_ok());
+        CHECK(KernelDispatcher::activation_route() == ActivationRoute::F32);
+        bool ok = true;
+        {
+            auto k = kernel(GgufTensorType::Q8_0);
+            std::vector<int> q(32, 0);
+            q[0] = 1;
+            QuantTensor t(q8_0_block(2.0f, q), {1, 32}, GgufTensorType::Q8_0);
+            std::vector<float> x(32, 0.0f), y(1, -1.0f);
+            x[0] = 3.0f;
+            ok = ok && k->gemv(t, x, y).is_ok() && y[0] == 6.0f;  // Q/reference/q8_0.rs:175-190
+            q[0] = 4;
+            QuantTensor t2(q8_0_block(0.5f, q), {1, 32}, GgufTensorType::Q8_0);
+            std::vector<float> x2(64, 0.0f), y2(2, -1.0f);
+            x2[0] = 3.0f;
+            x2[32] = -3.0f;
+            ok = ok && k->gemm(t2, x2, y2, 2, 1, 32).is_ok() && y2[0] == 6.0f && y2[1] == -6.0f;  // q8_0.rs:216-232
+        }
+        {
+            auto k = kernel(GgufTensorType::Q4K);
+            QuantTensor t(q4_k_block(1.0f, 0.0f, {1, 1, 1, 1, 0, 0, 0, 0, 1, 1, 1, 1}, 0x11), {1, 256}, GgufTensorType::Q4K);
+            std::vector<float> x(256, 1.0f), y(1);
+            ok = ok && k->gemv(t, x, y).is_ok() && y[0] == 256.0f;  // Q/reference/q4_k.rs:411-436
+        }
+        (void)KernelDispatcher::select_activation_route(ActivationRoute::Q8);  // back before any CHECK can return
+        CHECK(ok);
+        CHECK(KernelDispatcher::activation_route() == ActivationRoute::Q8);
+    });
+
     run("gemv equals quantize + fused into zeros, bit for bit", [&] {
         auto k = kernel(GgufTensorType::Q4K);
         std::vector<uint8_t> w;
