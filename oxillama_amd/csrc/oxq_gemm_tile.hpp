@@ -324,7 +324,10 @@ __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict_
                                                      uint32_t mpad, uint32_t nsb, float *__restrict__ p16) {
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= mpad * nsb) return;
-    const uint32_t j = idx / mpad, t = idx % mpad;
+    // eight consecutive threads take eight consecutive blocks of one token (272 contiguous bytes), the next eight
+    // the next token: reads in runs of a token row's bytes, writes in runs of eight tokens (256 bytes) per sub-block
+    // (nsb is a multiple of 8: the tile kernel wants k % 256 == 0)
+    const uint32_t grp = idx >> 3, t = grp % mpad, j = (grp / mpad) * 8 + (idx & 7);
     u32x4 q[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
     uint32_t dbits = 0;
     if (t < m) {
