@@ -146,6 +146,30 @@ def launch_phases(torch, dev, quant, linear, upload, synth):
             out.append((blocks, unroll, best * 1e3 / 32))
         return out
 
+    def empty_launch_us():
+        """us per launch of a kernel that does nothing (the read-only kernel over 0 bytes), 32 launches in a graph."""
+        out = []
+        for blocks in (512, 2048):
+            def body():
+                for _ in range(32):
+                    kit.oxq_benchkit_read(big.data_ptr(), sink.data_ptr(), 0, blocks, 1, side.cuda_stream)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                body()
+                side.synchronize()
+                with torch.cuda.graph(g, stream=side):
+                    body()
+                best = 1e9
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(side)
+                    g.replay()
+                    e1.record(side)
+                    e1.synchronize()
+                    best = min(best, e0.elapsed_time(e1))
+            out.append((blocks, best * 1e3 / 32))
+        return out
+
     print("Launch phases of the decode GEMV kernels on MI355X: python bench.py --launch-phases")
     print("Every wave stamps the 100 MHz wall clock (10 ns steps) at kernel entry (t0), when its first row batch is stored (t1)")
     print("and when its last is (t2).  One launch at a time (device synchronised before each), %d launches per shape, each on" % n_sets)
@@ -154,6 +178,9 @@ def launch_phases(torch, dev, quant, linear, upload, synth):
     print("  entry: when waves enter the kernel (the dispatcher fills the chip);  first: first rows stored;  last: a wave's end.")
     print("  steady: sum over waves of (bytes the wave streams after its first batch) / (t2 - t1): the rate the waves sustain")
     print("  between ramp and tail;  span: last t2 - first t0;  whole: weight bytes / span.")
+    print("  A launch that does nothing, back to back in a HIP graph (what every launch pays before its first wave runs and")
+    print("  after its last has ended): " + ", ".join(f"{b_} work groups {us_:.2f} us" for b_, us_ in empty_launch_us()) + " per launch.")
+    graph_us = {}
     for name, wbytes, fn in cases:
         rows, by_load = [], []
         for i in range(n_sets):  # first touch of a buffer pays for its page-table walks (66 MB: 17 us against 13)
@@ -199,6 +226,26 @@ def launch_phases(torch, dev, quant, linear, upload, synth):
             "%d waves/CU: %d waves, last median %.2f latest %.2f" % (
                 c, int(np.median([d[c][0] for d in by_load if c in d])), np.median([d[c][1] for d in by_load if c in d]),
                 np.median([d[c][2] for d in by_load if c in d])) for c in loads))
+        # the same launch timed the way the bench times it: 32 launches over the 16 sets in a HIP graph
+        def body():
+            for i in range(32):
+                fn(i % n_sets)
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            body()
+            side.synchronize()
+            with torch.cuda.graph(g, stream=side):
+                body()
+            best = 1e9
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(side)
+                g.replay()
+                e1.record(side)
+                e1.synchronize()
+                best = min(best, e0.elapsed_time(e1))
+        print(f"  back to back in a HIP graph: {best * 1e3 / 32:.2f} us per launch, i.e. {best * 1e3 / 32 - span:.2f} us between one launch's "
+              f"last store and the next one's first wave")
         print(f"  the same bytes with a kernel that only reads (16 bytes per lane, coalesced; graph of 32 launches over "
               f"distinct buffers): " + ", ".join(f"{b_}x{u_}: {us_:.2f} us" for b_, u_, us_ in read_only(wbytes)))
 
