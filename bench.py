@@ -18,6 +18,7 @@ Prints ONE JSON line.  Extra objects:
   kernels      the same figure for each GEMV shape, the lm_head and C1 shapes
   prefill      batch-512 Q4_K prefill matmul, int8 TOPS vs the 5.0 POPS peak
   moe          IQ4_XS grouped expert matmuls (8 experts, 64 tokens, top-2), weight GB/s
+  moe_32_tokens  the same layer for a decode batch of 32 tokens (the few-token grouped kernel)
   cpu_baseline the CPU restatement of the reference's fused rows on this host
 """
 import argparse
@@ -618,43 +619,51 @@ def main():
 
     # ---- C5: Mixtral-shaped IQ4_XS expert matmuls, 64 tokens, top-2 of 8 experts ------------
     moe_out = None
+    moe_small = None
     if not args.no_moe:
         from oxillama_amd import moe
-        E, NTOK, TOPK = 8, 64, 2
+        E, TOPK = 8, 2
 
         def expert_set(seed, n_rows, n_cols):
             return torch.from_numpy(np.stack([synth.weights(IQ4_XS, seed + e, n_rows, n_cols) for e in range(E)])).to(dev)
         wg, wu, wd = expert_set(7000, F, H), expert_set(7100, F, H), expert_set(7200, H, F)
         stride = wg[0].numel()
-        xt = torch.from_numpy(synth.normal_f32(7, NTOK * H)).to(dev)
         router = torch.from_numpy(synth.normal_f32(9, E * H, 0.05)).to(dev)
-        rows = NTOK * TOPK
-        d_exp = torch.empty(rows, dtype=torch.int32, device=dev)
-        d_wt = torch.empty(rows, dtype=torch.float32, device=dev)
-        d_off = torch.empty(E + 1, dtype=torch.int32, device=dev)
-        d_tok = torch.empty(rows, dtype=torch.int32, device=dev)
-        d_rows = torch.empty(rows, dtype=torch.int32, device=dev)
-        d_y = torch.empty(NTOK * H, dtype=torch.float32, device=dev)
         types3 = (IQ4_XS, IQ4_XS, IQ4_XS)
-        wsm = torch.empty(moe.moe_ffn_workspace_bytes(types3, rows, H, F), dtype=torch.uint8, device=dev)
 
-        def moe_step():
-            moe.route_dev(router, xt, NTOK, E, H, TOPK, d_exp, d_wt, d_off, d_tok, d_rows)
-            moe.moe_ffn_dev((IQ4_XS, wg, stride), (IQ4_XS, wu, stride), (IQ4_XS, wd, stride), E, xt, NTOK, TOPK, d_off,
-                            d_tok, d_rows, d_wt, 0, d_y, H, F, wsm)
+        def moe_leg(NTOK):
+            xt = torch.from_numpy(synth.normal_f32(7, NTOK * H)).to(dev)
+            rows = NTOK * TOPK
+            d_exp = torch.empty(rows, dtype=torch.int32, device=dev)
+            d_wt = torch.empty(rows, dtype=torch.float32, device=dev)
+            d_off = torch.empty(E + 1, dtype=torch.int32, device=dev)
+            d_tok = torch.empty(rows, dtype=torch.int32, device=dev)
+            d_rows = torch.empty(rows, dtype=torch.int32, device=dev)
+            d_y = torch.empty(NTOK * H, dtype=torch.float32, device=dev)
+            wsm = torch.empty(moe.moe_ffn_workspace_bytes(types3, rows, H, F), dtype=torch.uint8, device=dev)
 
-        with torch.cuda.stream(stream):
-            moe_step()
-            stream.synchronize()
-            offsets = d_off.cpu().numpy()
-            reps = 6
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(reps):
+            def moe_step():
+                moe.route_dev(router, xt, NTOK, E, H, TOPK, d_exp, d_wt, d_off, d_tok, d_rows)
+                moe.moe_ffn_dev((IQ4_XS, wg, stride), (IQ4_XS, wu, stride), (IQ4_XS, wd, stride), E, xt, NTOK, TOPK,
+                                d_off, d_tok, d_rows, d_wt, 0, d_y, H, F, wsm)
+
+            with torch.cuda.stream(stream):
                 moe_step()
-            e1.record(stream)
-            e1.synchronize()
-            moe_us = e0.elapsed_time(e1) * 1e3 / reps
+                stream.synchronize()
+                offsets = d_off.cpu().numpy()
+                reps = 6
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    moe_step()
+                e1.record(stream)
+                e1.synchronize()
+            return e0.elapsed_time(e1) * 1e3 / reps, offsets
+
+        NTOK = 64
+        rows = NTOK * TOPK
+        moe_us, offsets = moe_leg(NTOK)
+        small_us, small_offsets = moe_leg(32)
         moe_bytes = 3 * E * stride
         moe_ops = 2 * rows * 3 * F * H
         moe_out = {"workload": "IQ4_XS, 8 experts x (gate, up 14336x4096; down 4096x14336), 64 tokens, top-2 "
@@ -666,6 +675,11 @@ def main():
                    "timed": "the whole layer: router + softmax + top-2 + grouping, gather + quantize, 3 grouped int8-MFMA "
                             "matmuls, SwiGLU + quantize, weighted combine (the 749 MB of expert weights exceed the "
                             "256 MB Infinity Cache, so every step streams them from HBM)"}
+        moe_small = {"workload": "the same layer for a decode batch of 32 tokens (64 pairs): with a mean of 8 rows per "
+                                 "expert the grouped matmuls take the few-token kernel (16 x 16 x 32 MFMA tiles)",
+                     "rows_per_expert": np.diff(small_offsets).tolist(), "us_per_step": round(small_us, 1),
+                     "weight_GBps": round(moe_bytes / small_us / 1e3, 1),
+                     "frac_hbm_peak": round(moe_bytes / small_us / 1e3 / HBM_PEAK_GBPS, 4)}
         del wg, wu, wd
 
     # ---- CPU baseline: the reference's fused rows restated in C, same layer -------------
@@ -787,6 +801,7 @@ def main():
         "kernels": kernels,
         "prefill": prefill,
         "moe": moe_out,
+        "moe_32_tokens": moe_small,
         "device": {"name": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
                    "clock_mhz": info["clock_khz"] / 1000.0, "weight_generation_s": round(gen_s, 1)},
     }

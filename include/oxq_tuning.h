@@ -28,7 +28,11 @@ int oxq_set_gemv_waves_per_row(unsigned waves);
 /* Fewest activation rows for which oxq_gemm_q8_dev / oxq_gemm take the tile kernel; below it
  * they run GEMV launches, two to four rows per launch (tuning knob; 0 restores the default). */
 int oxq_set_gemm_tile_min_rows(unsigned rows);
-/* Tile shape / prefetch depth of the prefill kernel (tuning knob; 0 restores the default). */
+/* Which kernel and launch shape the batched matmuls take (tuning knob; 0 restores the default, the measured choice
+ * per shape).  1..23: a fixed tile shape / prefetch depth of the int8-MFMA tile kernel; 99: the tile kernel's own
+ * choice, never the few-token kernel; 100 and up: the LDS-streamed form of the tile kernel; 200..205: the
+ * few-token kernel (16 x 16 x 32 MFMA, groups of at most 32 token rows) in a fixed shape.  A value a format or
+ * shape cannot take falls back to the default tile choice. */
 int oxq_set_gemm_variant(int variant);
 /* Launch-phase probe of the decode GEMV (Q4_0, Q8_0, Q4_K, Q6_K rows of at most two 64-unit steps, and the
  * fused gate + up launch): while d_buffer is set, those launches run an instantiation of the same kernel in

@@ -2,6 +2,7 @@
 // side, and the tile kernel instantiated for Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS.  Kernel and launch
 // templates: oxq_gemm_tile.hpp; further formats: oxq_gemm_more.hip.
 #include "oxq_gemm_stream.hpp"
+#include "oxq_gemm_skinny.hpp"
 
 namespace oxq {
 

@@ -7,6 +7,7 @@
 #define OXQ_TILE_DEFAULT_SHAPES_ONLY
 #include "oxq_formats_more.hpp"
 #include "oxq_gemm_stream.hpp"
+#include "oxq_gemm_skinny.hpp"
 
 namespace oxq {
 

@@ -1,0 +1,394 @@
+// Few tokens per weight matrix (a mixture-of-experts group of up to 32 token rows): the batched fused matvec
+//   out[m x n] (+)= A_q8[m rows of Q8_0 blocks] x W[n x k]^T
+// (the reference's gemm loop over matvec_q8_fused, crates/oxillama-quant/src/reference/q4_k.rs:186-201, :218-333)
+// built around what the counters say bounds the tile kernel in this case: not HBM, not the matrix core, but the
+// texture unit -- every lane of a weight load reads its own row (64 separate accesses per instruction), and the
+// token bytes are fetched again by every work group.
+//
+//  * Weights: a wave owns NT tiles of 16 weight rows.  It reads them as contiguous runs -- consecutive lanes take
+//    consecutive 16-byte pieces of a row's two next super-blocks -- into registers, one step ahead, and from there
+//    into a private strip of LDS; the lanes then pick their B operands out of LDS in the matrix core's layout.  No
+//    barrier: the strip belongs to one wave, whose LDS operations execute in order.
+//  * Tokens: the work group copies the Q8_0 bytes, scales and block sums of its (at most 32) tokens for the whole
+//    k chunk into LDS once, already in operand order; all waves read them from there.  Rows of k that do not fit
+//    beside the weight strips are taken in chunks, one launch per chunk, each adding to the last one's output in a
+//    fixed order.
+//  * v_mfma_i32_16x16x32_i8 with the tokens as the A operand (16 tokens x 32 k) and the weights as B (32 k x 16
+//    rows): lane l = (c = l % 16, q = l / 16) supplies k-values 8q..8q+7 of token c and of weight row c and
+//    receives the sums of row c against tokens 4q..4q+3.  All of a lane's results belong to the one weight row
+//    whose block header it reads itself, so the weight-side factors need no exchange.
+// Arithmetic per result as in the tile kernel (oxq_gemm_tile.hpp): fl(dsc * isum) by the 1.5 * 2^23 trick, then
+// one fma with the token's scale; the zero-point term one more fma with d_a * sum(q_a).
+#pragma once
+#include "oxq_gemm_tile.hpp"
+
+namespace oxq {
+
+typedef int v4i32 __attribute__((ext_vector_type(4)));
+
+template <class F>
+struct Skinny {
+    static constexpr bool OK = false;
+};
+
+// Q4_K (reference/q4_k.rs:27-99,218-333): 144 B = d, dmin, 12 B of scales / mins, 4 runs of 32 bytes whose low
+// nibbles are sub-block 2g and high nibbles sub-block 2g + 1.  Lane (c, q) takes bytes 8q..8q+7 of each run.
+template <>
+struct Skinny<TileQ4K> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 144, ROW_STRIDE = 304;  // LDS bytes per row of a step (2 blocks + pad)
+    static constexpr bool HAS_MIN = true;
+    struct Raw {
+        u32x4 hdr;
+        u32x2 qs[4];
+    };
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk) {
+        w.hdr = *reinterpret_cast<const u32x4 *>(blk);
+    }
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) w.qs[g] = *reinterpret_cast<const u32x2 *>(blk + 16 + 32 * g + 8 * q);
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const u32x2 v = w.qs[s >> 1];
+        const uint32_t lo = (s & 1) ? (v[0] >> 4) & 0x0F0F0F0Fu : v[0] & 0x0F0F0F0Fu;
+        const uint32_t hi = (s & 1) ? (v[1] >> 4) & 0x0F0F0F0Fu : v[1] & 0x0F0F0F0Fu;
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+    static __device__ __forceinline__ void factors(const Raw &w, int s, float &dsc, float &qneg) {
+        TileQ4K::Hdr hd;
+        hd.w = w.hdr;
+        float d1[1];
+        TileQ4K::factors(hd, 0, (uint32_t)s, d1, qneg);
+        dsc = d1[0];
+    }
+};
+
+// IQ4_XS (reference/iq4_xs.rs:47-97): 136 B = d, scales_h, scales_l, 8 pieces of 16 bytes, one per sub-block, byte
+// j = codebook indices of weights 2j (low nibble) and 2j + 1 (high).  Lane (c, q) takes bytes 4q..4q+3 of each
+// piece: weights 8q + {0,2,4,6} from the low nibbles, 8q + {1,3,5,7} from the high ones -- the order the
+// preparation kernel gives the token bytes for this format (even bytes, then odd bytes, inside each 8).
+template <>
+struct Skinny<TileIQ4XS> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 136, ROW_STRIDE = 288;
+    static constexpr bool HAS_MIN = false;
+    struct Raw {
+        u32x2 hdr;
+        uint32_t qs[8];
+    };
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk) {
+        w.hdr = *reinterpret_cast<const u32x2 *>(blk);
+    }
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) w.qs[s] = *reinterpret_cast<const uint32_t *>(blk + 8 + 16 * s + 4 * q);
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const uint32_t lo = FmtIQ4XS::lut4(w.qs[s] & 0x0F0F0F0Fu);
+        const uint32_t hi = FmtIQ4XS::lut4((w.qs[s] >> 4) & 0x0F0F0F0Fu);
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+    static __device__ __forceinline__ void factors(const Raw &w, int s, float &dsc, float &qneg) {
+        TileIQ4XS::Hdr hd;
+        hd.w = u32x4{w.hdr[0], w.hdr[1], 0, 0};
+        float d1[1];
+        TileIQ4XS::factors(hd, 0, (uint32_t)s, d1, qneg);
+        dsc = d1[0];
+    }
+};
+
+constexpr uint32_t SKINNY_ACT_BYTES = 512 + 64 + 64;  // per (sub-block, token tile): int8 operands, fp32 scales, fp32 P
+constexpr uint32_t SKINNY_FAC_STRIDE = 17;            // floats per weight row in a wave's factor tables (16 + pad)
+
+typedef float v4f32 __attribute__((ext_vector_type(4)));
+
+// Work group = WAVES waves, each with its own NT x 16 weight rows; all of them the same token tiles (at most TT of
+// 16 tokens).  k is walked in chunks of `per` super-blocks (even): the work group stages the chunk's token bytes,
+// every wave runs its rows over the chunk, accumulators staying in registers; the weight prefetch runs on across
+// the chunk boundary.  blockIdx.x = row group, blockIdx.y = expert (grouped form) or 0, blockIdx.z = token pass.
+// LDS: [A operands | fp32 token scales | P] of a chunk, then per wave [weight strip | dsc table | zero-point table].
+// Waves per SIMD the shape is meant to run at: two work groups on a compute unit where their LDS allows it.
+template <class F, int NT, int WAVES, int TT, int PER>
+constexpr int skinny_waves_per_simd() {
+    constexpr size_t lds = (size_t)PER * 8 * TT * SKINNY_ACT_BYTES +
+                           (size_t)WAVES * NT * 16 * (Skinny<F>::ROW_STRIDE + SKINNY_FAC_STRIDE * 4 * (Skinny<F>::HAS_MIN ? 2 : 1));
+    return lds <= 80 * 1024 ? WAVES / 2 : WAVES / 4;
+}
+
+template <class F, int NT, int WAVES, int TT, int PER, bool DUMP>
+__global__ __launch_bounds__(64 * WAVES)
+__attribute__((amdgpu_waves_per_eu(skinny_waves_per_simd<F, NT, WAVES, TT, PER>(), skinny_waves_per_simd<F, NT, WAVES, TT, PER>())))
+void gemm_skinny_kernel(
+    const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,
+    const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m, uint32_t mpad,
+    uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride) {
+    using S = Skinny<F>;
+    constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: as_float(0x4B400000 + i) == MAGIC + i for |i| < 2^22
+    constexpr uint32_t RS = S::ROW_STRIDE, SEG = 2 * S::BLOCK, PPR = SEG / 16;  // 16-byte pieces per row per step
+    constexpr uint32_t PIECES = NT * 16 * PPR, NL = (PIECES + 63) / 64;
+    constexpr uint32_t THREADS = 64 * WAVES, FS = SKINNY_FAC_STRIDE;
+    constexpr uint32_t WAVE_LDS = NT * 16 * (RS + FS * 4 * (S::HAS_MIN ? 2 : 1));
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    const uint32_t lane = threadIdx.x & 63, c = lane & 15, q = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    uint32_t tok0 = 0, tok_end = m;
+    if (offsets) {
+        tok0 = (uint32_t)offsets[blockIdx.y];
+        tok_end = (uint32_t)offsets[blockIdx.y + 1];
+    }
+    // blockIdx.z = which 16 * TT token rows of the group: the launch is shaped for the usual group, a larger one
+    // takes further work groups per row group (each its own pass over the weights); the rest exit here
+    const uint32_t tokb = tok0 + blockIdx.z * (16 * TT);
+    if (tokb >= tok_end) return;  // the whole work group
+    const uint32_t n_super = k / 256;
+    constexpr uint32_t per = PER, nblk_max = PER * 8;  // sub-blocks (Q8_0 blocks per token) of a full chunk
+    uint8_t *const ldsA = lds;
+    float *const ldsD = reinterpret_cast<float *>(ldsA + (size_t)nblk_max * TT * 512);
+    float *const ldsP = ldsD + (size_t)nblk_max * TT * 16;
+    uint8_t *const strip = reinterpret_cast<uint8_t *>(ldsP + (size_t)nblk_max * TT * 16) + wave * WAVE_LDS;
+    float *const dscT = reinterpret_cast<float *>(strip + NT * 16 * RS);
+    float *const minT = dscT + NT * 16 * FS;
+
+    // ---- a chunk's tokens: from the workspace into registers (requested a chunk ahead, in flight while the last
+    // chunk is computed), from there into LDS in operand order.  Token rows past the group's end: whatever the
+    // padded workspace holds there; their results are never stored. ----
+    constexpr uint32_t KA = (nblk_max * TT * 64 + THREADS - 1) / THREADS, KS = (nblk_max * TT * 16 + THREADS - 1) / THREADS;
+    u32x2 tokA[KA];
+    uint32_t tokD[KS];
+    float tokP[KS];
+    auto load_tokens = [&](uint32_t sb0, uint32_t nblk) {
+        const uint32_t total = nblk * TT * 64, total_s = nblk * TT * 16;
+#pragma unroll
+        for (uint32_t i = 0; i < KA; i++) {
+            const uint32_t idx = min(threadIdx.x + i * THREADS, total - 1);
+            const uint32_t l = idx & 63, t = (idx >> 6) % TT, b = (idx >> 6) / TT;
+            const uint32_t cc = l >> 2, qq = l & 3;  // consecutive threads: consecutive 8 bytes of a token's block
+            tokA[i] = ld8(q8t + ((size_t)(sb0 * 8 + b) * mpad + tokb + 16 * t + cc) * 32 + 8 * qq);
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < KS; i++) {
+            const uint32_t idx = min(threadIdx.x + i * THREADS, total_s - 1);
+            const uint32_t cc = idx & 15, t = (idx >> 4) % TT, b = (idx >> 4) / TT;
+            const size_t src = (size_t)(sb0 * 8 + b) * mpad + tokb + 16 * t + cc;
+            tokD[i] = da16[src];
+            tokP[i] = S::HAS_MIN ? P[src] : 0.0f;
+        }
+    };
+    auto store_tokens = [&](uint32_t nblk) {
+        const uint32_t total = nblk * TT * 64, total_s = nblk * TT * 16;
+#pragma unroll
+        for (uint32_t i = 0; i < KA; i++) {
+            const uint32_t idx = min(threadIdx.x + i * THREADS, total - 1);
+            const uint32_t l = idx & 63, cc = l >> 2, qq = l & 3;
+            *reinterpret_cast<u32x2 *>(ldsA + ((size_t)(idx >> 6) * 64 + qq * 16 + cc) * 8) = tokA[i];
+        }
+#pragma unroll
+        for (uint32_t i = 0; i < KS; i++) {
+            const uint32_t idx = min(threadIdx.x + i * THREADS, total_s - 1);
+            ldsD[idx] = h2f(tokD[i]);
+            if (S::HAS_MIN) ldsP[idx] = tokP[i];
+        }
+    };
+
+    const uint32_t rbase = (blockIdx.x * WAVES + wave) * (16 * NT);
+    const bool active = rbase < n;  // a wave past the last row still stages tokens and meets the barriers
+    const uint8_t *We = W + (offsets ? (size_t)blockIdx.y * w_stride : 0);
+    const size_t row_bytes = (size_t)(k / 256) * S::BLOCK;
+    // the lane's pieces of a step: where they come from (less the step's offset) and where they go
+    const uint8_t *src[NL];
+    uint32_t dst[NL];
+#pragma unroll
+    for (uint32_t i = 0; i < NL; i++) {
+        const uint32_t p = min(i * 64 + lane, PIECES - 1), r = p / PPR, piece = p % PPR;
+        src[i] = We + (size_t)min(rbase + r, n - 1) * row_bytes + piece * 16;
+        dst[i] = r * RS + piece * 16;
+    }
+    const uint32_t tiles_here = min((uint32_t)TT, (tok_end - tokb + 15) / 16);
+    v4f32 acc[TT][NT];
+#pragma unroll
+    for (int t = 0; t < TT; t++)
+#pragma unroll
+        for (int j = 0; j < NT; j++) acc[t][j] = v4f32{0.0f, 0.0f, 0.0f, 0.0f};
+
+    u32x4 stage[NL];
+#pragma unroll
+    for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i]);
+    const uint32_t steps = n_super / 2;
+    load_tokens(0, min(per, n_super) * 8);
+    for (uint32_t sb0 = 0; sb0 < n_super; sb0 += per) {
+    const uint32_t nsbc = min(per, n_super - sb0);
+    __syncthreads();  // every wave is done with the last chunk's tokens
+    store_tokens(nsbc * 8);
+    __syncthreads();
+    if (sb0 + per < n_super) load_tokens(sb0 + per, min(per, n_super - sb0 - per) * 8);
+    if (active)
+    for (uint32_t st = sb0 / 2; st < (sb0 + nsbc) / 2; st++) {
+        // the step's bytes to the strip (pieces past the end, on the last load: the last piece again, same value)
+#pragma unroll
+        for (uint32_t i = 0; i < NL; i++) *reinterpret_cast<u32x4 *>(strip + dst[i]) = stage[i];
+        if (st + 1 < steps) {
+#pragma unroll
+            for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i] + (size_t)(st + 1) * SEG);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // scale factors of the step, decoded once: lane (c, q) takes row c, super-block q / 2, sub-blocks
+        // 4 (q % 2) .. + 3, for each tile
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            typename S::Raw hd;
+            S::read_hdr(hd, strip + (16 * j + c) * RS + (q >> 1) * S::BLOCK);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float dsc, qneg;
+                S::factors(hd, 4 * (q & 1) + i, dsc, qneg);
+                dscT[(16 * j + c) * FS + 4 * q + i] = dsc;
+                if (S::HAS_MIN) minT[(16 * j + c) * FS + 4 * q + i] = qneg;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            typename S::Raw raw[NT];
+#pragma unroll
+            for (int j = 0; j < NT; j++) S::read(raw[j], strip + (16 * j + c) * RS + u * S::BLOCK, q);
+            const uint32_t b0 = (st * 2 + u - sb0) * 8;
+            if (S::HAS_MIN) {
+                // zero-point term: per four sub-blocks one 16 x 16 x 4 fp32 product of P (tokens x sub-blocks) and the
+                // rows' factors, straight into the accumulators
+#pragma unroll
+                for (int hf = 0; hf < 2; hf++)
+#pragma unroll
+                    for (int t = 0; t < TT; t++)
+                        if (t < (int)tiles_here) {
+                            const float pa = ldsP[((b0 + 4 * hf + q) * TT + t) * 16 + c];
+#pragma unroll
+                            for (int j = 0; j < NT; j++) {
+                                const float zb = minT[(16 * j + c) * FS + u * 8 + 4 * hf + q];
+                                acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa, zb, acc[t][j], 0, 0, 0);
+                            }
+                        }
+            }
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                float dsc[NT], corr[NT];
+                long bop[NT];
+#pragma unroll
+                for (int j = 0; j < NT; j++) {
+                    dsc[j] = dscT[(16 * j + c) * FS + u * 8 + s];
+                    corr[j] = -(MAGIC * dsc[j]);
+                    bop[j] = S::operand(raw[j], s);
+                }
+#pragma unroll
+                for (int t = 0; t < TT; t++) {
+                    if (t < (int)tiles_here) {
+                        const uint32_t e = (b0 + s) * TT + t;
+                        const u32x2 av = *reinterpret_cast<const u32x2 *>(ldsA + ((size_t)e * 64 + lane) * 8);
+                        const long a = (long)(((uint64_t)av[1] << 32) | av[0]);
+                        const v4f32 da = *reinterpret_cast<const v4f32 *>(ldsD + (size_t)e * 16 + 4 * q);
+#pragma unroll
+                        for (int j = 0; j < NT; j++) {
+                            const v4i32 magic = {0x4B400000, 0x4B400000, 0x4B400000, 0x4B400000};
+                            const v4i32 r = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bop[j], magic, 0, 0, 0);
+#pragma unroll
+                            for (int v = 0; v < 4; v++) {
+                                const int ri = r[v];
+                                const float tt = fmaf(__builtin_bit_cast(float, ri), dsc[j], corr[j]);  // fl(dsc * isum)
+                                acc[t][j][v] = fmaf(tt, da[v], acc[t][j][v]);
+                                if (DUMP) {  // the integer sum of (token, weight row, sub-block)
+                                    const uint32_t tok = tokb + 16 * t + 4 * q + v, row = rbase + 16 * j + c;
+                                    if (tok < tok_end && row < n)
+                                        sums[((size_t)tok * n + row) * (k / 32) + (st * 2 + u) * 8 + s] = ri - 0x4B400000;
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    }
+    }
+#pragma unroll
+    for (int t = 0; t < TT; t++)
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+            const uint32_t row = rbase + 16 * j + c;
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const uint32_t tok = tokb + 16 * t + 4 * q + v;
+                if (row < n && tok < tok_end && t < (int)tiles_here) {
+                    float *o = out + (size_t)tok * n + row;
+                    const float y = acc[t][j][v];
+                    *o = accumulate ? *o + y : bias ? y + bias[row] : y;
+                }
+            }
+        }
+}
+
+template <class F, int NT, int WAVES, int TT, int PER, bool DUMP = false>
+static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
+    using S = Skinny<F>;
+    const size_t strips = (size_t)WAVES * NT * 16 * (S::ROW_STRIDE + SKINNY_FAC_STRIDE * 4 * (S::HAS_MIN ? 2 : 1));
+    auto kern = &gemm_skinny_kernel<F, NT, WAVES, TT, PER, DUMP>;
+    const size_t lds = (size_t)PER * 8 * TT * SKINNY_ACT_BYTES + strips;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds);
+    if (e != hipSuccess) return e;
+    // token passes: as many as the largest group can need (max_rows is the caller's bound, all rows if unknown)
+    const uint32_t group_rows = a.offsets ? a.max_rows : a.m;
+    const dim3 grid((a.n + 16 * NT * WAVES - 1) / (16 * NT * WAVES), a.offsets ? a.n_experts : 1,
+                    (group_rows + 16 * TT - 1) / (16 * TT));
+    if (grid.z > 65535) return hipErrorNotSupported;
+    note_launch("gemm_skinny_kernel", F::TYPE, NT, WAVES, TT, PER, grid.x, grid.y * grid.z, 64 * WAVES);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES), lds, stream, a.W, p.q8t, p.P, p.da16, a.out, a.sums, a.m, p.mpad, a.n, a.k,
+                       a.accumulate, a.bias, a.offsets, a.w_stride);
+    return hipGetLastError();
+}
+
+// hipErrorNotSupported: not this format / shape, or one the tile kernel serves better.  rows = the token rows per
+// group the launch is shaped for.  variant 0: the measured choice; 200..205: a fixed shape (tuning, tests).
+// Measured on MI355X, 8 experts of Mixtral's shapes (IQ4_XS; Q4_K alike), cold weights, against the tile kernel:
+//  * up to 16 rows per expert: 14336 x 4096 84 us against 106, 4096 x 14336 90 against 107;
+//  * 17..32 rows: two token tiles double the arithmetic per weight byte.  With a mean of 12 rows (most experts still
+//    one tile) 14336 x 4096 takes 88 us against 102; with a mean of 16 it is 98-107 against 101-106, no gain, and
+//    4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106;
+//  * one matrix, no experts: too few row groups for this shape (14336 x 4096, 16 tokens: 24 us against 19).
+template <class F>
+static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_t stream, uint32_t rows, int variant) {
+    if constexpr (Skinny<F>::OK) {
+        // whole steps of two super-blocks
+        if (a.k % 512 != 0 || rows > 32) return hipErrorNotSupported;
+        const bool two = rows > 16;
+        // <NT, WAVES, TT, PER>; LDS = PER * 8 * TT * 640 + WAVES * NT * 7 KB
+        if (a.sums && variant != 0 && variant != 200) return hipErrorNotSupported;
+        switch (variant) {
+        case 0: {
+            if (!a.offsets) return hipErrorNotSupported;
+            const bool many = (size_t)((a.n + 127) / 128) * a.n_experts >= 2 * (size_t)device_cus();
+            // two token tiles: only with many row groups and a mean of at most 12 rows per expert
+            if (two && (!many || 4 * (size_t)a.m > 3 * 16 * (size_t)a.n_experts)) return hipErrorNotSupported;
+            // debug dump: one shape per token-tile count (every shape adds a result's terms in the same order)
+            if (a.sums) return two ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream);
+            if (two) return launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream);
+            return many ? launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 8>(a, p, stream);
+        }
+        case 200:
+            if (a.sums) return two ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream);
+            return two ? launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream);
+        case 201: return two ? launch_skinny_shape<F, 1, 8, 2, 8>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 16>(a, p, stream);
+        case 203: return two ? launch_skinny_shape<F, 1, 4, 2, 4>(a, p, stream) : launch_skinny_shape<F, 1, 4, 1, 8>(a, p, stream);
+        case 204: return two ? launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream);
+        case 205: return two ? launch_skinny_shape<F, 1, 8, 2, 4>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 8>(a, p, stream);
+        default: return hipErrorNotSupported;
+        }
+    }
+    return hipErrorNotSupported;
+}
+
+}  // namespace oxq

@@ -1,0 +1,156 @@
+"""The few-token grouped matmul kernel (oxq_gemm_skinny.hpp: 16 x 16 x 32 int8 MFMA, weight rows read as contiguous
+runs through a per-wave LDS strip, a group's tokens staged in LDS) through the C ABI against the CPU oracle:
+integer sub-block sums bit-exact, fp32 within 1e-5 * |y_ref|_inf.  Every case asserts that the library really took
+this kernel (oxq_last_launch), so a change of launch policy cannot quietly turn these into tests of the tile kernel."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle as O
+from oxillama_amd import synth
+from test_gpu_parity import assert_close, canonical_ref, say
+
+pytestmark = pytest.mark.gpu
+
+FORMATS = [O.Q4_K, O.IQ4_XS]
+
+
+def last_launch():
+    from oxillama_amd import capi
+    buf = C.create_string_buffer(256)
+    capi.load().oxq_last_launch(buf, 256)
+    return buf.value.decode()
+
+
+def _case(ref, t, counts, n, k_, seed):
+    """Experts with the given token-row counts: offsets, Q8_0 activation rows, weights."""
+    offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    rows = int(offsets[-1])
+    x = synth.normal_f32(seed, rows * k_).reshape(rows, k_)
+    acts = ref.quantize_q8_0(x.reshape(-1)).reshape(rows, k_ // 32 * 34)
+    w = np.stack([synth.weights(t, seed + 10 + e, n, k_) for e in range(len(counts))])
+    return offsets, acts, w
+
+
+def _oracle_rows(ref, t, w, acts, offsets, n, k_, sample):
+    y, s = {}, {}
+    for r in sample:
+        e = int(np.searchsorted(offsets, r, side="right") - 1)
+        y[r] = canonical_ref(ref, t, w[e], acts[r], n, k_, threads=16)
+        s[r] = ref.block_sums(t, w[e], acts[r], n, k_)
+    return y, s
+
+
+def _run(hip, t, w, acts, offsets, n, k_, max_rows, sums=False, accumulate=False, out=None):
+    import torch
+    rows = int(offsets[-1])
+    kern = hip.HipKernel(t)
+    ws = torch.empty(kern.moe_gemm_workspace_bytes(rows, n, k_), dtype=torch.uint8, device="cuda")
+    dw, da, doff = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda(), torch.from_numpy(offsets).cuda()
+    dy = out if out is not None else torch.full((rows + 2, n), 7.0, dtype=torch.float32, device="cuda")
+    dsum = torch.full((rows, n, k_ // 32), -1, dtype=torch.int32, device="cuda") if sums else None
+    kern.moe_gemm_q8_dev(dw, w[0].nbytes, len(offsets) - 1, da, doff, rows, max_rows, dy, n, k_, ws,
+                         accumulate=accumulate, d_sums=dsum)
+    torch.cuda.synchronize()
+    return dy, dsum
+
+
+# (row counts per expert, n, k, max_rows handed to the call): one token tile / two (the default takes two only with
+# many row groups and a mean of at most 12 rows per expert); few row groups / at least two per compute unit; an expert without rows; ragged n (a wave past the last row, a tile cut at n % 16); k of one step, of a
+# whole number of chunks and with a short last chunk; groups larger than the launch is shaped for (max_rows = 0: the
+# shape follows twice the mean, the largest group takes further passes over its weights)
+CASES = [
+    ([3, 0, 16, 1], 300, 512, 16),
+    ([5, 9, 2, 16, 7, 1, 0, 11], 72, 1536, 16),
+    ([16, 16], 128, 2560, 16),
+    ([12, 7, 16, 3, 9, 14, 2, 5], 8192, 512, 16),
+    ([20, 3, 15, 4, 17, 1, 19, 12], 8192, 1024, 20),
+    ([32, 1, 17, 0, 8, 30, 2, 5], 8200, 512, 32),
+    ([2, 1, 40, 1, 3, 0, 1, 2], 96, 1024, 0),
+    ([9, 50, 3, 2, 1, 0, 20, 5], 8192, 512, 0),
+]
+
+
+@pytest.mark.parametrize("t", FORMATS, ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "r%d_n%d_k%d_max%d" % (sum(c[0]), c[1], c[2], c[3]))
+def test_skinny_grouped_against_oracle(hip, ref, t, case):
+    counts, n, k_, max_rows = case
+    say("skinny", O.NAMES[t], case)
+    offsets, acts, w = _case(ref, t, counts, n, k_, 4100 + n + k_)
+    rows = int(offsets[-1])
+    dy, dsum = _run(hip, t, w, acts, offsets, n, k_, max_rows, sums=True)
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    y, s = dy.cpu().numpy(), dsum.cpu().numpy()
+    assert np.all(y[rows:] == 7.0)  # guard rows
+    sample = range(rows) if n <= 512 else sorted(set(list(range(0, rows, 7)) + [int(o) for o in offsets[:-1] if o < rows] +
+                                                      [int(o) - 1 for o in offsets[1:] if o > 0]))
+    y_ref, s_ref = _oracle_rows(ref, t, w, acts, offsets, n, k_, sample)
+    for r in sample:
+        assert_close(y[r], y_ref[r], f"skinny {case} row {r}")
+        assert np.array_equal(s[r], s_ref[r]), f"integer sums of row {r}"
+    # the production launch (no sums): the same bits; overwrite then accumulate: twice them
+    dy2, _ = _run(hip, t, w, acts, offsets, n, k_, max_rows)
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    import torch
+    assert torch.equal(dy2, dy)
+    dy3, _ = _run(hip, t, w, acts, offsets, n, k_, max_rows, accumulate=True, out=dy2.clone())
+    assert torch.equal(dy3[:rows], dy[:rows] + dy[:rows]) and torch.equal(dy3[rows:], dy[rows:])
+
+
+@pytest.mark.parametrize("t", FORMATS, ids=lambda t: O.NAMES[t])
+def test_skinny_shapes_give_the_same_bits(hip, ref, tuning, t):
+    """Every launch shape of the kernel (waves per work group, super-blocks per chunk) adds a result's terms in the same
+    order; the tile kernel (another order) agrees within the fp32 bar."""
+    import torch
+    counts, n, k_ = [20, 3, 16, 0, 31, 9], 400, 3584
+    offsets, acts, w = _case(ref, t, counts, n, k_, 977)
+    rows = int(offsets[-1])
+    outs = {}
+    for variant in (0, 200, 201, 203, 204, 205, 99):
+        tuning("gemm_variant", variant)
+        dy, _ = _run(hip, t, w, acts, offsets, n, k_, 31)
+        say(" variant", variant, last_launch())
+        assert last_launch().startswith("gemm_tile_kernel" if variant in (0, 99) else "gemm_skinny_kernel"), last_launch()
+        outs[variant] = dy[:rows].clone()
+    for variant in (201, 203, 204, 205):
+        assert torch.equal(outs[variant], outs[200]), variant
+    assert torch.equal(outs[0], outs[99])  # two token tiles on few row groups: the default is the tile kernel
+    assert_close(outs[200].cpu().numpy(), outs[99].cpu().numpy(), "skinny against tile kernel")
+
+
+@pytest.mark.parametrize("t", FORMATS, ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("m", [1, 16, 17, 32])
+def test_skinny_plain_matmul_forced(hip, ref, tuning, t, m):
+    """One matrix, no experts (the default there is the tile kernel; the kernel is selectable), ragged n."""
+    import torch
+    n, k_ = 1000, 2048
+    w = synth.weights(t, 31, n, k_)
+    x = synth.normal_f32(32 + m, m * k_)
+    acts = ref.quantize_q8_0(x).reshape(m, k_ // 32 * 34)
+    kern = hip.HipKernel(t)
+    tuning("gemm_tile_min_rows", 1)
+    tuning("gemm_variant", 204)
+    ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
+    dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    kern.gemm_q8_dev(torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda(), dy, m, n, k_, workspace=ws)
+    torch.cuda.synchronize()
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    y = dy.cpu().numpy()
+    for r in range(m):
+        assert_close(y[r], canonical_ref(ref, t, w, acts[r], n, k_), f"plain m={m} row {r}")
+
+
+def test_skinny_full_size_c5_gate(hip, ref):
+    """C5's gate shape, 8 experts of IQ4_XS 14336 x 4096, up to 16 rows each and up to 32: oracle on sampled rows."""
+    t, n, k_ = O.IQ4_XS, 14336, 4096
+    for counts in ([11, 11, 9, 6, 10, 3, 9, 5], [20, 3, 15, 4, 17, 1, 19, 12]):
+        offsets, acts, w = _case(ref, t, counts, n, k_, 6000 + counts[0])
+        rows = int(offsets[-1])
+        dy, _ = _run(hip, t, w, acts, offsets, n, k_, max(counts))
+        assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+        y = dy.cpu().numpy()
+        for r in list(range(0, rows, 13)) + [rows - 1]:
+            e = int(np.searchsorted(offsets, r, side="right") - 1)
+            assert_close(y[r], canonical_ref(ref, t, w[e], acts[r], n, k_, threads=16), f"c5 gate row {r} expert {e}")
+        del dy
