@@ -71,7 +71,8 @@ struct Skinny<TileQ4K> {
 template <>
 struct Skinny<TileIQ4XS> {
     static constexpr bool OK = true;
-    static constexpr uint32_t BLOCK = 136, ROW_STRIDE = 288;
+    // 272 bytes = 68 dwords per row: lane (c, q) reads dword 68 c + q + const, bank 4 c + q -- all 64 distinct
+    static constexpr uint32_t BLOCK = 136, ROW_STRIDE = 272;
     static constexpr bool HAS_MIN = false;
     struct Raw {
         u32x2 hdr;
@@ -211,6 +212,11 @@ void gemm_skinny_kernel(
 #pragma unroll
         for (int j = 0; j < NT; j++) acc[t][j] = v4f32{0.0f, 0.0f, 0.0f, 0.0f};
 
+    // the MFMA's addend, 1.5 * 2^23 in every element: made opaque so that it stays in one register quad for the whole
+    // walk (as a plain constant the compiler rebuilds three of the four registers before every MFMA)
+    v4i32 magic;
+    asm volatile("v_mov_b32 %0, 0x4b400000\n\tv_mov_b32 %1, 0x4b400000\n\tv_mov_b32 %2, 0x4b400000\n\tv_mov_b32 %3, 0x4b400000"
+                 : "=v"(magic[0]), "=v"(magic[1]), "=v"(magic[2]), "=v"(magic[3]));
     u32x4 stage[NL];
 #pragma unroll
     for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i]);
@@ -298,7 +304,6 @@ void gemm_skinny_kernel(
                         const v4f32 da = *reinterpret_cast<const v4f32 *>(ldsD + (size_t)e * 16 + 4 * q);
 #pragma unroll
                         for (int j = 0; j < NT; j++) {
-                            const v4i32 magic = {0x4B400000, 0x4B400000, 0x4B400000, 0x4B400000};
                             const v4i32 r = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bop[j], magic, 0, 0, 0);
 #pragma unroll
                             for (int v = 0; v < 4; v++) {
