@@ -302,7 +302,9 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
  * expert_stride_bytes and writes the same rows of d_out [total_rows x n].  d_row_offsets is
  * device memory (n_experts + 1 ascending int32 values, last = total_rows), so the call neither
  * copies nor synchronises; max_rows_per_expert bounds any one group (0 = total_rows) and only
- * sizes the launch.  k must be a multiple of 256; needs oxq_moe_gemm_q8_workspace_bytes() bytes of
+ * sizes the launch (which kernel and tile shape serve the call follows from it and from the mean
+ * group size: fp32 summation order, hence the last bits, can differ between two bounds; every
+ * choice meets the 1e-5 bar).  k must be a multiple of 256; needs oxq_moe_gemm_q8_workspace_bytes() bytes of
  * 256-byte-aligned device scratch.  d_sums (optional, else NULL): exact int32 group sums
  * [(row * n + c) * (k/32) + g] as in oxq_gemm_block_sums_dev. */
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k);
