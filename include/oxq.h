@@ -276,7 +276,7 @@ int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
 /* oxq_gemm_q8_dev for callers that cannot allocate device memory and have no workspace to pass
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
  * counterpart in the reference.  The tile kernel's workspace is a static array in device
- * memory that the library holds on each GPU it was initialised on (8 MiB:
+ * memory that the library holds on each GPU it was initialised on (16 MiB:
  * oxq_gemm_q8_static_max_workspace_bytes()); the call allocates nothing, synchronises nothing and
  * gives the bits of oxq_gemm_q8_dev.  Shapes whose oxq_gemm_q8_workspace_bytes exceeds the
  * array return OXQ_ERR_BUFFER_TOO_SMALL (needed, available); oxq_init must have run (the call

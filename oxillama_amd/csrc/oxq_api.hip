@@ -19,7 +19,7 @@ hipError_t launch_dequant(uint32_t type, const uint8_t *blocks, size_t n_blocks,
 // f16 scales) live here instead of in a caller's or the library's allocation.  Every GPU the library runs on holds
 // its own copy at its own address until the process ends; host code reaches it only through the address that
 // hipGetSymbolAddress returned for that device (static_scratch_ptr), never through this name.
-constexpr size_t STATIC_SCRATCH_BYTES = (size_t)8 << 20;
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)16 << 20;
 static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
 
 namespace {
@@ -668,8 +668,10 @@ static int gemm_host(uint32_t type, const uint8_t *data, size_t data_len, const 
     ga.sums = nullptr;
     ga.workspace = nullptr;
     if (oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n_rows, (uint32_t)n_cols)) {
-        if ((st = g.s_work.reserve(oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)n_cols))) != OXQ_OK) return st;
+        const size_t wbytes = oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)n_cols, (uint32_t)n_rows, type);
+        if ((st = g.s_work.reserve(wbytes)) != OXQ_OK) return st;
         ga.workspace = (uint8_t *)g.s_work.ptr;
+        ga.workspace_bytes = wbytes;
     }
     ga.m = (uint32_t)m;
     ga.n = (uint32_t)n_rows;
@@ -870,7 +872,7 @@ size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k) 
     if (m > 0xFFFFFFFFull || n > 0xFFFFFFFFull || k > 0xFFFFFFFFull ||
         !oxq::gemm_tiles_supported(type, (uint32_t)m, (uint32_t)k))
         return 0;
-    return oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k);
+    return oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k, (uint32_t)n, type);
 }
 
 static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out, int32_t *d_sums,
@@ -895,12 +897,13 @@ static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
     // one reading of the tuning knobs per call: tile kernel, or GEMV launches (which need no workspace)
     const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k);
     ga.by_rows = !tiles;
-    const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k) : 0;
+    const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k, (uint32_t)n, type) : 0;
     if (need && d_workspace) {
         if (workspace_bytes < need) return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, workspace_bytes, "workspace too small");
         if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
             return fail(OXQ_ERR_KERNEL, 256, reinterpret_cast<uintptr_t>(d_workspace) & 255, "workspace must be 256-byte aligned");
         ga.workspace = (uint8_t *)d_workspace;
+        ga.workspace_bytes = workspace_bytes;
         OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
         return OXQ_OK;
     }
@@ -910,6 +913,7 @@ static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
         std::lock_guard<std::mutex> lock(g.mu);
         if ((st = g.s_work.reserve(need)) != OXQ_OK) return st;
         ga.workspace = (uint8_t *)g.s_work.ptr;
+        ga.workspace_bytes = need;
         OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
         OXQ_HIP(hipStreamSynchronize((hipStream_t)stream));
         return OXQ_OK;
@@ -937,7 +941,7 @@ int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_
         return fail(OXQ_ERR_NO_DEVICE, 0, 0, "call oxq_init first: this entry point sets nothing up by itself");
     if (m == 0 || n == 0 || k == 0) return OXQ_OK;
     const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k);
-    const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k) : 0;
+    const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k, (uint32_t)n, type) : 0;
     if (need > STATIC_SCRATCH_BYTES)
         return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, STATIC_SCRATCH_BYTES,
                     "shape needs more workspace than the static scratch holds: use oxq_gemm_q8_dev with a workspace");
@@ -946,6 +950,7 @@ int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_
     ga.A = d_acts_q8;
     ga.out = d_out;
     ga.sums = nullptr;
+    ga.workspace_bytes = tiles ? STATIC_SCRATCH_BYTES : 0;
     ga.workspace = tiles ? static_scratch_ptr[g.device] : nullptr;  // every byte the tile kernel reads is written
     ga.by_rows = !tiles;                                            // by the preparation kernel of this same call
     ga.m = (uint32_t)m;

@@ -54,10 +54,20 @@ static hipError_t gemm_by_rows(uint32_t type, const GemmArgs &a, hipStream_t str
 
 std::atomic<int> g_gemm_variant{0};  // tuning: 0 = default
 
-size_t gemm_workspace_bytes(uint32_t m, uint32_t k) {
+static size_t gemm_planes_bytes(uint32_t m, uint32_t k) {
     // token rows are padded so that a 128-token tile starting at any row stays inside
     const size_t mpad = ((size_t)m + 127) / 128 * 128 + 128, nsb = k / 32;
     return nsb * mpad * (32 + 4 + 2 + 8);  // activation bytes, P, f16 scales, the two half-block planes of P
+}
+// Bytes of the few-token kernel's per-split sums for this call, 0 if it would not split k.
+static size_t gemm_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
+    if ((type != OXQ_TYPE_Q4_K && type != OXQ_TYPE_IQ4_XS) || m > 16 || n == 0) return 0;
+    const uint32_t splits = skinny_splits(n, k);
+    return splits > 1 ? (size_t)splits * m * n * sizeof(float) : 0;
+}
+size_t gemm_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t type) {
+    const size_t planes = (gemm_planes_bytes(m, k) + 255) & ~(size_t)255;
+    return planes + gemm_partial_bytes(type, m, n, k);
 }
 
 std::atomic<uint32_t> g_gemm_tile_min_rows{0};  // tuning: 0 = default
@@ -72,7 +82,7 @@ bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
                        type == OXQ_TYPE_Q3_K || type == OXQ_TYPE_Q2_K;
     // the 32-weight formats are walked eight blocks at a time
     return known && k % 256 == 0 && m >= 1 && (size_t)(k / 32) * 256 <= 128 * 1024 &&
-           gemm_workspace_bytes(m, k) < 0x7FFFFFFFull;
+           gemm_planes_bytes(m, k) < 0x7FFFFFFFull;
 }
 
 // ... and is the faster way for m activation rows.  Below the threshold GEMV launches that take up
@@ -102,7 +112,10 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
                : (t == OXQ_TYPE_Q4_K || t == OXQ_TYPE_Q8_0) ? 0 : tile_act_perm_more(t);
     };
     const int perm = act_perm(type);
-    const TilePlan plan = {q8t, P, da16, mpad};
+    TilePlan plan = {q8t, P, da16, mpad};
+    if (!a.offsets && gemm_partial_bytes(type, a.m, a.n, a.k) &&
+        a.workspace_bytes >= gemm_workspace_bytes(a.m, a.k, a.n, type))
+        plan.partial = reinterpret_cast<float *>(a.workspace + ((gemm_planes_bytes(a.m, a.k) + 255) & ~(size_t)255));
     // the previous call left the same activations in the same byte order (and the half-block planes if this
     // format needs them): go straight to the tile kernel
     const bool prepared = a.prepared_for != 0 && act_perm(a.prepared_for) == perm &&

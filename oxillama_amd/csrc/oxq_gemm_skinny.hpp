@@ -107,7 +107,10 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 // Work group = WAVES waves, each with its own NT x 16 weight rows; all of them the same token tiles (at most TT of
 // 16 tokens).  k is walked in chunks of `per` super-blocks (even): the work group stages the chunk's token bytes,
 // every wave runs its rows over the chunk, accumulators staying in registers; the weight prefetch runs on across
-// the chunk boundary.  blockIdx.x = row group, blockIdx.y = expert (grouped form) or 0, blockIdx.z = token pass.
+// the chunk boundary.  blockIdx.x = row group, blockIdx.y = expert (grouped form), blockIdx.z = token pass.
+// One matrix (no experts) with too few row groups to fill the chip: blockIdx.y = which sb_per_split super-blocks of
+// k the work group walks; it stores its sums to partial[blockIdx.y][token][row] and gemm_skinny_reduce adds the
+// splits in index order.
 // LDS: [A operands | fp32 token scales | P] of a chunk, then per wave [weight strip | dsc table | zero-point table].
 // Waves per SIMD the shape is meant to run at: two work groups on a compute unit where their LDS allows it.
 template <class F, int NT, int WAVES, int TT, int PER>
@@ -123,7 +126,8 @@ __attribute__((amdgpu_waves_per_eu(skinny_waves_per_simd<F, NT, WAVES, TT, PER>(
 void gemm_skinny_kernel(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,
     const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m, uint32_t mpad,
-    uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride) {
+    uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
+    float *__restrict__ partial, uint32_t sb_per_split) {
     using S = Skinny<F>;
     constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: as_float(0x4B400000 + i) == MAGIC + i for |i| < 2^22
     constexpr uint32_t RS = S::ROW_STRIDE, SEG = 2 * S::BLOCK, PPR = SEG / 16;  // 16-byte pieces per row per step
@@ -142,7 +146,9 @@ void gemm_skinny_kernel(
     // takes further work groups per row group (each its own pass over the weights); the rest exit here
     const uint32_t tokb = tok0 + blockIdx.z * (16 * TT);
     if (tokb >= tok_end) return;  // the whole work group
-    const uint32_t n_super = k / 256;
+    // super-blocks [sb_lo, n_super) of this work group (all of k, or its split)
+    const uint32_t sb_lo = partial ? blockIdx.y * sb_per_split : 0;
+    const uint32_t n_super = partial ? min(k / 256, sb_lo + sb_per_split) : k / 256;
     constexpr uint32_t per = PER, nblk_max = PER * 8;  // sub-blocks (Q8_0 blocks per token) of a full chunk
     uint8_t *const ldsA = lds;
     float *const ldsD = reinterpret_cast<float *>(ldsA + (size_t)nblk_max * TT * 512);
@@ -219,10 +225,10 @@ void gemm_skinny_kernel(
                  : "=v"(magic[0]), "=v"(magic[1]), "=v"(magic[2]), "=v"(magic[3]));
     u32x4 stage[NL];
 #pragma unroll
-    for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i]);
+    for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i] + (size_t)(sb_lo / 2) * SEG);
     const uint32_t steps = n_super / 2;
-    load_tokens(0, min(per, n_super) * 8);
-    for (uint32_t sb0 = 0; sb0 < n_super; sb0 += per) {
+    load_tokens(sb_lo, min(per, n_super - sb_lo) * 8);
+    for (uint32_t sb0 = sb_lo; sb0 < n_super; sb0 += per) {
     const uint32_t nsbc = min(per, n_super - sb0);
     __syncthreads();  // every wave is done with the last chunk's tokens
     store_tokens(nsbc * 8);
@@ -335,16 +341,50 @@ void gemm_skinny_kernel(
             for (int v = 0; v < 4; v++) {
                 const uint32_t tok = tokb + 16 * t + 4 * q + v;
                 if (row < n && tok < tok_end && t < (int)tiles_here) {
-                    float *o = out + (size_t)tok * n + row;
                     const float y = acc[t][j][v];
-                    *o = accumulate ? *o + y : bias ? y + bias[row] : y;
+                    if (partial) {
+                        partial[((size_t)blockIdx.y * m + tok) * n + row] = y;
+                    } else {
+                        float *o = out + (size_t)tok * n + row;
+                        *o = accumulate ? *o + y : bias ? y + bias[row] : y;
+                    }
                 }
             }
         }
 }
 
+// out[i] (+)= partial[0][i] + partial[1][i] + ... in that order, i over m x n; bias[row] instead of the old value
+// when the call overwrites.
+static __global__ __launch_bounds__(256) void gemm_skinny_reduce(const float *__restrict__ partial, float *__restrict__ out,
+                                                         const float *__restrict__ bias, size_t total, uint32_t n,
+                                                         uint32_t splits, int accumulate) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float y = partial[i];
+    for (uint32_t s = 1; s < splits; s++) y += partial[(size_t)s * total + i];
+    out[i] = accumulate ? out[i] + y : bias ? y + bias[i % n] : y;
+}
+
+// Super-blocks per split of k for one matrix of n rows (0: no split): enough splits for about 1.75 work groups of 128
+// rows per compute unit of a 256-CU part, at least two steps (four super-blocks) each, at most 16.  A function of the
+// shape alone, so that the workspace size is.
+static inline uint32_t skinny_sb_per_split(uint32_t n, uint32_t k) {
+    const uint32_t n_super = k / 256, groups = (n + 127) / 128;
+    // below 2^25 weights the three launches (token re-layout, this kernel, the reduction) cost more than they save
+    if (k % 512 != 0 || groups >= 448 || (uint64_t)n * k < (1ull << 25)) return 0;
+    uint32_t splits = (448 + groups - 1) / groups;
+    if (splits > 16) splits = 16;
+    if (splits > n_super / 4) splits = n_super / 4;
+    if (splits < 2) return 0;
+    return ((n_super + splits - 1) / splits + 1) & ~1u;
+}
+static inline uint32_t skinny_splits(uint32_t n, uint32_t k) {
+    const uint32_t per = skinny_sb_per_split(n, k);
+    return per ? (k / 256 + per - 1) / per : 1;
+}
+
 template <class F, int NT, int WAVES, int TT, int PER, bool DUMP = false>
-static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
+static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipStream_t stream, bool split_k = false) {
     using S = Skinny<F>;
     const size_t strips = (size_t)WAVES * NT * 16 * (S::ROW_STRIDE + SKINNY_FAC_STRIDE * 4 * (S::HAS_MIN ? 2 : 1));
     auto kern = &gemm_skinny_kernel<F, NT, WAVES, TT, PER, DUMP>;
@@ -354,12 +394,20 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
     if (e != hipSuccess) return e;
     // token passes: as many as the largest group can need (max_rows is the caller's bound, all rows if unknown)
     const uint32_t group_rows = a.offsets ? a.max_rows : a.m;
-    const dim3 grid((a.n + 16 * NT * WAVES - 1) / (16 * NT * WAVES), a.offsets ? a.n_experts : 1,
+    const uint32_t splits = split_k ? skinny_splits(a.n, a.k) : 1;
+    float *const partial = splits > 1 ? p.partial : nullptr;
+    if (splits > 1 && (a.offsets || !partial)) return hipErrorNotSupported;
+    const dim3 grid((a.n + 16 * NT * WAVES - 1) / (16 * NT * WAVES), a.offsets ? a.n_experts : splits,
                     (group_rows + 16 * TT - 1) / (16 * TT));
     if (grid.z > 65535) return hipErrorNotSupported;
     note_launch("gemm_skinny_kernel", F::TYPE, NT, WAVES, TT, PER, grid.x, grid.y * grid.z, 64 * WAVES);
     hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES), lds, stream, a.W, p.q8t, p.P, p.da16, a.out, a.sums, a.m, p.mpad, a.n, a.k,
-                       a.accumulate, a.bias, a.offsets, a.w_stride);
+                       a.accumulate, a.bias, a.offsets, a.w_stride, partial, skinny_sb_per_split(a.n, a.k));
+    e = hipGetLastError();
+    if (e != hipSuccess || !partial) return e;
+    const size_t total = (size_t)a.m * a.n;
+    hipLaunchKernelGGL(gemm_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, partial, a.out, a.bias,
+                       total, a.n, splits, a.accumulate);
     return hipGetLastError();
 }
 
@@ -370,7 +418,10 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 //  * 17..32 rows: two token tiles double the arithmetic per weight byte.  With a mean of 12 rows (most experts still
 //    one tile) 14336 x 4096 takes 88 us against 102; with a mean of 16 it is 98-107 against 101-106, no gain, and
 //    4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106;
-//  * one matrix, no experts: too few row groups for this shape (14336 x 4096, 16 tokens: 24 us against 19).
+//  * one matrix, no experts, up to 16 token rows: too few row groups as it is (14336 x 4096: 24 us against 19);
+//    with k split over work groups and the splits added by a second launch (call totals, with the token re-layout):
+//    14336 x 4096 18.0 us against 19.6, 4096 x 14336 21.4 against 29.5, 28672 x 8192 40 against 49; 4096 x 4096
+//    14.4 against 12.3 (not taken below 2^25 weights); 17..32 rows 24.6 against 19.7 (not taken).
 template <class F>
 static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_t stream, uint32_t rows, int variant) {
     if constexpr (Skinny<F>::OK) {
@@ -381,7 +432,12 @@ static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_
         if (a.sums && variant != 0 && variant != 200) return hipErrorNotSupported;
         switch (variant) {
         case 0: {
-            if (!a.offsets) return hipErrorNotSupported;
+            if (!a.offsets) {
+                // one matrix: up to 16 token rows, k split over work groups (the workspace has room for the sums)
+                if (two || !p.partial || skinny_splits(a.n, a.k) < 2) return hipErrorNotSupported;
+                if (a.sums) return launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream, true);
+                return launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream, true);
+            }
             const bool many = (size_t)((a.n + 127) / 128) * a.n_experts >= 2 * (size_t)device_cus();
             // two token tiles: only with many row groups and a mean of at most 12 rows per expert
             if (two && (!many || 4 * (size_t)a.m > 3 * 16 * (size_t)a.n_experts)) return hipErrorNotSupported;

@@ -737,6 +737,7 @@ struct TilePlan {
     const float *P;
     const uint16_t *da16;
     uint32_t mpad;
+    float *partial = nullptr;  // room for the few-token kernel's per-split sums (one matrix, k split), or null
 };
 // The formats instantiated in the second translation unit, and the activation byte order they need.
 hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream);

@@ -140,6 +140,8 @@ struct GemmArgs {
     float *out;         // [m x n] row-major
     int32_t *sums;      // optional debug dump [m][n][k/32]
     uint8_t *workspace; // gemm_workspace_bytes(m, k) bytes, 256-byte aligned; null: row-by-row matvecs
+    size_t workspace_bytes = 0;  // what the workspace really holds, if known: gemm_workspace_bytes(m, k, n, type)
+                                 // bytes leave room for the few-token kernel's split-k sums
     bool by_rows = false;  // plain matmul: take the GEMV launches even though a workspace is there (the caller's
                            // snapshot of gemm_uses_tiles, so that one call reads the tuning knobs once)
     uint32_t m, n, k;   // m = all token rows (of all experts in the grouped form)
@@ -157,7 +159,9 @@ struct GemmArgs {
 };
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
 // Device scratch the tile kernel needs for m tokens of k columns (activation re-layout).
-size_t gemm_workspace_bytes(uint32_t m, uint32_t k);
+// With n and the format: plus, for a matmul of at most 32 token rows that the few-token kernel would split over k,
+// the room for its per-split sums (behind the re-tiled activations, 256-byte aligned).
+size_t gemm_workspace_bytes(uint32_t m, uint32_t k, uint32_t n = 0, uint32_t type = 0);
 // Tuning knobs (oxq_tuning.h), read once per call.
 extern std::atomic<int> g_gemm_variant;              // 0 = default tile shape
 extern std::atomic<uint32_t> g_gemm_tile_min_rows;   // 0 = default threshold

@@ -154,3 +154,54 @@ def test_skinny_full_size_c5_gate(hip, ref):
             e = int(np.searchsorted(offsets, r, side="right") - 1)
             assert_close(y[r], canonical_ref(ref, t, w[e], acts[r], n, k_, threads=16), f"c5 gate row {r} expert {e}")
         del dy
+
+
+@pytest.mark.parametrize("t", FORMATS, ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("shape", [(16, 4096, 8192), (9, 8200, 4096), (6, 16384, 2048), (13, 2100, 16384), (11, 16384, 3584)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_skinny_one_matrix_split_k(hip, ref, t, shape):
+    """One matrix, up to 16 token rows, at least 2^25 weights: k is split over work groups, each writes its sums for its
+    part of k, a second launch adds the parts in index order.  Integer sums ==, fp32 1e-5, bias, accumulate, ragged n,
+    splits of unequal length."""
+    import torch
+    from oxillama_amd import linear
+    m, n, k_ = shape
+    say("skinny split-k", O.NAMES[t], shape)
+    w = synth.weights(t, 71, n, k_)
+    acts = ref.quantize_q8_0(synth.normal_f32(72 + m, m * k_)).reshape(m, k_ // 32 * 34)
+    bias = synth.normal_f32(73, n)
+    kern = hip.HipKernel(t)
+    dw, da, db = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda(), torch.from_numpy(bias).cuda()
+    ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
+    dy = torch.full((m + 1, n), 7.0, dtype=torch.float32, device="cuda")
+    dsum = torch.full((m, n, k_ // 32), -1, dtype=torch.int32, device="cuda")
+    kern.gemm_block_sums_dev(dw, da, dy, dsum, m, n, k_, workspace=ws)
+    torch.cuda.synchronize()
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    y, s = dy.cpu().numpy(), dsum.cpu().numpy()
+    assert np.all(y[m:] == 7.0)
+    rows = sorted(set([0, m - 1, m // 2]))
+    y_ref = {r: canonical_ref(ref, t, w, acts[r], n, k_, threads=16) for r in rows}
+    for r in rows:
+        assert_close(y[r], y_ref[r], f"split-k {shape} row {r}")
+        assert np.array_equal(s[r], ref.block_sums(t, w, acts[r], n, k_)), f"integer sums of row {r}"
+    # production launch: the same bits; accumulate: twice them; bias in the reduction
+    dy2 = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    kern.gemm_q8_dev(dw, da, dy2, m, n, k_, workspace=ws)
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    kern.gemm_q8_dev(dw, da, dy2, m, n, k_, accumulate=True, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(dy2, dy[:m] + dy[:m])
+    dy3 = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    linear.linear_forward_batch_dev(t, dw, da, dy3, m, n, k_, d_bias=db, workspace=ws)
+    torch.cuda.synchronize()
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    assert torch.equal(dy3, dy[:m] + db[None, :])
+    # a workspace of the re-tiled activations' size alone, without room for the per-split sums, is refused
+    from oxillama_amd import capi
+    planes = ((k_ // 32) * (((m + 127) // 128) * 128 + 128) * 46 + 255) // 256 * 256
+    dy4 = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    small = ws[:planes]
+    st = capi.load().oxq_gemm_q8_dev(t, dw.data_ptr(), da.data_ptr(), dy4.data_ptr(), m, n, k_, 0, small.data_ptr(),
+                                     small.numel(), None)
+    assert st == capi.ERR_BUFFER_TOO_SMALL

@@ -43,11 +43,13 @@ def _case(hip, ref, t, m, n, k_, seed):
 
 def test_static_scratch_matmul_equals_workspace_matmul_twice_in_a_row(hip, ref):
     lib = capi.load()
-    assert lib.oxq_gemm_q8_static_max_workspace_bytes() == 8 << 20
+    assert lib.oxq_gemm_q8_static_max_workspace_bytes() == 16 << 20
     # a larger call first, then smaller ones on the same array (stale bytes of the first call lie behind them),
-    # then one below the tile kernel's row threshold (GEMV launches, no workspace at all)
+    # then one below the tile kernel's row threshold (GEMV launches, no workspace at all), then a few-token
+    # shape whose k is split over work groups (per-split sums in the array too) and a small one after it
     for t, m, n, k_, seed in ((O.Q4_K, 200, 257, 2048, 31), (O.Q4_K, 40, 100, 512, 33), (O.IQ4_XS, 130, 129, 1024, 35),
-                              (O.Q6_K, 33, 64, 768, 37), (O.Q8_0, 16, 96, 256, 39), (O.Q4_K, 3, 64, 512, 41)):
+                              (O.Q6_K, 33, 64, 768, 37), (O.Q8_0, 16, 96, 256, 39), (O.Q4_K, 3, 64, 512, 41),
+                              (O.Q4_K, 12, 4096, 8192, 43), (O.IQ4_XS, 16, 200, 1024, 45)):
         say(O.NAMES[t], m, n, k_)
         _case(hip, ref, t, m, n, k_, seed)
 
@@ -59,11 +61,11 @@ def test_static_scratch_limits(hip, ref):
     # 4096 tokens of 4096 columns need 25 MB of workspace: refused, with the sizes, before anything is launched
     m, n, k_ = 4096, 64, 4096
     need = hip.HipKernel(t).gemm_workspace_bytes(m, n, k_)
-    assert need > 8 << 20
+    assert need > 16 << 20
     d = torch.zeros(16, dtype=torch.uint8, device="cuda")
     with pytest.raises(quant.BufferTooSmall) as e:
         hip.HipKernel(t).gemm_q8_static_dev(d, d, d, m, n, k_)
-    assert (e.value.needed, e.value.available) == (need, 8 << 20)
+    assert (e.value.needed, e.value.available) == (need, 16 << 20)
     # the shape checks of oxq_gemm_q8_dev come first
     assert lib.oxq_gemm_q8_static_dev(15, d.data_ptr(), d.data_ptr(), d.data_ptr(), 8, 64, 256, 0, None) == \
         capi.ERR_UNSUPPORTED_TYPE
