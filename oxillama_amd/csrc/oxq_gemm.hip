@@ -116,9 +116,23 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
     if (!a.offsets && gemm_partial_bytes(type, a.m, a.n, a.k) &&
         a.workspace_bytes >= gemm_workspace_bytes(a.m, a.k, a.n, type))
         plan.partial = reinterpret_cast<float *>(a.workspace + ((gemm_planes_bytes(a.m, a.k) + 255) & ~(size_t)255));
+    // The few-token kernel (oxq_gemm_skinny.hpp), where it pays: it reads the caller's Q8_0 rows itself, no re-layout.
+    const int variant = g_gemm_variant.load(std::memory_order_relaxed);
+    const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
+    auto skinny_of = [&](uint32_t t) {
+        return t == OXQ_TYPE_Q4_K     ? skinny_shape<TileQ4K>(a, plan.partial != nullptr, rows, variant)
+               : t == OXQ_TYPE_IQ4_XS ? skinny_shape<TileIQ4XS>(a, plan.partial != nullptr, rows, variant)
+                                      : (int)SK_NONE;
+    };
+    if (const int shape = skinny_of(type)) {
+        const hipError_t e = type == OXQ_TYPE_Q4_K ? launch_skinny<TileQ4K>(a, plan, stream, shape)
+                                                   : launch_skinny<TileIQ4XS>(a, plan, stream, shape);
+        if (e != hipErrorNotSupported) return e;
+    }
     // the previous call left the same activations in the same byte order (and the half-block planes if this
-    // format needs them): go straight to the tile kernel
-    const bool prepared = a.prepared_for != 0 && act_perm(a.prepared_for) == perm &&
+    // format needs them) -- unless it was served by the few-token kernel, which prepares nothing: go straight to
+    // the tile kernel
+    const bool prepared = a.prepared_for != 0 && act_perm(a.prepared_for) == perm && !skinny_of(a.prepared_for) &&
                           (!tile_needs_p16_more(type) || tile_needs_p16_more(a.prepared_for));
     if (!prepared) {
         // formats with a 16-weight zero-point term also need P per half block

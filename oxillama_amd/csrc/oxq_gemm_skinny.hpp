@@ -9,10 +9,9 @@
 //    consecutive 16-byte pieces of a row's two next super-blocks -- into registers, one step ahead, and from there
 //    into a private strip of LDS; the lanes then pick their B operands out of LDS in the matrix core's layout.  No
 //    barrier: the strip belongs to one wave, whose LDS operations execute in order.
-//  * Tokens: the work group copies the Q8_0 bytes, scales and block sums of its (at most 32) tokens for the whole
-//    k chunk into LDS once, already in operand order; all waves read them from there.  Rows of k that do not fit
-//    beside the weight strips are taken in chunks, one launch per chunk, each adding to the last one's output in a
-//    fixed order.
+//  * Tokens: the work group copies the Q8_0 bytes, scales and block sums of its (at most 32) tokens for a chunk of
+//    k into LDS, already in operand order (straight from the caller's Q8_0 rows: no re-layout launch); all waves
+//    read them from there.
 //  * v_mfma_i32_16x16x32_i8 with the tokens as the A operand (16 tokens x 32 k) and the weights as B (32 k x 16
 //    rows): lane l = (c = l % 16, q = l / 16) supplies k-values 8q..8q+7 of token c and of weight row c and
 //    receives the sums of row c against tokens 4q..4q+3.  All of a lane's results belong to the one weight row
@@ -38,6 +37,7 @@ struct Skinny<TileQ4K> {
     static constexpr bool OK = true;
     static constexpr uint32_t BLOCK = 144, ROW_STRIDE = 304;  // LDS bytes per row of a step (2 blocks + pad)
     static constexpr bool HAS_MIN = true;
+    static constexpr int ACT_PERM = 0;
     struct Raw {
         u32x4 hdr;
         u32x2 qs[4];
@@ -74,6 +74,7 @@ struct Skinny<TileIQ4XS> {
     // 272 bytes = 68 dwords per row: lane (c, q) reads dword 68 c + q + const, bank 4 c + q -- all 64 distinct
     static constexpr uint32_t BLOCK = 136, ROW_STRIDE = 272;
     static constexpr bool HAS_MIN = false;
+    static constexpr int ACT_PERM = 1;
     struct Raw {
         u32x2 hdr;
         uint32_t qs[8];
@@ -124,9 +125,8 @@ template <class F, int NT, int WAVES, int TT, int PER, bool DUMP>
 __global__ __launch_bounds__(64 * WAVES)
 __attribute__((amdgpu_waves_per_eu(skinny_waves_per_simd<F, NT, WAVES, TT, PER>(), skinny_waves_per_simd<F, NT, WAVES, TT, PER>())))
 void gemm_skinny_kernel(
-    const uint8_t *__restrict__ W, const uint8_t *__restrict__ q8t, const float *__restrict__ P,
-    const uint16_t *__restrict__ da16, float *__restrict__ out, int32_t *__restrict__ sums, uint32_t m, uint32_t mpad,
-    uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
+    const uint8_t *__restrict__ W, const uint8_t *__restrict__ A, float *__restrict__ out, int32_t *__restrict__ sums,
+    uint32_t m, uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
     float *__restrict__ partial, uint32_t sb_per_split) {
     using S = Skinny<F>;
     constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: as_float(0x4B400000 + i) == MAGIC + i for |i| < 2^22
@@ -157,44 +157,53 @@ void gemm_skinny_kernel(
     float *const dscT = reinterpret_cast<float *>(strip + NT * 16 * RS);
     float *const minT = dscT + NT * 16 * FS;
 
-    // ---- a chunk's tokens: from the workspace into registers (requested a chunk ahead, in flight while the last
-    // chunk is computed), from there into LDS in operand order.  Token rows past the group's end: whatever the
-    // padded workspace holds there; their results are never stored. ----
-    constexpr uint32_t KA = (nblk_max * TT * 64 + THREADS - 1) / THREADS, KS = (nblk_max * TT * 16 + THREADS - 1) / THREADS;
+    // ---- a chunk's tokens: their Q8_0 blocks (34 bytes: f16 scale, 32 int8) from the caller's rows into registers
+    // (requested a chunk ahead, in flight while the last chunk is computed), from there into LDS in operand order,
+    // with what gemm_prep_acts would have made of them: the bytes of each 8 in the format's order, the scale as
+    // fp32, P = d * sum(q) (exact integer sum, one rounding).  Thread (cc, qq) of a 64-thread unit takes bytes
+    // 8 qq .. 8 qq + 7 of token cc's block; token rows past the group's end read as zeros. ----
+    constexpr uint32_t KA = (nblk_max * TT * 64 + THREADS - 1) / THREADS;
+    const size_t arow = (size_t)(k / 32) * Q8_BLOCK_BYTES;
     u32x2 tokA[KA];
-    uint32_t tokD[KS];
-    float tokP[KS];
+    uint32_t tokD[KA];
     auto load_tokens = [&](uint32_t sb0, uint32_t nblk) {
-        const uint32_t total = nblk * TT * 64, total_s = nblk * TT * 16;
+        const uint32_t total = nblk * TT * 64;
 #pragma unroll
         for (uint32_t i = 0; i < KA; i++) {
-            const uint32_t idx = min(threadIdx.x + i * THREADS, total - 1);
+            const uint32_t idx = threadIdx.x + i * THREADS;
             const uint32_t l = idx & 63, t = (idx >> 6) % TT, b = (idx >> 6) / TT;
-            const uint32_t cc = l >> 2, qq = l & 3;  // consecutive threads: consecutive 8 bytes of a token's block
-            tokA[i] = ld8(q8t + ((size_t)(sb0 * 8 + b) * mpad + tokb + 16 * t + cc) * 32 + 8 * qq);
-        }
-#pragma unroll
-        for (uint32_t i = 0; i < KS; i++) {
-            const uint32_t idx = min(threadIdx.x + i * THREADS, total_s - 1);
-            const uint32_t cc = idx & 15, t = (idx >> 4) % TT, b = (idx >> 4) / TT;
-            const size_t src = (size_t)(sb0 * 8 + b) * mpad + tokb + 16 * t + cc;
-            tokD[i] = da16[src];
-            tokP[i] = S::HAS_MIN ? P[src] : 0.0f;
+            const uint32_t cc = l >> 2, qq = l & 3, tok = tokb + 16 * t + cc;
+            tokA[i] = u32x2{0, 0};
+            tokD[i] = 0;
+            if (idx < total && tok < tok_end) {
+                const uint8_t *blk = A + (size_t)tok * arow + (size_t)(sb0 * 8 + b) * Q8_BLOCK_BYTES;
+                tokA[i] = ld8(blk + 2 + 8 * qq);
+                tokD[i] = ld2(blk);
+            }
         }
     };
     auto store_tokens = [&](uint32_t nblk) {
-        const uint32_t total = nblk * TT * 64, total_s = nblk * TT * 16;
+        const uint32_t total = nblk * TT * 64;
 #pragma unroll
         for (uint32_t i = 0; i < KA; i++) {
-            const uint32_t idx = min(threadIdx.x + i * THREADS, total - 1);
+            const uint32_t idx = threadIdx.x + i * THREADS;
+            if (idx >= total) continue;  // whole waves: total and THREADS are multiples of 64
             const uint32_t l = idx & 63, cc = l >> 2, qq = l & 3;
-            *reinterpret_cast<u32x2 *>(ldsA + ((size_t)(idx >> 6) * 64 + qq * 16 + cc) * 8) = tokA[i];
-        }
-#pragma unroll
-        for (uint32_t i = 0; i < KS; i++) {
-            const uint32_t idx = min(threadIdx.x + i * THREADS, total_s - 1);
-            ldsD[idx] = h2f(tokD[i]);
-            if (S::HAS_MIN) ldsP[idx] = tokP[i];
+            u32x2 v = tokA[i];
+            const float d = h2f(tokD[i]);
+            if (S::HAS_MIN) {
+                int sum = sdot4(v[0], 0x01010101u, sdot4(v[1], 0x01010101u, 0));
+                sum += xor1_i(sum);  // the four threads of a block
+                sum += xor2_i(sum);
+                if (qq == 0) ldsP[(idx >> 6) * 16 + cc] = d * (float)sum;
+            }
+            if (S::ACT_PERM == 1) {  // even bytes, then odd bytes
+                const uint32_t x0 = v[0], x1 = v[1];
+                v[0] = __builtin_amdgcn_perm(x1, x0, 0x06040200u);
+                v[1] = __builtin_amdgcn_perm(x1, x0, 0x07050301u);
+            }
+            *reinterpret_cast<u32x2 *>(ldsA + ((size_t)(idx >> 6) * 64 + qq * 16 + cc) * 8) = v;
+            if (qq == 0) ldsD[(idx >> 6) * 16 + cc] = d;
         }
     };
 
@@ -401,7 +410,7 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
                     (group_rows + 16 * TT - 1) / (16 * TT));
     if (grid.z > 65535) return hipErrorNotSupported;
     note_launch("gemm_skinny_kernel", F::TYPE, NT, WAVES, TT, PER, grid.x, grid.y * grid.z, 64 * WAVES);
-    hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES), lds, stream, a.W, p.q8t, p.P, p.da16, a.out, a.sums, a.m, p.mpad, a.n, a.k,
+    hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES), lds, stream, a.W, a.A, a.out, a.sums, a.m, a.n, a.k,
                        a.accumulate, a.bias, a.offsets, a.w_stride, partial, skinny_sb_per_split(a.n, a.k));
     e = hipGetLastError();
     if (e != hipSuccess || !partial) return e;
@@ -411,8 +420,9 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
     return hipGetLastError();
 }
 
-// hipErrorNotSupported: not this format / shape, or one the tile kernel serves better.  rows = the token rows per
-// group the launch is shaped for.  variant 0: the measured choice; 200..205: a fixed shape (tuning, tests).
+// Which launch shape serves a call: 0 = none (not this format / shape, or one the tile kernel serves better).  rows =
+// the token rows per group the launch is shaped for; has_partial: the workspace has room for split-k sums.
+// variant 0: the measured choice; 200..205: a fixed shape (tuning, tests).
 // Measured on MI355X, 8 experts of Mixtral's shapes (IQ4_XS; Q4_K alike), cold weights, against the tile kernel:
 //  * up to 16 rows per expert: 14336 x 4096 84 us against 106, 4096 x 14336 90 against 107;
 //  * 17..32 rows: two token tiles double the arithmetic per weight byte.  With a mean of 12 rows (most experts still
@@ -422,38 +432,52 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 //    with k split over work groups and the splits added by a second launch (call totals, with the token re-layout):
 //    14336 x 4096 18.0 us against 19.6, 4096 x 14336 21.4 against 29.5, 28672 x 8192 40 against 49; 4096 x 4096
 //    14.4 against 12.3 (not taken below 2^25 weights); 17..32 rows 24.6 against 19.7 (not taken).
+enum SkinnyShape { SK_NONE = 0, SK_1_4, SK_1_8, SK_2_2, SK_1_4_SPLIT, SK_1_16, SK_2_8, SK_W4_1_8, SK_W4_2_4, SK_2_4 };
+
 template <class F>
-static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_t stream, uint32_t rows, int variant) {
+static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int variant) {
     if constexpr (Skinny<F>::OK) {
         // whole steps of two super-blocks
-        if (a.k % 512 != 0 || rows > 32) return hipErrorNotSupported;
+        if (a.k % 512 != 0 || rows > 32) return SK_NONE;
         const bool two = rows > 16;
-        // <NT, WAVES, TT, PER>; LDS = PER * 8 * TT * 640 + WAVES * NT * 7 KB
-        if (a.sums && variant != 0 && variant != 200) return hipErrorNotSupported;
+        if (a.sums && variant != 0 && variant != 200) return SK_NONE;  // the dump exists for the default shapes
         switch (variant) {
         case 0: {
-            if (!a.offsets) {
-                // one matrix: up to 16 token rows, k split over work groups (the workspace has room for the sums)
-                if (two || !p.partial || skinny_splits(a.n, a.k) < 2) return hipErrorNotSupported;
-                if (a.sums) return launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream, true);
-                return launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream, true);
-            }
+            if (!a.offsets)  // one matrix: up to 16 token rows, k split over work groups (the workspace has room for the sums)
+                return (!two && has_partial && skinny_splits(a.n, a.k) >= 2) ? SK_1_4_SPLIT : SK_NONE;
             const bool many = (size_t)((a.n + 127) / 128) * a.n_experts >= 2 * (size_t)device_cus();
             // two token tiles: only with many row groups and a mean of at most 12 rows per expert
-            if (two && (!many || 4 * (size_t)a.m > 3 * 16 * (size_t)a.n_experts)) return hipErrorNotSupported;
-            // debug dump: one shape per token-tile count (every shape adds a result's terms in the same order)
-            if (a.sums) return two ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream);
-            if (two) return launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream);
-            return many ? launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 8>(a, p, stream);
+            if (two) return (many && 4 * (size_t)a.m <= 3 * 16 * (size_t)a.n_experts) ? SK_2_2 : SK_NONE;
+            // (the debug dump: one shape per token-tile count; every shape adds a result's terms in the same order)
+            return (many || a.sums) ? SK_1_4 : SK_1_8;
         }
-        case 200:
-            if (a.sums) return two ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream);
-            return two ? launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream);
-        case 201: return two ? launch_skinny_shape<F, 1, 8, 2, 8>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 16>(a, p, stream);
-        case 203: return two ? launch_skinny_shape<F, 1, 4, 2, 4>(a, p, stream) : launch_skinny_shape<F, 1, 4, 1, 8>(a, p, stream);
-        case 204: return two ? launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream);
-        case 205: return two ? launch_skinny_shape<F, 1, 8, 2, 4>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 8>(a, p, stream);
-        default: return hipErrorNotSupported;
+        case 200: return two ? SK_2_2 : SK_1_4;
+        case 201: return two ? SK_2_8 : SK_1_16;
+        case 203: return two ? SK_W4_2_4 : SK_W4_1_8;
+        case 204: return two ? SK_2_2 : SK_1_4;
+        case 205: return two ? SK_2_4 : SK_1_8;
+        default: return SK_NONE;
+        }
+    }
+    return SK_NONE;
+}
+
+// <NT, WAVES, TT, PER>; LDS = PER * 8 * TT * 640 + WAVES * NT * 7 KB
+template <class F>
+static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_t stream, int shape) {
+    if constexpr (Skinny<F>::OK) {
+        switch (shape) {
+        case SK_1_4: return a.sums ? launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream);
+        case SK_2_2: return a.sums ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream);
+        case SK_1_4_SPLIT:
+            return a.sums ? launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream, true) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream, true);
+        case SK_1_8: return launch_skinny_shape<F, 1, 8, 1, 8>(a, p, stream);
+        case SK_1_16: return launch_skinny_shape<F, 1, 8, 1, 16>(a, p, stream);
+        case SK_2_8: return launch_skinny_shape<F, 1, 8, 2, 8>(a, p, stream);
+        case SK_2_4: return launch_skinny_shape<F, 1, 8, 2, 4>(a, p, stream);
+        case SK_W4_1_8: return launch_skinny_shape<F, 1, 4, 1, 8>(a, p, stream);
+        case SK_W4_2_4: return launch_skinny_shape<F, 1, 4, 2, 4>(a, p, stream);
+        default: break;
         }
     }
     return hipErrorNotSupported;

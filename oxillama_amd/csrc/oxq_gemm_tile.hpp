@@ -766,8 +766,6 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
 
 template <class F>
 static hipError_t launch_streamed(const GemmArgs &a, const TilePlan &p, hipStream_t stream, uint32_t rows, int variant);
-template <class F>
-static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_t stream, uint32_t rows, int variant);
 
 // Tile shape by use: many tokens (prefill) take 128-token work-group tiles; few tokens (a
 // mixture-of-experts group, a short prompt, a decode batch) take 32-token tiles with the
@@ -776,10 +774,7 @@ template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
     const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
     const int variant = g_gemm_variant.load(std::memory_order_relaxed);
-    if (variant == 0 || (variant >= 200 && variant < 300)) {  // the few-token kernel (oxq_gemm_skinny.hpp), where it pays
-        const hipError_t e = launch_skinny<F>(a, p, stream, rows, variant);
-        if (e != hipErrorNotSupported) return e;
-    } else if (variant >= 100) {  // the streamed kernel (opt-in: oxq_gemm_stream.hpp says why), where the format and shape allow it
+    if (variant >= 100 && variant < 200) {  // the streamed kernel (opt-in: oxq_gemm_stream.hpp says why), where the format and shape allow it
         const hipError_t e = launch_streamed<F>(a, p, stream, rows, variant);
         if (e != hipErrorNotSupported) return e;
     }
