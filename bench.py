@@ -543,6 +543,36 @@ def main():
         kernels["f32_route_q8_0_q_proj_4096x4096"] = time_f32(k_q8, Q8_0, [w["q"] for w in layers], x, yq, H, H)
         kernels["f32_route_c1_q4_0_4096x4096"] = time_f32(k_q40, Q4_0, c1, x, yq, H, H)
         del c1
+        # a decode batch of 16 token rows on the Q4_K FFN shapes (oxq_gemm_q8_dev: the few-token kernel with k split
+        # over work groups, then the reduction launch), over the layers' distinct weights
+        def time_batch(kern, t, mats, m, n_rows, n_cols):
+            xb = torch.from_numpy(synth.normal_f32(11, m * n_cols)).to(dev)
+            xbq = torch.empty(m * (n_cols // 32 * 34), dtype=torch.uint8, device=dev)
+            quant.quantize_q8_0_dev(xb, xbq)
+            yb = torch.zeros(m * n_rows, dtype=torch.float32, device=dev)
+            wsb = torch.empty(max(kern.gemm_workspace_bytes(m, n_rows, n_cols), 256), dtype=torch.uint8, device=dev)
+            n = max(len(mats), 32)
+
+            def body():
+                for i in range(n):
+                    kern.gemm_q8_dev(mats[i % len(mats)], xbq, yb, m, n_rows, n_cols, workspace=wsb)
+            g = capture(body)
+            timed_replay(g)
+            us = min(timed_replay(g) for _ in range(3)) * 1e3 / n
+            launch = last_launch()
+            # the same calls on the int8-MFMA tile kernel (tuning knob 99: never the few-token kernel)
+            from oxillama_amd import capi
+            capi.load().oxq_set_gemm_variant(99)
+            g2 = capture(body)
+            timed_replay(g2)
+            tile_us = min(timed_replay(g2) for _ in range(3)) * 1e3 / n
+            capi.load().oxq_set_gemm_variant(0)
+            wb = n_rows * row_bytes(t, n_cols)
+            return {"us_per_call": round(us, 3), "token_rows": m, "launches": n, "distinct_weight_sets": len(mats),
+                    "launch": launch, "weight_GBps": round(wb / us / 1e3, 1),
+                    "frac_hbm_peak": round(wb / us / 1e3 / HBM_PEAK_GBPS, 4), "tile_kernel_us_per_call": round(tile_us, 3)}
+        kernels["batch16_q4k_gate_14336x4096"] = time_batch(k_q4k, Q4_K, [w["gate"] for w in layers], 16, F, H)
+        kernels["batch16_q4k_down_shape_4096x14336"] = time_batch(k_q4k, Q4_K, [w["gate"] for w in layers], 16, H, F)
         V = 128256
         lm = [upload(Q6_K, 6000 + i, V, H) for i in range(2)]
         logits = torch.zeros(V, dtype=torch.float32, device=dev)
