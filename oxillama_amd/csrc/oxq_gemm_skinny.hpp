@@ -363,15 +363,26 @@ void gemm_skinny_kernel(
 }
 
 // out[i] (+)= partial[0][i] + partial[1][i] + ... in that order, i over m x n; bias[row] instead of the old value
-// when the call overwrites.
+// when the call overwrites.  V = 4: four consecutive elements per thread (n a multiple of 4, buffers 16-byte aligned).
+template <int V>
 static __global__ __launch_bounds__(256) void gemm_skinny_reduce(const float *__restrict__ partial, float *__restrict__ out,
-                                                         const float *__restrict__ bias, size_t total, uint32_t n,
-                                                         uint32_t splits, int accumulate) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+                                                                const float *__restrict__ bias, size_t total, uint32_t n,
+                                                                uint32_t splits, int accumulate) {
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * V;
     if (i >= total) return;
-    float y = partial[i];
-    for (uint32_t s = 1; s < splits; s++) y += partial[(size_t)s * total + i];
-    out[i] = accumulate ? out[i] + y : bias ? y + bias[i % n] : y;
+    float y[V];
+    if (V == 4) {
+        const v4f32 p0 = *reinterpret_cast<const v4f32 *>(partial + i);
+        for (int v = 0; v < V; v++) y[v] = p0[v];
+        for (uint32_t s = 1; s < splits; s++) {
+            const v4f32 ps = *reinterpret_cast<const v4f32 *>(partial + (size_t)s * total + i);
+            for (int v = 0; v < V; v++) y[v] += ps[v];
+        }
+    } else {
+        y[0] = partial[i];
+        for (uint32_t s = 1; s < splits; s++) y[0] += partial[(size_t)s * total + i];
+    }
+    for (int v = 0; v < V; v++) out[i + v] = accumulate ? out[i + v] + y[v] : bias ? y[v] + bias[(i + v) % n] : y[v];
 }
 
 // Super-blocks per split of k for one matrix of n rows (0: no split): enough splits for about 1.75 work groups of 128
@@ -415,8 +426,12 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
     e = hipGetLastError();
     if (e != hipSuccess || !partial) return e;
     const size_t total = (size_t)a.m * a.n;
-    hipLaunchKernelGGL(gemm_skinny_reduce, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, partial, a.out, a.bias,
-                       total, a.n, splits, a.accumulate);
+    if (a.n % 4 == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0)
+        hipLaunchKernelGGL(gemm_skinny_reduce<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, partial,
+                           a.out, a.bias, total, a.n, splits, a.accumulate);
+    else
+        hipLaunchKernelGGL(gemm_skinny_reduce<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, partial, a.out,
+                           a.bias, total, a.n, splits, a.accumulate);
     return hipGetLastError();
 }
 

@@ -157,7 +157,7 @@ def test_skinny_full_size_c5_gate(hip, ref):
 
 
 @pytest.mark.parametrize("t", FORMATS, ids=lambda t: O.NAMES[t])
-@pytest.mark.parametrize("shape", [(16, 4096, 8192), (9, 8200, 4096), (6, 16384, 2048), (13, 2100, 16384), (11, 16384, 3584)],
+@pytest.mark.parametrize("shape", [(16, 4096, 8192), (9, 8200, 4096), (6, 16384, 2048), (13, 2100, 16384), (11, 16384, 3584), (7, 8201, 4096)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_skinny_one_matrix_split_k(hip, ref, t, shape):
     """One matrix, up to 16 token rows, at least 2^25 weights: k is split over work groups, each writes its sums for its
