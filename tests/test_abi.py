@@ -157,3 +157,26 @@ def test_moe_forward_argument_errors_before_touching_the_gpu():
     assert lib.oxq_moe_route_dev(None, None, 1, 2000, 4, 1, None, None, None, None, None, None) == capi.ERR_UNSUPPORTED_SHAPE
     assert lib.oxq_moe_ffn_workspace_bytes(t, t, t, 8, 288, 256) == 0  # the grouped kernel walks 256 columns at a time
     assert lib.oxq_moe_ffn_workspace_bytes(t, t, t, 8, 256, 512) > 0
+
+
+def test_gemm_workspace_size_is_a_function_of_the_shape():
+    """oxq_gemm_q8_workspace_bytes: the re-tiled activations (token rows padded to 128 and 128 more, 46 bytes per
+    token block, rounded to 256), plus -- for at most 16 token rows of Q4_K / IQ4_XS on a matrix of at least 2^25
+    weights that yields fewer than 448 groups of 128 rows -- the room for the few-token kernel's per-split sums:
+    splits x m x n floats, splits = min(ceil(448 / groups), k / 1024, 16) taken in even numbers of super-blocks."""
+    lib = capi.load()
+
+    def planes(m, k):
+        return ((k // 32) * ((m + 127) // 128 * 128 + 128) * 46 + 255) // 256 * 256
+
+    q4k, iq4xs, q6k = 12, 23, 14
+    w = lib.oxq_gemm_q8_workspace_bytes
+    assert w(q4k, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4            # 112 groups -> 4 splits of 4
+    assert w(iq4xs, 9, 4096, 14336) == planes(9, 14336) + 14 * 9 * 4096 * 4            # 32 groups -> 14 splits of 4
+    assert w(q4k, 11, 16384, 3584) == planes(11, 3584) + 3 * 11 * 16384 * 4            # 14 super-blocks: 6 + 6 + 2
+    assert w(q4k, 16, 4096, 4096) == planes(16, 4096)                                  # below 2^25 weights
+    assert w(q4k, 17, 14336, 4096) == planes(17, 4096)                                 # more than 16 rows
+    assert w(q6k, 16, 14336, 4096) == planes(16, 4096)                                 # no few-token kernel for Q6_K
+    assert w(q4k, 16, 128256, 4096) == planes(16, 4096)                                # 1002 groups fill the chip
+    assert w(q4k, 512, 14336, 4096) == planes(512, 4096)
+    assert w(q4k, 16, 14336, 4000) == 0                                                # k not a multiple of 256
