@@ -1,4 +1,5 @@
-// Few tokens per weight matrix (a mixture-of-experts group of up to 32 token rows): the batched fused matvec
+// Few tokens per weight matrix (a mixture-of-experts group of up to 32 token rows, a decode batch of up to 16 on one
+// matrix): the batched fused matvec
 //   out[m x n] (+)= A_q8[m rows of Q8_0 blocks] x W[n x k]^T
 // (the reference's gemm loop over matvec_q8_fused, crates/oxillama-quant/src/reference/q4_k.rs:186-201, :218-333)
 // built around what the counters say bounds the tile kernel in this case: not HBM, not the matrix core, but the
@@ -14,10 +15,11 @@
 //    read them from there.
 //  * v_mfma_i32_16x16x32_i8 with the tokens as the A operand (16 tokens x 32 k) and the weights as B (32 k x 16
 //    rows): lane l = (c = l % 16, q = l / 16) supplies k-values 8q..8q+7 of token c and of weight row c and
-//    receives the sums of row c against tokens 4q..4q+3.  All of a lane's results belong to the one weight row
-//    whose block header it reads itself, so the weight-side factors need no exchange.
+//    receives the sums of row c against tokens 4q..4q+3.  All of a lane's results belong to one weight row, so its
+//    weight-side factor is one value per sub-block (decoded once per step by the wave, kept in a small LDS table).
 // Arithmetic per result as in the tile kernel (oxq_gemm_tile.hpp): fl(dsc * isum) by the 1.5 * 2^23 trick, then
-// one fma with the token's scale; the zero-point term one more fma with d_a * sum(q_a).
+// one fma with the token's scale; the zero-point term (Q4_K) as a 16 x 16 x 4 fp32 MFMA per four sub-blocks over
+// P = d_a * sum(q_a) and the rows' -dmin * mn.
 #pragma once
 #include "oxq_gemm_tile.hpp"
 
