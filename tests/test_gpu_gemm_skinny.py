@@ -205,3 +205,25 @@ def test_skinny_one_matrix_split_k(hip, ref, t, shape):
     st = capi.load().oxq_gemm_q8_dev(t, dw.data_ptr(), da.data_ptr(), dy4.data_ptr(), m, n, k_, 0, small.data_ptr(),
                                      small.numel(), None)
     assert st == capi.ERR_BUFFER_TOO_SMALL
+
+
+def test_skinny_split_k_on_the_host_routes(hip, ref):
+    """The routes that size their own scratch -- QuantKernel::gemm on host slices, oxq_gemm_q8_dev without a
+    workspace -- leave room for the per-split sums and take the same kernel."""
+    import torch
+    t, m, n, k_ = O.Q4_K, 8, 8192, 4096
+    w = synth.weights(t, 81, n, k_)
+    x = synth.normal_f32(82, m * k_)
+    acts = ref.quantize_q8_0(x).reshape(m, k_ // 32 * 34)
+    kern = hip.HipKernel(t)
+    y = np.zeros(m * n, dtype=np.float32)
+    kern.gemm(hip.QuantTensor(w, [n, k_], t), x, y, m, n, k_)
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    y = y.reshape(m, n)
+    for r in (0, 3, m - 1):
+        assert_close(y[r], canonical_ref(ref, t, w, acts[r], n, k_, threads=16), f"host gemm row {r}")
+    dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    kern.gemm_q8_dev(torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda(), dy, m, n, k_)  # library-owned scratch
+    torch.cuda.synchronize()
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    assert np.array_equal(dy.cpu().numpy(), y)
