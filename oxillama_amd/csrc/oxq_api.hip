@@ -667,7 +667,8 @@ static int gemm_host(uint32_t type, const uint8_t *data, size_t data_len, const 
     ga.out = (float *)g.s_out.ptr;
     ga.sums = nullptr;
     ga.workspace = nullptr;
-    if (oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n_rows, (uint32_t)n_cols)) {
+    if (oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n_rows, (uint32_t)n_cols) ||
+        oxq::gemm_few_rows_pay(type, (uint32_t)m, (uint32_t)n_rows, (uint32_t)n_cols)) {
         const size_t wbytes = oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)n_cols, (uint32_t)n_rows, type);
         if ((st = g.s_work.reserve(wbytes)) != OXQ_OK) return st;
         ga.workspace = (uint8_t *)g.s_work.ptr;
@@ -895,7 +896,13 @@ static int gemm_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
     ga.accumulate = accumulate ? 1 : 0;
     ga.bias = d_bias;
     // one reading of the tuning knobs per call: tile kernel, or GEMV launches (which need no workspace)
-    const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k);
+    bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k);
+    // a few rows fewer still pay on the few-token kernel, if the caller's workspace has the room (without one the
+    // call would have to take the library's scratch and wait for the stream: the GEMV launches stay)
+    if (!tiles && d_workspace && !d_sums && oxq::gemm_few_rows_pay(type, (uint32_t)m, (uint32_t)n, (uint32_t)k) &&
+        workspace_bytes >= oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k, (uint32_t)n, type) &&
+        (reinterpret_cast<uintptr_t>(d_workspace) & 255) == 0)
+        tiles = true;
     ga.by_rows = !tiles;
     const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k, (uint32_t)n, type) : 0;
     if (need && d_workspace) {
@@ -940,7 +947,9 @@ int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_
         !static_scratch_ptr[g.device])
         return fail(OXQ_ERR_NO_DEVICE, 0, 0, "call oxq_init first: this entry point sets nothing up by itself");
     if (m == 0 || n == 0 || k == 0) return OXQ_OK;
-    const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k);
+    const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k) ||
+                       (oxq::gemm_few_rows_pay(type, (uint32_t)m, (uint32_t)n, (uint32_t)k) &&
+                        oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k, (uint32_t)n, type) <= STATIC_SCRATCH_BYTES);
     const size_t need = tiles ? oxq::gemm_workspace_bytes((uint32_t)m, (uint32_t)k, (uint32_t)n, type) : 0;
     if (need > STATIC_SCRATCH_BYTES)
         return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, STATIC_SCRATCH_BYTES,

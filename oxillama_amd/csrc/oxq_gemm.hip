@@ -95,6 +95,18 @@ bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
     return gemm_tiles_supported(type, m, k) && m >= min_rows;
 }
 
+// Fewer rows than that, on a shape the few-token kernel serves with k split over work groups: it still beats the
+// GEMV launches, whose time grows with every four rows (measured, us, GEMV launches against the few-token kernel:
+// Q4_K 14336 x 4096 4 rows 14.3 / 16.8, 5 rows 20.6 / 16.5; 4096 x 14336 5 rows 20.5 / 19.4, 8 rows 26.7 / 19.6;
+// IQ4_XS 14336 x 4096 2 rows 14.1 / 16.2, 3 rows 23.2 / 16.1, 5 rows 33.2 / 16.2; 4096 x 14336 3 rows 23.3 / 19.5).
+// Only where the caller has a workspace with room for the per-split sums, and with the knobs at their defaults.
+bool gemm_few_rows_pay(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
+    if (g_gemm_tile_min_rows.load(std::memory_order_relaxed) != 0 || g_gemm_variant.load(std::memory_order_relaxed) != 0)
+        return false;
+    return gemm_tiles_supported(type, m, k) && gemm_partial_bytes(type, m, n, k) != 0 &&
+           m >= (type == OXQ_TYPE_IQ4_XS ? 3u : 5u);
+}
+
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) {
     const bool tiles = a.workspace != nullptr && gemm_tiles_supported(type, a.m, a.k) && (a.offsets || !a.by_rows);
     if (!tiles) {

@@ -167,6 +167,9 @@ extern std::atomic<int> g_gemm_variant;              // 0 = default tile shape
 extern std::atomic<uint32_t> g_gemm_tile_min_rows;   // 0 = default threshold
 // True when (type, m, k) is served by the int8-MFMA tile kernel.
 bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k);
+// Below gemm_uses_tiles' row threshold, but the few-token kernel (k split over work groups) still beats the GEMV
+// launches: for callers that hold a workspace of gemm_workspace_bytes(m, k, n, type).
+bool gemm_few_rows_pay(uint32_t type, uint32_t m, uint32_t n, uint32_t k);
 // True when the tile kernel can take (type, m, k) at all (the grouped form always uses it).
 bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k);
 

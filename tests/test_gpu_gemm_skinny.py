@@ -227,3 +227,32 @@ def test_skinny_split_k_on_the_host_routes(hip, ref):
     torch.cuda.synchronize()
     assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
     assert np.array_equal(dy.cpu().numpy(), y)
+
+
+@pytest.mark.parametrize("case", [(O.IQ4_XS, 3, 8192, 4096), (O.Q4_K, 5, 4096, 8192), (O.Q4_K, 4, 8192, 4096)],
+                         ids=lambda c: "%s_m%d_%dx%d" % (O.NAMES[c[0]], c[1], c[2], c[3]))
+def test_few_rows_take_the_few_token_kernel_when_a_workspace_has_room(hip, ref, case):
+    """Below the tile kernel's row threshold the GEMV launches serve a matmul, four rows per pass -- except where the
+    few-token kernel is faster still (IQ4_XS from 3 rows, Q4_K from 5, on shapes it splits over k) and the caller's
+    workspace has room for its sums.  Without a workspace, or with a small one, the GEMV launches stay."""
+    import torch
+    t, m, n, k_ = case
+    w = synth.weights(t, 91, n, k_)
+    acts = ref.quantize_q8_0(synth.normal_f32(92, m * k_)).reshape(m, k_ // 32 * 34)
+    kern = hip.HipKernel(t)
+    dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
+    ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
+    expect_skinny = (t == O.IQ4_XS and m >= 3) or (t == O.Q4_K and m >= 5)
+    outs = []
+    for workspace in (ws, ws[:4096], None):
+        dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+        kern.gemm_q8_dev(dw, da, dy, m, n, k_, workspace=workspace)
+        torch.cuda.synchronize()
+        took = last_launch()
+        say(" ", O.NAMES[t], m, "workspace", None if workspace is None else workspace.numel(), "->", took)
+        assert took.startswith("gemm_skinny_kernel") == (expect_skinny and workspace is ws), took
+        outs.append(dy.cpu().numpy())
+    for r in range(m):
+        y_ref = canonical_ref(ref, t, w, acts[r], n, k_, threads=16)
+        for y in outs:
+            assert_close(y[r], y_ref, f"few rows {case} row {r}")
