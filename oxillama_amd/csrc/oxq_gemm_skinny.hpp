@@ -448,7 +448,8 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 //  * one matrix, no experts, up to 16 token rows: too few row groups as it is (14336 x 4096: 24 us against 19);
 //    with k split over work groups and the splits added by a second launch (call totals, with the token re-layout):
 //    14336 x 4096 18.0 us against 19.6, 4096 x 14336 21.4 against 29.5, 28672 x 8192 40 against 49; 4096 x 4096
-//    14.4 against 12.3 (not taken below 2^25 weights); 17..32 rows 24.6 against 19.7 (not taken).
+//    14.4 against 12.3 (not taken below 2^25 weights); 17..32 rows 24.6 against 19.7 (not taken).  From 512 row
+//    groups on no split is needed (57344 x 4096, 16 rows: 44 us against 56).
 enum SkinnyShape { SK_NONE = 0, SK_1_4, SK_1_8, SK_2_2, SK_1_4_SPLIT, SK_1_16, SK_2_8, SK_W4_1_8, SK_W4_2_4, SK_2_4 };
 
 template <class F>
@@ -460,8 +461,13 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
         if (a.sums && variant != 0 && variant != 200) return SK_NONE;  // the dump exists for the default shapes
         switch (variant) {
         case 0: {
-            if (!a.offsets)  // one matrix: up to 16 token rows, k split over work groups (the workspace has room for the sums)
-                return (!two && has_partial && skinny_splits(a.n, a.k) >= 2) ? SK_1_4_SPLIT : SK_NONE;
+            if (!a.offsets) {
+                // one matrix, up to 16 token rows: enough row groups by themselves (a vocabulary projection), or k
+                // split over work groups (the workspace has room for the sums)
+                if (two) return SK_NONE;
+                if ((size_t)((a.n + 127) / 128) >= 2 * (size_t)device_cus()) return SK_1_4;
+                return (has_partial && skinny_splits(a.n, a.k) >= 2) ? SK_1_4_SPLIT : SK_NONE;
+            }
             const bool many = (size_t)((a.n + 127) / 128) * a.n_experts >= 2 * (size_t)device_cus();
             // two token tiles: only with many row groups and a mean of at most 12 rows per expert
             if (two) return (many && 4 * (size_t)a.m <= 3 * 16 * (size_t)a.n_experts) ? SK_2_2 : SK_NONE;

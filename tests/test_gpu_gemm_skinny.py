@@ -207,6 +207,27 @@ def test_skinny_one_matrix_split_k(hip, ref, t, shape):
     assert st == capi.ERR_BUFFER_TOO_SMALL
 
 
+def test_skinny_one_matrix_with_many_row_groups(hip, ref):
+    """One matrix with at least two groups of 128 rows per compute unit (a vocabulary projection) and up to 16 token
+    rows: the few-token kernel without a split of k."""
+    import torch
+    t, m, n, k_ = O.Q4_K, 9, 65600, 512
+    w = synth.weights(t, 85, n, k_)
+    acts = ref.quantize_q8_0(synth.normal_f32(86, m * k_)).reshape(m, k_ // 32 * 34)
+    kern = hip.HipKernel(t)
+    ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
+    dy = torch.full((m + 1, n), 7.0, dtype=torch.float32, device="cuda")
+    dsum = torch.full((m, n, k_ // 32), -1, dtype=torch.int32, device="cuda")
+    kern.gemm_block_sums_dev(torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda(), dy, dsum, m, n, k_, workspace=ws)
+    torch.cuda.synchronize()
+    assert last_launch().startswith("gemm_skinny_kernel"), last_launch()
+    y, s = dy.cpu().numpy(), dsum.cpu().numpy()
+    assert np.all(y[m:] == 7.0)
+    for r in (0, 4, m - 1):
+        assert_close(y[r], canonical_ref(ref, t, w, acts[r], n, k_, threads=16), f"many row groups, row {r}")
+        assert np.array_equal(s[r], ref.block_sums(t, w, acts[r], n, k_))
+
+
 def test_skinny_split_k_on_the_host_routes(hip, ref):
     """The routes that size their own scratch -- QuantKernel::gemm on host slices, oxq_gemm_q8_dev without a
     workspace -- leave room for the per-split sums and take the same kernel."""
