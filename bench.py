@@ -19,6 +19,7 @@ Prints ONE JSON line.  Extra objects:
   prefill      batch-512 Q4_K prefill matmul, int8 TOPS vs the 5.0 POPS peak
   moe          IQ4_XS grouped expert matmuls (8 experts, 64 tokens, top-2), weight GB/s
   moe_32_tokens  the same layer for a decode batch of 32 tokens (the few-token grouped kernel)
+  moe_1_token    the same layer for one token (one GEMV launch per projection over the chosen experts)
   cpu_baseline the CPU restatement of the reference's fused rows on this host
 """
 import argparse
@@ -650,6 +651,7 @@ def main():
     # ---- C5: Mixtral-shaped IQ4_XS expert matmuls, 64 tokens, top-2 of 8 experts ------------
     moe_out = None
     moe_small = None
+    moe_one = None
     if not args.no_moe:
         from oxillama_amd import moe
         E, TOPK = 8, 2
@@ -694,6 +696,7 @@ def main():
         rows = NTOK * TOPK
         moe_us, offsets = moe_leg(NTOK)
         small_us, small_offsets = moe_leg(32)
+        one_us, one_offsets = moe_leg(1)
         moe_bytes = 3 * E * stride
         moe_ops = 2 * rows * 3 * F * H
         moe_out = {"workload": "IQ4_XS, 8 experts x (gate, up 14336x4096; down 4096x14336), 64 tokens, top-2 "
@@ -710,6 +713,12 @@ def main():
                      "rows_per_expert": np.diff(small_offsets).tolist(), "us_per_step": round(small_us, 1),
                      "weight_GBps": round(moe_bytes / small_us / 1e3, 1),
                      "frac_hbm_peak": round(moe_bytes / small_us / 1e3 / HBM_PEAK_GBPS, 4)}
+        live = int((np.diff(one_offsets) > 0).sum())
+        moe_one = {"workload": "the same layer for ONE token (MoeFfn::forward's own call: top-2, two expert rows): every "
+                               "projection is one GEMV launch over the two chosen experts' matrices",
+                   "us_per_step": round(one_us, 1), "experts_read": live, "weight_bytes": 3 * live * stride,
+                   "weight_GBps": round(3 * live * stride / one_us / 1e3, 1),
+                   "frac_hbm_peak": round(3 * live * stride / one_us / 1e3 / HBM_PEAK_GBPS, 4)}
         del wg, wu, wd
 
     # ---- CPU baseline: the reference's fused rows restated in C, same layer -------------
@@ -832,6 +841,7 @@ def main():
         "prefill": prefill,
         "moe": moe_out,
         "moe_32_tokens": moe_small,
+        "moe_1_token": moe_one,
         "device": {"name": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
                    "clock_mhz": info["clock_khz"] / 1000.0, "weight_generation_s": round(gen_s, 1)},
     }

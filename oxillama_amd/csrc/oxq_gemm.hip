@@ -107,7 +107,39 @@ bool gemm_few_rows_pay(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
            m >= (type == OXQ_TYPE_IQ4_XS ? 3u : 5u);
 }
 
+// Expert groups with at most this many token rows in all: one GEMV launch, a matvec per row against its expert's
+// matrix (each row streams a whole matrix, so this pays only while rows are fewer than about the experts they hit).
+// Measured on MI355X (IQ4_XS, 8 experts of Mixtral's shapes, us per matmul, GEMV launch / few-token kernel / tile
+// kernel): see the table in the few-token kernel's notes.
+constexpr uint32_t GROUPED_GEMV_MAX_ROWS = 8;
+
+static hipError_t gemm_grouped_by_gemv(uint32_t type, const GemmArgs &a, hipStream_t stream) {
+    GemvArgs g;
+    g.W = a.W;
+    g.A = a.A;
+    g.out = a.out;
+    g.sums = nullptr;
+    g.n_rows = a.n;
+    g.n_cols = a.k;
+    g.accumulate = a.accumulate;
+    g.bias = nullptr;
+    g.waves_per_cu = 0;
+    g.rows_per_batch = 0;
+    g.waves_per_row = 0;
+    g.group_offsets = a.offsets;
+    g.n_groups = a.n_experts;
+    g.n_pairs = a.m;
+    g.w_stride = a.w_stride;
+    g.a_stride = (size_t)(a.k / 32) * 34;
+    return launch_gemv_q8(type, g, stream);
+}
+
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) {
+    if (a.offsets && !a.sums && !a.bias && a.m <= GROUPED_GEMV_MAX_ROWS && a.n_experts <= 64 &&
+        g_gemm_variant.load(std::memory_order_relaxed) == 0) {
+        const hipError_t e = gemm_grouped_by_gemv(type, a, stream);
+        if (e != hipErrorNotSupported) return e;
+    }
     const bool tiles = a.workspace != nullptr && gemm_tiles_supported(type, a.m, a.k) && (a.offsets || !a.by_rows);
     if (!tiles) {
         if (a.offsets) return hipErrorInvalidValue;  // grouped form exists for the tile kernel only

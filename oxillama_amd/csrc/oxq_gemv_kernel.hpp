@@ -86,7 +86,9 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
                                                      const void *__restrict__ A, int32_t *__restrict__ sums,
                                                      uint32_t n_rows0, uint32_t n_rows1, uint32_t n_rows2,
                                                      uint32_t n_rows3, uint32_t units, uint32_t groups_per_row,
-                                                     size_t row_bytes, uint32_t n_cols, uint64_t *__restrict__ phases) {
+                                                     size_t row_bytes, uint32_t n_cols, uint64_t *__restrict__ phases,
+                                                     const int32_t *__restrict__ group_offsets, uint32_t n_groups_e,
+                                                     size_t w_stride, size_t a_stride) {
     static_assert(KS == 1 || KS == 2 || KS == 4, "waves per row");
     uint64_t ph_t0 = 0, ph_t1 = 0;
     if constexpr (PH) ph_t0 = wall_clock64();
@@ -98,7 +100,19 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
     const uint8_t *__restrict__ W = mat == 0 ? W0 : mat == 1 ? W1 : mat == 2 ? W2 : W3;
     float *__restrict__ out = mat == 0 ? out0 : mat == 1 ? out1 : mat == 2 ? out2 : out3;
     const float *__restrict__ old = mat == 0 ? old0 : mat == 1 ? old1 : mat == 2 ? old2 : old3;
-    const uint32_t n_rows = mat == 0 ? n_rows0 : mat == 1 ? n_rows1 : mat == 2 ? n_rows2 : n_rows3;
+    uint32_t n_rows = mat == 0 ? n_rows0 : mat == 1 ? n_rows1 : mat == 2 ? n_rows2 : n_rows3;
+    if (group_offsets) {
+        // Grouped form: blockIdx.y is a token row p; its group e (an expert) is the number of groups that end at or
+        // before p (one load per lane and a ballot; at most 64 groups).  Matrix e, activation row p, output row p.
+        const uint32_t ln = threadIdx.x & 63;
+        const int32_t end = ln < n_groups_e ? group_offsets[ln + 1] : 0x7FFFFFFF;
+        const uint32_t e = min((uint32_t)__builtin_popcountll(__ballot(end <= (int32_t)mat)), n_groups_e - 1);
+        W = W0 + (size_t)e * w_stride;
+        A = static_cast<const uint8_t *>(A) + (size_t)mat * a_stride;
+        out = out0 + (size_t)mat * n_rows0;
+        old = old0 ? old0 + (size_t)mat * n_rows0 : nullptr;
+        n_rows = n_rows0;
+    }
     constexpr uint32_t G = 4 / KS;  // row groups per work group
     __shared__ float part_sums[2][4][4];
     const uint32_t lane = threadIdx.x & 63;

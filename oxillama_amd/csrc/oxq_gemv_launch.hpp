@@ -27,14 +27,14 @@ template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP>
 static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t groups_per_row, size_t row_bytes,
                                 hipStream_t stream) {
     constexpr uint32_t G = 4 / KS;  // row groups per work group
-    const uint32_t n_mats = a.n_mats ? a.n_mats : 1;
+    const uint32_t n_mats = a.group_offsets ? a.n_pairs : a.n_mats ? a.n_mats : 1;
     const uint8_t *w[4];
     float *o[4];
     const float *old[4];  // what a row's sum is added to: the output (accumulate), a bias, or nothing
     uint32_t rows[4];
     uint32_t max_rows = a.n_rows;
     for (uint32_t i = 0; i < 4; i++) {
-        const bool more = i > 0 && i < n_mats;
+        const bool more = i > 0 && i < n_mats && !a.group_offsets;
         w[i] = more ? a.W_more[i - 1] : a.W;
         o[i] = more ? a.out_more[i - 1] : a.out;
         old[i] = a.accumulate ? o[i] : more ? a.bias_more[i - 1] : a.bias;
@@ -44,7 +44,7 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     const uint32_t n_batches = (max_rows + RB - 1) / RB;
     // the launch width is shared by the matrices of the call
     uint64_t total_rows = 0;
-    for (uint32_t i = 0; i < n_mats; i++) total_rows += rows[i];
+    for (uint32_t i = 0; i < n_mats; i++) total_rows += rows[i < 4 ? i : 0];
     // each matrix gets gridDim.x work groups, sized so that the whole launch fills the chip once
     uint32_t max_groups = (uint32_t)((uint64_t)(device_cus() * launch_width<F>(a) / KS) * max_rows / (total_rows ? total_rows : 1));
     if (max_groups == 0) max_groups = 1;
@@ -60,7 +60,8 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
         if (ph && (size_t)blocks * n_mats * 4 * 4 * 8 <= g_phase_cap.load(std::memory_order_relaxed)) {
             hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP, true>), dim3(blocks, n_mats), dim3(256), 0, stream,
                                w[0], w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums,
-                               rows[0], rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols, ph);
+                               rows[0], rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols, ph,
+                               a.group_offsets, a.n_groups, a.w_stride, a.a_stride);
             note_launch("gemv_q8_cached_phases", F::TYPE_ID, STEPS, RB, KS, DUMP, blocks, n_mats, 256);
             return hipGetLastError();
         }
@@ -71,7 +72,8 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
                 blocks, n_mats, 256);
     hipLaunchKernelGGL((gemv_q8_cached<F, SRC, STEPS, RB, KS, DUMP>), dim3(blocks, n_mats), dim3(256), lds, stream, w[0],
                        w[1], w[2], w[3], o[0], o[1], o[2], o[3], old[0], old[1], old[2], old[3], acts, a.sums, rows[0],
-                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols, (uint64_t *)nullptr);
+                       rows[1], rows[2], rows[3], units, groups_per_row, row_bytes, a.n_cols, (uint64_t *)nullptr,
+                       a.group_offsets, a.n_groups, a.w_stride, a.a_stride);
     return hipGetLastError();
 }
 
@@ -136,7 +138,7 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     case 8: return launch_steps<F, 8, 1>(a, units, groups_per_row, row_bytes, rb, stream);
     default: break;
     }
-    if (a.X) return hipErrorNotSupported;  // rows this long re-read the activations: Q8_0 blocks only
+    if (a.X || a.group_offsets) return hipErrorNotSupported;  // rows this long re-read the activations: Q8_0 blocks only
     const uint32_t max_waves = device_cus() * launch_width<F>(a);
     uint32_t waves = a.n_rows < max_waves ? a.n_rows : max_waves;
     uint32_t blocks = (waves + 3) / 4;

@@ -44,6 +44,13 @@ struct GemvArgs {
     float *out_more[3] = {nullptr, nullptr, nullptr};
     const float *bias_more[3] = {nullptr, nullptr, nullptr};
     uint32_t n_rows_more[3] = {0, 0, 0};
+    // Grouped (mixture-of-experts) form for a handful of token rows: n_pairs matvecs in one launch, pair p = the
+    // matrix at W + e * w_stride (e: the group whose rows group_offsets[e] .. group_offsets[e+1]-1 hold p) times
+    // the activation row A + p * a_stride, into out + p * n_rows.  group_offsets: device memory, n_groups + 1
+    // entries, n_groups <= 64.  n_mats, the *_more fields, X and sums are not used in this form.
+    const int32_t *group_offsets = nullptr;
+    uint32_t n_groups = 0, n_pairs = 0;
+    size_t w_stride = 0, a_stride = 0;
 };
 
 // What the calling thread launched last (kernel template, its integer parameters, grid): kept as plain fields,

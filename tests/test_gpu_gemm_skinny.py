@@ -277,3 +277,29 @@ def test_few_rows_take_the_few_token_kernel_when_a_workspace_has_room(hip, ref, 
         y_ref = canonical_ref(ref, t, w, acts[r], n, k_, threads=16)
         for y in outs:
             assert_close(y[r], y_ref, f"few rows {case} row {r}")
+
+
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+@pytest.mark.parametrize("counts", [[1, 0, 0, 1, 0, 0, 0, 0], [2, 0, 1, 0, 0, 3, 0, 2], [0, 0, 8]], ids=lambda c: "r%d" % sum(c))
+def test_grouped_matmul_of_a_handful_of_rows_is_one_gemv_launch(hip, ref, t, counts):
+    """Up to 8 token rows in all (a single token's top-2, a decode batch of a few): one GEMV launch, a matvec per row
+    against its expert's matrix -- the bits of oxq_matvec_q8_fused_dev on that row, for every format."""
+    import torch
+    n, k_ = 300, 2048
+    offsets, acts, w = _case(ref, t, counts, n, k_, 7000 + sum(counts))
+    rows = int(offsets[-1])
+    dy, _ = _run(hip, t, w, acts, offsets, n, k_, max(counts))
+    assert last_launch().startswith("gemv_q8_cached"), last_launch()
+    y = dy.cpu().numpy()
+    assert np.all(y[rows:] == 7.0)
+    kern = hip.HipKernel(t)
+    for r in range(rows):
+        e = int(np.searchsorted(offsets, r, side="right") - 1)
+        assert_close(y[r], canonical_ref(ref, t, w[e], acts[r], n, k_), f"row {r} expert {e}")
+        d1 = torch.zeros(n, dtype=torch.float32, device="cuda")
+        kern.matvec_q8_fused_dev(torch.from_numpy(w[e]).cuda(), torch.from_numpy(acts[r]).cuda(), d1, n, k_, accumulate=False)
+        torch.cuda.synchronize()
+        assert np.array_equal(d1.cpu().numpy(), y[r]), f"row {r}: not the single matvec's bits"
+    # accumulate
+    dy2, _ = _run(hip, t, w, acts, offsets, n, k_, max(counts), accumulate=True, out=dy.clone())
+    assert torch.equal(dy2[:rows], dy[:rows] + dy[:rows]) and torch.equal(dy2[rows:], dy[rows:])

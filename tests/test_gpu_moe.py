@@ -297,7 +297,9 @@ def test_moe_forward_host_slices(hip, ref):
         one = layer.forward(x[:hidden])
         assert_close(one, want(x[:hidden]), "one token", tol=2e-3)
         many = layer.forward_batch(x, 5).reshape(5, hidden)
-        assert np.array_equal(many[0].view(np.uint32), one.view(np.uint32))  # a row does not depend on the batch
+        # one token is two rows (one GEMV launch per projection), five tokens ten (the matmul kernels): another
+        # summation order, so the same row agrees to the layer's bar rather than bit for bit
+        assert_close(many[0], one, "a token alone and in a batch", tol=2e-3)
         for i in range(5):
             assert_close(many[i], want(x[i * hidden:(i + 1) * hidden]), f"token {i}", tol=2e-3)
     lib.oxq_weight_cache_enable(0)

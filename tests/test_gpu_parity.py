@@ -690,12 +690,20 @@ def test_moe_grouped_matmul(hip, ref, t, cfg):
             s_ref[r] = ref.block_sums(t, w[e], acts[r], n, k_)
     assert_close(y[:rows], y_ref, f"moe {cfg}")
     assert np.array_equal(dsum.cpu().numpy() - _tile_zero_point(t, acts.reshape(-1), rows, k_), s_ref)
-    # production launch (no sums), overwrite then accumulate: the same bits as the dump launch
-    dy2 = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
-    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy2, n, k_, ws)
+    # production launch (no sums): the same bits as the dump launch -- except for a handful of rows in all, which one
+    # GEMV launch serves (a matvec per row; the dump is the matmul kernels'): the same values within the bar.
+    # Overwrite then accumulate: twice the production launch's bits.
+    dy1 = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
+    kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy1, n, k_, ws)
+    torch.cuda.synchronize()
+    if rows > 8:
+        assert torch.equal(dy1, dy[:rows])
+    else:
+        assert_close(dy1.cpu().numpy(), y_ref, f"moe {cfg} production launch")
+    dy2 = dy1.clone()
     kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, max_rows, dy2, n, k_, ws, accumulate=True)
     torch.cuda.synchronize()
-    assert torch.equal(dy2, dy[:rows] + dy[:rows])
+    assert torch.equal(dy2, dy1 + dy1)
     # max_rows = 0 (unknown) sizes the launch for the worst case: another tile shape and fp32
     # summation order, the same values within the bar
     dy3 = torch.zeros((rows, n), dtype=torch.float32, device="cuda")
