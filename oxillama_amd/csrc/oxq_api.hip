@@ -1330,6 +1330,24 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
     hipStream_t s = (hipStream_t)stream;
     OXQ_HIP(oxq::launch_moe_gather_quantize(d_x, d_pair_token, acts, pairs, (uint32_t)hidden, s));
     const size_t gws = workspace_bytes - l.gemm;
+    // A handful of rows (one token's top-k, a decode batch of a few): gate, up, SwiGLU and the quantizer of h in one
+    // GEMV launch over the rows' experts, where the format and row length have that kernel (the bits of the
+    // separate launches below).
+    bool fused = false;
+    if (pairs <= oxq::GROUPED_GEMV_MAX_ROWS && gate_type == up_type && n_experts <= 64 && intermediate % 32 == 0 &&
+        oxq::g_gemm_variant.load(std::memory_order_relaxed) == 0 && g.fuse_swiglu.load(std::memory_order_relaxed)) {
+        oxq::GateUpGroups grp;
+        grp.offsets = d_row_offsets;
+        grp.n_groups = (uint32_t)n_experts;
+        grp.n_pairs = (uint32_t)pairs;
+        grp.wg_stride = gate_stride_bytes;
+        grp.wu_stride = up_stride_bytes;
+        const hipError_t e = oxq::launch_gate_up_swiglu(gate_type, d_gate, d_up, acts, hq, nullptr, (uint32_t)intermediate,
+                                                        (uint32_t)hidden, s, grp);
+        if (e == hipSuccess) fused = true;
+        else if (e != hipErrorNotSupported) return fail_hip(e, "launch_gate_up_swiglu (grouped)");
+    }
+    if (!fused) {
     if ((st = oxq_moe_gemm_q8_dev(gate_type, d_gate, gate_stride_bytes, n_experts, acts, d_row_offsets, pairs,
                                   max_rows_per_expert, gate, nullptr, intermediate, hidden, 0, ws + l.gemm, gws,
                                   stream)) != OXQ_OK)
@@ -1339,6 +1357,7 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
                             nullptr, intermediate, hidden, 0, ws + l.gemm, gws, stream, gate_type)) != OXQ_OK)
         return st;
     OXQ_HIP(oxq::launch_swiglu_quantize(gate, up, pairs * intermediate, nullptr, hq, s));
+    }
     if ((st = oxq_moe_gemm_q8_dev(down_type, d_down, down_stride_bytes, n_experts, hq, d_row_offsets, pairs,
                                   max_rows_per_expert, y, nullptr, hidden, intermediate, 0, ws + l.gemm, gws,
                                   stream)) != OXQ_OK)

@@ -111,8 +111,6 @@ bool gemm_few_rows_pay(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
 // matrix (each row streams a whole matrix, so this pays only while rows are fewer than about the experts they hit).
 // Measured on MI355X (IQ4_XS, 8 experts of Mixtral's shapes, us per matmul, GEMV launch / few-token kernel / tile
 // kernel): see the table in the few-token kernel's notes.
-constexpr uint32_t GROUPED_GEMV_MAX_ROWS = 8;
-
 static hipError_t gemm_grouped_by_gemv(uint32_t type, const GemmArgs &a, hipStream_t stream) {
     GemvArgs g;
     g.W = a.W;

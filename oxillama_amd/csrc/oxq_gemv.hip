@@ -76,16 +76,17 @@ bool gemv_takes_f32(uint32_t type, uint32_t n_cols) {
 }
 
 hipError_t launch_gate_up_swiglu(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts, uint8_t *hq,
-                                 float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream) {
+                                 float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream,
+                                 const GateUpGroups &grp) {
     switch (type) {
-    case OXQ_TYPE_Q4_0: return launch_gate_up_swiglu_format<FmtQ4_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    case OXQ_TYPE_Q8_0: return launch_gate_up_swiglu_format<FmtQ8_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    case OXQ_TYPE_Q4_K: return launch_gate_up_swiglu_format<FmtQ4K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    case OXQ_TYPE_Q4_0: return launch_gate_up_swiglu_format<FmtQ4_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
+    case OXQ_TYPE_Q8_0: return launch_gate_up_swiglu_format<FmtQ8_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
+    case OXQ_TYPE_Q4_K: return launch_gate_up_swiglu_format<FmtQ4K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
     case OXQ_TYPE_Q6_K:
         if (misaligned(Wg) || misaligned(Wu)) return hipErrorInvalidDevicePointer;
-        return launch_gate_up_swiglu_format<FmtQ6K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    case OXQ_TYPE_IQ4_XS: return launch_gate_up_swiglu_format<FmtIQ4XS>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    default: return launch_gate_up_swiglu_more(type, Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+        return launch_gate_up_swiglu_format<FmtQ6K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
+    case OXQ_TYPE_IQ4_XS: return launch_gate_up_swiglu_format<FmtIQ4XS>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
+    default: return launch_gate_up_swiglu_more(type, Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
     }
 }
 

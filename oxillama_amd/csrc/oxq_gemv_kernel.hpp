@@ -229,15 +229,32 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
 // up (RB rows per batch, the next batch's loads in flight while one is reduced; one wave per row,
 // so the sums are those of gemv_q8_cached with KS = 1, bit for bit), the 64 sums meet in LDS and
 // eight lanes encode the block.  h_out (optional) receives h in fp32.
-template <class F, int STEPS, int RB, int WAVES, bool PH = false>
+// GRP: the grouped (mixture-of-experts) form for a handful of token rows -- blockIdx.y is a token row p, its expert e
+// the group of group_offsets that holds p (found as in gemv_q8_cached); gate matrix Wg + e * wg_stride, up matrix
+// Wu + e * wu_stride, activation row A + p * a_stride, block of h at hq + p * hq_stride.  The arguments after
+// `phases` are read in that form only.
+template <class F, int STEPS, int RB, int WAVES, bool PH = false, bool GRP = false>
 __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8_t *__restrict__ Wg,
                                                              const uint8_t *__restrict__ Wu,
                                                              const void *__restrict__ A, uint8_t *__restrict__ hq,
                                                              float *__restrict__ h_out, uint32_t n_rows, uint32_t units,
-                                                             size_t row_bytes, uint64_t *__restrict__ phases) {
+                                                             size_t row_bytes, uint64_t *__restrict__ phases,
+                                                             const int32_t *__restrict__ group_offsets,
+                                                             uint32_t n_groups_e, size_t wg_stride, size_t wu_stride,
+                                                             size_t a_stride, size_t hq_stride) {
     static_assert((RB == 1 || RB == 2) && (WAVES == 4 || WAVES == 8), "configuration");
     uint64_t ph_t0 = 0, ph_t1 = 0;
     if constexpr (PH) ph_t0 = wall_clock64();
+    if constexpr (GRP) {
+        const uint32_t p = blockIdx.y, ln = threadIdx.x & 63;
+        const int32_t end = ln < n_groups_e ? group_offsets[ln + 1] : 0x7FFFFFFF;
+        const uint32_t e = min((uint32_t)__builtin_popcountll(__ballot(end <= (int32_t)p)), n_groups_e - 1);
+        Wg += (size_t)e * wg_stride;
+        Wu += (size_t)e * wu_stride;
+        A = static_cast<const uint8_t *>(A) + (size_t)p * a_stride;
+        hq += (size_t)p * hq_stride;
+        if (h_out) h_out += (size_t)p * n_rows;
+    }
     constexpr int RPW = 32 / WAVES;  // rows of each matrix per wave
     constexpr int NB = RPW / RB;     // batches per matrix and wave
     __shared__ float row_sums[2][32];

@@ -156,12 +156,30 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
 // configurations launch_format gives KS = 1 and at most two steps), a whole number of 32-row blocks.
 template <class F>
 static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts, uint8_t *hq,
-                                               float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream) {
+                                               float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream,
+                                               const GateUpGroups &grp = GateUpGroups()) {
     const uint32_t units = n_cols / F::UNIT_COLS;
     const size_t row_bytes = (size_t)(n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
     const uint32_t steps = (units + 63) / 64;
     if (steps > 2 || n_rows % 32 != 0 || n_rows == 0) return hipErrorNotSupported;
     const bool two = row_bytes <= F::TWO_ROW_BATCH_BYTES;
+    if (grp.offsets) {
+        if (grp.n_groups > 64 || grp.n_pairs == 0 || grp.n_pairs > 65535) return hipErrorNotSupported;
+        const dim3 grid(n_rows / 32, grp.n_pairs);
+        const size_t a_stride = (size_t)(n_cols / 32) * 34, hq_stride = (size_t)(n_rows / 32) * 34;
+#define OXQ_LAUNCH_GRP(ST, RBV)                                                                                      \
+    note_launch("gemv_q8_gate_up_swiglu_grouped", F::TYPE_ID, ST, RBV, 4, 0, grid.x, grid.y, 256);                   \
+    hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4, false, true>), grid, dim3(256), 0, stream, Wg, Wu,    \
+                       acts, hq, h, n_rows, units, row_bytes, (uint64_t *)nullptr, grp.offsets, grp.n_groups,         \
+                       grp.wg_stride, grp.wu_stride, a_stride, hq_stride)
+        if (steps == 1) {
+            if (two) { OXQ_LAUNCH_GRP(1, 2); } else { OXQ_LAUNCH_GRP(1, 1); }
+        } else {
+            if (two) { OXQ_LAUNCH_GRP(2, 2); } else { OXQ_LAUNCH_GRP(2, 1); }
+        }
+#undef OXQ_LAUNCH_GRP
+        return hipGetLastError();
+    }
     const dim3 grid(n_rows / 32);
     uint64_t *ph = nullptr;
     if constexpr (phase_probe_format<F>::value) {
@@ -173,12 +191,14 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
     if constexpr (phase_probe_format<F>::value) {                                                                    \
         if (ph) {                                                                                                    \
             hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4, true>), grid, dim3(256), 0, stream, Wg, Wu,    \
-                               acts, hq, h, n_rows, units, row_bytes, ph);                                           \
+                               acts, hq, h, n_rows, units, row_bytes, ph, (const int32_t *)nullptr, 0u, (size_t)0,   \
+                               (size_t)0, (size_t)0, (size_t)0);                                                     \
             return hipGetLastError();                                                                                \
         }                                                                                                            \
     }                                                                                                                \
     hipLaunchKernelGGL((gemv_q8_gate_up_swiglu<F, ST, RBV, 4>), grid, dim3(256), 0, stream, Wg, Wu, acts, hq, h,     \
-                       n_rows, units, row_bytes, (uint64_t *)nullptr)
+                       n_rows, units, row_bytes, (uint64_t *)nullptr, (const int32_t *)nullptr, 0u, (size_t)0,       \
+                       (size_t)0, (size_t)0, (size_t)0)
     if (steps == 1) {
         if (two) { OXQ_LAUNCH(1, 2); } else { OXQ_LAUNCH(1, 1); }
     } else {

@@ -22,12 +22,13 @@ hipError_t launch_gemv_vecs_more(uint32_t type, const GemvVecsArgs &a, hipStream
 }
 
 hipError_t launch_gate_up_swiglu_more(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts,
-                                      uint8_t *hq, float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream) {
+                                      uint8_t *hq, float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream,
+                                 const GateUpGroups &grp) {
     switch (type) {
-    case OXQ_TYPE_Q5_K: return launch_gate_up_swiglu_format<FmtQ5K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    case OXQ_TYPE_Q4_1: return launch_gate_up_swiglu_format<FmtQ4_1>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    case OXQ_TYPE_Q5_0: return launch_gate_up_swiglu_format<FmtQ5_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
-    case OXQ_TYPE_Q5_1: return launch_gate_up_swiglu_format<FmtQ5_1>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream);
+    case OXQ_TYPE_Q5_K: return launch_gate_up_swiglu_format<FmtQ5K>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
+    case OXQ_TYPE_Q4_1: return launch_gate_up_swiglu_format<FmtQ4_1>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
+    case OXQ_TYPE_Q5_0: return launch_gate_up_swiglu_format<FmtQ5_0>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
+    case OXQ_TYPE_Q5_1: return launch_gate_up_swiglu_format<FmtQ5_1>(Wg, Wu, acts, hq, h, n_rows, n_cols, stream, grp);
     default: return hipErrorNotSupported;  // the caller runs the two projections and the SwiGLU kernel
     }
 }

@@ -105,10 +105,20 @@ uint32_t gemv_group_cols(uint32_t type);
 hipError_t launch_gemv_q8_more(uint32_t type, const GemvArgs &a, hipStream_t stream);
 // ffn_gate, ffn_up, SwiGLU and the Q8_0 quantizer of h in one launch (both matrices of `type`, n_rows a
 // multiple of 32).  hipErrorNotSupported: no such kernel for this type / row length.
+// grp.offsets set: the grouped (mixture-of-experts) form for a handful of token rows -- row p of acts (n_pairs rows)
+// against the gate and up matrices of its expert e (the group of grp.offsets that holds p), Wg + e * wg_stride and
+// Wu + e * wu_stride; row p of hq / h.
+struct GateUpGroups {
+    const int32_t *offsets = nullptr;  // device memory, n_groups + 1 entries, n_groups <= 64; null: the dense form
+    uint32_t n_groups = 0, n_pairs = 0;
+    size_t wg_stride = 0, wu_stride = 0;
+};
 hipError_t launch_gate_up_swiglu(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts, uint8_t *hq,
-                                 float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream);
+                                 float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream,
+                                 const GateUpGroups &grp = GateUpGroups());
 hipError_t launch_gate_up_swiglu_more(uint32_t type, const uint8_t *Wg, const uint8_t *Wu, const uint8_t *acts,
-                                      uint8_t *hq, float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream);
+                                      uint8_t *hq, float *h, uint32_t n_rows, uint32_t n_cols, hipStream_t stream,
+                                      const GateUpGroups &grp = GateUpGroups());
 hipError_t launch_gemv_vecs_more(uint32_t type, const GemvVecsArgs &a, hipStream_t stream);
 
 // x: n floats (n % 32 == 0) -> n/32 Q8_0 blocks of 34 bytes.
@@ -174,6 +184,8 @@ extern std::atomic<int> g_gemm_variant;              // 0 = default tile shape
 extern std::atomic<uint32_t> g_gemm_tile_min_rows;   // 0 = default threshold
 // True when (type, m, k) is served by the int8-MFMA tile kernel.
 bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k);
+// Grouped (mixture-of-experts) matmuls of at most this many token rows in all take one GEMV launch, a matvec per row.
+constexpr uint32_t GROUPED_GEMV_MAX_ROWS = 8;
 // Below gemm_uses_tiles' row threshold, but the few-token kernel (k split over work groups) still beats the GEMV
 // launches: for callers that hold a workspace of gemm_workspace_bytes(m, k, n, type).
 bool gemm_few_rows_pay(uint32_t type, uint32_t m, uint32_t n, uint32_t k);
