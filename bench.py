@@ -666,23 +666,18 @@ def main():
         def moe_leg(NTOK):
             xt = torch.from_numpy(synth.normal_f32(7, NTOK * H)).to(dev)
             rows = NTOK * TOPK
-            d_exp = torch.empty(rows, dtype=torch.int32, device=dev)
-            d_wt = torch.empty(rows, dtype=torch.float32, device=dev)
-            d_off = torch.empty(E + 1, dtype=torch.int32, device=dev)
-            d_tok = torch.empty(rows, dtype=torch.int32, device=dev)
-            d_rows = torch.empty(rows, dtype=torch.int32, device=dev)
             d_y = torch.empty(NTOK * H, dtype=torch.float32, device=dev)
-            wsm = torch.empty(moe.moe_ffn_workspace_bytes(types3, rows, H, F), dtype=torch.uint8, device=dev)
+            wsm = torch.empty(moe.moe_forward_workspace_bytes(types3, NTOK, TOPK, E, H, F), dtype=torch.uint8, device=dev)
+            off_at = 2 * ((4 * rows + 255) & ~255)  # the workspace starts with experts | weights | offsets | ...
 
             def moe_step():
-                moe.route_dev(router, xt, NTOK, E, H, TOPK, d_exp, d_wt, d_off, d_tok, d_rows)
-                moe.moe_ffn_dev((IQ4_XS, wg, stride), (IQ4_XS, wu, stride), (IQ4_XS, wd, stride), E, xt, NTOK, TOPK,
-                                d_off, d_tok, d_rows, d_wt, 0, d_y, H, F, wsm)
+                moe.moe_forward_dev((IQ4_XS, wg, stride), (IQ4_XS, wu, stride), (IQ4_XS, wd, stride), E, router, xt, NTOK,
+                                    TOPK, d_y, H, F, wsm)
 
             with torch.cuda.stream(stream):
                 moe_step()
                 stream.synchronize()
-                offsets = d_off.cpu().numpy()
+                offsets = wsm[off_at:off_at + 4 * (E + 1)].cpu().numpy().view(np.int32)
                 reps = 6
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)

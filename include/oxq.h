@@ -456,14 +456,33 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
                     size_t max_rows_per_expert, float *d_out, size_t hidden, size_t intermediate,
                     void *d_workspace, size_t workspace_bytes, void *stream);
 
+/* MoeFfn::forward (crates/oxillama-arch/src/common/moe.rs:184-258) on device pointers, for
+ * n_tokens input vectors at once: oxq_moe_route_dev + oxq_moe_ffn_dev in one call, with the
+ * routing tables kept in the workspace.  d_router fp32 [n_experts x hidden]; d_x, d_out fp32
+ * [n_tokens x hidden]; expert e's matrices at d_gate + e * gate_stride_bytes, etc.  top_k == 0
+ * is KernelError (moe.rs:168-172), top_k above n_experts is clamped (moe.rs:233); no expert or
+ * intermediate == 0 gives the zeroed output (moe.rs:240-242).  The same bits as the two calls.
+ * For one token (the reference's own call) the router's launch also groups the choices and
+ * writes the quantized activation rows, so the layer is four launches plus the combine.  No
+ * allocation, no synchronisation; needs oxq_moe_forward_workspace_bytes() bytes of 256-byte-
+ * aligned scratch (0: no grouped kernel for a type / shape). */
+size_t oxq_moe_forward_workspace_bytes(uint32_t gate_type, uint32_t up_type, uint32_t down_type,
+                                       size_t n_tokens, size_t top_k, size_t n_experts,
+                                       size_t hidden, size_t intermediate);
+int oxq_moe_forward_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_bytes,
+                        uint32_t up_type, const uint8_t *d_up, size_t up_stride_bytes,
+                        uint32_t down_type, const uint8_t *d_down, size_t down_stride_bytes,
+                        size_t n_experts, const float *d_router, const float *d_x, size_t n_tokens,
+                        size_t top_k, float *d_out, size_t hidden, size_t intermediate,
+                        void *d_workspace, size_t workspace_bytes, void *stream);
+
 /* MoeFfn::forward on host slices, for n_tokens input vectors at once (n_tokens = 1 is the
  * reference's call): experts' matrices as raw blocks, expert after expert (gate_len = n_experts *
  * bytes of one [intermediate x hidden] matrix, etc.), fp32 router [n_experts x hidden].  Checks
  * in the reference's order (moe.rs:151-173: router size, top_k; moe.rs:33-58: gate, up, down
  * sizes) as DimensionMismatch {expected, got} / KernelError; hidden and intermediate must be
  * multiples of 256 (UnsupportedShape otherwise).  Stages everything to the device (weights
- * through the weight cache when it is on), runs oxq_moe_route_dev + oxq_moe_ffn_dev, copies the
- * output back. */
+ * through the weight cache when it is on), runs oxq_moe_forward_dev, copies the output back. */
 int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, uint32_t up_type,
                     const uint8_t *up, size_t up_len, uint32_t down_type, const uint8_t *down,
                     size_t down_len, const float *router, size_t router_len, size_t n_experts,

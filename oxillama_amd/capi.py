@@ -172,6 +172,12 @@ SIGNATURES = {
                                   C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p,
                                   C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t,
                                   C.c_void_p, C.c_size_t, C.c_void_p]),
+    "oxq_moe_forward_workspace_bytes": (C.c_size_t, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_size_t, C.c_size_t,
+                                                     C.c_size_t, C.c_size_t, C.c_size_t]),
+    "oxq_moe_forward_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.c_uint32, C.c_void_p, C.c_size_t,
+                                      C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p,
+                                      C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p,
+                                      C.c_size_t, C.c_void_p]),
     "oxq_topk_workspace_bytes": (C.c_size_t, [C.c_size_t, C.c_size_t]),
     "oxq_topk_dev": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                C.c_void_p]),

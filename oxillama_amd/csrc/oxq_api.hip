@@ -1299,12 +1299,15 @@ size_t oxq_moe_ffn_workspace_bytes(uint32_t gate_type, uint32_t up_type, uint32_
     return moe_ffn_layout(gate_type, up_type, down_type, n_pairs, hidden, intermediate, &l) ? l.total : 0;
 }
 
-int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_bytes, uint32_t up_type,
-                    const uint8_t *d_up, size_t up_stride_bytes, uint32_t down_type, const uint8_t *d_down,
-                    size_t down_stride_bytes, size_t n_experts, const float *d_x, size_t n_tokens, size_t top_k,
-                    const int32_t *d_row_offsets, const int32_t *d_pair_token, const int32_t *d_token_rows,
-                    const float *d_weights, size_t max_rows_per_expert, float *d_out, size_t hidden,
-                    size_t intermediate, void *d_workspace, size_t workspace_bytes, void *stream) {
+namespace {
+// acts_ready: the grouped Q8_0 activation rows already sit at their place in the workspace (the one-token
+// router launch wrote them); otherwise the gather launch comes first.
+int moe_ffn_impl(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_bytes, uint32_t up_type,
+                 const uint8_t *d_up, size_t up_stride_bytes, uint32_t down_type, const uint8_t *d_down,
+                 size_t down_stride_bytes, size_t n_experts, const float *d_x, size_t n_tokens, size_t top_k,
+                 const int32_t *d_row_offsets, const int32_t *d_pair_token, const int32_t *d_token_rows,
+                 const float *d_weights, size_t max_rows_per_expert, float *d_out, size_t hidden, size_t intermediate,
+                 void *d_workspace, size_t workspace_bytes, void *stream, bool acts_ready) {
     int st;
     if ((st = check_dev_shape(gate_type, intermediate, hidden)) != OXQ_OK) return st;
     if ((st = check_dev_shape(up_type, intermediate, hidden)) != OXQ_OK) return st;
@@ -1328,7 +1331,7 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
     uint8_t *acts = ws + l.acts, *hq = ws + l.hq;
     float *gate = (float *)(ws + l.gate), *up = (float *)(ws + l.up), *y = (float *)(ws + l.y);
     hipStream_t s = (hipStream_t)stream;
-    OXQ_HIP(oxq::launch_moe_gather_quantize(d_x, d_pair_token, acts, pairs, (uint32_t)hidden, s));
+    if (!acts_ready) OXQ_HIP(oxq::launch_moe_gather_quantize(d_x, d_pair_token, acts, pairs, (uint32_t)hidden, s));
     const size_t gws = workspace_bytes - l.gemm;
     // A handful of rows (one token's top-k, a decode batch of a few): gate, up, SwiGLU and the quantizer of h in one
     // GEMV launch over the rows' experts, where the format and row length have that kernel (the bits of the
@@ -1367,6 +1370,94 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
     return OXQ_OK;
 }
 
+// Tables of the layer in front of the feed-forward workspace: experts | weights | offsets | pair_token | token_rows.
+struct MoeTables {
+    size_t experts, weights, offsets, pair_token, token_rows, ffn, total;
+};
+bool moe_forward_layout(uint32_t gate_type, uint32_t up_type, uint32_t down_type, size_t n_tokens, size_t k,
+                        size_t n_experts, size_t hidden, size_t inter, MoeTables *t, MoeFfnLayout *l) {
+    const size_t pairs = n_tokens * k;
+    if (!moe_ffn_layout(gate_type, up_type, down_type, pairs, hidden, inter, l)) return false;
+    size_t off = 0;
+    t->experts = off; off += align256(pairs * 4);
+    t->weights = off; off += align256(pairs * 4);
+    t->offsets = off; off += align256((n_experts + 1) * 4);
+    t->pair_token = off; off += align256(pairs * 4);
+    t->token_rows = off; off += align256(pairs * 4);
+    t->ffn = off;
+    t->total = off + l->total;
+    return true;
+}
+}  // namespace
+
+int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_bytes, uint32_t up_type,
+                    const uint8_t *d_up, size_t up_stride_bytes, uint32_t down_type, const uint8_t *d_down,
+                    size_t down_stride_bytes, size_t n_experts, const float *d_x, size_t n_tokens, size_t top_k,
+                    const int32_t *d_row_offsets, const int32_t *d_pair_token, const int32_t *d_token_rows,
+                    const float *d_weights, size_t max_rows_per_expert, float *d_out, size_t hidden,
+                    size_t intermediate, void *d_workspace, size_t workspace_bytes, void *stream) {
+    return moe_ffn_impl(gate_type, d_gate, gate_stride_bytes, up_type, d_up, up_stride_bytes, down_type, d_down,
+                        down_stride_bytes, n_experts, d_x, n_tokens, top_k, d_row_offsets, d_pair_token, d_token_rows,
+                        d_weights, max_rows_per_expert, d_out, hidden, intermediate, d_workspace, workspace_bytes, stream,
+                        false);
+}
+
+size_t oxq_moe_forward_workspace_bytes(uint32_t gate_type, uint32_t up_type, uint32_t down_type, size_t n_tokens,
+                                       size_t top_k, size_t n_experts, size_t hidden, size_t intermediate) {
+    MoeTables t;
+    MoeFfnLayout l;
+    const size_t k = top_k < n_experts ? top_k : n_experts;
+    return moe_forward_layout(gate_type, up_type, down_type, n_tokens, k, n_experts, hidden, intermediate, &t, &l)
+               ? t.total
+               : 0;
+}
+
+int oxq_moe_forward_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_bytes, uint32_t up_type,
+                        const uint8_t *d_up, size_t up_stride_bytes, uint32_t down_type, const uint8_t *d_down,
+                        size_t down_stride_bytes, size_t n_experts, const float *d_router, const float *d_x,
+                        size_t n_tokens, size_t top_k, float *d_out, size_t hidden, size_t intermediate,
+                        void *d_workspace, size_t workspace_bytes, void *stream) {
+    int st;
+    if ((st = check_dev_shape(gate_type, intermediate, hidden)) != OXQ_OK) return st;
+    if ((st = check_dev_shape(up_type, intermediate, hidden)) != OXQ_OK) return st;
+    if ((st = check_dev_shape(down_type, hidden, intermediate)) != OXQ_OK) return st;
+    if (top_k == 0) return fail(OXQ_ERR_KERNEL, 1, 0, "MoeFfn top_k must be >= 1");  // moe.rs:168-172
+    if (n_experts > 1024) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 1024, n_experts, "at most 1024 experts");
+    const size_t k = top_k < n_experts ? top_k : n_experts;  // moe.rs:233
+    if (n_tokens * k > 0x7FFFFFFFull || hidden > 0xFFFFFFFFull)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0x7FFFFFFFull, n_tokens * k, "too many (token, expert) pairs");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (n_tokens == 0 || hidden == 0) return OXQ_OK;
+    if (!d_x || !d_out) return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (n_experts == 0 || intermediate == 0) {  // no expert to add: the zeroed output (moe.rs:240-242)
+        OXQ_HIP(oxq::launch_fill_zero(d_out, n_tokens * hidden, s));
+        return OXQ_OK;
+    }
+    if (!d_router || !d_gate || !d_up || !d_down) return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer");
+    MoeTables t;
+    MoeFfnLayout l;
+    if (!moe_forward_layout(gate_type, up_type, down_type, n_tokens, k, n_experts, hidden, intermediate, &t, &l))
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, hidden, "no grouped kernel for this type/shape");
+    if (!d_workspace || workspace_bytes < t.total)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, t.total, d_workspace ? workspace_bytes : 0, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
+        return fail(OXQ_ERR_KERNEL, 256, reinterpret_cast<uintptr_t>(d_workspace) & 255,
+                    "workspace must be 256-byte aligned");
+    uint8_t *ws = (uint8_t *)d_workspace;
+    int32_t *experts = (int32_t *)(ws + t.experts), *offsets = (int32_t *)(ws + t.offsets);
+    int32_t *pair_token = (int32_t *)(ws + t.pair_token), *token_rows = (int32_t *)(ws + t.token_rows);
+    float *weights = (float *)(ws + t.weights);
+    // One token with a handful of choices: the router's launch also groups and writes the activation rows.
+    const bool one = n_tokens == 1 && k <= oxq::GROUPED_GEMV_MAX_ROWS;
+    OXQ_HIP(oxq::launch_moe_route(d_router, d_x, experts, weights, (uint32_t)n_tokens, (uint32_t)n_experts,
+                                  (uint32_t)hidden, (uint32_t)k, offsets, pair_token, token_rows, s,
+                                  one ? ws + t.ffn + l.acts : nullptr));
+    return moe_ffn_impl(gate_type, d_gate, gate_stride_bytes, up_type, d_up, up_stride_bytes, down_type, d_down,
+                        down_stride_bytes, n_experts, d_x, n_tokens, k, offsets, pair_token, token_rows, weights, 0, d_out,
+                        hidden, intermediate, ws + t.ffn, workspace_bytes - t.ffn, stream, one);
+}
+
 // MoeFfn::forward on host slices (the drop-in route): everything is staged to the device, the layer
 // runs there, the output comes back.  Validation in the reference's order (moe.rs:151-173, 33-58).
 int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, uint32_t up_type, const uint8_t *up,
@@ -1400,8 +1491,8 @@ int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, ui
         std::memset(output, 0, n_tokens * hidden * sizeof(float));
         return OXQ_OK;
     }
-    const size_t k = top_k < n_experts ? top_k : n_experts, pairs = n_tokens * k;
-    const size_t ws_bytes = oxq_moe_ffn_workspace_bytes(gate_type, up_type, down_type, pairs, hidden, intermediate);
+    const size_t ws_bytes =
+        oxq_moe_forward_workspace_bytes(gate_type, up_type, down_type, n_tokens, top_k, n_experts, hidden, intermediate);
     if (ws_bytes == 0)
         return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, hidden % 256 ? hidden : intermediate,
                     "no grouped kernel for this type/shape (dimensions must be multiples of 256)");
@@ -1420,27 +1511,16 @@ int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, ui
     if ((st = stage(g.s_weights, gate_type, gate, gate_len, &dg)) != OXQ_OK) return st;
     if ((st = stage(g.s_moe_up, up_type, up, up_len, &du)) != OXQ_OK) return st;
     if ((st = stage(g.s_moe_down, down_type, down, down_len, &dd)) != OXQ_OK) return st;
-    // tables: router | experts | weights | offsets | pair_token | token_rows, each 256-byte aligned
-    size_t off = 0;
-    auto take = [&](size_t bytes) { const size_t at = off; off += align256(bytes); return at; };
-    const size_t o_router = take(router_len * sizeof(float)), o_exp = take(pairs * 4), o_wt = take(pairs * 4);
-    const size_t o_off = take((n_experts + 1) * 4), o_tok = take(pairs * 4), o_rows = take(pairs * 4);
-    if ((st = g.s_moe_tables.reserve(off)) != OXQ_OK) return st;
+    if ((st = g.s_moe_tables.reserve(router_len * sizeof(float))) != OXQ_OK) return st;
     if ((st = g.s_x.reserve(n_tokens * hidden * sizeof(float))) != OXQ_OK) return st;
     if ((st = g.s_out.reserve(n_tokens * hidden * sizeof(float))) != OXQ_OK) return st;
     if ((st = g.s_work.reserve(ws_bytes + 256)) != OXQ_OK) return st;
-    uint8_t *tb = (uint8_t *)g.s_moe_tables.ptr;
     uint8_t *ws = (uint8_t *)((reinterpret_cast<uintptr_t>(g.s_work.ptr) + 255) & ~(uintptr_t)255);
-    OXQ_HIP(hipMemcpy(tb + o_router, router, router_len * sizeof(float), hipMemcpyHostToDevice));
+    OXQ_HIP(hipMemcpy(g.s_moe_tables.ptr, router, router_len * sizeof(float), hipMemcpyHostToDevice));
     OXQ_HIP(hipMemcpy(g.s_x.ptr, input, n_tokens * hidden * sizeof(float), hipMemcpyHostToDevice));
-    if ((st = oxq_moe_route_dev((const float *)(tb + o_router), (const float *)g.s_x.ptr, n_tokens, n_experts, hidden,
-                                top_k, (int32_t *)(tb + o_exp), (float *)(tb + o_wt), (int32_t *)(tb + o_off),
-                                (int32_t *)(tb + o_tok), (int32_t *)(tb + o_rows), nullptr)) != OXQ_OK)
-        return st;
-    if ((st = oxq_moe_ffn_dev(gate_type, dg, g_one, up_type, du, u_one, down_type, dd, d_one, n_experts,
-                              (const float *)g.s_x.ptr, n_tokens, k, (const int32_t *)(tb + o_off),
-                              (const int32_t *)(tb + o_tok), (const int32_t *)(tb + o_rows), (const float *)(tb + o_wt), 0,
-                              (float *)g.s_out.ptr, hidden, intermediate, ws, ws_bytes, nullptr)) != OXQ_OK)
+    if ((st = oxq_moe_forward_dev(gate_type, dg, g_one, up_type, du, u_one, down_type, dd, d_one, n_experts,
+                                  (const float *)g.s_moe_tables.ptr, (const float *)g.s_x.ptr, n_tokens, top_k,
+                                  (float *)g.s_out.ptr, hidden, intermediate, ws, ws_bytes, nullptr)) != OXQ_OK)
         return st;
     OXQ_HIP(hipMemcpy(output, g.s_out.ptr, n_tokens * hidden * sizeof(float), hipMemcpyDeviceToHost));
     return OXQ_OK;

@@ -19,34 +19,47 @@ namespace oxq {
 // 64-bit wave maximum over keys (weight bits, complemented index); weights divided by the sum of
 // the selected ones in selection order (1/k when that sum is <= 1e-9).  Lane l owns experts l,
 // l + 64, ... in LDS.  5 * n_exp floats of dynamic LDS.
+//
+// ONE (a launch for a single token, k <= n_exp): the work group goes on to what the grouping and
+// the gather kernels would do for that token -- the k chosen experts in ascending order are the
+// grouped rows (offsets[e] = how many chosen experts lie below e), every row belongs to token 0,
+// and each row's activations are the token's Q8_0 blocks, written k times.  Same tables and bytes
+// as the separate launches.
+template <bool ONE>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict__ router, const float *__restrict__ x,
                                                        int32_t *__restrict__ experts, float *__restrict__ weights,
-                                                       uint32_t n_exp, uint32_t hidden, uint32_t k) {
+                                                       uint32_t n_exp, uint32_t hidden, uint32_t k,
+                                                       int32_t *__restrict__ offsets, int32_t *__restrict__ pair_token,
+                                                       int32_t *__restrict__ token_rows, uint8_t *__restrict__ acts) {
     extern __shared__ float lds[];
     float *probs = lds, *part = lds + n_exp;
     const uint32_t t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const float *xr = x + (size_t)t * hidden;
     const uint32_t n4 = (hidden & 3) == 0 ? hidden / 4 : 0;
-    for (uint32_t e0 = 0; e0 < n_exp; e0 += 4) {  // four experts per pass: their loads are in flight together
-        const float *rr[4];
-        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        for (int q = 0; q < 4; q++) rr[q] = router + (size_t)min(e0 + q, n_exp - 1) * hidden;
+    constexpr int EP = 8;  // experts per pass: their loads are in flight together
+    for (uint32_t e0 = 0; e0 < n_exp; e0 += EP) {
+        const float *rr[EP];
+        float acc[EP];
+        for (int q = 0; q < EP; q++) {
+            rr[q] = router + (size_t)min(e0 + q, n_exp - 1) * hidden;
+            acc[q] = 0.0f;
+        }
         if (n4) {
             for (uint32_t c = threadIdx.x; c < n4; c += 256) {
-                float xv[4], rv[4][4];
+                float xv[4], rv[EP][4];
                 load4(xv, xr + 4 * c);
 #pragma unroll
-                for (int q = 0; q < 4; q++) load4(rv[q], rr[q] + 4 * c);
+                for (int q = 0; q < EP; q++) load4(rv[q], rr[q] + 4 * c);
 #pragma unroll
-                for (int q = 0; q < 4; q++)
+                for (int q = 0; q < EP; q++)
                     for (int i = 0; i < 4; i++) acc[q] += rv[q][i] * xv[i];
             }
         } else {
             for (uint32_t c = threadIdx.x; c < hidden; c += 256)
-                for (int q = 0; q < 4; q++) acc[q] += rr[q][c] * xr[c];
+                for (int q = 0; q < EP; q++) acc[q] += rr[q][c] * xr[c];
         }
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
+        for (int q = 0; q < EP; q++) {
             const float v = wave_sum(acc[q]);
             if (lane == 0 && e0 + q < n_exp) part[4 * (e0 + q) + wave] = v;
         }
@@ -55,47 +68,74 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict_
     for (uint32_t e = threadIdx.x; e < n_exp; e += 256)
         probs[e] = (part[4 * e] + part[4 * e + 1]) + (part[4 * e + 2] + part[4 * e + 3]);
     __syncthreads();
-    if (wave != 0) return;
+    int32_t *chosen = reinterpret_cast<int32_t *>(part);  // ONE: the selection, for the other waves (part is free now)
 
-    float m = -INFINITY;
-    for (uint32_t e = lane; e < n_exp; e += 64) m = fmaxf(m, probs[e]);
-    m = fmaxf(m, dpp_f<0xB1>(m));
-    m = fmaxf(m, dpp_f<0x4E>(m));
-    m = fmaxf(m, dpp_f<0x124>(m));
-    m = fmaxf(m, dpp_f<0x128>(m));
-    const float max_logit = fmaxf(fmaxf(readlane_f(m, 0), readlane_f(m, 16)), fmaxf(readlane_f(m, 32), readlane_f(m, 48)));
-    float s = 0.0f;
-    for (uint32_t e = lane; e < n_exp; e += 64) {
-        const float v = expf(probs[e] - max_logit);
-        probs[e] = v;
-        s += v;
-    }
-    const float exp_sum = wave_sum(s);
-    const float uniform = 1.0f / (float)n_exp;
-    for (uint32_t e = lane; e < n_exp; e += 64) probs[e] = exp_sum > 0.0f ? probs[e] / exp_sum : uniform;
-
-    int32_t *sel = experts + (size_t)t * k;
-    float *wt = weights + (size_t)t * k;
-    float selected_sum = 0.0f;
-    for (uint32_t r = 0; r < k; r++) {
-        uint64_t best = 0;
+    if (wave == 0) {
+        float m = -INFINITY;
+        for (uint32_t e = lane; e < n_exp; e += 64) m = fmaxf(m, probs[e]);
+        m = fmaxf(m, dpp_f<0xB1>(m));
+        m = fmaxf(m, dpp_f<0x4E>(m));
+        m = fmaxf(m, dpp_f<0x124>(m));
+        m = fmaxf(m, dpp_f<0x128>(m));
+        const float max_logit =
+            fmaxf(fmaxf(readlane_f(m, 0), readlane_f(m, 16)), fmaxf(readlane_f(m, 32), readlane_f(m, 48)));
+        float s = 0.0f;
         for (uint32_t e = lane; e < n_exp; e += 64) {
-            const float v = probs[e];  // >= 0 (or NaN, which ranks first and is taken once); taken entries are -1
-            const uint64_t key = v < 0.0f ? 0 : ((uint64_t)__builtin_bit_cast(uint32_t, v) << 32) | (0xFFFFFFFFu - e);
-            best = max_u64(best, key);
+            const float v = expf(probs[e] - max_logit);
+            probs[e] = v;
+            s += v;
         }
-        best = wave_max_u64(best);
-        const uint32_t e = 0xFFFFFFFFu - (uint32_t)best;
-        const float v = __builtin_bit_cast(float, (uint32_t)(best >> 32));
-        if ((e & 63) == lane) probs[e] = -1.0f;  // the owner lane is the only one that reads it again
-        selected_sum += v;
-        if (lane == 0) {
-            sel[r] = (int32_t)e;
-            wt[r] = v;
+        const float exp_sum = wave_sum(s);
+        const float uniform = 1.0f / (float)n_exp;
+        for (uint32_t e = lane; e < n_exp; e += 64) probs[e] = exp_sum > 0.0f ? probs[e] / exp_sum : uniform;
+
+        int32_t *sel = experts + (size_t)t * k;
+        float *wt = weights + (size_t)t * k;
+        float selected_sum = 0.0f;
+        for (uint32_t r = 0; r < k; r++) {
+            uint64_t best = 0;
+            for (uint32_t e = lane; e < n_exp; e += 64) {
+                const float v = probs[e];  // >= 0 (or NaN, which ranks first and is taken once); taken entries are -1
+                const uint64_t key =
+                    v < 0.0f ? 0 : ((uint64_t)__builtin_bit_cast(uint32_t, v) << 32) | (0xFFFFFFFFu - e);
+                best = max_u64(best, key);
+            }
+            best = wave_max_u64(best);
+            const uint32_t e = 0xFFFFFFFFu - (uint32_t)best;
+            const float v = __builtin_bit_cast(float, (uint32_t)(best >> 32));
+            if ((e & 63) == lane) probs[e] = -1.0f;  // the owner lane is the only one that reads it again
+            selected_sum += v;
+            if (lane == 0) {
+                sel[r] = (int32_t)e;
+                wt[r] = v;
+                if (ONE) chosen[r] = (int32_t)e;
+            }
         }
+        if (lane == 0)
+            for (uint32_t r = 0; r < k; r++) wt[r] = selected_sum > 1e-9f ? wt[r] / selected_sum : 1.0f / (float)k;
     }
-    if (lane == 0)
-        for (uint32_t r = 0; r < k; r++) wt[r] = selected_sum > 1e-9f ? wt[r] / selected_sum : 1.0f / (float)k;
+    if (!ONE) return;
+
+    __syncthreads();
+    for (uint32_t e = threadIdx.x; e <= n_exp; e += 256) {
+        int32_t below = 0;
+        for (uint32_t r = 0; r < k; r++) below += chosen[r] < (int32_t)e ? 1 : 0;
+        offsets[e] = below;
+    }
+    for (uint32_t p = threadIdx.x; p < k; p += 256) {
+        int32_t row = 0;
+        for (uint32_t r = 0; r < k; r++) row += chosen[r] < chosen[p] ? 1 : 0;
+        token_rows[p] = row;
+        pair_token[row] = 0;
+    }
+    const uint32_t bpr = hidden / 32, j = threadIdx.x & 7;
+    for (uint32_t b0 = 0; b0 < bpr; b0 += 32) {  // eight lanes per block as in the quantizer
+        const uint32_t b = b0 + (threadIdx.x >> 3);
+        const bool valid = b < bpr;
+        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (valid) load4(v, xr + (size_t)b * 32 + 4 * j);
+        for (uint32_t r = 0; r < k; r++) encode_q8_0_lanes(v, valid, acts + ((size_t)r * bpr + b) * 34, j);
+    }
 }
 
 // One work group per expert e.  Pass 1 counts the pairs routed to experts below e (the first
@@ -179,6 +219,18 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restric
     out[i] = o;
 }
 
+__global__ __launch_bounds__(256) void fill_zero_kernel(float *__restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = 0.0f;
+}
+
+// A fill by a kernel, not a memset node: callers may be capturing the stream into a graph.
+hipError_t launch_fill_zero(float *out, size_t n, hipStream_t stream) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, out, n);
+    return hipGetLastError();
+}
+
 hipError_t launch_moe_gather_quantize(const float *x, const int32_t *pair_token, uint8_t *out, size_t n_pairs,
                                       uint32_t hidden, hipStream_t stream) {
     const uint32_t bpr = hidden / 32;
@@ -200,10 +252,16 @@ hipError_t launch_moe_combine(const float *y_pairs, const int32_t *token_rows, c
 
 hipError_t launch_moe_route(const float *router, const float *x, int32_t *experts, float *weights, uint32_t n_tokens,
                             uint32_t n_exp, uint32_t hidden, uint32_t k, int32_t *offsets, int32_t *pair_token,
-                            int32_t *token_rows, hipStream_t stream) {
+                            int32_t *token_rows, hipStream_t stream, uint8_t *acts_one) {
     if (n_tokens == 0 || n_exp == 0) return hipSuccess;
-    hipLaunchKernelGGL(moe_route_kernel, dim3(n_tokens), dim3(256), 5 * n_exp * sizeof(float), stream, router, x, experts,
-                       weights, n_exp, hidden, k);
+    const size_t lds = 5 * n_exp * sizeof(float);
+    if (acts_one) {  // the caller checked: one token, a handful of choices, whole blocks
+        hipLaunchKernelGGL(moe_route_kernel<true>, dim3(1), dim3(256), lds, stream, router, x, experts, weights, n_exp,
+                           hidden, k, offsets, pair_token, token_rows, acts_one);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(moe_route_kernel<false>, dim3(n_tokens), dim3(256), lds, stream, router, x, experts, weights,
+                       n_exp, hidden, k, offsets, pair_token, token_rows, acts_one);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(moe_group_kernel, dim3(n_exp), dim3(256), 0, stream, experts, n_tokens * k, k, offsets,

@@ -92,6 +92,25 @@ def moe_ffn_dev(gate, up, down, n_experts, d_x, n_tokens, top_k, d_offsets, d_pa
                                        workspace.numel(), HipKernel._stream()))
 
 
+def moe_forward_workspace_bytes(types, n_tokens, top_k, n_experts, hidden, intermediate):
+    from . import capi
+    tg, tu, td = (int(t) for t in types)
+    return capi.load().oxq_moe_forward_workspace_bytes(tg, tu, td, n_tokens, top_k, n_experts, hidden, intermediate)
+
+
+def moe_forward_dev(gate, up, down, n_experts, d_router, d_x, n_tokens, top_k, d_out, hidden, intermediate, workspace):
+    """MoeFfn::forward (moe.rs:184-258) for n_tokens tokens on torch CUDA tensors, current stream: routing and
+    the experts in one call, tables in the workspace.  gate / up / down as in moe_ffn_dev."""
+    from . import capi
+    from .quant import HipKernel, _check
+    args = []
+    for t, d_w, stride in (gate, up, down):
+        args += [int(t), d_w.data_ptr(), stride]
+    _check(capi.load().oxq_moe_forward_dev(*args, n_experts, d_router.data_ptr(), d_x.data_ptr(), n_tokens, top_k,
+                                           d_out.data_ptr(), hidden, intermediate, workspace.data_ptr(),
+                                           workspace.numel(), HipKernel._stream()))
+
+
 class MoeFfn:
     """MoeFfn of the reference (moe.rs:129-258) with the experts' projections as GGUF blocks.
 

@@ -377,3 +377,64 @@ def test_moe_layer_full_size_c5(hip, ref):
             eo = ref.matvec_q8_fused_mt(t, wd[e * stride:(e + 1) * stride], hq, hidden, inter, 16)
             acc = acc + weights[tk, j] * eo
         assert_close(got[tk], acc, f"token {tk}", tol=2e-3)
+
+
+@pytest.mark.parametrize("cfg", [(8, 2, 1, 512, 256, O.IQ4_XS), (8, 1, 1, 256, 512, O.Q4_K), (8, 8, 1, 256, 256, O.Q6_K),
+                                 (16, 9, 1, 256, 256, O.Q4_K), (3, 5, 1, 256, 256, O.Q8_0), (8, 2, 5, 256, 512, O.IQ4_XS),
+                                 (8, 2, 40, 512, 256, O.Q4_K), (70, 2, 1, 256, 256, O.Q4_K)], ids=str)
+def test_moe_forward_on_device_pointers(hip, ref, cfg):
+    """oxq_moe_forward_dev (routing and experts in one call; for one token the router's launch also groups the
+    choices and writes the activation rows) against oxq_moe_route_dev + oxq_moe_ffn_dev: the same bits, on a
+    workspace that held other contents before; one token against the oracle's layer as well."""
+    n_exp, top_k, n_tok, hidden, inter, t = cfg
+    say("moe forward dev", cfg)
+    wg = expert_weights(t, 100, n_exp, inter, hidden)
+    wu = expert_weights(t, 200, n_exp, inter, hidden)
+    wd = expert_weights(t, 300, n_exp, hidden, inter)
+    stride_gu, stride_d = wg.size // n_exp, wd.size // n_exp
+    router = synth.normal_f32(15, n_exp * hidden, 0.05)
+    x = synth.normal_f32(16, n_tok * hidden)
+    d_x, d_router, d_wg, d_wu, d_wd = dev(x), dev(router), dev(wg), dev(wu), dev(wd)
+    d, k = route_on_device(router, x, n_tok, n_exp, hidden, top_k)
+    ws = torch.empty(moe.moe_ffn_workspace_bytes((t, t, t), n_tok * k, hidden, inter), dtype=torch.uint8, device=DEV)
+    want = torch.empty(n_tok * hidden, dtype=torch.float32, device=DEV)
+    moe.moe_ffn_dev((t, d_wg, stride_gu), (t, d_wu, stride_gu), (t, d_wd, stride_d), n_exp, d_x, n_tok, k, d["offsets"],
+                    d["pair_token"], d["token_rows"], d["weights"], 0, want, hidden, inter, ws)
+    need = moe.moe_forward_workspace_bytes((t, t, t), n_tok, top_k, n_exp, hidden, inter)
+    assert need > ws.numel()
+    ws2 = torch.full((need,), 0xA5, dtype=torch.uint8, device=DEV)
+    got = torch.full((n_tok * hidden,), 7.0, dtype=torch.float32, device=DEV)
+    for _ in range(2):  # the second call finds the first one's tables and rows in the workspace
+        moe.moe_forward_dev((t, d_wg, stride_gu), (t, d_wu, stride_gu), (t, d_wd, stride_d), n_exp, d_router, d_x, n_tok,
+                            top_k, got, hidden, inter, ws2)
+        assert np.array_equal(host(got).view(np.uint32), host(want).view(np.uint32))
+    # the tables at the head of the workspace: experts | weights | offsets | pair_token | token_rows, 256-byte slots
+    al = lambda n: (n + 255) & ~255
+    raw = host(ws2)
+    o = 0
+    for name, n in (("experts", n_tok * k), ("weights", n_tok * k), ("offsets", n_exp + 1), ("pair_token", n_tok * k),
+                    ("token_rows", n_tok * k)):
+        assert np.array_equal(raw[o:o + 4 * n], host(d[name]).ravel().view(np.uint8)), name
+        o += al(4 * n)
+    with pytest.raises(Exception):
+        moe.moe_forward_dev((t, d_wg, stride_gu), (t, d_wu, stride_gu), (t, d_wd, stride_d), n_exp, d_router, d_x, n_tok,
+                            top_k, got, hidden, inter, ws2[:need - 256])
+    if n_tok == 1:
+        y_ref, sel, _ = ref.moe_forward_q(t, router, wg, wu, wd, n_exp, hidden, inter, top_k, x)
+        assert np.array_equal(host(d["experts"]).ravel(), sel.astype(np.int32))
+        assert_close(host(got), y_ref, "one token against the oracle", tol=2e-3)
+
+
+def test_moe_forward_on_device_pointers_degenerate(hip):
+    """No experts or no intermediate columns: the zeroed output (moe.rs:240-242); top_k == 0: InvalidConfig."""
+    from oxillama_amd.quant import KernelError
+    hidden = 256
+    d_x = dev(synth.normal_f32(3, 2 * hidden))
+    out = torch.full((2 * hidden,), 7.0, dtype=torch.float32, device=DEV)
+    empty = torch.empty(256, dtype=torch.uint8, device=DEV)
+    moe.moe_forward_dev((O.Q4_K, empty, 0), (O.Q4_K, empty, 0), (O.Q4_K, empty, 0), 0, empty, d_x, 2, 2, out, hidden, 256,
+                        empty)
+    assert not host(out).any()
+    with pytest.raises(KernelError):
+        moe.moe_forward_dev((O.Q4_K, empty, 0), (O.Q4_K, empty, 0), (O.Q4_K, empty, 0), 4, empty, d_x, 2, 0, out, hidden,
+                            256, empty)
