@@ -263,7 +263,8 @@ int oxq_activation_route(void);
 
 /* Prefill / decode batch: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched
  * form of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  From 6 rows up
- * (9 where n < 8192), with k a multiple of 256, every format but Q2_K / Q3_K runs on the int8-MFMA tile
+ * (9 where n < 8192), with k a multiple of 256 (the formats of 32-weight blocks: any multiple of
+ * 32 from 256 up), every format runs on the int8-MFMA tile
  * kernel, which needs oxq_gemm_q8_workspace_bytes() bytes of 256-byte-aligned device scratch:
  * pass it and the call is asynchronous and allocation-free; pass NULL and the library uses
  * its own scratch (the call then serialises and waits for the stream).  Fewer rows, and
@@ -304,7 +305,8 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
  * copies nor synchronises; max_rows_per_expert bounds any one group (0 = total_rows) and only
  * sizes the launch (which kernel and tile shape serve the call follows from it and from the mean
  * group size: fp32 summation order, hence the last bits, can differ between two bounds; every
- * choice meets the 1e-5 bar).  k must be a multiple of 256; needs oxq_moe_gemm_q8_workspace_bytes() bytes of
+ * choice meets the 1e-5 bar).  k must be a multiple of 256 (the formats of 32-weight blocks: of
+ * 32, and at least 256); needs oxq_moe_gemm_q8_workspace_bytes() bytes of
  * 256-byte-aligned device scratch.  d_sums (optional, else NULL): exact int32 group sums
  * [(row * n + c) * (k/32) + g] as in oxq_gemm_block_sums_dev. */
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k);
@@ -481,7 +483,8 @@ int oxq_moe_forward_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_s
  * bytes of one [intermediate x hidden] matrix, etc.), fp32 router [n_experts x hidden].  Checks
  * in the reference's order (moe.rs:151-173: router size, top_k; moe.rs:33-58: gate, up, down
  * sizes) as DimensionMismatch {expected, got} / KernelError; hidden and intermediate must be
- * multiples of 256 (UnsupportedShape otherwise).  Stages everything to the device (weights
+ * multiples of 256, or of 32 from 256 up where the matrices they are the row length of are in
+ * formats of 32-weight blocks (UnsupportedShape otherwise).  Stages everything to the device (weights
  * through the weight cache when it is on), runs oxq_moe_forward_dev, copies the output back. */
 int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, uint32_t up_type,
                     const uint8_t *up, size_t up_len, uint32_t down_type, const uint8_t *down,

@@ -56,7 +56,7 @@ std::atomic<int> g_gemm_variant{0};  // tuning: 0 = default
 
 static size_t gemm_planes_bytes(uint32_t m, uint32_t k) {
     // token rows are padded so that a 128-token tile starting at any row stays inside
-    const size_t mpad = ((size_t)m + 127) / 128 * 128 + 128, nsb = k / 32;
+    const size_t mpad = ((size_t)m + 127) / 128 * 128 + 128, nsb = tile_padded_sub_blocks(k);
     return nsb * mpad * (32 + 4 + 2 + 8);  // activation bytes, P, f16 scales, the two half-block planes of P
 }
 // Bytes of the few-token kernel's per-split sums for this call, 0 if it would not split k.
@@ -80,8 +80,12 @@ bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
                        type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q5_K || type == OXQ_TYPE_Q4_1 ||
                        type == OXQ_TYPE_IQ4_NL || type == OXQ_TYPE_Q8_1 || type == OXQ_TYPE_Q5_0 || type == OXQ_TYPE_Q5_1 ||
                        type == OXQ_TYPE_Q3_K || type == OXQ_TYPE_Q2_K;
-    // the 32-weight formats are walked eight blocks at a time
-    return known && k % 256 == 0 && m >= 1 && (size_t)(k / 32) * 256 <= 128 * 1024 &&
+    // the 32-weight formats are walked eight blocks at a time; their rows may end inside the last eight (the
+    // kernel then reads that step through the window of the row's last eight blocks), the others' may not
+    const bool blocks32 = type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q4_1 ||
+                          type == OXQ_TYPE_IQ4_NL || type == OXQ_TYPE_Q8_1 || type == OXQ_TYPE_Q5_0 || type == OXQ_TYPE_Q5_1;
+    const bool whole = k % 256 == 0 || (blocks32 && k % 32 == 0 && k >= 256);
+    return known && whole && m >= 1 && (size_t)tile_padded_sub_blocks(k) * 256 <= 128 * 1024 &&
            gemm_planes_bytes(m, k) < 0x7FFFFFFFull;
 }
 
@@ -143,7 +147,7 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
         if (a.offsets) return hipErrorInvalidValue;  // grouped form exists for the tile kernel only
         return gemm_by_rows(type, a, stream);
     }
-    const uint32_t mpad = (a.m + 127) / 128 * 128 + 128, nsb = a.k / 32;
+    const uint32_t mpad = (a.m + 127) / 128 * 128 + 128, nsb = tile_padded_sub_blocks(a.k), nsb_row = a.k / 32;
     uint8_t *q8t = a.workspace;
     float *P = reinterpret_cast<float *>(q8t + (size_t)nsb * mpad * 32);
     uint16_t *da16 = reinterpret_cast<uint16_t *>(q8t + (size_t)nsb * mpad * 36);
@@ -182,11 +186,11 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
                          ? reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(P) + tile_p16_offset(nsb, mpad))
                          : nullptr;
         if (perm == 2)
-            hipLaunchKernelGGL(gemm_prep_acts<2>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
+            hipLaunchKernelGGL(gemm_prep_acts<2>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16, nsb_row);
         else if (perm == 1)
-            hipLaunchKernelGGL(gemm_prep_acts<1>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
+            hipLaunchKernelGGL(gemm_prep_acts<1>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16, nsb_row);
         else
-            hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16);
+            hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16, nsb_row);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }

@@ -48,6 +48,7 @@ struct TileQ5K {
 template <uint32_t TYPE_ID, uint32_t STRIDE, uint32_t PAYLOAD, bool LUT, bool WITH_M>
 struct TileNibbles32 {
     static constexpr uint32_t TYPE = TYPE_ID, BLOCK_BYTES = 8 * STRIDE;
+    static constexpr bool RAGGED_K = true;
     static constexpr bool HAS_MIN = WITH_M;
     static constexpr int ACT_PERM = 1, NQ = 1, KSPLIT = 1;
     struct Hdr {
@@ -92,6 +93,7 @@ using TileIQ4NL = TileNibbles32<OXQ_TYPE_IQ4_NL, 18, 2, true, false>;
 // Q8_1 (reference/q8_1.rs:36-42): 36 B = d, s (unused), 32 int8; the payload is the B operand.
 struct TileQ8_1 {
     static constexpr uint32_t TYPE = OXQ_TYPE_Q8_1, BLOCK_BYTES = 8 * 36;
+    static constexpr bool RAGGED_K = true;
     static constexpr bool HAS_MIN = false;
     static constexpr int ACT_PERM = 0, NQ = 2, KSPLIT = 1;
     using Hdr = TileQ8_0::Hdr;
@@ -126,6 +128,7 @@ struct TileQ8_1 {
 template <uint32_t TYPE_ID, uint32_t STRIDE, bool WITH_M>
 struct TileQ5x {
     static constexpr uint32_t TYPE = TYPE_ID, BLOCK_BYTES = 8 * STRIDE;
+    static constexpr bool RAGGED_K = true;
     static constexpr uint32_t QH = WITH_M ? 4 : 2, PAYLOAD = QH + 4;
     static constexpr bool HAS_MIN = true;
     static constexpr int ACT_PERM = 2, NQ = 2, KSPLIT = 1;

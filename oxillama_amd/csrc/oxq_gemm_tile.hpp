@@ -193,6 +193,7 @@ struct TileIQ4XS {
 // IQ4_XS; the "- 8" goes through the zero-point term: sum (q-8) a = sum q a - 8 sum a.
 struct TileQ4_0 {
     static constexpr uint32_t TYPE = OXQ_TYPE_Q4_0, BLOCK_BYTES = 8 * 18;
+    static constexpr bool RAGGED_K = true;  // eight independent 32-weight blocks: rows of any whole number of them
     static constexpr bool HAS_MIN = true;
     static constexpr int ACT_PERM = 1, NQ = 1, KSPLIT = 1;
     struct Hdr {
@@ -230,6 +231,7 @@ struct TileQ4_0 {
 // 256-weight step; the payload is the B operand as it is.
 struct TileQ8_0 {
     static constexpr uint32_t TYPE = OXQ_TYPE_Q8_0, BLOCK_BYTES = 8 * 34;
+    static constexpr bool RAGGED_K = true;
     static constexpr bool HAS_MIN = false;
     static constexpr int ACT_PERM = 0, NQ = 2, KSPLIT = 1;
     struct Hdr {
@@ -321,17 +323,24 @@ struct TileQ6K {
 template <int PERM>
 __global__ __launch_bounds__(256) void gemm_prep_acts(const uint8_t *__restrict__ A, uint8_t *__restrict__ q8t,
                                                      float *__restrict__ P, uint16_t *__restrict__ da16, uint32_t m,
-                                                     uint32_t mpad, uint32_t nsb, float *__restrict__ p16) {
+                                                     uint32_t mpad, uint32_t nsb, float *__restrict__ p16,
+                                                     uint32_t nsb_row) {
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= mpad * nsb) return;
     // eight consecutive threads take eight consecutive blocks of one token (272 contiguous bytes), the next eight
-    // the next token: reads in runs of a token row's bytes, writes in runs of eight tokens (256 bytes) per sub-block
-    // (nsb is a multiple of 8: the tile kernel wants k % 256 == 0)
+    // the next token: reads in runs of a token row's bytes, writes in runs of eight tokens (256 bytes) per sub-block.
+    // nsb is a multiple of 8 (the tile kernel walks 256 columns at a time); a token row holds nsb_row <= nsb blocks.
+    // When the row ends inside the last group of eight, that group is the row's LAST eight blocks (the window the
+    // kernel reads its weights through, so that no read leaves the row), and the blocks of it that the group
+    // before already covers are written as zeros.
     const uint32_t grp = idx >> 3, t = grp % mpad, j = (grp / mpad) * 8 + (idx & 7);
+    const uint32_t shift = nsb - nsb_row, last = nsb - 8;
+    const uint32_t src = j >= last ? j - shift : j;
+    const bool live = j < last || (idx & 7) >= shift;
     u32x4 q[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
     uint32_t dbits = 0;
-    if (t < m) {
-        const uint8_t *blk = A + ((size_t)t * nsb + j) * Q8_BLOCK_BYTES;
+    if (t < m && live) {
+        const uint8_t *blk = A + ((size_t)t * nsb_row + src) * Q8_BLOCK_BYTES;
         dbits = ld2(blk);
         q[0] = ld16(blk + 2);
         q[1] = ld16(blk + 18);
@@ -373,6 +382,14 @@ template <class F, class = void> struct tile_min_planes { static constexpr int v
 template <class F> struct tile_min_planes<F, std::void_t<decltype(F::MIN_PLANES)>> {
     static constexpr int value = F::MIN_PLANES;
 };
+// Formats made of independent 32-weight blocks (the policy says RAGGED_K) take rows of any whole number of blocks
+// (at least eight); the others need whole 256-weight super-blocks.
+template <class F, class = void> struct tile_ragged_k { static constexpr bool value = false; };
+template <class F> struct tile_ragged_k<F, std::void_t<decltype(F::RAGGED_K)>> {
+    static constexpr bool value = F::RAGGED_K;
+};
+// Sub-blocks the planes of the workspace hold for a row of k weights: whole groups of eight.
+__host__ __device__ __forceinline__ uint32_t tile_padded_sub_blocks(uint32_t k) { return (k + 255) / 256 * 8; }
 // Byte offset, from the start of the P plane, of the two half-block planes (the workspace holds the
 // activation bytes, P, the f16 scales, then the half planes: 32 + 4 + 2 bytes per token block before them).
 __host__ __device__ __forceinline__ size_t tile_p16_offset(size_t nsb, size_t mpad) { return nsb * mpad * 6; }
@@ -420,7 +437,13 @@ __device__ __forceinline__ void gemm_tile_body(
     constexpr size_t RED_BYTES = SPLITK ? sizeof(float) * 4 * MT * NT * 16 * 64 : 0;
     __shared__ __align__(16) uint8_t lds_static[SC_BYTES > RED_BYTES ? SC_BYTES : RED_BYTES];
     float (*lds_sc)[8][NP][W_ROWS] = reinterpret_cast<float (*)[8][NP][W_ROWS]>(lds_static);
-    const uint32_t nsb = k / 32, nblk = k / 256, ngrp = nblk * 4;
+    // A row that ends inside its last group of eight blocks (formats of independent 32-weight blocks only): the
+    // last group is read through the window of the row's last eight blocks, so that no load leaves the row, and
+    // the `dead` sub-blocks of that window, which the group before has covered, get zero factors (their token
+    // bytes and scales in the workspace are zeros as well).
+    constexpr bool RAG = tile_ragged_k<F>::value;
+    const uint32_t nsb_row = k / 32, nblk = RAG ? (k + 255) / 256 : k / 256, nsb = nblk * 8, ngrp = nblk * 4;
+    const uint32_t dead = nsb - nsb_row;
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     // split k: the wave index as a scalar -- everything derived from it (the wave's k range, hence the scalar
     // offsets of its buffer loads) must be known to be wave-uniform, or every load is wrapped in a waterfall
@@ -483,7 +506,9 @@ __device__ __forceinline__ void gemm_tile_body(
     // per-lane offset and a scalar offset that advances with k, so the loop spends no
     // vector instructions on addressing.  Rows past n are clamped for loads and masked
     // at the store.
-    const uint32_t row_bytes = nblk * F::BLOCK_BYTES;
+    const uint32_t row_bytes = RAG ? nsb_row * (F::BLOCK_BYTES / 8) : nblk * F::BLOCK_BYTES;
+    const uint32_t last_window = row_bytes - F::BLOCK_BYTES;
+    auto blk_off = [&](uint32_t blk) { return RAG ? min(blk * F::BLOCK_BYTES, last_window) : blk * F::BLOCK_BYTES; };
     const uint32_t n_base = min(n_wg, n - 1);
     const size_t w_left = (size_t)(n - n_base) * row_bytes;
     const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
@@ -499,7 +524,7 @@ __device__ __forceinline__ void gemm_tile_body(
     // factors of the next super-block after its last read of the current ones.
     const uint32_t drow = lane % W_ROWS, ds0 = SPL * (lane / W_ROWS);
     const uint32_t hrow_off = (min(n_wave + drow, n - 1) - n_base) * row_bytes;
-    auto decode = [&](const typename F::Hdr &hd) {
+    auto decode = [&](const typename F::Hdr &hd, uint32_t blk) {
 #pragma unroll
         for (int e = 0; e < SPL; e++) {
             const uint32_t s = ds0 + e;
@@ -508,6 +533,10 @@ __device__ __forceinline__ void gemm_tile_body(
                 F::factors2(hd, e, s, dsc, qneg);
             else
                 F::factors(hd, e, s, dsc, qneg[0]);
+            if (RAG && blk == nblk - 1 && s < dead) {
+                for (int is = 0; is < KS; is++) dsc[is] = 0.0f;
+                for (int ip = 0; ip < MINP; ip++) qneg[ip] = 0.0f;
+            }
 #pragma unroll
             for (int is = 0; is < KS; is++) {
                 lds_sc[wave][s][is][drow] = dsc[is];
@@ -519,8 +548,8 @@ __device__ __forceinline__ void gemm_tile_body(
     };
     {
         typename F::Hdr hd;
-        F::template load_hdr<SPL>(rs_w, hrow_off, min(blk_begin, nblk - 1) * F::BLOCK_BYTES, ds0, hd);
-        decode(hd);
+        F::template load_hdr<SPL>(rs_w, hrow_off, blk_off(min(blk_begin, nblk - 1)), ds0, hd);
+        decode(hd, min(blk_begin, nblk - 1));
     }
 
     v16f acc[MT][NT];
@@ -552,7 +581,7 @@ __device__ __forceinline__ void gemm_tile_body(
     // group index G = 4*blk + g; groups past the end re-read the last one (result unused)
     auto fetch_w = [&](Wq &w, uint32_t G) {
         G = min(G, ngrp - 1);
-        for (int nt = 0; nt < NT; nt++) F::fetch(rs_w, wq_off[nt], h, (G >> 2) * F::BLOCK_BYTES, G & 3, w.q[nt]);
+        for (int nt = 0; nt < NT; nt++) F::fetch(rs_w, wq_off[nt], h, blk_off(G >> 2), G & 3, w.q[nt]);
     };
     auto fetch_a = [&](Ops &o, uint32_t G) {
         G = min(G, ngrp - 1);
@@ -610,8 +639,11 @@ __device__ __forceinline__ void gemm_tile_body(
                 acc[mt][nt][i] = fmaf(tt, da, acc[mt][nt][i]);
                 if (DUMP) {
                     const uint32_t row = m_wave + mt * 32 + 8 * (i >> 2) + 4 * h + (i & 3);
-                    if (row < row_end && nrow[nt] < n)
-                        sums[((size_t)row * n + nrow[nt]) * (nsb * KS) + j * KS + is] = (int)(dbits - MAGIC_BITS);
+                    // (a row's last window: sub-block s of it is block j - dead of the row; dead ones are skipped)
+                    const bool shifted = RAG && blk == nblk - 1;
+                    if (row < row_end && nrow[nt] < n && !(shifted && s < dead))
+                        sums[((size_t)row * n + nrow[nt]) * (nsb_row * KS) + (j - (shifted ? dead : 0)) * KS + is] =
+                            (int)(dbits - MAGIC_BITS);
                 }
             }
             if (t + 2 < T) dq[t & 1] = mfma_tile(t + 2);
@@ -651,7 +683,7 @@ __device__ __forceinline__ void gemm_tile_body(
             for (int i = 0; i < 4; i++) fetch_w(incoming[i], blk * 4 + DIST + i);
         }
         typename F::Hdr hd;
-        F::template load_hdr<SPL>(rs_w, hrow_off, nxt * F::BLOCK_BYTES, ds0, hd);
+        F::template load_hdr<SPL>(rs_w, hrow_off, blk_off(nxt), ds0, hd);
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const Wq w = DIST < 4 ? wring[g % (DIST < 4 ? DIST : 1)] : wring[DIST < 4 ? 0 : g];
@@ -669,7 +701,7 @@ __device__ __forceinline__ void gemm_tile_body(
             for (int i = 0; i < 4; i++) wring[DIST - 4 + i] = incoming[i];
         }
         __builtin_amdgcn_wave_barrier();  // the wave's reads of this super-block's factors come first
-        decode(hd);
+        decode(hd, nxt);
         __builtin_amdgcn_wave_barrier();
     }
 
@@ -750,7 +782,7 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
     const uint32_t rows = a.offsets ? a.max_rows : a.m;
     const uint32_t m_tiles = (rows + WG_TOK - 1) / WG_TOK, n_tiles = (a.n + WG_ROWS - 1) / WG_ROWS;
     const dim3 grid(8 * ((n_tiles + 7) / 8) * m_tiles, a.offsets ? a.n_experts : 1);
-    const size_t lds = (size_t)(a.k / 32) * WG_TOK * 2;
+    const size_t lds = (size_t)tile_padded_sub_blocks(a.k) * WG_TOK * 2;
     auto kern = &gemm_tile_kernel<F, MT, NT, WM, DIST, DUMP, ADIST>;
     if constexpr (OCC == 3) kern = &gemm_tile_kernel_occ3<F, MT, NT, WM, DIST, DUMP, ADIST>;
     if (lds > 32 * 1024) {  // beyond the default dynamic LDS limit: opt in (up to the 160 KB of a CU)

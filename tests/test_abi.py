@@ -157,6 +157,10 @@ def test_moe_forward_argument_errors_before_touching_the_gpu():
     assert lib.oxq_moe_route_dev(None, None, 1, 2000, 4, 1, None, None, None, None, None, None) == capi.ERR_UNSUPPORTED_SHAPE
     assert lib.oxq_moe_ffn_workspace_bytes(t, t, t, 8, 288, 256) == 0  # the grouped kernel walks 256 columns at a time
     assert lib.oxq_moe_ffn_workspace_bytes(t, t, t, 8, 256, 512) > 0
+    # the formats of independent 32-weight blocks (8: Q8_0) take rows of any whole number of blocks from eight up
+    assert lib.oxq_moe_ffn_workspace_bytes(8, 8, 8, 8, 288, 352) > 0
+    assert lib.oxq_moe_ffn_workspace_bytes(8, 8, 8, 8, 224, 352) == 0
+    assert lib.oxq_moe_ffn_workspace_bytes(8, 8, 8, 8, 300, 352) == 0
 
 
 def test_gemm_workspace_size_is_a_function_of_the_shape():

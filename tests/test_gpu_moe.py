@@ -128,6 +128,20 @@ def expert_weights(t, seed, n_exp, n_rows, n_cols):
                                    (O.Q5_K, O.Q5_K, O.Q5_K)], ids=["q4k_q4k_q6k", "q8_0", "q4_0_iq4xs", "q5k"])
 @pytest.mark.parametrize("shape", [(4, 2, 1, 256, 512), (8, 2, 3, 512, 256), (8, 2, 40, 512, 256), (6, 3, 130, 256, 768)], ids=str)
 def test_moe_ffn_layer(hip, ref, types, shape):
+    _moe_ffn_layer_case(hip, ref, types, shape)
+
+
+@pytest.mark.parametrize("types", [(O.Q8_0, O.Q8_0, O.Q8_0), (O.Q4_0, O.Q5_0, O.Q8_1), (O.Q5_1, O.Q4_1, O.IQ4_NL)],
+                         ids=["q8_0", "q4_0_q5_0_q8_1", "q5_1_q4_1_iq4nl"])
+@pytest.mark.parametrize("shape", [(4, 2, 3, 288, 352), (4, 2, 40, 288, 352), (6, 3, 130, 352, 1408)], ids=str)
+def test_moe_ffn_layer_rows_of_whole_32_blocks(hip, ref, types, shape):
+    """Hidden and intermediate sizes that are multiples of 32 but not of 256 (expert matrices in the 32-weight
+    formats, as GGUF files store tensors whose rows the 256-weight formats cannot take): the same layer, the same
+    bars."""
+    _moe_ffn_layer_case(hip, ref, types, shape)
+
+
+def _moe_ffn_layer_case(hip, ref, types, shape):
     n_exp, top_k, n_tok, hidden, inter = shape
     tg, tu, td = types
     say("moe ffn", [O.NAMES[t] for t in types], shape)
@@ -259,10 +273,11 @@ def test_moe_ffn_with_host_tables_and_errors(hip, ref):
     with pytest.raises(hip.BufferTooSmall) as e:
         moe.moe_ffn_dev(*args, ws[:256])
     assert e.value.needed == ws.numel()
-    with pytest.raises(hip.UnsupportedShape):  # the grouped kernel walks 256 columns at a time
+    with pytest.raises(hip.UnsupportedShape):  # the grouped kernel walks 256 columns at a time: rows of at least that
         moe.moe_ffn_dev((O.Q8_0, args[0][1], stride), (O.Q8_0, args[1][1], stride), (O.Q8_0, args[2][1], stride),
-                        *args[3:-2], 288, inter, ws)
-    assert moe.moe_ffn_workspace_bytes((O.Q8_0, O.Q8_0, O.Q8_0), n_tok * k, 288, inter) == 0
+                        *args[3:-2], 224, inter, ws)
+    assert moe.moe_ffn_workspace_bytes((O.Q8_0, O.Q8_0, O.Q8_0), n_tok * k, 224, inter) == 0
+    assert moe.moe_ffn_workspace_bytes((O.Q8_0, O.Q8_0, O.Q8_0), n_tok * k, 288, inter) > 0
     with pytest.raises(hip.KernelError):  # top_k = 0, moe.rs:168-172
         moe.moe_ffn_dev(*args[:6], 0, *args[7:], ws)
 

@@ -254,10 +254,13 @@ def test_device_route_forms(hip, ref, t):
 
 def test_grouped_form_reports_unsupported(hip):
     z = torch.zeros(4096, dtype=torch.uint8, device=DEV)
-    k = hip.HipKernel(O.Q5_0)  # the tile kernel walks 256 columns at a time
-    assert k.moe_gemm_workspace_bytes(64, 256, 288) == 0
+    k = hip.HipKernel(O.Q5_0)  # the tile kernel walks 256 columns at a time: rows of at least eight blocks
+    assert k.moe_gemm_workspace_bytes(64, 256, 288) > 0
+    assert k.moe_gemm_workspace_bytes(64, 256, 224) == 0
     with pytest.raises(hip.UnsupportedShape):
-        k.moe_gemm_q8_dev(z, 256 * 9 * 22, 1, z, z, 4, 4, z, 256, 288, z)
+        k.moe_gemm_q8_dev(z, 256 * 7 * 22, 1, z, z, 4, 4, z, 256, 224, z)
+    k = hip.HipKernel(O.Q5_K)  # ... and the 256-weight formats whole super-blocks, which the shape check says first
+    assert k.moe_gemm_workspace_bytes(64, 256, 288) == 0
 
 
 def _tile_zero_point(t, acts, rows, k_):
@@ -275,9 +278,24 @@ def _tile_zero_point(t, acts, rows, k_):
 def test_prefill_tile_kernel(hip, ref, tuning, shape, t):
     """The int8-MFMA tile kernel on the added formats: integer sub-block sums bit-exact, fp32 within 1e-5 of
     the reference's fused kernel, every tile shape (split k, 64 x 128, 128 x 64), ragged edges, accumulate."""
-    m, n, k_ = shape
     say("prefill", O.NAMES[t], shape)
     tuning("gemm_tile_min_rows", 1)
+    _prefill_tile_case(hip, ref, shape, t)
+
+
+@pytest.mark.parametrize("shape", [(8, 32, 288), (33, 100, 416), (130, 129, 352), (40, 64, 1408), (450, 140, 480)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("t", [t for t in TILE_TYPES if O.BLOCK[t][0] == 32], ids=ids)
+def test_prefill_tile_kernel_rows_of_whole_32_blocks(hip, ref, tuning, shape, t):
+    """Rows of whole 32-weight blocks that are not whole 256-weight steps, on the added formats of independent
+    blocks: the same bars."""
+    say("prefill, ragged k", O.NAMES[t], shape)
+    tuning("gemm_tile_min_rows", 1)
+    _prefill_tile_case(hip, ref, shape, t)
+
+
+def _prefill_tile_case(hip, ref, shape, t):
+    m, n, k_ = shape
     if True:
         w = O.random_blocks(t, 900 + m, n, k_)
         x = synth.normal_f32(950 + n, m * k_)

@@ -561,6 +561,21 @@ def test_prefill_tile_kernel(hip, ref, tuning, shape, t):
     _prefill_tile_case(hip, ref, shape, t)
 
 
+BLOCKS32 = [t for t in O.ALL_TYPES if O.BLOCK[t][0] == 32]
+
+
+@pytest.mark.parametrize("shape", [(8, 32, 288), (33, 100, 416), (130, 129, 352), (40, 64, 1408), (200, 130, 480),
+                                   (450, 140, 288)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("t", BLOCKS32, ids=lambda t: O.NAMES[t])
+def test_prefill_tile_kernel_rows_of_whole_32_blocks(hip, ref, tuning, shape, t):
+    """Rows that are whole 32-weight blocks but not whole 256-weight steps (the formats of independent blocks):
+    the last step reads the row's last eight blocks and counts only those the step before has not covered.
+    Integer sums bit-exact, fp32 within 1e-5, every tile shape's row count."""
+    say("prefill, ragged k", O.NAMES[t], shape)
+    tuning("gemm_tile_min_rows", 1)
+    _prefill_tile_case(hip, ref, shape, t)
+
+
 def _prefill_tile_case(hip, ref, shape, t):
     import torch
     m, n, k_ = shape
