@@ -19,7 +19,8 @@ Prints ONE JSON line.  Extra objects:
   prefill      batch-512 Q4_K prefill matmul, int8 TOPS vs the 5.0 POPS peak
   moe          IQ4_XS grouped expert matmuls (8 experts, 64 tokens, top-2), weight GB/s
   moe_32_tokens  the same layer for a decode batch of 32 tokens (the few-token grouped kernel)
-  moe_1_token    the same layer for one token (one GEMV launch per projection over the chosen experts)
+  moe_1_token    the same layer for one token (one GEMV launch per projection over the chosen experts);
+                 the MoE legs call oxq_moe_forward_dev and are timed as replayed HIP graphs of six layers
   cpu_baseline the CPU restatement of the reference's fused rows on this host
 """
 import argparse
@@ -674,44 +675,51 @@ def main():
                 moe.moe_forward_dev((IQ4_XS, wg, stride), (IQ4_XS, wu, stride), (IQ4_XS, wd, stride), E, router, xt, NTOK,
                                     TOPK, d_y, H, F, wsm)
 
+            reps = 6
             with torch.cuda.stream(stream):
                 moe_step()
                 stream.synchronize()
                 offsets = wsm[off_at:off_at + 4 * (E + 1)].cpu().numpy().view(np.int32)
-                reps = 6
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record(stream)
                 for _ in range(reps):
                     moe_step()
                 e1.record(stream)
                 e1.synchronize()
-            return e0.elapsed_time(e1) * 1e3 / reps, offsets
+            eager_us = e0.elapsed_time(e1) * 1e3 / reps
+            # the same launches recorded once and replayed, as the decode step above is timed: the figure reported
+            g = capture(lambda: [moe_step() for _ in range(reps)])
+            graph_us = float(np.median([timed_replay(g) for _ in range(3)])) * 1e3 / reps
+            return graph_us, offsets, eager_us
 
         NTOK = 64
         rows = NTOK * TOPK
-        moe_us, offsets = moe_leg(NTOK)
-        small_us, small_offsets = moe_leg(32)
-        one_us, one_offsets = moe_leg(1)
+        moe_us, offsets, moe_eager_us = moe_leg(NTOK)
+        small_us, small_offsets, small_eager_us = moe_leg(32)
+        one_us, one_offsets, one_eager_us = moe_leg(1)
         moe_bytes = 3 * E * stride
         moe_ops = 2 * rows * 3 * F * H
         moe_out = {"workload": "IQ4_XS, 8 experts x (gate, up 14336x4096; down 4096x14336), 64 tokens, top-2 "
                                "(seeded fp32 router), pairs grouped per expert on the device",
                    "pairs": rows, "rows_per_expert": np.diff(offsets).tolist(), "us_per_step": round(moe_us, 1),
+                   "us_per_step_launched_eagerly": round(moe_eager_us, 1),
                    "weight_bytes": moe_bytes, "weight_GBps": round(moe_bytes / moe_us / 1e3, 1),
                    "frac_hbm_peak": round(moe_bytes / moe_us / 1e3 / HBM_PEAK_GBPS, 4),
                    "int8_TOPS": round(moe_ops / moe_us / 1e6, 1),
-                   "timed": "the whole layer: router + softmax + top-2 + grouping, gather + quantize, 3 grouped int8-MFMA "
+                   "timed": "six layers in a replayed HIP graph (median of three replays); the whole layer: router + softmax + top-2 + grouping, gather + quantize, 3 grouped int8-MFMA "
                             "matmuls, SwiGLU + quantize, weighted combine (the 749 MB of expert weights exceed the "
                             "256 MB Infinity Cache, so every step streams them from HBM)"}
         moe_small = {"workload": "the same layer for a decode batch of 32 tokens (64 pairs): with a mean of 8 rows per "
                                  "expert the grouped matmuls take the few-token kernel (16 x 16 x 32 MFMA tiles)",
                      "rows_per_expert": np.diff(small_offsets).tolist(), "us_per_step": round(small_us, 1),
+                     "us_per_step_launched_eagerly": round(small_eager_us, 1),
                      "weight_GBps": round(moe_bytes / small_us / 1e3, 1),
                      "frac_hbm_peak": round(moe_bytes / small_us / 1e3 / HBM_PEAK_GBPS, 4)}
         live = int((np.diff(one_offsets) > 0).sum())
         moe_one = {"workload": "the same layer for ONE token (MoeFfn::forward's own call: top-2, two expert rows): every "
                                "projection is one GEMV launch over the two chosen experts' matrices",
-                   "us_per_step": round(one_us, 1), "experts_read": live, "weight_bytes": 3 * live * stride,
+                   "us_per_step": round(one_us, 1), "us_per_step_launched_eagerly": round(one_eager_us, 1),
+                   "experts_read": live, "weight_bytes": 3 * live * stride,
                    "weight_GBps": round(3 * live * stride / one_us / 1e3, 1),
                    "frac_hbm_peak": round(3 * live * stride / one_us / 1e3 / HBM_PEAK_GBPS, 4)}
         del wg, wu, wd
