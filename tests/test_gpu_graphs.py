@@ -120,3 +120,30 @@ def test_moe_layer_replays(hip, ref):
 
     say("mixture-of-experts layer under graph replay")
     replay_and_compare(hip, record, [out], lambda o: torch.full_like(o, 9.0), between)
+
+
+@pytest.mark.parametrize("n_tok", [1, 24], ids=["one_token", "24_tokens"])
+def test_moe_forward_on_device_pointers_replays(hip, ref, n_tok):
+    """oxq_moe_forward_dev (routing tables in the workspace; for one token the router's launch writes the activation
+    rows too) captured once and replayed over a workspace that eager work overwrites in between."""
+    n_exp, top_k, hidden, inter = 8, 2, 512, 1024
+    t = O.IQ4_XS
+    wg, wu, wd = (np.concatenate([synth.weights(t, s + e, inter if s < 300 else hidden, hidden if s < 300 else inter)
+                                  for e in range(n_exp)]) for s in (100, 200, 300))
+    stride_gu, stride_d = wg.size // n_exp, wd.size // n_exp
+    router = dev(synth.normal_f32(41, n_exp * hidden, 0.05))
+    x = dev(synth.normal_f32(42, n_tok * hidden))
+    ws = torch.empty(moe.moe_forward_workspace_bytes((t, t, t), n_tok, top_k, n_exp, hidden, inter), dtype=torch.uint8,
+                     device=DEV)
+    out = torch.empty(n_tok * hidden, dtype=torch.float32, device=DEV)
+    args = ((t, dev(wg), stride_gu), (t, dev(wu), stride_gu), (t, dev(wd), stride_d), n_exp, router, x, n_tok, top_k, out,
+            hidden, inter)
+
+    def record():
+        moe.moe_forward_dev(*args, ws)
+
+    def between(rep):
+        ws.fill_(rep + 1)
+
+    say("MoeFfn::forward on device pointers under graph replay,", n_tok, "token(s)")
+    replay_and_compare(hip, record, [out], lambda o: torch.full_like(o, 9.0), between)
