@@ -467,7 +467,10 @@ int oxq_moe_ffn_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_strid
  * For one token (the reference's own call) the router's launch also groups the choices and
  * writes the quantized activation rows, so the layer is four launches plus the combine.  No
  * allocation, no synchronisation; needs oxq_moe_forward_workspace_bytes() bytes of 256-byte-
- * aligned scratch (0: no grouped kernel for a type / shape). */
+ * aligned scratch (0: no grouped kernel for a type / shape).  After the call the workspace
+ * starts with the routing tables of oxq_moe_route_dev, each rounded up to 256 bytes: experts
+ * [n_tokens x k] int32 | weights [n_tokens x k] fp32 | row offsets [n_experts + 1] int32 |
+ * pair_token [n_tokens * k] int32 | token_rows [n_tokens x k] int32 (k = min(top_k, n_experts)). */
 size_t oxq_moe_forward_workspace_bytes(uint32_t gate_type, uint32_t up_type, uint32_t down_type,
                                        size_t n_tokens, size_t top_k, size_t n_experts,
                                        size_t hidden, size_t intermediate);
