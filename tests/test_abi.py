@@ -184,3 +184,12 @@ def test_gemm_workspace_size_is_a_function_of_the_shape():
     assert w(q4k, 16, 128256, 4096) == planes(16, 4096)                                # 1002 groups fill the chip
     assert w(q4k, 512, 14336, 4096) == planes(512, 4096)
     assert w(q4k, 16, 14336, 4000) == 0                                                # k not a multiple of 256
+    # the formats of independent 32-weight blocks: any whole number of blocks from eight up, planes padded to whole
+    # groups of eight blocks
+    q8_0, q5_0 = 8, 6
+    assert w(q8_0, 64, 4864, 896) == planes(64, 1024)
+    assert w(q5_0, 64, 896, 4864) == planes(64, 4864)                                  # 152 blocks: whole groups
+    assert w(q8_0, 64, 4864, 288) == planes(64, 512)
+    assert w(q8_0, 64, 4864, 224) == 0                                                 # fewer than eight blocks
+    assert w(q8_0, 64, 4864, 300) == 0                                                 # ends inside a block
+    assert w(q6k, 64, 4864, 288) == 0
