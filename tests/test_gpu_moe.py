@@ -392,6 +392,22 @@ def test_moe_layer_full_size_c5(hip, ref):
             eo = ref.matvec_q8_fused_mt(t, wd[e * stride:(e + 1) * stride], hq, hidden, inter, 16)
             acc = acc + weights[tk, j] * eo
         assert_close(got[tk], acc, f"token {tk}", tol=2e-3)
+    # the one-call entry point at the same size: the same bits for the batch; and the reference's own call, one
+    # token (router launch that also groups and writes the activation rows, one GEMV launch per projection over the
+    # two chosen experts), against the same oracle result
+    say("moe layer C5 full size: oxq_moe_forward_dev, 64 tokens and one token")
+    d_router, d_x = dev(router), dev(x)
+    ws2 = torch.empty(moe.moe_forward_workspace_bytes((t, t, t), n_tok, top_k, n_exp, hidden, inter), dtype=torch.uint8,
+                      device=DEV)
+    d_out2 = torch.full((n_tok * hidden,), 7.0, dtype=torch.float32, device=DEV)
+    moe.moe_forward_dev((t, d_wg, stride), (t, d_wu, stride), (t, d_wd, stride), n_exp, d_router, d_x, n_tok, top_k, d_out2,
+                        hidden, inter, ws2)
+    assert np.array_equal(host(d_out2).view(np.uint32), got.ravel().view(np.uint32))
+    one = torch.full((hidden,), 7.0, dtype=torch.float32, device=DEV)
+    moe.moe_forward_dev((t, d_wg, stride), (t, d_wu, stride), (t, d_wd, stride), n_exp, d_router, d_x[63 * hidden:], 1, top_k,
+                        one, hidden, inter, ws2)
+    assert_close(host(one), acc, "token 63 alone", tol=2e-3)
+    assert_close(host(one), got[63], "token 63 alone against its row of the batch", tol=2e-3)
 
 
 @pytest.mark.parametrize("cfg", [(8, 2, 1, 512, 256, O.IQ4_XS), (8, 1, 1, 256, 512, O.Q4_K), (8, 8, 1, 256, 256, O.Q6_K),
