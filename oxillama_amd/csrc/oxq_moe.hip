@@ -23,8 +23,8 @@ namespace oxq {
 // ONE (a launch for a single token, k <= n_exp): the work group goes on to what the grouping and
 // the gather kernels would do for that token -- the k chosen experts in ascending order are the
 // grouped rows (offsets[e] = how many chosen experts lie below e), every row belongs to token 0,
-// and each row's activations are the token's Q8_0 blocks, written k times.  Same tables and bytes
-// as the separate launches.
+// and each row's activations are the token's Q8_0 blocks, written k times while the logits are
+// formed.  Same tables and bytes as the separate launches.
 template <bool ONE>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict__ router, const float *__restrict__ x,
                                                        int32_t *__restrict__ experts, float *__restrict__ weights,
@@ -53,6 +53,13 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict_
 #pragma unroll
                 for (int q = 0; q < EP; q++)
                     for (int i = 0; i < 4; i++) acc[q] += rv[q][i] * xv[i];
+                if (ONE && e0 == 0) {
+                    // the activation rows are k copies of the token's Q8_0 blocks whichever experts get chosen:
+                    // written from the values in hand (eight consecutive lanes hold one block, as in the quantizer;
+                    // hidden is a multiple of 32 here, so a block's lanes are in the loop together)
+                    for (uint32_t r = 0; r < k; r++)
+                        encode_q8_0_lanes(xv, true, acts + ((size_t)r * (hidden / 32) + c / 8) * 34, c & 7);
+                }
             }
         } else {
             for (uint32_t c = threadIdx.x; c < hidden; c += 256)
@@ -127,14 +134,6 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict_
         for (uint32_t r = 0; r < k; r++) row += chosen[r] < chosen[p] ? 1 : 0;
         token_rows[p] = row;
         pair_token[row] = 0;
-    }
-    const uint32_t bpr = hidden / 32, j = threadIdx.x & 7;
-    for (uint32_t b0 = 0; b0 < bpr; b0 += 32) {  // eight lanes per block as in the quantizer
-        const uint32_t b = b0 + (threadIdx.x >> 3);
-        const bool valid = b < bpr;
-        float v[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-        if (valid) load4(v, xr + (size_t)b * 32 + 4 * j);
-        for (uint32_t r = 0; r < k; r++) encode_q8_0_lanes(v, valid, acts + ((size_t)r * bpr + b) * 34, j);
     }
 }
 
