@@ -264,6 +264,9 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra-kernels", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--moe-tile-only", action="store_true",
+                    help="run the 64-token MoE leg's grouped matmuls on the tile kernel alone (for profiles that set it "
+                         "beside the few-token kernel)")
     ap.add_argument("--unfused-swiglu", action="store_true",
                     help="gate + up in one launch, SwiGLU + quantize in a second (default: all of it in one launch)")
     ap.add_argument("--fused-quantize", action="store_true",
@@ -664,7 +667,15 @@ def main():
         router = torch.from_numpy(synth.normal_f32(9, E * H, 0.05)).to(dev)
         types3 = (IQ4_XS, IQ4_XS, IQ4_XS)
 
-        def moe_leg(NTOK):
+        def moe_leg(NTOK, tile_only=False):
+            from oxillama_amd import capi
+            capi.load().oxq_set_gemm_variant(99 if tile_only else 0)  # 99: the tile kernel's own choice of shape
+            try:
+                return moe_leg_timed(NTOK)
+            finally:
+                capi.load().oxq_set_gemm_variant(0)
+
+        def moe_leg_timed(NTOK):
             xt = torch.from_numpy(synth.normal_f32(7, NTOK * H)).to(dev)
             rows = NTOK * TOPK
             d_y = torch.empty(NTOK * H, dtype=torch.float32, device=dev)
@@ -694,13 +705,14 @@ def main():
 
         NTOK = 64
         rows = NTOK * TOPK
-        moe_us, offsets, moe_eager_us = moe_leg(NTOK)
+        moe_us, offsets, moe_eager_us = moe_leg(NTOK, args.moe_tile_only)
         small_us, small_offsets, small_eager_us = moe_leg(32)
         one_us, one_offsets, one_eager_us = moe_leg(1)
         moe_bytes = 3 * E * stride
         moe_ops = 2 * rows * 3 * F * H
         moe_out = {"workload": "IQ4_XS, 8 experts x (gate, up 14336x4096; down 4096x14336), 64 tokens, top-2 "
-                               "(seeded fp32 router), pairs grouped per expert on the device",
+                               "(seeded fp32 router), pairs grouped per expert on the device"
+                               + (" [--moe-tile-only: grouped matmuls on the tile kernel alone]" if args.moe_tile_only else ""),
                    "pairs": rows, "rows_per_expert": np.diff(offsets).tolist(), "us_per_step": round(moe_us, 1),
                    "us_per_step_launched_eagerly": round(moe_eager_us, 1),
                    "weight_bytes": moe_bytes, "weight_GBps": round(moe_bytes / moe_us / 1e3, 1),

@@ -443,8 +443,9 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 // Measured on MI355X, 8 experts of Mixtral's shapes (IQ4_XS; Q4_K alike), cold weights, against the tile kernel:
 //  * up to 16 rows per expert: 14336 x 4096 84 us against 106, 4096 x 14336 90 against 107;
 //  * 17..32 rows: two token tiles double the arithmetic per weight byte.  With a mean of 12 rows (most experts still
-//    one tile) 14336 x 4096 takes 88 us against 102; with a mean of 16 it is 98-107 against 101-106, no gain, and
-//    4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106;
+//    one tile) 14336 x 4096 takes 88 us against 102; with a mean of 16 the kernel alone is 99 us against 103, and
+//    the tile kernel's token re-layout launch (5 us) is not needed: the layer of 64 tokens 316-324 us against
+//    340-343; 4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106;
 //  * one matrix, no experts, up to 16 token rows: too few row groups as it is (14336 x 4096: 24 us against 19);
 //    with k split over work groups and the splits added by a second launch (call totals, with the token re-layout):
 //    14336 x 4096 18.0 us against 19.6, 4096 x 14336 21.4 against 29.5, 28672 x 8192 40 against 49; 4096 x 4096
@@ -469,8 +470,8 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
                 return (has_partial && skinny_splits(a.n, a.k) >= 2) ? SK_1_4_SPLIT : SK_NONE;
             }
             const bool many = (size_t)((a.n + 127) / 128) * a.n_experts >= 2 * (size_t)device_cus();
-            // two token tiles: only with many row groups and a mean of at most 12 rows per expert
-            if (two) return (many && 4 * (size_t)a.m <= 3 * 16 * (size_t)a.n_experts) ? SK_2_2 : SK_NONE;
+            // two token tiles: only with many row groups and a mean of at most 16 rows per expert
+            if (two) return (many && (size_t)a.m <= 16 * (size_t)a.n_experts) ? SK_2_2 : SK_NONE;
             // (the debug dump: one shape per token-tile count; every shape adds a result's terms in the same order)
             return (many || a.sums) ? SK_1_4 : SK_1_8;
         }

@@ -57,7 +57,7 @@ def _run(hip, t, w, acts, offsets, n, k_, max_rows, sums=False, accumulate=False
 
 
 # (row counts per expert, n, k, max_rows handed to the call): one token tile / two (the default takes two only with
-# many row groups and a mean of at most 12 rows per expert); few row groups / at least two per compute unit; an expert without rows; ragged n (a wave past the last row, a tile cut at n % 16); k of one step, of a
+# many row groups and a mean of at most 16 rows per expert); few row groups / at least two per compute unit; an expert without rows; ragged n (a wave past the last row, a tile cut at n % 16); k of one step, of a
 # whole number of chunks and with a short last chunk; groups larger than the launch is shaped for (max_rows = 0: the
 # shape follows twice the mean, the largest group takes further passes over its weights)
 CASES = [
