@@ -123,13 +123,13 @@ constexpr int skinny_waves_per_simd() {
     return lds <= 80 * 1024 ? WAVES / 2 : WAVES / 4;
 }
 
+// The work of one work group on the token rows tokb .. tok_end - 1 (at most 16 * TT of them) of its group.
 template <class F, int NT, int WAVES, int TT, int PER, bool DUMP>
-__global__ __launch_bounds__(64 * WAVES)
-__attribute__((amdgpu_waves_per_eu(skinny_waves_per_simd<F, NT, WAVES, TT, PER>(), skinny_waves_per_simd<F, NT, WAVES, TT, PER>())))
-void gemm_skinny_kernel(
+__device__ __forceinline__ void gemm_skinny_body(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ A, float *__restrict__ out, int32_t *__restrict__ sums,
     uint32_t m, uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
-    float *__restrict__ partial, uint32_t sb_per_split) {
+    float *__restrict__ partial, uint32_t sb_per_split, const uint32_t tokb, const uint32_t tok_end, const uint32_t rg,
+    const uint32_t gy) {
     using S = Skinny<F>;
     constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: as_float(0x4B400000 + i) == MAGIC + i for |i| < 2^22
     constexpr uint32_t RS = S::ROW_STRIDE, SEG = 2 * S::BLOCK, PPR = SEG / 16;  // 16-byte pieces per row per step
@@ -139,17 +139,8 @@ void gemm_skinny_kernel(
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lane = threadIdx.x & 63, c = lane & 15, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    uint32_t tok0 = 0, tok_end = m;
-    if (offsets) {
-        tok0 = (uint32_t)offsets[blockIdx.y];
-        tok_end = (uint32_t)offsets[blockIdx.y + 1];
-    }
-    // blockIdx.z = which 16 * TT token rows of the group: the launch is shaped for the usual group, a larger one
-    // takes further work groups per row group (each its own pass over the weights); the rest exit here
-    const uint32_t tokb = tok0 + blockIdx.z * (16 * TT);
-    if (tokb >= tok_end) return;  // the whole work group
     // super-blocks [sb_lo, n_super) of this work group (all of k, or its split)
-    const uint32_t sb_lo = partial ? blockIdx.y * sb_per_split : 0;
+    const uint32_t sb_lo = partial ? gy * sb_per_split : 0;
     const uint32_t n_super = partial ? min(k / 256, sb_lo + sb_per_split) : k / 256;
     constexpr uint32_t per = PER, nblk_max = PER * 8;  // sub-blocks (Q8_0 blocks per token) of a full chunk
     uint8_t *const ldsA = lds;
@@ -209,9 +200,9 @@ void gemm_skinny_kernel(
         }
     };
 
-    const uint32_t rbase = (blockIdx.x * WAVES + wave) * (16 * NT);
+    const uint32_t rbase = (rg * WAVES + wave) * (16 * NT);
     const bool active = rbase < n;  // a wave past the last row still stages tokens and meets the barriers
-    const uint8_t *We = W + (offsets ? (size_t)blockIdx.y * w_stride : 0);
+    const uint8_t *We = W + (offsets ? (size_t)gy * w_stride : 0);
     const size_t row_bytes = (size_t)(k / 256) * S::BLOCK;
     // the lane's pieces of a step: where they come from (less the step's offset) and where they go
     const uint8_t *src[NL];
@@ -354,7 +345,7 @@ void gemm_skinny_kernel(
                 if (row < n && tok < tok_end && t < (int)tiles_here) {
                     const float y = acc[t][j][v];
                     if (partial) {
-                        partial[((size_t)blockIdx.y * m + tok) * n + row] = y;
+                        partial[((size_t)gy * m + tok) * n + row] = y;
                     } else {
                         float *o = out + (size_t)tok * n + row;
                         *o = accumulate ? *o + y : bias ? y + bias[row] : y;
@@ -362,6 +353,37 @@ void gemm_skinny_kernel(
                 }
             }
         }
+}
+
+// The kernel: finds the work group's token rows and runs the body.  A launch shaped for two token tiles runs the
+// one-tile body (same LDS bytes: twice the chunk length) for a group that has rows in the first tile only -- the
+// branch-free step instead of the two-tile step's branches, for what is most of the groups when the mean is 16 rows.
+template <class F, int NT, int WAVES, int TT, int PER, bool DUMP>
+__global__ __launch_bounds__(64 * WAVES)
+__attribute__((amdgpu_waves_per_eu(skinny_waves_per_simd<F, NT, WAVES, TT, PER>(), skinny_waves_per_simd<F, NT, WAVES, TT, PER>())))
+void gemm_skinny_kernel(
+    const uint8_t *__restrict__ W, const uint8_t *__restrict__ A, float *__restrict__ out, int32_t *__restrict__ sums,
+    uint32_t m, uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
+    float *__restrict__ partial, uint32_t sb_per_split) {
+    const uint32_t rg = blockIdx.x, gy = blockIdx.y;  // row group; expert (grouped form) or split of k
+    uint32_t tok0 = 0, tok_end = m;
+    if (offsets) {
+        tok0 = (uint32_t)offsets[gy];
+        tok_end = (uint32_t)offsets[gy + 1];
+    }
+    // blockIdx.z = which 16 * TT token rows of the group: the launch is shaped for the usual group, a larger one
+    // takes further work groups per row group (each its own pass over the weights); the rest exit here
+    const uint32_t tokb = tok0 + blockIdx.z * (16 * TT);
+    if (tokb >= tok_end) return;  // the whole work group
+    if constexpr (TT == 2) {
+        if (tok_end - tokb <= 16) {
+            gemm_skinny_body<F, NT, WAVES, 1, 2 * PER, DUMP>(W, A, out, sums, m, n, k, accumulate, bias, offsets, w_stride,
+                                                            partial, sb_per_split, tokb, tok_end, rg, gy);
+            return;
+        }
+    }
+    gemm_skinny_body<F, NT, WAVES, TT, PER, DUMP>(W, A, out, sums, m, n, k, accumulate, bias, offsets, w_stride, partial,
+                                                  sb_per_split, tokb, tok_end, rg, gy);
 }
 
 // out[i] (+)= partial[0][i] + partial[1][i] + ... in that order, i over m x n; bias[row] instead of the old value
@@ -419,8 +441,8 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
     const uint32_t splits = split_k ? skinny_splits(a.n, a.k) : 1;
     float *const partial = splits > 1 ? p.partial : nullptr;
     if (splits > 1 && (a.offsets || !partial)) return hipErrorNotSupported;
-    const dim3 grid((a.n + 16 * NT * WAVES - 1) / (16 * NT * WAVES), a.offsets ? a.n_experts : splits,
-                    (group_rows + 16 * TT - 1) / (16 * TT));
+    const uint32_t row_groups = (a.n + 16 * NT * WAVES - 1) / (16 * NT * WAVES);
+    const dim3 grid(row_groups, a.offsets ? a.n_experts : splits, (group_rows + 16 * TT - 1) / (16 * TT));
     if (grid.z > 65535) return hipErrorNotSupported;
     note_launch("gemm_skinny_kernel", F::TYPE, NT, WAVES, TT, PER, grid.x, grid.y * grid.z, 64 * WAVES);
     hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES), lds, stream, a.W, a.A, a.out, a.sums, a.m, a.n, a.k,
@@ -443,8 +465,8 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 // Measured on MI355X, 8 experts of Mixtral's shapes (IQ4_XS; Q4_K alike), cold weights, against the tile kernel:
 //  * up to 16 rows per expert: 14336 x 4096 84 us against 106, 4096 x 14336 90 against 107;
 //  * 17..32 rows: two token tiles double the arithmetic per weight byte.  With a mean of 12 rows (most experts still
-//    one tile) 14336 x 4096 takes 88 us against 102; with a mean of 16 the kernel alone is 99 us against 103, and
-//    the tile kernel's token re-layout launch (5 us) is not needed: the layer of 64 tokens 316-324 us against
+//    one tile) 14336 x 4096 takes 88 us against 102; with a mean of 16 the kernel alone is 93 us against 103, and
+//    the tile kernel's token re-layout launch (5 us) is not needed: the layer of 64 tokens 311-317 us against
 //    340-343; 4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106;
 //  * one matrix, no experts, up to 16 token rows: too few row groups as it is (14336 x 4096: 24 us against 19);
 //    with k split over work groups and the splits added by a second launch (call totals, with the token re-layout):
