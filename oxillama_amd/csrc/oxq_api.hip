@@ -981,10 +981,10 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
 }
 
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k) {
-    (void)n;
-    if (total_rows > 0x7FFFFFFFull || k > 0xFFFFFFFFull || !oxq::gemm_tiles_supported(type, (uint32_t)total_rows, (uint32_t)k))
+    if (total_rows > 0x7FFFFFFFull || k > 0xFFFFFFFFull || n > 0xFFFFFFFFull ||
+        !oxq::gemm_tiles_supported(type, (uint32_t)total_rows, (uint32_t)k))
         return 0;
-    return oxq::gemm_workspace_bytes((uint32_t)total_rows, (uint32_t)k);
+    return oxq::gemm_grouped_workspace_bytes((uint32_t)total_rows, (uint32_t)k, (uint32_t)n, type);
 }
 
 // prepared_for: format id of an immediately preceding call on the same activations and workspace (0: none).
@@ -1014,6 +1014,7 @@ static int moe_gemm_impl(uint32_t type, const uint8_t *d_weights, size_t expert_
     ga.out = d_out;
     ga.sums = d_sums;
     ga.workspace = (uint8_t *)d_workspace;
+    ga.workspace_bytes = workspace_bytes;
     ga.m = (uint32_t)total_rows;
     ga.n = (uint32_t)n;
     ga.k = (uint32_t)k;

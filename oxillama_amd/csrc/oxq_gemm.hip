@@ -65,6 +65,18 @@ static size_t gemm_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t
     const uint32_t splits = skinny_splits(n, k);
     return splits > 1 ? (size_t)splits * m * n * sizeof(float) : 0;
 }
+// The same for the grouped form, which splits k in two where an expert's matrix has few row groups: a function of
+// (type, rows, n, k) only, as the caller sizes the workspace without the number of experts.
+static size_t gemm_grouped_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
+    if ((type != OXQ_TYPE_Q4_K && type != OXQ_TYPE_IQ4_XS) || k % 1024 != 0 || n == 0 || n > SKINNY_GROUPED_SPLIT_MAX_N)
+        return 0;
+    const size_t bytes = (size_t)2 * m * n * sizeof(float);
+    return bytes <= ((size_t)64 << 20) ? bytes : 0;
+}
+size_t gemm_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t type) {
+    const size_t planes = (gemm_planes_bytes(m, k) + 255) & ~(size_t)255;
+    return planes + gemm_grouped_partial_bytes(type, m, n, k);
+}
 size_t gemm_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t type) {
     const size_t planes = (gemm_planes_bytes(m, k) + 255) & ~(size_t)255;
     return planes + gemm_partial_bytes(type, m, n, k);
@@ -161,6 +173,9 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
     TilePlan plan = {q8t, P, da16, mpad};
     if (!a.offsets && gemm_partial_bytes(type, a.m, a.n, a.k) &&
         a.workspace_bytes >= gemm_workspace_bytes(a.m, a.k, a.n, type))
+        plan.partial = reinterpret_cast<float *>(a.workspace + ((gemm_planes_bytes(a.m, a.k) + 255) & ~(size_t)255));
+    if (a.offsets && gemm_grouped_partial_bytes(type, a.m, a.n, a.k) &&
+        a.workspace_bytes >= gemm_grouped_workspace_bytes(a.m, a.k, a.n, type))
         plan.partial = reinterpret_cast<float *>(a.workspace + ((gemm_planes_bytes(a.m, a.k) + 255) & ~(size_t)255));
     // The few-token kernel (oxq_gemm_skinny.hpp), where it pays: it reads the caller's Q8_0 rows itself, no re-layout.
     const int variant = g_gemm_variant.load(std::memory_order_relaxed);

@@ -129,7 +129,7 @@ __device__ __forceinline__ void gemm_skinny_body(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ A, float *__restrict__ out, int32_t *__restrict__ sums,
     uint32_t m, uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
     float *__restrict__ partial, uint32_t sb_per_split, const uint32_t tokb, const uint32_t tok_end, const uint32_t rg,
-    const uint32_t gy) {
+    const uint32_t gy, const uint32_t ks) {
     using S = Skinny<F>;
     constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: as_float(0x4B400000 + i) == MAGIC + i for |i| < 2^22
     constexpr uint32_t RS = S::ROW_STRIDE, SEG = 2 * S::BLOCK, PPR = SEG / 16;  // 16-byte pieces per row per step
@@ -140,7 +140,7 @@ __device__ __forceinline__ void gemm_skinny_body(
     const uint32_t lane = threadIdx.x & 63, c = lane & 15, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     // super-blocks [sb_lo, n_super) of this work group (all of k, or its split)
-    const uint32_t sb_lo = partial ? gy * sb_per_split : 0;
+    const uint32_t sb_lo = partial ? ks * sb_per_split : 0;
     const uint32_t n_super = partial ? min(k / 256, sb_lo + sb_per_split) : k / 256;
     constexpr uint32_t per = PER, nblk_max = PER * 8;  // sub-blocks (Q8_0 blocks per token) of a full chunk
     uint8_t *const ldsA = lds;
@@ -345,7 +345,7 @@ __device__ __forceinline__ void gemm_skinny_body(
                 if (row < n && tok < tok_end && t < (int)tiles_here) {
                     const float y = acc[t][j][v];
                     if (partial) {
-                        partial[((size_t)gy * m + tok) * n + row] = y;
+                        partial[((size_t)ks * m + tok) * n + row] = y;
                     } else {
                         float *o = out + (size_t)tok * n + row;
                         *o = accumulate ? *o + y : bias ? y + bias[row] : y;
@@ -364,8 +364,12 @@ __attribute__((amdgpu_waves_per_eu(skinny_waves_per_simd<F, NT, WAVES, TT, PER>(
 void gemm_skinny_kernel(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ A, float *__restrict__ out, int32_t *__restrict__ sums,
     uint32_t m, uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
-    float *__restrict__ partial, uint32_t sb_per_split) {
-    const uint32_t rg = blockIdx.x, gy = blockIdx.y;  // row group; expert (grouped form) or split of k
+    float *__restrict__ partial, uint32_t sb_per_split, uint32_t grouped_splits) {
+    // row group; expert (grouped form); split of k: blockIdx.y is the expert, or the split (one matrix), or, in the
+    // grouped form with k split, expert * grouped_splits + split
+    const uint32_t rg = blockIdx.x;
+    const uint32_t gy = !offsets ? 0 : partial ? blockIdx.y / grouped_splits : blockIdx.y;
+    const uint32_t ks = !partial ? 0 : offsets ? blockIdx.y % grouped_splits : blockIdx.y;
     uint32_t tok0 = 0, tok_end = m;
     if (offsets) {
         tok0 = (uint32_t)offsets[gy];
@@ -378,12 +382,12 @@ void gemm_skinny_kernel(
     if constexpr (TT == 2) {
         if (tok_end - tokb <= 16) {
             gemm_skinny_body<F, NT, WAVES, 1, 2 * PER, DUMP>(W, A, out, sums, m, n, k, accumulate, bias, offsets, w_stride,
-                                                            partial, sb_per_split, tokb, tok_end, rg, gy);
+                                                            partial, sb_per_split, tokb, tok_end, rg, gy, ks);
             return;
         }
     }
     gemm_skinny_body<F, NT, WAVES, TT, PER, DUMP>(W, A, out, sums, m, n, k, accumulate, bias, offsets, w_stride, partial,
-                                                  sb_per_split, tokb, tok_end, rg, gy);
+                                                  sb_per_split, tokb, tok_end, rg, gy, ks);
 }
 
 // out[i] (+)= partial[0][i] + partial[1][i] + ... in that order, i over m x n; bias[row] instead of the old value
@@ -427,6 +431,10 @@ static inline uint32_t skinny_splits(uint32_t n, uint32_t k) {
     return per ? (k / 256 + per - 1) / per : 1;
 }
 
+// Grouped form: an expert's k is split in two where its matrix has too few row groups to fill the chip by experts
+// alone (at most this many rows per expert; the workspace size follows the same bound).
+constexpr uint32_t SKINNY_GROUPED_SPLITS = 2, SKINNY_GROUPED_SPLIT_MAX_N = 8192;
+
 template <class F, int NT, int WAVES, int TT, int PER, bool DUMP = false>
 static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipStream_t stream, bool split_k = false) {
     using S = Skinny<F>;
@@ -438,15 +446,18 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
     if (e != hipSuccess) return e;
     // token passes: as many as the largest group can need (max_rows is the caller's bound, all rows if unknown)
     const uint32_t group_rows = a.offsets ? a.max_rows : a.m;
-    const uint32_t splits = split_k ? skinny_splits(a.n, a.k) : 1;
+    const uint32_t splits = !split_k ? 1 : a.offsets ? SKINNY_GROUPED_SPLITS : skinny_splits(a.n, a.k);
     float *const partial = splits > 1 ? p.partial : nullptr;
-    if (splits > 1 && (a.offsets || !partial)) return hipErrorNotSupported;
+    if (splits > 1 && !partial) return hipErrorNotSupported;
+    // super-blocks per split: the grouped form halves k (a multiple of 1024: whole steps in both halves)
+    const uint32_t sb_per_split = a.offsets ? a.k / 256 / SKINNY_GROUPED_SPLITS : skinny_sb_per_split(a.n, a.k);
+    if (splits > 1 && a.offsets && a.k % (512 * SKINNY_GROUPED_SPLITS) != 0) return hipErrorNotSupported;
     const uint32_t row_groups = (a.n + 16 * NT * WAVES - 1) / (16 * NT * WAVES);
-    const dim3 grid(row_groups, a.offsets ? a.n_experts : splits, (group_rows + 16 * TT - 1) / (16 * TT));
-    if (grid.z > 65535) return hipErrorNotSupported;
+    const dim3 grid(row_groups, a.offsets ? a.n_experts * splits : splits, (group_rows + 16 * TT - 1) / (16 * TT));
+    if (grid.z > 65535 || grid.y > 65535) return hipErrorNotSupported;
     note_launch("gemm_skinny_kernel", F::TYPE, NT, WAVES, TT, PER, grid.x, grid.y * grid.z, 64 * WAVES);
     hipLaunchKernelGGL(kern, grid, dim3(64 * WAVES), lds, stream, a.W, a.A, a.out, a.sums, a.m, a.n, a.k,
-                       a.accumulate, a.bias, a.offsets, a.w_stride, partial, skinny_sb_per_split(a.n, a.k));
+                       a.accumulate, a.bias, a.offsets, a.w_stride, partial, sb_per_split, splits);
     e = hipGetLastError();
     if (e != hipSuccess || !partial) return e;
     const size_t total = (size_t)a.m * a.n;
@@ -467,13 +478,15 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 //  * 17..32 rows: two token tiles double the arithmetic per weight byte.  With a mean of 12 rows (most experts still
 //    one tile) 14336 x 4096 takes 88 us against 102; with a mean of 16 the kernel alone is 93 us against 103, and
 //    the tile kernel's token re-layout launch (5 us) is not needed: the layer of 64 tokens 311-317 us against
-//    340-343; 4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106;
+//    340-343; 4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106,
+//    and with each expert's k in two halves (twice the work groups, a reduction launch) 90 + 5 against 103 + 5: the
+//    layer 293-298 us;
 //  * one matrix, no experts, up to 16 token rows: too few row groups as it is (14336 x 4096: 24 us against 19);
 //    with k split over work groups and the splits added by a second launch (call totals, with the token re-layout):
 //    14336 x 4096 18.0 us against 19.6, 4096 x 14336 21.4 against 29.5, 28672 x 8192 40 against 49; 4096 x 4096
 //    14.4 against 12.3 (not taken below 2^25 weights); 17..32 rows 24.6 against 19.7 (not taken).  From 512 row
 //    groups on no split is needed (57344 x 4096, 16 rows: 44 us against 56).
-enum SkinnyShape { SK_NONE = 0, SK_1_4, SK_1_8, SK_2_2, SK_1_4_SPLIT, SK_1_16, SK_2_8, SK_W4_1_8, SK_W4_2_4, SK_2_4 };
+enum SkinnyShape { SK_NONE = 0, SK_1_4, SK_1_8, SK_2_2, SK_1_4_SPLIT, SK_1_16, SK_2_8, SK_W4_1_8, SK_W4_2_4, SK_2_4, SK_2_2_SPLIT };
 
 template <class F>
 static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int variant) {
@@ -493,7 +506,15 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
             }
             const bool many = (size_t)((a.n + 127) / 128) * a.n_experts >= 2 * (size_t)device_cus();
             // two token tiles: only with many row groups and a mean of at most 16 rows per expert
-            if (two) return (many && (size_t)a.m <= 16 * (size_t)a.n_experts) ? SK_2_2 : SK_NONE;
+            if (two) {
+                if ((size_t)a.m > 16 * (size_t)a.n_experts) return SK_NONE;
+                if (many) return SK_2_2;
+                // few row groups per expert: each expert's k in two halves, where that gives every compute unit a
+                // work group and the workspace has room for the halves' sums
+                const bool can_split = has_partial && a.n <= SKINNY_GROUPED_SPLIT_MAX_N && a.k % 1024 == 0 &&
+                                       (size_t)((a.n + 127) / 128) * a.n_experts * SKINNY_GROUPED_SPLITS >= device_cus();
+                return can_split ? SK_2_2_SPLIT : SK_NONE;
+            }
             // (the debug dump: one shape per token-tile count; every shape adds a result's terms in the same order)
             return (many || a.sums) ? SK_1_4 : SK_1_8;
         }
@@ -517,6 +538,8 @@ static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_
         case SK_2_2: return a.sums ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream);
         case SK_1_4_SPLIT:
             return a.sums ? launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream, true) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream, true);
+        case SK_2_2_SPLIT:
+            return a.sums ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream, true) : launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream, true);
         case SK_1_8: return launch_skinny_shape<F, 1, 8, 1, 8>(a, p, stream);
         case SK_1_16: return launch_skinny_shape<F, 1, 8, 1, 16>(a, p, stream);
         case SK_2_8: return launch_skinny_shape<F, 1, 8, 2, 8>(a, p, stream);

@@ -183,6 +183,9 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
 // With n and the format: plus, for a matmul of at most 32 token rows that the few-token kernel would split over k,
 // the room for its per-split sums (behind the re-tiled activations, 256-byte aligned).
 size_t gemm_workspace_bytes(uint32_t m, uint32_t k, uint32_t n = 0, uint32_t type = 0);
+// ... of the grouped form: the planes, plus room for two per-split sums of [m x n] where the few-token kernel may
+// split an expert's k in two (Q4_K / IQ4_XS, k a multiple of 1024, at most 8192 rows per expert).
+size_t gemm_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t type);
 // Tuning knobs (oxq_tuning.h), read once per call.
 extern std::atomic<int> g_gemm_variant;              // 0 = default tile shape
 extern std::atomic<uint32_t> g_gemm_tile_min_rows;   // 0 = default threshold

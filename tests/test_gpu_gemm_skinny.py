@@ -57,7 +57,7 @@ def _run(hip, t, w, acts, offsets, n, k_, max_rows, sums=False, accumulate=False
 
 
 # (row counts per expert, n, k, max_rows handed to the call): one token tile / two (the default takes two only with
-# many row groups and a mean of at most 16 rows per expert); few row groups / at least two per compute unit; an expert without rows; ragged n (a wave past the last row, a tile cut at n % 16); k of one step, of a
+# many row groups, or enough for every compute unit once k is halved, and a mean of at most 16 rows per expert); few row groups / at least two per compute unit; an expert without rows; ragged n (a wave past the last row, a tile cut at n % 16); k of one step, of a
 # whole number of chunks and with a short last chunk; groups larger than the launch is shaped for (max_rows = 0: the
 # shape follows twice the mean, the largest group takes further passes over its weights)
 CASES = [
@@ -69,6 +69,10 @@ CASES = [
     ([32, 1, 17, 0, 8, 30, 2, 5], 8200, 512, 32),
     ([2, 1, 40, 1, 3, 0, 1, 2], 96, 1024, 0),
     ([9, 50, 3, 2, 1, 0, 20, 5], 8192, 512, 0),
+    # two token tiles on few row groups per expert: each expert's k in two halves, the halves' sums added by a second
+    # launch (one step per half; several chunks per half and groups of unknown size)
+    ([20, 3, 17, 0, 32, 16, 9, 25], 2048, 1024, 32),
+    ([22, 10, 17, 13, 20, 16, 9, 15], 4096, 3072, 0),
 ]
 
 
