@@ -480,7 +480,7 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 //    the tile kernel's token re-layout launch (5 us) is not needed: the layer of 64 tokens 311-317 us against
 //    340-343; 4096 x 14336 (one work group per compute unit, the longer per-step chain uncovered) 126 against 106,
 //    and with each expert's k in two halves (twice the work groups, a reduction launch) 90 + 5 against 103 + 5: the
-//    layer 293-298 us;
+//    layer 293-303 us;
 //  * one matrix, no experts, up to 16 token rows: too few row groups as it is (14336 x 4096: 24 us against 19);
 //    with k split over work groups and the splits added by a second launch (call totals, with the token re-layout):
 //    14336 x 4096 18.0 us against 19.6, 4096 x 14336 21.4 against 29.5, 28672 x 8192 40 against 49; 4096 x 4096
