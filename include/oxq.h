@@ -307,7 +307,8 @@ int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8
  * group size: fp32 summation order, hence the last bits, can differ between two bounds; every
  * choice meets the 1e-5 bar).  k must be a multiple of 256 (the formats of 32-weight blocks: of
  * 32, and at least 256); needs oxq_moe_gemm_q8_workspace_bytes() bytes of
- * 256-byte-aligned device scratch.  d_sums (optional, else NULL): exact int32 group sums
+ * 256-byte-aligned device scratch (the re-tiled activations and, for Q4_K / IQ4_XS experts of
+ * at most 8192 rows, room for the sums of two halves of k).  d_sums (optional, else NULL): exact int32 group sums
  * [(row * n + c) * (k/32) + g] as in oxq_gemm_block_sums_dev. */
 size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t n, size_t k);
 int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes,
