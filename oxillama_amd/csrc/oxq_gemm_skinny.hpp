@@ -368,8 +368,25 @@ void gemm_skinny_kernel(
     // row group; expert (grouped form); split of k: blockIdx.y is the expert, or the split (one matrix), or, in the
     // grouped form with k split, expert * grouped_splits + split
     const uint32_t rg = blockIdx.x;
-    const uint32_t gy = !offsets ? 0 : partial ? blockIdx.y / grouped_splits : blockIdx.y;
+    uint32_t gy = !offsets ? 0 : partial ? blockIdx.y / grouped_splits : blockIdx.y;
     const uint32_t ks = !partial ? 0 : offsets ? blockIdx.y % grouped_splits : blockIdx.y;
+    if constexpr (TT == 2) {
+        // Groups of two token tiles take longer than groups of one: hand the experts out largest group first
+        // (ties by index), so that the long work groups start in the first round and the short ones fill the end.
+        // Lane e ranks expert e; the work group takes the expert whose rank is its place in the grid.
+        const uint32_t n_e = offsets ? gridDim.y / (partial ? grouped_splits : 1u) : 0u;
+        if (n_e > 1 && n_e <= 64) {
+            const uint32_t lane = threadIdx.x & 63, e = min(lane, n_e - 1);
+            const int size_e = offsets[e + 1] - offsets[e];
+            uint32_t rank = 0;
+            for (uint32_t o = 0; o < n_e; o++) {
+                const int so = __builtin_amdgcn_readlane(size_e, (int)o);
+                rank += (so > size_e || (so == size_e && o < e)) ? 1u : 0u;
+            }
+            const unsigned long long hit = __ballot(lane < n_e && rank == gy);
+            gy = (uint32_t)__builtin_amdgcn_readfirstlane((int)(__ffsll((long long)hit) - 1));
+        }
+    }
     uint32_t tok0 = 0, tok_end = m;
     if (offsets) {
         tok0 = (uint32_t)offsets[gy];
