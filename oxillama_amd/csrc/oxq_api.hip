@@ -991,7 +991,8 @@ size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t 
 static int moe_gemm_impl(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
                          const uint8_t *d_acts_q8, const int32_t *d_row_offsets, size_t total_rows,
                          size_t max_rows_per_expert, float *d_out, int32_t *d_sums, size_t n, size_t k, int accumulate,
-                         void *d_workspace, size_t workspace_bytes, void *stream, uint32_t prepared_for) {
+                         void *d_workspace, size_t workspace_bytes, void *stream, uint32_t prepared_for,
+                         oxq::GemmArgs::SplitSums *defer_reduce = nullptr) {
     int st = check_dev_shape(type, n, k);
     if (st != OXQ_OK) return st;
     if (total_rows > 0x7FFFFFFFull || n_experts > 65535)
@@ -1032,6 +1033,7 @@ static int moe_gemm_impl(uint32_t type, const uint8_t *d_weights, size_t expert_
     }
     ga.w_stride = expert_stride_bytes;
     ga.prepared_for = prepared_for;
+    ga.defer_reduce = defer_reduce;
     OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
     return OXQ_OK;
 }
@@ -1362,12 +1364,17 @@ int moe_ffn_impl(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_b
         return st;
     OXQ_HIP(oxq::launch_swiglu_quantize(gate, up, pairs * intermediate, nullptr, hq, s));
     }
-    if ((st = oxq_moe_gemm_q8_dev(down_type, d_down, down_stride_bytes, n_experts, hq, d_row_offsets, pairs,
-                                  max_rows_per_expert, y, nullptr, hidden, intermediate, 0, ws + l.gemm, gws,
-                                  stream)) != OXQ_OK)
+    // where the down matmul splits k it leaves the halves' sums for the combine launch to add
+    oxq::GemmArgs::SplitSums halves;
+    if ((st = moe_gemm_impl(down_type, d_down, down_stride_bytes, n_experts, hq, d_row_offsets, pairs, max_rows_per_expert,
+                            y, nullptr, hidden, intermediate, 0, ws + l.gemm, gws, stream, 0, &halves)) != OXQ_OK)
         return st;
-    OXQ_HIP(oxq::launch_moe_combine(y, d_token_rows, d_weights, d_out, (uint32_t)n_tokens, (uint32_t)top_k,
-                                    (uint32_t)hidden, s));
+    if (halves.splits > 1)
+        OXQ_HIP(oxq::launch_moe_combine(halves.partial, d_token_rows, d_weights, d_out, (uint32_t)n_tokens, (uint32_t)top_k,
+                                        (uint32_t)hidden, s, halves.splits, pairs * hidden));
+    else
+        OXQ_HIP(oxq::launch_moe_combine(y, d_token_rows, d_weights, d_out, (uint32_t)n_tokens, (uint32_t)top_k,
+                                        (uint32_t)hidden, s));
     return OXQ_OK;
 }
 

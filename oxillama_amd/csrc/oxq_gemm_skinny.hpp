@@ -477,6 +477,11 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
                        a.accumulate, a.bias, a.offsets, a.w_stride, partial, sb_per_split, splits);
     e = hipGetLastError();
     if (e != hipSuccess || !partial) return e;
+    if (a.defer_reduce && !a.accumulate && !a.bias) {  // the caller adds the splits' sums (in index order, as below)
+        a.defer_reduce->partial = partial;
+        a.defer_reduce->splits = splits;
+        return hipSuccess;
+    }
     const size_t total = (size_t)a.m * a.n;
     if (a.n % 4 == 0 && (reinterpret_cast<uintptr_t>(a.out) & 15) == 0)
         hipLaunchKernelGGL(gemm_skinny_reduce<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream, partial,

@@ -139,7 +139,8 @@ hipError_t launch_lora_apply(const float *a, const float *b, float *r, uint32_t 
 hipError_t launch_moe_gather_quantize(const float *x, const int32_t *pair_token, uint8_t *out, size_t n_pairs,
                                       uint32_t hidden, hipStream_t stream);
 hipError_t launch_moe_combine(const float *y_pairs, const int32_t *token_rows, const float *weights, float *out,
-                              uint32_t n_tokens, uint32_t top_k, uint32_t hidden, hipStream_t stream);
+                              uint32_t n_tokens, uint32_t top_k, uint32_t hidden, hipStream_t stream,
+                              uint32_t splits = 1, size_t split_stride = 0);
 
 hipError_t launch_fill_zero(float *out, size_t n, hipStream_t stream);
 
@@ -177,6 +178,14 @@ struct GemmArgs {
     uint32_t prepared_for = 0;         // tile kernel: the workspace already holds these activations, re-laid out for
                                        // this format id by the previous call (0: none); same layout -> no second pass
     size_t w_stride = 0;
+    // Grouped form whose caller adds the per-split sums itself (the mixture-of-experts layer's combine launch):
+    // where the few-token kernel splits k it then leaves `out` untouched, skips its reduction launch and reports
+    // the sums ([splits][m][n] floats) and their count here.  Null: the call always finishes `out`.
+    struct SplitSums {
+        const float *partial = nullptr;
+        uint32_t splits = 0;
+    };
+    SplitSums *defer_reduce = nullptr;
 };
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream);
 // Device scratch the tile kernel needs for m tokens of k columns (activation re-layout).

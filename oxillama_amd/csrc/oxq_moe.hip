@@ -202,16 +202,21 @@ __global__ __launch_bounds__(256) void moe_gather_quantize_kernel(const float *_
 
 // out[t][c] = sum over the token's selected experts, in selection order, of weight * expert_out
 // (moe.rs:236-254: output zeroed, then `*o += weight * e` per expert; multiply and add rounded separately).
+// splits > 1: an expert output is the sum, in index order, of `splits` partial results split_stride floats apart
+// (the down matmul left its halves of k unadded).
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float *__restrict__ y_pairs,
                                                          const int32_t *__restrict__ token_rows,
                                                          const float *__restrict__ weights, float *__restrict__ out,
-                                                         uint32_t n_tokens, uint32_t top_k, uint32_t hidden) {
+                                                         uint32_t n_tokens, uint32_t top_k, uint32_t hidden,
+                                                         uint32_t splits, size_t split_stride) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (size_t)n_tokens * hidden) return;
     const uint32_t t = (uint32_t)(i / hidden), c = (uint32_t)(i % hidden);
     float o = 0.0f;
     for (uint32_t j = 0; j < top_k; j++) {
-        const float e = y_pairs[(size_t)token_rows[t * top_k + j] * hidden + c];
+        const size_t at = (size_t)token_rows[t * top_k + j] * hidden + c;
+        float e = y_pairs[at];
+        for (uint32_t s = 1; s < splits; s++) e += y_pairs[at + s * split_stride];
         const float p = weights[t * top_k + j] * e;
         o += p;
     }
@@ -241,11 +246,12 @@ hipError_t launch_moe_gather_quantize(const float *x, const int32_t *pair_token,
 }
 
 hipError_t launch_moe_combine(const float *y_pairs, const int32_t *token_rows, const float *weights, float *out,
-                              uint32_t n_tokens, uint32_t top_k, uint32_t hidden, hipStream_t stream) {
+                              uint32_t n_tokens, uint32_t top_k, uint32_t hidden, hipStream_t stream, uint32_t splits,
+                              size_t split_stride) {
     const size_t n = (size_t)n_tokens * hidden;
     if (n == 0) return hipSuccess;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, y_pairs, token_rows,
-                       weights, out, n_tokens, top_k, hidden);
+                       weights, out, n_tokens, top_k, hidden, splits, split_stride);
     return hipGetLastError();
 }
 
