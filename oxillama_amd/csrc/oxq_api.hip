@@ -107,6 +107,7 @@ struct State {
     std::unordered_map<CacheKey, CacheEntry, CacheKeyHash> cache;
     size_t cache_bytes = 0, cache_limit = (size_t)16 << 30;
     uint64_t cache_tick = 0, cache_hits = 0, cache_uploads = 0;
+    uint64_t cache_pin = UINT64_MAX;  // entries used after this tick belong to the call in progress: not evicted
     Scratch s_weights, s_acts, s_x, s_out, s_sums, s_work, s_bias, s_lora_a, s_lora_b, s_lora_r;
     Scratch s_moe_up, s_moe_down, s_moe_tables;
     std::atomic<bool> fuse_swiglu{true};  // oxq_ffn_swiglu_dev: gate, up, SwiGLU and the quantizer of h in one launch where possible
@@ -172,9 +173,11 @@ int stage_weights(uint32_t type, const uint8_t *host, size_t len, const uint8_t 
             g.cache.erase(it);
         }
         while (!g.cache.empty() && g.cache_bytes + len > g.cache_limit) {  // byte cap: least recently used first
-            auto lru = g.cache.begin();
+            auto lru = g.cache.end();
             for (auto jt = g.cache.begin(); jt != g.cache.end(); ++jt)
-                if (jt->second.last_use < lru->second.last_use) lru = jt;
+                if (jt->second.last_use <= g.cache_pin && (lru == g.cache.end() || jt->second.last_use < lru->second.last_use))
+                    lru = jt;
+            if (lru == g.cache.end()) break;  // what is left was staged by this very call and is about to be read
             (void)hipFree(lru->second.dev);
             g.cache_bytes -= lru->first.len;
             g.cache.erase(lru);
@@ -987,12 +990,12 @@ size_t oxq_moe_gemm_q8_workspace_bytes(uint32_t type, size_t total_rows, size_t 
     return oxq::gemm_grouped_workspace_bytes((uint32_t)total_rows, (uint32_t)k, (uint32_t)n, type);
 }
 
-// prepared_for: format id of an immediately preceding call on the same activations and workspace (0: none).
+// prep_state: what an earlier call of the same sequence left in the workspace (GemmArgs::Prepared), or null.
 static int moe_gemm_impl(uint32_t type, const uint8_t *d_weights, size_t expert_stride_bytes, size_t n_experts,
                          const uint8_t *d_acts_q8, const int32_t *d_row_offsets, size_t total_rows,
                          size_t max_rows_per_expert, float *d_out, int32_t *d_sums, size_t n, size_t k, int accumulate,
-                         void *d_workspace, size_t workspace_bytes, void *stream, uint32_t prepared_for,
-                         oxq::GemmArgs::SplitSums *defer_reduce = nullptr) {
+                         void *d_workspace, size_t workspace_bytes, void *stream,
+                         oxq::GemmArgs::Prepared *prep_state, oxq::GemmArgs::SplitSums *defer_reduce = nullptr) {
     int st = check_dev_shape(type, n, k);
     if (st != OXQ_OK) return st;
     if (total_rows > 0x7FFFFFFFull || n_experts > 65535)
@@ -1032,7 +1035,7 @@ static int moe_gemm_impl(uint32_t type, const uint8_t *d_weights, size_t expert_
         ga.shape_rows = (uint32_t)(2 * mean < total_rows ? 2 * mean : total_rows);
     }
     ga.w_stride = expert_stride_bytes;
-    ga.prepared_for = prepared_for;
+    ga.prep_state = prep_state;
     ga.defer_reduce = defer_reduce;
     OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
     return OXQ_OK;
@@ -1043,7 +1046,7 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
                         size_t max_rows_per_expert, float *d_out, int32_t *d_sums, size_t n, size_t k, int accumulate,
                         void *d_workspace, size_t workspace_bytes, void *stream) {
     return moe_gemm_impl(type, d_weights, expert_stride_bytes, n_experts, d_acts_q8, d_row_offsets, total_rows,
-                         max_rows_per_expert, d_out, d_sums, n, k, accumulate, d_workspace, workspace_bytes, stream, 0);
+                         max_rows_per_expert, d_out, d_sums, n, k, accumulate, d_workspace, workspace_bytes, stream, nullptr);
 }
 
 // ---- the callers' side: QuantLinear, SwiGLU feed-forward, RMSNorm ------------------------
@@ -1354,20 +1357,21 @@ int moe_ffn_impl(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_b
         else if (e != hipErrorNotSupported) return fail_hip(e, "launch_gate_up_swiglu (grouped)");
     }
     if (!fused) {
-    if ((st = oxq_moe_gemm_q8_dev(gate_type, d_gate, gate_stride_bytes, n_experts, acts, d_row_offsets, pairs,
-                                  max_rows_per_expert, gate, nullptr, intermediate, hidden, 0, ws + l.gemm, gws,
-                                  stream)) != OXQ_OK)
+    // up reads the activations that gate re-laid out in the workspace, if gate's launch did that and in up's order
+    oxq::GemmArgs::Prepared prep;
+    if ((st = moe_gemm_impl(gate_type, d_gate, gate_stride_bytes, n_experts, acts, d_row_offsets, pairs,
+                            max_rows_per_expert, gate, nullptr, intermediate, hidden, 0, ws + l.gemm, gws, stream,
+                            &prep)) != OXQ_OK)
         return st;
-    // up reads the activations gate just re-laid out in the workspace
     if ((st = moe_gemm_impl(up_type, d_up, up_stride_bytes, n_experts, acts, d_row_offsets, pairs, max_rows_per_expert, up,
-                            nullptr, intermediate, hidden, 0, ws + l.gemm, gws, stream, gate_type)) != OXQ_OK)
+                            nullptr, intermediate, hidden, 0, ws + l.gemm, gws, stream, &prep)) != OXQ_OK)
         return st;
     OXQ_HIP(oxq::launch_swiglu_quantize(gate, up, pairs * intermediate, nullptr, hq, s));
     }
     // where the down matmul splits k it leaves the halves' sums for the combine launch to add
     oxq::GemmArgs::SplitSums halves;
     if ((st = moe_gemm_impl(down_type, d_down, down_stride_bytes, n_experts, hq, d_row_offsets, pairs, max_rows_per_expert,
-                            y, nullptr, hidden, intermediate, 0, ws + l.gemm, gws, stream, 0, &halves)) != OXQ_OK)
+                            y, nullptr, hidden, intermediate, 0, ws + l.gemm, gws, stream, nullptr, &halves)) != OXQ_OK)
         return st;
     if (halves.splits > 1)
         OXQ_HIP(oxq::launch_moe_combine(halves.partial, d_token_rows, d_weights, d_out, (uint32_t)n_tokens, (uint32_t)top_k,
@@ -1508,8 +1512,16 @@ int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, ui
     if ((st = ensure_init()) != OXQ_OK) return st;
     std::lock_guard<std::mutex> lock(g.mu);
     const uint8_t *dg = nullptr, *du = nullptr, *dd = nullptr;
+    // The cache serves this call only if the three tensors fit under its byte cap together, and what the call has
+    // staged is pinned until it returns: staging `down` must not evict (and free) the `gate` the kernels will read.
+    const bool cached = g.cache_mode != 0 && gate_len + up_len + down_len <= g.cache_limit;
+    struct Pin {
+        uint64_t &pin;
+        explicit Pin(uint64_t &p, uint64_t tick) : pin(p) { pin = tick; }
+        ~Pin() { pin = UINT64_MAX; }
+    } pin(g.cache_pin, g.cache_tick);
     auto stage = [&](Scratch &slot, uint32_t t, const uint8_t *host, size_t len, const uint8_t **dev) -> int {
-        if (g.cache_mode != 0 && len <= g.cache_limit) return stage_weights(t, host, len, dev);
+        if (cached) return stage_weights(t, host, len, dev);
         int r = slot.reserve(len);
         if (r != OXQ_OK) return r;
         OXQ_HIP(hipMemcpy(slot.ptr, host, len, hipMemcpyHostToDevice));

@@ -52,6 +52,35 @@ __device__ __forceinline__ uint32_t f2h(float f) {
     return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)f);
 }
 
+// expf as the C library computes it (the routine behind Rust's f32::exp on Linux, which the reference's
+// swiglu.rs:18 and moe.rs softmax call): exp(x) = 2^(k/32) * 2^(r/32) in double with a 32-entry table of 2^(i/32) and a
+// cubic in r, one rounding to float at the end.  The device's own expf differs from it in the last place for a
+// large share of arguments, and a last-place difference of h can move a Q8_0 byte of the down projection's input
+// by a whole step; this form agrees with the host's on all but a few arguments in 10^8.
+static __device__ __constant__ const uint64_t EXP2_TAB[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull, 0x3fef72b83c7d517bull,
+    0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull, 0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull,
+    0x3feedea64c123422ull, 0x3feece086061892dull, 0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull,
+    0x3feea47eb03a5585ull, 0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull, 0x3feee89f995ad3adull,
+    0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull, 0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full,
+    0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};  // bits of 2^(i/32) minus i << 47
+__device__ __forceinline__ float expf_libm(float x) {
+    if (x > 0x1.62e42ep6f) return __builtin_inff();  // overflow
+    if (x < -0x1.9fe368p6f) return 0.0f;             // below the smallest subnormal
+    constexpr double N = 32.0, INV_LN2_N = 0x1.71547652b82fep+0 * N, SHIFT = 0x1.8p52;
+    constexpr double C0 = 0x1.c6af84b912394p-5 / N / N / N, C1 = 0x1.ebfce50fac4f3p-3 / N / N, C2 = 0x1.62e42ff0c52d6p-1 / N;
+    double z = INV_LN2_N * (double)x, kd = z + SHIFT;  // kd: z rounded to an integer, in the low mantissa bits
+    const uint64_t ki = __builtin_bit_cast(uint64_t, kd);
+    kd -= SHIFT;
+    const double r = z - kd;
+    const double s = __builtin_bit_cast(double, EXP2_TAB[ki & 31] + (ki << 47));
+    z = C0 * r + C1;
+    double y = C2 * r + 1.0;
+    y = z * (r * r) + y;
+    return (float)(y * s);
+}
+
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
 }

@@ -1,7 +1,6 @@
 // The batched form of the fused matvec (prefill, decode batch, mixture-of-experts group): host
 // side, and the tile kernel instantiated for Q4_0, Q8_0, Q4_K, Q6_K, IQ4_XS.  Kernel and launch
 // templates: oxq_gemm_tile.hpp; further formats: oxq_gemm_more.hip.
-#include "oxq_gemm_stream.hpp"
 #include "oxq_gemm_skinny.hpp"
 
 namespace oxq {
@@ -190,14 +189,14 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
                                                    : launch_skinny<TileIQ4XS>(a, plan, stream, shape);
         if (e != hipErrorNotSupported) return e;
     }
-    // the previous call left the same activations in the same byte order (and the half-block planes if this
-    // format needs them) -- unless it was served by the few-token kernel, which prepares nothing: go straight to
-    // the tile kernel
-    const bool prepared = a.prepared_for != 0 && act_perm(a.prepared_for) == perm && !skinny_of(a.prepared_for) &&
-                          (!tile_needs_p16_more(type) || tile_needs_p16_more(a.prepared_for));
+    // an earlier call of the same sequence left these activations in the workspace in the byte order this format
+    // needs (with the half-block planes if it needs them): go straight to the tile kernel
+    const bool need_p16 = tile_needs_p16_more(type);
+    const bool prepared = a.prep_state && a.prep_state->valid && a.prep_state->perm == perm &&
+                          (!need_p16 || a.prep_state->p16);
     if (!prepared) {
         // formats with a 16-weight zero-point term also need P per half block
-        float *p16 = tile_needs_p16_more(type)
+        float *p16 = need_p16
                          ? reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(P) + tile_p16_offset(nsb, mpad))
                          : nullptr;
         if (perm == 2)
@@ -208,6 +207,7 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
             hipLaunchKernelGGL(gemm_prep_acts<0>, pgrid, dim3(256), 0, stream, a.A, q8t, P, da16, a.m, mpad, nsb, p16, nsb_row);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
+        if (a.prep_state) *a.prep_state = GemmArgs::Prepared{true, perm, need_p16};
     }
     switch (type) {
     case OXQ_TYPE_Q4_K: return launch_tiles<TileQ4K>(a, plan, stream);

@@ -6,7 +6,6 @@
 // shapes are instantiated here.
 #define OXQ_TILE_DEFAULT_SHAPES_ONLY
 #include "oxq_formats_more.hpp"
-#include "oxq_gemm_stream.hpp"
 #include "oxq_gemm_skinny.hpp"
 
 namespace oxq {

@@ -796,9 +796,6 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
     return hipGetLastError();
 }
 
-template <class F>
-static hipError_t launch_streamed(const GemmArgs &a, const TilePlan &p, hipStream_t stream, uint32_t rows, int variant);
-
 // Tile shape by use: many tokens (prefill) take 128-token work-group tiles; few tokens (a
 // mixture-of-experts group, a short prompt, a decode batch) take 32-token tiles with the
 // weight bytes fetched further ahead, because that case is paced by the weight stream.
@@ -806,10 +803,6 @@ template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
     const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
     const int variant = g_gemm_variant.load(std::memory_order_relaxed);
-    if (variant >= 100 && variant < 200) {  // the streamed kernel (opt-in: oxq_gemm_stream.hpp says why), where the format and shape allow it
-        const hipError_t e = launch_streamed<F>(a, p, stream, rows, variant);
-        if (e != hipErrorNotSupported) return e;
-    }
     if (a.sums)  // debug dump: the same tile layout (and fp32 summation order) as the production choice below
         return rows > 384  ? launch_tile<F, 2, 1, 2, 1, true>(a, p, stream)
                : rows > 64 ? launch_tile<F, 2, 1, 1, 2, true>(a, p, stream)

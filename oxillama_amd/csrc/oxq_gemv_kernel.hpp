@@ -303,7 +303,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
     float v[4];
     for (int i = 0; i < 4; i++) {
         const float g = row_sums[0][4 * j + i], u = row_sums[1][4 * j + i];
-        const float sigmoid = 1.0f / (1.0f + expf(-g));  // swiglu.rs:18
+        const float sigmoid = 1.0f / (1.0f + expf_libm(-g));  // swiglu.rs:18
         v[i] = g * sigmoid * u;                          // swiglu.rs:19
     }
     const bool writer = lane < 8;

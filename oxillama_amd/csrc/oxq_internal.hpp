@@ -175,8 +175,16 @@ struct GemmArgs {
     uint32_t n_experts = 0;
     uint32_t max_rows = 0;             // upper bound of the rows of any one expert (sizes the grid)
     uint32_t shape_rows = 0;           // rows per expert the tile shape is chosen for (<= max_rows)
-    uint32_t prepared_for = 0;         // tile kernel: the workspace already holds these activations, re-laid out for
-                                       // this format id by the previous call (0: none); same layout -> no second pass
+    // Tile kernel, calls in a row on the same activations and workspace (gate then up): what the workspace holds.
+    // A call that runs the re-layout pass records it here; a later call whose format needs the same byte order
+    // (and no plane the earlier pass left out) skips its own pass.  Calls served by a kernel that reads the
+    // caller's Q8_0 rows itself leave the record as it is.  Null: always re-lay out.
+    struct Prepared {
+        bool valid = false;
+        int perm = 0;      // byte order of the activation payload
+        bool p16 = false;  // the half-block planes of P were written as well
+    };
+    Prepared *prep_state = nullptr;
     size_t w_stride = 0;
     // Grouped form whose caller adds the per-split sums itself (the mixture-of-experts layer's combine launch):
     // where the few-token kernel splits k it then leaves `out` untouched, skips its reduction launch and reports

@@ -31,7 +31,7 @@ __global__ __launch_bounds__(256) void swiglu_quantize_kernel(const float *__res
         load4(g, gate + blk * 32 + 4 * j);
         load4(u, up + blk * 32 + 4 * j);
         for (int i = 0; i < 4; i++) {
-            const float sigmoid = 1.0f / (1.0f + expf(-g[i]));  // swiglu.rs:18
+            const float sigmoid = 1.0f / (1.0f + expf_libm(-g[i]));  // swiglu.rs:18
             v[i] = g[i] * sigmoid * u[i];                       // swiglu.rs:19
         }
         if (h_out) {

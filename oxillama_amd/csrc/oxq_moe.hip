@@ -88,7 +88,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict_
             fmaxf(fmaxf(readlane_f(m, 0), readlane_f(m, 16)), fmaxf(readlane_f(m, 32), readlane_f(m, 48)));
         float s = 0.0f;
         for (uint32_t e = lane; e < n_exp; e += 64) {
-            const float v = expf(probs[e] - max_logit);
+            const float v = expf_libm(probs[e] - max_logit);
             probs[e] = v;
             s += v;
         }

@@ -66,8 +66,10 @@ def test_swiglu_quantize(hip, ref):
         h, q = host(d_h), host(d_q)
         want = ref.swiglu(g, u)
         assert np.all(np.isfinite(h))
-        # elementwise: a few ulp from expf
+        # elementwise: the device evaluates exp as the C library does, so h is the oracle's value bit for bit (but
+        # for a handful of arguments in 10^8 on which the library's own last place differs)
         assert np.all(np.abs(h - want) <= 4e-7 * np.abs(want) + 1e-37), "swiglu fp32"
+        assert np.count_nonzero(h.view(np.uint32) != want.view(np.uint32)) <= 2, "swiglu fp32, bit for bit"
         # the bytes are the quantizer's bytes for the values the kernel itself produced
         assert np.array_equal(q, ref.quantize_q8_0(h))
         # each output alone gives the same result

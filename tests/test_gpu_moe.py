@@ -6,9 +6,11 @@ Bars: the routing tables (experts, offsets, rows) exact; weights within 1e-5 (th
 products are summed lane-strided, the reference's in index order); grouped Q8_0
 activation bytes bit-exact; the combine bit-exact given the experts' outputs; the composed layer
 bit-identical to the same steps through the plain entry points; fp32 against the oracle within
-1e-5 * |y_ref|_inf per stage.  End to end the Q8_0 re-quantization of the intermediate vector
-turns last-place differences of gate/up (device expf vs libm) into whole quantization steps of a
-few elements, so the end-to-end bar against the oracle is 2e-3 * |y_ref|_inf."""
+1e-5 * |y_ref|_inf per stage; on identical gate / up values the Q8_0 bytes of h equal the oracle's.
+End to end a token is held to 2e-5 * |y_ref|_inf where its h bytes equal those of the oracle's own chain;
+where the last-place difference between the device's and the oracle's gate / up (another summation
+order) moved a byte of h across a rounding boundary, that is a whole quantization step and the bar is
+2e-3 * |y_ref|_inf."""
 import sys
 
 import numpy as np
@@ -131,6 +133,16 @@ def test_moe_ffn_layer(hip, ref, types, shape):
     _moe_ffn_layer_case(hip, ref, types, shape)
 
 
+@pytest.mark.parametrize("types", [(O.Q4_K, O.Q8_0, O.Q4_K), (O.IQ4_XS, O.Q4_0, O.IQ4_XS), (O.Q8_0, O.Q4_K, O.Q6_K)],
+                         ids=["q4k_q8_0_q4k", "iq4xs_q4_0_iq4xs", "q8_0_q4k_q6k"])
+@pytest.mark.parametrize("shape", [(8, 2, 24, 512, 256), (8, 2, 40, 1024, 512)], ids=str)
+def test_moe_ffn_layer_gate_and_up_on_different_kernels(hip, ref, types, shape):
+    """Gate in a format that the few-token kernel serves (it reads the caller's Q8_0 rows and re-lays nothing out) and
+    up in a format of the same activation byte order that only the tile kernel serves, and the other way round: up
+    must not take the workspace for prepared when gate's launch did not prepare it."""
+    _moe_ffn_layer_case(hip, ref, types, shape)
+
+
 @pytest.mark.parametrize("types", [(O.Q8_0, O.Q8_0, O.Q8_0), (O.Q4_0, O.Q5_0, O.Q8_1), (O.Q5_1, O.Q4_1, O.IQ4_NL)],
                          ids=["q8_0", "q4_0_q5_0_q8_1", "q5_1_q4_1_iq4nl"])
 @pytest.mark.parametrize("shape", [(4, 2, 3, 288, 352), (4, 2, 40, 288, 352), (6, 3, 130, 352, 1408)], ids=str)
@@ -195,6 +207,7 @@ def _moe_ffn_layer_case(hip, ref, types, shape):
         sel, wt = ref.moe_route(router, n_exp, hidden, top_k, xt)
         assert experts[t].tolist() == sel.tolist() and np.max(np.abs(weights[t] - wt)) <= 1e-5
         acc = np.zeros(hidden, np.float32)
+        chain_before = flipped_chain + scales_chain
         for j, e in enumerate(sel):
             r = rows[t, j]
             acts = q8[r * a_row:(r + 1) * a_row]
@@ -205,8 +218,8 @@ def _moe_ffn_layer_case(hip, ref, types, shape):
             assert_close(uh[r * inter:(r + 1) * inter], u_ref, f"up t{t} e{e}")
             hq_ref = ref.quantize_q8_0(ref.swiglu(gh[r * inter:(r + 1) * inter], uh[r * inter:(r + 1) * inter]))
             mine = hqh[r * h_row:(r + 1) * h_row]
-            # device expf vs libm: h differs in the last place now and then, and a few of those differences cross a
-            # rounding boundary of the Q8_0 encoder -- one step of one weight each, never a scale
+            # the device evaluates exp the way the C library does (oxq_device.hpp expf_libm), so on identical gate / up
+            # values the bytes of h are the oracle's
             mb, rb_ = mine.reshape(-1, 34), hq_ref.reshape(-1, 34)
             assert np.array_equal(mb[:, :2], rb_[:, :2]), f"h scales t{t} e{e}"
             step = mb[:, 2:].view(np.int8).astype(np.int32) - rb_[:, 2:].view(np.int8).astype(np.int32)
@@ -233,11 +246,14 @@ def _moe_ffn_layer_case(hip, ref, types, shape):
         want, sel2, _ = ref.moe_forward_q(tg, router, wg, wu, wd, n_exp, hidden, inter, top_k, xt) \
             if tg == tu == td else (None, None, None)
         if want is not None:
-            assert_close(got[t], want, f"end to end t{t}", tol=2e-3)
-    # the flipped bytes are what separates the 2e-3 end-to-end bar from the 1e-5 per-stage bar: far below 0.1 % of h
+            # a token whose h bytes are the oracle chain's bytes: the layer's output within the fp32 bar (2e-5: the
+            # routing weights carry up to 1e-5 of their own); a byte of h that the last-place difference between the
+            # device's and the oracle's gate / up moved across a rounding boundary is a whole quantization step
+            same_h = flipped_chain + scales_chain == chain_before
+            assert_close(got[t], want, f"end to end t{t}", tol=2e-5 if same_h else 2e-3)
     say(f"h bytes one step off the oracle's: {flipped_h} of {bytes_h} (same gate/up); oracle's gate/up: {flipped_chain} bytes, "
         f"{scales_chain} of {bytes_h // 34} block scales one f16 step off")
-    assert flipped_h <= max(1, bytes_h // 1000), f"{flipped_h} of {bytes_h} Q8_0 bytes of h differ"
+    assert flipped_h == 0, f"{flipped_h} of {bytes_h} Q8_0 bytes of h differ on identical gate / up values"
     assert flipped_chain <= max(2, bytes_h // 1000), f"{flipped_chain} of {bytes_h} Q8_0 bytes of h differ from the oracle's chain"
     assert scales_chain <= max(2, bytes_h // 34 // 100), f"{scales_chain} of {bytes_h // 34} block scales of h differ"
 
@@ -317,6 +333,20 @@ def test_moe_forward_host_slices(hip, ref):
         assert_close(many[0], one, "a token alone and in a batch", tol=2e-3)
         for i in range(5):
             assert_close(many[i], want(x[i * hidden:(i + 1) * hidden]), f"token {i}", tol=2e-3)
+    # a byte cap that the three tensors do not fit under together: staging `down` must not evict (and free) the
+    # `gate` or `up` that the same call staged a moment earlier -- such a call goes round the cache; and with room
+    # for exactly the three, an older entry goes, not one of the call's own
+    plain = layer.forward_batch(x, 5)
+    other = synth.weights(t, 77, 64, hidden)
+    xa = ref.quantize_q8_0(x[:hidden])
+    for limit in (wg.nbytes + wu.nbytes + wd.nbytes - 1, 2 * wg.nbytes, wg.nbytes + wu.nbytes + wd.nbytes):
+        lib.oxq_weight_cache_clear()
+        lib.oxq_weight_cache_enable(1)
+        lib.oxq_weight_cache_set_limit(limit)
+        hip.HipKernel(t).matvec_q8_fused(other, xa, np.zeros(64, dtype=np.float32), 64, hidden)  # an older entry
+        for _ in range(2):
+            assert np.array_equal(layer.forward_batch(x, 5).view(np.uint32), plain.view(np.uint32)), limit
+    lib.oxq_weight_cache_set_limit(16 << 30)
     lib.oxq_weight_cache_enable(0)
     lib.oxq_weight_cache_clear()
     # the reference's error cases (moe.rs:403-450, 307-322) after a working call
