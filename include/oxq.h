@@ -269,7 +269,10 @@ int oxq_activation_route(void);
  * pass it and the call is asynchronous and allocation-free; pass NULL and the library uses
  * its own scratch (the call then serialises and waits for the stream).  Fewer rows, and
  * shapes for which the workspace size is 0, run GEMV launches (up to four rows per pass over
- * the weights) and ignore the workspace. */
+ * the weights) and ignore the workspace.  Q4_K matmuls of many token rows whose 128-token x
+ * 256-row work groups fill the chip (the prefill shapes) run on the f16 matrix cores instead,
+ * with the 6-bit sub-block scale inside the weight operand (exact) and d / dmin applied per
+ * super-block: the same integers, fp32 inside the same 1e-5 bar; the workspace size covers both. */
 size_t oxq_gemm_q8_workspace_bytes(uint32_t type, size_t m, size_t n, size_t k);
 int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                     float *d_out, size_t m, size_t n, size_t k, int accumulate,
@@ -294,6 +297,14 @@ int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_
 int oxq_gemm_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                             float *d_out, int32_t *d_sums, size_t m, size_t n, size_t k,
                             void *d_workspace, size_t workspace_bytes, void *stream);
+/* Debug: the same for the prefill kernel of the formats whose scaled weights are exact in f16 (Q4_K), which
+ * oxq_gemm_q8_dev takes for many token rows: its matrix-core result per (token, row, 32-weight sub-block) is the
+ * 6-bit sub-block scale times the integer group sum, an exact integer, written to
+ * d_sums[(r * n + c) * (k/32) + g]; d_out as oxq_gemm_q8_dev (overwrite).  Any m >= 1 runs on that kernel here.
+ * OXQ_ERR_UNSUPPORTED_SHAPE when the format or shape has no such kernel; a workspace is required. */
+int oxq_gemm_scaled_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
+                             float *d_out, int32_t *d_sums, size_t m, size_t n, size_t k,
+                             void *d_workspace, size_t workspace_bytes, void *stream);
 
 /* Grouped (mixture-of-experts) matmul: the batched form of the per-token expert calls of
  * MoeFfn::forward (crates/oxillama-arch/src/common/moe.rs:236-252: for each selected expert,

@@ -30,7 +30,8 @@ int oxq_set_gemv_waves_per_row(unsigned waves);
 int oxq_set_gemm_tile_min_rows(unsigned rows);
 /* Which kernel and launch shape the batched matmuls take (tuning knob; 0 restores the default, the measured choice
  * per shape).  1..23: a fixed tile shape / prefetch depth of the int8-MFMA tile kernel; 99: the tile kernel's own
- * choice, never the few-token kernel; 200..205: the
+ * choice, never the few-token kernel nor the prefill kernel; 300: the prefill kernel (f16 matrix cores, Q4_K) for any
+ * number of token rows; 200..205: the
  * few-token kernel (16 x 16 x 32 MFMA, groups of at most 32 token rows) in a fixed shape.  A value a format or
  * shape cannot take falls back to the default tile choice. */
 int oxq_set_gemm_variant(int variant);

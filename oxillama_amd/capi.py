@@ -128,6 +128,8 @@ SIGNATURES = {
                                   C.c_size_t, C.c_size_t, C.c_int, C.c_void_p, C.c_size_t, C.c_void_p]),
     "oxq_gemm_block_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                           C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "oxq_gemm_scaled_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
+                                           C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p]),
     "oxq_moe_gemm_q8_workspace_bytes": (C.c_size_t, [C.c_uint32, C.c_size_t, C.c_size_t, C.c_size_t]),
     "oxq_moe_gemm_q8_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p,
                                       C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int,

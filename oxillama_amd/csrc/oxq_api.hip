@@ -1049,6 +1049,36 @@ int oxq_moe_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, size_t expert_s
                          max_rows_per_expert, d_out, d_sums, n, k, accumulate, d_workspace, workspace_bytes, stream, nullptr);
 }
 
+int oxq_gemm_scaled_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_out,
+                             int32_t *d_sums, size_t m, size_t n, size_t k, void *d_workspace, size_t workspace_bytes,
+                             void *stream) {
+    if (!d_sums) return fail(OXQ_ERR_INTERNAL, 0, 0, "null sums");
+    int st = check_dev_shape(type, n, k, true);
+    if (st != OXQ_OK) return st;
+    if (m == 0 || m > 0xFFFFFFFFull || !oxq::gemm_prefill_supported(type, (uint32_t)m, (uint32_t)n, (uint32_t)k))
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0, m, "no prefill kernel for this type/shape");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    const size_t need = oxq::gemm_prefill_workspace_bytes((uint32_t)m, (uint32_t)k);
+    if (!d_workspace || workspace_bytes < need)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, d_workspace ? workspace_bytes : 0, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(d_workspace) & 255)
+        return fail(OXQ_ERR_KERNEL, 256, reinterpret_cast<uintptr_t>(d_workspace) & 255, "workspace must be 256-byte aligned");
+    oxq::GemmArgs ga;
+    ga.W = d_weights;
+    ga.A = d_acts_q8;
+    ga.out = d_out;
+    ga.sums = d_sums;
+    ga.scaled_sums = true;
+    ga.workspace = (uint8_t *)d_workspace;
+    ga.workspace_bytes = workspace_bytes;
+    ga.m = (uint32_t)m;
+    ga.n = (uint32_t)n;
+    ga.k = (uint32_t)k;
+    ga.accumulate = 0;
+    OXQ_HIP(oxq::launch_gemm_q8(type, ga, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
 // ---- the callers' side: QuantLinear, SwiGLU feed-forward, RMSNorm ------------------------
 
 static int check_lora(const oxq_lora *lora) {

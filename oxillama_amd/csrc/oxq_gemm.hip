@@ -78,7 +78,21 @@ size_t gemm_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t
 }
 size_t gemm_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t type) {
     const size_t planes = (gemm_planes_bytes(m, k) + 255) & ~(size_t)255;
-    return planes + gemm_partial_bytes(type, m, n, k);
+    const size_t tiles = planes + gemm_partial_bytes(type, m, n, k);
+    // the prefill kernel lays its own planes (f16 token operands) over the head of the same workspace; the size is
+    // a function of the shape, whichever kernel a call then takes
+    const size_t prefill = gemm_prefill_supported(type, m, n ? n : 1, k) ? gemm_prefill_workspace_bytes(m, k) : 0;
+    return tiles > prefill ? tiles : prefill;
+}
+
+// A plain matmul takes the prefill kernel where its work groups (128 tokens x 256 rows, one per compute unit, each
+// about as long whatever the others do) fill their rounds of the chip: measured at k = 4096 against the tile
+// kernel, 224 / 448 / 672 work groups on 256 compute units 110 / 202 / 298 us against 126 / 228 / 332, but 280 work
+// groups 194 against 172, 168 a tie, 128 and fewer far behind (the tile kernel's smaller tiles spread better).
+static bool gemm_prefill_pays(uint32_t m, uint32_t n) {
+    const uint64_t wgs = (uint64_t)((m + 127) / 128) * ((n + 255) / 256), cus = device_cus();
+    const uint64_t rounds = (wgs + cus - 1) / cus;
+    return 100 * wgs >= 85 * rounds * cus;
 }
 
 std::atomic<uint32_t> g_gemm_tile_min_rows{0};  // tuning: 0 = default
@@ -158,6 +172,17 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
         if (a.offsets) return hipErrorInvalidValue;  // grouped form exists for the tile kernel only
         return gemm_by_rows(type, a, stream);
     }
+    const int variant = g_gemm_variant.load(std::memory_order_relaxed);
+    // many token rows of a format whose scaled weights are exact in f16: the prefill kernel (oxq_gemm_prefill.hip).
+    // The debug dump of the integer sums stays on the tile kernel; the dump of the scaled sums is this kernel's.
+    if (!a.offsets && (variant == 0 || variant == 300) && (!a.sums || a.scaled_sums) &&
+        gemm_prefill_supported(type, a.m, a.n, a.k) && a.workspace_bytes >= gemm_prefill_workspace_bytes(a.m, a.k)) {
+        if (a.scaled_sums || variant == 300 || gemm_prefill_pays(a.m, a.n)) {
+            const hipError_t e = launch_gemm_prefill(type, a, stream);
+            if (e != hipErrorNotSupported) return e;
+        }
+    }
+    if (a.scaled_sums) return hipErrorNotSupported;
     const uint32_t mpad = (a.m + 127) / 128 * 128 + 128, nsb = tile_padded_sub_blocks(a.k), nsb_row = a.k / 32;
     uint8_t *q8t = a.workspace;
     float *P = reinterpret_cast<float *>(q8t + (size_t)nsb * mpad * 32);
@@ -177,7 +202,6 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
         a.workspace_bytes >= gemm_grouped_workspace_bytes(a.m, a.k, a.n, type))
         plan.partial = reinterpret_cast<float *>(a.workspace + ((gemm_planes_bytes(a.m, a.k) + 255) & ~(size_t)255));
     // The few-token kernel (oxq_gemm_skinny.hpp), where it pays: it reads the caller's Q8_0 rows itself, no re-layout.
-    const int variant = g_gemm_variant.load(std::memory_order_relaxed);
     const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
     auto skinny_of = [&](uint32_t t) {
         return t == OXQ_TYPE_Q4_K     ? skinny_shape<TileQ4K>(a, plan.partial != nullptr, rows, variant)

@@ -161,6 +161,7 @@ struct GemmArgs {
     const uint8_t *A;   // Q8_0 blocks of the m activation rows, row-major, k/32 blocks per row
     float *out;         // [m x n] row-major
     int32_t *sums;      // optional debug dump [m][n][k/32]
+    bool scaled_sums = false;  // the dump is the prefill kernel's: sub-block scale times integer sum (exact integers)
     uint8_t *workspace; // gemm_workspace_bytes(m, k) bytes, 256-byte aligned; null: row-by-row matvecs
     size_t workspace_bytes = 0;  // what the workspace really holds, if known: gemm_workspace_bytes(m, k, n, type)
                                  // bytes leave room for the few-token kernel's split-k sums
@@ -203,6 +204,12 @@ size_t gemm_workspace_bytes(uint32_t m, uint32_t k, uint32_t n = 0, uint32_t typ
 // ... of the grouped form: the planes, plus room for two per-split sums of [m x n] where the few-token kernel may
 // split an expert's k in two (Q4_K / IQ4_XS, k a multiple of 1024, at most 8192 rows per expert).
 size_t gemm_grouped_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t type);
+// The prefill kernel of the formats whose scaled weights are exact in f16 (oxq_gemm_prefill.hip): plain matmuls of
+// many token rows.  Its workspace (f16 token operands, scale pairs, bf16 pieces of the block sums) replaces the tile
+// kernel's planes at the head of the caller's workspace.  hipErrorNotSupported: not this format / shape.
+bool gemm_prefill_supported(uint32_t type, uint32_t m, uint32_t n, uint32_t k);
+size_t gemm_prefill_workspace_bytes(uint32_t m, uint32_t k);
+hipError_t launch_gemm_prefill(uint32_t type, const GemmArgs &a, hipStream_t stream);
 // Tuning knobs (oxq_tuning.h), read once per call.
 extern std::atomic<int> g_gemm_variant;              // 0 = default tile shape
 extern std::atomic<uint32_t> g_gemm_tile_min_rows;   // 0 = default threshold

@@ -294,6 +294,12 @@ class HipKernel:
                                                  d_out.data_ptr(), d_sums.data_ptr(), m, n, k, ws_ptr, ws_len,
                                                  self._stream()))
 
+    def gemm_scaled_sums_dev(self, d_weights, d_acts, d_out, d_sums, m, n, k, workspace):
+        """The prefill kernel's debug dump: sub-block scale times integer group sum per (token, row, sub-block)."""
+        _check(self._lib.oxq_gemm_scaled_sums_dev(self.tensor_type, d_weights.data_ptr(), d_acts.data_ptr(),
+                                                  d_out.data_ptr(), d_sums.data_ptr(), m, n, k, workspace.data_ptr(),
+                                                  workspace.numel(), self._stream()))
+
     def moe_gemm_workspace_bytes(self, total_rows, n, k):
         return self._lib.oxq_moe_gemm_q8_workspace_bytes(self.tensor_type, total_rows, n, k)
 

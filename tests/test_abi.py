@@ -167,7 +167,8 @@ def test_gemm_workspace_size_is_a_function_of_the_shape():
     """oxq_gemm_q8_workspace_bytes: the re-tiled activations (token rows padded to 128 and 128 more, 46 bytes per
     token block, rounded to 256), plus -- for at most 16 token rows of Q4_K / IQ4_XS on a matrix of at least 2^25
     weights that yields fewer than 448 groups of 128 rows -- the room for the few-token kernel's per-split sums:
-    splits x m x n floats, splits = min(ceil(448 / groups), k / 1024, 16) taken in even numbers of super-blocks."""
+    splits x m x n floats, splits = min(ceil(448 / groups), k / 1024, 16) taken in even numbers of super-blocks.
+    For Q4_K the size is at least what the prefill kernel's planes take."""
     lib = capi.load()
 
     def planes(m, k):
@@ -182,7 +183,11 @@ def test_gemm_workspace_size_is_a_function_of_the_shape():
     assert w(q4k, 17, 14336, 4096) == planes(17, 4096)                                 # more than 16 rows
     assert w(q6k, 16, 14336, 4096) == planes(16, 4096)                                 # no few-token kernel for Q6_K
     assert w(q4k, 16, 128256, 4096) == planes(16, 4096)                                # 1002 groups fill the chip
-    assert w(q4k, 512, 14336, 4096) == planes(512, 4096)
+    # Q4_K: never less than the prefill kernel's planes (74 bytes per token block, token rows padded to 128)
+    def prefill(m, k):
+        return (k // 32) * ((m + 127) // 128 * 128) * 74
+    assert w(q4k, 512, 14336, 4096) == max(planes(512, 4096), prefill(512, 4096)) == prefill(512, 4096)
+    assert w(q6k, 512, 14336, 4096) == planes(512, 4096)
     assert w(q4k, 16, 14336, 4000) == 0                                                # k not a multiple of 256
     # the formats of independent 32-weight blocks: any whole number of blocks from eight up, planes padded to whole
     # groups of eight blocks

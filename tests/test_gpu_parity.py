@@ -625,6 +625,8 @@ def test_prefill_full_size_c4(hip, ref):
     dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
     kern.gemm_q8_dev(dw, da, dy, m, n, k_, accumulate=False, workspace=ws)
     torch.cuda.synchronize()
+    from test_gpu_prefill_f16 import last_launch, q4k_sub_block_scales
+    assert "gemm_prefill_q4k" in last_launch(), last_launch()  # C4 is the shape the f16 prefill kernel is for
     rows = list(range(0, m, 16)) + [m - 1]
     y_ref = _oracle_prefill(ref, t, w, acts, m, n, k_, rows=rows)
     assert_close(dy.cpu().numpy()[rows], y_ref, "C4 prefill")
@@ -644,8 +646,16 @@ def test_prefill_full_size_c4(hip, ref):
         got = dsum.cpu().numpy()
         for r in range(m):
             assert np.array_equal(got[r], ref.block_sums(t, w_slab, acts[r * arb:(r + 1) * arb], 512, k_)), (r0, r)
-        # the slab on its own goes through the same tile arithmetic as inside the full matrix
+        # the slab on its own (the int8 tile kernel at this size) meets the same bar
         assert_close(dy_slab.cpu().numpy(), y_slab, f"C4 slab launch, rows {r0}")
+        # and the prefill kernel's own matrix-core results on the slab: sub-block scale x integer sum, exactly
+        kern.gemm_scaled_sums_dev(dw_slab, da, dy_slab, dsum, m, 512, k_, ws)
+        torch.cuda.synchronize()
+        got = dsum.cpu().numpy()
+        sc = q4k_sub_block_scales(w_slab, 512, k_)
+        for r in range(0, m, 7):
+            assert np.array_equal(got[r], sc * ref.block_sums(t, w_slab, acts[r * arb:(r + 1) * arb], 512, k_)), (r0, r)
+        assert_close(dy_slab.cpu().numpy(), y_slab, f"C4 slab on the prefill kernel, rows {r0}")
         del dsum, got
     # every token row also equals the batch-1 fused matvec of the same activations, to fp32 order
     yv = torch.zeros(n, dtype=torch.float32, device="cuda")
