@@ -264,6 +264,12 @@ def main():
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-extra-kernels", action="store_true")
     ap.add_argument("--no-moe", action="store_true")
+    ap.add_argument("--f32-route", action="store_true",
+                    help="also time the projections on the fp32-activation route (QuantKernel::gemv's own arithmetic); "
+                         "the figures go to the --detail file, not to the result line")
+    ap.add_argument("--detail", metavar="FILE", default=None,
+                    help="write every leg's full record (launch names, sample descriptions, byte counts) as JSON to FILE; "
+                         "the result line on stdout stays compact")
     ap.add_argument("--moe-tile-only", action="store_true",
                     help="run the 64-token MoE leg's grouped matmuls on the tile kernel alone (for profiles that set it "
                          "beside the few-token kernel)")
@@ -543,10 +549,11 @@ def main():
             wb = n_rows * row_bytes(t, n_cols)
             return {"us_per_call": round(us, 3), "launches": n, "distinct_weight_sets": len(mats),
                     "weight_GBps": round(wb / us / 1e3, 1), "frac_hbm_peak": round((wb + 4 * n_cols + 4 * n_rows) / us / 1e3 / HBM_PEAK_GBPS, 4)}
-        kernels["f32_route_q4k_gate_14336x4096"] = time_f32(k_q4k, Q4_K, [w["gate"] for w in layers], x, yg, F, H)
-        kernels["f32_route_q6k_down_4096x14336"] = time_f32(k_q6k, Q6_K, [w["down"] for w in layers], h, yd, H, F)
-        kernels["f32_route_q8_0_q_proj_4096x4096"] = time_f32(k_q8, Q8_0, [w["q"] for w in layers], x, yq, H, H)
-        kernels["f32_route_c1_q4_0_4096x4096"] = time_f32(k_q40, Q4_0, c1, x, yq, H, H)
+        if args.f32_route:
+            kernels["f32_route_q4k_gate_14336x4096"] = time_f32(k_q4k, Q4_K, [w["gate"] for w in layers], x, yg, F, H)
+            kernels["f32_route_q6k_down_4096x14336"] = time_f32(k_q6k, Q6_K, [w["down"] for w in layers], h, yd, H, F)
+            kernels["f32_route_q8_0_q_proj_4096x4096"] = time_f32(k_q8, Q8_0, [w["q"] for w in layers], x, yq, H, H)
+            kernels["f32_route_c1_q4_0_4096x4096"] = time_f32(k_q40, Q4_0, c1, x, yq, H, H)
         del c1
         # a decode batch of 16 token rows on the Q4_K FFN shapes (oxq_gemm_q8_dev: the few-token kernel with k split
         # over work groups, then the reduction launch), over the layers' distinct weights
@@ -597,6 +604,7 @@ def main():
             quant.quantize_q8_0_dev(xs, xsq)
             k_q4k.gemm_q8_dev(wp[0], xsq, ys, M, F, H, workspace=ws)
             stream.synchronize()
+            prefill_launch = last_launch()
             reps = 8
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record(stream)
@@ -644,7 +652,21 @@ def main():
             e1.record(stream)
             e1.synchronize()
         mfma_only_tops = mf_blocks * 4 * mf_iters * 4 * 2 * 32 ** 3 / (e0.elapsed_time(e1) * 1e3) / 1e6
-        prefill = {"workload": "Q4_K 14336x4096 x Q8_0 acts 512x4096", "int8_ops": ops,
+        # the int8 tile kernel on the same calls (tuning knob 99), beside the kernel the library chooses
+        from oxillama_amd import capi as _capi
+        _capi.load().oxq_set_gemm_variant(99)
+        with torch.cuda.stream(stream):
+            k_q4k.gemm_q8_dev(wp[0], xsq, ys, M, F, H, workspace=ws)
+            stream.synchronize()
+            e0.record(stream)
+            for i in range(reps):
+                k_q4k.gemm_q8_dev(wp[i % len(wp)], xsq, ys, M, F, H, workspace=ws)
+            e1.record(stream)
+            e1.synchronize()
+        _capi.load().oxq_set_gemm_variant(0)
+        tile_gemm_us = e0.elapsed_time(e1) * 1e3 / reps
+        prefill = {"workload": "Q4_K 14336x4096 x Q8_0 acts 512x4096", "int8_ops": ops, "launch": prefill_launch,
+                   "int8_tile_kernel_gemm_us": round(tile_gemm_us, 2),
                    "gemm_us": round(gemm_us, 2), "quantize_us": round(quant_us, 2),
                    "TOPS": round(ops / gemm_us / 1e6, 2), "peak_TOPS": INT8_PEAK_TOPS,
                    "frac_int8_peak": round(ops / gemm_us / 1e6 / INT8_PEAK_TOPS, 4),
@@ -819,6 +841,8 @@ def main():
         s_1t, n_1t = time_cpu(1, 8.0)
         cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "host_cores": host_cores,
                "kind": "port",
+               "sample_short": f"one layer of the timed step, {n_mt} repeats, {cores} threads (static row split); " +
+                               ("AVX2 twin of the reference's fused rows" if avx2 else "scalar C restatement"),
                "sample": f"one layer (same 4 matrices, quantization of x, SwiGLU + quantization of h), {n_mt} repeats, static row split over "
                          f"{cores} threads; " + ("AVX2 intrinsics twin of the reference's fused rows (Q6_K body is scalar "
                          "there too)" if avx2 else "scalar C restatement of the reference's AVX2-tier fused rows"),
@@ -826,6 +850,38 @@ def main():
                "single_thread": {"value": round(step_weight_bytes / s_1t / 1e9, 3), "ms_per_step": round(s_1t * 1e3, 3),
                                  "repeats": n_1t}}
 
+    detail = {"timing": timing, "roofline": roofline, "cpu_baseline": cpu, "parity": parity, "kernels": kernels,
+              "prefill": prefill, "moe": moe_out, "moe_32_tokens": moe_small, "moe_1_token": moe_one,
+              "device": {"name": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
+                         "clock_mhz": info["clock_khz"] / 1000.0, "weight_generation_s": round(gen_s, 1)}}
+    if args.detail:
+        with open(args.detail, "w") as f:
+            json.dump(detail, f, indent=1)
+
+    def short(k):  # per-kernel legs: time and fraction of the 8 TB/s peak (algorithmic bytes where the leg has them)
+        return {"us": k["us_per_call"], "frac": k["frac_hbm_peak"]}
+
+    def get(d, *path):
+        for p in path:
+            if d is None:
+                return None
+            d = d.get(p)
+        return d
+
+    launch_words = ("quantize x, q_proj, gate+up+SwiGLU+quantize (one launch), down" if not (args.fused_quantize or args.unfused_swiglu)
+                    else "quantize x, q_proj, gate+up (one launch), SwiGLU+quantize, down" if not args.fused_quantize
+                    else "q_proj, gate+up (one launch), SwiGLU, down, each quantizing its fp32 input itself")
+    # where the targets of this path stand, in one flat object (fractions of the 8 TB/s HBM peak, of the 5 POPS int8 peak)
+    targets = {"q4k_gate_up_swiglu_frac": pair_swiglu["frac_hbm_peak"], "q4k_gate_up_frac": pair["frac_hbm_peak"],
+               "q4k_gate_frac": get(kernels, "q4k_gate_up_14336x4096", "frac_hbm_peak"),
+               "q6k_down_frac": get(kernels, "q6k_down_4096x14336", "frac_hbm_peak"),
+               "q8_0_q_proj_frac": get(kernels, "q8_0_q_proj_4096x4096", "frac_hbm_peak"),
+               "c1_q4_0_frac": get(kernels, "c1_q4_0_4096x4096", "frac_hbm_peak"),
+               "c3_lm_head_frac": get(kernels, "c3_lm_head_q6k_128256x4096", "frac_hbm_peak"),
+               "c3_lm_head_us": get(kernels, "c3_lm_head_q6k_128256x4096", "us_per_call"),
+               "prefill_frac_int8_peak": get(prefill, "frac_int8_peak"), "prefill_gemm_us": get(prefill, "gemm_us"),
+               "prefill_TOPS": get(prefill, "TOPS"), "moe_us": get(moe_out, "us_per_step"),
+               "moe_frac": get(moe_out, "frac_hbm_peak")}
     out = {
         "metric": "Q4_K GEMV weight GB/s (% HBM peak); batch-512 prefill int8-MFMA TOPS",
         "value": round(value, 1),
@@ -834,32 +890,48 @@ def main():
         "steps": K,
         "warmup": W,
         "ms_per_step": round(ms_per_step, 5),
-        "timing": timing,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8 dot (v_dot4_i32_i8) -> int32 group sums -> f32",
+        "dtype": "int8 dot -> int32 group sums -> f32",
         "data": "synthetic",
-        "config": {"workload": "Llama-3-8B decode projections, batch 1: q_proj 4096x4096 Q8_0, "
-                               "ffn_gate/ffn_up 14336x4096 Q4_K, ffn_down 4096x14336 Q6_K, Q8_0 activations",
+        "config": {"workload": "Llama-3-8B decode projections, batch 1: q_proj 4096x4096 Q8_0, ffn_gate/ffn_up "
+                               "14336x4096 Q4_K, ffn_down 4096x14336 Q6_K, Q8_0 activations",
                    "weight_bytes_per_step": step_weight_bytes, "distinct_layers": L,
                    "frac_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
-                   "launch": "one HIP graph of all timed steps; per step " +
-                             ("quantize x, q_proj, gate+up+SwiGLU+quantize (one launch), down" if not (args.fused_quantize or args.unfused_swiglu)
-                              else "quantize x, q_proj, gate+up (one launch), SwiGLU + quantize, down" if not args.fused_quantize
-                              else "q_proj, gate+up (one launch), SwiGLU, down, each projection quantizing its fp32 "
-                                   "input vector to Q8_0 itself")},
-        "roofline": roofline,
-        "cpu_baseline": cpu,
-        "parity": parity,
-        "kernels": kernels,
-        "prefill": prefill,
-        "moe": moe_out,
-        "moe_32_tokens": moe_small,
-        "moe_1_token": moe_one,
-        "device": {"name": info["name"], "arch": info["arch"], "compute_units": info["compute_units"],
-                   "clock_mhz": info["clock_khz"] / 1000.0, "weight_generation_s": round(gen_s, 1)},
+                   "launch": "one HIP graph of all timed steps; per step " + launch_words,
+                   "timing": {"replays": R, "reported": "median wall time of the replays / steps",
+                              "ms_min": timing["ms_per_step_min"], "ms_max": timing["ms_per_step_max"],
+                              "ms_hip_events": timing["ms_per_step_hip_events_median"]},
+                   "targets": targets},
+        "roofline": {"bound": "hbm", "kernel": dom_launch, "achieved": roofline["achieved"], "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": roofline["frac"], "traffic": roofline["traffic"],
+                     "us_per_call": roofline["us_per_call"], "algorithmic_bytes": roofline["algorithmic_bytes"],
+                     "others": {k: short(v) for k, v in kernels.items() if "frac_hbm_peak" in v}},
+        "cpu_baseline": None if cpu is None else {
+            "value": cpu["value"], "unit": "GB/s", "cores": cpu["cores"], "kind": "port",
+            "sample": "",
+            "ms_per_step": cpu["ms_per_step"], "single_thread_value": cpu["single_thread"]["value"]},
+        "parity": None if parity is None else {
+            "pass": parity["pass"], "acts_q8_bytes_equal": parity["acts_q8_bytes_equal"],
+            "h_q8_bytes_equal_fraction": parity["h_q8_bytes_equal_fraction"],
+            "fp32_max_err_over_ymax": parity["fp32_max_err_over_ymax"], "tolerance": 1e-5},
+        "prefill": None if prefill is None else {
+            "gemm_us": prefill["gemm_us"], "quantize_us": prefill["quantize_us"], "TOPS": prefill["TOPS"],
+            "frac_int8_peak": prefill["frac_int8_peak"], "kernel": prefill["launch"].split(" ")[0],
+            "int8_tile_kernel_gemm_us": prefill["int8_tile_kernel_gemm_us"], "mfma_only_TOPS": prefill["mfma_only_TOPS"],
+            "other_formats_gemm_us": {k: v["gemm_us"] for k, v in prefill["same_shape_other_formats"].items()}},
+        "moe": None if moe_out is None else {
+            "us_64_tokens": moe_out["us_per_step"], "frac_64_tokens": moe_out["frac_hbm_peak"],
+            "rows_per_expert": moe_out["rows_per_expert"], "us_32_tokens": moe_small["us_per_step"],
+            "frac_32_tokens": moe_small["frac_hbm_peak"], "us_1_token": moe_one["us_per_step"],
+            "frac_1_token": moe_one["frac_hbm_peak"]},
+        "batch16": {k: {"us": v["us_per_call"], "tile_kernel_us": v["tile_kernel_us_per_call"]}
+                    for k, v in kernels.items() if "tile_kernel_us_per_call" in v},
+        "device": {"name": info["name"], "compute_units": info["compute_units"]},
     }
+    if cpu is not None:
+        out["cpu_baseline"]["sample"] = cpu["sample_short"]
     print(json.dumps(out), flush=True)
     if parity is not None and not parity["pass"]:
         sys.exit(3)  # the line above is still printed; a fast kernel with wrong results is not a result

@@ -513,8 +513,9 @@ int oxq_moe_forward(uint32_t gate_type, const uint8_t *gate, size_t gate_len, ui
  * 500-509); k = 1 is its argmax (mod.rs:652-662: the first of equal maxima).  Exactly equal values
  * come out lower index first (the reference's unstable sort leaves that open); NaNs rank last.
  * 1 <= k <= 256, k <= n <= 2^20.  Needs oxq_topk_workspace_bytes() bytes of 8-byte-aligned device
- * scratch; one or two launches (from k = 40 a one-launch radix select that leaves the scratch
- * untouched), no allocation, no synchronisation. */
+ * scratch; one or two launches (from k = 16 on vectors of more than 4096 values: slices of the
+ * vector selected side by side, then their survivors by one work group), no allocation, no
+ * synchronisation. */
 size_t oxq_topk_workspace_bytes(size_t n, size_t k);
 int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
                  uint32_t *d_out_indices, void *d_workspace, size_t workspace_bytes, void *stream);

@@ -299,13 +299,17 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
     }
     __syncthreads();
     if (wave != 0) return;
+    // one element of h per lane (the exp is a chain of double-precision operations: 32 lanes side by side, not four
+    // in a row on eight lanes), then the encoder's layout: lane j of eight holds elements 4j..4j+3
+    float hv;
+    {
+        const float g = row_sums[0][lane & 31], u = row_sums[1][lane & 31];
+        const float sigmoid = 1.0f / (1.0f + expf_libm(-g));  // swiglu.rs:18
+        hv = g * sigmoid * u;                                 // swiglu.rs:19
+    }
     const uint32_t j = lane & 7;
     float v[4];
-    for (int i = 0; i < 4; i++) {
-        const float g = row_sums[0][4 * j + i], u = row_sums[1][4 * j + i];
-        const float sigmoid = 1.0f / (1.0f + expf_libm(-g));  // swiglu.rs:18
-        v[i] = g * sigmoid * u;                          // swiglu.rs:19
-    }
+    for (int i = 0; i < 4; i++) v[i] = __shfl(hv, (int)(4 * j + i), 64);
     const bool writer = lane < 8;
     if (writer && h_out)
         for (int i = 0; i < 4; i++) h_out[(size_t)blockIdx.x * 32 + 4 * j + i] = v[i];

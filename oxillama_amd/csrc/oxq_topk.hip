@@ -92,6 +92,7 @@ constexpr uint32_t SEL_CAP = 8192, SEL_THREADS = 1024;
 
 // Suffix scan over the bins from the top: the digit d with count(bins > d) < want <= count(bins >= d), and
 // those two counts.  All threads call; nb <= 4 * SEL_THREADS bins; result broadcast through `res`.
+template <uint32_t THREADS = SEL_THREADS>
 __device__ __forceinline__ void select_digit(const uint32_t *hist, uint32_t nb, uint32_t want, uint32_t *wave_tot,
                                              uint32_t *res, uint32_t &digit, uint32_t &above, uint32_t &equal) {
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -105,7 +106,7 @@ __device__ __forceinline__ void select_digit(const uint32_t *hist, uint32_t nb, 
     if (lane == 0) wave_tot[wave] = v;
     __syncthreads();
     uint32_t higher = 0;
-    for (uint32_t w = wave + 1; w < SEL_THREADS / 64; w++) higher += wave_tot[w];
+    for (uint32_t w = wave + 1; w < THREADS / 64; w++) higher += wave_tot[w];
     const uint32_t incl = v + higher, excl = incl - p;
     if (excl < want && incl >= want) {  // exactly one thread: the crossing is inside its four bins
         uint32_t run = excl;
@@ -151,14 +152,15 @@ struct SelectShared {
 // The smallest threshold t (low bits zero) such that exactly `want` of the keys `each` visits are >= t, found
 // W bits at a time from the top.  `each(fn)` calls fn(key, valid) for every key, the same number of times in every
 // thread of a wave; all threads of the work group call this function.
-template <int W, class Each>
+template <int W, uint32_t THREADS = SEL_THREADS, class Each>
 __device__ __forceinline__ uint64_t kth_threshold(Each &&each, uint32_t want, SelectShared &sh) {
+    static_assert((1u << W) <= 4 * THREADS, "a thread sums four bins in the scan");
     const uint32_t tid = threadIdx.x;
     uint64_t prefix = 0;  // the digits found so far
     uint32_t done = 0;    // how many bits that is
     while (true) {
         const uint32_t w = min((uint32_t)W, 64u - done), nb = 1u << w;
-        for (uint32_t b = tid; b < (nb < 4 ? 4 : nb); b += SEL_THREADS) sh.hist[b] = 0;
+        for (uint32_t b = tid; b < (nb < 4 ? 4 : nb); b += THREADS) sh.hist[b] = 0;
         __syncthreads();
         const uint32_t shift = 64 - done - w;
         each([&](uint64_t key, bool valid) {
@@ -167,7 +169,7 @@ __device__ __forceinline__ uint64_t kth_threshold(Each &&each, uint32_t want, Se
         });
         __syncthreads();
         uint32_t digit, above, equal;
-        select_digit(sh.hist, nb, want, sh.wave_tot, sh.res, digit, above, equal);
+        select_digit<THREADS>(sh.hist, nb, want, sh.wave_tot, sh.res, digit, above, equal);
         prefix = (prefix << w) | digit;
         done += w;
         want -= above;  // the threshold is the want-th largest of the keys that match the prefix
@@ -279,24 +281,117 @@ __global__ __launch_bounds__(SEL_THREADS) void topk_select_kernel(const float *_
     }
 }
 
+// ---- the same selection spread over the chip: two launches -------------------------------------------------------
+// One work group reading 128256 logits twice is what the kernel above spends its time on (31-39 us).  Here the vector
+// is cut into G slices; a work group per slice keeps its slice's keys in LDS and selects the slice's k largest with
+// the same digit search (a slice with at most k keys passes them all on); the G * k survivors (<= SEL_CAP) go to the
+// workspace, and one work group selects and ranks the k largest of those.  Exact for the same reason: every key of
+// the overall top k is among its own slice's top k.  12-bit digits: two rounds settle 24 bits of the value, which
+// separates a few thousand logits (8-bit digits take three; measured 14.6 us against 19.1 for k = 40 in a replayed
+// graph, 23.9 against 27.8 for k = 256).  After the lm_head GEMV (71 us): 87 us for the pair with k = 40.
+constexpr uint32_t SPREAD_THREADS = 1024;  // (four waves instead of sixteen measured slower: the key loops get longer)
+__global__ __launch_bounds__(SPREAD_THREADS) void topk_slice_select_kernel(const float *__restrict__ x, uint32_t n, uint32_t k,
+                                                                       uint32_t slice_len, uint64_t *__restrict__ ws) {
+    __shared__ SelectShared sh;
+    __shared__ uint64_t cand[SEL_CAP];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lo = blockIdx.x * slice_len, hi = min(n, lo + slice_len);
+    const uint32_t n_cand = hi > lo ? hi - lo : 0;
+    for (uint32_t j = tid; j < n_cand; j += SPREAD_THREADS) cand[j] = topk_key(x[lo + j], lo + j);
+    if (tid == 0) sh.counter = 0;
+    __syncthreads();
+    auto each_in_lds = [&](auto &&fn) {
+        for (uint32_t j0 = 0; j0 < n_cand; j0 += SPREAD_THREADS) {
+            const uint32_t j = j0 + tid;
+            fn(j < n_cand ? cand[j] : 0, j < n_cand);
+        }
+    };
+    uint64_t *out = ws + (size_t)blockIdx.x * k;
+    if (n_cand <= k) {  // the whole slice, padded with keys that rank below everything
+        for (uint32_t j = tid; j < k; j += SPREAD_THREADS) out[j] = j < n_cand ? cand[j] : 0;
+        return;
+    }
+    const uint64_t t = kth_threshold<12, SPREAD_THREADS>(each_in_lds, k, sh);
+    for (uint32_t j = tid; j < n_cand; j += SPREAD_THREADS) {
+        const uint64_t key = cand[j];
+        if (key >= t) out[atomicAdd(&sh.counter, 1u)] = key;  // exactly k of them
+    }
+}
+
+// The k largest of n_cand (<= SEL_CAP) keys, ranked, to the outputs.
+__global__ __launch_bounds__(SPREAD_THREADS) void topk_final_kernel(const uint64_t *__restrict__ ws, uint32_t n_cand, uint32_t k,
+                                                                float *__restrict__ out_vals, uint32_t *__restrict__ out_idx) {
+    __shared__ SelectShared sh;
+    __shared__ uint64_t cand[SEL_CAP];
+    __shared__ uint64_t sel[256];
+    const uint32_t tid = threadIdx.x;
+    for (uint32_t j = tid; j < n_cand; j += SPREAD_THREADS) cand[j] = ws[j];
+    if (tid == 0) sh.counter = 0;
+    __syncthreads();
+    auto each_in_lds = [&](auto &&fn) {
+        for (uint32_t j0 = 0; j0 < n_cand; j0 += SPREAD_THREADS) {
+            const uint32_t j = j0 + tid;
+            fn(j < n_cand ? cand[j] : 0, j < n_cand);
+        }
+    };
+    const uint64_t t = kth_threshold<12, SPREAD_THREADS>(each_in_lds, k, sh);
+    for (uint32_t j = tid; j < n_cand; j += SPREAD_THREADS) {
+        const uint64_t key = cand[j];
+        if (key >= t) sel[atomicAdd(&sh.counter, 1u)] = key;
+    }
+    __syncthreads();
+    if (tid < k) {
+        const uint64_t mine = sel[tid];
+        uint32_t rank = 0;
+        for (uint32_t j = 0; j < k; j++) rank += sel[j] > mine ? 1u : 0u;
+        out_vals[rank] = topk_value(mine);
+        out_idx[rank] = 0xFFFFFFFFu - (uint32_t)mine;
+    }
+}
+
+// Slices of the two-launch form for (n, k): 0 if it does not apply (every slice must fit the LDS key buffer, and the
+// slices' survivors together as well).
+static uint32_t topk_spread_slices(size_t n, size_t k) {
+    if (k == 0 || k > 256 || n <= 4096 || n > 0xFFFFFFFFull) return 0;  // a short vector: one work group does it
+    uint32_t g = (uint32_t)(SEL_CAP / k);
+    if (g > 64) g = 64;  // 16 to 128 slices measured alike (128256 logits: 17-19 us with 8-bit digits); 64 is the flat middle
+    const size_t len = (n + g - 1) / g;
+    return len <= SEL_CAP ? g : 0;
+}
+
 uint32_t topk_items(size_t n) {  // elements per lane in stage 1 so that at most 256 slices (of 64 lanes) result
     const size_t per = (n + 16383) / 16384;
     return per <= 8 ? 8 : per <= 16 ? 16 : per <= 32 ? 32 : per <= 64 ? 64 : 0;
 }
 
-// From this k on the radix select is the faster of the two (128256 logits: 31-39 us whatever k, against 13 us at
+// From this k on the radix select is the faster of the two one-work-group forms (128256 logits: 31-39 us whatever k, against 13 us at
 // k = 8, 26 us at 32, 36 us at 48, 47 us at 64, 173 us at 256 for the two-stage kernels).
 constexpr uint32_t TOPK_SELECT_MIN_K = 40;
+// ... and from this k on, for vectors of more than 4096 values whose slices fit, the two-launch form is faster still.
+constexpr uint32_t TOPK_SPREAD_MIN_K = 16;
 
 size_t topk_workspace_bytes(size_t n, size_t k) {
     const uint32_t items = topk_items(n);
     if (items == 0 || k == 0 || k > 256 || k > n) return 0;
     const size_t slices = (n + 64 * items - 1) / (64 * items);
-    return slices * k * sizeof(uint64_t);
+    const size_t spread = (size_t)topk_spread_slices(n, k) * k * sizeof(uint64_t);
+    const size_t waves = slices * k * sizeof(uint64_t);
+    return spread > waves ? spread : waves;
 }
 
 hipError_t launch_topk(const float *x, uint32_t n, uint32_t k, float *out_vals, uint32_t *out_idx, void *workspace,
                        hipStream_t stream) {
+    if (k >= TOPK_SPREAD_MIN_K) {
+        if (const uint32_t g = topk_spread_slices(n, k)) {  // slices selected side by side, then their survivors
+            const uint32_t len = (n + g - 1) / g;
+            uint64_t *ws = static_cast<uint64_t *>(workspace);
+            hipLaunchKernelGGL(topk_slice_select_kernel, dim3(g), dim3(SPREAD_THREADS), 0, stream, x, n, k, len, ws);
+            hipError_t e = hipGetLastError();
+            if (e != hipSuccess) return e;
+            hipLaunchKernelGGL(topk_final_kernel, dim3(1), dim3(SPREAD_THREADS), 0, stream, ws, g * k, k, out_vals, out_idx);
+            return hipGetLastError();
+        }
+    }
     if (k >= TOPK_SELECT_MIN_K) {  // radix select by one work group; needs no workspace
         hipLaunchKernelGGL(topk_select_kernel, dim3(1), dim3(SEL_THREADS), 0, stream, x, n, k, out_vals, out_idx);
         return hipGetLastError();
