@@ -39,7 +39,7 @@ struct Skinny<TileQ4K> {
     static constexpr bool OK = true;
     static constexpr uint32_t BLOCK = 144, ROW_STRIDE = 304;  // LDS bytes per row of a step (2 blocks + pad)
     static constexpr bool HAS_MIN = true;
-    static constexpr int ACT_PERM = 0;
+    static constexpr int ACT_PERM = 0, KSPLIT = 1;
     struct Raw {
         u32x4 hdr;
         u32x2 qs[4];
@@ -47,6 +47,7 @@ struct Skinny<TileQ4K> {
     static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk) {
         w.hdr = *reinterpret_cast<const u32x4 *>(blk);
     }
+    template <int U>
     static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
 #pragma unroll
         for (int g = 0; g < 4; g++) w.qs[g] = *reinterpret_cast<const u32x2 *>(blk + 16 + 32 * g + 8 * q);
@@ -76,7 +77,7 @@ struct Skinny<TileIQ4XS> {
     // 272 bytes = 68 dwords per row: lane (c, q) reads dword 68 c + q + const, bank 4 c + q -- all 64 distinct
     static constexpr uint32_t BLOCK = 136, ROW_STRIDE = 272;
     static constexpr bool HAS_MIN = false;
-    static constexpr int ACT_PERM = 1;
+    static constexpr int ACT_PERM = 1, KSPLIT = 1;
     struct Raw {
         u32x2 hdr;
         uint32_t qs[8];
@@ -84,6 +85,7 @@ struct Skinny<TileIQ4XS> {
     static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk) {
         w.hdr = *reinterpret_cast<const u32x2 *>(blk);
     }
+    template <int U>
     static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
 #pragma unroll
         for (int s = 0; s < 8; s++) w.qs[s] = *reinterpret_cast<const uint32_t *>(blk + 8 + 16 * s + 4 * q);
@@ -102,10 +104,93 @@ struct Skinny<TileIQ4XS> {
     }
 };
 
-constexpr uint32_t SKINNY_ACT_BYTES = 512 + 64 + 64;  // per (sub-block, token tile): int8 operands, fp32 scales, fp32 P
-constexpr uint32_t SKINNY_FAC_STRIDE = 17;            // floats per weight row in a wave's factor tables (16 + pad)
+// Q6_K (reference/q6_k.rs:25-75): 210 B = ql[128], qh[64], 16 int8 scales, d.  Sub-block s = 4 hh + p + 2 e of 32
+// weights has its low 4 bits in ql[64 hh + 32 p + l] (low nibble e = 0, high nibble e = 1) and its upper 2 bits in
+// qh[32 hh + l] at bit 2 p + 4 e; its two halves of 16 weights have their own scales, scales[2 s] and [2 s + 1].
+// Lane (c, q) takes weights 8q..8q+7 of every sub-block: 8 bytes of ql per (hh, p), 8 of qh per hh.
+//  * The step's second block starts 210 bytes into the row's strip: 2 past a multiple of 8.  Its fields are read as
+//    the aligned 8 bytes below plus the next dword, funnel-shifted.
+//  * One MFMA per half: the lanes of the other half (q / 2) supply zeros.  Each half's result is scaled by its own
+//    factor, as the reference scales 16 weights at a time (q6_k.rs:62-70).
+//  * The operand is q (0..63), not q - 32: the MFMA's addend carries -32 * sum of the token's 16 activations
+//    (integers, exact), so the result is the reference's sum of (q - 32) * a.
+template <>
+struct Skinny<TileQ6K> {
+    static constexpr bool OK = true;
+    // 432 bytes = 108 dwords per row: rows start on multiples of 16 bytes
+    static constexpr uint32_t BLOCK = 210, ROW_STRIDE = 432;
+    static constexpr bool HAS_MIN = false;
+    static constexpr int ACT_PERM = 0, KSPLIT = 2;
+    struct Raw {
+        u32x2 ql[4], qh[2];
+    };
+    struct __attribute__((packed, aligned(8), may_alias)) A8 { u32x2 v; };
+    struct __attribute__((packed, aligned(4), may_alias)) A4 { uint32_t v; };
+    struct __attribute__((packed, aligned(2), may_alias)) A2 { uint16_t v; };
+    // 8 bytes at p: U = 0 a multiple of 8, U = 1 two past one
+    template <int U>
+    static __device__ __forceinline__ u32x2 get8(const uint8_t *p) {
+        if constexpr (U == 0) {
+            return reinterpret_cast<const A8 *>(p)->v;
+        } else {
+            const u32x2 lo = reinterpret_cast<const A8 *>(p - 2)->v;
+            const uint32_t hi = reinterpret_cast<const A4 *>(p + 6)->v;
+            return u32x2{__builtin_amdgcn_alignbit(lo[1], lo[0], 16), __builtin_amdgcn_alignbit(hi, lo[1], 16)};
+        }
+    }
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) w.ql[g] = get8<U>(blk + 32 * g + 8 * q);
+#pragma unroll
+        for (int hh = 0; hh < 2; hh++) w.qh[hh] = get8<U>(blk + 128 + 32 * hh + 8 * q);
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const int hh = s >> 2, p = s & 1, e = (s >> 1) & 1, sh = 2 * p + 4 * e;
+        const u32x2 l = w.ql[2 * hh + p], h = w.qh[hh];
+        uint32_t v[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const uint32_t lo = e ? (l[i] >> 4) & 0x0F0F0F0Fu : l[i] & 0x0F0F0F0Fu;
+            const uint32_t hs = sh < 4 ? h[i] << (4 - sh) : h[i] >> (sh - 4);  // the 2-bit field to bits 4, 5
+            v[i] = (hs & 0x30303030u) | lo;
+        }
+        return (long)(((uint64_t)v[1] << 32) | v[0]);
+    }
+    // The factors of a block, decoded by the wave once: lane (c, q) takes row c's sub-blocks 2q and 2q + 1, both
+    // halves of each -- scales[4q .. 4q + 3], table slots 4q .. 4q + 3 (slot = 2 * sub-block + half).
+    template <int U>
+    static __device__ __forceinline__ void block_factors(const uint8_t *blk, uint32_t q, float (&f)[4]) {
+        uint32_t sc;
+        if constexpr (U == 0) {
+            sc = reinterpret_cast<const A4 *>(blk + 192 + 4 * q)->v;
+        } else {
+            const uint32_t lo = reinterpret_cast<const A4 *>(blk + 190 + 4 * q)->v;
+            const uint32_t hi = reinterpret_cast<const A4 *>(blk + 194 + 4 * q)->v;
+            sc = __builtin_amdgcn_alignbit(hi, lo, 16);
+        }
+        const float d = h2f(reinterpret_cast<const A2 *>(blk + 208)->v);
+#pragma unroll
+        for (int b = 0; b < 4; b++) f[b] = d * (float)(int)(int8_t)((sc >> (8 * b)) & 0xFF);  // reference/q6_k.rs:62, exact
+    }
+};
+
+// LDS bytes per (sub-block, token tile): int8 operands, fp32 scales, and fp32 P (one factor per sub-block) or the
+// MFMA addends of the two halves (two factors)
+template <class F>
+constexpr uint32_t skinny_act_bytes() {
+    return 512 + 64 + (Skinny<F>::KSPLIT == 2 ? 128 : 64);
+}
+constexpr uint32_t SKINNY_FAC_STRIDE = 17;  // floats per weight row in a wave's factor tables (16 + pad)
+// LDS bytes of a wave: the strip of its rows' bytes of a step, and the factor tables (one factor per sub-block: of
+// the step's 16 sub-blocks, and a second table where the format has a zero-point term; two factors: of one block's)
+template <class F, int NT>
+constexpr uint32_t skinny_wave_lds() {
+    return NT * 16 * (Skinny<F>::ROW_STRIDE + SKINNY_FAC_STRIDE * 4 * (Skinny<F>::HAS_MIN ? 2 : 1));
+}
 
 typedef float v4f32 __attribute__((ext_vector_type(4)));
+struct __attribute__((packed, aligned(4))) StripA4 { u32x4 v; };
 
 // Work group = WAVES waves, each with its own NT x 16 weight rows; all of them the same token tiles (at most TT of
 // 16 tokens).  k is walked in chunks of `per` super-blocks (even): the work group stages the chunk's token bytes,
@@ -118,8 +203,7 @@ typedef float v4f32 __attribute__((ext_vector_type(4)));
 // Waves per SIMD the shape is meant to run at: two work groups on a compute unit where their LDS allows it.
 template <class F, int NT, int WAVES, int TT, int PER>
 constexpr int skinny_waves_per_simd() {
-    constexpr size_t lds = (size_t)PER * 8 * TT * SKINNY_ACT_BYTES +
-                           (size_t)WAVES * NT * 16 * (Skinny<F>::ROW_STRIDE + SKINNY_FAC_STRIDE * 4 * (Skinny<F>::HAS_MIN ? 2 : 1));
+    constexpr size_t lds = (size_t)PER * 8 * TT * skinny_act_bytes<F>() + (size_t)WAVES * skinny_wave_lds<F, NT>();
     return lds <= 80 * 1024 ? WAVES / 2 : WAVES / 4;
 }
 
@@ -132,10 +216,14 @@ __device__ __forceinline__ void gemm_skinny_body(
     const uint32_t gy, const uint32_t ks) {
     using S = Skinny<F>;
     constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: as_float(0x4B400000 + i) == MAGIC + i for |i| < 2^22
-    constexpr uint32_t RS = S::ROW_STRIDE, SEG = 2 * S::BLOCK, PPR = SEG / 16;  // 16-byte pieces per row per step
-    constexpr uint32_t PIECES = NT * 16 * PPR, NL = (PIECES + 63) / 64;
+    constexpr int KS = S::KSPLIT;  // MFMAs (and scale factors) per sub-block
+    // a row's bytes of a step as 16-byte pieces: FULL whole ones from the start, and where the step's length is not
+    // a multiple of 16 one more that ends with the step (overlapping the last whole one).  The whole pieces of all
+    // rows come first in the lanes' order, then the rows' last pieces.
+    constexpr uint32_t RS = S::ROW_STRIDE, SEG = 2 * S::BLOCK, FULL = SEG / 16, TAIL = SEG % 16 ? 1 : 0;
+    constexpr uint32_t NFULL = NT * 16 * FULL, PIECES = NFULL + TAIL * NT * 16, NL = (PIECES + 63) / 64;
     constexpr uint32_t THREADS = 64 * WAVES, FS = SKINNY_FAC_STRIDE;
-    constexpr uint32_t WAVE_LDS = NT * 16 * (RS + FS * 4 * (S::HAS_MIN ? 2 : 1));
+    constexpr uint32_t WAVE_LDS = skinny_wave_lds<F, NT>();
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t lane = threadIdx.x & 63, c = lane & 15, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -145,8 +233,9 @@ __device__ __forceinline__ void gemm_skinny_body(
     constexpr uint32_t per = PER, nblk_max = PER * 8;  // sub-blocks (Q8_0 blocks per token) of a full chunk
     uint8_t *const ldsA = lds;
     float *const ldsD = reinterpret_cast<float *>(ldsA + (size_t)nblk_max * TT * 512);
-    float *const ldsP = ldsD + (size_t)nblk_max * TT * 16;
-    uint8_t *const strip = reinterpret_cast<uint8_t *>(ldsP + (size_t)nblk_max * TT * 16) + wave * WAVE_LDS;
+    float *const ldsP = ldsD + (size_t)nblk_max * TT * 16;       // one factor per sub-block: P
+    int *const ldsC = reinterpret_cast<int *>(ldsP);             // two: the MFMA addends, [block][tile][half][16 tokens]
+    uint8_t *const strip = reinterpret_cast<uint8_t *>(ldsP + (size_t)nblk_max * TT * 16 * KS) + wave * WAVE_LDS;
     float *const dscT = reinterpret_cast<float *>(strip + NT * 16 * RS);
     float *const minT = dscT + NT * 16 * FS;
 
@@ -190,6 +279,13 @@ __device__ __forceinline__ void gemm_skinny_body(
                 sum += xor2_i(sum);
                 if (qq == 0) ldsP[(idx >> 6) * 16 + cc] = d * (float)sum;
             }
+            if (KS == 2) {
+                // per half of the block (threads 0, 1 and 2, 3): the addend that turns sum(q a) into sum((q - 32) a),
+                // on top of the 1.5 * 2^23 every result carries
+                int sum = sdot4(v[0], 0x01010101u, sdot4(v[1], 0x01010101u, 0));
+                sum += xor1_i(sum);
+                if ((qq & 1) == 0) ldsC[((idx >> 6) * 2 + (qq >> 1)) * 16 + cc] = 0x4B400000 - 32 * sum;
+            }
             if (S::ACT_PERM == 1) {  // even bytes, then odd bytes
                 const uint32_t x0 = v[0], x1 = v[1];
                 v[0] = __builtin_amdgcn_perm(x1, x0, 0x06040200u);
@@ -209,9 +305,10 @@ __device__ __forceinline__ void gemm_skinny_body(
     uint32_t dst[NL];
 #pragma unroll
     for (uint32_t i = 0; i < NL; i++) {
-        const uint32_t p = min(i * 64 + lane, PIECES - 1), r = p / PPR, piece = p % PPR;
-        src[i] = We + (size_t)min(rbase + r, n - 1) * row_bytes + piece * 16;
-        dst[i] = r * RS + piece * 16;
+        const uint32_t p = min(i * 64 + lane, PIECES - 1);
+        const uint32_t r = p < NFULL ? p / FULL : p - NFULL, at = p < NFULL ? (p % FULL) * 16 : SEG - 16;
+        src[i] = We + (size_t)min(rbase + r, n - 1) * row_bytes + at;
+        dst[i] = r * RS + at;
     }
     const uint32_t tiles_here = min((uint32_t)TT, (tok_end - tokb + 15) / 16);
     v4f32 acc[TT][NT];
@@ -225,6 +322,7 @@ __device__ __forceinline__ void gemm_skinny_body(
     v4i32 magic;
     asm volatile("v_mov_b32 %0, 0x4b400000\n\tv_mov_b32 %1, 0x4b400000\n\tv_mov_b32 %2, 0x4b400000\n\tv_mov_b32 %3, 0x4b400000"
                  : "=v"(magic[0]), "=v"(magic[1]), "=v"(magic[2]), "=v"(magic[3]));
+    const uint64_t half_mask = q < 2 ? ~0ull : 0ull;
     u32x4 stage[NL];
 #pragma unroll
     for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i] + (size_t)(sb_lo / 2) * SEG);
@@ -246,7 +344,12 @@ __device__ __forceinline__ void gemm_skinny_body(
     for (uint32_t st = sb0 / 2; st < (sb0 + nsbc) / 2; st++) {
         // the step's bytes to the strip (pieces past the end, on the last load: the last piece again, same value)
 #pragma unroll
-        for (uint32_t i = 0; i < NL; i++) *reinterpret_cast<u32x4 *>(strip + dst[i]) = stage[i];
+        for (uint32_t i = 0; i < NL; i++) {
+            if (TAIL && (i + 1) * 64 > NFULL)  // rows' last pieces among them: on dword boundaries only
+                reinterpret_cast<StripA4 *>(strip + dst[i])->v = stage[i];
+            else
+                *reinterpret_cast<u32x4 *>(strip + dst[i]) = stage[i];
+        }
         if (st + 1 < steps) {
 #pragma unroll
             for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i] + (size_t)(st + 1) * SEG);
@@ -255,7 +358,8 @@ __device__ __forceinline__ void gemm_skinny_body(
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // scale factors of the step, decoded once: lane (c, q) takes row c, super-block q / 2, sub-blocks
-        // 4 (q % 2) .. + 3, for each tile
+        // 4 (q % 2) .. + 3, for each tile (two factors per sub-block: per block, below)
+        if constexpr (KS == 1)
 #pragma unroll
         for (int j = 0; j < NT; j++) {
             typename S::Raw hd;
@@ -275,8 +379,29 @@ __device__ __forceinline__ void gemm_skinny_body(
         for (int u = 0; u < 2; u++) {
             typename S::Raw raw[NT];
 #pragma unroll
-            for (int j = 0; j < NT; j++) S::read(raw[j], strip + (16 * j + c) * RS + u * S::BLOCK, q);
+            for (int j = 0; j < NT; j++) {  // (u is a constant once the loop is unrolled)
+                const uint8_t *blk = strip + (16 * j + c) * RS + u * S::BLOCK;
+                if (u == 0) S::template read<0>(raw[j], blk, q);
+                else S::template read<1>(raw[j], blk, q);
+            }
             const uint32_t b0 = (st * 2 + u - sb0) * 8;
+            if constexpr (KS == 2) {
+                // the block's factors (the table holds one block's: the last block's readers are done)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int j = 0; j < NT; j++) {
+                    float f[4];
+                    const uint8_t *blk = strip + (16 * j + c) * RS + u * S::BLOCK;
+                    if (u == 0) S::template block_factors<0>(blk, q, f);
+                    else S::template block_factors<1>(blk, q, f);
+#pragma unroll
+                    for (int b = 0; b < 4; b++) dscT[(16 * j + c) * FS + 4 * q + b] = f[b];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            }
             if (S::HAS_MIN) {
                 // zero-point term: per four sub-blocks one 16 x 16 x 4 fp32 product of P (tokens x sub-blocks) and the
                 // rows' factors, straight into the accumulators
@@ -295,13 +420,18 @@ __device__ __forceinline__ void gemm_skinny_body(
             }
 #pragma unroll
             for (int s = 0; s < 8; s++) {
-                float dsc[NT], corr[NT];
-                long bop[NT];
+                float dsc[NT][KS], corr[NT][KS];
+                long bop[NT][KS];
 #pragma unroll
                 for (int j = 0; j < NT; j++) {
-                    dsc[j] = dscT[(16 * j + c) * FS + u * 8 + s];
-                    corr[j] = -(MAGIC * dsc[j]);
-                    bop[j] = S::operand(raw[j], s);
+                    const long op = S::operand(raw[j], s);
+#pragma unroll
+                    for (int is = 0; is < KS; is++) {
+                        dsc[j][is] = dscT[(16 * j + c) * FS + (KS == 2 ? 2 * s + is : u * 8 + s)];
+                        corr[j][is] = -(MAGIC * dsc[j][is]);
+                        // two factors: k-values 0..15 come from the lanes q = 0, 1, the others supply zeros; and so on
+                        bop[j][is] = KS == 2 ? (long)((uint64_t)op & (is == 0 ? half_mask : ~half_mask)) : op;
+                    }
                 }
 #pragma unroll
                 for (int t = 0; t < TN; t++) {
@@ -311,17 +441,23 @@ __device__ __forceinline__ void gemm_skinny_body(
                         const long a = (long)(((uint64_t)av[1] << 32) | av[0]);
                         const v4f32 da = *reinterpret_cast<const v4f32 *>(ldsD + (size_t)e * 16 + 4 * q);
 #pragma unroll
-                        for (int j = 0; j < NT; j++) {
-                            const v4i32 r = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bop[j], magic, 0, 0, 0);
+                        for (int is = 0; is < KS; is++) {
+                            v4i32 addend = magic;
+                            if constexpr (KS == 2) addend = *reinterpret_cast<const v4i32 *>(ldsC + ((size_t)e * 2 + is) * 16 + 4 * q);
 #pragma unroll
-                            for (int v = 0; v < 4; v++) {
-                                const int ri = r[v];
-                                const float tt = fmaf(__builtin_bit_cast(float, ri), dsc[j], corr[j]);  // fl(dsc * isum)
-                                acc[t][j][v] = fmaf(tt, da[v], acc[t][j][v]);
-                                if (DUMP) {  // the integer sum of (token, weight row, sub-block)
-                                    const uint32_t tok = tokb + 16 * t + 4 * q + v, row = rbase + 16 * j + c;
-                                    if (tok < tok_end && row < n)
-                                        sums[((size_t)tok * n + row) * (k / 32) + (st * 2 + u) * 8 + s] = ri - 0x4B400000;
+                            for (int j = 0; j < NT; j++) {
+                                const v4i32 r = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bop[j][is], addend, 0, 0, 0);
+#pragma unroll
+                                for (int v = 0; v < 4; v++) {
+                                    const int ri = r[v];
+                                    const float tt = fmaf(__builtin_bit_cast(float, ri), dsc[j][is], corr[j][is]);  // fl(dsc * isum)
+                                    acc[t][j][v] = fmaf(tt, da[v], acc[t][j][v]);
+                                    if (DUMP) {  // the integer sum of (token, weight row, sub-block or half of one)
+                                        const uint32_t tok = tokb + 16 * t + 4 * q + v, row = rbase + 16 * j + c;
+                                        if (tok < tok_end && row < n)
+                                            sums[((size_t)tok * n + row) * (k / 32 * KS) + ((st * 2 + u) * 8 + s) * KS + is] =
+                                                ri - 0x4B400000;
+                                    }
                                 }
                             }
                         }
@@ -455,9 +591,9 @@ constexpr uint32_t SKINNY_GROUPED_SPLITS = 2, SKINNY_GROUPED_SPLIT_MAX_N = 8192;
 template <class F, int NT, int WAVES, int TT, int PER, bool DUMP = false>
 static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipStream_t stream, bool split_k = false) {
     using S = Skinny<F>;
-    const size_t strips = (size_t)WAVES * NT * 16 * (S::ROW_STRIDE + SKINNY_FAC_STRIDE * 4 * (S::HAS_MIN ? 2 : 1));
+    const size_t strips = (size_t)WAVES * skinny_wave_lds<F, NT>();
     auto kern = &gemm_skinny_kernel<F, NT, WAVES, TT, PER, DUMP>;
-    const size_t lds = (size_t)PER * 8 * TT * SKINNY_ACT_BYTES + strips;
+    const size_t lds = (size_t)PER * 8 * TT * skinny_act_bytes<F>() + strips;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        (int)lds);
     if (e != hipSuccess) return e;
@@ -516,6 +652,8 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
         // whole steps of two super-blocks
         if (a.k % 512 != 0 || rows > 32) return SK_NONE;
         const bool two = rows > 16;
+        // two factors per sub-block: the one-tile shapes only (see launch_skinny)
+        if (Skinny<F>::KSPLIT == 2 && (two || (variant != 0 && variant != 200))) return SK_NONE;
         if (a.sums && variant != 0 && variant != 200) return SK_NONE;  // the dump exists for the default shapes
         switch (variant) {
         case 0: {
@@ -554,7 +692,17 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
 // <NT, WAVES, TT, PER>; LDS = PER * 8 * TT * 640 + WAVES * NT * 7 KB
 template <class F>
 static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_t stream, int shape) {
-    if constexpr (Skinny<F>::OK) {
+    if constexpr (Skinny<F>::OK && Skinny<F>::KSPLIT == 2) {
+        // Q6_K: 8 KB of LDS per wave; with chunks of two super-blocks of one token tile two work groups still share
+        // a compute unit (75 KB each)
+        switch (shape) {
+        case SK_1_4:
+        case SK_1_8: return a.sums ? launch_skinny_shape<F, 1, 8, 1, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 2>(a, p, stream);
+        case SK_1_4_SPLIT:
+            return a.sums ? launch_skinny_shape<F, 1, 8, 1, 2, true>(a, p, stream, true) : launch_skinny_shape<F, 1, 8, 1, 2>(a, p, stream, true);
+        default: break;
+        }
+    } else if constexpr (Skinny<F>::OK) {
         switch (shape) {
         case SK_1_4: return a.sums ? launch_skinny_shape<F, 1, 8, 1, 4, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 4>(a, p, stream);
         case SK_2_2: return a.sums ? launch_skinny_shape<F, 1, 8, 2, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 2, 2>(a, p, stream);
