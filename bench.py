@@ -585,6 +585,7 @@ def main():
                     "frac_hbm_peak": round(wb / us / 1e3 / HBM_PEAK_GBPS, 4), "tile_kernel_us_per_call": round(tile_us, 3)}
         kernels["batch16_q4k_gate_14336x4096"] = time_batch(k_q4k, Q4_K, [w["gate"] for w in layers], 16, F, H)
         kernels["batch16_q4k_down_shape_4096x14336"] = time_batch(k_q4k, Q4_K, [w["gate"] for w in layers], 16, H, F)
+        kernels["batch16_q6k_down_4096x14336"] = time_batch(k_q6k, Q6_K, [w["down"] for w in layers], 16, H, F)
         V = 128256
         lm = [upload(Q6_K, 6000 + i, V, H) for i in range(2)]
         logits = torch.zeros(V, dtype=torch.float32, device=dev)
@@ -881,7 +882,9 @@ def main():
                "c3_lm_head_us": get(kernels, "c3_lm_head_q6k_128256x4096", "us_per_call"),
                "prefill_frac_int8_peak": get(prefill, "frac_int8_peak"), "prefill_gemm_us": get(prefill, "gemm_us"),
                "prefill_TOPS": get(prefill, "TOPS"), "moe_us": get(moe_out, "us_per_step"),
-               "moe_frac": get(moe_out, "frac_hbm_peak")}
+               "moe_frac": get(moe_out, "frac_hbm_peak"),
+               "batch16_q4k_4096x14336_us": get(kernels, "batch16_q4k_down_shape_4096x14336", "us_per_call"),
+               "batch16_q6k_4096x14336_us": get(kernels, "batch16_q6k_down_4096x14336", "us_per_call")}
     out = {
         "metric": "Q4_K GEMV weight GB/s (% HBM peak); batch-512 prefill int8-MFMA TOPS",
         "value": round(value, 1),

@@ -272,11 +272,12 @@ def test_skinny_split_k_on_the_host_routes(hip, ref):
     assert np.array_equal(dy.cpu().numpy(), y)
 
 
-@pytest.mark.parametrize("case", [(O.IQ4_XS, 3, 8192, 4096), (O.Q4_K, 5, 4096, 8192), (O.Q4_K, 4, 8192, 4096)],
+@pytest.mark.parametrize("case", [(O.IQ4_XS, 3, 8192, 4096), (O.Q4_K, 5, 4096, 8192), (O.Q4_K, 4, 8192, 4096),
+                                  (O.Q6_K, 5, 4096, 8192), (O.Q6_K, 4, 4096, 8192)],
                          ids=lambda c: "%s_m%d_%dx%d" % (O.NAMES[c[0]], c[1], c[2], c[3]))
 def test_few_rows_take_the_few_token_kernel_when_a_workspace_has_room(hip, ref, case):
     """Below the tile kernel's row threshold the GEMV launches serve a matmul, four rows per pass -- except where the
-    few-token kernel is faster still (IQ4_XS from 3 rows, Q4_K from 5, on shapes it splits over k) and the caller's
+    few-token kernel is faster still (IQ4_XS from 3 rows, Q4_K and Q6_K from 5, on shapes it splits over k) and the caller's
     workspace has room for its sums.  Without a workspace, or with a small one, the GEMV launches stay."""
     import torch
     t, m, n, k_ = case
@@ -285,7 +286,7 @@ def test_few_rows_take_the_few_token_kernel_when_a_workspace_has_room(hip, ref, 
     kern = hip.HipKernel(t)
     dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
     ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
-    expect_skinny = (t == O.IQ4_XS and m >= 3) or (t == O.Q4_K and m >= 5)
+    expect_skinny = (t == O.IQ4_XS and m >= 3) or (t in (O.Q4_K, O.Q6_K) and m >= 5)
     outs = []
     for workspace in (ws, ws[:4096], None):
         dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
