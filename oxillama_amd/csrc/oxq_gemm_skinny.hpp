@@ -38,13 +38,13 @@ template <>
 struct Skinny<TileQ4K> {
     static constexpr bool OK = true;
     static constexpr uint32_t BLOCK = 144, ROW_STRIDE = 304;  // LDS bytes per row of a step (2 blocks + pad)
-    static constexpr bool HAS_MIN = true;
+    static constexpr bool HAS_MIN = true, TABLE = true, ONE_TILE = false;
     static constexpr int ACT_PERM = 0, KSPLIT = 1;
     struct Raw {
         u32x4 hdr;
         u32x2 qs[4];
     };
-    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk) {
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk, uint32_t) {
         w.hdr = *reinterpret_cast<const u32x4 *>(blk);
     }
     template <int U>
@@ -58,11 +58,12 @@ struct Skinny<TileQ4K> {
         const uint32_t hi = (s & 1) ? (v[1] >> 4) & 0x0F0F0F0Fu : v[1] & 0x0F0F0F0Fu;
         return (long)(((uint64_t)hi << 32) | lo);
     }
-    static __device__ __forceinline__ void factors(const Raw &w, int s, float &dsc, float &qneg) {
+    // factors of sub-block 4 * half + i
+    static __device__ __forceinline__ void factors(const Raw &w, uint32_t half, int i, float &dsc, float &qneg) {
         TileQ4K::Hdr hd;
         hd.w = w.hdr;
         float d1[1];
-        TileQ4K::factors(hd, 0, (uint32_t)s, d1, qneg);
+        TileQ4K::factors(hd, 0, 4 * half + i, d1, qneg);
         dsc = d1[0];
     }
 };
@@ -76,13 +77,13 @@ struct Skinny<TileIQ4XS> {
     static constexpr bool OK = true;
     // 272 bytes = 68 dwords per row: lane (c, q) reads dword 68 c + q + const, bank 4 c + q -- all 64 distinct
     static constexpr uint32_t BLOCK = 136, ROW_STRIDE = 272;
-    static constexpr bool HAS_MIN = false;
+    static constexpr bool HAS_MIN = false, TABLE = true, ONE_TILE = false;
     static constexpr int ACT_PERM = 1, KSPLIT = 1;
     struct Raw {
         u32x2 hdr;
         uint32_t qs[8];
     };
-    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk) {
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk, uint32_t) {
         w.hdr = *reinterpret_cast<const u32x2 *>(blk);
     }
     template <int U>
@@ -95,13 +96,114 @@ struct Skinny<TileIQ4XS> {
         const uint32_t hi = FmtIQ4XS::lut4((w.qs[s] >> 4) & 0x0F0F0F0Fu);
         return (long)(((uint64_t)hi << 32) | lo);
     }
-    static __device__ __forceinline__ void factors(const Raw &w, int s, float &dsc, float &qneg) {
+    static __device__ __forceinline__ void factors(const Raw &w, uint32_t half, int i, float &dsc, float &qneg) {
         TileIQ4XS::Hdr hd;
         hd.w = u32x4{w.hdr[0], w.hdr[1], 0, 0};
         float d1[1];
-        TileIQ4XS::factors(hd, 0, (uint32_t)s, d1, qneg);
+        TileIQ4XS::factors(hd, 0, 4 * half + i, d1, qneg);
         dsc = d1[0];
     }
+};
+
+// LDS accesses of the strip at less than their natural alignment (the formats whose fields sit at odd multiples of 2)
+struct __attribute__((packed, aligned(8), may_alias)) StripR8 { u32x2 v; };
+struct __attribute__((packed, aligned(4), may_alias)) StripR4 { uint32_t v; };
+struct __attribute__((packed, aligned(2), may_alias)) StripR2 { uint16_t v; };
+// 8 bytes at p, which is MIS (0, 2, 4, 6) past a multiple of 8.  2 or 6 past: the three dwords from p - 2 on (an
+// aligned 8 bytes and a dword, in this order or the other), funnel-shifted; 4 past: two dwords as they are
+template <int MIS>
+__device__ __forceinline__ u32x2 strip_get8(const uint8_t *p) {
+    if constexpr (MIS == 0) {
+        return reinterpret_cast<const StripR8 *>(p)->v;
+    } else if constexpr (MIS == 4) {
+        return u32x2{reinterpret_cast<const StripR4 *>(p)->v, reinterpret_cast<const StripR4 *>(p + 4)->v};
+    } else if constexpr (MIS == 2) {
+        const u32x2 lo = reinterpret_cast<const StripR8 *>(p - 2)->v;
+        const uint32_t hi = reinterpret_cast<const StripR4 *>(p + 6)->v;
+        return u32x2{__builtin_amdgcn_alignbit(lo[1], lo[0], 16), __builtin_amdgcn_alignbit(hi, lo[1], 16)};
+    } else {
+        const uint32_t lo = reinterpret_cast<const StripR4 *>(p - 2)->v;
+        const u32x2 hi = reinterpret_cast<const StripR8 *>(p + 2)->v;
+        return u32x2{__builtin_amdgcn_alignbit(hi[0], lo, 16), __builtin_amdgcn_alignbit(hi[1], hi[0], 16)};
+    }
+}
+// 4 bytes at p, MIS (0 or 2) past a multiple of 4
+template <int MIS>
+__device__ __forceinline__ uint32_t strip_get4(const uint8_t *p) {
+    if constexpr (MIS == 0) {
+        return reinterpret_cast<const StripR4 *>(p)->v;
+    } else {
+        return __builtin_amdgcn_alignbit(reinterpret_cast<const StripR4 *>(p + 2)->v, reinterpret_cast<const StripR4 *>(p - 2)->v, 16);
+    }
+}
+
+// Q4_0 (reference/q4_0.rs:22-49): 18 B = d, 16 bytes of nibbles, byte j = weights 2j (low) and 2j + 1 (high), each
+// minus 8.  Eight blocks (144 B) stand for a super-block.  Lane (c, q) takes bytes 4q..4q+3 of each block, as for
+// IQ4_XS; they sit 2 past a dword boundary in the even blocks.  The operand is the unsigned nibble; the "- 8" goes
+// through the zero-point term (P times -8 d), as in the tile kernel.
+template <>
+struct Skinny<TileQ4_0> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 144, ROW_STRIDE = 304;
+    static constexpr bool HAS_MIN = true, TABLE = true, ONE_TILE = false;
+    static constexpr int ACT_PERM = 1, KSPLIT = 1;
+    struct Raw {
+        uint32_t d[4];
+        uint32_t qs[8];
+    };
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk, uint32_t half) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) w.d[i] = reinterpret_cast<const StripR2 *>(blk + 18 * (4 * half + i))->v;
+    }
+    static __device__ __forceinline__ void factors(const Raw &w, uint32_t, int i, float &dsc, float &qneg) {
+        dsc = h2f(w.d[i]);
+        qneg = -(8.0f * dsc);  // exact
+    }
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int s = 0; s < 8; s += 2) {
+            w.qs[s] = strip_get4<2>(blk + 18 * s + 2 + 4 * q);
+            w.qs[s + 1] = strip_get4<0>(blk + 18 * (s + 1) + 2 + 4 * q);
+        }
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const uint32_t lo = w.qs[s] & 0x0F0F0F0Fu, hi = (w.qs[s] >> 4) & 0x0F0F0F0Fu;
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+};
+
+// Q8_0 weights (reference/q8_0.rs:22-47): 34 B = d, 32 int8, the operand as it is.  Eight blocks (272 B) stand for a
+// super-block; a row's step is 544 bytes, and the strip rows are packed at that stride: with it, the token bytes
+// of a chunk of two super-blocks and no factor table, two work groups still share a compute unit's LDS.  The
+// scale is read from the strip with the block's bytes.  Lane (c, q) takes payload bytes 8q..8q+7, which sit 2, 4, 6
+// or 0 bytes past a multiple of 8 as the block index goes up.
+template <>
+struct Skinny<TileQ8_0> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 272, ROW_STRIDE = 544;
+    static constexpr bool HAS_MIN = false, TABLE = false, ONE_TILE = true;
+    static constexpr int ACT_PERM = 0, KSPLIT = 1;
+    struct Raw {
+        uint32_t d[8];
+        u32x2 qs[8];
+    };
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int s = 0; s < 8; s += 4) {
+            w.qs[s] = strip_get8<2>(blk + 34 * s + 2 + 8 * q);
+            w.qs[s + 1] = strip_get8<4>(blk + 34 * (s + 1) + 2 + 8 * q);
+            w.qs[s + 2] = strip_get8<6>(blk + 34 * (s + 2) + 2 + 8 * q);
+            w.qs[s + 3] = strip_get8<0>(blk + 34 * (s + 3) + 2 + 8 * q);
+        }
+#pragma unroll
+        for (int s = 0; s < 8; s++) w.d[s] = reinterpret_cast<const StripR2 *>(blk + 34 * s)->v;
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        return (long)(((uint64_t)w.qs[s][1] << 32) | w.qs[s][0]);
+    }
+    static __device__ __forceinline__ float scale(const Raw &w, int s) { return h2f(w.d[s]); }
 };
 
 // Q6_K (reference/q6_k.rs:25-75): 210 B = ql[128], qh[64], 16 int8 scales, d.  Sub-block s = 4 hh + p + 2 e of 32
@@ -119,31 +221,18 @@ struct Skinny<TileQ6K> {
     static constexpr bool OK = true;
     // 432 bytes = 108 dwords per row: rows start on multiples of 16 bytes
     static constexpr uint32_t BLOCK = 210, ROW_STRIDE = 432;
-    static constexpr bool HAS_MIN = false;
+    static constexpr bool HAS_MIN = false, TABLE = true, ONE_TILE = true;
     static constexpr int ACT_PERM = 0, KSPLIT = 2;
     struct Raw {
         u32x2 ql[4], qh[2];
     };
-    struct __attribute__((packed, aligned(8), may_alias)) A8 { u32x2 v; };
-    struct __attribute__((packed, aligned(4), may_alias)) A4 { uint32_t v; };
-    struct __attribute__((packed, aligned(2), may_alias)) A2 { uint16_t v; };
-    // 8 bytes at p: U = 0 a multiple of 8, U = 1 two past one
-    template <int U>
-    static __device__ __forceinline__ u32x2 get8(const uint8_t *p) {
-        if constexpr (U == 0) {
-            return reinterpret_cast<const A8 *>(p)->v;
-        } else {
-            const u32x2 lo = reinterpret_cast<const A8 *>(p - 2)->v;
-            const uint32_t hi = reinterpret_cast<const A4 *>(p + 6)->v;
-            return u32x2{__builtin_amdgcn_alignbit(lo[1], lo[0], 16), __builtin_amdgcn_alignbit(hi, lo[1], 16)};
-        }
-    }
+    // U: the step's first block (fields on multiples of 8) or its second (2 past)
     template <int U>
     static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
 #pragma unroll
-        for (int g = 0; g < 4; g++) w.ql[g] = get8<U>(blk + 32 * g + 8 * q);
+        for (int g = 0; g < 4; g++) w.ql[g] = strip_get8<2 * U>(blk + 32 * g + 8 * q);
 #pragma unroll
-        for (int hh = 0; hh < 2; hh++) w.qh[hh] = get8<U>(blk + 128 + 32 * hh + 8 * q);
+        for (int hh = 0; hh < 2; hh++) w.qh[hh] = strip_get8<2 * U>(blk + 128 + 32 * hh + 8 * q);
     }
     static __device__ __forceinline__ long operand(const Raw &w, int s) {
         const int hh = s >> 2, p = s & 1, e = (s >> 1) & 1, sh = 2 * p + 4 * e;
@@ -161,15 +250,8 @@ struct Skinny<TileQ6K> {
     // halves of each -- scales[4q .. 4q + 3], table slots 4q .. 4q + 3 (slot = 2 * sub-block + half).
     template <int U>
     static __device__ __forceinline__ void block_factors(const uint8_t *blk, uint32_t q, float (&f)[4]) {
-        uint32_t sc;
-        if constexpr (U == 0) {
-            sc = reinterpret_cast<const A4 *>(blk + 192 + 4 * q)->v;
-        } else {
-            const uint32_t lo = reinterpret_cast<const A4 *>(blk + 190 + 4 * q)->v;
-            const uint32_t hi = reinterpret_cast<const A4 *>(blk + 194 + 4 * q)->v;
-            sc = __builtin_amdgcn_alignbit(hi, lo, 16);
-        }
-        const float d = h2f(reinterpret_cast<const A2 *>(blk + 208)->v);
+        const uint32_t sc = strip_get4<2 * U>(blk + 192 + 4 * q);
+        const float d = h2f(reinterpret_cast<const StripR2 *>(blk + 208)->v);
 #pragma unroll
         for (int b = 0; b < 4; b++) f[b] = d * (float)(int)(int8_t)((sc >> (8 * b)) & 0xFF);  // reference/q6_k.rs:62, exact
     }
@@ -186,7 +268,7 @@ constexpr uint32_t SKINNY_FAC_STRIDE = 17;  // floats per weight row in a wave's
 // the step's 16 sub-blocks, and a second table where the format has a zero-point term; two factors: of one block's)
 template <class F, int NT>
 constexpr uint32_t skinny_wave_lds() {
-    return NT * 16 * (Skinny<F>::ROW_STRIDE + SKINNY_FAC_STRIDE * 4 * (Skinny<F>::HAS_MIN ? 2 : 1));
+    return NT * 16 * (Skinny<F>::ROW_STRIDE + (Skinny<F>::TABLE ? SKINNY_FAC_STRIDE * 4 * (Skinny<F>::HAS_MIN ? 2 : 1) : 0));
 }
 
 typedef float v4f32 __attribute__((ext_vector_type(4)));
@@ -218,10 +300,12 @@ __device__ __forceinline__ void gemm_skinny_body(
     constexpr float MAGIC = 12582912.0f;  // 1.5 * 2^23: as_float(0x4B400000 + i) == MAGIC + i for |i| < 2^22
     constexpr int KS = S::KSPLIT;  // MFMAs (and scale factors) per sub-block
     // a row's bytes of a step as 16-byte pieces: FULL whole ones from the start, and where the step's length is not
-    // a multiple of 16 one more that ends with the step (overlapping the last whole one).  The whole pieces of all
-    // rows come first in the lanes' order, then the rows' last pieces.
+    // a multiple of 16 one more that ends with the step (overlapping the last whole one).  Four lanes share a row:
+    // a load instruction takes 64 consecutive bytes of each of 16 rows, the next one the next 64, so that a lane's
+    // pieces sit at fixed distances from its first (one address register, one LDS offset register); only the last
+    // instruction of a row, where the pieces run out, has offsets of its own.
     constexpr uint32_t RS = S::ROW_STRIDE, SEG = 2 * S::BLOCK, FULL = SEG / 16, TAIL = SEG % 16 ? 1 : 0;
-    constexpr uint32_t NFULL = NT * 16 * FULL, PIECES = NFULL + TAIL * NT * 16, NL = (PIECES + 63) / 64;
+    constexpr uint32_t PPR = FULL + TAIL, ITR = (PPR + 3) / 4, NL = NT * ITR;
     constexpr uint32_t THREADS = 64 * WAVES, FS = SKINNY_FAC_STRIDE;
     constexpr uint32_t WAVE_LDS = skinny_wave_lds<F, NT>();
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -301,15 +385,26 @@ __device__ __forceinline__ void gemm_skinny_body(
     const uint8_t *We = W + (offsets ? (size_t)gy * w_stride : 0);
     const size_t row_bytes = (size_t)(k / 256) * S::BLOCK;
     // the lane's pieces of a step: where they come from (less the step's offset) and where they go
-    const uint8_t *src[NL];
-    uint32_t dst[NL];
+    const uint32_t lrow = lane >> 2, sub = lane & 3;
+    const uint8_t *src[NT];
+    uint32_t dst[NT];
 #pragma unroll
-    for (uint32_t i = 0; i < NL; i++) {
-        const uint32_t p = min(i * 64 + lane, PIECES - 1);
-        const uint32_t r = p < NFULL ? p / FULL : p - NFULL, at = p < NFULL ? (p % FULL) * 16 : SEG - 16;
-        src[i] = We + (size_t)min(rbase + r, n - 1) * row_bytes + at;
-        dst[i] = r * RS + at;
+    for (uint32_t j = 0; j < NT; j++) {
+        src[j] = We + (size_t)min(rbase + 16 * j + lrow, n - 1) * row_bytes + 16 * sub;
+        dst[j] = (16 * j + lrow) * RS + 16 * sub;
     }
+    // the row's last instruction: piece sub + 4 (ITR - 1), or the row's last piece where that is past it (loaded by
+    // several lanes then, and stored to the same place with the same value)
+    const uint32_t last_piece = min(sub + 4 * (ITR - 1), PPR - 1);
+    const uint32_t last_at = ((TAIL && last_piece == PPR - 1) ? SEG - 16 : 16 * last_piece) - 16 * sub;
+    auto load_step = [&](u32x4 (&stage)[NL], uint32_t st) {
+#pragma unroll
+        for (uint32_t j = 0; j < NT; j++) {
+            const uint8_t *sp = src[j] + (size_t)st * SEG;
+#pragma unroll
+            for (uint32_t i = 0; i < ITR; i++) stage[j * ITR + i] = ld16(sp + (i + 1 < ITR ? 64 * i : last_at));
+        }
+    };
     const uint32_t tiles_here = min((uint32_t)TT, (tok_end - tokb + 15) / 16);
     v4f32 acc[TT][NT];
 #pragma unroll
@@ -324,8 +419,7 @@ __device__ __forceinline__ void gemm_skinny_body(
                  : "=v"(magic[0]), "=v"(magic[1]), "=v"(magic[2]), "=v"(magic[3]));
     const uint64_t half_mask = q < 2 ? ~0ull : 0ull;
     u32x4 stage[NL];
-#pragma unroll
-    for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i] + (size_t)(sb_lo / 2) * SEG);
+    load_step(stage, sb_lo / 2);
     const uint32_t steps = n_super / 2;
     load_tokens(sb_lo, min(per, n_super - sb_lo) * 8);
     for (uint32_t sb0 = sb_lo; sb0 < n_super; sb0 += per) {
@@ -344,30 +438,31 @@ __device__ __forceinline__ void gemm_skinny_body(
     for (uint32_t st = sb0 / 2; st < (sb0 + nsbc) / 2; st++) {
         // the step's bytes to the strip (pieces past the end, on the last load: the last piece again, same value)
 #pragma unroll
-        for (uint32_t i = 0; i < NL; i++) {
-            if (TAIL && (i + 1) * 64 > NFULL)  // rows' last pieces among them: on dword boundaries only
-                reinterpret_cast<StripA4 *>(strip + dst[i])->v = stage[i];
-            else
-                *reinterpret_cast<u32x4 *>(strip + dst[i]) = stage[i];
-        }
-        if (st + 1 < steps) {
+        for (uint32_t j = 0; j < NT; j++)
 #pragma unroll
-            for (uint32_t i = 0; i < NL; i++) stage[i] = ld16(src[i] + (size_t)(st + 1) * SEG);
-        }
+            for (uint32_t i = 0; i < ITR; i++) {
+                if (i + 1 < ITR)
+                    *reinterpret_cast<u32x4 *>(strip + dst[j] + 64 * i) = stage[j * ITR + i];
+                else if (TAIL)  // the rows' last pieces among them: on dword boundaries only
+                    reinterpret_cast<StripA4 *>(strip + dst[j] + last_at)->v = stage[j * ITR + i];
+                else
+                    *reinterpret_cast<u32x4 *>(strip + dst[j] + last_at) = stage[j * ITR + i];
+            }
+        if (st + 1 < steps) load_step(stage, st + 1);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         // scale factors of the step, decoded once: lane (c, q) takes row c, super-block q / 2, sub-blocks
         // 4 (q % 2) .. + 3, for each tile (two factors per sub-block: per block, below)
-        if constexpr (KS == 1)
+        if constexpr (KS == 1 && S::TABLE)
 #pragma unroll
         for (int j = 0; j < NT; j++) {
             typename S::Raw hd;
-            S::read_hdr(hd, strip + (16 * j + c) * RS + (q >> 1) * S::BLOCK);
+            S::read_hdr(hd, strip + (16 * j + c) * RS + (q >> 1) * S::BLOCK, q & 1);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 float dsc, qneg;
-                S::factors(hd, 4 * (q & 1) + i, dsc, qneg);
+                S::factors(hd, q & 1, i, dsc, qneg);
                 dscT[(16 * j + c) * FS + 4 * q + i] = dsc;
                 if (S::HAS_MIN) minT[(16 * j + c) * FS + 4 * q + i] = qneg;
             }
@@ -427,7 +522,8 @@ __device__ __forceinline__ void gemm_skinny_body(
                     const long op = S::operand(raw[j], s);
 #pragma unroll
                     for (int is = 0; is < KS; is++) {
-                        dsc[j][is] = dscT[(16 * j + c) * FS + (KS == 2 ? 2 * s + is : u * 8 + s)];
+                        if constexpr (S::TABLE) dsc[j][is] = dscT[(16 * j + c) * FS + (KS == 2 ? 2 * s + is : u * 8 + s)];
+                        else dsc[j][is] = S::scale(raw[j], s);
                         corr[j][is] = -(MAGIC * dsc[j][is]);
                         // two factors: k-values 0..15 come from the lanes q = 0, 1, the others supply zeros; and so on
                         bop[j][is] = KS == 2 ? (long)((uint64_t)op & (is == 0 ? half_mask : ~half_mask)) : op;
@@ -652,8 +748,8 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
         // whole steps of two super-blocks
         if (a.k % 512 != 0 || rows > 32) return SK_NONE;
         const bool two = rows > 16;
-        // two factors per sub-block: the one-tile shapes only (see launch_skinny)
-        if (Skinny<F>::KSPLIT == 2 && (two || (variant != 0 && variant != 200))) return SK_NONE;
+        // the formats with the long strips: the one-tile shapes only (see launch_skinny)
+        if (Skinny<F>::ONE_TILE && (two || (variant != 0 && variant != 200))) return SK_NONE;
         if (a.sums && variant != 0 && variant != 200) return SK_NONE;  // the dump exists for the default shapes
         switch (variant) {
         case 0: {
@@ -692,9 +788,9 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
 // <NT, WAVES, TT, PER>; LDS = PER * 8 * TT * 640 + WAVES * NT * 7 KB
 template <class F>
 static hipError_t launch_skinny(const GemmArgs &a, const TilePlan &p, hipStream_t stream, int shape) {
-    if constexpr (Skinny<F>::OK && Skinny<F>::KSPLIT == 2) {
-        // Q6_K: 8 KB of LDS per wave; with chunks of two super-blocks of one token tile two work groups still share
-        // a compute unit (75 KB each)
+    if constexpr (Skinny<F>::OK && Skinny<F>::ONE_TILE) {
+        // Q6_K, Q8_0: 8 KB of LDS and more per wave; with chunks of two super-blocks of one token tile two work
+        // groups still share a compute unit (75 and 78 KB each)
         switch (shape) {
         case SK_1_4:
         case SK_1_8: return a.sums ? launch_skinny_shape<F, 1, 8, 1, 2, true>(a, p, stream) : launch_skinny_shape<F, 1, 8, 1, 2>(a, p, stream);

@@ -13,13 +13,25 @@ from test_gpu_parity import assert_close, canonical_ref, say
 
 pytestmark = pytest.mark.gpu
 
-FORMATS = [O.Q4_K, O.IQ4_XS]
-# Q6_K (a scale per 16 weights: two MFMAs per sub-block, the integer sums per half): the kernel's one-token-tile shapes
-FORMATS_1TILE = FORMATS + [O.Q6_K]
+FORMATS = [O.Q4_K, O.IQ4_XS, O.Q4_0]
+# Q6_K (a scale per 16 weights: two MFMAs per sub-block, the integer sums per half) and Q8_0 (544 bytes of a row per
+# step): the kernel's one-token-tile shapes only
+ONE_TILE = [O.Q6_K, O.Q8_0]
+FORMATS_1TILE = FORMATS + ONE_TILE
 
 
 def sum_groups(t, k_):
     return k_ // 16 if t == O.Q6_K else k_ // 32
+
+
+def ref_sums(ref, t, w, act_row, n, k_):
+    """The integer sums the kernel's dump holds: the reference's; for Q4_0 of the unsigned nibbles (sum q a = sum (q - 8) a
+    + 8 sum a: the "- 8" enters in fp32, as in the tile kernel)."""
+    s = ref.block_sums(t, w, act_row, n, k_)
+    if t == O.Q4_0:
+        a = act_row.reshape(k_ // 32, 34)[:, 2:].view(np.int8).astype(np.int32).sum(axis=1)
+        s = s + 8 * a[None, :]
+    return s
 
 
 def shaped_rows(counts, max_rows):
@@ -52,7 +64,7 @@ def _oracle_rows(ref, t, w, acts, offsets, n, k_, sample):
     for r in sample:
         e = int(np.searchsorted(offsets, r, side="right") - 1)
         y[r] = canonical_ref(ref, t, w[e], acts[r], n, k_, threads=16)
-        s[r] = ref.block_sums(t, w[e], acts[r], n, k_)
+        s[r] = ref_sums(ref, t, w[e], acts[r], n, k_)
     return y, s
 
 
@@ -95,7 +107,7 @@ CASES = [
 def test_skinny_grouped_against_oracle(hip, ref, t, case):
     counts, n, k_, max_rows = case
     say("skinny", O.NAMES[t], case)
-    if t == O.Q6_K and shaped_rows(counts, max_rows) > 16:
+    if t in ONE_TILE and shaped_rows(counts, max_rows) > 16:
         pytest.skip("two token tiles: the tile kernel's case for this format")
     offsets, acts, w = _case(ref, t, counts, n, k_, 4100 + n + k_)
     rows = int(offsets[-1])
@@ -144,7 +156,7 @@ def test_skinny_shapes_give_the_same_bits(hip, ref, tuning, t):
 def test_skinny_plain_matmul_forced(hip, ref, tuning, t, m):
     """One matrix, no experts (the default there is the tile kernel; the kernel is selectable), ragged n."""
     import torch
-    if t == O.Q6_K and m > 16:
+    if t in ONE_TILE and m > 16:
         pytest.skip("two token tiles: the tile kernel's case for this format")
     n, k_ = 1000, 2048
     w = synth.weights(t, 31, n, k_)
@@ -152,7 +164,7 @@ def test_skinny_plain_matmul_forced(hip, ref, tuning, t, m):
     acts = ref.quantize_q8_0(x).reshape(m, k_ // 32 * 34)
     kern = hip.HipKernel(t)
     tuning("gemm_tile_min_rows", 1)
-    tuning("gemm_variant", 200 if t == O.Q6_K else 204)
+    tuning("gemm_variant", 200 if t in ONE_TILE else 204)
     ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
     dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
     kern.gemm_q8_dev(torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda(), dy, m, n, k_, workspace=ws)
@@ -206,7 +218,7 @@ def test_skinny_one_matrix_split_k(hip, ref, t, shape):
     y_ref = {r: canonical_ref(ref, t, w, acts[r], n, k_, threads=16) for r in rows}
     for r in rows:
         assert_close(y[r], y_ref[r], f"split-k {shape} row {r}")
-        assert np.array_equal(s[r], ref.block_sums(t, w, acts[r], n, k_)), f"integer sums of row {r}"
+        assert np.array_equal(s[r], ref_sums(ref, t, w, acts[r], n, k_)), f"integer sums of row {r}"
     # production launch: the same bits; accumulate: twice them; bias in the reduction
     dy2 = torch.zeros((m, n), dtype=torch.float32, device="cuda")
     kern.gemm_q8_dev(dw, da, dy2, m, n, k_, workspace=ws)
