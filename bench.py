@@ -284,6 +284,9 @@ def main():
                     help="launch a 256 MiB copy kernel 3 times, then gate+up (one launch) over 8 distinct layers, "
                          "lm_head twice and the prefill matmul twice, and exit: the workload of the rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE runs (the copy kernel scales the counters)")
+    ap.add_argument("--mfma-valu-probe", action="store_true",
+                    help="time a kernel of f16 MFMAs and fp32 fmas on register operands in several proportions, one "
+                         "work group of 8 waves per compute unit, and exit: how much vector work the matrix work hides")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives or sharding here)",
@@ -303,6 +306,30 @@ def main():
     L = max(1, args.layers)
 
     k_q8, k_q4k, k_q6k = quant.HipKernel(Q8_0), quant.HipKernel(Q4_K), quant.HipKernel(Q6_K)
+
+    if args.mfma_valu_probe:
+        import ctypes as C
+        kit = C.CDLL(os.path.join(ROOT, "oxillama_amd", "liboxq_benchkit.so"))
+        kit.oxq_benchkit_mfma_valu.argtypes = [C.c_void_p, C.c_uint, C.c_int, C.c_int, C.c_int, C.c_void_p]
+        iters = 4000
+        rows = []
+        for blocks in (info["compute_units"], 8):  # the whole chip busy, and 8 compute units of it
+            buf = torch.zeros(max(blocks, 2) * 512, dtype=torch.float32, device=dev)
+            for n_mfma, n_fma in ((0, 16), (0, 32), (2, 0), (2, 8), (2, 16), (2, 32)):
+                best = 1e9
+                for _ in range(3):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    st = kit.oxq_benchkit_mfma_valu(buf.data_ptr(), blocks, iters, n_mfma, n_fma, None)
+                    e1.record()
+                    e1.synchronize()
+                    assert st == 0, st
+                    best = min(best, e0.elapsed_time(e1))
+                # a SIMD runs two waves of the work group: 2 * iters trips
+                rows.append({"work_groups": blocks, "mfma_32x32x16_f16_per_trip": n_mfma, "fma_f32_per_trip": n_fma,
+                             "ns_per_trip_per_simd": round(best * 1e6 / (2 * iters), 1)})
+        print(json.dumps({"probe": "mfma_valu", "waves_per_simd": 2, "trips": iters, "rows": rows}))
+        return
 
     if args.traffic_probe:
         import ctypes as C

@@ -1,8 +1,10 @@
 // Measurement helpers (not part of the quantized-matmul ABI): a plain copy kernel of
 // known size, used to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters, a
 // streaming read kernel that marks the practical HBM read ceiling for a given
-// footprint and launch shape, and a kernel of nothing but int8 MFMAs on register
-// operands, which marks what the matrix cores deliver when nothing else is in the way.
+// footprint and launch shape, a kernel of nothing but int8 MFMAs on register
+// operands, which marks what the matrix cores deliver when nothing else is in the way,
+// and a kernel of f16 MFMAs and fp32 fmas in chosen proportion, which shows how much of
+// the vector work the matrix work hides.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -54,7 +56,59 @@ __global__ __launch_bounds__(256) void benchkit_mfma_i8_kernel(int *__restrict__
     out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
 }
 
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// How matrix and vector instructions share a SIMD's time: per trip NM v_mfma_f32_32x32x16_f16 on independent
+// accumulators and NV fp32 fmas on registers the MFMAs do not touch, all operands in registers.  512 threads: two
+// waves per SIMD when one work group sits on a compute unit.
+template <int NM, int NV>
+__global__ __launch_bounds__(512) void benchkit_mfma_valu_kernel(float *__restrict__ out, int iters) {
+    const int lane = threadIdx.x;
+    h8 a, b;
+    for (int i = 0; i < 8; i++) a[i] = (_Float16)(lane + i), b[i] = (_Float16)(lane * 3 + i);
+    v16f acc[2];
+    for (int c = 0; c < 2; c++)
+        for (int i = 0; i < 16; i++) acc[c][i] = 0.0f;
+    float v[32];
+    for (int i = 0; i < 32; i++) v[i] = out[lane + i];
+    const float da = out[lane + 77];
+    for (int it = 0; it < iters; it++) {
+        if (NM > 0) {
+#pragma unroll
+            for (int c = 0; c < NM; c++) {
+                acc[c & 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[c & 1], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < NV / (NM ? NM : 1); i++) v[(c * 16 + i) & 31] = fmaf(v[(c * 16 + i) & 31], da, 1.0f);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NV; i++) v[i & 31] = fmaf(v[i & 31], da, 1.0f);
+        }
+    }
+    float r = 0.0f;
+    for (int c = 0; c < 2; c++)
+        for (int i = 0; i < 16; i++) r += acc[c][i];
+    for (int i = 0; i < 32; i++) r += v[i];
+    out[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = r;
+}
+
 extern "C" {
+
+// blocks x 8 waves x iters trips of n_mfma (0 or 2) MFMAs and n_fma (0, 8, 16, 32) fmas; out: blocks * 512 floats, the
+// first 512 read as inputs.  Returns hipErrorInvalidValue for a combination that is not instantiated.
+int oxq_benchkit_mfma_valu(void *out, unsigned blocks, int iters, int n_mfma, int n_fma, void *stream) {
+    hipStream_t st = (hipStream_t)stream;
+    float *o = (float *)out;
+#define OXQ_MV(NM, NV)                                                                                      \
+    if (n_mfma == NM && n_fma == NV) {                                                                      \
+        hipLaunchKernelGGL((benchkit_mfma_valu_kernel<NM, NV>), dim3(blocks), dim3(512), 0, st, o, iters);  \
+        return (int)hipGetLastError();                                                                      \
+    }
+    OXQ_MV(0, 16) OXQ_MV(0, 32) OXQ_MV(2, 0) OXQ_MV(2, 8) OXQ_MV(2, 16) OXQ_MV(2, 32)
+#undef OXQ_MV
+    return (int)hipErrorInvalidValue;
+}
 
 // blocks x 4 waves x iters x 4 MFMAs of 2 * 32 * 32 * 32 int8 operations; out: blocks * 256 ints.
 int oxq_benchkit_mfma_i8(void *out, unsigned blocks, int iters, void *stream) {
