@@ -284,6 +284,10 @@ def main():
                     help="launch a 256 MiB copy kernel 3 times, then gate+up (one launch) over 8 distinct layers, "
                          "lm_head twice and the prefill matmul twice, and exit: the workload of the rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE runs (the copy kernel scales the counters)")
+    ap.add_argument("--prefetch-probe", action="store_true",
+                    help="the timed decode steps again with a small kernel on a second stream that, while a GEMV launch "
+                         "runs, touches the first MB of the NEXT launch's weights (one dword per 128-byte line); prints "
+                         "ms per step for several prefetch sizes and exits")
     ap.add_argument("--mfma-valu-probe", action="store_true",
                     help="time a kernel of f16 MFMAs and fp32 fmas on register operands in several proportions, one "
                          "work group of 8 waves per compute unit, and exit: how much vector work the matrix work hides")
@@ -452,6 +456,48 @@ def main():
             e1.record(stream)
             e1.synchronize()
         return e0.elapsed_time(e1)  # ms
+
+    if args.prefetch_probe:
+        import ctypes as C
+        kit = C.CDLL(os.path.join(ROOT, "oxillama_amd", "liboxq_benchkit.so"))
+        kit.oxq_benchkit_touch.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint, C.c_void_p]
+        side = torch.cuda.Stream()
+        sink = torch.zeros(4096, dtype=torch.int32, device=dev)
+        quant.quantize_q8_0_dev(x, xq)
+        quant.quantize_q8_0_dev(h, hq)
+        torch.cuda.synchronize()
+
+        def launches_of(i):
+            """The three weight-streaming launches of step i: (weights the launch reads, the call)."""
+            w = layers[i % L]
+            return [([w["q"]], lambda: k_q8.matvec_q8_fused_dev(w["q"], xq, yq, H, H, accumulate=False)),
+                    ([w["gate"], w["up"]], lambda: linear.gate_up_swiglu_dev(Q4_K, w["gate"], w["up"], xq, None, hq, F, H)),
+                    ([w["down"]], lambda: k_q6k.matvec_q8_fused_dev(w["down"], hq, yd, H, F, accumulate=False))]
+
+        def steps_with_prefetch(n_steps, mb, blocks):
+            seq = [l for i in range(n_steps) for l in launches_of(i)]
+            for j, (_, call) in enumerate(seq):
+                if mb and j + 1 < len(seq):
+                    # while launch j runs: the head of launch j + 1's weights, on the second stream
+                    side.wait_stream(stream)
+                    nxt = seq[j + 1][0]
+                    for t in nxt:
+                        nb = min(t.numel(), (mb << 20) // len(nxt)) // 128 * 128
+                        kit.oxq_benchkit_touch(t.data_ptr(), sink.data_ptr(), nb, blocks, side.cuda_stream)
+                call()
+            stream.wait_stream(side)
+
+        rows = []
+        for mb, blocks in ((0, 0), (2, 16), (4, 16), (8, 32), (16, 32), (16, 64), (32, 64)):
+            g = capture(lambda: steps_with_prefetch(args.steps, mb, blocks))
+            timed_replay(g)
+            ms = sorted(timed_replay(g) for _ in range(5))[2] / args.steps
+            rows.append({"prefetch_MB_per_launch": mb, "touch_work_groups": blocks, "ms_per_step": round(ms, 5)})
+            print(json.dumps(rows[-1]), file=sys.stderr, flush=True)
+        print(json.dumps({"probe": "prefetch", "steps": args.steps, "launches_per_step": 3,
+                          "note": "activations pre-quantized (no quantize launch): compare the rows with each other, "
+                                  "not with the default run", "rows": rows}))
+        return
 
     # ---- the timed region: W warm-up steps, then exactly K steps ----------------------
     K, W = args.steps, args.warmup

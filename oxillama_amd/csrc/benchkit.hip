@@ -36,6 +36,16 @@ __global__ __launch_bounds__(256) void benchkit_read_kernel(const u32x4 *__restr
     if (r == 0x9E3779B9u) out[blockIdx.x] = r;  // practically never: keeps the loads alive
 }
 
+// One dword of every 128-byte line of a buffer: pulls the lines through the memory-side cache at the least cost to
+// the texture units (a wave instruction covers 8 KB).
+__global__ __launch_bounds__(256) void benchkit_touch_kernel(const uint32_t *__restrict__ src, uint32_t *__restrict__ out,
+                                                            size_t n_lines) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    uint32_t acc = 0;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_lines; i += stride) acc ^= src[i * 32];
+    if (acc == 0x9E3779B9u) out[blockIdx.x] = acc;  // practically never: keeps the loads alive
+}
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
@@ -113,6 +123,12 @@ int oxq_benchkit_mfma_valu(void *out, unsigned blocks, int iters, int n_mfma, in
 // blocks x 4 waves x iters x 4 MFMAs of 2 * 32 * 32 * 32 int8 operations; out: blocks * 256 ints.
 int oxq_benchkit_mfma_i8(void *out, unsigned blocks, int iters, void *stream) {
     hipLaunchKernelGGL(benchkit_mfma_i8_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (int *)out, iters);
+    return (int)hipGetLastError();
+}
+
+int oxq_benchkit_touch(const void *src, void *out, size_t bytes, unsigned blocks, void *stream) {
+    hipLaunchKernelGGL(benchkit_touch_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const uint32_t *)src,
+                       (uint32_t *)out, bytes / 128);
     return (int)hipGetLastError();
 }
 
