@@ -284,8 +284,10 @@ int oxq_gemm_q8_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_ac
  * oxq_gemm_q8_static_max_workspace_bytes()); the call allocates nothing, synchronises nothing and
  * gives the bits of oxq_gemm_q8_dev.  Shapes whose oxq_gemm_q8_workspace_bytes exceeds the
  * array return OXQ_ERR_BUFFER_TOO_SMALL (needed, available); oxq_init must have run (the call
- * does not initialise lazily: OXQ_ERR_NO_DEVICE).  All calls on one GPU share the array: calls
- * that overlap in time on one GPU (different streams or threads) race on it. */
+ * does not initialise lazily: OXQ_ERR_NO_DEVICE) for the device the calling thread has current,
+ * whose copy of the array the call uses.  All calls on one GPU share the array: issue them on
+ * ONE stream per GPU (or order the streams with events yourself) -- calls that overlap in time
+ * on one GPU race on it, and nothing in the library detects that. */
 size_t oxq_gemm_q8_static_max_workspace_bytes(void);
 int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                            float *d_out, size_t m, size_t n, size_t k, int accumulate,

@@ -946,9 +946,13 @@ int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_
     if (st != OXQ_OK) return st;
     if (m > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, m, "dimension exceeds 2^32-1");
     // no lazy initialisation here: that would be the one path of this call that allocates
-    if (!g.initialised.load(std::memory_order_acquire) || g.device < 0 || g.device >= MAX_DEVICES ||
-        !static_scratch_ptr[g.device])
-        return fail(OXQ_ERR_NO_DEVICE, 0, 0, "call oxq_init first: this entry point sets nothing up by itself");
+    // the array of the device the calling thread has current (where the stream's work runs), not of the last one
+    // oxq_init was called for: each device holds its own copy
+    int device = -1;
+    if (!g.initialised.load(std::memory_order_acquire) || hipGetDevice(&device) != hipSuccess || device < 0 ||
+        device >= MAX_DEVICES || !static_scratch_ptr[device])
+        return fail(OXQ_ERR_NO_DEVICE, 0, 0,
+                    "call oxq_init for this device first: this entry point sets nothing up by itself");
     if (m == 0 || n == 0 || k == 0) return OXQ_OK;
     const bool tiles = oxq::gemm_uses_tiles(type, (uint32_t)m, (uint32_t)n, (uint32_t)k) ||
                        (oxq::gemm_few_rows_pay(type, (uint32_t)m, (uint32_t)n, (uint32_t)k) &&
@@ -963,7 +967,7 @@ int oxq_gemm_q8_static_dev(uint32_t type, const uint8_t *d_weights, const uint8_
     ga.out = d_out;
     ga.sums = nullptr;
     ga.workspace_bytes = tiles ? STATIC_SCRATCH_BYTES : 0;
-    ga.workspace = tiles ? static_scratch_ptr[g.device] : nullptr;  // every byte the tile kernel reads is written
+    ga.workspace = tiles ? static_scratch_ptr[device] : nullptr;    // every byte the tile kernel reads is written
     ga.by_rows = !tiles;                                            // by the preparation kernel of this same call
     ga.m = (uint32_t)m;
     ga.n = (uint32_t)n;

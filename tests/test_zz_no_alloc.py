@@ -26,10 +26,15 @@ def _case(hip, ref, t, m, n, k_, seed):
     torch.cuda.synchronize()
     for acc in (False, True):
         kern.gemm_q8_dev(dw, da, want, m, n, k_, accumulate=acc, workspace=ws)
-        before = torch.cuda.memory_stats()["allocation.all.allocated"]
-        kern.gemm_q8_static_dev(dw, da, got, m, n, k_, accumulate=acc)
-        assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
         torch.cuda.synchronize()
+        # neither torch's allocator nor the device's own (free bytes as the driver reports them: a hipMalloc inside
+        # the library would lower them) moves across the call
+        before = torch.cuda.memory_stats()["allocation.all.allocated"]
+        free_before = torch.cuda.mem_get_info()[0]
+        kern.gemm_q8_static_dev(dw, da, got, m, n, k_, accumulate=acc)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
         assert torch.equal(got, want), (O.NAMES[t], m, n, k_, acc)
     # and against the oracle, so that "equal" cannot mean "equally wrong"
     arb = k_ // 32 * 34
@@ -52,6 +57,35 @@ def test_static_scratch_matmul_equals_workspace_matmul_twice_in_a_row(hip, ref):
                               (O.Q4_K, 12, 4096, 8192, 43), (O.IQ4_XS, 16, 200, 1024, 45)):
         say(O.NAMES[t], m, n, k_)
         _case(hip, ref, t, m, n, k_, seed)
+
+
+def test_static_scratch_matmul_under_stream_capture(hip, ref):
+    """Recorded into a HIP graph (where an allocation or a synchronisation inside the call would end the capture with an
+    error) and replayed three times with eager work between the replays: every replay gives the eager call's bits."""
+    import torch
+    t, m, n, k_ = O.Q4_K, 24, 512, 1024
+    w = synth.weights(t, 51, n, k_)
+    acts = ref.quantize_q8_0(synth.normal_f32(52, m * k_))
+    kern = hip.HipKernel(t)
+    dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
+    want = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    got = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    other = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+    kern.gemm_q8_static_dev(dw, da, want, m, n, k_)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(g, stream=stream):
+            kern.gemm_q8_static_dev(dw, da, got, m, n, k_)
+        for i in range(3):
+            got.zero_()
+            # eager work on the same array between the replays: another shape's bytes lie in it when the graph runs
+            kern.gemm_q8_static_dev(dw, da[:8 * (k_ // 32 * 34)], other[:8], 8, n, k_)
+            stream.synchronize()
+            g.replay()
+            stream.synchronize()
+            assert torch.equal(got, want), i
 
 
 def test_static_scratch_limits(hip, ref):
