@@ -522,6 +522,24 @@ size_t oxq_topk_workspace_bytes(size_t n, size_t k);
 int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
                  uint32_t *d_out_indices, void *d_workspace, size_t workspace_bytes, void *stream);
 
+/* The rest of the sampler on those candidates (sample_with_rng from its greedy shortcut on,
+ * crates/oxillama-runtime/src/sampling/mod.rs:487-564): temperature <= 0 or k == 1 returns the
+ * first candidate; otherwise every value times 1/temperature, softmax over the k candidates
+ * (mod.rs:617-638), min-p (keep p >= min_p * p[0]; 0 = off), top-p (cut after the cumulative sum
+ * reaches top_p; 1 = off), renormalisation, and the draw against one value of the reference's
+ * Xorshift64 (mod.rs:669-690), whose state *d_rng_state holds and which advances only when more
+ * than one candidate survives, as in the reference.  d_values / d_indices: k candidates, largest
+ * value first (oxq_topk_dev's output; the values are the logits after whatever bias, penalty or
+ * mask the caller applies -- those steps of the reference are not here).  *d_token receives the
+ * token id; d_probs (optional, k floats) the final probabilities, zeros past the survivors.
+ * 1 <= k <= 256.  Every fp32 operation is the reference's, in its order, so token and generator
+ * state are the reference's for the same candidates (equal logits: see oxq_topk_dev).  One
+ * launch, no allocation, no synchronisation.  Seed the state as Xorshift64::new does: the seed,
+ * or 0x517cc1b727220a95 for a zero seed. */
+int oxq_sample_candidates_dev(const float *d_values, const uint32_t *d_indices, size_t k,
+                              float temperature, float min_p, float top_p, uint64_t *d_rng_state,
+                              uint32_t *d_token, float *d_probs, void *stream);
+
 int oxq_block_sums_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8,
                        int32_t *d_sums, size_t n_rows, size_t n_cols, void *stream);
 

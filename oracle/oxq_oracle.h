@@ -152,6 +152,18 @@ oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w,
  * crates/oxillama-runtime/src/sampling/mod.rs:500-509,652-662 */
 uint32_t oxq_ref_argmax(const float *values, size_t n);
 void oxq_ref_topk(const float *values, size_t n, size_t k, float *out_vals, uint32_t *out_idx);
+/* Xorshift64::new / next_u64 / next_f32, sampling/mod.rs:669-690: the sampler's generator.  *state is
+ * advanced; a zero seed is replaced as new() does. */
+uint64_t oxq_ref_xorshift64_seed(uint64_t seed);
+float oxq_ref_xorshift64_next_f32(uint64_t *state);
+/* The tail of sample_with_rng, sampling/mod.rs:487-564, on the k candidates that steps 5 and 6 (sort, truncate to
+ * top_k) leave, largest logit first: greedy shortcut (temperature <= 0 or k == 1), temperature scaling, softmax
+ * over the candidates, min-p, top-p, renormalisation, and the draw against one rng.next_f32() -- which is taken
+ * only when more than one candidate is left, as in the reference.  probs_out (optional, k floats) receives the
+ * final probabilities, zeros past the survivors; n_left_out (optional) their count.  Returns the token id. */
+uint32_t oxq_ref_sample_candidates(const float *vals, const uint32_t *idx, size_t k, float temperature,
+                                   float min_p, float top_p, uint64_t *rng_state, float *probs_out,
+                                   size_t *n_left_out);
 
 /* ---- mixture-of-experts feed-forward (oxq_oracle_moe.c), crates/oxillama-arch/src/common/moe.rs ---- */
 

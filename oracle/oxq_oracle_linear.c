@@ -194,3 +194,135 @@ void oxq_ref_topk(const float *values, size_t n, size_t k, float *out_vals, uint
     }
     free(taken);
 }
+
+/* Xorshift64, sampling/mod.rs:669-690 */
+uint64_t oxq_ref_xorshift64_seed(uint64_t seed) { return seed == 0 ? 0x517cc1b727220a95ull : seed; }
+
+float oxq_ref_xorshift64_next_f32(uint64_t *state) {
+    uint64_t x = *state;
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    *state = x;
+    return (float)(x >> 40) / (float)(1ull << 24); /* mod.rs:687-689 */
+}
+
+/* sample_with_rng from step 3 on, sampling/mod.rs:487-564; softmax_candidates, mod.rs:617-638.  The candidate
+ * values are the logits after steps 0-2 (bias, penalties, grammar), which leave this restatement's scope. */
+uint32_t oxq_ref_sample_candidates(const float *vals, const uint32_t *idx, size_t k, float temperature,
+                                   float min_p, float top_p, uint64_t *rng_state, float *probs_out,
+                                   size_t *n_left_out) {
+    if (probs_out) {
+        for (size_t i = 0; i < k; i++) {
+            probs_out[i] = 0.0f;
+        }
+    }
+    if (n_left_out) {
+        *n_left_out = k ? 1 : 0;
+    }
+    if (k == 0) {
+        return 0;
+    }
+    /* step 3: greedy shortcut; the first candidate is argmax (largest value, lowest index) */
+    if (temperature <= 0.0f || k == 1) {
+        if (probs_out) {
+            probs_out[0] = 1.0f;
+        }
+        return idx[0];
+    }
+    float *p = (float *)malloc(k * sizeof(float));
+    uint32_t *ids = (uint32_t *)malloc(k * sizeof(uint32_t));
+    memcpy(ids, idx, k * sizeof(uint32_t));
+    /* step 4: every logit times 1 / temperature (the order of the candidates does not change) */
+    if (temperature != 1.0f) {
+        const float inv_temp = 1.0f / temperature;
+        for (size_t i = 0; i < k; i++) {
+            p[i] = vals[i] * inv_temp;
+        }
+    } else {
+        for (size_t i = 0; i < k; i++) {
+            p[i] = vals[i];
+        }
+    }
+    /* step 7: softmax_candidates */
+    float max_logit = -INFINITY;
+    for (size_t i = 0; i < k; i++) {
+        max_logit = fmaxf(max_logit, p[i]); /* f32::max: a NaN operand is ignored */
+    }
+    float sum = 0.0f;
+    for (size_t i = 0; i < k; i++) {
+        p[i] = expf(p[i] - max_logit);
+        sum += p[i];
+    }
+    if (sum > 0.0f) {
+        for (size_t i = 0; i < k; i++) {
+            p[i] /= sum;
+        }
+    }
+    size_t n = k;
+    /* step 8: min-p, retain p >= min_p * p[0] (order kept) */
+    if (min_p > 0.0f && n > 0) {
+        const float threshold = min_p * p[0];
+        size_t w = 0;
+        for (size_t i = 0; i < n; i++) {
+            if (p[i] >= threshold) {
+                p[w] = p[i];
+                ids[w] = ids[i];
+                w++;
+            }
+        }
+        n = w;
+    }
+    /* step 9: top-p */
+    if (top_p < 1.0f && n > 0) {
+        float cumulative = 0.0f;
+        size_t cutoff = n;
+        for (size_t i = 0; i < n; i++) {
+            cumulative += p[i];
+            if (cumulative >= top_p) {
+                cutoff = i + 1;
+                break;
+            }
+        }
+        n = cutoff;
+    }
+    /* step 10: renormalise */
+    float total = 0.0f;
+    for (size_t i = 0; i < n; i++) {
+        total += p[i];
+    }
+    if (total > 0.0f && total != 1.0f) {
+        for (size_t i = 0; i < n; i++) {
+            p[i] /= total;
+        }
+    }
+    if (probs_out) {
+        for (size_t i = 0; i < n; i++) {
+            probs_out[i] = p[i];
+        }
+    }
+    if (n_left_out) {
+        *n_left_out = n;
+    }
+    /* step 11: the draw */
+    uint32_t token;
+    if (n == 0) {
+        token = idx[0]; /* argmax of the processed logits */
+    } else if (n == 1) {
+        token = ids[0];
+    } else {
+        const float r = oxq_ref_xorshift64_next_f32(rng_state);
+        float cumulative = 0.0f;
+        token = ids[n - 1]; /* fallback: the last candidate */
+        for (size_t i = 0; i < n; i++) {
+            cumulative += p[i];
+            if (r < cumulative) {
+                token = ids[i];
+                break;
+            }
+        }
+    }
+    free(p);
+    free(ids);
+    return token;
+}

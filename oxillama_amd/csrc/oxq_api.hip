@@ -1598,6 +1598,17 @@ int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
     return OXQ_OK;
 }
 
+int oxq_sample_candidates_dev(const float *d_values, const uint32_t *d_indices, size_t k, float temperature, float min_p,
+                              float top_p, uint64_t *d_rng_state, uint32_t *d_token, float *d_probs, void *stream) {
+    if (k == 0 || k > 256) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, k, "between 1 and 256 candidates");
+    if (!d_values || !d_indices || !d_rng_state || !d_token) return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_sample_candidates(d_values, d_indices, (uint32_t)k, temperature, min_p, top_p, d_rng_state,
+                                          d_token, d_probs, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
 // QuantLinear::forward on host slices (drop-in route: everything is staged per call).
 int oxq_linear_forward(uint32_t type, const uint8_t *data, size_t data_len, const size_t *shape, size_t n_dims,
                        const float *bias, size_t bias_len, const float *lora_a, size_t lora_a_len, const float *lora_b,

@@ -686,7 +686,6 @@ constexpr uint32_t SKINNY_GROUPED_SPLITS = 2, SKINNY_GROUPED_SPLIT_MAX_N = 8192;
 
 template <class F, int NT, int WAVES, int TT, int PER, bool DUMP = false>
 static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipStream_t stream, bool split_k = false) {
-    using S = Skinny<F>;
     const size_t strips = (size_t)WAVES * skinny_wave_lds<F, NT>();
     auto kern = &gemm_skinny_kernel<F, NT, WAVES, TT, PER, DUMP>;
     const size_t lds = (size_t)PER * 8 * TT * skinny_act_bytes<F>() + strips;

@@ -413,4 +413,121 @@ hipError_t launch_topk(const float *x, uint32_t n, uint32_t k, float *out_vals, 
     return hipGetLastError();
 }
 
+// The sampler from its candidate list on: sample_with_rng's steps 3 to 11 (crates/oxillama-runtime/src/sampling/
+// mod.rs:487-564; softmax_candidates :617-638; Xorshift64 :669-690) on the k <= 256 candidates that the top-k above
+// leaves, largest logit first -- so that a token id, not a candidate list, leaves the device.  One work group.  What
+// the reference does element by element is done by all threads (the scaling, the exponentials, the divisions), what
+// it does as a running sum in candidate order (softmax sum, top-p, renormalisation, the draw) by thread 0 in that
+// order, so that every fp32 value is the reference's: exp is the C library's (expf_libm), the divisions are
+// correctly rounded.  rng_state is advanced only when more than one candidate survives, as in the reference.
+__global__ __launch_bounds__(256) void sample_candidates_kernel(const float *__restrict__ vals, const uint32_t *__restrict__ idx,
+                                                                uint32_t k, float temperature, float min_p, float top_p,
+                                                                uint64_t *__restrict__ rng_state, uint32_t *__restrict__ token_out,
+                                                                float *__restrict__ probs_out) {
+    __shared__ float p[256];
+    __shared__ uint32_t ids[256];
+    __shared__ float s_val;
+    __shared__ uint32_t s_n;
+    const uint32_t t = threadIdx.x;
+    if (temperature <= 0.0f || k == 1) {  // step 3: greedy; the first candidate is the argmax
+        if (t == 0) *token_out = idx[0];
+        if (probs_out && t < k) probs_out[t] = t == 0 ? 1.0f : 0.0f;
+        return;
+    }
+    if (t < k) {
+        float v = vals[t];
+        if (temperature != 1.0f) v = v * (1.0f / temperature);  // step 4
+        p[t] = v;
+        ids[t] = idx[t];
+    }
+    __syncthreads();
+    if (t == 0) {  // step 7: the maximum (f32::max: a NaN operand is ignored)
+        float m = -INFINITY;
+        for (uint32_t i = 0; i < k; i++) m = fmaxf(m, p[i]);
+        s_val = m;
+    }
+    __syncthreads();
+    const float max_logit = s_val;
+    if (t < k) p[t] = expf_libm(p[t] - max_logit);
+    __syncthreads();
+    if (t == 0) {
+        float sum = 0.0f;
+        for (uint32_t i = 0; i < k; i++) sum += p[i];
+        s_val = sum;
+    }
+    __syncthreads();
+    const float sum = s_val;
+    if (t < k && sum > 0.0f) p[t] = p[t] / sum;
+    __syncthreads();
+    if (t == 0) {
+        uint32_t n = k;
+        if (min_p > 0.0f) {  // step 8
+            const float threshold = min_p * p[0];
+            uint32_t w = 0;
+            for (uint32_t i = 0; i < n; i++)
+                if (p[i] >= threshold) {
+                    p[w] = p[i];
+                    ids[w] = ids[i];
+                    w++;
+                }
+            n = w;
+        }
+        if (top_p < 1.0f && n > 0) {  // step 9
+            float cumulative = 0.0f;
+            uint32_t cutoff = n;
+            for (uint32_t i = 0; i < n; i++) {
+                cumulative += p[i];
+                if (cumulative >= top_p) {
+                    cutoff = i + 1;
+                    break;
+                }
+            }
+            n = cutoff;
+        }
+        float total = 0.0f;  // step 10
+        for (uint32_t i = 0; i < n; i++) total += p[i];
+        s_val = total;
+        s_n = n;
+    }
+    __syncthreads();
+    const uint32_t n = s_n;
+    const float total = s_val;
+    if (t < n && total > 0.0f && total != 1.0f) p[t] = p[t] / total;
+    __syncthreads();
+    if (probs_out && t < k) probs_out[t] = t < n ? p[t] : 0.0f;
+    if (t == 0) {  // step 11
+        uint32_t token;
+        if (n == 0) {
+            token = idx[0];
+        } else if (n == 1) {
+            token = ids[0];
+        } else {
+            uint64_t x = *rng_state;
+            x ^= x << 13;
+            x ^= x >> 7;
+            x ^= x << 17;
+            *rng_state = x;
+            const float r = (float)(x >> 40) / 16777216.0f;
+            float cumulative = 0.0f;
+            token = ids[n - 1];
+            for (uint32_t i = 0; i < n; i++) {
+                cumulative += p[i];
+                if (r < cumulative) {
+                    token = ids[i];
+                    break;
+                }
+            }
+        }
+        *token_out = token;
+    }
+}
+
+hipError_t launch_sample_candidates(const float *vals, const uint32_t *idx, uint32_t k, float temperature, float min_p,
+                                    float top_p, uint64_t *rng_state, uint32_t *token_out, float *probs_out,
+                                    hipStream_t stream) {
+    hipLaunchKernelGGL(sample_candidates_kernel, dim3(1), dim3(256), 0, stream, vals, idx, k, temperature, min_p, top_p,
+                       rng_state, token_out, probs_out);
+    return hipGetLastError();
+}
+
 }  // namespace oxq

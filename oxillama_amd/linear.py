@@ -157,5 +157,14 @@ def topk_dev(d_values, k, d_out_values, d_out_indices, workspace):
                             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream()))
 
 
+def sample_candidates_dev(d_values, d_indices, k, temperature, min_p, top_p, d_rng_state, d_token, d_probs=None):
+    """The sampler after its candidate list (sampling/mod.rs:487-564): temperature, softmax, min-p, top-p, the draw.
+    d_rng_state: one uint64 (the reference's Xorshift64 state), d_token: one uint32, d_probs: optional k floats."""
+    lib = capi.load()
+    _check(lib.oxq_sample_candidates_dev(d_values.data_ptr(), d_indices.data_ptr(), k, temperature, min_p, top_p,
+                                         d_rng_state.data_ptr(), d_token.data_ptr(),
+                                         d_probs.data_ptr() if d_probs is not None else None, _stream()))
+
+
 def topk_workspace_bytes(n, k):
     return capi.load().oxq_topk_workspace_bytes(n, k)

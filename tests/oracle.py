@@ -134,6 +134,12 @@ def load():
     lib.oxq_ref_argmax.argtypes = [vp, sz]
     lib.oxq_ref_topk.restype = None
     lib.oxq_ref_topk.argtypes = [vp, sz, sz, vp, vp]
+    lib.oxq_ref_xorshift64_seed.restype = C.c_uint64
+    lib.oxq_ref_xorshift64_seed.argtypes = [C.c_uint64]
+    lib.oxq_ref_xorshift64_next_f32.restype = C.c_float
+    lib.oxq_ref_xorshift64_next_f32.argtypes = [vp]
+    lib.oxq_ref_sample_candidates.restype = C.c_uint32
+    lib.oxq_ref_sample_candidates.argtypes = [vp, vp, sz, C.c_float, C.c_float, C.c_float, vp, vp, vp]
     lib.oxq_ref_rmsnorm_forward_to.restype = None
     lib.oxq_ref_rmsnorm_forward_to.argtypes = [vp, vp, C.c_float, sz, vp]
     _lib = lib
@@ -419,6 +425,28 @@ def topk(values, k):
     vals, idx = np.zeros(k, dtype=np.float32), np.zeros(k, dtype=np.uint32)
     load().oxq_ref_topk(_p(v), v.size, k, _p(vals), _p(idx))
     return vals, idx
+
+
+def xorshift64_seed(seed):
+    return int(load().oxq_ref_xorshift64_seed(seed))
+
+
+def xorshift64_next_f32(state):
+    """(value in [0, 1), new state)"""
+    st = C.c_uint64(state)
+    v = load().oxq_ref_xorshift64_next_f32(C.byref(st))
+    return float(v), int(st.value)
+
+
+def sample_candidates(vals, idx, temperature, min_p, top_p, rng_state):
+    """The sampler after its candidate list: (token, new rng state, final probabilities, survivors)."""
+    v = np.ascontiguousarray(vals, dtype=np.float32).ravel()
+    i = np.ascontiguousarray(idx, dtype=np.uint32).ravel()
+    probs = np.zeros(v.size, dtype=np.float32)
+    st, n_left = C.c_uint64(rng_state), C.c_size_t(0)
+    tok = load().oxq_ref_sample_candidates(_p(v), _p(i), v.size, temperature, min_p, top_p, C.byref(st), _p(probs),
+                                           C.byref(n_left))
+    return int(tok), int(st.value), probs, int(n_left.value)
 
 
 # ---- mixture-of-experts feed-forward (oracle/oxq_oracle_moe.c) ----

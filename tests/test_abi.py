@@ -165,7 +165,7 @@ def test_moe_forward_argument_errors_before_touching_the_gpu():
 
 def test_gemm_workspace_size_is_a_function_of_the_shape():
     """oxq_gemm_q8_workspace_bytes: the re-tiled activations (token rows padded to 128 and 128 more, 46 bytes per
-    token block, rounded to 256), plus -- for at most 16 token rows of Q4_K / IQ4_XS on a matrix of at least 2^25
+    token block, rounded to 256), plus -- for at most 16 token rows of Q4_K / IQ4_XS / Q4_0 / Q6_K / Q8_0 on a matrix of at least 2^25
     weights that yields fewer than 448 groups of 128 rows -- the room for the few-token kernel's per-split sums:
     splits x m x n floats, splits = min(ceil(448 / groups), k / 1024, 16) taken in even numbers of super-blocks.
     For Q4_K the size is at least what the prefill kernel's planes take."""
@@ -181,7 +181,8 @@ def test_gemm_workspace_size_is_a_function_of_the_shape():
     assert w(q4k, 11, 16384, 3584) == planes(11, 3584) + 3 * 11 * 16384 * 4            # 14 super-blocks: 6 + 6 + 2
     assert w(q4k, 16, 4096, 4096) == planes(16, 4096)                                  # below 2^25 weights
     assert w(q4k, 17, 14336, 4096) == planes(17, 4096)                                 # more than 16 rows
-    assert w(q6k, 16, 14336, 4096) == planes(16, 4096)                                 # no few-token kernel for Q6_K
+    assert w(q6k, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4            # Q6_K, Q8_0, Q4_0 alike
+    assert w(13, 16, 14336, 4096) == planes(16, 4096)                                  # Q5_K: no few-token kernel
     assert w(q4k, 16, 128256, 4096) == planes(16, 4096)                                # 1002 groups fill the chip
     # Q4_K: never less than the prefill kernel's planes (74 bytes per token block, token rows padded to 128)
     def prefill(m, k):
