@@ -911,6 +911,16 @@ def main():
             if not parity["pass"]:
                 print("bench.py: PARITY GATE FAILED: " + json.dumps(parity), file=sys.stderr, flush=True)
 
+        if args.f32_route:
+            # the reference's other method on the CPU: gemv on unquantized fp32 activations (the scalar restatement of
+            # Q/reference/q4_k.rs:135-178; one thread, one call of ffn_gate) beside the GPU's f32_route_* legs
+            t_begin = time.perf_counter()
+            O.gemv(O.Q4_K, hw["gate"], F, H, hx)
+            el = time.perf_counter() - t_begin
+            kernels["f32_route_cpu_q4k_gate_14336x4096"] = {
+                "us_per_call": round(el * 1e6, 1), "launches": 1, "distinct_weight_sets": 1,
+                "weight_GBps": round(F * row_bytes(Q4_K, H) / el / 1e9, 3), "frac_hbm_peak": None, "cores": 1,
+                "kind": "port", "sample": "one gemv of ffn_gate 14336x4096 on one host thread (scalar C restatement)"}
         s_mt, n_mt = time_cpu(cores, 8.0)
         s_1t, n_1t = time_cpu(1, 8.0)
         cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "host_cores": host_cores,
