@@ -92,10 +92,13 @@ size_t gemm_workspace_bytes(uint32_t m, uint32_t k, uint32_t n, uint32_t type) {
 // about as long whatever the others do) fill their rounds of the chip: measured at k = 4096 against the tile
 // kernel, 224 / 448 / 672 work groups on 256 compute units 110 / 202 / 298 us against 126 / 228 / 332, but 280 work
 // groups 194 against 172, 168 a tie, 128 and fewer far behind (the tile kernel's smaller tiles spread better).
+// And its token tiles must be mostly full: a work group costs the same with 32 of its 128 token rows in use (128256 x
+// 4096: 32 / 64 / 96 / 128 tokens 208 / 220 / 234 / 245 us against 115 / 185 / 275 / 285 on the tile kernel).
 static bool gemm_prefill_pays(uint32_t m, uint32_t n) {
-    const uint64_t wgs = (uint64_t)((m + 127) / 128) * ((n + 255) / 256), cus = device_cus();
+    const uint64_t token_tiles = (m + 127) / 128;
+    const uint64_t wgs = token_tiles * ((n + 255) / 256), cus = device_cus();
     const uint64_t rounds = (wgs + cus - 1) / cus;
-    return 100 * wgs >= 85 * rounds * cus;
+    return 100 * wgs >= 85 * rounds * cus && 100 * (uint64_t)m >= 70 * 128 * token_tiles;
 }
 
 std::atomic<uint32_t> g_gemm_tile_min_rows{0};  // tuning: 0 = default

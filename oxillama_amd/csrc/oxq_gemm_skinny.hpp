@@ -290,7 +290,10 @@ constexpr int skinny_waves_per_simd() {
 }
 
 // The work of one work group on the token rows tokb .. tok_end - 1 (at most 16 * TT of them) of its group.
-template <class F, int NT, int WAVES, int TT, int PER, bool DUMP>
+// SPREAD_LOG (two token tiles only): the second tile's rows sit in every 2^SPREAD_LOG-th of its 16 slots.  A lane's four
+// results of an MFMA are the slots 4q .. 4q + 3, so with up to 4 (8) rows in the second tile only one (two) of them
+// is a token and the two fmas of each of the others are not compiled in.
+template <class F, int NT, int WAVES, int TT, int PER, bool DUMP, int SPREAD_LOG = 0>
 __device__ __forceinline__ void gemm_skinny_body(
     const uint8_t *__restrict__ W, const uint8_t *__restrict__ A, float *__restrict__ out, int32_t *__restrict__ sums,
     uint32_t m, uint32_t n, uint32_t k, int accumulate, const float *__restrict__ bias, const int32_t *__restrict__ offsets, size_t w_stride,
@@ -330,6 +333,13 @@ __device__ __forceinline__ void gemm_skinny_body(
     // 8 qq .. 8 qq + 7 of token cc's block; token rows past the group's end read as zeros. ----
     constexpr uint32_t KA = (nblk_max * TT * 64 + THREADS - 1) / THREADS;
     const size_t arow = (size_t)(k / 32) * Q8_BLOCK_BYTES;
+    static_assert(SPREAD_LOG == 0 || TT == 2, "spread slots: the second token tile");
+    constexpr uint32_t DEAD_SLOTS = (1u << SPREAD_LOG) - 1;  // the second tile's slot holds a token where slot & DEAD_SLOTS == 0
+    // token row of slot `slot` of tile t, or tok_end (none)
+    auto token_of = [&](uint32_t t, uint32_t slot) {
+        if (SPREAD_LOG != 0 && t == 1) return (slot & DEAD_SLOTS) ? tok_end : tokb + 16 + (slot >> SPREAD_LOG);
+        return tokb + 16 * t + slot;
+    };
     u32x2 tokA[KA];
     uint32_t tokD[KA];
     auto load_tokens = [&](uint32_t sb0, uint32_t nblk) {
@@ -338,7 +348,7 @@ __device__ __forceinline__ void gemm_skinny_body(
         for (uint32_t i = 0; i < KA; i++) {
             const uint32_t idx = threadIdx.x + i * THREADS;
             const uint32_t l = idx & 63, t = (idx >> 6) % TT, b = (idx >> 6) / TT;
-            const uint32_t cc = l >> 2, qq = l & 3, tok = tokb + 16 * t + cc;
+            const uint32_t cc = l >> 2, qq = l & 3, tok = token_of(t, cc);
             tokA[i] = u32x2{0, 0};
             tokD[i] = 0;
             if (idx < total && tok < tok_end) {
@@ -545,11 +555,12 @@ __device__ __forceinline__ void gemm_skinny_body(
                                 const v4i32 r = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, bop[j][is], addend, 0, 0, 0);
 #pragma unroll
                                 for (int v = 0; v < 4; v++) {
+                                    if (SPREAD_LOG != 0 && t == 1 && (v & DEAD_SLOTS)) continue;  // a slot without a token
                                     const int ri = r[v];
                                     const float tt = fmaf(__builtin_bit_cast(float, ri), dsc[j][is], corr[j][is]);  // fl(dsc * isum)
                                     acc[t][j][v] = fmaf(tt, da[v], acc[t][j][v]);
                                     if (DUMP) {  // the integer sum of (token, weight row, sub-block or half of one)
-                                        const uint32_t tok = tokb + 16 * t + 4 * q + v, row = rbase + 16 * j + c;
+                                        const uint32_t tok = token_of(t, 4 * q + v), row = rbase + 16 * j + c;
                                         if (tok < tok_end && row < n)
                                             sums[((size_t)tok * n + row) * (k / 32 * KS) + ((st * 2 + u) * 8 + s) * KS + is] =
                                                 ri - 0x4B400000;
@@ -573,7 +584,7 @@ __device__ __forceinline__ void gemm_skinny_body(
             const uint32_t row = rbase + 16 * j + c;
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const uint32_t tok = tokb + 16 * t + 4 * q + v;
+                const uint32_t tok = token_of(t, 4 * q + v);
                 if (row < n && tok < tok_end && t < (int)tiles_here) {
                     const float y = acc[t][j][v];
                     if (partial) {
@@ -632,6 +643,19 @@ void gemm_skinny_kernel(
         if (tok_end - tokb <= 16) {
             gemm_skinny_body<F, NT, WAVES, 1, 2 * PER, DUMP>(W, A, out, sums, m, n, k, accumulate, bias, offsets, w_stride,
                                                             partial, sb_per_split, tokb, tok_end, rg, gy, ks);
+            return;
+        }
+    }
+    if constexpr (TT == 2 && !DUMP) {
+        // a second tile of up to 4 (8) rows: the body that spreads them over the slots (same sums, same order)
+        if (tok_end - tokb <= 20) {
+            gemm_skinny_body<F, NT, WAVES, TT, PER, DUMP, 2>(W, A, out, sums, m, n, k, accumulate, bias, offsets, w_stride,
+                                                             partial, sb_per_split, tokb, tok_end, rg, gy, ks);
+            return;
+        }
+        if (tok_end - tokb <= 24) {
+            gemm_skinny_body<F, NT, WAVES, TT, PER, DUMP, 1>(W, A, out, sums, m, n, k, accumulate, bias, offsets, w_stride,
+                                                             partial, sb_per_split, tokb, tok_end, rg, gy, ks);
             return;
         }
     }

@@ -92,10 +92,12 @@ def test_prefill_f16_kernel(hip, ref, tuning, shape):
 
 def test_prefill_f16_kernel_is_the_default_where_it_fills_the_chip(hip, ref):
     """Without any knob: a Q4_K matmul whose 128-token x 256-row work groups fill 7/8 of the compute units takes this
-    kernel; one that fills 40 % of them, and any Q6_K matmul, stays on the int8 tile kernel."""
+    kernel (also with 96 of a tile's 128 token rows in use); one that fills 40 % of them, one with 64 token rows (half
+    of every work group's token tile empty), and any Q6_K matmul, stay on the int8 tile kernel."""
     cus = hip.device_info()["compute_units"]
     k = 256
     for t, m, n, expect in ((O.Q4_K, 128, 256 * (cus * 7 // 8), True), (O.Q4_K, 128, 256 * (cus * 2 // 5), False),
+                            (O.Q4_K, 96, 256 * (cus * 7 // 8), True), (O.Q4_K, 64, 256 * (cus * 7 // 8), False),
                             (O.Q6_K, 128, 256 * (cus * 7 // 8), False)):
         say("default kernel", O.NAMES[t], m, n, k)
         w = synth.weights(t, 5, n, k)
@@ -107,7 +109,7 @@ def test_prefill_f16_kernel_is_the_default_where_it_fills_the_chip(hip, ref):
                          workspace=ws)
         torch.cuda.synchronize()
         assert ("gemm_prefill_q4k" in last_launch()) == expect, (O.NAMES[t], m, n, last_launch())
-        rows = [0, 1, 63, 127]
+        rows = [0, 1, 63, m - 1]
         y_ref = oracle_rows(ref, t, w, acts, n, k, rows)
         assert np.abs(dy.cpu().numpy()[rows] - y_ref).max() <= FP32_REL_TOL * np.abs(y_ref).max()
 
