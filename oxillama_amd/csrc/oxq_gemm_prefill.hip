@@ -82,13 +82,15 @@ __host__ __device__ inline size_t pf_pbf_bytes(size_t nsb, size_t mpad) { return
 // unpack takes bytes 0 and 2 of a dword together (they sit in the two 16-bit halves), then bytes 1 and 3.
 __device__ __forceinline__ constexpr int pf_slot_byte(int j) { return (j & 4) | ((j & 1) << 1) | ((j >> 1) & 1); }
 
-// One thread per (sub-block j, token t); consecutive threads are consecutive tokens.
+// One thread per (sub-block j, token t).  Eight consecutive threads take the eight sub-blocks of one super-block of one
+// token (272 contiguous bytes of its row; their eight bf16 pieces of P make one 16-byte run), the next eight the next
+// token: reads in runs of a row's bytes, operand writes in runs of eight tokens per sub-block.
 __global__ __launch_bounds__(256) void prefill_prep_acts(const uint8_t *__restrict__ A, uint8_t *__restrict__ tokf,
                                                         uint16_t *__restrict__ dag, uint16_t *__restrict__ pbf, uint32_t m,
                                                         uint32_t mpad, uint32_t nsb) {
     const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= mpad * nsb) return;
-    const uint32_t j = idx / mpad, t = idx % mpad;
+    const uint32_t grp = idx >> 3, t = grp % mpad, j = (grp / mpad) * 8 + (idx & 7);
     u32x4 q[2] = {{0, 0, 0, 0}, {0, 0, 0, 0}};
     uint32_t dbits = 0;
     if (t < m) {
