@@ -814,6 +814,9 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     case 3: return launch_tile<F, 2, 2, 2, 1, false>(a, p, stream);
     case 4: return launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
     case 5: return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
+    case 6: return launch_tile<F, 4, 1, 1, 2, false>(a, p, stream);
+    case 7: return launch_tile<F, 4, 1, 1, 1, false>(a, p, stream);
+    case 8: return launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
     case 12: return launch_tile<F, 1, 2, 1, 2, false>(a, p, stream);
     case 13: return launch_tile<F, 1, 2, 1, 4, false>(a, p, stream);
     case 14: return launch_tile<F, 1, 1, 1, 2, false>(a, p, stream);
@@ -834,7 +837,17 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
             // chip one and a half work groups per compute unit: 14336 x 4096, 512 tokens 123 us against 125 us,
             // 2048 tokens 383 us against 422 us; 4096 x 14336 has too few such tiles (214 us against 140 us)
             const size_t wgs = (size_t)((rows + 127) / 128) * ((a.n + 127) / 128) * (a.offsets ? a.n_experts : 1);
-            if (2 * wgs >= 3 * (size_t)device_cus()) return launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
+            // Within the 128 x 128 tile a wave takes 128 tokens x 32 rows (four token tiles against ONE weight-row
+            // tile) rather than 64 x 64: half the weight loads per MFMA, and those are the loads in which every lane
+            // reads its own row.  Same bits.  512 x 14336 x 4096: Q8_0 122 us against 158, Q4_0 122 against 141,
+            // IQ4_XS 107 against 118, Q6_K 168 against 189; 2048 tokens: Q8_0 388 against 503.  Q4_K, whose weight
+            // loads are the lightest per MFMA, is the exception (114 against 111) and keeps 64 x 64.
+            constexpr bool wide = F::TYPE != OXQ_TYPE_Q4_K;
+            if (2 * wgs >= 3 * (size_t)device_cus())
+                return wide ? launch_tile<F, 4, 1, 1, 1, false>(a, p, stream) : launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
+            // one to one and a half work groups per compute unit: still the better shape for the formats of a
+            // byte and more per weight (512 x 8192 x 8192 Q8_0: 149 us against 180)
+            if (wide && F::BLOCK_BYTES >= 256 && wgs >= (size_t)device_cus()) return launch_tile<F, 4, 1, 1, 1, false>(a, p, stream);
             return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
         }
         if (rows > 64) return launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);

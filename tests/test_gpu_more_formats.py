@@ -294,6 +294,42 @@ def test_prefill_tile_kernel_rows_of_whole_32_blocks(hip, ref, tuning, shape, t)
     _prefill_tile_case(hip, ref, shape, t)
 
 
+@pytest.mark.parametrize("t", TILE_TYPES, ids=ids)
+def test_prefill_many_tokens_takes_the_wide_tile_shape(hip, ref, t):
+    """More than 384 tokens on a matrix whose 128 x 128 work-group tiles give every compute unit one and a half: the
+    library's own choice is the shape with four token tiles against one weight-row tile per wave.  Sampled tokens
+    against the oracle on all outputs (ragged n); the debug dump's launch (another shape) gives the same bits."""
+    from oxillama_amd import capi
+    import ctypes as C
+    cus = hip.device_info()["compute_units"]
+    m, k_ = 400, 256
+    n = 128 * ((3 * cus + 7) // 8) - 5
+    say("prefill, wide tiles", O.NAMES[t], (m, n, k_))
+    w = O.random_blocks(t, 990, n, k_)
+    acts = ref.quantize_q8_0(synth.normal_f32(991, m * k_))
+    kern = hip.HipKernel(t)
+    dw, da = dev(w), dev(acts)
+    ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device=DEV)
+    dy = torch.full((m + 1, n), 7.0, dtype=torch.float32, device=DEV)
+    kern.gemm_q8_dev(dw, da, dy, m, n, k_, accumulate=False, workspace=ws)
+    torch.cuda.synchronize()
+    buf = C.create_string_buffer(256)
+    capi.load().oxq_last_launch(buf, 256)
+    took = buf.value.decode()
+    assert took.startswith("gemm_tile_kernel") and ",4,1,1,1>" in took, took
+    rows = sorted(set(list(range(0, m, 37)) + [127, 128, 383, 384, m - 1]))
+    arb = k_ // 32 * 34
+    y = host(dy)
+    assert np.all(y[m] == 7.0)
+    y_ref = np.stack([ref.matvec_q8_fused_mt(t, w, acts[r * arb:(r + 1) * arb], n, k_, 16) for r in rows])
+    assert_close(y[rows], y_ref, f"wide tiles {O.NAMES[t]}")
+    dsum = torch.empty((m, n, k_ // O.GROUP_COLS[t]), dtype=torch.int32, device=DEV)
+    dy2 = torch.empty((m, n), dtype=torch.float32, device=DEV)
+    kern.gemm_block_sums_dev(dw, da, dy2, dsum, m, n, k_, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(dy2, dy[:m])
+
+
 def _prefill_tile_case(hip, ref, shape, t):
     m, n, k_ = shape
     if True:

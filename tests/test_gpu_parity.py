@@ -561,6 +561,42 @@ def test_prefill_tile_kernel(hip, ref, tuning, shape, t):
     _prefill_tile_case(hip, ref, shape, t)
 
 
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_prefill_many_tokens_takes_the_wide_tile_shape(hip, ref, t):
+    """More than 384 tokens on a matrix whose 128 x 128 work-group tiles give every compute unit one and a half: the tile
+    kernel with four token tiles against one weight-row tile per wave (every format but Q4_K).  The library's own choice, no knob; sampled tokens against the oracle on all outputs, ragged n."""
+    import torch
+    from test_gpu_prefill_f16 import last_launch
+    cus = hip.device_info()["compute_units"]
+    m, k_ = 400, 256
+    n = 128 * ((3 * cus + 7) // 8) - 5
+    say("prefill, wide tiles", O.NAMES[t], (m, n, k_))
+    w = synth.weights(t, 650, n, k_)
+    acts = ref.quantize_q8_0(synth.normal_f32(651, m * k_))
+    kern = hip.HipKernel(t)
+    dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
+    ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
+    dy = torch.full((m + 1, n), 7.0, dtype=torch.float32, device="cuda")
+    kern.gemm_q8_dev(dw, da, dy, m, n, k_, accumulate=False, workspace=ws)
+    torch.cuda.synchronize()
+    took = last_launch()
+    if t == O.Q4_K:  # its f16 kernel where that fills the chip, else the tile kernel's 64 x 64 waves
+        assert "gemm_prefill_q4k" in took or took.startswith("gemm_tile_kernel<Q4_K,2,2,2,2>"), took
+    else:
+        assert took.startswith("gemm_tile_kernel") and ",4,1,1,1>" in took, took
+    rows = sorted(set(list(range(0, m, 37)) + [127, 128, 383, 384, m - 1]))
+    y = dy.cpu().numpy()
+    assert np.all(y[m] == 7.0)
+    assert_close(y[rows], _oracle_prefill(ref, t, w, acts, m, n, k_, rows=rows), f"wide tiles {O.NAMES[t]}")
+    # the debug dump's launch (another tile shape) gives the same bits and the oracle's integer sums
+    if t != O.Q4_K:
+        dsum = torch.empty((m, n, k_ // (16 if t in (O.Q6_K, O.Q2_K, O.Q3_K) else 32)), dtype=torch.int32, device="cuda")
+        dy2 = torch.empty((m, n), dtype=torch.float32, device="cuda")
+        kern.gemm_block_sums_dev(dw, da, dy2, dsum, m, n, k_, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(dy2, dy[:m])
+
+
 BLOCKS32 = [t for t in O.ALL_TYPES if O.BLOCK[t][0] == 32]
 
 
