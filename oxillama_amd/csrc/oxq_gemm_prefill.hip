@@ -325,7 +325,6 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         static_for(std::make_integer_sequence<int, 32>{}, [&](auto qc) __attribute__((always_inline)) {
             constexpr int q = decltype(qc)::value;
             constexpr int g = q >> 3, ts = q & 7, e = ts >> 2, mt = ts & 3;
-            const uint8_t *const buf = tokbuf(g);
             if constexpr (ts == 0) {
                 // the buffer of the stage before is free since the barrier that ended it: it takes the stage three ahead
                 request_stage(tokbuf(g + 3), min(S0 + g + 3, Slast));

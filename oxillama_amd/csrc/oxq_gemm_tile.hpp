@@ -803,6 +803,7 @@ template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
     const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
     const int variant = g_gemm_variant.load(std::memory_order_relaxed);
+    (void)variant;  // (read by the fixed-shape knobs, which the second translation unit leaves out)
     if (a.sums)  // debug dump: the same tile layout (and fp32 summation order) as the production choice below
         return rows > 384  ? launch_tile<F, 2, 1, 2, 1, true>(a, p, stream)
                : rows > 64 ? launch_tile<F, 2, 1, 1, 2, true>(a, p, stream)
