@@ -522,6 +522,17 @@ size_t oxq_topk_workspace_bytes(size_t n, size_t k);
 int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
                  uint32_t *d_out_indices, void *d_workspace, size_t workspace_bytes, void *stream);
 
+/* The sampler's edits of the logits BEFORE the candidate list, in place (sample_with_rng steps 0 and 1,
+ * crates/oxillama-runtime/src/sampling/mod.rs:573-613): banned tokens to -inf; d_bias_values[i] added
+ * to logit d_bias_tokens[i] where that logit is still finite (each token at most once: the
+ * reference's map); the repetition penalty over the last `window` of the n_recent recent tokens --
+ * once per occurrence, a positive logit divided by the penalty, any other multiplied; nothing for
+ * a penalty of 1.  Token ids >= n are skipped, as in the reference.  Any list may be empty (NULL,
+ * 0).  window <= 4096 entries in effect.  One launch; the grammar mask of the reference is not here. */
+int oxq_logits_edit_dev(float *d_logits, size_t n, const uint32_t *d_banned, size_t n_banned,
+                        const uint32_t *d_bias_tokens, const float *d_bias_values, size_t n_bias,
+                        const uint32_t *d_recent, size_t n_recent, size_t window,
+                        float repetition_penalty, void *stream);
 /* The rest of the sampler on those candidates (sample_with_rng from its greedy shortcut on,
  * crates/oxillama-runtime/src/sampling/mod.rs:487-564): temperature <= 0 or k == 1 returns the
  * first candidate; otherwise every value times 1/temperature, softmax over the k candidates

@@ -152,6 +152,14 @@ oxq_ref_status oxq_ref_linear_forward(uint32_t type, int tier, const uint8_t *w,
  * crates/oxillama-runtime/src/sampling/mod.rs:500-509,652-662 */
 uint32_t oxq_ref_argmax(const float *values, size_t n);
 void oxq_ref_topk(const float *values, size_t n, size_t k, float *out_vals, uint32_t *out_idx);
+/* Steps 0 and 1 of sample_with_rng on the logits, in place: apply_logit_bias_and_banned_tokens (sampling/mod.rs:
+ * 573-593: banned tokens to -inf, then bias added where the logit is still finite) and apply_repetition_penalty
+ * (mod.rs:596-613: for every token of the last `window` entries of recent, in order and once per occurrence, a
+ * positive logit is divided by the penalty, any other multiplied; nothing for penalty == 1).  Token ids past n are
+ * skipped.  bias_tokens holds each token once (the reference's map). */
+void oxq_ref_logits_edit(float *logits, size_t n, const uint32_t *banned, size_t n_banned,
+                         const uint32_t *bias_tokens, const float *bias_values, size_t n_bias,
+                         const uint32_t *recent, size_t n_recent, size_t window, float repetition_penalty);
 /* Xorshift64::new / next_u64 / next_f32, sampling/mod.rs:669-690: the sampler's generator.  *state is
  * advanced; a zero seed is replaced as new() does. */
 uint64_t oxq_ref_xorshift64_seed(uint64_t seed);

@@ -326,3 +326,34 @@ uint32_t oxq_ref_sample_candidates(const float *vals, const uint32_t *idx, size_
     free(ids);
     return token;
 }
+
+/* apply_logit_bias_and_banned_tokens, sampling/mod.rs:573-593; apply_repetition_penalty, mod.rs:596-613 */
+void oxq_ref_logits_edit(float *logits, size_t n, const uint32_t *banned, size_t n_banned,
+                         const uint32_t *bias_tokens, const float *bias_values, size_t n_bias,
+                         const uint32_t *recent, size_t n_recent, size_t window, float repetition_penalty) {
+    for (size_t i = 0; i < n_banned; i++) {
+        if (banned[i] < n) {
+            logits[banned[i]] = -INFINITY;
+        }
+    }
+    for (size_t i = 0; i < n_bias; i++) {
+        const size_t idx = bias_tokens[i];
+        if (idx < n && isfinite(logits[idx])) {
+            logits[idx] += bias_values[i];
+        }
+    }
+    if (repetition_penalty == 1.0f || n_recent == 0) {
+        return;
+    }
+    const size_t start = n_recent > window ? n_recent - window : 0; /* saturating_sub */
+    for (size_t i = start; i < n_recent; i++) {
+        const size_t idx = recent[i];
+        if (idx < n) {
+            if (logits[idx] > 0.0f) {
+                logits[idx] /= repetition_penalty;
+            } else {
+                logits[idx] *= repetition_penalty;
+            }
+        }
+    }
+}

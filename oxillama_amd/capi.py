@@ -180,6 +180,8 @@ SIGNATURES = {
                                       C.c_uint32, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p,
                                       C.c_size_t, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p,
                                       C.c_size_t, C.c_void_p]),
+    "oxq_logits_edit_dev": (C.c_int, [C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p, C.c_size_t,
+                                      C.c_void_p, C.c_size_t, C.c_size_t, C.c_float, C.c_void_p]),
     "oxq_sample_candidates_dev": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_float, C.c_float,
                                             C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "oxq_topk_workspace_bytes": (C.c_size_t, [C.c_size_t, C.c_size_t]),

@@ -1598,6 +1598,24 @@ int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
     return OXQ_OK;
 }
 
+int oxq_logits_edit_dev(float *d_logits, size_t n, const uint32_t *d_banned, size_t n_banned, const uint32_t *d_bias_tokens,
+                        const float *d_bias_values, size_t n_bias, const uint32_t *d_recent, size_t n_recent,
+                        size_t window, float repetition_penalty, void *stream) {
+    if (!d_logits || n == 0 || n > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n, "1 .. 2^32-1 logits");
+    if ((n_banned && !d_banned) || (n_bias && (!d_bias_tokens || !d_bias_values)) || (n_recent && !d_recent))
+        return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer");
+    if (n_banned > 0xFFFFFFFFull || n_bias > 0xFFFFFFFFull) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 0xFFFFFFFFull, n_banned, "list too long");
+    // the window is the tail of the recent tokens (saturating_sub, sampling/mod.rs:601-603)
+    const size_t n_window = n_recent < window ? n_recent : window;
+    if (n_window > 4096) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 4096, n_window, "repetition window of at most 4096 tokens");
+    int st = ensure_init();
+    if (st != OXQ_OK) return st;
+    OXQ_HIP(oxq::launch_logits_edit(d_logits, (uint32_t)n, d_banned, (uint32_t)n_banned, d_bias_tokens, d_bias_values,
+                                    (uint32_t)n_bias, d_recent ? d_recent + (n_recent - n_window) : nullptr,
+                                    (uint32_t)n_window, repetition_penalty, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
 int oxq_sample_candidates_dev(const float *d_values, const uint32_t *d_indices, size_t k, float temperature, float min_p,
                               float top_p, uint64_t *d_rng_state, uint32_t *d_token, float *d_probs, void *stream) {
     if (k == 0 || k > 256) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, k, "between 1 and 256 candidates");

@@ -155,6 +155,10 @@ hipError_t launch_moe_route(const float *router, const float *x, int32_t *expert
 size_t topk_workspace_bytes(size_t n, size_t k);
 hipError_t launch_topk(const float *x, uint32_t n, uint32_t k, float *out_vals, uint32_t *out_idx, void *workspace,
                        hipStream_t stream);
+// The sampler's steps before the candidate list: banned tokens, logit bias, repetition penalty, on the logits in place.
+hipError_t launch_logits_edit(float *logits, uint32_t n, const uint32_t *banned, uint32_t n_banned, const uint32_t *bias_tokens,
+                              const float *bias_values, uint32_t n_bias, const uint32_t *recent, uint32_t n_window,
+                              float penalty, hipStream_t stream);
 // The sampler's steps after the candidate list (temperature, softmax, min-p, top-p, draw) on k <= 256 candidates.
 hipError_t launch_sample_candidates(const float *vals, const uint32_t *idx, uint32_t k, float temperature, float min_p,
                                     float top_p, uint64_t *rng_state, uint32_t *token_out, float *probs_out,

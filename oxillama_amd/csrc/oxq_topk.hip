@@ -522,6 +522,58 @@ __global__ __launch_bounds__(256) void sample_candidates_kernel(const float *__r
     }
 }
 
+// Steps 0 and 1 of sample_with_rng on the logits in place (sampling/mod.rs:573-613): banned tokens to -inf, the
+// bias added where the logit is still finite (each biased token once: the reference's map), then the repetition
+// penalty over the last `window` recent tokens.  One work group; the three steps are ordered by barriers (they may
+// touch the same logit).  The reference applies the penalty once per OCCURRENCE of a token, in order: here the lane
+// that holds a token's first occurrence in the window applies it as many times as the token occurs, to the value
+// in a register -- the same operations on the same value in the same order.
+__global__ __launch_bounds__(256) void logits_edit_kernel(float *__restrict__ logits, uint32_t n,
+                                                          const uint32_t *__restrict__ banned, uint32_t n_banned,
+                                                          const uint32_t *__restrict__ bias_tokens,
+                                                          const float *__restrict__ bias_values, uint32_t n_bias,
+                                                          const uint32_t *__restrict__ recent, uint32_t n_window,
+                                                          float penalty) {
+    const uint32_t t = threadIdx.x;
+    for (uint32_t i = t; i < n_banned; i += 256)
+        if (banned[i] < n) logits[banned[i]] = -INFINITY;
+    __threadfence_block();
+    __syncthreads();
+    for (uint32_t i = t; i < n_bias; i += 256) {
+        const uint32_t idx = bias_tokens[i];
+        if (idx < n) {
+            const float v = logits[idx];
+            if (__builtin_isfinite(v)) logits[idx] = v + bias_values[i];
+        }
+    }
+    __threadfence_block();
+    __syncthreads();
+    if (penalty == 1.0f || n_window == 0) return;
+    for (uint32_t i = t; i < n_window; i += 256) {
+        const uint32_t tok = recent[i];
+        if (tok >= n) continue;
+        uint32_t count = 0;
+        bool first = true;
+        for (uint32_t j = 0; j < n_window; j++) {
+            const bool same = recent[j] == tok;
+            count += same ? 1u : 0u;
+            first = first && !(same && j < i);
+        }
+        if (!first) continue;
+        float v = logits[tok];
+        for (uint32_t c = 0; c < count; c++) v = v > 0.0f ? v / penalty : v * penalty;
+        logits[tok] = v;
+    }
+}
+
+hipError_t launch_logits_edit(float *logits, uint32_t n, const uint32_t *banned, uint32_t n_banned, const uint32_t *bias_tokens,
+                              const float *bias_values, uint32_t n_bias, const uint32_t *recent, uint32_t n_window,
+                              float penalty, hipStream_t stream) {
+    hipLaunchKernelGGL(logits_edit_kernel, dim3(1), dim3(256), 0, stream, logits, n, banned, n_banned, bias_tokens,
+                       bias_values, n_bias, recent, n_window, penalty);
+    return hipGetLastError();
+}
+
 hipError_t launch_sample_candidates(const float *vals, const uint32_t *idx, uint32_t k, float temperature, float min_p,
                                     float top_p, uint64_t *rng_state, uint32_t *token_out, float *probs_out,
                                     hipStream_t stream) {

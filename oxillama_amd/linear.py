@@ -157,6 +157,20 @@ def topk_dev(d_values, k, d_out_values, d_out_indices, workspace):
                             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream()))
 
 
+def logits_edit_dev(d_logits, d_banned=None, d_bias_tokens=None, d_bias_values=None, d_recent=None, window=0,
+                    repetition_penalty=1.0):
+    """The sampler's edits of the logits before the candidate list (sampling/mod.rs:573-613), in place: banned tokens,
+    logit bias, repetition penalty over the last `window` of d_recent.  Token lists: int32 / uint32 CUDA tensors."""
+    def ptr(t):
+        return t.data_ptr() if t is not None and t.numel() else None
+
+    def cnt(t):
+        return t.numel() if t is not None else 0
+    _check(capi.load().oxq_logits_edit_dev(d_logits.data_ptr(), d_logits.numel(), ptr(d_banned), cnt(d_banned),
+                                           ptr(d_bias_tokens), ptr(d_bias_values), cnt(d_bias_tokens), ptr(d_recent),
+                                           cnt(d_recent), window, repetition_penalty, _stream()))
+
+
 def sample_candidates_dev(d_values, d_indices, k, temperature, min_p, top_p, d_rng_state, d_token, d_probs=None):
     """The sampler after its candidate list (sampling/mod.rs:487-564): temperature, softmax, min-p, top-p, the draw.
     d_rng_state: one uint64 (the reference's Xorshift64 state), d_token: one uint32, d_probs: optional k floats."""

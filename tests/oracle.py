@@ -134,6 +134,8 @@ def load():
     lib.oxq_ref_argmax.argtypes = [vp, sz]
     lib.oxq_ref_topk.restype = None
     lib.oxq_ref_topk.argtypes = [vp, sz, sz, vp, vp]
+    lib.oxq_ref_logits_edit.restype = None
+    lib.oxq_ref_logits_edit.argtypes = [vp, sz, vp, sz, vp, vp, sz, vp, sz, sz, C.c_float]
     lib.oxq_ref_xorshift64_seed.restype = C.c_uint64
     lib.oxq_ref_xorshift64_seed.argtypes = [C.c_uint64]
     lib.oxq_ref_xorshift64_next_f32.restype = C.c_float
@@ -425,6 +427,19 @@ def topk(values, k):
     vals, idx = np.zeros(k, dtype=np.float32), np.zeros(k, dtype=np.uint32)
     load().oxq_ref_topk(_p(v), v.size, k, _p(vals), _p(idx))
     return vals, idx
+
+
+def logits_edit(logits, banned=(), bias=None, recent=(), window=0, repetition_penalty=1.0):
+    """Steps 0 and 1 of the sampler on a copy of the logits: banned tokens, logit bias (dict token -> bias), repetition
+    penalty over the last `window` of `recent`."""
+    out = np.array(logits, dtype=np.float32).ravel().copy()
+    bn = np.ascontiguousarray(banned, dtype=np.uint32)
+    bt = np.ascontiguousarray(list((bias or {}).keys()), dtype=np.uint32)
+    bv = np.ascontiguousarray(list((bias or {}).values()), dtype=np.float32)
+    rc = np.ascontiguousarray(recent, dtype=np.uint32)
+    load().oxq_ref_logits_edit(_p(out), out.size, _p(bn), bn.size, _p(bt), _p(bv), bt.size, _p(rc), rc.size, window,
+                               repetition_penalty)
+    return out
 
 
 def xorshift64_seed(seed):

@@ -119,3 +119,76 @@ def test_sampler_in_a_graph_continues_the_sequence(hip, ref):
             stream.synchronize()
             tok, state, _, _ = ref.sample_candidates(vals, idx, *cfg, state)
             assert int(d_tok.item()) == tok and int(d_state.item()) & ((1 << 64) - 1) == state, i
+
+
+def _edit_on_device(logits, banned, bias, recent, window, penalty):
+    import torch
+
+    def u32(v):
+        return torch.from_numpy(np.ascontiguousarray(v, dtype=np.uint32).view(np.int32)).cuda() if len(v) else None
+    d = torch.from_numpy(np.ascontiguousarray(logits, dtype=np.float32)).cuda()
+    bt, bv = list(bias.keys()), list(bias.values())
+    linear.logits_edit_dev(d, u32(banned), u32(bt), torch.tensor(bv, dtype=torch.float32, device="cuda") if bv else None,
+                           u32(recent), window, penalty)
+    torch.cuda.synchronize()
+    return d.cpu().numpy()
+
+
+def test_logits_edit_follows_the_oracle(hip, ref):
+    """Banned tokens, logit bias and the repetition penalty (a token that occurs several times in the window is
+    penalised that many times) on the device: every logit bit for bit the oracle's."""
+    rng = np.random.default_rng(11)
+    for trial in range(25):
+        n = int(rng.choice([7, 300, 32000, 128256]))
+        logits = (rng.standard_normal(n) * 4).astype(np.float32)
+        logits[rng.integers(0, n, size=3)] = -np.inf
+        banned = rng.integers(0, n + 3, size=int(rng.integers(0, 40))).tolist()
+        bias = {int(t): float(rng.standard_normal() * 10) for t in rng.choice(n + 2, size=int(rng.integers(0, min(30, n))), replace=False)}
+        recent = rng.integers(0, min(n + 2, 40), size=int(rng.integers(0, 600))).tolist()
+        window = int(rng.choice([0, 1, 64, 300, 5000]))
+        if min(window, len(recent)) > 4096:
+            window = 64
+        penalty = float(rng.choice([1.0, 1.1, 1.3, 0.8]))
+        got = _edit_on_device(logits, banned, bias, recent, window, penalty)
+        want = ref.logits_edit(logits, banned, bias, recent, window, penalty)
+        assert np.array_equal(got, want), (trial, n, window, penalty)
+
+
+def test_default_sampler_config_end_to_end(hip, ref):
+    """The reference's default configuration (repetition penalty 1.1 over 64 tokens, temperature 0.7, top-k 40, top-p
+    0.9: SamplerConfig::default, mod.rs:140-160) as three launches -- logit edits, candidate list, draw -- against the
+    oracle's three functions, thirty tokens in a row with the sampled token joining the recent ones."""
+    import torch
+    n, k = 32000, 40
+    state = O.xorshift64_seed(2024)
+    d_state = torch.tensor([state], dtype=torch.int64, device="cuda")
+    d_tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    d_vals = torch.empty(k, dtype=torch.float32, device="cuda")
+    d_idx = torch.empty(k, dtype=torch.int32, device="cuda")
+    ws = torch.empty(linear.topk_workspace_bytes(n, k) // 8 + 1, dtype=torch.int64, device="cuda")
+    recent = []
+    for step in range(30):
+        logits = (synth.normal_f32(9000 + step, n) * 3.0).astype(np.float32)
+        want_logits = ref.logits_edit(logits, recent=recent, window=64, repetition_penalty=1.1)
+        vals, idx = ref.topk(want_logits, k)
+        tok, state, _, _ = ref.sample_candidates(vals, idx, 0.7, 0.0, 0.9, state)
+        d_logits = torch.from_numpy(logits).cuda()
+        d_recent = torch.tensor(recent, dtype=torch.int32, device="cuda") if recent else None
+        linear.logits_edit_dev(d_logits, d_recent=d_recent, window=64, repetition_penalty=1.1)
+        linear.topk_dev(d_logits, k, d_vals, d_idx, ws)
+        linear.sample_candidates_dev(d_vals, d_idx, k, 0.7, 0.0, 0.9, d_state, d_tok)
+        torch.cuda.synchronize()
+        assert int(d_tok.item()) == tok and int(d_state.item()) & ((1 << 64) - 1) == state, step
+        recent.append(tok)
+        if step % 3 == 0:
+            recent.append(tok)  # repeats in the window
+
+
+def test_reference_bias_and_ban_cases_on_the_device(hip, ref):
+    out = _edit_on_device([1.0, 5.0, 4.9, 1.0], [], {}, [1], 64, 100.0)
+    assert int(np.argmax(out)) == 2
+    out = _edit_on_device(np.arange(5, dtype=np.float32), [0, 1, 2, 4], {}, [], 0, 1.0)
+    assert np.all(np.isneginf(out[[0, 1, 2, 4]])) and out[3] == 3.0
+    assert int(np.argmax(_edit_on_device([10.0, -20.0, -20.0, -20.0], [], {1: 100.0}, [], 0, 1.0))) == 1
+    assert int(np.argmax(_edit_on_device([100.0, 1.0, 0.5, 0.1], [], {0: -200.0}, [], 0, 1.0))) == 1
+    assert np.isneginf(_edit_on_device([1.0, 2.0], [1], {1: 50.0}, [], 0, 1.0)[1])

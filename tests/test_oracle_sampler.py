@@ -140,3 +140,50 @@ def test_edges():
     # outside; the partition is checked instead: cumulative sums of the final probabilities end within 1e-6 of one
     _, _, probs, n = O.sample_candidates(np.linspace(5, -5, 200), np.arange(200), 1.3, 0.0, 1.0, 3)
     assert n == 200 and abs(float(np.cumsum(probs.astype(np.float64))[-1]) - 1.0) < 1e-6
+
+
+def py_logits_edit(logits, banned, bias, recent, window, penalty):
+    """The reference's two functions (mod.rs:573-613) as plain Python over numpy float32 scalars."""
+    out = [np.float32(v) for v in logits]
+    for tkn in banned:
+        if tkn < len(out):
+            out[tkn] = np.float32(-np.inf)
+    for tkn, b in bias.items():
+        if tkn < len(out) and np.isfinite(out[tkn]):
+            out[tkn] = np.float32(out[tkn] + np.float32(b))
+    if penalty != 1.0 and len(recent):
+        for tkn in recent[max(0, len(recent) - window):]:
+            if tkn < len(out):
+                out[tkn] = np.float32(out[tkn] / np.float32(penalty)) if out[tkn] > 0 else np.float32(out[tkn] * np.float32(penalty))
+    return np.array(out, dtype=np.float32)
+
+
+def test_logits_edit_reference_cases():
+    # test_repetition_penalty (mod.rs:789-806): token 1 penalised, token 2 wins
+    out = O.logits_edit([1.0, 5.0, 4.9, 1.0], recent=[1], window=64, repetition_penalty=100.0)
+    assert int(np.argmax(out)) == 2 and out[1] == np.float32(5.0) / np.float32(100.0)
+    # banned_tokens_never_sampled (mod.rs:956-983): everything but token 3 at -inf
+    out = O.logits_edit(np.arange(5, dtype=np.float32), banned=[0, 1, 2, 4])
+    assert np.all(np.isneginf(out[[0, 1, 2, 4]])) and out[3] == 3.0
+    # positive_bias / negative_bias (mod.rs:986-1028)
+    assert int(np.argmax(O.logits_edit([10.0, -20.0, -20.0, -20.0], bias={1: 100.0}))) == 1
+    assert int(np.argmax(O.logits_edit([100.0, 1.0, 0.5, 0.1], bias={0: -200.0}))) == 1
+    # logit_bias_empty_config_no_op (mod.rs:1031-1044)
+    assert np.array_equal(O.logits_edit([1.0, 2.0, 3.0, 0.5]), np.float32([1.0, 2.0, 3.0, 0.5]))
+    # a banned token stays banned whatever its bias (mod.rs:586-590)
+    assert np.isneginf(O.logits_edit([1.0, 2.0], banned=[1], bias={1: 50.0})[1])
+
+
+def test_logits_edit_against_plain_python():
+    rng = np.random.default_rng(5)
+    for trial in range(30):
+        n = int(rng.integers(5, 300))
+        logits = (rng.standard_normal(n) * 4).astype(np.float32)
+        banned = rng.integers(0, n + 3, size=int(rng.integers(0, 6))).tolist()  # some ids past the vocabulary
+        bias = {int(t): float(rng.standard_normal() * 10) for t in rng.choice(n + 2, size=int(rng.integers(0, 6)), replace=False)}
+        recent = rng.integers(0, min(n + 2, 12), size=int(rng.integers(0, 90))).tolist()  # few distinct ids: repeats
+        window = int(rng.integers(0, 100))
+        penalty = float(rng.choice([1.0, 1.1, 1.3, 0.8]))
+        got = O.logits_edit(logits, banned, bias, recent, window, penalty)
+        want = py_logits_edit(logits, banned, bias, recent, window, penalty)
+        assert np.array_equal(got, want, equal_nan=True), trial
