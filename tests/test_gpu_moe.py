@@ -200,7 +200,7 @@ def _moe_ffn_layer_case(hip, ref, types, shape):
     experts, weights, rows = host(d["experts"]), host(d["weights"]), host(d["token_rows"])
     q8, gh, uh, hqh, yh = host(d_q8), host(g), host(u), host(hq), host(y).reshape(pairs, hidden)
     a_row, h_row = hidden // 32 * 34, inter // 32 * 34
-    sample = sorted(set([0, n_tok - 1, n_tok // 2] + list(range(0, n_tok, 17))))
+    sample = sorted(set([0, n_tok - 1, n_tok // 2] + list(range(0, n_tok, 4))))
     flipped_h = bytes_h = flipped_chain = scales_chain = 0
     for t in sample:
         xt = x[t * hidden:(t + 1) * hidden]

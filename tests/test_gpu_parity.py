@@ -645,8 +645,8 @@ def _prefill_tile_case(hip, ref, shape, t):
 
 
 def test_prefill_full_size_c4(hip, ref):
-    """C4: 512 tokens x Q4_K 14336 x 4096.  Oracle on every 16th token (all 14336 outputs each), on all tokens for two
-    512-row slabs of W, and bit-exact integer sums on those slabs."""
+    """C4: 512 tokens x Q4_K 14336 x 4096.  Oracle on every token and every output, and bit-exact integer sums (the tile
+    kernel's, and the prefill kernel's scaled ones) on two 512-row slabs of W."""
     import torch
     m, n, k_, t = 512, 14336, 4096, O.Q4_K
     w = synth.weights(t, 31, n, k_)
@@ -663,7 +663,7 @@ def test_prefill_full_size_c4(hip, ref):
     torch.cuda.synchronize()
     from test_gpu_prefill_f16 import last_launch, q4k_sub_block_scales
     assert "gemm_prefill_q4k" in last_launch(), last_launch()  # C4 is the shape the f16 prefill kernel is for
-    rows = list(range(0, m, 16)) + [m - 1]
+    rows = list(range(m))  # every token, every output: 512 oracle matvecs of 14336 x 4096 on the host's threads
     y_ref = _oracle_prefill(ref, t, w, acts, m, n, k_, rows=rows)
     assert_close(dy.cpu().numpy()[rows], y_ref, "C4 prefill")
     # two 512-row slabs of W (one that straddles tile boundaries in the middle, and the last rows): the oracle
@@ -775,7 +775,7 @@ def test_moe_grouped_matmul(hip, ref, t, cfg):
 
 def test_moe_full_size_c5_one_projection(hip, ref):
     """C5 shapes: 8 experts of IQ4_XS 14336 x 4096 (gate) and 4096 x 14336 (down), 64 tokens top-2.
-    Oracle on a sample of pairs (every row of the sampled pairs)."""
+    Oracle on every pair row, every output."""
     import torch
     t, n_experts, n_tok, top_k = O.IQ4_XS, 8, 64, 2
     kern = hip.HipKernel(t)
@@ -788,7 +788,7 @@ def test_moe_full_size_c5_one_projection(hip, ref):
         kern.moe_gemm_q8_dev(dw, w[0].nbytes, n_experts, da, doff, rows, int(np.diff(offsets).max()), dy, n, k_, ws)
         torch.cuda.synchronize()
         y = dy.cpu().numpy()
-        for r in range(0, rows, 9):
+        for r in range(rows):
             e = int(np.searchsorted(offsets, r, side="right") - 1)
             y_ref = canonical_ref(ref, t, w[e], acts[r], n, k_, threads=16)
             assert_close(y[r], y_ref, f"c5 {n}x{k_} pair row {r} expert {e}")
