@@ -385,7 +385,7 @@ def want_all(ref, layer, router, wg, wu, wd, xt):
 
 def test_moe_layer_full_size_c5(hip, ref):
     """The whole layer at the C5 size (IQ4_XS, 8 experts of 14336 x 4096 / 4096 x 14336, 64 tokens, top-2): routing
-    exact for every token; for three tokens the layer's output against the oracle's MoeFfn::forward on quantized
+    exact for every token; for every token the layer's output against the oracle's MoeFfn::forward on quantized
     experts (end-to-end bar), and the size-independent property that the weights of a token sum to one."""
     n_exp, top_k, n_tok, hidden, inter = 8, 2, 64, 4096, 14336
     t = O.IQ4_XS
@@ -410,8 +410,9 @@ def test_moe_layer_full_size_c5(hip, ref):
                     d["pair_token"], d["token_rows"], d["weights"], 0, d_out, hidden, inter, ws)
     got = host(d_out).reshape(n_tok, hidden)
     assert np.all(np.isfinite(got))
-    for tk in (0, 31, 63):
-        say("moe layer C5 full size: oracle token", tk)
+    for tk in range(n_tok):  # every token (threaded oracle matvecs: a few seconds)
+        if tk % 16 == 0:
+            say("moe layer C5 full size: oracle token", tk)
         xt = x[tk * hidden:(tk + 1) * hidden]
         xq = ref.quantize_q8_0(xt)
         acc = np.zeros(hidden, np.float32)
