@@ -18,9 +18,16 @@ template <class F> struct phase_probe_format {
                                   F::TYPE_ID == OXQ_TYPE_Q4_0;
 };
 
+// A launch over at most this many weight bytes is "small": it ends within a few microseconds, most of which are the
+// ramp of its waves, and runs faster on fewer, longer-lived waves (measured on MI355X at 4096 x 4096 and 6144 x 4096:
+// 3-7 % faster with one work group per compute unit than with two; from 14336 x 4096 on the wider launch wins).
+constexpr uint64_t SMALL_LAUNCH_BYTES = 28ull << 20;
+
 template <class F>
-static uint32_t launch_width(const GemvArgs &a) {
-    return a.waves_per_cu ? a.waves_per_cu : format_waves_per_cu<F>::value;
+static uint32_t launch_width(const GemvArgs &a, uint64_t weight_bytes) {
+    if (a.waves_per_cu) return a.waves_per_cu;
+    const uint32_t w = format_waves_per_cu<F>::value;
+    return weight_bytes <= SMALL_LAUNCH_BYTES && w > 4 ? 4 : w;
 }
 
 template <class F, class SRC, int STEPS, int RB, int KS, bool DUMP>
@@ -46,7 +53,9 @@ static hipError_t launch_cached_src(const GemvArgs &a, uint32_t units, uint32_t 
     uint64_t total_rows = 0;
     for (uint32_t i = 0; i < n_mats; i++) total_rows += rows[i < 4 ? i : 0];
     // each matrix gets gridDim.x work groups, sized so that the whole launch fills the chip once
-    uint32_t max_groups = (uint32_t)((uint64_t)(device_cus() * launch_width<F>(a) / KS) * max_rows / (total_rows ? total_rows : 1));
+    // (several matrices in one launch keep the format's width: not measured otherwise)
+    const uint32_t width = launch_width<F>(a, n_mats == 1 ? total_rows * row_bytes : ~0ull);
+    uint32_t max_groups = (uint32_t)((uint64_t)(device_cus() * width / KS) * max_rows / (total_rows ? total_rows : 1));
     if (max_groups == 0) max_groups = 1;
     // Equal share per group: ceil(n_batches / passes) groups, each doing `passes` batches.
     const uint32_t passes = (n_batches + max_groups - 1) / max_groups;
@@ -114,7 +123,12 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     // Rows per batch: two while a wave's slice of a row is at most ~3.4 KB, else one
     // (measured on MI355X: more in flight per wave does not pay beyond that); Q6_K always one.
     uint32_t rb = a.rows_per_batch;
-    if (rb == 0) rb = row_bytes / (ks >= 4 ? 4 : 1) <= F::TWO_ROW_BATCH_BYTES ? 2 : 1;
+    if (rb == 0) {
+        const size_t slice = row_bytes / (ks >= 4 ? 4 : 1);
+        // a small launch (few trips per wave) keeps two rows in flight up to a slightly longer slice: Q8_0 at 4096 columns
+        const bool small = (uint64_t)a.n_rows * row_bytes <= SMALL_LAUNCH_BYTES && a.n_mats <= 1 && !a.group_offsets;
+        rb = slice <= F::TWO_ROW_BATCH_BYTES || (small && slice <= 4400) ? 2 : 1;
+    }
     // Q8_0 activations and a row that ends inside a block: the kernel that masks the activations
     const bool ragged_q8 = a.n_cols % F::BLOCK_COLS != 0 && !a.X;
     if (ks >= 4 && steps <= 32 && !ragged_q8) {
@@ -139,7 +153,7 @@ static hipError_t launch_format(const GemvArgs &a, uint32_t group_cols, hipStrea
     default: break;
     }
     if (a.X || a.group_offsets) return hipErrorNotSupported;  // rows this long re-read the activations: Q8_0 blocks only
-    const uint32_t max_waves = device_cus() * launch_width<F>(a);
+    const uint32_t max_waves = device_cus() * launch_width<F>(a, ~0ull);
     uint32_t waves = a.n_rows < max_waves ? a.n_rows : max_waves;
     uint32_t blocks = (waves + 3) / 4;
     if (blocks == 0) blocks = 1;
