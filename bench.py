@@ -912,15 +912,29 @@ def main():
                 print("bench.py: PARITY GATE FAILED: " + json.dumps(parity), file=sys.stderr, flush=True)
 
         if args.f32_route:
-            # the reference's other method on the CPU: gemv on unquantized fp32 activations (the scalar restatement of
-            # Q/reference/q4_k.rs:135-178; one thread, one call of ffn_gate) beside the GPU's f32_route_* legs
-            t_begin = time.perf_counter()
-            O.gemv(O.Q4_K, hw["gate"], F, H, hx)
-            el = time.perf_counter() - t_begin
+            # the reference's other method on the CPU: gemv on unquantized fp32 activations, one call of ffn_gate,
+            # beside the GPU's f32_route_* legs.  Where the host has AVX-512F: the intrinsics twin of the reference's
+            # AVX-512 row (Q/simd/avx512/q4_k.rs:279-415) on `cores` threads, best of a few calls; else the scalar
+            # restatement (Q/reference/q4_k.rs:135-178) on one thread.
+            if O.load_avx512() is not None:
+                O.avx512_gemv_q4_k(hw["gate"], hx, F, H, threads=cores)
+                el, reps = 1e9, 0
+                t_stop = time.perf_counter() + 3.0
+                while time.perf_counter() < t_stop:
+                    t_begin = time.perf_counter()
+                    O.avx512_gemv_q4_k(hw["gate"], hx, F, H, threads=cores)
+                    el = min(el, time.perf_counter() - t_begin)
+                    reps += 1
+                used, what = cores, f"AVX-512 twin of the reference's gemv row, {cores} threads (static row split), best of {reps} calls (the 33 MB matrix stays in the host's caches between them)"
+            else:
+                t_begin = time.perf_counter()
+                O.gemv(O.Q4_K, hw["gate"], F, H, hx)
+                el = time.perf_counter() - t_begin
+                used, what = 1, "scalar C restatement on one host thread, one call"
             kernels["f32_route_cpu_q4k_gate_14336x4096"] = {
                 "us_per_call": round(el * 1e6, 1), "launches": 1, "distinct_weight_sets": 1,
-                "weight_GBps": round(F * row_bytes(Q4_K, H) / el / 1e9, 3), "frac_hbm_peak": None, "cores": 1,
-                "kind": "port", "sample": "one gemv of ffn_gate 14336x4096 on one host thread (scalar C restatement)"}
+                "weight_GBps": round(F * row_bytes(Q4_K, H) / el / 1e9, 3), "frac_hbm_peak": None, "cores": used,
+                "kind": "port", "sample": "gemv of ffn_gate 14336x4096 on fp32 activations: " + what}
         s_mt, n_mt = time_cpu(cores, 8.0)
         s_1t, n_1t = time_cpu(1, 8.0)
         cpu = {"value": round(step_weight_bytes / s_mt / 1e9, 3), "unit": "GB/s", "cores": cores, "host_cores": host_cores,

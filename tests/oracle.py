@@ -87,6 +87,37 @@ def avx2_matvec_q8_fused(t, w, acts, n_rows, n_cols, threads=1, out=None):
     return out[:n_rows]
 
 
+_avx512 = None
+AVX512_PATH = os.path.join(ORACLE_DIR, "liboxq_cpu_avx512.so")
+
+
+def load_avx512():
+    """AVX-512 intrinsics twin of the reference's fp32-activation gemv for Q4_K (CPU baseline of that route);
+    None when the host CPU lacks AVX-512F."""
+    global _avx512
+    if _avx512 is not None:
+        return _avx512
+    if not (host_has("avx512f") and host_has("fma") and host_has("f16c")):
+        return None
+    if not os.path.exists(AVX512_PATH):
+        subprocess.run(["make", "-C", ORACLE_DIR, "-s", "liboxq_cpu_avx512.so"], check=True)
+    lib = C.CDLL(AVX512_PATH)
+    lib.oxq_avx512_gemv_q4_k.restype = C.c_int
+    lib.oxq_avx512_gemv_q4_k.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_int]
+    _avx512 = lib
+    return lib
+
+
+def avx512_gemv_q4_k(w, x, n_rows, n_cols, threads=1):
+    lib = load_avx512()
+    w = _u8(w)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.zeros(max(n_rows, 1), dtype=np.float32)
+    if lib.oxq_avx512_gemv_q4_k(_p(w), _p(x), _p(out), n_rows, n_cols, threads) != 0:
+        raise ValueError("partial block")
+    return out[:n_rows]
+
+
 def load():
     global _lib
     if _lib is not None:

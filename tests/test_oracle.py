@@ -537,3 +537,25 @@ def test_avx2_twin_is_bit_identical_to_the_avx2_tier_restatement(ref, t):
     want = ref.matvec_q8_fused(t, w, a, n_rows, n_cols, tier=O.TIER_AVX2)
     assert np.array_equal(ref.avx2_matvec_q8_fused(t, w, a, n_rows, n_cols, threads=1), want)
     assert np.array_equal(ref.avx2_matvec_q8_fused(t, w, a, n_rows, n_cols, threads=3), want)
+
+
+def test_avx512_twin_of_the_f32_gemv_matches_the_scalar_restatement(ref):
+    """The AVX-512 twin timed as the CPU figure of the fp32-activation route (Q/simd/avx512/q4_k.rs:279-415) against the
+    scalar gemv (Q/reference/q4_k.rs:135-178): sixteen partial sums and a fused multiply-subtract instead of one chain,
+    so within 1e-5 of the largest |y|, not bit for bit; threads split rows and change nothing.  A dequantized dot
+    product in float64 bounds both from the other side (a wrong nibble order or scale index would be off by far more)."""
+    from oxillama_amd import synth
+    if ref.load_avx512() is None:
+        pytest.skip("host CPU lacks AVX-512F")
+    n_rows, n_cols = 23, 2048
+    w = synth.weights(O.Q4_K, 97, n_rows, n_cols)
+    x = synth.normal_f32(98, n_cols)
+    want = ref.gemv(O.Q4_K, w, n_rows, n_cols, x)
+    got = ref.avx512_gemv_q4_k(w, x, n_rows, n_cols, threads=1)
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    assert np.array_equal(ref.avx512_gemv_q4_k(w, x, n_rows, n_cols, threads=3), got)
+    deq = ref.dequant_rows(O.Q4_K, w, n_rows, n_cols).astype(np.float64)
+    exact = deq @ x.astype(np.float64)
+    assert np.abs(got - exact).max() <= 1e-5 * np.abs(exact).max()
+    with pytest.raises(ValueError):
+        ref.avx512_gemv_q4_k(w, x, n_rows, 2000)
