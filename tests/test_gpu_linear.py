@@ -422,7 +422,8 @@ def test_ffn_swiglu_errors(hip):
 
 def test_topk_matches_oracle(hip, ref):
     rng = np.random.default_rng(21)
-    for n, ks in ((128256, (1, 40, 256)), (1000, (1, 7, 256)), (5, (1, 5)), (300000, (2, 50)), (1 << 20, (1, 64))):
+    for n, ks in ((128256, (1, 40, 256)), (1000, (1, 7, 256)), (5, (1, 5)), (300000, (2, 50)), (1 << 20, (1, 64)),
+                  (151936, (1, 40, 64)), (262144, (40,)), (4097, (3, 64))):
         v = (rng.standard_normal(n) * 3).astype(np.float32)
         if n > 2000:
             v[1000:1010] = v[17]          # exact ties across and inside slices
