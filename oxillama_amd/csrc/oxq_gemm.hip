@@ -69,7 +69,8 @@ static size_t gemm_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t
 // The same for the grouped form, which splits k in two where an expert's matrix has few row groups: a function of
 // (type, rows, n, k) only, as the caller sizes the workspace without the number of experts.
 static size_t gemm_grouped_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
-    if ((type != OXQ_TYPE_Q4_K && type != OXQ_TYPE_IQ4_XS && type != OXQ_TYPE_Q4_0) || k % 1024 != 0 || n == 0 ||
+    if ((type != OXQ_TYPE_Q4_K && type != OXQ_TYPE_IQ4_XS && type != OXQ_TYPE_Q4_0 && type != OXQ_TYPE_Q6_K &&
+         type != OXQ_TYPE_Q8_0) || k % 1024 != 0 || n == 0 ||
         n > SKINNY_GROUPED_SPLIT_MAX_N)
         return 0;
     const size_t bytes = (size_t)2 * m * n * sizeof(float);

@@ -637,7 +637,9 @@ void gemm_skinny_kernel(
     }
     // blockIdx.z = which 16 * TT token rows of the group: the launch is shaped for the usual group, a larger one
     // takes further work groups per row group (each its own pass over the weights); the rest exit here
-    const uint32_t tokb = tok0 + blockIdx.z * (16 * TT);
+    // (the last pass is dispatched first: the few work groups of the groups that overflow run beside the first pass
+    // instead of after it)
+    const uint32_t tokb = tok0 + (gridDim.z - 1 - blockIdx.z) * (16 * TT);
     if (tokb >= tok_end) return;  // the whole work group
     if constexpr (TT == 2) {
         if (tok_end - tokb <= 16) {
@@ -772,7 +774,7 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
         if (a.k % 512 != 0 || rows > 32) return SK_NONE;
         const bool two = rows > 16;
         // the formats with the long strips: the one-tile shapes only (see launch_skinny)
-        if (Skinny<F>::ONE_TILE && (two || (variant != 0 && variant != 200))) return SK_NONE;
+        if (Skinny<F>::ONE_TILE && variant != 0 && variant != 200) return SK_NONE;
         if (a.sums && variant != 0 && variant != 200) return SK_NONE;  // the dump exists for the default shapes
         switch (variant) {
         case 0: {
@@ -786,6 +788,20 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
             const bool many = (size_t)((a.n + 127) / 128) * a.n_experts >= 2 * (size_t)device_cus();
             // two token tiles: only with many row groups and a mean of at most 16 rows per expert
             if (two) {
+                // one tile per work group: a group of 17..32 rows takes a second pass over its expert's weights (the
+                // launch's second layer of work groups; those of the smaller groups exit at once).  8 experts of
+                // 14336 x 4096, 11..23 rows: Q6_K 152 us, Q8_0 155 against 195 / 227 on the tile kernel; a pass costs
+                // 117 / 8 us per expert, so up to a mean of 17 rows (two passes for about half the experts).
+                if (Skinny<F>::ONE_TILE) {
+                    if ((size_t)a.m > 17 * (size_t)a.n_experts) return SK_NONE;
+                    if (many) return SK_1_4;
+                    // few row groups per expert (one work group per compute unit in the first pass): the second
+                    // pass's work groups would double up on some compute units and set the time; with each expert's
+                    // k in two halves the launch spreads evenly
+                    const bool can_split = has_partial && a.n <= SKINNY_GROUPED_SPLIT_MAX_N && a.k % 1024 == 0 &&
+                                           (size_t)((a.n + 127) / 128) * a.n_experts * SKINNY_GROUPED_SPLITS >= device_cus();
+                    return can_split ? SK_1_4_SPLIT : SK_1_8;
+                }
                 if ((size_t)a.m > 16 * (size_t)a.n_experts) return SK_NONE;
                 if (many) return SK_2_2;
                 // few row groups per expert: each expert's k in two halves, where that gives every compute unit a
@@ -794,10 +810,13 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
                                        (size_t)((a.n + 127) / 128) * a.n_experts * SKINNY_GROUPED_SPLITS >= device_cus();
                 return can_split ? SK_2_2_SPLIT : SK_NONE;
             }
+            if (Skinny<F>::ONE_TILE && !many && has_partial && a.n <= SKINNY_GROUPED_SPLIT_MAX_N && a.k % 1024 == 0 &&
+                (size_t)((a.n + 127) / 128) * a.n_experts * SKINNY_GROUPED_SPLITS >= device_cus())
+                return SK_1_4_SPLIT;
             // (the debug dump: one shape per token-tile count; every shape adds a result's terms in the same order)
             return (many || a.sums) ? SK_1_4 : SK_1_8;
         }
-        case 200: return two ? SK_2_2 : SK_1_4;
+        case 200: return two && !Skinny<F>::ONE_TILE ? SK_2_2 : SK_1_4;
         case 201: return two ? SK_2_8 : SK_1_16;
         case 203: return two ? SK_W4_2_4 : SK_W4_1_8;
         case 204: return two ? SK_2_2 : SK_1_4;

@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 
 FORMATS = [O.Q4_K, O.IQ4_XS, O.Q4_0]
 # Q6_K (a scale per 16 weights: two MFMAs per sub-block, the integer sums per half) and Q8_0 (544 bytes of a row per
-# step): the kernel's one-token-tile shapes only
+# step): the kernel's one-token-tile shapes only; expert groups of more than 16 rows take further passes
 ONE_TILE = [O.Q6_K, O.Q8_0]
 FORMATS_1TILE = FORMATS + ONE_TILE
 
@@ -99,6 +99,8 @@ CASES = [
     # launch (one step per half; several chunks per half and groups of unknown size)
     ([20, 3, 17, 0, 32, 16, 9, 25], 2048, 1024, 32),
     ([22, 10, 17, 13, 20, 16, 9, 15], 4096, 3072, 0),
+    # one token tile on few row groups per expert (Q6_K, Q8_0: k in two halves there as well)
+    ([16, 5, 0, 9, 12, 1, 16, 7], 2048, 2048, 16),
 ]
 
 
@@ -107,8 +109,7 @@ CASES = [
 def test_skinny_grouped_against_oracle(hip, ref, t, case):
     counts, n, k_, max_rows = case
     say("skinny", O.NAMES[t], case)
-    if t in ONE_TILE and shaped_rows(counts, max_rows) > 16:
-        pytest.skip("two token tiles: the tile kernel's case for this format")
+    # (Q6_K, Q8_0 shaped for 17..32 rows: the one-tile kernel, a second pass over the weights for the larger groups)
     offsets, acts, w = _case(ref, t, counts, n, k_, 4100 + n + k_)
     rows = int(offsets[-1])
     dy, dsum = _run(hip, t, w, acts, offsets, n, k_, max_rows, sums=True)
