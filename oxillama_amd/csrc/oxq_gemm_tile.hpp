@@ -852,7 +852,13 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
             // IQ4_XS 107 against 118, Q6_K 168 against 189; 2048 tokens: Q8_0 388 against 503.  Q4_K, whose weight
             // loads are the lightest per MFMA, is the exception (114 against 111) and keeps 64 x 64.
             constexpr bool wide = F::TYPE != OXQ_TYPE_Q4_K;
-            if (2 * wgs >= 3 * (size_t)device_cus())
+            // ... or where the 128 x 64 tiles below would come to between one and two per compute unit: a compute unit
+            // with two of them takes twice as long as one with one, so 129..256 of the larger tiles, one per compute
+            // unit, finish first (4096 x 14336, 768 tokens: Q8_0 248 us against 348, Q6_K 339 against 397, Q4_K 228
+            // against 266; 1024 tokens Q6_K 368 against 421)
+            const size_t cus = device_cus();
+            // (Q4_K on rows of 4096 columns is the exception: 4096 x 4096, 768 / 1024 tokens 72 / 77 us against 76 / 82)
+            if (2 * wgs >= 3 * cus || (2 * wgs > cus && wgs <= cus && (wide || a.k >= 8192)))
                 return wide ? launch_tile<F, 4, 1, 1, 1, false>(a, p, stream) : launch_tile<F, 2, 2, 2, 2, false>(a, p, stream);
             // one to one and a half work groups per compute unit: still the better shape for the formats of a
             // byte and more per weight (512 x 8192 x 8192 Q8_0: 149 us against 180)
