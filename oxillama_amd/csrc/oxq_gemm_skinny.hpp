@@ -785,7 +785,12 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
             if (!a.offsets) {
                 // one matrix, up to 16 token rows: enough row groups by themselves (a vocabulary projection), or k
                 // split over work groups (the workspace has room for the sums)
-                if (two) return SK_NONE;
+                if (two) {
+                    // 17..32 token rows: only where the tile kernel's 32 x 32 tiles leave half the chip idle (fewer
+                    // than 8192 weight rows) and k is long enough to split
+                    if (a.n >= 8192 || !has_partial || skinny_splits(a.n, a.k) < 2) return SK_NONE;
+                    return Skinny<F>::ONE_TILE ? SK_1_4_SPLIT : SK_2_2_SPLIT;
+                }
                 if ((size_t)((a.n + 127) / 128) >= 2 * (size_t)device_cus()) return SK_1_4;
                 return (has_partial && skinny_splits(a.n, a.k) >= 2) ? SK_1_4_SPLIT : SK_NONE;
             }

@@ -192,10 +192,12 @@ def test_skinny_full_size_c5_gate(hip, ref):
 
 
 @pytest.mark.parametrize("t", FORMATS_1TILE, ids=lambda t: O.NAMES[t])
-@pytest.mark.parametrize("shape", [(16, 4096, 8192), (9, 8200, 4096), (6, 16384, 2048), (13, 2100, 16384), (11, 16384, 3584), (7, 8201, 4096)],
+@pytest.mark.parametrize("shape", [(16, 4096, 8192), (9, 8200, 4096), (6, 16384, 2048), (13, 2100, 16384), (11, 16384, 3584), (7, 8201, 4096),
+                                   # 17..32 rows on fewer than 8192 weight rows: two token tiles (Q6_K, Q8_0: two passes)
+                                   (21, 4096, 8192), (32, 2100, 16384), (17, 4100, 8192)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_skinny_one_matrix_split_k(hip, ref, t, shape):
-    """One matrix, up to 16 token rows, at least 2^25 weights: k is split over work groups, each writes its sums for its
+    """One matrix, up to 16 token rows (32 on fewer than 8192 weight rows), at least 2^25 weights: k is split over work groups, each writes its sums for its
     part of k, a second launch adds the parts in index order.  Integer sums ==, fp32 1e-5, bias, accumulate, ragged n,
     splits of unequal length."""
     import torch
