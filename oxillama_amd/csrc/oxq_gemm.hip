@@ -106,8 +106,9 @@ std::atomic<uint32_t> g_gemm_tile_min_rows{0};  // tuning: 0 = default
 
 // The tile kernel can take this format and shape at all.
 bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
-    // LDS holds the f16 token scales of up to 128 tokens for the whole k (k/32 * 256 bytes)
-    // beside up to 24 KB of decoded weight scales; up to k = 8192 two work groups share a CU
+    // LDS holds the f16 token scales of a work group's tokens for the whole k (k/32 * 2 bytes per token) beside up
+    // to 24 KB of decoded weight scales: 128-token tiles up to k = 16384, 64-token tiles up to 32768, 32-token tiles
+    // up to 65536 (launch_tiles picks among them); up to k = 8192 two work groups of 128 tokens share a CU
     const bool known = type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K ||
                        type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q5_K || type == OXQ_TYPE_Q4_1 ||
                        type == OXQ_TYPE_IQ4_NL || type == OXQ_TYPE_Q8_1 || type == OXQ_TYPE_Q5_0 || type == OXQ_TYPE_Q5_1 ||
@@ -117,7 +118,7 @@ bool gemm_tiles_supported(uint32_t type, uint32_t m, uint32_t k) {
     const bool blocks32 = type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q4_1 ||
                           type == OXQ_TYPE_IQ4_NL || type == OXQ_TYPE_Q8_1 || type == OXQ_TYPE_Q5_0 || type == OXQ_TYPE_Q5_1;
     const bool whole = k % 256 == 0 || (blocks32 && k % 32 == 0 && k >= 256);
-    return known && whole && m >= 1 && (size_t)tile_padded_sub_blocks(k) * 256 <= 128 * 1024 &&
+    return known && whole && m >= 1 && (size_t)tile_padded_sub_blocks(k) * 64 <= 128 * 1024 &&
            gemm_planes_bytes(m, k) < 0x7FFFFFFFull;
 }
 

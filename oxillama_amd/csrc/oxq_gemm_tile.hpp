@@ -804,19 +804,26 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
     const int variant = g_gemm_variant.load(std::memory_order_relaxed);
     (void)variant;  // (read by the fixed-shape knobs, which the second translation unit leaves out)
-    // 65..384 tokens: 64 x 128 tiles (a wave per 32 weight rows) where they give the chip 1.75 work groups per compute
+    // The f16 token scales of a work group's tokens for the whole k sit in LDS (k / 32 * 2 bytes per token): 128-token
+    // tiles up to k = 16384, 64-token tiles up to 32768, 32-token tiles beyond (up to 65536).
+    const uint32_t nsb_pad = tile_padded_sub_blocks(a.k);
+    const bool fits128 = (size_t)nsb_pad * 256 <= 128 * 1024, fits64 = (size_t)nsb_pad * 128 <= 128 * 1024;
+    const bool big = rows > 384 && fits128;
+    const bool mid = !big && rows > 64 && fits64;
+    // 65..384 tokens (more where k is too long for the 128-token tiles): 64 x 128 tiles (a wave per 32 weight rows)
+    // where they give the chip 1.75 work groups per compute
     // unit, else 64 x 32 tiles whose four waves split k -- four times the work groups.  Measured (us, the first
     // against the second): 4096 x 14336, 128 / 256 / 384 tokens, Q4_K 131 / 136 / 143 against 47 / 87 / 127, Q6_K
     // 196 / 198 / 206 against 66 / 125 / 183; 4096 x 4096 Q4_K 44 / 45 / 48 against 19 / 27 / 37, Q8_0 51 / 51 / 54
     // against 21 / 33 / 46; 14336 x 4096 Q4_K 128 / 192 tokens 49 / 70 against 45 / 63, 256 a tie, 384 108 against 113.
-    const bool mid_split_k = rows > 64 && rows <= 384 &&
-                             (size_t)((rows + 63) / 64) * ((a.n + 127) / 128) * (a.offsets ? a.n_experts : 1) * 4 < 7 * (size_t)device_cus();
+    const bool mid_split_k = mid && (size_t)((rows + 63) / 64) * ((a.n + 127) / 128) * (a.offsets ? a.n_experts : 1) * 4 <
+                                        7 * (size_t)device_cus();
     if (a.sums)  // debug dump: the same tile layout (and fp32 summation order) as the production choice below
-        return rows > 384  ? launch_tile<F, 2, 1, 2, 1, true>(a, p, stream)
-               : rows > 64 ? (mid_split_k ? launch_tile<F, 2, 1, 0, 2, true, 2, 2>(a, p, stream)
-                                          : launch_tile<F, 2, 1, 1, 2, true>(a, p, stream))
-               : rows > 32 ? launch_tile<F, 2, 1, 0, 2, true, 2, 2>(a, p, stream)
-                           : launch_tile<F, 1, 2, 0, 2, true, 2, 2>(a, p, stream);
+        return big   ? launch_tile<F, 2, 1, 2, 1, true>(a, p, stream)
+               : mid ? (mid_split_k ? launch_tile<F, 2, 1, 0, 2, true, 2, 2>(a, p, stream)
+                                    : launch_tile<F, 2, 1, 1, 2, true>(a, p, stream))
+               : (rows > 32 && fits64) ? launch_tile<F, 2, 1, 0, 2, true, 2, 2>(a, p, stream)
+                                       : launch_tile<F, 1, 2, 0, 2, true, 2, 2>(a, p, stream);
 #ifndef OXQ_TILE_DEFAULT_SHAPES_ONLY
     switch (variant) {
     case 1: return launch_tile<F, 2, 1, 2, 1, false>(a, p, stream);
@@ -841,7 +848,7 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
         // tokens the four waves of a work group share one tile and split k (most work groups, shortest
         // dependency chain per wave); up to 384 tokens 64 x 128 tiles (64 x 32 with k split where those are too
         // few); beyond that 128 x 64 tiles at three waves per SIMD.
-        if (rows > 384) {
+        if (big) {
             // 128 x 128 tiles (two waves per SIMD, weight bytes fetched two steps ahead) where they still give the
             // chip one and a half work groups per compute unit: 14336 x 4096, 512 tokens 123 us against 125 us,
             // 2048 tokens 383 us against 422 us; 4096 x 14336 has too few such tiles (214 us against 140 us)
@@ -865,18 +872,19 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
             if (wide && F::BLOCK_BYTES >= 256 && wgs >= (size_t)device_cus()) return launch_tile<F, 4, 1, 1, 1, false>(a, p, stream);
             return launch_tile<F, 2, 1, 2, 1, false, 3>(a, p, stream);
         }
-        if (rows > 64)
+        if (mid)
             return mid_split_k ? launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream) : launch_tile<F, 2, 1, 1, 2, false>(a, p, stream);
         // split k; 64 weight rows (or 64 tokens) per work group only where that still leaves every
         // compute unit at least one work group, else 32 x 32
         const size_t groups = a.offsets ? a.n_experts : 1;
         // 33..64 tokens: one 64-token tile where 32-row tiles still give every compute unit a work group
         // (14336 x 4096, 64 rows: 26.6 us against 31.1 with 32 x 32 tiles; 4096 rows: 61 against 50)
-        if (rows > 32 && (size_t)((a.n + 31) / 32) * groups >= device_cus())
+        if (rows > 32 && fits64 && (size_t)((a.n + 31) / 32) * groups >= device_cus())
             return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
         if ((size_t)((a.n + 63) / 64) * groups < device_cus())
             return launch_tile<F, 1, 1, 0, 2, false, 2, 2>(a, p, stream);
-        if (rows > 32) return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
+        if (rows > 32 && fits64) return launch_tile<F, 2, 1, 0, 2, false, 2, 2>(a, p, stream);
+        // (also: any number of tokens on rows of more than 32768 columns)
         return launch_tile<F, 1, 2, 0, 2, false, 2, 2>(a, p, stream);
     }
 }

@@ -597,6 +597,20 @@ def test_prefill_many_tokens_takes_the_wide_tile_shape(hip, ref, t):
         assert torch.equal(dy2, dy[:m])
 
 
+@pytest.mark.parametrize("shape", [(40, 40, 28672), (100, 72, 17408), (400, 40, 28672), (70, 33, 36864), (400, 36, 36864),
+                                   (9, 48, 65536)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("t", O.ALL_TYPES, ids=lambda t: O.NAMES[t])
+def test_prefill_tile_kernel_long_rows(hip, ref, tuning, shape, t):
+    """Rows of more than 16384 columns (the down projections of the large models: 17408, 28672, ...): the token scales of
+    a 128-token tile for the whole row no longer fit LDS, and the library takes 64-token tiles (up to 32768 columns) or
+    32-token tiles (up to 65536) instead of falling back to one GEMV launch per four rows.  Same checks as above."""
+    from test_gpu_prefill_f16 import last_launch
+    say("prefill, long rows", O.NAMES[t], shape)
+    tuning("gemm_tile_min_rows", 1)
+    _prefill_tile_case(hip, ref, shape, t)
+    assert last_launch().startswith("gemm_tile_kernel"), last_launch()  # (the last call there is the sums' dump)
+
+
 BLOCKS32 = [t for t in O.ALL_TYPES if O.BLOCK[t][0] == 32]
 
 
