@@ -142,8 +142,11 @@ bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
 bool gemm_few_rows_pay(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
     if (g_gemm_tile_min_rows.load(std::memory_order_relaxed) != 0 || g_gemm_variant.load(std::memory_order_relaxed) != 0)
         return false;
+    // from 5 rows (a second GEMV pass); from 3 where a GEMV launch takes two vectors at most (rows of two or of five
+    // to eight 64-lane steps: IQ4_XS and the 32-weight formats at 4096 columns, everything at 8192 and beyond --
+    // Q4_K 28672 x 8192 3 / 4 rows 52.6 / 56.7 against 38.4 / 38.8, Q8_0 14336 x 4096 24.1 / 25.6 against 21.6 / 22.0)
     return gemm_tiles_supported(type, m, k) && gemm_partial_bytes(type, m, n, k) != 0 &&
-           m >= (type == OXQ_TYPE_IQ4_XS ? 3u : 5u);
+           m >= (gemv_vecs_max(type, k) <= 2 ? 3u : 5u);
 }
 
 // Expert groups with at most this many token rows in all: one GEMV launch, a matvec per row against its expert's

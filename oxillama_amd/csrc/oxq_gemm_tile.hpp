@@ -801,7 +801,18 @@ static hipError_t launch_tile(const GemmArgs &a, const TilePlan &p, hipStream_t 
 // weight bytes fetched further ahead, because that case is paced by the weight stream.
 template <class F>
 static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t stream) {
-    const uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
+    uint32_t rows = a.offsets ? (a.shape_rows ? a.shape_rows : a.max_rows) : a.m;
+    // Expert groups whose sizes only the device knows (the launch is shaped for twice the mean, the grid covers the
+    // worst case): the tile follows the mean -- a larger group takes more tiles, while a tile twice the usual group
+    // is half empty everywhere.  8 experts of 14336 x 4096 / 4096 x 14336, IQ4_XS, 12..25 rows each: 108 / 108 us on
+    // 32-token tiles against 152 / 164 on 64-token ones; 24..42 rows 136 / 140 against 155 / 167; 38..63 rows on
+    // 64 x 32 split-k tiles 163 / 172 against 159 / 258 on 64 x 128.
+    // (a mean of 49..64 rows spills over 64 in half the groups: the shapes for 65 rows and more; 256 tokens on those
+    // experts 743 us per layer against 781)
+    if (a.offsets && a.n_experts && a.shape_rows && a.shape_rows < a.max_rows) {
+        const uint32_t mean = (a.m + a.n_experts - 1) / a.n_experts;
+        rows = mean > 48 && mean < 65 ? 65 : mean;
+    }
     const int variant = g_gemm_variant.load(std::memory_order_relaxed);
     (void)variant;  // (read by the fixed-shape knobs, which the second translation unit leaves out)
     // The f16 token scales of a work group's tokens for the whole k sit in LDS (k / 32 * 2 bytes per token): 128-token

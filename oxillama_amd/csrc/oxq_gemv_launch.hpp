@@ -243,6 +243,7 @@ static hipError_t launch_vecs_k(const GemvVecsArgs &a, uint32_t units, size_t ro
     const uint32_t groups = (n_batches + passes - 1) / passes;
     uint32_t blocks = (groups + G - 1) / G;
     if (blocks == 0) blocks = 1;
+    note_launch("gemv_q8_vecs", F::TYPE_ID, STEPS, KS, NV, RB, blocks, 1, 256);
     hipLaunchKernelGGL((gemv_q8_vecs<F, STEPS, KS, NV, RB>), dim3(blocks), dim3(256), 0, stream, a.W, a.A, a.a_stride,
                        a.out, a.out_stride, a.n_rows, units, row_bytes, a.accumulate, a.n_vecs, a.bias);
     return hipGetLastError();

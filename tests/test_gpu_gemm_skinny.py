@@ -292,7 +292,7 @@ def test_skinny_split_k_on_the_host_routes(hip, ref):
                          ids=lambda c: "%s_m%d_%dx%d" % (O.NAMES[c[0]], c[1], c[2], c[3]))
 def test_few_rows_take_the_few_token_kernel_when_a_workspace_has_room(hip, ref, case):
     """Below the tile kernel's row threshold the GEMV launches serve a matmul, four rows per pass -- except where the
-    few-token kernel is faster still (IQ4_XS from 3 rows, Q4_K and Q6_K from 5, on shapes it splits over k) and the caller's
+    few-token kernel is faster still (from 3 rows where a GEMV launch takes two vectors at most, else from 5, on shapes it splits over k) and the caller's
     workspace has room for its sums.  Without a workspace, or with a small one, the GEMV launches stay."""
     import torch
     t, m, n, k_ = case
@@ -301,7 +301,9 @@ def test_few_rows_take_the_few_token_kernel_when_a_workspace_has_room(hip, ref, 
     kern = hip.HipKernel(t)
     dw, da = torch.from_numpy(w).cuda(), torch.from_numpy(acts).cuda()
     ws = torch.empty(kern.gemm_workspace_bytes(m, n, k_), dtype=torch.uint8, device="cuda")
-    expect_skinny = (t == O.IQ4_XS and m >= 3) or (t in (O.Q4_K, O.Q6_K) and m >= 5)
+    # from 3 rows where a GEMV launch takes at most two vectors (rows of 2 or 5..8 steps of 64 lanes), else from 5
+    steps = -(-(k_ // (32 if t == O.IQ4_XS else 64)) // 64)
+    expect_skinny = m >= (5 if steps in (1, 3, 4) else 3)
     outs = []
     for workspace in (ws, ws[:4096], None):
         dy = torch.zeros((m, n), dtype=torch.float32, device="cuda")
