@@ -101,6 +101,8 @@ CASES = [
     ([22, 10, 17, 13, 20, 16, 9, 15], 4096, 3072, 0),
     # one token tile on few row groups per expert (Q6_K, Q8_0: k in two halves there as well)
     ([16, 5, 0, 9, 12, 1, 16, 7], 2048, 2048, 16),
+    # a mean of 17 rows, sizes unknown to the host: shaped for twice that, more than two token tiles hold
+    ([25, 18, 19, 16, 12, 21, 10, 15], 8192, 1024, 0),
 ]
 
 
