@@ -130,7 +130,8 @@ bool gemm_uses_tiles(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
     const uint32_t knob = g_gemm_tile_min_rows.load(std::memory_order_relaxed);
     // (GEMV launches of four rows per pass against the tile kernel, us: 4096 x 4096 Q4_K 6 / 8 rows 13.8 / 16.6 against
     // 12.5, Q8_0 17.5 / 23.0 against 16.9, Q6_K 20.3 / 25.0 against 17.1; 2048 x 4096 9.3 / 10.9 against 12.3)
-    const uint32_t min_rows = knob ? knob : ((n >= 8192 || (uint64_t)n * k >= (1ull << 24)) ? 6 : 9);
+    // 14336 x 4096, 5 rows (two GEMV passes): Q5_K 23.1 against 22.0, Q5_0 32.5 against 28.6, Q2_K 25.3 against 24.0
+    const uint32_t min_rows = knob ? knob : n >= 8192 ? 5 : (uint64_t)n * k >= (1ull << 24) ? 6 : 9;
     return gemm_tiles_supported(type, m, k) && m >= min_rows;
 }
 
