@@ -819,7 +819,13 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     // tiles up to k = 16384, 64-token tiles up to 32768, 32-token tiles beyond (up to 65536).
     const uint32_t nsb_pad = tile_padded_sub_blocks(a.k);
     const bool fits128 = (size_t)nsb_pad * 256 <= 128 * 1024, fits64 = (size_t)nsb_pad * 128 <= 128 * 1024;
-    const bool big = rows > 384 && fits128;
+    // more than 384 tokens on a matrix so narrow that even 128 x 64 tiles leave compute units without one (the key /
+    // value projections of grouped-query attention): the 64 x 32 split-k tiles of the mid range -- 1024 x 4096 at
+    // 512 / 1024 tokens 20.7 / 30.7 us against 45.7 / 49.0, 1024 x 8192 Q8_0 35.7 against 98.9, 3072 x 3072 30.7
+    // against 38.5; from one tile per compute unit on (1024 x 4096, 2048 tokens) a tie
+    const bool narrow = rows > 384 && fits128 &&
+                        (size_t)((rows + 127) / 128) * ((a.n + 63) / 64) * (a.offsets ? a.n_experts : 1) < (size_t)device_cus();
+    const bool big = rows > 384 && fits128 && !narrow;
     const bool mid = !big && rows > 64 && fits64;
     // 65..384 tokens (more where k is too long for the 128-token tiles): 64 x 128 tiles (a wave per 32 weight rows)
     // where they give the chip 1.75 work groups per compute
@@ -827,8 +833,8 @@ static hipError_t launch_tiles(const GemmArgs &a, const TilePlan &p, hipStream_t
     // against the second): 4096 x 14336, 128 / 256 / 384 tokens, Q4_K 131 / 136 / 143 against 47 / 87 / 127, Q6_K
     // 196 / 198 / 206 against 66 / 125 / 183; 4096 x 4096 Q4_K 44 / 45 / 48 against 19 / 27 / 37, Q8_0 51 / 51 / 54
     // against 21 / 33 / 46; 14336 x 4096 Q4_K 128 / 192 tokens 49 / 70 against 45 / 63, 256 a tie, 384 108 against 113.
-    const bool mid_split_k = mid && (size_t)((rows + 63) / 64) * ((a.n + 127) / 128) * (a.offsets ? a.n_experts : 1) * 4 <
-                                        7 * (size_t)device_cus();
+    const bool mid_split_k = mid && (narrow || (size_t)((rows + 63) / 64) * ((a.n + 127) / 128) * (a.offsets ? a.n_experts : 1) * 4 <
+                                                   7 * (size_t)device_cus());
     if (a.sums)  // debug dump: the same tile layout (and fp32 summation order) as the production choice below
         return big   ? launch_tile<F, 2, 1, 2, 1, true>(a, p, stream)
                : mid ? (mid_split_k ? launch_tile<F, 2, 1, 0, 2, true, 2, 2>(a, p, stream)
