@@ -99,7 +99,10 @@ static bool gemm_prefill_pays(uint32_t m, uint32_t n) {
     const uint64_t token_tiles = (m + 127) / 128;
     const uint64_t wgs = token_tiles * ((n + 255) / 256), cus = device_cus();
     const uint64_t rounds = (wgs + cus - 1) / cus;
-    return 100 * wgs >= 85 * rounds * cus && 100 * (uint64_t)m >= 70 * 128 * token_tiles;
+    // (three quarters of a round still pays -- 192 work groups: 4096 x 14336 at 1536 tokens 345 us against 425, 8192 x
+    // 8192 at 768 tokens 205 against 255, 6144 x 4096 at 1024 tokens 111 against 122; 560 of 768: 565 against 606 --
+    // two thirds does not: 336 of 512, 14336 x 4096 at 768 tokens, 204 against 180)
+    return 100 * wgs >= 72 * rounds * cus && 100 * (uint64_t)m >= 70 * 128 * token_tiles;
 }
 
 std::atomic<uint32_t> g_gemm_tile_min_rows{0};  // tuning: 0 = default
