@@ -317,6 +317,7 @@ __device__ __forceinline__ void gemm_skinny_body(
     // super-blocks [sb_lo, n_super) of this work group (all of k, or its split)
     const uint32_t sb_lo = partial ? ks * sb_per_split : 0;
     const uint32_t n_super = partial ? min(k / 256, sb_lo + sb_per_split) : k / 256;
+    const bool odd_super = (n_super & 1) != 0;  // (sb_lo is even: only the end of k can leave half a step)
     constexpr uint32_t per = PER, nblk_max = PER * 8;  // sub-blocks (Q8_0 blocks per token) of a full chunk
     uint8_t *const ldsA = lds;
     float *const ldsD = reinterpret_cast<float *>(ldsA + (size_t)nblk_max * TT * 512);
@@ -351,8 +352,13 @@ __device__ __forceinline__ void gemm_skinny_body(
             const uint32_t cc = l >> 2, qq = l & 3, tok = token_of(t, cc);
             tokA[i] = u32x2{0, 0};
             tokD[i] = 0;
-            if (idx < total && tok < tok_end) {
-                const uint8_t *blk = A + (size_t)tok * arow + (size_t)(sb0 * 8 + b) * Q8_BLOCK_BYTES;
+            // an odd number of super-blocks: the last step's strip holds the last two super-blocks, the one before the
+            // last (done by the step before) in its first half -- that half meets zeros, the second the last one's tokens
+            uint32_t sbi = sb0 + (b >> 3);
+            const bool dead = odd_super && sbi == n_super - 1;
+            if (odd_super && sbi == n_super) sbi = n_super - 1;
+            if (idx < total && tok < tok_end && !dead) {
+                const uint8_t *blk = A + (size_t)tok * arow + (size_t)(sbi * 8 + (b & 7)) * Q8_BLOCK_BYTES;
                 tokA[i] = ld8(blk + 2 + 8 * qq);
                 tokD[i] = ld2(blk);
             }
@@ -390,6 +396,7 @@ __device__ __forceinline__ void gemm_skinny_body(
         }
     };
 
+    const uint32_t steps = (n_super + 1) / 2;
     const uint32_t rbase = (rg * WAVES + wave) * (16 * NT);
     const bool active = rbase < n;  // a wave past the last row still stages tokens and meets the barriers
     const uint8_t *We = W + (offsets ? (size_t)gy * w_stride : 0);
@@ -410,7 +417,7 @@ __device__ __forceinline__ void gemm_skinny_body(
     auto load_step = [&](u32x4 (&stage)[NL], uint32_t st) {
 #pragma unroll
         for (uint32_t j = 0; j < NT; j++) {
-            const uint8_t *sp = src[j] + (size_t)st * SEG;
+            const uint8_t *sp = src[j] + (odd_super && st == steps - 1 ? (size_t)(n_super - 2) * S::BLOCK : (size_t)st * SEG);
 #pragma unroll
             for (uint32_t i = 0; i < ITR; i++) stage[j * ITR + i] = ld16(sp + (i + 1 < ITR ? 64 * i : last_at));
         }
@@ -430,14 +437,15 @@ __device__ __forceinline__ void gemm_skinny_body(
     const uint64_t half_mask = q < 2 ? ~0ull : 0ull;
     u32x4 stage[NL];
     load_step(stage, sb_lo / 2);
-    const uint32_t steps = n_super / 2;
-    load_tokens(sb_lo, min(per, n_super - sb_lo) * 8);
+    // (token blocks are staged by whole steps: an odd last super-block brings a dead one along)
+    auto chunk_blocks = [&](uint32_t from) { return ((min(per, n_super - from) + 1) & ~1u) * 8; };
+    load_tokens(sb_lo, chunk_blocks(sb_lo));
     for (uint32_t sb0 = sb_lo; sb0 < n_super; sb0 += per) {
-    const uint32_t nsbc = min(per, n_super - sb0);
+    const uint32_t nsbc = (min(per, n_super - sb0) + 1) & ~1u;
     __syncthreads();  // every wave is done with the last chunk's tokens
     store_tokens(nsbc * 8);
     __syncthreads();
-    if (sb0 + per < n_super) load_tokens(sb0 + per, min(per, n_super - sb0 - per) * 8);
+    if (sb0 + per < n_super) load_tokens(sb0 + per, chunk_blocks(sb0 + per));
     // The chunk's steps.  One token tile: no branch inside a step, so the LDS reads, the MFMAs and the fmas of
     // different sub-blocks interleave.  Two: each tile's work sits behind a branch on the group's tile count --
     // measured faster than the branch-free form, which needs more registers than two work groups per
@@ -561,8 +569,11 @@ __device__ __forceinline__ void gemm_skinny_body(
                                     acc[t][j][v] = fmaf(tt, da[v], acc[t][j][v]);
                                     if (DUMP) {  // the integer sum of (token, weight row, sub-block or half of one)
                                         const uint32_t tok = token_of(t, 4 * q + v), row = rbase + 16 * j + c;
-                                        if (tok < tok_end && row < n)
-                                            sums[((size_t)tok * n + row) * (k / 32 * KS) + ((st * 2 + u) * 8 + s) * KS + is] =
+                                        // (the odd last step: its first half is the dead one, its second the last super-block)
+                                        const bool last_odd = odd_super && st == steps - 1;
+                                        const uint32_t sbi = last_odd ? n_super - 1 : st * 2 + u;
+                                        if (tok < tok_end && row < n && !(last_odd && u == 0))
+                                            sums[((size_t)tok * n + row) * (k / 32 * KS) + (sbi * 8 + s) * KS + is] =
                                                 ri - 0x4B400000;
                                     }
                                 }
@@ -698,7 +709,7 @@ static __global__ __launch_bounds__(256) void gemm_skinny_reduce(const float *__
 static inline uint32_t skinny_sb_per_split(uint32_t n, uint32_t k) {
     const uint32_t n_super = k / 256, groups = (n + 127) / 128;
     // below 2^25 weights the three launches (token re-layout, this kernel, the reduction) cost more than they save
-    if (k % 512 != 0 || groups >= 448 || (uint64_t)n * k < (1ull << 25)) return 0;
+    if (k % 256 != 0 || groups >= 448 || (uint64_t)n * k < (1ull << 25)) return 0;
     uint32_t splits = (448 + groups - 1) / groups;
     if (splits > 16) splits = 16;
     if (splits > n_super / 4) splits = n_super / 4;
@@ -777,7 +788,7 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
         // whole steps of two super-blocks
         // (expert groups of a mean of up to 20 rows: the launch may be shaped for more than 32 -- twice the mean --
         // and the groups beyond 32 rows take further passes)
-        if (a.k % 512 != 0 || (rows > 32 && !(a.offsets && (size_t)a.m <= 20 * (size_t)a.n_experts))) return SK_NONE;
+        if (a.k % 256 != 0 || a.k < 512 || (rows > 32 && !(a.offsets && (size_t)a.m <= 20 * (size_t)a.n_experts))) return SK_NONE;
         const bool two = rows > 16;
         // the formats with the long strips: the one-tile shapes only (see launch_skinny)
         if (Skinny<F>::ONE_TILE && variant != 0 && variant != 200) return SK_NONE;

@@ -103,6 +103,10 @@ CASES = [
     ([16, 5, 0, 9, 12, 1, 16, 7], 2048, 2048, 16),
     # a mean of 17 rows, sizes unknown to the host: shaped for twice that, more than two token tiles hold
     ([25, 18, 19, 16, 12, 21, 10, 15], 8192, 1024, 0),
+    # an odd number of super-blocks (the last step has one live half): three, five (a chunk boundary inside), eleven
+    ([3, 0, 16, 1], 300, 768, 16),
+    ([12, 7, 16, 3, 9, 14, 2, 5], 8192, 1280, 16),
+    ([20, 3, 15, 4, 17, 1, 19, 12], 8192, 2816, 20),
 ]
 
 
@@ -196,7 +200,9 @@ def test_skinny_full_size_c5_gate(hip, ref):
 @pytest.mark.parametrize("t", FORMATS_1TILE, ids=lambda t: O.NAMES[t])
 @pytest.mark.parametrize("shape", [(16, 4096, 8192), (9, 8200, 4096), (6, 16384, 2048), (13, 2100, 16384), (11, 16384, 3584), (7, 8201, 4096),
                                    # 17..32 rows on fewer than 8192 weight rows: two token tiles (Q6_K, Q8_0: two passes)
-                                   (21, 4096, 8192), (32, 2100, 16384), (17, 4100, 8192)],
+                                   (21, 4096, 8192), (32, 2100, 16384), (17, 4100, 8192),
+                                   # an odd number of super-blocks (43, 17): the last split ends on half a step
+                                   (16, 4096, 11008), (9, 8200, 4352), (21, 4096, 11008)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_skinny_one_matrix_split_k(hip, ref, t, shape):
     """One matrix, up to 16 token rows (32 on fewer than 8192 weight rows), at least 2^25 weights: k is split over work groups, each writes its sums for its
