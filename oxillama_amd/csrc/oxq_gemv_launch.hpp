@@ -176,7 +176,7 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
     const size_t row_bytes = (size_t)(n_cols / F::BLOCK_COLS) * F::BLOCK_BYTES;
     const uint32_t steps = (units + 63) / 64;
     if (steps > 2 || n_rows % 32 != 0 || n_rows == 0) return hipErrorNotSupported;
-    const bool two = row_bytes <= F::TWO_ROW_BATCH_BYTES;
+    const bool two = row_bytes <= F::TWO_ROW_BATCH_BYTES && steps == 1;
     if (grp.offsets) {
         if (grp.n_groups > 64 || grp.n_pairs == 0 || grp.n_pairs > 65535) return hipErrorNotSupported;
         const dim3 grid(n_rows / 32, grp.n_pairs);
