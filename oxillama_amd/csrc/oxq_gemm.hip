@@ -61,7 +61,7 @@ static size_t gemm_planes_bytes(uint32_t m, uint32_t k) {
 // Bytes of the few-token kernel's per-split sums for this call, 0 if it would not split k.
 static size_t gemm_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
     const bool few_token = type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K ||
-                           type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0;
+                           type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q5_K;
     if (!few_token || m > 32 || (m > 16 && n >= 8192) || n == 0) return 0;
     const uint32_t splits = skinny_splits(n, k);
     return splits > 1 ? (size_t)splits * m * n * sizeof(float) : 0;
@@ -70,7 +70,7 @@ static size_t gemm_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t
 // (type, rows, n, k) only, as the caller sizes the workspace without the number of experts.
 static size_t gemm_grouped_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
     if ((type != OXQ_TYPE_Q4_K && type != OXQ_TYPE_IQ4_XS && type != OXQ_TYPE_Q4_0 && type != OXQ_TYPE_Q6_K &&
-         type != OXQ_TYPE_Q8_0) || k % 1024 != 0 || n == 0 ||
+         type != OXQ_TYPE_Q8_0 && type != OXQ_TYPE_Q5_K) || k % 1024 != 0 || n == 0 ||
         n > SKINNY_GROUPED_SPLIT_MAX_N)
         return 0;
     const size_t bytes = (size_t)2 * m * n * sizeof(float);
@@ -226,14 +226,15 @@ hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) 
                : t == OXQ_TYPE_Q6_K   ? skinny_shape<TileQ6K>(a, plan.partial != nullptr, rows, variant)
                : t == OXQ_TYPE_Q8_0   ? skinny_shape<TileQ8_0>(a, plan.partial != nullptr, rows, variant)
                : t == OXQ_TYPE_Q4_0   ? skinny_shape<TileQ4_0>(a, plan.partial != nullptr, rows, variant)
-                                      : (int)SK_NONE;
+                                      : skinny_shape_more(t, a, plan.partial != nullptr, rows, variant);
     };
     if (const int shape = skinny_of(type)) {
         const hipError_t e = type == OXQ_TYPE_Q4_K     ? launch_skinny<TileQ4K>(a, plan, stream, shape)
                              : type == OXQ_TYPE_IQ4_XS ? launch_skinny<TileIQ4XS>(a, plan, stream, shape)
                              : type == OXQ_TYPE_Q6_K   ? launch_skinny<TileQ6K>(a, plan, stream, shape)
                              : type == OXQ_TYPE_Q8_0   ? launch_skinny<TileQ8_0>(a, plan, stream, shape)
-                                                       : launch_skinny<TileQ4_0>(a, plan, stream, shape);
+                             : type == OXQ_TYPE_Q4_0   ? launch_skinny<TileQ4_0>(a, plan, stream, shape)
+                                                       : launch_skinny_more(type, a, plan, stream, shape);
         if (e != hipErrorNotSupported) return e;
     }
     // an earlier call of the same sequence left these activations in the workspace in the byte order this format

@@ -41,6 +41,45 @@ struct TileQ5K {
     }
 };
 
+// The few-token kernel's view of the same block (oxq_gemm_skinny.hpp): lane (c, q) takes bytes 8q..8q+7 of each run of
+// 32 nibble bytes and of qh (the fifth bits of weights 8q..8q+7 of every sub-block: bits g and g + 4 of byte l belong to
+// weight l of sub-blocks 2g and 2g + 1).  352 bytes of a row per step leave LDS for one token tile at two work groups per compute unit.
+template <>
+struct Skinny<TileQ5K> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 176, ROW_STRIDE = 368;
+    static constexpr bool HAS_MIN = true, TABLE = true, ONE_TILE = true;
+    static constexpr int ACT_PERM = 0, KSPLIT = 1;
+    struct Raw {
+        u32x4 hdr;
+        u32x2 qh;
+        u32x2 qs[4];
+    };
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk, uint32_t) {
+        w.hdr = *reinterpret_cast<const u32x4 *>(blk);
+    }
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+        w.qh = *reinterpret_cast<const u32x2 *>(blk + 16 + 8 * q);
+#pragma unroll
+        for (int g = 0; g < 4; g++) w.qs[g] = *reinterpret_cast<const u32x2 *>(blk + 48 + 32 * g + 8 * q);
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const u32x2 v = w.qs[s >> 1];
+        const int bit = (s >> 1) + 4 * (s & 1);  // (reference/q5_k.rs:86,93: bit g for the low nibbles of run g, g + 4 for the high)
+        const uint32_t lo = ((s & 1) ? (v[0] >> 4) & 0x0F0F0F0Fu : v[0] & 0x0F0F0F0Fu) | (((w.qh[0] >> bit) & 0x01010101u) << 4);
+        const uint32_t hi = ((s & 1) ? (v[1] >> 4) & 0x0F0F0F0Fu : v[1] & 0x0F0F0F0Fu) | (((w.qh[1] >> bit) & 0x01010101u) << 4);
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+    static __device__ __forceinline__ void factors(const Raw &w, uint32_t half, int i, float &dsc, float &qneg) {
+        TileQ4K::Hdr hd;
+        hd.w = w.hdr;
+        float d1[1];
+        TileQ4K::factors(hd, 0, 4 * half + i, d1, qneg);  // (the header of Q4_K)
+        dsc = d1[0];
+    }
+};
+
 // 32-weight blocks of interleaved nibbles (byte j = weights 2j, 2j+1), eight blocks per 256-weight
 // step: Q4_1 (reference/q4_1.rs:37-46: 20 B = d, m, 16 B; w = d * q + m, the "+ m" through the
 // zero-point term) and IQ4_NL (reference/iq4_nl.rs:43-51: 18 B = d, 16 B of codebook indices).
@@ -286,6 +325,15 @@ int tile_act_perm_more(uint32_t type) {
 }
 
 bool tile_needs_p16_more(uint32_t type) { return type == OXQ_TYPE_Q2_K; }
+
+// The few-token kernel for the formats of this translation unit: the launch shape that serves a call (0: none), and
+// the launch.
+int skinny_shape_more(uint32_t type, const GemmArgs &a, bool has_partial, uint32_t rows, int variant) {
+    return type == OXQ_TYPE_Q5_K ? skinny_shape<TileQ5K>(a, has_partial, rows, variant) : (int)SK_NONE;
+}
+hipError_t launch_skinny_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream, int shape) {
+    return type == OXQ_TYPE_Q5_K ? launch_skinny<TileQ5K>(a, plan, stream, shape) : hipErrorNotSupported;
+}
 
 hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream) {
     switch (type) {

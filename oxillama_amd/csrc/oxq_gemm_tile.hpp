@@ -773,6 +773,8 @@ struct TilePlan {
 };
 // The formats instantiated in the second translation unit, and the activation byte order they need.
 hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream);
+int skinny_shape_more(uint32_t type, const GemmArgs &a, bool has_partial, uint32_t rows, int variant);
+hipError_t launch_skinny_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream, int shape);
 int tile_act_perm_more(uint32_t type);
 bool tile_needs_p16_more(uint32_t type);
 

@@ -16,8 +16,15 @@ pytestmark = pytest.mark.gpu
 FORMATS = [O.Q4_K, O.IQ4_XS, O.Q4_0]
 # Q6_K (a scale per 16 weights: two MFMAs per sub-block, the integer sums per half) and Q8_0 (544 bytes of a row per
 # step): the kernel's one-token-tile shapes only; expert groups of more than 16 rows take further passes
-ONE_TILE = [O.Q6_K, O.Q8_0]
+ONE_TILE = [O.Q6_K, O.Q8_0, O.Q5_K]
 FORMATS_1TILE = FORMATS + ONE_TILE
+
+
+def weights(t, seed, n, k_):
+    """Synthetic weights: the package's generator for the five formats it knows, the oracle's random blocks otherwise."""
+    if t in synth.BLOCK:
+        return synth.weights(t, seed, n, k_)
+    return O.random_blocks(t, seed, n, k_)
 
 
 def sum_groups(t, k_):
@@ -55,7 +62,7 @@ def _case(ref, t, counts, n, k_, seed):
     rows = int(offsets[-1])
     x = synth.normal_f32(seed, rows * k_).reshape(rows, k_)
     acts = ref.quantize_q8_0(x.reshape(-1)).reshape(rows, k_ // 32 * 34)
-    w = np.stack([synth.weights(t, seed + 10 + e, n, k_) for e in range(len(counts))])
+    w = np.stack([weights(t, seed + 10 + e, n, k_) for e in range(len(counts))])
     return offsets, acts, w
 
 
@@ -166,7 +173,7 @@ def test_skinny_plain_matmul_forced(hip, ref, tuning, t, m):
     if t in ONE_TILE and m > 16:
         pytest.skip("two token tiles: the tile kernel's case for this format")
     n, k_ = 1000, 2048
-    w = synth.weights(t, 31, n, k_)
+    w = weights(t, 31, n, k_)
     x = synth.normal_f32(32 + m, m * k_)
     acts = ref.quantize_q8_0(x).reshape(m, k_ // 32 * 34)
     kern = hip.HipKernel(t)
@@ -212,7 +219,7 @@ def test_skinny_one_matrix_split_k(hip, ref, t, shape):
     from oxillama_amd import linear
     m, n, k_ = shape
     say("skinny split-k", O.NAMES[t], shape)
-    w = synth.weights(t, 71, n, k_)
+    w = weights(t, 71, n, k_)
     acts = ref.quantize_q8_0(synth.normal_f32(72 + m, m * k_)).reshape(m, k_ // 32 * 34)
     bias = synth.normal_f32(73, n)
     kern = hip.HipKernel(t)
@@ -278,7 +285,7 @@ def test_skinny_split_k_on_the_host_routes(hip, ref):
     workspace -- leave room for the per-split sums and take the same kernel."""
     import torch
     t, m, n, k_ = O.Q4_K, 8, 8192, 4096
-    w = synth.weights(t, 81, n, k_)
+    w = weights(t, 81, n, k_)
     x = synth.normal_f32(82, m * k_)
     acts = ref.quantize_q8_0(x).reshape(m, k_ // 32 * 34)
     kern = hip.HipKernel(t)
