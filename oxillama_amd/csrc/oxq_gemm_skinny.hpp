@@ -708,8 +708,12 @@ static __global__ __launch_bounds__(256) void gemm_skinny_reduce(const float *__
 // shape alone, so that the workspace size is.
 static inline uint32_t skinny_sb_per_split(uint32_t n, uint32_t k) {
     const uint32_t n_super = k / 256, groups = (n + 127) / 128;
-    // below 2^25 weights the three launches (token re-layout, this kernel, the reduction) cost more than they save
-    if (k % 256 != 0 || groups >= 448 || (uint64_t)n * k < (1ull << 25)) return 0;
+    // Small matrices: with rows of 4096 columns and more the split still beats the tile kernel's few, long work groups
+    // (16 rows, us: 2048 x 8192 12.1 against 18.3, 1536 x 8960 13.4 against 20.0, 512 x 8192 10.8 against 17.2, 4096 x
+    // 4096 10.9 against 12.6, 1024 x 4096 9.5 against 11.7); with shorter rows it is a tie (2048 x 2048 9.1 against
+    // 8.9), and below 2^22 weights the two launches cost more than they save
+    const uint64_t weights = (uint64_t)n * k;
+    if (k % 256 != 0 || groups >= 448 || weights < (1ull << 22) || (k < 4096 && weights < (1ull << 25))) return 0;
     uint32_t splits = (448 + groups - 1) / groups;
     if (splits > 16) splits = 16;
     if (splits > n_super / 4) splits = n_super / 4;

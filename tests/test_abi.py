@@ -165,8 +165,9 @@ def test_moe_forward_argument_errors_before_touching_the_gpu():
 
 def test_gemm_workspace_size_is_a_function_of_the_shape():
     """oxq_gemm_q8_workspace_bytes: the re-tiled activations (token rows padded to 128 and 128 more, 46 bytes per
-    token block, rounded to 256), plus -- for at most 16 token rows of Q4_K / IQ4_XS / Q4_0 / Q6_K / Q8_0 on a matrix of at least 2^25
-    weights that yields fewer than 448 groups of 128 rows -- the room for the few-token kernel's per-split sums:
+    token block, rounded to 256), plus -- for at most 16 token rows (32 on fewer than 8192 weight rows) of Q4_K / IQ4_XS / Q4_0 /
+    Q6_K / Q8_0 / Q5_K on a matrix of at least 2^22 weights (2^25 where rows are shorter than 4096)
+    that yields fewer than 448 groups of 128 rows -- the room for the few-token kernel's per-split sums:
     splits x m x n floats, splits = min(ceil(448 / groups), k / 1024, 16) taken in even numbers of super-blocks.
     For Q4_K the size is at least what the prefill kernel's planes take."""
     lib = capi.load()
@@ -179,10 +180,14 @@ def test_gemm_workspace_size_is_a_function_of_the_shape():
     assert w(q4k, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4            # 112 groups -> 4 splits of 4
     assert w(iq4xs, 9, 4096, 14336) == planes(9, 14336) + 14 * 9 * 4096 * 4            # 32 groups -> 14 splits of 4
     assert w(q4k, 11, 16384, 3584) == planes(11, 3584) + 3 * 11 * 16384 * 4            # 14 super-blocks: 6 + 6 + 2
-    assert w(q4k, 16, 4096, 4096) == planes(16, 4096)                                  # below 2^25 weights
-    assert w(q4k, 17, 14336, 4096) == planes(17, 4096)                                 # more than 16 rows
+    assert w(q4k, 16, 4096, 4096) == planes(16, 4096) + 4 * 16 * 4096 * 4              # 2^24 weights, rows of 4096: 4 splits of 4
+    assert w(q4k, 16, 4096, 2048) == planes(16, 2048)                                  # below 2^25 weights in rows shorter than 4096
+    assert w(q4k, 16, 512, 4096) == planes(16, 4096)                                   # below 2^22 weights
+    assert w(q4k, 17, 14336, 4096) == planes(17, 4096)                                 # more than 16 rows on 8192 weight rows and more
+    assert w(q4k, 17, 4096, 14336) == planes(17, 14336) + 14 * 17 * 4096 * 4           # ... up to 32 rows on fewer
     assert w(q6k, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4            # Q6_K, Q8_0, Q4_0 alike
-    assert w(13, 16, 14336, 4096) == planes(16, 4096)                                  # Q5_K: no few-token kernel
+    assert w(13, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4             # Q5_K too
+    assert w(10, 16, 14336, 4096) == planes(16, 4096)                                  # Q2_K: no few-token kernel
     assert w(q4k, 16, 128256, 4096) == planes(16, 4096)                                # 1002 groups fill the chip
     # Q4_K: never less than the prefill kernel's planes (74 bytes per token block, token rows padded to 128)
     def prefill(m, k):
