@@ -291,6 +291,10 @@ def main():
     ap.add_argument("--mfma-valu-probe", action="store_true",
                     help="time a kernel of f16 MFMAs and fp32 fmas on register operands in several proportions, one "
                          "work group of 8 waves per compute unit, and exit: how much vector work the matrix work hides")
+    ap.add_argument("--token-sweep", action="store_true",
+                    help="time oxq_gemm_q8_dev (the library's own choice of kernel) over 1..2048 token rows on the matrix "
+                         "shapes of a 7-8 B model (Q4_K; Q6_K on the down shape), three rotating weight sets, replayed "
+                         "graphs; prints one line per (format, shape, rows) with the launch the library took, and exits")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives or sharding here)",
@@ -310,6 +314,42 @@ def main():
     L = max(1, args.layers)
 
     k_q8, k_q4k, k_q6k = quant.HipKernel(Q8_0), quant.HipKernel(Q4_K), quant.HipKernel(Q6_K)
+
+    if args.token_sweep:
+        sweep_stream = torch.cuda.Stream()
+        for t, n, k in ((Q4_K, 4096, 4096), (Q4_K, 1024, 4096), (Q4_K, 14336, 4096), (Q4_K, 4096, 14336), (Q6_K, 4096, 14336)):
+            kern = quant.HipKernel(t)
+            sets = [torch.from_numpy(synth.weights(t, 100 + i, n, k)).to(dev) for i in range(3)]
+            for m in (1, 2, 4, 5, 8, 16, 17, 32, 33, 64, 65, 128, 256, 384, 385, 512, 768, 1024, 2048):
+                xq = torch.empty(m * (k // 32 * 34), dtype=torch.uint8, device=dev)
+                quant.quantize_q8_0_dev(torch.from_numpy(synth.normal_f32(3, m * k)).to(dev), xq)
+                y = torch.zeros(m * n, dtype=torch.float32, device=dev)
+                wk = torch.empty(max(kern.gemm_workspace_bytes(m, n, k), 256), dtype=torch.uint8, device=dev)
+                calls = [0]
+
+                def call():
+                    kern.gemm_q8_dev(sets[calls[0] % 3], xq, y, m, n, k, workspace=wk)
+                    calls[0] += 1
+                reps = 12
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.stream(sweep_stream):
+                    call()
+                    sweep_stream.synchronize()
+                    with torch.cuda.graph(g, stream=sweep_stream):
+                        for _ in range(reps):
+                            call()
+                    best = 1e9
+                    for _ in range(3):
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record(sweep_stream)
+                        g.replay()
+                        e1.record(sweep_stream)
+                        e1.synchronize()
+                        best = min(best, e0.elapsed_time(e1) * 1e3 / reps)
+                print(json.dumps({"format": {Q4_K: "Q4_K", Q6_K: "Q6_K"}[t], "n": n, "k": k, "rows": m, "us": round(best, 1),
+                                  "us_per_row": round(best / m, 3), "launch": last_launch()}), flush=True)
+            del sets
+        return
 
     if args.mfma_valu_probe:
         import ctypes as C

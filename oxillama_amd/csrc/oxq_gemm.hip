@@ -62,7 +62,7 @@ static size_t gemm_planes_bytes(uint32_t m, uint32_t k) {
 static size_t gemm_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
     const bool few_token = type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K ||
                            type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q5_K;
-    if (!few_token || m > 32 || (m > 16 && n >= 8192) || n == 0) return 0;
+    if (!few_token || m > 32 || (m > 16 && (n >= 8192 || (uint64_t)n * k < (1ull << 25))) || n == 0) return 0;
     const uint32_t splits = skinny_splits(n, k);
     return splits > 1 ? (size_t)splits * m * n * sizeof(float) : 0;
 }
