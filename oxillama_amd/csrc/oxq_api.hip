@@ -1377,7 +1377,7 @@ int moe_ffn_impl(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_b
     // GEMV launch over the rows' experts, where the format and row length have that kernel (the bits of the
     // separate launches below).
     bool fused = false;
-    if (pairs <= oxq::GROUPED_GEMV_MAX_ROWS && gate_type == up_type && n_experts <= 64 && intermediate % 32 == 0 &&
+    if (pairs <= oxq::GROUPED_GEMV_MAX_ROWS && gate_type == up_type && n_experts <= 4096 && intermediate % 32 == 0 &&
         oxq::g_gemm_variant.load(std::memory_order_relaxed) == 0 && g.fuse_swiglu.load(std::memory_order_relaxed)) {
         oxq::GateUpGroups grp;
         grp.offsets = d_row_offsets;
@@ -1496,9 +1496,11 @@ int oxq_moe_forward_dev(uint32_t gate_type, const uint8_t *d_gate, size_t gate_s
     float *weights = (float *)(ws + t.weights);
     // One token with a handful of choices: the router's launch also groups and writes the activation rows.
     const bool one = n_tokens == 1 && k <= oxq::GROUPED_GEMV_MAX_ROWS;
+    // (the router's logits may lie, until the experts run, where the gate projection's outputs will)
+    float *logits_scratch = n_tokens * n_experts <= n_tokens * k * intermediate ? (float *)(ws + t.ffn + l.gate) : nullptr;
     OXQ_HIP(oxq::launch_moe_route(d_router, d_x, experts, weights, (uint32_t)n_tokens, (uint32_t)n_experts,
                                   (uint32_t)hidden, (uint32_t)k, offsets, pair_token, token_rows, s,
-                                  one ? ws + t.ffn + l.acts : nullptr));
+                                  one ? ws + t.ffn + l.acts : nullptr, logits_scratch));
     return moe_ffn_impl(gate_type, d_gate, gate_stride_bytes, up_type, d_up, up_stride_bytes, down_type, d_down,
                         down_stride_bytes, n_experts, d_x, n_tokens, k, offsets, pair_token, token_rows, weights, 0, d_out,
                         hidden, intermediate, ws + t.ffn, workspace_bytes - t.ffn, stream, one);

@@ -103,10 +103,14 @@ __global__ __launch_bounds__(256) void gemv_q8_cached(const uint8_t *__restrict_
     uint32_t n_rows = mat == 0 ? n_rows0 : mat == 1 ? n_rows1 : mat == 2 ? n_rows2 : n_rows3;
     if (group_offsets) {
         // Grouped form: blockIdx.y is a token row p; its group e (an expert) is the number of groups that end at or
-        // before p (one load per lane and a ballot; at most 64 groups).  Matrix e, activation row p, output row p.
+        // before p (one load per lane and a ballot per 64 groups).  Matrix e, activation row p, output row p.
         const uint32_t ln = threadIdx.x & 63;
-        const int32_t end = ln < n_groups_e ? group_offsets[ln + 1] : 0x7FFFFFFF;
-        const uint32_t e = min((uint32_t)__builtin_popcountll(__ballot(end <= (int32_t)mat)), n_groups_e - 1);
+        uint32_t below = 0;
+        for (uint32_t base = 0; base < n_groups_e; base += 64) {  // (64 groups per ballot)
+            const int32_t end = base + ln < n_groups_e ? group_offsets[base + ln + 1] : 0x7FFFFFFF;
+            below += (uint32_t)__builtin_popcountll(__ballot(end <= (int32_t)mat));
+        }
+        const uint32_t e = min(below, n_groups_e - 1);
         W = W0 + (size_t)e * w_stride;
         A = static_cast<const uint8_t *>(A) + (size_t)mat * a_stride;
         out = out0 + (size_t)mat * n_rows0;
@@ -247,8 +251,12 @@ __global__ __launch_bounds__(64 * WAVES) void gemv_q8_gate_up_swiglu(const uint8
     if constexpr (PH) ph_t0 = wall_clock64();
     if constexpr (GRP) {
         const uint32_t p = blockIdx.y, ln = threadIdx.x & 63;
-        const int32_t end = ln < n_groups_e ? group_offsets[ln + 1] : 0x7FFFFFFF;
-        const uint32_t e = min((uint32_t)__builtin_popcountll(__ballot(end <= (int32_t)p)), n_groups_e - 1);
+        uint32_t below = 0;
+        for (uint32_t base = 0; base < n_groups_e; base += 64) {  // (64 groups per ballot)
+            const int32_t end = base + ln < n_groups_e ? group_offsets[base + ln + 1] : 0x7FFFFFFF;
+            below += (uint32_t)__builtin_popcountll(__ballot(end <= (int32_t)p));
+        }
+        const uint32_t e = min(below, n_groups_e - 1);
         Wg += (size_t)e * wg_stride;
         Wu += (size_t)e * wu_stride;
         A = static_cast<const uint8_t *>(A) + (size_t)p * a_stride;

@@ -178,7 +178,7 @@ static hipError_t launch_gate_up_swiglu_format(const uint8_t *Wg, const uint8_t 
     if (steps > 2 || n_rows % 32 != 0 || n_rows == 0) return hipErrorNotSupported;
     const bool two = row_bytes <= F::TWO_ROW_BATCH_BYTES && steps == 1;
     if (grp.offsets) {
-        if (grp.n_groups > 64 || grp.n_pairs == 0 || grp.n_pairs > 65535) return hipErrorNotSupported;
+        if (grp.n_groups > 4096 || grp.n_pairs == 0 || grp.n_pairs > 65535) return hipErrorNotSupported;
         const dim3 grid(n_rows / 32, grp.n_pairs);
         const size_t a_stride = (size_t)(n_cols / 32) * 34, hq_stride = (size_t)(n_rows / 32) * 34;
 #define OXQ_LAUNCH_GRP(ST, RBV)                                                                                      \

@@ -149,7 +149,8 @@ hipError_t launch_fill_zero(float *out, size_t n, hipStream_t stream);
 // grouped Q8_0 activation rows there, k copies of the token's blocks, so that no gather launch is needed.
 hipError_t launch_moe_route(const float *router, const float *x, int32_t *experts, float *weights, uint32_t n_tokens,
                             uint32_t n_exp, uint32_t hidden, uint32_t k, int32_t *offsets, int32_t *pair_token,
-                            int32_t *token_rows, hipStream_t stream, uint8_t *acts_one = nullptr);
+                            int32_t *token_rows, hipStream_t stream, uint8_t *acts_one = nullptr,
+                            float *logits_scratch = nullptr);  // (room for n_tokens x n_exp floats, or null)
 
 // Exact top-k (k <= 256, n <= 2^20) of an fp32 vector; workspace of topk_workspace_bytes(n, k) bytes (0: unsupported).
 size_t topk_workspace_bytes(size_t n, size_t k);

@@ -25,55 +25,87 @@ namespace oxq {
 // grouped rows (offsets[e] = how many chosen experts lie below e), every row belongs to token 0,
 // and each row's activations are the token's Q8_0 blocks, written k times while the logits are
 // formed.  Same tables and bytes as the separate launches.
+// The logits of experts e0 .. e0 + 7 for one token, by the 256 threads of a work group: per-thread sums over the
+// columns (16-byte loads), lane sums, one partial per wave into part[4 * q + wave].
+constexpr int ROUTE_EP = 8;  // experts per pass: their loads are in flight together
+template <bool ONE>
+__device__ __forceinline__ void route_logits_pass(const float *__restrict__ router, const float *__restrict__ xr, uint32_t e0,
+                                                  uint32_t n_exp, uint32_t hidden, uint32_t k, uint8_t *__restrict__ acts,
+                                                  float *part) {
+    constexpr int EP = ROUTE_EP;
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const uint32_t n4 = (hidden & 3) == 0 ? hidden / 4 : 0;
+    const float *rr[EP];
+    float acc[EP];
+    for (int q = 0; q < EP; q++) {
+        rr[q] = router + (size_t)min(e0 + q, n_exp - 1) * hidden;
+        acc[q] = 0.0f;
+    }
+    if (n4) {
+        for (uint32_t c = threadIdx.x; c < n4; c += 256) {
+            float xv[4], rv[EP][4];
+            load4(xv, xr + 4 * c);
+#pragma unroll
+            for (int q = 0; q < EP; q++) load4(rv[q], rr[q] + 4 * c);
+#pragma unroll
+            for (int q = 0; q < EP; q++)
+                for (int i = 0; i < 4; i++) acc[q] += rv[q][i] * xv[i];
+            if (ONE && e0 == 0) {
+                // the activation rows are k copies of the token's Q8_0 blocks whichever experts get chosen:
+                // written from the values in hand (eight consecutive lanes hold one block, as in the quantizer;
+                // hidden is a multiple of 32 here, so a block's lanes are in the loop together)
+                for (uint32_t r = 0; r < k; r++)
+                    encode_q8_0_lanes(xv, true, acts + ((size_t)r * (hidden / 32) + c / 8) * 34, c & 7);
+            }
+        }
+    } else {
+        for (uint32_t c = threadIdx.x; c < hidden; c += 256)
+            for (int q = 0; q < EP; q++) acc[q] += rr[q][c] * xr[c];
+    }
+#pragma unroll
+    for (int q = 0; q < EP; q++) {
+        const float v = wave_sum(acc[q]);
+        if (lane == 0 && e0 + q < n_exp) part[4 * q + wave] = v;
+    }
+}
+
+// Many experts: the logits by a launch of their own, a work group per (token, eight experts) -- the same sums in the
+// same order as inside moe_route_kernel, which then starts from them.  (One work group per token walks 128 experts of
+// 2048 columns in 35 us.)
+template <bool ONE>
+__global__ __launch_bounds__(256) void moe_logits_kernel(const float *__restrict__ router, const float *__restrict__ x,
+                                                        float *__restrict__ logits, uint32_t n_exp, uint32_t hidden,
+                                                        uint32_t k, uint8_t *__restrict__ acts) {
+    __shared__ float part[4 * ROUTE_EP];
+    const uint32_t t = blockIdx.x, e0 = blockIdx.y * ROUTE_EP;
+    route_logits_pass<ONE>(router, x + (size_t)t * hidden, e0, n_exp, hidden, k, acts, part);
+    __syncthreads();
+    if (threadIdx.x < ROUTE_EP && e0 + threadIdx.x < n_exp) {
+        const uint32_t q = threadIdx.x;
+        logits[(size_t)t * n_exp + e0 + q] = (part[4 * q] + part[4 * q + 1]) + (part[4 * q + 2] + part[4 * q + 3]);
+    }
+}
+
 template <bool ONE>
 __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict__ router, const float *__restrict__ x,
                                                        int32_t *__restrict__ experts, float *__restrict__ weights,
                                                        uint32_t n_exp, uint32_t hidden, uint32_t k,
                                                        int32_t *__restrict__ offsets, int32_t *__restrict__ pair_token,
-                                                       int32_t *__restrict__ token_rows, uint8_t *__restrict__ acts) {
+                                                       int32_t *__restrict__ token_rows, uint8_t *__restrict__ acts,
+                                                       const float *__restrict__ logits) {
     extern __shared__ float lds[];
     float *probs = lds, *part = lds + n_exp;
     const uint32_t t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const float *xr = x + (size_t)t * hidden;
-    const uint32_t n4 = (hidden & 3) == 0 ? hidden / 4 : 0;
-    constexpr int EP = 8;  // experts per pass: their loads are in flight together
-    for (uint32_t e0 = 0; e0 < n_exp; e0 += EP) {
-        const float *rr[EP];
-        float acc[EP];
-        for (int q = 0; q < EP; q++) {
-            rr[q] = router + (size_t)min(e0 + q, n_exp - 1) * hidden;
-            acc[q] = 0.0f;
-        }
-        if (n4) {
-            for (uint32_t c = threadIdx.x; c < n4; c += 256) {
-                float xv[4], rv[EP][4];
-                load4(xv, xr + 4 * c);
-#pragma unroll
-                for (int q = 0; q < EP; q++) load4(rv[q], rr[q] + 4 * c);
-#pragma unroll
-                for (int q = 0; q < EP; q++)
-                    for (int i = 0; i < 4; i++) acc[q] += rv[q][i] * xv[i];
-                if (ONE && e0 == 0) {
-                    // the activation rows are k copies of the token's Q8_0 blocks whichever experts get chosen:
-                    // written from the values in hand (eight consecutive lanes hold one block, as in the quantizer;
-                    // hidden is a multiple of 32 here, so a block's lanes are in the loop together)
-                    for (uint32_t r = 0; r < k; r++)
-                        encode_q8_0_lanes(xv, true, acts + ((size_t)r * (hidden / 32) + c / 8) * 34, c & 7);
-                }
-            }
-        } else {
-            for (uint32_t c = threadIdx.x; c < hidden; c += 256)
-                for (int q = 0; q < EP; q++) acc[q] += rr[q][c] * xr[c];
-        }
-#pragma unroll
-        for (int q = 0; q < EP; q++) {
-            const float v = wave_sum(acc[q]);
-            if (lane == 0 && e0 + q < n_exp) part[4 * (e0 + q) + wave] = v;
-        }
+    if (logits) {  // formed by moe_logits_kernel
+        for (uint32_t e = threadIdx.x; e < n_exp; e += 256) probs[e] = logits[(size_t)t * n_exp + e];
+    } else {
+        const float *xr = x + (size_t)t * hidden;
+        for (uint32_t e0 = 0; e0 < n_exp; e0 += ROUTE_EP) route_logits_pass<ONE>(router, xr, e0, n_exp, hidden, k, acts, part + 4 * e0);
+        __syncthreads();
+        for (uint32_t e = threadIdx.x; e < n_exp; e += 256)
+            probs[e] = (part[4 * e] + part[4 * e + 1]) + (part[4 * e + 2] + part[4 * e + 3]);
     }
-    __syncthreads();
-    for (uint32_t e = threadIdx.x; e < n_exp; e += 256)
-        probs[e] = (part[4 * e] + part[4 * e + 1]) + (part[4 * e + 2] + part[4 * e + 3]);
+
     __syncthreads();
     int32_t *chosen = reinterpret_cast<int32_t *>(part);  // ONE: the selection, for the other waves (part is free now)
 
@@ -257,16 +289,31 @@ hipError_t launch_moe_combine(const float *y_pairs, const int32_t *token_rows, c
 
 hipError_t launch_moe_route(const float *router, const float *x, int32_t *experts, float *weights, uint32_t n_tokens,
                             uint32_t n_exp, uint32_t hidden, uint32_t k, int32_t *offsets, int32_t *pair_token,
-                            int32_t *token_rows, hipStream_t stream, uint8_t *acts_one) {
+                            int32_t *token_rows, hipStream_t stream, uint8_t *acts_one, float *logits_scratch) {
     if (n_tokens == 0 || n_exp == 0) return hipSuccess;
     const size_t lds = 5 * n_exp * sizeof(float);
+    // From 32 experts on (four passes of a token's work group and more), where the caller has room for n_tokens x n_exp
+    // floats: the logits by a launch of their own.
+    const float *logits = nullptr;
+    if (logits_scratch && n_exp >= 32 && n_tokens <= 65535) {
+        const dim3 grid(n_tokens, (n_exp + ROUTE_EP - 1) / ROUTE_EP);
+        if (acts_one)
+            hipLaunchKernelGGL(moe_logits_kernel<true>, grid, dim3(256), 0, stream, router, x, logits_scratch, n_exp, hidden, k,
+                               acts_one);
+        else
+            hipLaunchKernelGGL(moe_logits_kernel<false>, grid, dim3(256), 0, stream, router, x, logits_scratch, n_exp, hidden, k,
+                               acts_one);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        logits = logits_scratch;
+    }
     if (acts_one) {  // the caller checked: one token, a handful of choices, whole blocks
         hipLaunchKernelGGL(moe_route_kernel<true>, dim3(1), dim3(256), lds, stream, router, x, experts, weights, n_exp,
-                           hidden, k, offsets, pair_token, token_rows, acts_one);
+                           hidden, k, offsets, pair_token, token_rows, acts_one, logits);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(moe_route_kernel<false>, dim3(n_tokens), dim3(256), lds, stream, router, x, experts, weights,
-                       n_exp, hidden, k, offsets, pair_token, token_rows, acts_one);
+                       n_exp, hidden, k, offsets, pair_token, token_rows, acts_one, logits);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(moe_group_kernel, dim3(n_exp), dim3(256), 0, stream, experts, n_tokens * k, k, offsets,
