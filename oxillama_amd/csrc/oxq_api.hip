@@ -1377,7 +1377,7 @@ int moe_ffn_impl(uint32_t gate_type, const uint8_t *d_gate, size_t gate_stride_b
     // GEMV launch over the rows' experts, where the format and row length have that kernel (the bits of the
     // separate launches below).
     bool fused = false;
-    if (pairs <= oxq::GROUPED_GEMV_MAX_ROWS && gate_type == up_type && n_experts <= 4096 && intermediate % 32 == 0 &&
+    if (pairs <= oxq::grouped_gemv_max_rows(n_experts) && gate_type == up_type && n_experts <= 4096 && intermediate % 32 == 0 &&
         oxq::g_gemm_variant.load(std::memory_order_relaxed) == 0 && g.fuse_swiglu.load(std::memory_order_relaxed)) {
         oxq::GateUpGroups grp;
         grp.offsets = d_row_offsets;

@@ -179,7 +179,7 @@ static hipError_t gemm_grouped_by_gemv(uint32_t type, const GemmArgs &a, hipStre
 }
 
 hipError_t launch_gemm_q8(uint32_t type, const GemmArgs &a, hipStream_t stream) {
-    if (a.offsets && !a.sums && !a.bias && a.m <= GROUPED_GEMV_MAX_ROWS && a.n_experts <= 4096 &&
+    if (a.offsets && !a.sums && !a.bias && a.m <= grouped_gemv_max_rows(a.n_experts) && a.n_experts <= 4096 &&
         g_gemm_variant.load(std::memory_order_relaxed) == 0) {
         const hipError_t e = gemm_grouped_by_gemv(type, a, stream);
         if (e != hipErrorNotSupported) return e;
