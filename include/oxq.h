@@ -262,14 +262,18 @@ int oxq_select_activation_route(int route);
 int oxq_activation_route(void);
 
 /* Prefill / decode batch: d_out[m x n] (+)= acts[m rows of Q8_0] x W[n x k]^T, the batched
- * form of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  From 6 rows up
- * (9 where n < 8192), with k a multiple of 256 (the formats of 32-weight blocks: any multiple of
- * 32 from 256 up), every format runs on the int8-MFMA tile
+ * form of matvec_q8_fused (m fused matvecs, Q/reference/q4_k.rs:186-201).  From 5 rows up
+ * (6 where n < 8192, 9 on matrices of fewer than 2^24 weights), with k a multiple of 256 and at
+ * most 65536 (the formats of 32-weight blocks: any multiple of 32 from 256 up), every format runs
+ * on the int8-MFMA tile
  * kernel, which needs oxq_gemm_q8_workspace_bytes() bytes of 256-byte-aligned device scratch:
  * pass it and the call is asynchronous and allocation-free; pass NULL and the library uses
  * its own scratch (the call then serialises and waits for the stream).  Fewer rows, and
  * shapes for which the workspace size is 0, run GEMV launches (up to four rows per pass over
- * the weights) and ignore the workspace.  Q4_K matmuls of many token rows whose 128-token x
+ * the weights) and ignore the workspace.  Decode batches (3..16 rows, up to 32 on matrices of
+ * fewer than 8192 rows) of Q4_K, Q5_K, Q6_K, Q8_0, Q4_0 and IQ4_XS weights run on a kernel that
+ * reads the weights once and splits k over work groups; its per-split sums are part of the
+ * workspace size.  Q4_K matmuls of many token rows whose 128-token x
  * 256-row work groups fill the chip (the prefill shapes) run on the f16 matrix cores instead,
  * with the 6-bit sub-block scale inside the weight operand (exact) and d / dmin applied per
  * super-block: the same integers, fp32 inside the same 1e-5 bar; the workspace size covers both. */
