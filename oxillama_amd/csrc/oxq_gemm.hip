@@ -58,19 +58,23 @@ static size_t gemm_planes_bytes(uint32_t m, uint32_t k) {
     const size_t mpad = ((size_t)m + 127) / 128 * 128 + 128, nsb = tile_padded_sub_blocks(k);
     return nsb * mpad * (32 + 4 + 2 + 8);  // activation bytes, P, f16 scales, the two half-block planes of P
 }
+// The formats the few-token kernel has a policy for.
+static bool gemm_few_token_format(uint32_t type) {
+    return type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K || type == OXQ_TYPE_Q8_0 ||
+           type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q5_K || type == OXQ_TYPE_Q3_K || type == OXQ_TYPE_Q4_1 ||
+           type == OXQ_TYPE_IQ4_NL || type == OXQ_TYPE_Q5_0 || type == OXQ_TYPE_Q5_1 ||
+           type == OXQ_TYPE_Q2_K;
+}
 // Bytes of the few-token kernel's per-split sums for this call, 0 if it would not split k.
 static size_t gemm_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
-    const bool few_token = type == OXQ_TYPE_Q4_K || type == OXQ_TYPE_IQ4_XS || type == OXQ_TYPE_Q6_K ||
-                           type == OXQ_TYPE_Q8_0 || type == OXQ_TYPE_Q4_0 || type == OXQ_TYPE_Q5_K;
-    if (!few_token || m > 32 || (m > 16 && (n >= 8192 || (uint64_t)n * k < (1ull << 25))) || n == 0) return 0;
+    if (!gemm_few_token_format(type) || m > 32 || (m > 16 && (n >= 8192 || (uint64_t)n * k < (1ull << 25))) || n == 0) return 0;
     const uint32_t splits = skinny_splits(n, k);
     return splits > 1 ? (size_t)splits * m * n * sizeof(float) : 0;
 }
 // The same for the grouped form, which splits k in two where an expert's matrix has few row groups: a function of
 // (type, rows, n, k) only, as the caller sizes the workspace without the number of experts.
 static size_t gemm_grouped_partial_bytes(uint32_t type, uint32_t m, uint32_t n, uint32_t k) {
-    if ((type != OXQ_TYPE_Q4_K && type != OXQ_TYPE_IQ4_XS && type != OXQ_TYPE_Q4_0 && type != OXQ_TYPE_Q6_K &&
-         type != OXQ_TYPE_Q8_0 && type != OXQ_TYPE_Q5_K) || k % 1024 != 0 || n == 0 ||
+    if (!gemm_few_token_format(type) || k % 1024 != 0 || n == 0 ||
         n > SKINNY_GROUPED_SPLIT_MAX_N)
         return 0;
     const size_t bytes = (size_t)2 * m * n * sizeof(float);

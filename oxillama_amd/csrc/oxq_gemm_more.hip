@@ -1,5 +1,6 @@
 // The int8-MFMA tile kernel (oxq_gemm_tile.hpp) instantiated for further formats: Q5_K, Q4_1, Q5_0,
-// Q5_1, Q8_1, IQ4_NL.  Each is a small policy (which bytes a lane fetches per group of two
+// Q5_1, Q8_1, IQ4_NL, Q3_K, Q2_K, and the few-token kernel (oxq_gemm_skinny.hpp) for all of them
+// but Q8_1.  Each is a small policy (which bytes a lane fetches per group of two
 // sub-blocks, how they become int8 B operands, how the scale factors are decoded, which byte
 // order the activations need); kernel body, tile shapes and launch policy are shared.  A
 // translation unit of its own so that the two sets compile side by side; only the default tile
@@ -326,13 +327,236 @@ int tile_act_perm_more(uint32_t type) {
 
 bool tile_needs_p16_more(uint32_t type) { return type == OXQ_TYPE_Q2_K; }
 
+// Q3_K in the few-token kernel, as Q6_K there (two scale factors per 32-weight sub-block, one MFMA per 16-weight half,
+// the operand unsigned -- 0..7 -- and the "- 4" in the MFMA's addend).  Lane (c, q) takes weights 8q..8q+7 of every
+// sub-block: bytes 8q..8q+7 of hmask (bit s = sub-block s) and of each run of 32 bytes of 2-bit fields (run n,
+// bits 2j..2j+1 = sub-block 4n + j).  The step's second block starts 110 bytes into the row's strip, 6 past a multiple
+// of 8.  272 bytes = 68 dwords per row: the 64 lanes of an 8-byte read hit different banks.
+template <>
+struct Skinny<TileQ3K> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 110, ROW_STRIDE = 272;
+    static constexpr bool HAS_MIN = false, TABLE = true, ONE_TILE = true;
+    static constexpr int ACT_PERM = 0, KSPLIT = 2, OFFSET = 4;
+    struct Raw {
+        u32x2 hm, qs[2];
+    };
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+        w.hm = strip_get8<6 * U>(blk + 8 * q);
+#pragma unroll
+        for (int n = 0; n < 2; n++) w.qs[n] = strip_get8<6 * U>(blk + 32 + 32 * n + 8 * q);
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const u32x2 l = w.qs[s >> 2];
+        uint32_t v[2];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+            v[i] = ((l[i] >> (2 * (s & 3))) & 0x03030303u) | (((w.hm[i] >> s) & 0x01010101u) << 2);
+        return (long)(((uint64_t)v[1] << 32) | v[0]);
+    }
+    // Lane (c, q) decodes row c's scales 4q .. 4q + 3 (scale 2s + half belongs to that half of sub-block s):
+    // decode_scales, reference/q3_k.rs:30-59 -- index 8n + kk: n = 0 the low six bits of byte kk; n = 1 nibble kk / 4 of
+    // byte 8 + kk % 4, with the top two bits of byte kk above it; each minus 32.
+    template <int U>
+    static __device__ __forceinline__ void block_factors(const uint8_t *blk, uint32_t q, float (&f)[4]) {
+        const uint32_t sw = strip_get4<2 * U>(blk + 96 + 4 * (q & 1)), s2 = strip_get4<2 * U>(blk + 104);
+        const float d = h2f(reinterpret_cast<const StripR2 *>(blk + 108)->v);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const uint32_t byte = (sw >> (8 * b)) & 0xFF;
+            const uint32_t hi = ((s2 >> (8 * b + 4 * (q & 1))) & 0x0F) | ((byte >> 6) << 4);
+            f[b] = d * (float)((int)(q < 2 ? (byte & 0x3F) : hi) - 32);  // exact
+        }
+    }
+};
+
+// Q2_K in the few-token kernel: the walk of Q3_K without the high bit (lane (c, q): bytes 8q..8q+7 of each run of 32
+// bytes of 2-bit fields; the second block of a step starts 84 bytes into the strip row, 4 past a multiple of 8), the
+// operand the field itself, and per 16 weights a scale and a zero-point factor: the latter through a 16 x 16 x 4 fp32
+// MFMA per four halves against P of the tokens' halves.  176 bytes = 44 dwords per strip row.
+template <>
+struct Skinny<TileQ2K> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 84, ROW_STRIDE = 176;
+    static constexpr bool HAS_MIN = true, TABLE = true, ONE_TILE = true;
+    static constexpr int ACT_PERM = 0, KSPLIT = 2, OFFSET = 0;
+    struct Raw {
+        u32x2 qs[2];
+    };
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int n = 0; n < 2; n++) w.qs[n] = strip_get8<4 * U>(blk + 16 + 32 * n + 8 * q);
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const u32x2 l = w.qs[s >> 2];
+        const uint32_t lo = (l[0] >> (2 * (s & 3))) & 0x03030303u, hi = (l[1] >> (2 * (s & 3))) & 0x03030303u;
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+    // Lane (c, q): row c's scale bytes 4q .. 4q + 3 (byte 2s + half: low nibble the scale, high nibble the min of that
+    // half of sub-block s; reference/q2_k.rs:60-75)
+    template <int U>
+    static __device__ __forceinline__ void block_factors(const uint8_t *blk, uint32_t q, float (&f)[4], float (&mn)[4]) {
+        const uint32_t sc = *reinterpret_cast<const uint32_t *>(blk + 4 * q);
+        const uint32_t dd = *reinterpret_cast<const uint32_t *>(blk + 80);
+        const float d = h2f(dd & 0xFFFF), dmin = h2f(dd >> 16);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            const uint32_t byte = (sc >> (8 * b)) & 0xFF;
+            f[b] = d * (float)(byte & 0x0F);        // exact
+            mn[b] = -(dmin * (float)(byte >> 4));   // exact
+        }
+    }
+};
+
+// Q4_1 and IQ4_NL in the few-token kernel, as Q4_0 there: lane (c, q) takes bytes 4q..4q+3 of each block's nibbles
+// (weights 8q + {0,2,4,6} from the low nibbles, 8q + {1,3,5,7} from the high ones: the tokens' bytes even, then odd).
+// Q4_1 (20-byte blocks, every field on a dword boundary): the "+ m" through the zero-point term.  336 bytes = 84
+// dwords per strip row: the 64 lanes of a dword read hit different banks.
+template <>
+struct Skinny<TileQ4_1> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 160, ROW_STRIDE = 336;
+    static constexpr bool HAS_MIN = true, TABLE = true, ONE_TILE = false;
+    static constexpr int ACT_PERM = 1, KSPLIT = 1;
+    struct Raw {
+        uint32_t dm[4];  // d | m << 16 (f16 bits)
+        uint32_t qs[8];
+    };
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk, uint32_t half) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) w.dm[i] = *reinterpret_cast<const uint32_t *>(blk + 20 * (4 * half + i));
+    }
+    static __device__ __forceinline__ void factors(const Raw &w, uint32_t, int i, float &dsc, float &qneg) {
+        dsc = h2f(w.dm[i] & 0xFFFF);
+        qneg = h2f(w.dm[i] >> 16);
+    }
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) w.qs[s] = *reinterpret_cast<const uint32_t *>(blk + 20 * s + 4 + 4 * q);
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const uint32_t lo = w.qs[s] & 0x0F0F0F0Fu, hi = (w.qs[s] >> 4) & 0x0F0F0F0Fu;
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+};
+// IQ4_NL (18-byte blocks, the nibbles 2 past a dword boundary in the even blocks): the codebook byte is the operand.
+template <>
+struct Skinny<TileIQ4NL> {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 144, ROW_STRIDE = 304;
+    static constexpr bool HAS_MIN = false, TABLE = true, ONE_TILE = false;
+    static constexpr int ACT_PERM = 1, KSPLIT = 1;
+    struct Raw {
+        uint32_t d[4];
+        uint32_t qs[8];
+    };
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk, uint32_t half) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) w.d[i] = reinterpret_cast<const StripR2 *>(blk + 18 * (4 * half + i))->v;
+    }
+    static __device__ __forceinline__ void factors(const Raw &w, uint32_t, int i, float &dsc, float &qneg) {
+        dsc = h2f(w.d[i]);
+        qneg = 0.0f;
+    }
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int s = 0; s < 8; s += 2) {
+            w.qs[s] = strip_get4<2>(blk + 18 * s + 2 + 4 * q);
+            w.qs[s + 1] = strip_get4<0>(blk + 18 * (s + 1) + 2 + 4 * q);
+        }
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const uint32_t lo = FmtIQ4XS::lut4(w.qs[s] & 0x0F0F0F0Fu), hi = FmtIQ4XS::lut4((w.qs[s] >> 4) & 0x0F0F0F0Fu);
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+};
+
+// Q5_0 / Q5_1 in the few-token kernel: lane (c, q) takes bytes 4q..4q+3 of each block's nibbles -- weights 4q..4q+3
+// (low nibbles) and 16 + 4q..16 + 4q + 3 (high) -- and their fifth bits, bits 4q.. and 16 + 4q.. of qh; the tokens'
+// bytes are staged in that order (ACT_PERM = 2).  Q5_0's fields sit 2 past a dword boundary in the even blocks.
+// The "- 16" / "+ m" through the zero-point term.  Strip rows of 92 / 100 dwords: no bank conflicts among the 64
+// lanes of a dword read; one token tile (the strips leave LDS for that at two work groups per compute unit).
+template <uint32_t TYPE_ID, uint32_t STRIDE, bool WITH_M>
+struct SkinnyQ5x {
+    static constexpr bool OK = true;
+    static constexpr uint32_t BLOCK = 8 * STRIDE, ROW_STRIDE = 2 * BLOCK + 16;
+    static constexpr bool HAS_MIN = true, TABLE = true, ONE_TILE = true;
+    static constexpr int ACT_PERM = 2, KSPLIT = 1;
+    static constexpr uint32_t QH = WITH_M ? 4 : 2;
+    struct Raw {
+        uint32_t dm[4];
+        uint32_t qs[8], qh[8];
+    };
+    static __device__ __forceinline__ void read_hdr(Raw &w, const uint8_t *blk, uint32_t half) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const uint8_t *b = blk + STRIDE * (4 * half + i);
+            if constexpr (WITH_M) w.dm[i] = *reinterpret_cast<const uint32_t *>(b);
+            else w.dm[i] = reinterpret_cast<const StripR2 *>(b)->v;
+        }
+    }
+    static __device__ __forceinline__ void factors(const Raw &w, uint32_t, int i, float &dsc, float &qneg) {
+        dsc = h2f(w.dm[i] & 0xFFFF);
+        qneg = WITH_M ? h2f(w.dm[i] >> 16) : -(16.0f * dsc);  // exact
+    }
+    template <int U>
+    static __device__ __forceinline__ void read(Raw &w, const uint8_t *blk, uint32_t q) {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const uint8_t *b = blk + STRIDE * s;
+            if constexpr (WITH_M) {
+                w.qh[s] = *reinterpret_cast<const uint32_t *>(b + QH);
+                w.qs[s] = *reinterpret_cast<const uint32_t *>(b + QH + 4 + 4 * q);
+            } else if (s % 2 == 0) {
+                w.qh[s] = strip_get4<2>(b + QH);
+                w.qs[s] = strip_get4<2>(b + QH + 4 + 4 * q);
+            } else {
+                w.qh[s] = strip_get4<0>(b + QH);
+                w.qs[s] = strip_get4<0>(b + QH + 4 + 4 * q);
+            }
+            w.qh[s] >>= 4 * q;  // the lane's fifth bits: bits 0..3 (low nibbles) and 16..19 (high)
+        }
+    }
+    static __device__ __forceinline__ long operand(const Raw &w, int s) {
+        const uint32_t lo = (w.qs[s] & 0x0F0F0F0Fu) | (spread4(w.qh[s] & 0xFu) << 4);
+        const uint32_t hi = ((w.qs[s] >> 4) & 0x0F0F0F0Fu) | (spread4((w.qh[s] >> 16) & 0xFu) << 4);
+        return (long)(((uint64_t)hi << 32) | lo);
+    }
+};
+template <>
+struct Skinny<TileQ5_0> : SkinnyQ5x<OXQ_TYPE_Q5_0, 22, false> {};
+template <>
+struct Skinny<TileQ5_1> : SkinnyQ5x<OXQ_TYPE_Q5_1, 24, true> {};
+
 // The few-token kernel for the formats of this translation unit: the launch shape that serves a call (0: none), and
 // the launch.
 int skinny_shape_more(uint32_t type, const GemmArgs &a, bool has_partial, uint32_t rows, int variant) {
-    return type == OXQ_TYPE_Q5_K ? skinny_shape<TileQ5K>(a, has_partial, rows, variant) : (int)SK_NONE;
+    switch (type) {
+    case OXQ_TYPE_Q5_K: return skinny_shape<TileQ5K>(a, has_partial, rows, variant);
+    case OXQ_TYPE_Q3_K: return skinny_shape<TileQ3K>(a, has_partial, rows, variant);
+    case OXQ_TYPE_Q4_1: return skinny_shape<TileQ4_1>(a, has_partial, rows, variant);
+    case OXQ_TYPE_IQ4_NL: return skinny_shape<TileIQ4NL>(a, has_partial, rows, variant);
+    case OXQ_TYPE_Q2_K: return skinny_shape<TileQ2K>(a, has_partial, rows, variant);
+    case OXQ_TYPE_Q5_0: return skinny_shape<TileQ5_0>(a, has_partial, rows, variant);
+    case OXQ_TYPE_Q5_1: return skinny_shape<TileQ5_1>(a, has_partial, rows, variant);
+    default: return (int)SK_NONE;
+    }
 }
 hipError_t launch_skinny_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream, int shape) {
-    return type == OXQ_TYPE_Q5_K ? launch_skinny<TileQ5K>(a, plan, stream, shape) : hipErrorNotSupported;
+    switch (type) {
+    case OXQ_TYPE_Q5_K: return launch_skinny<TileQ5K>(a, plan, stream, shape);
+    case OXQ_TYPE_Q3_K: return launch_skinny<TileQ3K>(a, plan, stream, shape);
+    case OXQ_TYPE_Q4_1: return launch_skinny<TileQ4_1>(a, plan, stream, shape);
+    case OXQ_TYPE_IQ4_NL: return launch_skinny<TileIQ4NL>(a, plan, stream, shape);
+    case OXQ_TYPE_Q2_K: return launch_skinny<TileQ2K>(a, plan, stream, shape);
+    case OXQ_TYPE_Q5_0: return launch_skinny<TileQ5_0>(a, plan, stream, shape);
+    case OXQ_TYPE_Q5_1: return launch_skinny<TileQ5_1>(a, plan, stream, shape);
+    default: return hipErrorNotSupported;
+    }
 }
 
 hipError_t launch_tiles_more(uint32_t type, const GemmArgs &a, const TilePlan &plan, hipStream_t stream) {

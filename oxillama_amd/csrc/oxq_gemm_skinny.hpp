@@ -222,7 +222,7 @@ struct Skinny<TileQ6K> {
     // 432 bytes = 108 dwords per row: rows start on multiples of 16 bytes
     static constexpr uint32_t BLOCK = 210, ROW_STRIDE = 432;
     static constexpr bool HAS_MIN = false, TABLE = true, ONE_TILE = true;
-    static constexpr int ACT_PERM = 0, KSPLIT = 2;
+    static constexpr int ACT_PERM = 0, KSPLIT = 2, OFFSET = 32;
     struct Raw {
         u32x2 ql[4], qh[2];
     };
@@ -258,10 +258,10 @@ struct Skinny<TileQ6K> {
 };
 
 // LDS bytes per (sub-block, token tile): int8 operands, fp32 scales, and fp32 P (one factor per sub-block) or the
-// MFMA addends of the two halves (two factors)
+// MFMA addends of the two halves (two factors; with a zero-point term, P of each half as well)
 template <class F>
 constexpr uint32_t skinny_act_bytes() {
-    return 512 + 64 + (Skinny<F>::KSPLIT == 2 ? 128 : 64);
+    return 512 + 64 + (Skinny<F>::KSPLIT == 2 ? 128 : 64) + (Skinny<F>::KSPLIT == 2 && Skinny<F>::HAS_MIN ? 128 : 0);
 }
 constexpr uint32_t SKINNY_FAC_STRIDE = 17;  // floats per weight row in a wave's factor tables (16 + pad)
 // LDS bytes of a wave: the strip of its rows' bytes of a step, and the factor tables (one factor per sub-block: of
@@ -323,7 +323,8 @@ __device__ __forceinline__ void gemm_skinny_body(
     float *const ldsD = reinterpret_cast<float *>(ldsA + (size_t)nblk_max * TT * 512);
     float *const ldsP = ldsD + (size_t)nblk_max * TT * 16;       // one factor per sub-block: P
     int *const ldsC = reinterpret_cast<int *>(ldsP);             // two: the MFMA addends, [block][tile][half][16 tokens]
-    uint8_t *const strip = reinterpret_cast<uint8_t *>(ldsP + (size_t)nblk_max * TT * 16 * KS) + wave * WAVE_LDS;
+    float *const ldsP2 = ldsP + (size_t)nblk_max * TT * 16 * KS;  // two factors and a zero-point term: P per half
+    uint8_t *const strip = reinterpret_cast<uint8_t *>(ldsP2 + (KS == 2 && S::HAS_MIN ? (size_t)nblk_max * TT * 32 : 0)) + wave * WAVE_LDS;
     float *const dscT = reinterpret_cast<float *>(strip + NT * 16 * RS);
     float *const minT = dscT + NT * 16 * FS;
 
@@ -373,25 +374,37 @@ __device__ __forceinline__ void gemm_skinny_body(
             const uint32_t l = idx & 63, cc = l >> 2, qq = l & 3;
             u32x2 v = tokA[i];
             const float d = h2f(tokD[i]);
-            if (S::HAS_MIN) {
+            if constexpr (S::HAS_MIN && KS == 1) {
                 int sum = sdot4(v[0], 0x01010101u, sdot4(v[1], 0x01010101u, 0));
                 sum += xor1_i(sum);  // the four threads of a block
                 sum += xor2_i(sum);
                 if (qq == 0) ldsP[(idx >> 6) * 16 + cc] = d * (float)sum;
             }
-            if (KS == 2) {
-                // per half of the block (threads 0, 1 and 2, 3): the addend that turns sum(q a) into sum((q - 32) a),
+            if constexpr (S::HAS_MIN && KS == 2) {  // a zero-point factor per 16 weights: P of each half
+                int sum = sdot4(v[0], 0x01010101u, sdot4(v[1], 0x01010101u, 0));
+                sum += xor1_i(sum);
+                if ((qq & 1) == 0) ldsP2[((idx >> 6) * 2 + (qq >> 1)) * 16 + cc] = d * (float)sum;
+            }
+            if constexpr (KS == 2) {
+                // per half of the block (threads 0, 1 and 2, 3): the addend that turns sum(q a) into sum((q - OFFSET) a),
                 // on top of the 1.5 * 2^23 every result carries
                 int sum = sdot4(v[0], 0x01010101u, sdot4(v[1], 0x01010101u, 0));
                 sum += xor1_i(sum);
-                if ((qq & 1) == 0) ldsC[((idx >> 6) * 2 + (qq >> 1)) * 16 + cc] = 0x4B400000 - 32 * sum;
+                if ((qq & 1) == 0) ldsC[((idx >> 6) * 2 + (qq >> 1)) * 16 + cc] = 0x4B400000 - S::OFFSET * sum;
             }
             if (S::ACT_PERM == 1) {  // even bytes, then odd bytes
                 const uint32_t x0 = v[0], x1 = v[1];
                 v[0] = __builtin_amdgcn_perm(x1, x0, 0x06040200u);
                 v[1] = __builtin_amdgcn_perm(x1, x0, 0x07050301u);
             }
-            *reinterpret_cast<u32x2 *>(ldsA + ((size_t)(idx >> 6) * 64 + qq * 16 + cc) * 8) = v;
+            if constexpr (S::ACT_PERM == 2) {
+                // weights j and j + 16 share a byte: k-slot q holds token bytes 4q .. 4q + 3, then 16 + 4q .. 16 + 4q + 3
+#pragma unroll
+                for (uint32_t i = 0; i < 2; i++)
+                    *reinterpret_cast<uint32_t *>(ldsA + ((size_t)(idx >> 6) * 64 + (2 * (qq & 1) + i) * 16 + cc) * 8 + 4 * (qq >> 1)) = v[i];
+            } else {
+                *reinterpret_cast<u32x2 *>(ldsA + ((size_t)(idx >> 6) * 64 + qq * 16 + cc) * 8) = v;
+            }
             if (qq == 0) ldsD[(idx >> 6) * 16 + cc] = d;
         }
     };
@@ -506,8 +519,16 @@ __device__ __forceinline__ void gemm_skinny_body(
                 for (int j = 0; j < NT; j++) {
                     float f[4];
                     const uint8_t *blk = strip + (16 * j + c) * RS + u * S::BLOCK;
-                    if (u == 0) S::template block_factors<0>(blk, q, f);
-                    else S::template block_factors<1>(blk, q, f);
+                    if constexpr (S::HAS_MIN) {
+                        float mn[4];
+                        if (u == 0) S::template block_factors<0>(blk, q, f, mn);
+                        else S::template block_factors<1>(blk, q, f, mn);
+#pragma unroll
+                        for (int b = 0; b < 4; b++) minT[(16 * j + c) * FS + 4 * q + b] = mn[b];
+                    } else {
+                        if (u == 0) S::template block_factors<0>(blk, q, f);
+                        else S::template block_factors<1>(blk, q, f);
+                    }
 #pragma unroll
                     for (int b = 0; b < 4; b++) dscT[(16 * j + c) * FS + 4 * q + b] = f[b];
                 }
@@ -515,7 +536,23 @@ __device__ __forceinline__ void gemm_skinny_body(
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
             }
-            if (S::HAS_MIN) {
+            if constexpr (S::HAS_MIN && KS == 2) {
+                // zero-point term, a factor per 16 weights: per four halves (slot = 2 * sub-block + half) one
+                // 16 x 16 x 4 fp32 product of P (tokens x halves) and the rows' factors of the block
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+#pragma unroll
+                    for (int t = 0; t < TN; t++)
+                        if (TT == 1 || t < (int)tiles_here) {
+                            const float pa = ldsP2[(((b0 + 2 * g + (q >> 1)) * TT + t) * 2 + (q & 1)) * 16 + c];
+#pragma unroll
+                            for (int j = 0; j < NT; j++) {
+                                const float zb = minT[(16 * j + c) * FS + 4 * g + q];
+                                acc[t][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa, zb, acc[t][j], 0, 0, 0);
+                            }
+                        }
+            }
+            if constexpr (S::HAS_MIN && KS == 1) {
                 // zero-point term: per four sub-blocks one 16 x 16 x 4 fp32 product of P (tokens x sub-blocks) and the
                 // rows' factors, straight into the accumulators
 #pragma unroll

@@ -166,7 +166,7 @@ def test_moe_forward_argument_errors_before_touching_the_gpu():
 def test_gemm_workspace_size_is_a_function_of_the_shape():
     """oxq_gemm_q8_workspace_bytes: the re-tiled activations (token rows padded to 128 and 128 more, 46 bytes per
     token block, rounded to 256), plus -- for at most 16 token rows (32 on fewer than 8192 weight rows) of Q4_K / IQ4_XS / Q4_0 /
-    Q6_K / Q8_0 / Q5_K on a matrix of at least 2^22 weights (2^25 where rows are shorter than 4096)
+    Q6_K / Q8_0 / Q5_K and the other weight formats (all but Q8_1) on a matrix of at least 2^22 weights (2^25 where rows are shorter than 4096)
     that yields fewer than 448 groups of 128 rows -- the room for the few-token kernel's per-split sums:
     splits x m x n floats, splits = min(ceil(448 / groups), k / 1024, 16) taken in even numbers of super-blocks.
     For Q4_K the size is at least what the prefill kernel's planes take."""
@@ -187,7 +187,9 @@ def test_gemm_workspace_size_is_a_function_of_the_shape():
     assert w(q4k, 17, 4096, 14336) == planes(17, 14336) + 14 * 17 * 4096 * 4           # ... up to 32 rows on fewer
     assert w(q6k, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4            # Q6_K, Q8_0, Q4_0 alike
     assert w(13, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4             # Q5_K too
-    assert w(10, 16, 14336, 4096) == planes(16, 4096)                                  # Q2_K: no few-token kernel
+    assert w(11, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4             # Q3_K (and Q4_1, IQ4_NL, Q5_0, Q5_1)
+    assert w(10, 16, 14336, 4096) == planes(16, 4096) + 4 * 16 * 14336 * 4             # Q2_K
+    assert w(9, 16, 14336, 4096) == planes(16, 4096)                                   # Q8_1: no few-token kernel
     assert w(q4k, 16, 128256, 4096) == planes(16, 4096)                                # 1002 groups fill the chip
     # Q4_K: never less than the prefill kernel's planes (74 bytes per token block, token rows padded to 128)
     def prefill(m, k):

@@ -13,10 +13,11 @@ from test_gpu_parity import assert_close, canonical_ref, say
 
 pytestmark = pytest.mark.gpu
 
-FORMATS = [O.Q4_K, O.IQ4_XS, O.Q4_0]
-# Q6_K (a scale per 16 weights: two MFMAs per sub-block, the integer sums per half) and Q8_0 (544 bytes of a row per
-# step): the kernel's one-token-tile shapes only; expert groups of more than 16 rows take further passes
-ONE_TILE = [O.Q6_K, O.Q8_0, O.Q5_K]
+FORMATS = [O.Q4_K, O.IQ4_XS, O.Q4_0, O.Q4_1, O.IQ4_NL]
+# Q6_K, Q3_K, Q2_K (a scale per 16 weights: two MFMAs per sub-block, the integer sums per half), Q8_0 (544 bytes of a
+# row per step), Q5_K, Q5_0, Q5_1: the kernel's one-token-tile shapes only; expert groups of more than 16 rows take
+# further passes
+ONE_TILE = [O.Q6_K, O.Q8_0, O.Q5_K, O.Q3_K, O.Q2_K, O.Q5_0, O.Q5_1]
 FORMATS_1TILE = FORMATS + ONE_TILE
 
 
@@ -28,16 +29,16 @@ def weights(t, seed, n, k_):
 
 
 def sum_groups(t, k_):
-    return k_ // 16 if t == O.Q6_K else k_ // 32
+    return k_ // O.GROUP_COLS[t]
 
 
 def ref_sums(ref, t, w, act_row, n, k_):
     """The integer sums the kernel's dump holds: the reference's; for Q4_0 of the unsigned nibbles (sum q a = sum (q - 8) a
     + 8 sum a: the "- 8" enters in fp32, as in the tile kernel)."""
     s = ref.block_sums(t, w, act_row, n, k_)
-    if t == O.Q4_0:
+    if t in (O.Q4_0, O.Q5_0):  # (Q5_0: the unsigned 5-bit values, "- 16" in fp32)
         a = act_row.reshape(k_ // 32, 34)[:, 2:].view(np.int8).astype(np.int32).sum(axis=1)
-        s = s + 8 * a[None, :]
+        s = s + (8 if t == O.Q4_0 else 16) * a[None, :]
     return s
 
 
