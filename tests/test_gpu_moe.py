@@ -127,7 +127,8 @@ def expert_weights(t, seed, n_exp, n_rows, n_cols):
 
 
 @pytest.mark.parametrize("types", [(O.Q4_K, O.Q4_K, O.Q6_K), (O.Q8_0, O.Q8_0, O.Q8_0), (O.Q4_0, O.IQ4_XS, O.Q4_0),
-                                   (O.Q5_K, O.Q5_K, O.Q5_K)], ids=["q4k_q4k_q6k", "q8_0", "q4_0_iq4xs", "q5k"])
+                                   (O.Q5_K, O.Q5_K, O.Q5_K), (O.Q3_K, O.Q3_K, O.Q2_K), (O.Q5_0, O.Q5_1, O.Q4_1)],
+                         ids=["q4k_q4k_q6k", "q8_0", "q4_0_iq4xs", "q5k", "q3k_q3k_q2k", "q5_0_q5_1_q4_1"])
 @pytest.mark.parametrize("shape", [(4, 2, 1, 256, 512), (8, 2, 3, 512, 256), (8, 2, 40, 512, 256), (6, 3, 130, 256, 768),
                                    (128, 8, 20, 512, 768), (128, 8, 4, 512, 768)], ids=str)  # (the last two: more experts than a wave has
                                                                                             # lanes, most with one row or none; 32 rows: one GEMV per row)
