@@ -295,6 +295,10 @@ def main():
                     help="time oxq_gemm_q8_dev (the library's own choice of kernel) over 1..2048 token rows on the matrix "
                          "shapes of a 7-8 B model (Q4_K; Q6_K on the down shape), three rotating weight sets, replayed "
                          "graphs; prints one line per (format, shape, rows) with the launch the library took, and exits")
+    ap.add_argument("--format-sweep", action="store_true",
+                    help="time oxq_gemm_q8_dev on decode batches of 4 / 8 / 16 / 32 rows for all thirteen formats on the "
+                         "gate and down shapes of a 7-8 B model: the library's choice and, beside it, the int8 tile "
+                         "kernel forced (oxq_set_gemm_variant(99)); random valid blocks; prints one line per case, exits")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no collectives or sharding here)",
@@ -349,6 +353,63 @@ def main():
                 print(json.dumps({"format": {Q4_K: "Q4_K", Q6_K: "Q6_K"}[t], "n": n, "k": k, "rows": m, "us": round(best, 1),
                                   "us_per_row": round(best / m, 3), "launch": last_launch()}), flush=True)
             del sets
+        return
+
+    if args.format_sweep:
+        from oxillama_amd import capi
+        lib = capi.load()
+        # (type id, name, weights per block, bytes per block, offsets of the block's f16 fields)
+        formats = [(2, "Q4_0", 32, 18, (0,)), (3, "Q4_1", 32, 20, (0, 2)), (6, "Q5_0", 32, 22, (0,)), (7, "Q5_1", 32, 24, (0, 2)),
+                   (8, "Q8_0", 32, 34, (0,)), (9, "Q8_1", 32, 36, (0, 2)), (10, "Q2_K", 256, 84, (80, 82)),
+                   (11, "Q3_K", 256, 110, (108,)), (12, "Q4_K", 256, 144, (0, 2)), (13, "Q5_K", 256, 176, (0, 2)),
+                   (14, "Q6_K", 256, 210, (208,)), (20, "IQ4_NL", 32, 18, (0,)), (23, "IQ4_XS", 256, 136, (0,))]
+        sweep_stream = torch.cuda.Stream()
+        rng = np.random.default_rng(5)
+        for t, name, bs, bb, f16_at in formats:
+            assert lib.oxq_block_size(t) == bs and lib.oxq_block_bytes(t) == bb, name
+            kern = quant.HipKernel(t)
+            for n, k in ((F, H), (H, F)):
+                # every payload bit random, the f16 fields finite and small: any such bytes are a legal block
+                blocks = rng.integers(0, 256, size=(256 * (k // bs), bb), dtype=np.uint8)
+                for off in f16_at:
+                    v = rng.uniform(0.005, 0.02, blocks.shape[0]).astype(np.float16)
+                    blocks[:, off:off + 2] = v.view(np.uint8).reshape(-1, 2)
+                one = torch.from_numpy(blocks.reshape(-1)).to(dev)
+                sets = [one.repeat(n // 256) for _ in range(3)]
+                for m in (4, 8, 16, 32):
+                    xq = torch.empty(m * (k // 32 * 34), dtype=torch.uint8, device=dev)
+                    quant.quantize_q8_0_dev(torch.from_numpy(synth.normal_f32(3, m * k)).to(dev), xq)
+                    y = torch.zeros(m * n, dtype=torch.float32, device=dev)
+                    wk = torch.empty(max(kern.gemm_workspace_bytes(m, n, k), 256), dtype=torch.uint8, device=dev)
+                    row = {"format": name, "n": n, "k": k, "rows": m}
+                    for variant, key in ((0, "us"), (99, "tile_kernel_us")):
+                        lib.oxq_set_gemm_variant(variant)
+                        calls = [0]
+
+                        def call():
+                            kern.gemm_q8_dev(sets[calls[0] % 3], xq, y, m, n, k, workspace=wk)
+                            calls[0] += 1
+                        g = torch.cuda.CUDAGraph()
+                        with torch.cuda.stream(sweep_stream):
+                            call()
+                            sweep_stream.synchronize()
+                            if variant == 0:
+                                row["launch"] = last_launch()
+                            with torch.cuda.graph(g, stream=sweep_stream):
+                                for _ in range(12):
+                                    call()
+                            best = 1e9
+                            for _ in range(3):
+                                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                                e0.record(sweep_stream)
+                                g.replay()
+                                e1.record(sweep_stream)
+                                e1.synchronize()
+                                best = min(best, e0.elapsed_time(e1) * 1e3 / 12)
+                        row[key] = round(best, 1)
+                    lib.oxq_set_gemm_variant(0)
+                    print(json.dumps(row), flush=True)
+                del sets, one
         return
 
     if args.mfma_valu_probe:
