@@ -764,6 +764,27 @@ def main():
         lm = [upload(Q6_K, 6000 + i, V, H) for i in range(2)]
         logits = torch.zeros(V, dtype=torch.float32, device=dev)
         kernels["c3_lm_head_q6k_128256x4096"] = time_kernel(k_q6k, Q6_K, lm, xq, logits, V, H, launches=8)
+        # ... followed by the sampler's candidate list: top_k = 40 (the GEMV launch and the two top-k launches), and the
+        # argmax of greedy decoding as those launches and as the one launch in which the GEMV's waves select it
+        def lm_then_list(top_k, one_launch):
+            cand_v = torch.zeros(top_k, dtype=torch.float32, device=dev)
+            cand_i = torch.zeros(top_k, dtype=torch.int32, device=dev)
+            tws = torch.zeros(max(linear.topk_workspace_bytes(V, top_k), linear.lm_head_topk_workspace_bytes(Q6_K, V, H, top_k)) // 8 + 1,
+                              dtype=torch.int64, device=dev)
+
+            def body():
+                for i in range(8):
+                    if one_launch:
+                        linear.lm_head_topk_dev(Q6_K, lm[i % 2], xq, logits, V, H, top_k, cand_v, cand_i, tws)
+                    else:
+                        k_q6k.matvec_q8_fused_dev(lm[i % 2], xq, logits, V, H, accumulate=False)
+                        linear.topk_dev(logits, top_k, cand_v, cand_i, tws)
+            g = capture(body)
+            timed_replay(g)
+            return round(min(timed_replay(g) for _ in range(3)) * 1e3 / 8, 2)
+        kernels["c3_lm_head_then_candidates"] = {"top40_three_launches_us": lm_then_list(40, False),
+                                                 "argmax_one_launch_us": lm_then_list(1, True),
+                                                 "argmax_three_launches_us": lm_then_list(1, False)}
         del lm, logits
 
     # ---- prefill: 512 x 4096 activations times Q4_K 14336 x 4096 ---------------------------
@@ -1078,6 +1099,8 @@ def main():
                "c1_q4_0_frac": get(kernels, "c1_q4_0_4096x4096", "frac_hbm_peak"),
                "c3_lm_head_frac": get(kernels, "c3_lm_head_q6k_128256x4096", "frac_hbm_peak"),
                "c3_lm_head_us": get(kernels, "c3_lm_head_q6k_128256x4096", "us_per_call"),
+               "c3_lm_head_top40_us": get(kernels, "c3_lm_head_then_candidates", "top40_three_launches_us"),
+               "c3_lm_head_argmax_us": get(kernels, "c3_lm_head_then_candidates", "argmax_one_launch_us"),
                "prefill_frac_int8_peak": get(prefill, "frac_int8_peak"), "prefill_gemm_us": get(prefill, "gemm_us"),
                "prefill_TOPS": get(prefill, "TOPS"), "moe_us": get(moe_out, "us_per_step"),
                "moe_frac": get(moe_out, "frac_hbm_peak"),

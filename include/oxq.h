@@ -526,6 +526,26 @@ size_t oxq_topk_workspace_bytes(size_t n, size_t k);
 int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
                  uint32_t *d_out_indices, void *d_workspace, size_t workspace_bytes, void *stream);
 
+/* The vocabulary projection and the candidate list of its logits in one call: d_logits[n_rows] = W . x as
+ * oxq_matvec_q8_fused_dev computes it (accumulate = 0; the same bits), and the k largest logits with their row
+ * indices as oxq_topk_dev lists them (same order, same ties) -- the lm_head's forward followed by the sampler's sort
+ * and truncation (crates/oxillama-runtime/src/sampling/mod.rs:500-509; k = 1: its argmax, mod.rs:652-662) for a
+ * request that edits no logits first (no banned tokens, bias or repetition penalty: those go through
+ * oxq_logits_edit_dev between the two separate calls).  For k <= 8 (greedy decoding, small top_k) on Q6_K, Q8_0,
+ * Q4_K, Q5_K, Q4_0 matrices whose rows take one wave (up to 8192 columns of the 256-weight formats, 4096 of the
+ * others; at most 64 row batches per wave) this is ONE launch: every wave of the GEMV keeps its rows' logits as keys
+ * and selects its k largest after its last row, the work group merges its waves' lists, and the last work group to
+ * finish merges the work groups' lists (a ticket in library-owned device memory, which the launch leaves at zero;
+ * no work group waits for another) -- 128256 x 4096 Q6_K with k = 1: 74.7 us against 78.2 for the separate launches.
+ * Any other k, shape or format runs the GEMV launch and then oxq_topk_dev's launches, with the same results.
+ * 1 <= k <= 256, k <= n_rows <= 2^20.  Needs oxq_lm_head_topk_workspace_bytes() bytes of 8-byte-aligned device
+ * scratch.  No allocation, no synchronisation.  A HIP graph that holds such a launch must not run twice at the same
+ * time (the ticket's address is part of the recorded launch). */
+size_t oxq_lm_head_topk_workspace_bytes(uint32_t type, size_t n_rows, size_t n_cols, size_t k);
+int oxq_lm_head_topk_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_logits,
+                         size_t n_rows, size_t n_cols, size_t k, float *d_out_values, uint32_t *d_out_indices,
+                         void *d_workspace, size_t workspace_bytes, void *stream);
+
 /* The sampler's edits of the logits BEFORE the candidate list, in place (sample_with_rng steps 0 and 1,
  * crates/oxillama-runtime/src/sampling/mod.rs:573-613): banned tokens to -inf; d_bias_values[i] added
  * to logit d_bias_tokens[i] where that logit is still finite (each token at most once: the

@@ -13,7 +13,7 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
-HIP_SOURCES = ["oxq_api.hip", "oxq_gemv.hip", "oxq_gemv_more.hip", "oxq_gemv_f32.hip", "oxq_gemm.hip", "oxq_gemm_more.hip", "oxq_gemm_prefill.hip", "oxq_quantize.hip", "oxq_linear.hip", "oxq_gguf.hip", "oxq_topk.hip", "oxq_moe.hip"]
+HIP_SOURCES = ["oxq_api.hip", "oxq_gemv.hip", "oxq_gemv_more.hip", "oxq_gemv_f32.hip", "oxq_gemm.hip", "oxq_gemm_more.hip", "oxq_gemm_prefill.hip", "oxq_quantize.hip", "oxq_linear.hip", "oxq_gguf.hip", "oxq_topk.hip", "oxq_lm_head.hip", "oxq_moe.hip"]
 HIP_LIB = os.path.join(HERE, "liboxq_hip.so")
 SYNTH_LIB = os.path.join(HERE, "liboxq_synth.so")
 BENCHKIT_LIB = os.path.join(HERE, "liboxq_benchkit.so")

@@ -187,6 +187,9 @@ SIGNATURES = {
     "oxq_topk_workspace_bytes": (C.c_size_t, [C.c_size_t, C.c_size_t]),
     "oxq_topk_dev": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                C.c_void_p]),
+    "oxq_lm_head_topk_workspace_bytes": (C.c_size_t, [C.c_uint32, C.c_size_t, C.c_size_t, C.c_size_t]),
+    "oxq_lm_head_topk_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t,
+                                       C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
     "oxq_block_sums_dev": (C.c_int, [C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
                                      C.c_size_t, C.c_void_p]),
 }

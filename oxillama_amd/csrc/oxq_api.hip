@@ -1600,6 +1600,41 @@ int oxq_topk_dev(const float *d_values, size_t n, size_t k, float *d_out_values,
     return OXQ_OK;
 }
 
+size_t oxq_lm_head_topk_workspace_bytes(uint32_t type, size_t n_rows, size_t n_cols, size_t k) {
+    if (k == 0 || k > n_rows || n_rows > 0xFFFFFFFFull || n_cols > 0xFFFFFFFFull) return 0;
+    const size_t lists = oxq::lm_head_topk_lists_bytes(type, (uint32_t)n_rows, (uint32_t)n_cols, (uint32_t)k);
+    const size_t topk = oxq::topk_workspace_bytes(n_rows, k);
+    if (lists == 0 && topk == 0) return 0;
+    return lists > topk ? lists : topk;
+}
+
+int oxq_lm_head_topk_dev(uint32_t type, const uint8_t *d_weights, const uint8_t *d_acts_q8, float *d_logits, size_t n_rows,
+                         size_t n_cols, size_t k, float *d_out_values, uint32_t *d_out_indices, void *d_workspace,
+                         size_t workspace_bytes, void *stream) {
+    int st = check_dev_shape(type, n_rows, n_cols, true);
+    if (st != OXQ_OK) return st;
+    if (k == 0 || k > n_rows) return fail(OXQ_ERR_DIMENSION_MISMATCH, n_rows, k, "k must be between 1 and the number of rows");
+    const size_t need = oxq_lm_head_topk_workspace_bytes(type, n_rows, n_cols, k);
+    if (need == 0) return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, k, "k above 256 or more than 2^20 rows");
+    if (!d_workspace || workspace_bytes < need)
+        return fail(OXQ_ERR_BUFFER_TOO_SMALL, need, d_workspace ? workspace_bytes : 0, "workspace too small");
+    if (reinterpret_cast<uintptr_t>(d_workspace) & 7)
+        return fail(OXQ_ERR_KERNEL, 8, reinterpret_cast<uintptr_t>(d_workspace) & 7, "workspace must be 8-byte aligned");
+    if (!d_logits || !d_out_values || !d_out_indices) return fail(OXQ_ERR_INTERNAL, 0, 0, "null pointer");
+    if ((st = ensure_init()) != OXQ_OK) return st;
+    if (oxq::lm_head_topk_lists_bytes(type, (uint32_t)n_rows, (uint32_t)n_cols, (uint32_t)k) != 0) {
+        OXQ_HIP(oxq::launch_lm_head_topk(type, d_weights, d_acts_q8, d_logits, (uint32_t)n_rows, (uint32_t)n_cols, (uint32_t)k,
+                                         d_workspace, d_out_values, d_out_indices, (hipStream_t)stream));
+        return OXQ_OK;
+    }
+    // shapes the one-launch form does not take: the GEMV, then the top-k launches
+    OXQ_HIP(oxq::launch_gemv_q8(type, gemv_args(d_weights, d_acts_q8, d_logits, nullptr, n_rows, n_cols, 0), (hipStream_t)stream));
+    if (oxq::topk_workspace_bytes(n_rows, k) == 0)
+        return fail(OXQ_ERR_UNSUPPORTED_SHAPE, 256, k, "k above 256 or more than 2^20 rows");
+    OXQ_HIP(oxq::launch_topk(d_logits, (uint32_t)n_rows, (uint32_t)k, d_out_values, d_out_indices, d_workspace, (hipStream_t)stream));
+    return OXQ_OK;
+}
+
 int oxq_logits_edit_dev(float *d_logits, size_t n, const uint32_t *d_banned, size_t n_banned, const uint32_t *d_bias_tokens,
                         const float *d_bias_values, size_t n_bias, const uint32_t *d_recent, size_t n_recent,
                         size_t window, float repetition_penalty, void *stream) {

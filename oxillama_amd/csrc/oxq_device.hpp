@@ -131,4 +131,18 @@ __device__ __forceinline__ uint64_t wave_max_u64(uint64_t v) {
     return ((uint64_t)mh << 32) | ml;
 }
 
+// Top-k keys: the order-preserving bits of a float, then the complement of its index -- one unsigned maximum decides
+// value and tie (the lower index first) at once; NaN ranks below everything.
+__device__ __forceinline__ uint64_t topk_key(float v, uint32_t index) {
+    uint32_t b = __builtin_bit_cast(uint32_t, v);
+    b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);  // unsigned order == float order
+    if (v != v) b = 0;                                // NaN ranks below everything
+    return ((uint64_t)b << 32) | (uint64_t)(0xFFFFFFFFu - index);
+}
+__device__ __forceinline__ float topk_value(uint64_t key) {
+    uint32_t b = (uint32_t)(key >> 32);
+    b = (b & 0x80000000u) ? (b & 0x7FFFFFFFu) : ~b;
+    return __builtin_bit_cast(float, b);
+}
+
 }  // namespace oxq

@@ -152,6 +152,11 @@ hipError_t launch_moe_route(const float *router, const float *x, int32_t *expert
                             int32_t *token_rows, hipStream_t stream, uint8_t *acts_one = nullptr,
                             float *logits_scratch = nullptr);  // (room for n_tokens x n_exp floats, or null)
 
+// The vocabulary projection and the k largest logits in one launch (oxq_lm_head.hip): bytes of workspace it needs for
+// this shape (0: the one-launch form does not apply), and the launch (hipErrorNotSupported likewise).
+size_t lm_head_topk_lists_bytes(uint32_t type, uint32_t n_rows, uint32_t n_cols, uint32_t k);
+hipError_t launch_lm_head_topk(uint32_t type, const uint8_t *W, const uint8_t *A, float *out, uint32_t n_rows, uint32_t n_cols,
+                               uint32_t k, void *lists, float *out_vals, uint32_t *out_idx, hipStream_t stream);
 // Exact top-k (k <= 256, n <= 2^20) of an fp32 vector; workspace of topk_workspace_bytes(n, k) bytes (0: unsupported).
 size_t topk_workspace_bytes(size_t n, size_t k);
 hipError_t launch_topk(const float *x, uint32_t n, uint32_t k, float *out_vals, uint32_t *out_idx, void *workspace,

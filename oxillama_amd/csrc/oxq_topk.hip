@@ -13,18 +13,6 @@
 
 namespace oxq {
 
-__device__ __forceinline__ uint64_t topk_key(float v, uint32_t index) {
-    uint32_t b = __builtin_bit_cast(uint32_t, v);
-    b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);  // unsigned order == float order
-    if (v != v) b = 0;                                // NaN ranks below everything
-    return ((uint64_t)b << 32) | (uint64_t)(0xFFFFFFFFu - index);
-}
-__device__ __forceinline__ float topk_value(uint64_t key) {
-    uint32_t b = (uint32_t)(key >> 32);
-    b = (b & 0x80000000u) ? (b & 0x7FFFFFFFu) : ~b;
-    return __builtin_bit_cast(float, b);
-}
-
 // Slice s = elements [s * 64 * ITEMS, (s + 1) * 64 * ITEMS), one wave each: its k largest keys, largest
 // first, to cand[s * k .. s * k + k); slots beyond the slice's size hold key 0.  Waves work on their own.
 template <int ITEMS>

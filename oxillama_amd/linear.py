@@ -157,6 +157,18 @@ def topk_dev(d_values, k, d_out_values, d_out_indices, workspace):
                             workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream()))
 
 
+def lm_head_topk_workspace_bytes(quant_type, n_rows, n_cols, k):
+    return capi.load().oxq_lm_head_topk_workspace_bytes(quant_type, n_rows, n_cols, k)
+
+
+def lm_head_topk_dev(quant_type, d_weights, d_acts_q8, d_logits, n_rows, n_cols, k, d_out_values, d_out_indices, workspace):
+    """The vocabulary projection (logits to d_logits) and the k largest logits with their row indices, in one launch
+    where the shape allows it (oxq_lm_head_topk_dev)."""
+    _check(capi.load().oxq_lm_head_topk_dev(quant_type, d_weights.data_ptr(), d_acts_q8.data_ptr(), d_logits.data_ptr(),
+                                            n_rows, n_cols, k, d_out_values.data_ptr(), d_out_indices.data_ptr(),
+                                            workspace.data_ptr(), workspace.numel() * workspace.element_size(), _stream()))
+
+
 def logits_edit_dev(d_logits, d_banned=None, d_bias_tokens=None, d_bias_values=None, d_recent=None, window=0,
                     repetition_penalty=1.0):
     """The sampler's edits of the logits before the candidate list (sampling/mod.rs:573-613), in place: banned tokens,
