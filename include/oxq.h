@@ -271,7 +271,7 @@ int oxq_activation_route(void);
  * its own scratch (the call then serialises and waits for the stream).  Fewer rows, and
  * shapes for which the workspace size is 0, run GEMV launches (up to four rows per pass over
  * the weights) and ignore the workspace.  Decode batches (3..16 rows, up to 32 on matrices of
- * fewer than 8192 rows) of Q4_K, Q5_K, Q6_K, Q8_0, Q4_0 and IQ4_XS weights run on a kernel that
+ * fewer than 8192 rows) in every weight format but Q8_1 run on a kernel that
  * reads the weights once and splits k over work groups; its per-split sums are part of the
  * workspace size.  Q4_K matmuls of many token rows whose 128-token x
  * 256-row work groups fill the chip (the prefill shapes) run on the f16 matrix cores instead,
