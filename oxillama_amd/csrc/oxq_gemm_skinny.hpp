@@ -823,13 +823,25 @@ static hipError_t launch_skinny_shape(const GemmArgs &a, const TilePlan &p, hipS
 //    groups on no split is needed (57344 x 4096, 16 rows: 44 us against 56).
 enum SkinnyShape { SK_NONE = 0, SK_1_4, SK_1_8, SK_2_2, SK_1_4_SPLIT, SK_1_16, SK_2_8, SK_W4_1_8, SK_W4_2_4, SK_2_4, SK_2_2_SPLIT };
 
+// Expert groups of up to this many rows in the mean stay with the kernel's two-tile shapes (larger groups take further
+// passes over their expert's weights).  20 where the tile kernel is the alternative at its best (Q4_K, IQ4_XS: 8
+// experts of 14336 x 4096 with 13..28 rows 92-101 us against 105 + 5); the formats of 32-weight blocks, whose tile
+// kernel is bound by its many small loads, keep the few-token kernel up to 48 (the Mixtral-shaped layer at 96 / 128 /
+// 192 tokens, us: Q4_1 348 / 436 / 625 against 527 / 671 / 712 on the tile kernel, Q4_0 348 / 440 / 630 against 486 /
+// 619 / 663, IQ4_NL 331 / 438 / 627 against 490 / 628 / 648; at 256 tokens, a mean of 64, the tile kernel is level).
+template <class F>
+constexpr uint32_t skinny_grouped_mean_limit() {
+    return tile_ragged_k<F>::value ? 48 : 20;
+}
+
 template <class F>
 static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int variant) {
     if constexpr (Skinny<F>::OK) {
+        constexpr size_t MEAN_LIMIT = skinny_grouped_mean_limit<F>();
         // whole steps of two super-blocks
         // (expert groups of a mean of up to 20 rows: the launch may be shaped for more than 32 -- twice the mean --
         // and the groups beyond 32 rows take further passes)
-        if (a.k % 256 != 0 || a.k < 512 || (rows > 32 && !(a.offsets && (size_t)a.m <= 20 * (size_t)a.n_experts))) return SK_NONE;
+        if (a.k % 256 != 0 || a.k < 512 || (rows > 32 && !(a.offsets && (size_t)a.m <= MEAN_LIMIT * (size_t)a.n_experts))) return SK_NONE;
         const bool two = rows > 16;
         // the formats with the long strips: the one-tile shapes only (see launch_skinny)
         if (Skinny<F>::ONE_TILE && variant != 0 && variant != 200) return SK_NONE;
@@ -869,7 +881,7 @@ static int skinny_shape(const GemmArgs &a, bool has_partial, uint32_t rows, int 
                 }
                 // (a mean of up to 20 rows: 8 experts of 14336 x 4096 with 13..28 rows 92-101 us against 105 + 5 on
                 // the tile kernel and its token re-layout)
-                if ((size_t)a.m > 20 * (size_t)a.n_experts) return SK_NONE;
+                if ((size_t)a.m > MEAN_LIMIT * (size_t)a.n_experts) return SK_NONE;
                 if (many) return SK_2_2;
                 // few row groups per expert: each expert's k in two halves, where that gives every compute unit a
                 // work group and the workspace has room for the halves' sums

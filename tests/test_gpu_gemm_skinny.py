@@ -145,6 +145,26 @@ def test_skinny_grouped_against_oracle(hip, ref, t, case):
     assert torch.equal(dy3[:rows], dy[:rows] + dy[:rows]) and torch.equal(dy3[rows:], dy[rows:])
 
 
+@pytest.mark.parametrize("t", [O.Q4_0, O.Q4_1, O.IQ4_NL, O.Q4_K], ids=lambda t: O.NAMES[t])
+def test_skinny_grouped_larger_groups_in_the_formats_of_32_weight_blocks(hip, ref, t):
+    """A mean of 32 rows per expert (sizes unknown to the host: the launch is shaped for 64, groups beyond 32 rows take a
+    second pass): the formats of 32-weight blocks stay on the few-token kernel up to a mean of 48, Q4_K goes to the tile
+    kernel from 20."""
+    counts, n, k_ = [42, 24, 30, 29, 27, 34, 32, 38], 8192, 512
+    offsets, acts, w = _case(ref, t, counts, n, k_, 5100)
+    rows = int(offsets[-1])
+    dy, _ = _run(hip, t, w, acts, offsets, n, k_, 0)
+    took = last_launch()
+    say(O.NAMES[t], took)
+    assert took.startswith("gemm_skinny_kernel") == (t != O.Q4_K), took
+    y = dy.cpu().numpy()
+    assert np.all(y[rows:] == 7.0)
+    sample = sorted(set(list(range(0, rows, 11)) + [int(o) for o in offsets[:-1]] + [int(o) - 1 for o in offsets[1:]]))
+    y_ref, _ = _oracle_rows(ref, t, w, acts, offsets, n, k_, sample)
+    for r in sample:
+        assert_close(y[r], y_ref[r], f"row {r}")
+
+
 @pytest.mark.parametrize("t", FORMATS, ids=lambda t: O.NAMES[t])
 def test_skinny_shapes_give_the_same_bits(hip, ref, tuning, t):
     """Every launch shape of the kernel (waves per work group, super-blocks per chunk) adds a result's terms in the same
